@@ -1,0 +1,130 @@
+"""ctypes binding of libcrystalframer_hip.so (the C ABI declared in include/crystalframer_hip.h).
+
+There is no CPU fallback: if the library is missing, or an entry point reports an error, the call
+raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from typing import Optional
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
+ABI_VERSION = 1
+
+CFH_WINDOW_REFERENCE = 0
+CFH_WINDOW_WIDE = 1
+
+
+class CfhParams(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", ctypes.c_int32),
+        ("num_heads", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32),
+        ("dist_bins", ctypes.c_int32),
+        ("angle_bins", ctypes.c_int32),
+        ("cos_abs", ctypes.c_int32),
+        ("lattice_range", ctypes.c_int32),
+        ("minimum_range", ctypes.c_int32),
+        ("window_mode", ctypes.c_int32),
+        ("dist_max", ctypes.c_float),
+        ("dist_wscale", ctypes.c_float),
+        ("angle_wscale", ctypes.c_float),
+        ("dist_coef", ctypes.c_float),
+        ("angle_coef", ctypes.c_float),
+        ("cutoff_radius", ctypes.c_float),
+        ("prune_log2", ctypes.c_float),
+        ("symm_break_noise", ctypes.c_float),
+        ("noise_seed", ctypes.c_uint64),
+        ("grad_coef_quirk", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_frame_axis1",
+           "cfh_frame_axis2", "cfh_framed_pe_forward", "cfh_framed_pe_backward")
+
+_lib = None
+_lock = threading.Lock()
+_P = ctypes.c_void_p
+_I64 = ctypes.c_int64
+
+
+def load():
+    """Load the library once; raise if it is absent or its ABI version differs."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m crystalframer_amd.build` "
+                "(hipcc --offload-arch=gfx950). There is no fallback path.")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name in EXPORTS:
+            if not hasattr(lib, name):
+                raise RuntimeError(f"{LIB_PATH} does not export {name}")
+        lib.cfh_abi_version.restype = ctypes.c_int
+        lib.cfh_last_error.restype = ctypes.c_char_p
+        lib.cfh_workspace_bytes.restype = ctypes.c_size_t
+        lib.cfh_workspace_bytes.argtypes = [ctypes.POINTER(CfhParams), _I64, _I64]
+        pp = ctypes.POINTER(CfhParams)
+        lib.cfh_frame_axis1.restype = ctypes.c_int
+        lib.cfh_frame_axis1.argtypes = [pp] + [_P] * 10 + [_I64] * 3 + [_P, _P, ctypes.c_size_t, _P]
+        lib.cfh_frame_axis2.restype = ctypes.c_int
+        lib.cfh_frame_axis2.argtypes = [pp] + [_P] * 11 + [_I64] * 3 + [_P, _P, ctypes.c_size_t, _P]
+        lib.cfh_framed_pe_forward.restype = ctypes.c_int
+        lib.cfh_framed_pe_forward.argtypes = [pp] + [_P] * 13 + [_I64] * 3 + [_P] * 4 + [ctypes.c_size_t, _P]
+        lib.cfh_framed_pe_backward.restype = ctypes.c_int
+        lib.cfh_framed_pe_backward.argtypes = [pp] + [_P] * 16 + [_I64] * 3 + [_P] * 6 + [ctypes.c_size_t, _P]
+        if lib.cfh_abi_version() != ABI_VERSION:
+            raise RuntimeError(f"ABI version {lib.cfh_abi_version()} of {LIB_PATH} != {ABI_VERSION}")
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        msg = load().cfh_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"{what} failed (code {rc}): {msg}")
+
+
+def ptr(t: Optional[torch.Tensor]):
+    """Device pointer of a contiguous tensor (None -> NULL)."""
+    if t is None:
+        return None
+    if not t.is_contiguous():
+        raise ValueError("tensor passed to the HIP library must be contiguous")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def require_gpu(*tensors: torch.Tensor):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "crystalframer_amd operators run on a HIP device only (tensor on "
+                f"{t.device}); there is no CPU path")
+
+
+_workspaces = {}
+
+
+def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """Scratch buffer handed to the library, one per (device, stream): kernels of one stream run
+    in order, so they can share it; grown on demand, reused across calls."""
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def current_stream_ptr(device: torch.device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)

@@ -1,0 +1,325 @@
+// C ABI of the gfx950 kernels (see include/crystalframer_hip.h).  Host side: argument checks,
+// constant preparation, work-queue reset and kernel launches.  Nothing here allocates or
+// synchronises.
+#include "../../include/crystalframer_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "device_common.hpp"
+#include "frame_select.hpp"
+#include "framed_pe_bwd.hpp"
+#include "framed_pe_fwd.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+constexpr int MAX_HEADS = 64;
+constexpr size_t COUNTER_BYTES = 256;          // MAX_HEADS int32 work-queue heads
+constexpr int WAVES_PER_SIMD = 3;
+
+__global__ void reset_counters_kernel(int32_t* counters) { counters[threadIdx.x] = 0; }
+
+// number of compute units of the current device (cached per device)
+int device_cus() {
+    static int cus[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cus[dev] == 0) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cus[dev] = v;
+    }
+    return cus[dev];
+}
+
+// persistent wavefronts to launch: a multiple of H, enough to fill the device, no more than items
+int launch_waves(int64_t N, int H) {
+    int cus = device_cus();
+    if (cus <= 0) cus = 256;
+    int64_t want = (int64_t)cus * 4 * WAVES_PER_SIMD;
+    want = (want / H) * H;
+    if (want < H) want = H;
+    const int64_t items = N * H;
+    if (want > items) want = items;
+    return (int)want;
+}
+
+int check_params(const cfh_params* p) {
+    if (!p) return fail(CFH_EINVAL, "params is NULL");
+    if (p->struct_size != (int32_t)sizeof(cfh_params))
+        return fail(CFH_EINVAL, "cfh_params.struct_size %d != %zu (header/library mismatch)", p->struct_size,
+                    sizeof(cfh_params));
+    if (p->num_heads < 1 || p->num_heads > MAX_HEADS)
+        return fail(CFH_EINVAL, "num_heads %d outside 1..%d", p->num_heads, MAX_HEADS);
+    if (p->head_dim != cfh::DH) return fail(CFH_EINVAL, "head_dim %d not compiled (only %d)", p->head_dim, cfh::DH);
+    if (p->dist_bins != 0 && p->dist_bins != cfh::NBINS)
+        return fail(CFH_EINVAL, "dist_bins %d not compiled (0 or %d)", p->dist_bins, cfh::NBINS);
+    if (p->angle_bins != 0 && p->angle_bins != cfh::NBINS)
+        return fail(CFH_EINVAL, "angle_bins %d not compiled (0 or %d)", p->angle_bins, cfh::NBINS);
+    if (p->angle_bins != 0 && p->dist_bins == 0)
+        return fail(CFH_EINVAL, "angle encoding requires the distance encoding (dist_bins > 0)");
+    if (p->lattice_range < 0 || p->lattice_range > cfh::RMAX)
+        return fail(CFH_EINVAL, "lattice_range %d outside 0..%d", p->lattice_range, cfh::RMAX);
+    if (p->minimum_range < 0 || p->minimum_range > cfh::RMAX)
+        return fail(CFH_EINVAL, "minimum_range %d outside 0..%d", p->minimum_range, cfh::RMAX);
+    if (p->window_mode != CFH_WINDOW_REFERENCE && p->window_mode != CFH_WINDOW_WIDE)
+        return fail(CFH_EINVAL, "window_mode %d unknown", p->window_mode);
+    return CFH_OK;
+}
+
+// window widths for the configured scales; only (9,33) and (11,41) are instantiated
+int window_widths(const cfh_params* p, int* wl, int* wa) {
+    const int cut = (p->window_mode == CFH_WINDOW_WIDE) ? 5 : 4;
+    *wl = (int)std::ceil(2.0 * (double)p->dist_wscale * cut + 1.0);
+    *wa = (int)std::ceil(2.0 * (double)p->angle_wscale * cut + 1.0);
+    const int want_l = cut == 4 ? 9 : 11, want_a = cut == 4 ? 33 : 41;
+    if (p->dist_bins > 0 && *wl != want_l)
+        return fail(CFH_EINVAL, "dist_wscale %g gives a %d-bin window; only wscale 1.0 (%d bins) is compiled",
+                    (double)p->dist_wscale, *wl, want_l);
+    if (p->angle_bins > 0 && *wa != want_a)
+        return fail(CFH_EINVAL, "angle_wscale %g gives a %d-bin window; only wscale 4.0 (%d bins) is compiled",
+                    (double)p->angle_wscale, *wa, want_a);
+    return CFH_OK;
+}
+
+cfh::BasisConsts basis_consts(const cfh_params* p) {
+    cfh::BasisConsts bc;
+    std::memset(&bc, 0, sizeof(bc));
+    const double cut = (p->window_mode == CFH_WINDOW_WIDE) ? 5.0 : 4.0;
+    const double sl2e = std::sqrt(1.4426950408889634);
+    if (p->dist_bins > 0) {
+        const double interval = (double)p->dist_max / p->dist_bins;
+        bc.inv_interval = (float)(1.0 / interval);
+        bc.start_off = (float)(cut * p->dist_wscale + 1.0);
+        const double step = sl2e / ((double)p->dist_wscale * std::sqrt(2.0));
+        bc.len_step = (float)step;
+        bc.len_cc = (float)std::exp2(-2.0 * step * step);
+    }
+    if (p->angle_bins > 0) {
+        const int A = p->angle_bins;
+        const double interval = (p->cos_abs ? 1.0 : 2.0) / (A - 1);
+        const double sigma = (p->cos_abs ? 1.0 : 2.0) * (double)p->angle_wscale / (A - 1);
+        bc.ang_inv_interval = (float)(1.0 / interval);
+        bc.ang_end_off = (float)(1.0 + cut * sigma);
+        bc.ang_interval = (float)interval;
+        const double sinv = sl2e / (sigma * std::sqrt(2.0));
+        bc.ang_sigma_inv = (float)sinv;
+        bc.ang_step = (float)(interval * sinv);
+        bc.ang_cc = (float)std::exp2(-2.0 * interval * sinv * interval * sinv);
+        bc.ang_mu0 = p->cos_abs ? 0.0f : -1.0f;
+    }
+    return bc;
+}
+
+int check_geometry(const float* a_ih, const float* rpos, const float* tvecs, const int64_t* batch,
+                   const int64_t* edges, const int64_t* e_start, int64_t N, int64_t E, int64_t B) {
+    if (N < 0 || E < 0 || B < 0) return fail(CFH_EINVAL, "negative size N=%lld E=%lld B=%lld", (long long)N, (long long)E, (long long)B);
+    if (N > 0x7fffffffLL / 64 || E > 0x7fffffffLL / 64)
+        return fail(CFH_EINVAL, "N=%lld or E=%lld beyond the 32-bit index range of the kernels", (long long)N, (long long)E);
+    if (N == 0) return CFH_OK;
+    if (!a_ih || !rpos || !tvecs || !batch || !edges || !e_start)
+        return fail(CFH_EINVAL, "a_ih, rpos, tvecs, batch, edges and e_start must not be NULL");
+    return CFH_OK;
+}
+
+int check_workspace(void* ws, size_t have, size_t need) {
+    if (!ws || have < need) return fail(CFH_EWORKSPACE, "workspace of %zu bytes needed, %zu given", need, have);
+    if (((uintptr_t)ws & 255) != 0) return fail(CFH_EWORKSPACE, "workspace must be 256-byte aligned");
+    return CFH_OK;
+}
+
+void fill_common(cfh::KernelArgs& A, const cfh_params* p, const float* a_ih, const float* rpos,
+                 const float* tvecs, const float* rvlen, const int64_t* batch, const int64_t* edges,
+                 const int64_t* e_start, const int32_t* order, int64_t N, int64_t E, void* workspace) {
+    std::memset(&A, 0, sizeof(A));
+    A.a_ih = a_ih; A.rpos = rpos; A.tvecs = tvecs; A.rvlen = rvlen;
+    A.batch = batch; A.edges = edges; A.e_start = e_start; A.order = order;
+    A.counters = reinterpret_cast<int32_t*>(workspace);
+    A.N = (int32_t)N; A.E = (int32_t)E; A.H = p->num_heads;
+    A.cutoff_radius = rvlen ? p->cutoff_radius : 0.0f;
+    A.lattice_range = p->lattice_range; A.minimum_range = p->minimum_range;
+    A.prune_log2 = p->prune_log2;
+    A.dist_coef = p->dist_coef; A.angle_coef = p->angle_coef;
+    A.gz_coef = p->grad_coef_quirk ? p->dist_coef : 1.0f;
+    A.gw_dist_coef = p->grad_coef_quirk ? 1.0f : p->dist_coef;
+    A.noise = p->symm_break_noise;
+    A.seed_lo = (uint32_t)(p->noise_seed & 0xffffffffu);
+    A.seed_hi = (uint32_t)(p->noise_seed >> 32);
+    A.bc = basis_consts(p);
+}
+
+int finish_launch(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(CFH_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return CFH_OK;
+}
+
+template <typename Kern>
+int launch_persistent(Kern kern, const cfh::KernelArgs& A, int waves, hipStream_t st, const char* what) {
+    hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(MAX_HEADS), 0, st, A.counters);
+    hipLaunchKernelGGL(kern, dim3(waves), dim3(cfh::WAVE), 0, st, A);
+    return finish_launch(what);
+}
+
+}  // namespace
+
+extern "C" {
+
+int cfh_abi_version(void) { return CFH_ABI_VERSION; }
+
+const char* cfh_last_error(void) { return g_err; }
+
+size_t cfh_workspace_bytes(const cfh_params* p, int64_t N, int64_t E) {
+    (void)E;
+    if (check_params(p) != CFH_OK) return 0;
+    const int waves = launch_waves(N > 0 ? N : 1, p->num_heads);
+    return COUNTER_BYTES + (size_t)waves * 4 * cfh::DH * cfh::NBINS * sizeof(float);
+}
+
+int cfh_frame_axis1(const cfh_params* p, const float* q, const float* k, const float* a_ih,
+                    const float* rpos, const float* tvecs, const float* rvlen, const int64_t* batch,
+                    const int64_t* edges, const int64_t* e_start, const int32_t* order, int64_t N,
+                    int64_t E, int64_t B, float* frame1, void* workspace, size_t workspace_bytes,
+                    void* stream) {
+    int rc = check_params(p);
+    if (rc) return rc;
+    if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
+    if (N == 0) return CFH_OK;
+    if (!q || !k || !frame1) return fail(CFH_EINVAL, "q, k and frame1 must not be NULL");
+    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES))) return rc;
+    cfh::KernelArgs A;
+    fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
+    A.q = q; A.k = k; A.out_frame = frame1;
+    return launch_persistent(cfh::frame_axis_kernel<false>, A, launch_waves(N, p->num_heads),
+                             (hipStream_t)stream, "frame_axis1");
+}
+
+int cfh_frame_axis2(const cfh_params* p, const float* q, const float* k, const float* a_ih,
+                    const float* rpos, const float* tvecs, const float* rvlen, const int64_t* batch,
+                    const int64_t* edges, const int64_t* e_start, const int32_t* order,
+                    const float* frame1, int64_t N, int64_t E, int64_t B, float* frame2max,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_params(p);
+    if (rc) return rc;
+    if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
+    if (N == 0) return CFH_OK;
+    if (!q || !k || !frame1 || !frame2max) return fail(CFH_EINVAL, "q, k, frame1 and frame2max must not be NULL");
+    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES))) return rc;
+    cfh::KernelArgs A;
+    fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
+    A.q = q; A.k = k; A.frame1 = frame1; A.out_frame = frame2max;
+    return launch_persistent(cfh::frame_axis_kernel<true>, A, launch_waves(N, p->num_heads),
+                             (hipStream_t)stream, "frame_axis2");
+}
+
+#define CFH_DISPATCH_PE(KERNEL, HAS_LEN, HAS_ANG)                                                   \
+    do {                                                                                            \
+        if (wide) {                                                                                 \
+            if (p->cos_abs) rc = launch_persistent(KERNEL<11, 41, true, HAS_LEN, HAS_ANG>, A, waves, st, what);  \
+            else rc = launch_persistent(KERNEL<11, 41, false, HAS_LEN, HAS_ANG>, A, waves, st, what);            \
+        } else {                                                                                    \
+            if (p->cos_abs) rc = launch_persistent(KERNEL<9, 33, true, HAS_LEN, HAS_ANG>, A, waves, st, what);   \
+            else rc = launch_persistent(KERNEL<9, 33, false, HAS_LEN, HAS_ANG>, A, waves, st, what);             \
+        }                                                                                           \
+    } while (0)
+
+int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,
+                          const float* rvlen, const int64_t* batch, const int64_t* edges,
+                          const int64_t* e_start, const int32_t* order, const float* W_dist,
+                          const float* W_axis1, const float* W_axis2, const float* W_axis3,
+                          const float* frames, int64_t N, int64_t E, int64_t B, float* z, float* psi,
+                          float* d2min_out, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_params(p);
+    if (rc) return rc;
+    if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
+    if (N == 0) return CFH_OK;
+    if (!z) return fail(CFH_EINVAL, "z must not be NULL");
+    const bool has_len = p->dist_bins > 0 && W_dist != nullptr;
+    const bool has_ang = has_len && p->angle_bins > 0 && W_axis1 != nullptr;
+    if (p->dist_bins > 0 && !W_dist) return fail(CFH_EINVAL, "dist_bins > 0 but W_dist is NULL");
+    if (has_len && !psi) return fail(CFH_EINVAL, "psi must not be NULL when dist_bins > 0");
+    if (has_ang && (!W_axis2 || !W_axis3 || !frames))
+        return fail(CFH_EINVAL, "W_axis1..3 and frames must be given together");
+    int wl = 0, wa = 0;
+    if ((rc = window_widths(p, &wl, &wa))) return rc;
+    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES))) return rc;
+    cfh::KernelArgs A;
+    fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
+    A.W[0] = W_dist; A.W[1] = W_axis1; A.W[2] = W_axis2; A.W[3] = W_axis3;
+    A.frames = frames; A.out_z = z; A.out_psi = psi; A.out_d2min = d2min_out;
+    const int waves = launch_waves(N, p->num_heads);
+    const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+    hipStream_t st = (hipStream_t)stream;
+    const char* what = "framed_pe_forward";
+    if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_fwd_kernel, true, true);
+    else if (has_len) CFH_DISPATCH_PE(cfh::framed_pe_fwd_kernel, true, false);
+    else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, false, false>, A, waves, st, what);
+    return rc;
+}
+
+int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,
+                           const float* rvlen, const int64_t* batch, const int64_t* edges,
+                           const int64_t* e_start, const int32_t* order, const float* W_dist,
+                           const float* W_axis1, const float* W_axis2, const float* W_axis3,
+                           const float* frames, const float* z, const float* gz, const float* gpsi,
+                           int64_t N, int64_t E, int64_t B, float* ga, float* gW_dist, float* gW_axis1,
+                           float* gW_axis2, float* gW_axis3, void* workspace, size_t workspace_bytes,
+                           void* stream) {
+    int rc = check_params(p);
+    if (rc) return rc;
+    if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
+    const bool has_len = p->dist_bins > 0 && W_dist != nullptr;
+    const bool has_ang = has_len && p->angle_bins > 0 && W_axis1 != nullptr;
+    hipStream_t st = (hipStream_t)stream;
+    const size_t wbytes = (size_t)p->num_heads * cfh::DH * cfh::NBINS * sizeof(float);
+    if (N == 0) {     // no atoms: the weight gradients are zero
+        float* outs[4] = {gW_dist, gW_axis1, gW_axis2, gW_axis3};
+        for (float* o : outs)
+            if (o && hipMemsetAsync(o, 0, wbytes, st) != hipSuccess) return fail(CFH_ELAUNCH, "memset of an empty gradient failed");
+        return CFH_OK;
+    }
+    if (!z || !gz || !ga) return fail(CFH_EINVAL, "z, gz and ga must not be NULL");
+    if (has_len && !gpsi) return fail(CFH_EINVAL, "gpsi must not be NULL when dist_bins > 0");
+    if (has_ang && (!W_axis2 || !W_axis3 || !frames))
+        return fail(CFH_EINVAL, "W_axis1..3 and frames must be given together");
+    int wl = 0, wa = 0;
+    if ((rc = window_widths(p, &wl, &wa))) return rc;
+    const int waves = launch_waves(N, p->num_heads);
+    const size_t need = COUNTER_BYTES + (size_t)waves * 4 * cfh::DH * cfh::NBINS * sizeof(float);
+    if ((rc = check_workspace(workspace, workspace_bytes, need))) return rc;
+    cfh::KernelArgs A;
+    fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
+    A.W[0] = W_dist; A.W[1] = W_axis1; A.W[2] = W_axis2; A.W[3] = W_axis3;
+    A.frames = frames; A.z = z; A.gz = gz; A.gpsi = gpsi; A.out_ga = ga;
+    A.gw_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + COUNTER_BYTES);
+    const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+    const char* what = "framed_pe_backward";
+    if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, true);
+    else if (has_len) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, false);
+    else rc = launch_persistent(cfh::framed_pe_bwd_kernel<9, 33, false, false, false>, A, waves, st, what);
+    if (rc) return rc;
+    if (has_len) {
+        const int nenc = has_ang ? 4 : 1;
+        const int total = nenc * p->num_heads * cfh::DH * cfh::NBINS;
+        hipLaunchKernelGGL(cfh::gw_reduce_kernel, dim3((total + 255) / 256), dim3(256), 0, st, A.gw_partial,
+                           waves, p->num_heads, nenc, gW_dist, gW_axis1, gW_axis2, gW_axis3);
+        rc = finish_launch("gw_reduce");
+    }
+    return rc;
+}
+
+}  // extern "C"

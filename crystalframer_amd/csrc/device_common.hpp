@@ -1,0 +1,235 @@
+// Device-side building blocks shared by the lattice-sum kernels (gfx950, wave64).
+//
+// Execution model used by every kernel in this directory:
+//   * a workgroup is ONE 64-lane wavefront that owns one attention head h (= blockIdx.x % H, so
+//     all wavefronts of a head land on the same XCD and share its L2 copy of that head's weights);
+//   * wavefronts are persistent: each pulls (atom i) work items for its head from a per-head
+//     counter in global memory until the counter passes N -- an exit every wavefront reaches;
+//   * for an item (i,h) the integer translations n of the box [-R1,R1]x[-R2,R2]x[-R3,R3] are
+//     expanded once into an LDS table of Cartesian shifts n.L (TCAP entries at a time), lanes then
+//     run over table entries, so one pair (i,j) is processed 64 translations per step.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace cfh {
+
+constexpr int WAVE = 64;
+constexpr int TCAP = 512;      // translations staged in LDS per pass (8 KB of float4)
+constexpr int NBINS = 64;      // distance bins K and angle bins A the kernels are compiled for
+constexpr int DH = 16;         // head dimension the kernels are compiled for
+constexpr int HS = 72;         // padded row stride (floats) of the 4 x 64 histograms in LDS
+constexpr int RMAX = 32;       // safety clamp of a box half-width
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float SQRT_LOG2E = 1.2011224087864498f;
+constexpr float LN2 = 0.6931471805599453f;
+
+// ---- hardware transcendental units (quarter rate, ~1 ulp) -------------------------------------
+__device__ __forceinline__ float hw_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float hw_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float hw_rsq(float x) { return __builtin_amdgcn_rsqf(x); }
+__device__ __forceinline__ float hw_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float hw_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
+__device__ __forceinline__ float clampf(float x, float lo, float hi) { return fminf(fmaxf(x, lo), hi); }
+
+// ---- wave64 reductions ------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+// arg-min over (value, index): smallest value, then smallest index
+__device__ __forceinline__ void wave_argmin(float& v, int& idx) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        float ov = __shfl_xor(v, o, WAVE);
+        int oi = __shfl_xor(idx, o, WAVE);
+        if (ov < v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+    }
+}
+// arg-max over (value, index): largest value, then smallest index
+__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        float ov = __shfl_xor(v, o, WAVE);
+        int oi = __shfl_xor(idx, o, WAVE);
+        if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+    }
+}
+__device__ __forceinline__ int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ float uniform_f(float v) {
+    return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
+}
+__device__ __forceinline__ int lane_prefix(uint64_t mask) {   // set bits below this lane
+    return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+}
+
+// ---- per-(atom, head) geometry ----------------------------------------------------------------
+struct Box {
+    int R1, R2, R3;   // half-widths
+    int s2, s3;       // 2*R2+1, 2*R3+1
+    int T;            // number of translations
+};
+
+// Half-widths of the translation box.  Same operation order as the reference kernels
+// (models/kernels/real_enc_frame_proj_fwd_length.cu:59-86): float32 up to (cutoff+0.01f)*rvl,
+// double division by 2.0*CUDART_PI_F, ceil; no fused multiply-add.
+#pragma clang fp contract(off)
+__device__ __forceinline__ int half_width(float c1, float rvl, int minimum_range) {
+    const float prod = c1 * rvl;
+    const double v = (double)prod / (2.0 * (double)3.14159274101257324f);
+    int r = (v > 0.0 && v < (double)RMAX) ? (int)ceil(v) : (v >= (double)RMAX ? RMAX : 0);
+    if (minimum_range > 0) r = max(r, minimum_range);
+    return min(r, RMAX);
+}
+__device__ __forceinline__ Box translation_box(float a, float rvl1, float rvl2, float rvl3,
+                                               float cutoff_radius, int lattice_range,
+                                               int minimum_range) {
+    Box b;
+    b.R1 = b.R2 = b.R3 = lattice_range;
+    if (cutoff_radius != 0.0f) {
+        float cut = cutoff_radius;
+        if (cut < 0.0f) cut = __fsqrt_rn(__fdiv_rn(-0.5f, a)) * (-cut);
+        const float c1 = cut + 0.01f;
+        b.R1 = half_width(c1, rvl1, minimum_range);
+        b.R2 = half_width(c1, rvl2, minimum_range);
+        b.R3 = half_width(c1, rvl3, minimum_range);
+    }
+    b.s2 = 2 * b.R2 + 1; b.s3 = 2 * b.R3 + 1;
+    b.T = (2 * b.R1 + 1) * b.s2 * b.s3;
+    return b;
+}
+#pragma clang fp contract(fast)
+
+struct Lattice { float t[9]; };   // rows = lattice vectors
+
+// Fill tab[0..cnt) with the Cartesian shifts of translations t0..t0+cnt in the reference's loop
+// order (n1 outermost, n3 innermost, ascending).
+__device__ __forceinline__ void build_shift_table(float4* tab, int t0, int cnt, const Box& bx,
+                                                  const Lattice& L, int lane) {
+    for (int u = lane; u < cnt; u += WAVE) {
+        const int t = t0 + u;
+        const int i3 = t % bx.s3;
+        const int q = t / bx.s3;
+        const int i2 = q % bx.s2;
+        const int i1 = q / bx.s2;
+        const float n1 = (float)(i1 - bx.R1), n2 = (float)(i2 - bx.R2), n3 = (float)(i3 - bx.R3);
+        float4 v;
+        v.x = fmaf(L.t[6], n3, fmaf(L.t[3], n2, L.t[0] * n1));
+        v.y = fmaf(L.t[7], n3, fmaf(L.t[4], n2, L.t[1] * n1));
+        v.z = fmaf(L.t[8], n3, fmaf(L.t[5], n2, L.t[2] * n1));
+        v.w = 0.0f;
+        tab[u] = v;
+    }
+}
+
+// ---- truncated Gaussian windows by a two-sided multiplicative recurrence ------------------------
+// For W equally spaced bins with scaled offsets beta_m = beta_c + (m-C)*sig (C = W/2) the values
+// g_m = 2^(-beta_m^2) satisfy g_{m+1} = g_m r_m, r_{m+1} = r_m cc with cc = 2^(-2 sig^2), so a
+// window costs three hardware exponentials instead of W.  The chain starts at the centre bin and
+// runs outwards both ways (at most W/2 multiplications deep).  Exponents of the ratios are clamped
+// so that an underflowed centre (far outside the basis range) gives zeros instead of 0*inf.
+struct WindowSeed { float gc, rr, rl; };
+__device__ __forceinline__ WindowSeed window_seed(float beta_c, float sig, float weight) {
+    WindowSeed s;
+    const float tb = 2.0f * beta_c * sig;
+    const float s2 = sig * sig;
+    s.gc = hw_exp2(-beta_c * beta_c) * weight;
+    s.rr = hw_exp2(clampf(-(tb + s2), -100.0f, 100.0f));
+    s.rl = hw_exp2(clampf(tb - s2, -100.0f, 100.0f));
+    return s;
+}
+
+template <int W>
+__device__ __forceinline__ void window_scatter(float* base, const WindowSeed& s, float cc) {
+    constexpr int C = W / 2;
+    atomicAdd(base + C, s.gc);
+    float g = s.gc, r = s.rr;
+#pragma unroll
+    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; atomicAdd(base + m, g); }
+    g = s.gc; r = s.rl;
+#pragma unroll
+    for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; atomicAdd(base + m, g); }
+}
+
+// Scatter weight*g_m into hbase[m] and return sum_m weight*g_m*gbase[m].
+template <int W>
+__device__ __forceinline__ float window_scatter_gather(float* hbase, const float* gbase,
+                                                       const WindowSeed& s, float cc) {
+    constexpr int C = W / 2;
+    float acc = s.gc * gbase[C];
+    atomicAdd(hbase + C, s.gc);
+    float g = s.gc, r = s.rr;
+#pragma unroll
+    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); atomicAdd(hbase + m, g); }
+    g = s.gc; r = s.rl;
+#pragma unroll
+    for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); atomicAdd(hbase + m, g); }
+    return acc;
+}
+
+// Constants of the two bases, prepared on the host.
+struct BasisConsts {
+    // distance basis
+    float inv_interval;    // K/dist_max
+    float start_off;       // 4*wscale + 1  : start = trunc(d*inv_interval - start_off)
+    float len_step;        // sqrt(log2 e)/(wscale*sqrt 2) : scaled offset between neighbouring bins
+    float len_cc;          // 2^(-2 len_step^2)
+    // angle basis
+    float ang_inv_interval;  // (A-1)/2 (cos_abs: A-1)
+    float ang_end_off;       // 1 + 4*sigma_a
+    float ang_interval;      // 2/(A-1) (cos_abs: 1/(A-1))
+    float ang_sigma_inv;     // sqrt(log2 e)/(sigma_a*sqrt 2)
+    float ang_step;          // ang_interval*ang_sigma_inv
+    float ang_cc;            // 2^(-2 ang_step^2)
+    float ang_mu0;           // centre of bin 0: -1 (cos_abs: 0)
+};
+
+// Launch-wide arguments (by value in the kernarg segment).
+struct KernelArgs {
+    // geometry
+    const float* a_ih; const float* rpos; const float* tvecs; const float* rvlen;
+    const int64_t* batch; const int64_t* edges; const int64_t* e_start; const int32_t* order;
+    // attention operands for the frame search
+    const float* q; const float* k; const float* frame1;
+    // value-PE operands
+    const float* W[4]; const float* frames; const float* z; const float* gz; const float* gpsi;
+    // outputs
+    float* out_z; float* out_psi; float* out_d2min; float* out_frame; float* out_ga;
+    float* gw_partial;            // (waves, 4, DH, NBINS) per-wave weight-gradient partials
+    int32_t* counters;            // (H) work-queue heads
+    int32_t N, E, H;
+    float cutoff_radius; int32_t lattice_range, minimum_range;
+    float prune_log2;             // <= 0: keep every translation
+    float dist_coef, angle_coef, gz_coef, gw_dist_coef;
+    float noise; uint32_t seed_lo, seed_hi;
+    BasisConsts bc;
+};
+
+// Next work item of this wavefront's head: one lane takes it from the counter, all lanes get it.
+// The electing lane id passes through an empty asm so that the compiler cannot relate this branch
+// to the `if (lane == 0)` stores at the tail of the persistent loop: when it can, it threads the two
+// branches together across the back edge, lanes 1..63 re-enter the loop apart from lane 0 (reading
+// item 0 from the readfirstlane below), and the wavefront never leaves the loop.
+__device__ __forceinline__ int next_item(int32_t* counter, int lane) {
+    int elect = lane;
+    asm volatile("" : "+v"(elect));
+    int it = 0;
+    if (elect == 0) it = atomicAdd(counter, 1);
+    return uniform_i(it);
+}
+
+// Counter-based uniform in [0,1) for the optional tie-breaking noise of the frame search.
+__device__ __forceinline__ float hash_uniform(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    uint32_t x = a * 0x9E3779B1u ^ (b + 0x7F4A7C15u) * 0x85EBCA77u;
+    x ^= x >> 15; x *= 0xC2B2AE3Du; x ^= c * 0x27D4EB2Fu; x ^= x >> 13; x *= 0x165667B1u;
+    x ^= d; x ^= x >> 16; x *= 0x9E3779B1u; x ^= x >> 15;
+    return (float)(x >> 8) * (1.0f / 16777216.0f);
+}
+
+}  // namespace cfh

@@ -1,0 +1,265 @@
+"""Operator boundary: ``torch.autograd.Function`` classes with the names and positional signatures
+of the reference's ``models/cuda_funcs`` package, backed by the gfx950 HIP library.
+
+An attention layer written against the reference API
+(models/indexed_lattice_multi_head_attention_cuda.py:455-462,543-546) can import these instead and
+run unchanged on one MI355X.  The kernels' compile-time constants, which the reference sets
+globally through ``compile_kernels`` (models/cuda_funcs/kernel_manager.py:116-167), live in
+``KernelManager`` here as well.
+"""
+from __future__ import annotations
+
+import ctypes
+import weakref
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+CUPY_AVAILABLE = True   # name kept from the reference: "the native path is usable"
+
+
+class KernelManager:
+    """Global kernel constants (reference: models/cuda_funcs/kernel_manager.py:25-62,124-149)."""
+    MAX_SYSTEM_SIZE: int = 320          # kept for API parity; these kernels have no size limit
+    PE_THREAD_NUM: int = 64
+    LATTICE_RANGE: int = 2
+    MINIMUM_RANGE: int = 2
+    SYMM_BREAK_NOISE: float = 1e-5
+    NOISE_SEED: Optional[int] = None    # None: a fresh seed per call, as the reference draws one
+    # options of this implementation (no reference counterpart)
+    WINDOW_MODE: int = _lib.CFH_WINDOW_REFERENCE
+    PRUNE_LOG2: float = 32.0            # skip translations lighter than 2^-32 of their pair's heaviest
+    GRAD_COEF_QUIRK: bool = False
+    _compiled_for = None
+
+
+def compile_kernels(lattice_range: int, head_num: int, key_head_dim: int, value_pe_dim: int,
+                    dim_angle_enc: int, value_head_dim: int, set_minimum_range: bool, cos_abs: int,
+                    value_pe_dist_wscale: float, value_pe_angle_wscale: float,
+                    value_pe_dist_coef: float, value_pe_angle_coef: float, symm_break_noise: float):
+    """Same signature as the reference's run-time compiler.  The HIP kernels are built ahead of
+    time, so this records the global constants and checks that the requested combination is among
+    the compiled instantiations."""
+    if key_head_dim != 16 or value_head_dim != 16:
+        raise NotImplementedError(f"head dims ({key_head_dim},{value_head_dim}): only 16 is compiled")
+    if value_pe_dim not in (0, 64) or dim_angle_enc not in (0, 64):
+        raise NotImplementedError(f"value_pe_dist_real={value_pe_dim}, value_pe_angle_real={dim_angle_enc}: "
+                                  "only 0 or 64 bins are compiled")
+    if value_pe_dim > 0 and float(value_pe_dist_wscale) != 1.0:
+        raise NotImplementedError("value_pe_dist_wscale: only 1.0 is compiled")
+    if dim_angle_enc > 0 and float(value_pe_angle_wscale) != 4.0:
+        raise NotImplementedError("value_pe_angle_wscale: only 4.0 is compiled")
+    KernelManager.LATTICE_RANGE = int(lattice_range)
+    KernelManager.MINIMUM_RANGE = int(lattice_range) if set_minimum_range else 0
+    KernelManager.SYMM_BREAK_NOISE = float(symm_break_noise)
+    KernelManager._compiled_for = dict(head_num=head_num, cos_abs=cos_abs)
+    _lib.load()
+
+
+# --------------------------------------------------------------------------------------------------
+def _params(H: int, Dh: int, K: int, A: int, cos_abs: int, dist_max: float, wscale: float,
+            angle_wscale: float, dist_coef: float, angle_coef: float, cutoff_radius) -> _lib.CfhParams:
+    p = _lib.CfhParams()
+    p.struct_size = ctypes.sizeof(_lib.CfhParams)
+    p.num_heads, p.head_dim, p.dist_bins, p.angle_bins = H, Dh, K, A
+    p.cos_abs = int(cos_abs)
+    p.lattice_range = KernelManager.LATTICE_RANGE
+    p.minimum_range = KernelManager.MINIMUM_RANGE
+    p.window_mode = KernelManager.WINDOW_MODE
+    p.dist_max, p.dist_wscale, p.angle_wscale = float(dist_max), float(wscale), float(angle_wscale)
+    p.dist_coef, p.angle_coef = float(dist_coef), float(angle_coef)
+    p.cutoff_radius = 0.0 if cutoff_radius is None else float(cutoff_radius)
+    p.prune_log2 = float(KernelManager.PRUNE_LOG2)
+    p.symm_break_noise = float(KernelManager.SYMM_BREAK_NOISE)
+    if KernelManager.NOISE_SEED is None:
+        p.noise_seed = int(torch.randint(0, 2 ** 62, (1,)).item()) if p.symm_break_noise > 0 else 0
+    else:
+        p.noise_seed = int(KernelManager.NOISE_SEED)
+    p.grad_coef_quirk = int(bool(KernelManager.GRAD_COEF_QUIRK))
+    return p
+
+
+_edge_cache = {"ref": None, "version": None, "N": None, "val": None}
+
+
+def edge_schedule(edge_ij_e: torch.Tensor, N: int):
+    """(e_start (N+1) int64, order (N) int32) for an edge list whose edges are grouped by query atom.
+
+    e_start is built as the reference's backward does (models/cuda_funcs/real_space_framed_proj.py:
+    139-141); ``order`` lists atoms by descending neighbour count for the kernels' work queue.
+    The result is cached for the last edge tensor seen (every layer of a forward pass shares it).
+    """
+    c = _edge_cache
+    if c["ref"] is not None and c["ref"]() is edge_ij_e and c["version"] == edge_ij_e._version and c["N"] == N:
+        return c["val"]
+    cnt = torch.zeros(N + 1, dtype=torch.long, device=edge_ij_e.device)
+    cnt.scatter_add_(0, edge_ij_e[0] + 1, torch.ones_like(edge_ij_e[0]))
+    e_start = cnt.cumsum(0)
+    order = torch.argsort(e_start[1:] - e_start[:-1], descending=True, stable=True).to(torch.int32)
+    val = (e_start.contiguous(), order.contiguous())
+    c.update(ref=weakref.ref(edge_ij_e), version=edge_ij_e._version, N=N, val=val)
+    return val
+
+
+def _f32c(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    if t is None:
+        return None
+    return t.detach().to(torch.float32).contiguous()
+
+
+def _proj_weight(W: Optional[torch.Tensor], H: int, what: str) -> Optional[torch.Tensor]:
+    """(1,H,Dh,bins) or (H,Dh,bins) -> contiguous (H,Dh,bins); per-edge / per-atom weights unsupported."""
+    if W is None:
+        return None
+    if W.dim() not in (3, 4):
+        raise AssertionError(f"{what} must have 3 or 4 dimensions")
+    if W.dim() == 4:
+        if W.shape[0] != 1:
+            raise NotImplementedError(f"{what}: only one shared projection (leading dim 1) is supported")
+        W = W[0]
+    if W.shape[0] != H:
+        raise ValueError(f"{what}: expected {H} heads, got {W.shape[0]}")
+    return _f32c(W)
+
+
+def _frame_call(second: bool, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, frame1, rvlen_n,
+                cutoff_radius):
+    _lib.require_gpu(q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e)
+    lib = _lib.load()
+    N, H = a_ik.shape
+    E = edge_ij_e.shape[1]
+    Dh = q.shape[-1]
+    dev = a_ik.device
+    q, k, a = _f32c(q), _f32c(k), _f32c(a_ik)
+    rpos, tv = _f32c(rpos_ij_e), _f32c(tvecs_n)
+    rv = _f32c(rvlen_n)
+    batch, edges = batch_i.contiguous(), edge_ij_e.contiguous()
+    e_start, order = edge_schedule(edge_ij_e, N)
+    out = torch.zeros((N, H, 3), dtype=torch.float32, device=dev)
+    p = _params(H, Dh, 0, 0, 0, 1.0, 1.0, 1.0, 1.0, 1.0, cutoff_radius if rv is not None else None)
+    with torch.cuda.device(dev):
+        need = lib.cfh_workspace_bytes(ctypes.byref(p), N, E)
+        ws = _lib.workspace(dev, need)
+        st = _lib.current_stream_ptr(dev)
+        if not second:
+            rc = lib.cfh_frame_axis1(ctypes.byref(p), _lib.ptr(q), _lib.ptr(k), _lib.ptr(a), _lib.ptr(rpos),
+                                     _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges),
+                                     _lib.ptr(e_start), _lib.ptr(order), N, E, tv.shape[0], _lib.ptr(out),
+                                     _lib.ptr(ws), ws.numel(), st)
+        else:
+            f1 = _f32c(frame1)
+            rc = lib.cfh_frame_axis2(ctypes.byref(p), _lib.ptr(q), _lib.ptr(k), _lib.ptr(a), _lib.ptr(rpos),
+                                     _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges),
+                                     _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(f1), N, E, tv.shape[0],
+                                     _lib.ptr(out), _lib.ptr(ws), ws.numel(), st)
+    _lib.check(rc, "cfh_frame_axis2" if second else "cfh_frame_axis1")
+    return out
+
+
+class ComputeFrame1MaximumMethodCUDA(torch.autograd.Function):
+    """First frame axis (N,H,3).  Signature of models/cuda_funcs/calc_maximum_frame.py:24-91;
+    ``v``, ``dist2_min_e``, ``K``, ``dist_max`` and ``wscale`` are unused there as well."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max,
+                wscale, rvlen_n=None, cutoff_radius=None):
+        return _frame_call(False, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, None, rvlen_n,
+                           cutoff_radius)
+
+    @staticmethod
+    def backward(ctx, gframevec):
+        return (None,) * 14
+
+
+class ComputeFrame2MaximumMethodCUDA(torch.autograd.Function):
+    """Second frame axis before orthogonalisation (N,H,3).  Signature of
+    models/cuda_funcs/calc_maximum_frame.py:95-170."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max,
+                wscale, frame1, rvlen_n=None, cutoff_radius=None):
+        return _frame_call(True, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, frame1, rvlen_n,
+                           cutoff_radius)
+
+    @staticmethod
+    def backward(ctx, gframevec):
+        return (None,) * 15
+
+
+class RealEncodingWithFramedProjFuncCUDA(torch.autograd.Function):
+    """z (E,H) and the framed value position encoding (E,H,Dh).  Signature and return convention of
+    models/cuda_funcs/real_space_framed_proj.py:19-221: returns ``(z,)`` when ``K <= 0``, else
+    ``(z, v)``; gradients flow to ``a_ik`` and the four projection weights only."""
+
+    @staticmethod
+    def forward(ctx, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale,
+                W_k, W_k1, W_k2, W_k3, frame_vec_1, frame_vec_2, frame_vec_3, dim_angle_enc,
+                value_pe_angle_scale, cos_abs, length_rbf_mul, angle_rbf_mul, rvlen_n=None,
+                cutoff_radius=None):
+        _lib.require_gpu(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e)
+        lib = _lib.load()
+        N, H = a_ik.shape
+        E = edge_ij_e.shape[1]
+        dev = a_ik.device
+        K = int(K) if W_k is not None else 0
+        Wd = _proj_weight(W_k, H, "W_k") if K > 0 else None
+        use_angle = K > 0 and W_k1 is not None and int(dim_angle_enc) > 0
+        A = int(dim_angle_enc) if use_angle else 0
+        Wa = [_proj_weight(w, H, "W_k%d" % (n + 1)) for n, w in enumerate((W_k1, W_k2, W_k3))] if use_angle \
+            else [None, None, None]
+        Dh = Wd.shape[-2] if Wd is not None else 16
+        a = _f32c(a_ik)
+        rpos, tv, rv = _f32c(rpos_ij_e), _f32c(tvecs_n), _f32c(rvlen_n)
+        batch, edges = batch_i.contiguous(), edge_ij_e.contiguous()
+        e_start, order = edge_schedule(edge_ij_e, N)
+        frames = torch.stack([_f32c(frame_vec_1), _f32c(frame_vec_2), _f32c(frame_vec_3)], 0).contiguous() \
+            if use_angle else None
+        z = torch.empty((E, H), dtype=torch.float32, device=dev)
+        v = torch.empty((E, H, Dh), dtype=torch.float32, device=dev) if K > 0 else None
+        p = _params(H, Dh, K, A, cos_abs, float(dist_max), wscale, value_pe_angle_scale,
+                    length_rbf_mul, angle_rbf_mul, cutoff_radius if rv is not None else None)
+        with torch.cuda.device(dev):
+            ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
+            rc = lib.cfh_framed_pe_forward(
+                ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch),
+                _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd), _lib.ptr(Wa[0]),
+                _lib.ptr(Wa[1]), _lib.ptr(Wa[2]), _lib.ptr(frames), N, E, tv.shape[0], _lib.ptr(z),
+                _lib.ptr(v), None, _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_framed_pe_forward")
+        ctx.save_for_backward(a, rpos, tv, rv, batch, edges, e_start, order, Wd, Wa[0], Wa[1], Wa[2], frames, z)
+        ctx.params = p
+        ctx.w_shapes = [None if w is None else w.shape for w in (W_k, W_k1, W_k2, W_k3)]
+        ctx.n_inputs = 23
+        if K <= 0:
+            return z,
+        return z, v
+
+    @staticmethod
+    def backward(ctx, gz_ek, gv_ekd=None):
+        a, rpos, tv, rv, batch, edges, e_start, order, Wd, W1, W2, W3, frames, z = ctx.saved_tensors
+        lib = _lib.load()
+        p = ctx.params
+        N, H = a.shape
+        E = edges.shape[1]
+        dev = a.device
+        gz = _f32c(gz_ek) if gz_ek is not None else torch.zeros_like(z)
+        gv = None
+        if Wd is not None:
+            gv = _f32c(gv_ekd) if gv_ekd is not None else torch.zeros((E, H, Wd.shape[-2]), dtype=torch.float32, device=dev)
+        ga = torch.empty((N, H), dtype=torch.float32, device=dev)
+        gWd = torch.empty_like(Wd) if Wd is not None else None
+        gWa = [torch.empty_like(w) if w is not None else None for w in (W1, W2, W3)]
+        with torch.cuda.device(dev):
+            ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
+            rc = lib.cfh_framed_pe_backward(
+                ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch),
+                _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd), _lib.ptr(W1), _lib.ptr(W2),
+                _lib.ptr(W3), _lib.ptr(frames), _lib.ptr(z), _lib.ptr(gz), _lib.ptr(gv), N, E, tv.shape[0],
+                _lib.ptr(ga), _lib.ptr(gWd), _lib.ptr(gWa[0]), _lib.ptr(gWa[1]), _lib.ptr(gWa[2]),
+                _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_framed_pe_backward")
+        gws = [g if g is None else g.reshape(s) for g, s in zip([gWd] + gWa, ctx.w_shapes)]
+        return (ga, None, None, None, None, None, None, None, None, gws[0], gws[1], gws[2], gws[3],
+                None, None, None, None, None, None, None, None, None, None)

@@ -1,0 +1,154 @@
+/*
+ * crystalframer_hip.h -- C ABI of the MI355X (gfx950) kernels for CrystalFramer's periodic
+ * infinitely-connected attention: real-space lattice sums, Gaussian distance value encoding,
+ * dynamic max-frame selection and frame-projected angle value encoding, forward and backward.
+ *
+ * Every entry point takes plain device pointers and sizes, enqueues its kernels on the HIP stream
+ * it is given (NULL = the default stream) and returns without synchronising.  The return value is
+ * 0 on success or a negative CFH_E* code; cfh_last_error() then describes the failure.  The library
+ * allocates nothing: scratch memory comes in through the `workspace` argument, whose required
+ * size cfh_workspace_bytes() reports.  All floating-point tensors are contiguous float32, all
+ * index tensors contiguous int64, exactly as the reference passes them to its kernels.
+ *
+ * Tensor naming (N atoms, E ordered atom pairs, B crystals, H heads, Dh head dim, K distance bins,
+ * A angle bins):
+ *   a_ih    (N,H)      Gaussian coefficient, a < 0            rpos   (E,3)   pos[j]-pos[i]
+ *   tvecs   (B,3,3)    lattice vectors as rows                 rvlen  (B,3)   |reciprocal rows|
+ *   batch   (N)        crystal of each atom                    edges  (2,E)   (i,j); edges of one
+ *   e_start (N+1)      first edge of each atom                                 atom are contiguous
+ *   order   (N) int32  optional visiting order of atoms for the work queue (NULL = natural)
+ */
+#ifndef CRYSTALFRAMER_HIP_H
+#define CRYSTALFRAMER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CFH_ABI_VERSION 1
+
+enum {
+    CFH_OK = 0,
+    CFH_EINVAL = -1,       /* bad argument (null pointer, unsupported constant, size mismatch) */
+    CFH_EWORKSPACE = -2,   /* workspace missing or too small                                    */
+    CFH_ELAUNCH = -3,      /* HIP reported an error when launching                              */
+    CFH_EDEVICE = -4       /* no usable gfx950 device                                           */
+};
+
+/* Which truncation of the Gaussian bases the kernels use. */
+enum {
+    CFH_WINDOW_REFERENCE = 0,  /* +-4 sigma: ceil(8*wscale+1) bins, the reference kernels' rule
+                                  (models/cuda_funcs/kernel_manager.py:146-147)                 */
+    CFH_WINDOW_WIDE = 1        /* two more bins on each side; dropped tail < 4e-6 of the peak   */
+};
+
+/*
+ * Scalar parameters.  They are the values the reference bakes into its kernels by text
+ * substitution before NVRTC (models/cuda_funcs/kernel_manager.py:116-159) plus the scalar
+ * arguments of its launches (models/cuda_funcs/real_space_framed_proj.py:66-104).
+ */
+typedef struct cfh_params {
+    int32_t struct_size;     /* = sizeof(cfh_params), ABI check                                   */
+    int32_t num_heads;       /* H      (HEAD_NUM)                                                 */
+    int32_t head_dim;        /* Dh     (V_HEAD_DIM = K_HEAD_DIM); 16 is compiled                  */
+    int32_t dist_bins;       /* K      (VPE_DIM); 0 or 64                                         */
+    int32_t angle_bins;      /* A      (ANGLE_ENC_DIM); 0 or 64                                   */
+    int32_t cos_abs;         /* COS_ABS 0/1                                                       */
+    int32_t lattice_range;   /* LATTICE_RANGE: box half-width when cutoff_radius == 0             */
+    int32_t minimum_range;   /* MINIMUM_RANGE: lower bound of the adaptive half-width (0 = none)  */
+    int32_t window_mode;     /* CFH_WINDOW_*                                                      */
+    float dist_max;          /* angstrom; bin centres (k+1)*dist_max/K                            */
+    float dist_wscale;       /* sigma_dist = dist_wscale*dist_max/K                               */
+    float angle_wscale;      /* sigma_angle = (cos_abs?1:2)*angle_wscale/(A-1)                    */
+    float dist_coef;         /* length_rbf_mul                                                    */
+    float angle_coef;        /* angle_rbf_mul                                                     */
+    float cutoff_radius;     /* <0: -cutoff_radius sigmas of each head's Gaussian; 0: fixed box;
+                                >0: absolute radius in angstrom                                   */
+    float prune_log2;        /* translations whose weight is below 2^-prune_log2 of the largest
+                                one of their pair are skipped; <= 0 evaluates every translation   */
+    float symm_break_noise;  /* amplitude of the tie-breaking noise of the frame search (0 = the
+                                deterministic first-wins rule)                                    */
+    uint64_t noise_seed;     /* seed of that noise                                                */
+    int32_t grad_coef_quirk; /* 1: backward scales like the reference (d/dz part by dist_coef,
+                                dW_dist unscaled; real_space_framed_proj.py:183-184); 0: exact    */
+    int32_t reserved;
+} cfh_params;
+
+/* Version of this ABI; a mismatch with CFH_ABI_VERSION means header and library differ. */
+int cfh_abi_version(void);
+
+/* Text of the last error on the calling thread ("" if none). */
+const char* cfh_last_error(void);
+
+/* Bytes of device scratch the four entry points below need for (N atoms, E pairs). */
+size_t cfh_workspace_bytes(const cfh_params* p, int64_t N, int64_t E);
+
+/*
+ * First frame axis, f1 (N,H,3): unit vector towards the nearest periodic image (d^2 > 1e-5) of the
+ * neighbour j maximising  q_i.k_j + a_ih*d2min(i,j).  `q` (N,H,Dh) must already be divided by
+ * sqrt(Dh); `k` (N,H,Dh).
+ * Replaces ComputeFrame1MaximumMethodCUDA.forward: kernel compute_maximum_frame_each_edge, the
+ * gathered q.k product and torch_scatter.scatter_max
+ * (models/cuda_funcs/calc_maximum_frame.py:24-87, models/kernels/compute_maximum_frame_each_edge.cu).
+ */
+int cfh_frame_axis1(const cfh_params* p, const float* q, const float* k, const float* a_ih,
+                    const float* rpos, const float* tvecs, const float* rvlen,
+                    const int64_t* batch, const int64_t* edges, const int64_t* e_start,
+                    const int32_t* order, int64_t N, int64_t E, int64_t B,
+                    float* frame1, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Second frame axis before orthogonalisation, f2max (N,H,3): unit vector towards the image (over
+ * all neighbours j and translations n) maximising
+ *   q_i.k_j + a_ih*d^2 + log(max(1-|cos(image, f1)|, 1e-5)),   |cos| < 0.9999, d^2 > 1e-5.
+ * Replaces ComputeFrame2MaximumMethodCUDA.forward
+ * (models/cuda_funcs/calc_maximum_frame.py:95-166, models/kernels/compute_second_frame_each_edge.cu).
+ */
+int cfh_frame_axis2(const cfh_params* p, const float* q, const float* k, const float* a_ih,
+                    const float* rpos, const float* tvecs, const float* rvlen,
+                    const int64_t* batch, const int64_t* edges, const int64_t* e_start,
+                    const int32_t* order, const float* frame1, int64_t N, int64_t E, int64_t B,
+                    float* frame2max, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * z (E,H) = log sum_n exp(a_ih*|rpos + n.L|^2) and, when K > 0, the value position encoding
+ * psi (E,H,Dh) = dist_coef * W_dist.s_dist + angle_coef * sum_axis W_axis.s_axis, where s are the
+ * softmax-over-translations averages of the truncated Gaussian bases of the distance and of the
+ * cosine to each frame axis.  W_dist (H,Dh,K); W_axis[3] each (H,Dh,A) or all NULL; frames
+ * (3,N,H,3) or NULL.  d2min_out (E,H) is optional.
+ * Replaces RealEncodingWithFramedProjFuncCUDA.forward: kernels real_enc_frame_proj_fwd_length and
+ * real_enc_frame_proj_fwd_angle and the sums between them
+ * (models/cuda_funcs/real_space_framed_proj.py:21-120).
+ */
+int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* rpos,
+                          const float* tvecs, const float* rvlen, const int64_t* batch,
+                          const int64_t* edges, const int64_t* e_start, const int32_t* order,
+                          const float* W_dist, const float* W_axis1, const float* W_axis2,
+                          const float* W_axis3, const float* frames, int64_t N, int64_t E,
+                          int64_t B, float* z, float* psi, float* d2min_out, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/*
+ * Gradients of the above for upstream gz (E,H) and gpsi (E,H,Dh): ga (N,H), gW_dist (H,Dh,K),
+ * gW_axis[3] (H,Dh,A).  The per-translation weights are recomputed from z, not stored.  The
+ * weight gradients are returned already summed over atoms.  No gradient flows to the frames
+ * (the reference returns None for them).
+ * Replaces RealEncodingWithFramedProjFuncCUDA.backward: kernels real_enc_frame_proj_bwd_length and
+ * real_enc_frame_proj_bwd_angle (models/cuda_funcs/real_space_framed_proj.py:123-221).
+ */
+int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* rpos,
+                           const float* tvecs, const float* rvlen, const int64_t* batch,
+                           const int64_t* edges, const int64_t* e_start, const int32_t* order,
+                           const float* W_dist, const float* W_axis1, const float* W_axis2,
+                           const float* W_axis3, const float* frames, const float* z,
+                           const float* gz, const float* gpsi, int64_t N, int64_t E, int64_t B,
+                           float* ga, float* gW_dist, float* gW_axis1, float* gW_axis2,
+                           float* gW_axis3, void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CRYSTALFRAMER_HIP_H */

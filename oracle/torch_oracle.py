@@ -1,0 +1,415 @@
+"""CPU oracle (TEST INFRASTRUCTURE ONLY) for CrystalFramer's periodic attention terms.
+
+This file restates, in plain PyTorch on the CPU, the arithmetic of the reference's
+native kernels and of its pure-PyTorch layer.  It is written at the level of the
+mathematics (explicit translation lists, ``logsumexp``, softmax weights, Gaussian
+bases); gradients come from autograd in float64, so they do not share any formula
+with the hand-derived backward kernels they are used to check.
+
+Only tests, the smoke check and the CPU-baseline leg of the benchmark may import it.
+The product path (``crystalframer_amd``) never does.
+
+Reference files restated here (paths relative to the reference repository root):
+
+* translation-set rule ............ models/kernels/real_enc_frame_proj_fwd_length.cu:59-86
+* z, distance value-PE ............ models/kernels/real_enc_frame_proj_fwd_length.cu:88-194
+                                    models/indexed_lattice_multi_head_attention.py:276-322,580-588
+* angle value-PE .................. models/kernels/real_enc_frame_proj_fwd_angle.cu:106-209
+* first frame axis ................ models/kernels/compute_maximum_frame_each_edge.cu:78-111
+                                    models/cuda_funcs/calc_maximum_frame.py:72-86
+* second frame axis ............... models/kernels/compute_second_frame_each_edge.cu:81-142
+                                    models/cuda_funcs/calc_maximum_frame.py:146-164
+* orthogonalisation ............... models/indexed_lattice_multi_head_attention_cuda.py:475-481
+* softmax-over-neighbours ......... models/kernels/fused_dpa_fwd.cu:46-124
+* per-crystal mean ................ models/kernels/irregular_mean_fwd.cu:13-90
+* geometry preparation ............ models/indexed_latticeformer_encoder.py:15-44,175-245
+
+Pinning status (what independent fact checks each function; see tests/test_oracle_*.py):
+
+* ``lattice_logsumexp`` (z): Poisson/Ewald identity against a reciprocal-space sum,
+  orthorhombic factorisation into 1-D sums, lattice-vector shift and unimodular
+  basis-change invariance, sharp-Gaussian limit.
+* distance / angle value-PE: brute-force Python loops on tiny cells, one-atom cubic
+  cell with cosines in {0, +-1}, sharp-Gaussian limit, SE(3) invariance.
+* frames: brute-force enumeration, orthonormality / right-handedness, SE(3) equivariance.
+* window indices, the 1e3 / 1e-5 sentinels, the adaptive-range rounding and tie-break
+  order are fixed by the kernel text alone ("parity unpinned" beyond reading): no
+  executable reference exists for them.
+* ``torch_scatter.scatter_max`` (segmented arg-max, un-vendored, version unpinned in the
+  reference's Dockerfile) is restated as a plain arg-max with lowest-index tie-break:
+  parity unpinned on ties.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+CUDART_PI_F = float(np.float32(3.141592654))  # the float constant the kernels promote to double
+
+
+# --------------------------------------------------------------------------------------
+# geometry preparation
+# --------------------------------------------------------------------------------------
+def edge_index(sizes: Sequence[int]) -> torch.Tensor:
+    """All ordered pairs (i, j) inside each crystal, i-major.
+
+    Follows models/indexed_latticeformer_encoder.py:15-32.
+    """
+    rows, cols = [], []
+    off = 0
+    for n in sizes:
+        idx = torch.arange(off, off + n, dtype=torch.long)
+        rows.append(idx.repeat_interleave(n))
+        cols.append(idx.repeat(n))
+        off += n
+    return torch.stack([torch.cat(rows), torch.cat(cols)])
+
+
+def geometry(pos: torch.Tensor, trans: torch.Tensor, sizes: Sequence[int]):
+    """edges, rpos_ij = pos[j]-pos[i], reciprocal rows 2*pi*(t_b x t_c)/V, cell volume.
+
+    Follows models/indexed_latticeformer_encoder.py:34-44,175-245.
+    """
+    edges = edge_index(sizes)
+    m = trans
+    vcell = (m[:, 0, 0] * m[:, 1, 1] * m[:, 2, 2] + m[:, 0, 1] * m[:, 1, 2] * m[:, 2, 0]
+             + m[:, 0, 2] * m[:, 1, 0] * m[:, 2, 1] - m[:, 0, 2] * m[:, 1, 1] * m[:, 2, 0]
+             - m[:, 0, 0] * m[:, 1, 2] * m[:, 2, 1] - m[:, 0, 1] * m[:, 1, 0] * m[:, 2, 2])
+    recip = torch.stack([
+        torch.linalg.cross(m[:, 1], m[:, 2], dim=1),
+        torch.linalg.cross(m[:, 2], m[:, 0], dim=1),
+        torch.linalg.cross(m[:, 0], m[:, 1], dim=1),
+    ], dim=1) * (2.0 * math.pi / vcell[:, None, None])
+    rpos = pos[edges[1]] - pos[edges[0]]
+    return edges, rpos, recip, vcell
+
+
+# --------------------------------------------------------------------------------------
+# translation-set rule
+# --------------------------------------------------------------------------------------
+def translation_ranges(a_ih: torch.Tensor, rvlen: Optional[torch.Tensor], batch: torch.Tensor,
+                       cutoff_radius: Optional[float], lattice_range: int = 2,
+                       minimum_range: int = 2) -> torch.Tensor:
+    """Per-(atom, head) half-widths R_d of the translation box, int64 (N, H, 3).
+
+    Follows models/kernels/real_enc_frame_proj_fwd_length.cu:59-86: float32 arithmetic up to
+    ``(cutoff + 0.01f) * rvl``, then a double division by ``2.0 * CUDART_PI_F`` and ``ceil``.
+    ``cutoff_radius`` None or 0 selects the fixed box of half-width ``lattice_range``.
+    """
+    N, H = a_ih.shape
+    if cutoff_radius is None or float(cutoff_radius) == 0.0 or rvlen is None:
+        return torch.full((N, H, 3), int(lattice_range), dtype=torch.long)
+    a32 = a_ih.detach().to(torch.float32).numpy()
+    c = np.float32(cutoff_radius)
+    if c < 0:
+        cut = np.sqrt(np.float32(-0.5) / a32) * np.float32(-c)          # (N,H) float32
+    else:
+        cut = np.full_like(a32, c)
+    rv = rvlen.detach().to(torch.float32).numpy()[batch.numpy()]        # (N,3) float32
+    prod = (cut + np.float32(0.01))[:, :, None] * rv[:, None, :]        # float32
+    R = np.ceil(prod.astype(np.float64) / (2.0 * CUDART_PI_F)).astype(np.int64)
+    if minimum_range > 0:
+        R = np.maximum(R, int(minimum_range))
+    return torch.from_numpy(R)
+
+
+def _grid(Rmax: Sequence[int], dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Integer translations of the box, n1 outermost ... n3 innermost (the kernels' loop order)."""
+    axes = [torch.arange(-int(r), int(r) + 1, dtype=torch.long) for r in Rmax]
+    g = torch.stack(torch.meshgrid(*axes, indexing="ij"), dim=-1).reshape(-1, 3)
+    return g, g.to(dtype)
+
+
+# --------------------------------------------------------------------------------------
+# windows of the truncated Gaussian bases
+# --------------------------------------------------------------------------------------
+def reference_windows(K: int, dist_wscale: float, A: int, angle_wscale: float) -> Tuple[int, int]:
+    """(LENGTH_RANGE, ANGLE_RANGE) exactly as models/cuda_funcs/kernel_manager.py:146-147."""
+    cut_sigma = 4
+    return (math.ceil(2 * dist_wscale * cut_sigma + 1), math.ceil(2 * angle_wscale * cut_sigma + 1))
+
+
+def _length_basis(d: torch.Tensor, K: int, dist_max: float, wscale: float, window: Optional[int]):
+    """Gaussian radial basis of a distance, (..., K).
+
+    centres (k+1)*dist_max/K, sigma = wscale*dist_max/K
+    (models/indexed_lattice_multi_head_attention.py:580-588 and
+    models/kernels/real_enc_frame_proj_fwd_length.cu:130-160).  ``window`` = number of bins the
+    kernel keeps (start index rule of :139-142); None = full basis.
+    """
+    interval = dist_max / K
+    sig = interval * wscale
+    k = torch.arange(K, dtype=d.dtype)
+    b = ((k + 1) * interval - d[..., None]) / (math.sqrt(2.0) * sig)
+    g = torch.exp(-b * b)
+    if window is not None and K - window > 8:
+        start = torch.trunc((d - 4 * sig) / interval - 1).clamp(0, K - window)
+        kk = k.expand(g.shape)
+        keep = (kk >= start[..., None]) & (kk < start[..., None] + window)
+        g = g * keep
+    return g
+
+
+def _angle_basis(c: torch.Tensor, valid: torch.Tensor, A: int, angle_sigma: float, cos_abs: int,
+                 window: Optional[int]):
+    """Gaussian basis of a cosine, (..., A).
+
+    models/kernels/real_enc_frame_proj_fwd_angle.cu:136-175.  ``valid`` is False for the self image
+    (d^2 <= 1e-5) whose sentinel cosine 1e3 makes every Gaussian underflow to exactly 0.
+    cos_abs=0: centres -1+2m/(A-1); cos_abs=1: centres m/(A-1) on |cos|, and the windowed branch
+    keeps the top ``window`` bins whatever the cosine (the end_dim formula of :155 assumes [-1,1]).
+    """
+    if cos_abs:
+        c = c.abs()
+        interval = 1.0 / (A - 1)
+        mu = torch.arange(A, dtype=c.dtype) * interval
+    else:
+        interval = 2.0 / (A - 1)
+        mu = -1.0 + torch.arange(A, dtype=c.dtype) * interval
+    u = (mu - c[..., None]) / (math.sqrt(2.0) * angle_sigma)
+    g = torch.exp(-u * u)
+    if window is not None and A - window > 8:
+        end = torch.trunc(torch.clamp((c + 1.0 + 4 * angle_sigma) / interval + 1.0, max=float(A)))
+        end = end.clamp(min=float(window))
+        m = torch.arange(A, dtype=c.dtype).expand(g.shape)
+        keep = (m >= end[..., None] - window) & (m < end[..., None])
+        g = g * keep
+    return g * valid[..., None]
+
+
+# --------------------------------------------------------------------------------------
+# z and the value position encoding psi
+# --------------------------------------------------------------------------------------
+def framed_pe(a_ih, rpos, tvecs, batch, edges, W_k, W_axes, frames, *, K=64, dist_max=14.0,
+              wscale=1.0, A=64, angle_wscale=4.0, cos_abs=0, c_dist=1.0, c_angle=1.0,
+              rvlen=None, cutoff_radius=None, lattice_range=2, minimum_range=2,
+              windows="reference", return_parts=False):
+    """z (E,H) and psi (E,H,Dh) of RealEncodingWithFramedProjFuncCUDA.forward.
+
+    models/cuda_funcs/real_space_framed_proj.py:21-120 with the two kernels it launches.
+    ``W_k`` (1,H,Dh,K) or None; ``W_axes`` sequence of three (1,H,Dh,A) or None;
+    ``frames`` sequence of three (N,H,3).  ``windows``: "reference" (9/33-bin truncation, the
+    kernel's), "full" (no truncation, the pure-PyTorch layer's), or an explicit (Wl, Wa).
+    Differentiable in ``a_ih``, ``W_k`` and ``W_axes`` (float64 autograd = gradient oracle).
+    """
+    dt = a_ih.dtype
+    N, H = a_ih.shape
+    E = edges.shape[1]
+    if windows == "reference":
+        wl, wa = reference_windows(K, wscale, A, angle_wscale)
+    elif windows == "full":
+        wl = wa = None
+    else:
+        wl, wa = windows
+    if A > 0:
+        angle_sigma = (angle_wscale / (A - 1)) if cos_abs else (2.0 * angle_wscale / (A - 1))
+    R = translation_ranges(a_ih, rvlen, batch, cutoff_radius, lattice_range, minimum_range)
+    sizes = torch.bincount(batch, minlength=tvecs.shape[0]).tolist()
+    Dh = W_k.shape[-2] if W_k is not None else (W_axes[0].shape[-2] if W_axes is not None else 0)
+
+    z_out, psi_out, d2min_out, shat_len, shat_ang = [], [], [], [], []
+    n_off = 0
+    e_off = 0
+    for b, nb in enumerate(sizes):
+        if nb == 0:
+            continue
+        sl_n = slice(n_off, n_off + nb)
+        sl_e = slice(e_off, e_off + nb * nb)
+        Rb = R[sl_n]                                        # (nb,H,3)
+        gi, gf = _grid(Rb.reshape(-1, 3).max(0).values.tolist(), dt)
+        shift = gf @ tvecs[b].to(dt)                        # (T,3): n1*t1 + n2*t2 + n3*t3
+        delta = rpos[sl_e].to(dt)[:, None, :] + shift[None]  # (nb*nb, T, 3)
+        d2 = (delta * delta).sum(-1)                        # (e,T)
+        inbox = (gi.abs()[None, None] <= Rb[:, :, None, :]).all(-1)   # (nb,H,T)
+        inbox_e = inbox.repeat_interleave(nb, dim=0)        # (e,H,T) rows follow i
+        a_e = a_ih[sl_n].repeat_interleave(nb, dim=0)       # (e,H)
+        logit = a_e[:, :, None] * d2[:, None, :]
+        logit = torch.where(inbox_e, logit, torch.full_like(logit, -float("inf")))
+        z = torch.logsumexp(logit, dim=-1)                  # (e,H)
+        p = torch.exp(logit - z[..., None])                 # softmax over translations
+        z_out.append(z)
+        d2min_out.append(torch.where(inbox_e, d2[:, None, :].expand_as(logit),
+                                     torch.full_like(logit, 1e10)).min(-1).values)
+        psi = torch.zeros(nb * nb, H, Dh, dtype=dt)
+        d = torch.sqrt(d2)
+        if W_k is not None and K > 0:
+            g = _length_basis(d, K, dist_max, wscale, wl)    # (e,T,K)
+            s = torch.einsum("eht,etk->ehk", p, g)
+            shat_len.append(s)
+            psi = psi + c_dist * torch.einsum("hck,ehk->ehc", W_k.reshape(H, Dh, K).to(dt), s)
+        if W_axes is not None and A > 0:
+            valid = d2 > 1e-5
+            dsafe = torch.where(valid, d, torch.ones_like(d))
+            s_axes = []
+            for ax in range(3):
+                f = frames[ax][sl_n].to(dt).repeat_interleave(nb, dim=0)     # (e,H,3)
+                cosv = torch.einsum("etx,ehx->eht", delta, f) / dsafe[:, None, :]
+                g = _angle_basis(cosv, valid[:, None, :].expand_as(cosv), A, angle_sigma, cos_abs, wa)
+                s = torch.einsum("eht,ehtm->ehm", p, g)
+                s_axes.append(s)
+                psi = psi + c_angle * torch.einsum("hcm,ehm->ehc", W_axes[ax].reshape(H, Dh, A).to(dt), s)
+            shat_ang.append(torch.stack(s_axes))
+        psi_out.append(psi)
+        n_off += nb
+        e_off += nb * nb
+    z = torch.cat(z_out) if z_out else torch.zeros(0, H, dtype=dt)
+    psi = torch.cat(psi_out) if psi_out else torch.zeros(0, H, Dh, dtype=dt)
+    if return_parts:
+        parts = {
+            "d2min": torch.cat(d2min_out),
+            "shat_len": torch.cat(shat_len) if shat_len else None,
+            "shat_ang": torch.cat(shat_ang, dim=1) if shat_ang else None,
+            "R": R,
+        }
+        return z, psi, parts
+    return z, psi
+
+
+def lattice_logsumexp(a_ih, rpos, tvecs, batch, edges, **kw):
+    """z only (no value encoding)."""
+    N, H = a_ih.shape
+    z, _ = framed_pe(a_ih, rpos, tvecs, batch, edges, None, None, None, K=0, A=0, **kw)
+    return z
+
+
+# --------------------------------------------------------------------------------------
+# frames
+# --------------------------------------------------------------------------------------
+def _argmax_first(v: torch.Tensor):
+    """arg-max with the earliest index winning ties (strict '>' update while scanning upward)."""
+    m = v.max()
+    idx = int(torch.nonzero(v == m)[0, 0])
+    return idx, m
+
+
+def frame_axes_max(q, k, a_ih, rpos, tvecs, batch, edges, *, rvlen=None, cutoff_radius=None,
+                   lattice_range=2, minimum_range=2, return_gaps=False):
+    """First and second ("max" method) frame axes, noise-free tie rule.
+
+    ``q`` must already be divided by sqrt(head_dim)
+    (models/indexed_lattice_multi_head_attention_cuda.py:446-447).
+
+    frame1(i,h): unit direction of the nearest image with d^2 > 1e-5 of the neighbour j that
+    maximises  q_i.k_j + a*d2min(e)   (compute_maximum_frame_each_edge.cu:78-111 with zero noise:
+    strict '<' keeps the first image in loop order; calc_maximum_frame.py:72-86).
+    frame2max(i,h): per edge the image maximising a*(d^2-d2min)+log(max(1-|cos|,1e-5)) subject to
+    |cos| < 0.9999 and d^2 > 1e-5 (compute_second_frame_each_edge.cu:81-142), then the neighbour
+    maximising q.k + that value + a*d2min (calc_maximum_frame.py:146-164).
+    Ties across neighbours go to the lowest edge index (segmented arg-max; parity unpinned on ties).
+    ``return_gaps``: also return, per (i,h), winner-minus-runner-up scores (ambiguity measure).
+    """
+    dt = a_ih.dtype
+    N, H = a_ih.shape
+    R = translation_ranges(a_ih, rvlen, batch, cutoff_radius, lattice_range, minimum_range)
+    sizes = torch.bincount(batch, minlength=tvecs.shape[0]).tolist()
+    f1 = torch.zeros(N, H, 3, dtype=dt)
+    f2 = torch.zeros(N, H, 3, dtype=dt)
+    gap1 = torch.full((N, H), float("inf"), dtype=dt)
+    gap2 = torch.full((N, H), float("inf"), dtype=dt)
+    n_off = e_off = 0
+    for b, nb in enumerate(sizes):
+        if nb == 0:
+            continue
+        for il in range(nb):
+            i = n_off + il
+            es = slice(e_off + il * nb, e_off + (il + 1) * nb)
+            js = edges[1, es]
+            for h in range(H):
+                gi, gf = _grid(R[i, h].tolist(), dt)
+                shift = gf @ tvecs[b].to(dt)
+                delta = rpos[es].to(dt)[:, None, :] + shift[None]          # (nb,T,3)
+                d2 = (delta * delta).sum(-1)
+                ok = d2 > 1e-5
+                qk = (q[i, h].to(dt)[None, :] * k[js, h].to(dt)).sum(-1)   # (nb,)
+                a = a_ih[i, h]
+                # ---- first axis
+                d2nz = torch.where(ok, d2, torch.full_like(d2, 1e10))
+                d2min_nz = d2nz.min(dim=1).values
+                tmin = torch.stack([torch.nonzero(d2nz[r] == d2min_nz[r])[0, 0] for r in range(nb)])  # first in loop order
+                score1 = qk + a * d2min_nz
+                j1, _ = _argmax_first(score1)
+                v1 = delta[j1, tmin[j1]]
+                f1[i, h] = v1 / v1.norm()
+                if nb > 1:
+                    s = torch.sort(score1, descending=True).values
+                    gap1[i, h] = s[0] - s[1]
+                # runner-up image inside the winning edge (ties between +n/-n on self edges are
+                # structural and resolved by order, so they are not counted as ambiguity)
+                # ---- second axis
+                dsafe = torch.sqrt(torch.where(ok, d2, torch.ones_like(d2)))
+                unit = delta / dsafe[..., None]
+                cosv = (unit * f1[i, h]).sum(-1)
+                val = a * (d2 - d2min_nz[:, None]) + torch.log(torch.clamp(1 - cosv.abs(), min=1e-5))
+                cand = ok & (cosv.abs() < 0.9999)
+                val = torch.where(cand, val, torch.full_like(val, -float("inf")))
+                best_t = torch.stack([torch.nonzero(val[r] == val[r].max())[0, 0] for r in range(nb)])
+                best_v = val[torch.arange(nb), best_t] + a * d2min_nz
+                score2 = qk + best_v
+                j2, _ = _argmax_first(score2)
+                f2[i, h] = unit[j2, best_t[j2]]
+                allv = (val + (a * d2min_nz + qk)[:, None]).flatten()
+                s = torch.sort(allv, descending=True).values
+                # +n / -n images of the self edge tie exactly; skip exact duplicates of the winner
+                s = s[s < s[0]]
+                if s.numel() > 0:
+                    gap2[i, h] = (allv.max() - s[0])
+        n_off += nb
+        e_off += nb * nb
+    if return_gaps:
+        return f1, f2, gap1, gap2
+    return f1, f2
+
+
+def orthonormal_frame(f1, f2max):
+    """Gram-Schmidt + cross product (indexed_lattice_multi_head_attention_cuda.py:475-481)."""
+    dot = (f1 * f2max).sum(-1, keepdim=True)
+    f2 = torch.nn.functional.normalize(f2max - dot * f1, dim=2)
+    f3 = torch.linalg.cross(f1, f2)
+    return f1, f2, f3
+
+
+# --------------------------------------------------------------------------------------
+# consumer: softmax over neighbours, and pooling
+# --------------------------------------------------------------------------------------
+def softmax_attention(q, k, v, z, psi, batch, edges):
+    """o_i = sum_j softmax_j(q_i.k_j + z_ij) (v_j + psi_ij);  q pre-scaled by 1/sqrt(Dh).
+
+    models/kernels/fused_dpa_fwd.cu:46-124 (max-subtracted softmax per (i,h)).
+    Returns (out (N,H,Dh), prob (E,H)).
+    """
+    N, H, D = q.shape
+    logit = (q[edges[0]] * k[edges[1]]).sum(-1)
+    if z is not None:
+        logit = logit + z
+    m = torch.full((N, H), -float("inf"), dtype=q.dtype).scatter_reduce(
+        0, edges[0][:, None].expand(-1, H), logit, reduce="amax")
+    ex = torch.exp(logit - m[edges[0]])
+    den = torch.zeros(N, H, dtype=q.dtype).index_add(0, edges[0], ex)
+    prob = ex / den[edges[0]]
+    val = v[edges[1]]
+    if psi is not None:
+        val = val + psi
+    out = torch.zeros(N, H, v.shape[-1], dtype=q.dtype).index_add(0, edges[0], prob[..., None] * val)
+    return out, prob
+
+
+def crystal_mean(x, batch, nbatch):
+    """Per-crystal mean (models/kernels/irregular_mean_fwd.cu:13-90; summation order ignored)."""
+    s = torch.zeros((nbatch,) + x.shape[1:], dtype=x.dtype).index_add(0, batch, x)
+    cnt = torch.bincount(batch, minlength=nbatch).to(x.dtype)
+    return s / cnt.reshape((-1,) + (1,) * (x.dim() - 1))
+
+
+# --------------------------------------------------------------------------------------
+# alpha -> a
+# --------------------------------------------------------------------------------------
+def gaussian_coefficient(alpha, scale_real=1.4, gauss_lb=0.5, beta=0.1):
+    """a = [(1-lb)*elu(alpha*beta/(1-lb)) + 1] * (-1/2 r0^-2)
+
+    models/indexed_lattice_multi_head_attention_cuda.py:925,940.
+    """
+    f = (1.0 - gauss_lb) * torch.nn.functional.elu(alpha * (beta / (1.0 - gauss_lb))) + 1.0
+    return f * (-0.5 * scale_real ** -2)
