@@ -112,7 +112,8 @@ cfh::BasisConsts basis_consts(const cfh_params* p) {
     if (p->angle_bins > 0) {
         const int A = p->angle_bins;
         const double interval = (p->cos_abs ? 1.0 : 2.0) / (A - 1);
-        const double sigma = (p->cos_abs ? 1.0 : 2.0) * (double)p->angle_wscale / (A - 1);
+        // the reference passes sigma to its kernels as a float32 scalar
+        const double sigma = (double)(float)((p->cos_abs ? 1.0 : 2.0) * (double)p->angle_wscale / (A - 1));
         bc.ang_inv_interval = (float)(1.0 / interval);
         bc.ang_end_off = (float)(1.0 + cut * sigma);
         bc.ang_interval = (float)interval;

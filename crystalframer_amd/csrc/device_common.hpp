@@ -145,32 +145,56 @@ __device__ __forceinline__ WindowSeed window_seed(float beta_c, float sig, float
     return s;
 }
 
+// Histograms are accumulated in LDS as unsigned 32-bit fixed point (FIX_ONE = 1.0), with integer
+// atomics.  Measured on MI355X: a conflict-free wave64 ds_add_u32 costs about 6 LDS clocks per CU,
+// a ds_add_f32 costs 190-260 whatever the addresses (the float adder takes the lanes one at a time),
+// so float atomics are not usable in an inner loop.  The quantities accumulated are
+// softmax-normalised weights times Gaussians, so every bin stays within [0, 1]; one unit in the last
+// place is 4.7e-10, finer than a float32 accumulator.  Lanes spread over NREP replicas of the
+// histogram (lane & (NREP-1)), shifted by 4 banks each, which divides same-address collisions of
+// lanes whose windows coincide (clamped windows at the ends of the cosine range).
+constexpr int NREP = 8;
+constexpr int REP_STRIDE = 4 * HS + 4;            // words between replicas: 4 rows + a 4-bank shift
+constexpr float FIX_ONE = 2147483648.0f;          // 2^31
+constexpr float FIX_INV = 1.0f / 2147483648.0f;
+
 template <int W>
-__device__ __forceinline__ void window_scatter(float* base, const WindowSeed& s, float cc) {
+__device__ __forceinline__ void window_scatter(uint32_t* base, const WindowSeed& s, float cc) {
     constexpr int C = W / 2;
-    atomicAdd(base + C, s.gc);
+    atomicAdd(base + C, (uint32_t)s.gc);
     float g = s.gc, r = s.rr;
 #pragma unroll
-    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; atomicAdd(base + m, g); }
+    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; atomicAdd(base + m, (uint32_t)g); }
     g = s.gc; r = s.rl;
 #pragma unroll
-    for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; atomicAdd(base + m, g); }
+    for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; atomicAdd(base + m, (uint32_t)g); }
 }
 
 // Scatter weight*g_m into hbase[m] and return sum_m weight*g_m*gbase[m].
 template <int W>
-__device__ __forceinline__ float window_scatter_gather(float* hbase, const float* gbase,
+__device__ __forceinline__ float window_scatter_gather(uint32_t* hbase, const float* gbase,
                                                        const WindowSeed& s, float cc) {
     constexpr int C = W / 2;
     float acc = s.gc * gbase[C];
-    atomicAdd(hbase + C, s.gc);
+    atomicAdd(hbase + C, (uint32_t)s.gc);
     float g = s.gc, r = s.rr;
 #pragma unroll
-    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); atomicAdd(hbase + m, g); }
+    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); atomicAdd(hbase + m, (uint32_t)g); }
     g = s.gc; r = s.rl;
 #pragma unroll
-    for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); atomicAdd(hbase + m, g); }
+    for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); atomicAdd(hbase + m, (uint32_t)g); }
     return acc;
+}
+
+// Sum the NREP replicas of histogram word `idx` (idx < 4*HS), clear them, return the float value.
+__device__ __forceinline__ float take_bin(uint32_t* hist, int idx) {
+    uint32_t s = 0;
+#pragma unroll
+    for (int r = 0; r < NREP; r++) {
+        s += hist[r * REP_STRIDE + idx];
+        hist[r * REP_STRIDE + idx] = 0u;
+    }
+    return (float)s * FIX_INV;
 }
 
 // Constants of the two bases, prepared on the host.

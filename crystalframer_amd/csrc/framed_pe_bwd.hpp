@@ -20,13 +20,14 @@ template <int WL, int WA, bool COS_ABS, bool HAS_LEN, bool HAS_ANG>
 __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P) {
     __shared__ float4 tab[TCAP];
     __shared__ uint16_t list[TCAP];
-    __shared__ __attribute__((aligned(16))) float hist[4 * HS];   // sum_n p g_k per encoder
-    __shared__ __attribute__((aligned(16))) float Gs[4 * HS];     // projected upstream gradient
+    __shared__ uint32_t hist[NREP * REP_STRIDE];                  // fixed-point sum_n p g_k per encoder
+    __shared__ __attribute__((aligned(16))) float Gs[4 * HS];     // projected upstream gradient / 2^31
 
     constexpr int NENC = HAS_ANG ? 4 : (HAS_LEN ? 1 : 0);
     const int lane = threadIdx.x;
     const int H = P.H;
     const int h = blockIdx.x % H;
+    uint32_t* const myhist = hist + (lane & (NREP - 1)) * REP_STRIDE;
 
     // lane k: W_enc[h, c, k] for all (enc, c), and the gradient accumulators of the same shape
     float Wt[NENC > 0 ? NENC * DH : 1];
@@ -40,6 +41,10 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
         }
     const BasisConsts bc = P.bc;
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
+
+    for (int u = lane; u < NREP * REP_STRIDE; u += WAVE) hist[u] = 0u;
+    for (int u = lane; u < 4 * HS; u += WAVE) Gs[u] = 0.0f;
+    __syncthreads();
 
     for (;;) {
         const int it = next_item(P.counters + h, lane);
@@ -90,18 +95,13 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
 #pragma unroll
                 for (int c = 0; c < DH; c++) gp[c] = uniform_f(P.gpsi[((size_t)e * H + h) * DH + c]);
             }
-            __syncthreads();       // previous pair's reads of hist / Gs are done
+            __syncthreads();       // previous pair's reads of Gs are done
 #pragma unroll
             for (int en = 0; en < NENC; en++) {
                 float g = 0.0f;
 #pragma unroll
                 for (int c = 0; c < DH; c++) g = fmaf(Wt[en * DH + c], gp[c], g);
-                Gs[en * HS + lane] = g * (en == 0 ? P.dist_coef : P.angle_coef);
-                hist[en * HS + lane] = 0.0f;
-            }
-            if (lane < HS - NBINS) {     // padding columns (never read, kept defined)
-#pragma unroll
-                for (int en = 0; en < NENC; en++) { Gs[en * HS + NBINS + lane] = 0.0f; hist[en * HS + NBINS + lane] = 0.0f; }
+                Gs[en * HS + lane] = g * ((en == 0 ? P.dist_coef : P.angle_coef) * FIX_INV);
             }
             __syncthreads();
 
@@ -122,7 +122,9 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
                         const float4 v = tab[u];
                         const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
                         const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
-                        keep = fmaf(a2, d2, -z2) >= prune;
+                        const float ex = fmaf(a2, d2, -z2);
+                        keep = ex >= prune;
+                        if (!keep) A0 = fmaf(hw_exp2(ex), d2, A0);    // light terms still count in dz/da
                     }
                     const uint64_t m = __ballot(keep);
                     if (keep) list[nkeep + lane_prefix(m)] = (uint16_t)u;
@@ -135,6 +137,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
                         const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
                         const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
                         const float p = hw_exp2(fmaf(a2, d2, -z2));
+                        const float pf = p * FIX_ONE;
                         float pbg = 0.0f;
                         if (HAS_LEN) {
                             const float d = hw_sqrt(d2);
@@ -142,8 +145,8 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
                             int start = (int)(u - bc.start_off);
                             start = max(0, min(start, NBINS - WL));
                             const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
-                            const WindowSeed s = window_seed(beta_c, bc.len_step, p);
-                            pbg += window_scatter_gather<WL>(hist + start, Gs + start, s, bc.len_cc);
+                            const WindowSeed s = window_seed(beta_c, bc.len_step, pf);
+                            pbg += window_scatter_gather<WL>(myhist + start, Gs + start, s, bc.len_cc);
                         }
                         if (HAS_ANG) {
                             if (d2 > 1e-5f) {
@@ -158,8 +161,8 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
                                     const int start = end - WA;
                                     const float mu_c = bc.ang_mu0 + (float)(start + WA / 2) * bc.ang_interval;
                                     const float beta_c = (mu_c - cs) * bc.ang_sigma_inv;
-                                    const WindowSeed s = window_seed(beta_c, bc.ang_step, p);
-                                    pbg += window_scatter_gather<WA>(hist + (ax + 1) * HS + start,
+                                    const WindowSeed s = window_seed(beta_c, bc.ang_step, pf);
+                                    pbg += window_scatter_gather<WA>(myhist + (ax + 1) * HS + start,
                                                                      Gs + (ax + 1) * HS + start, s, bc.ang_cc);
                                 }
                             }
@@ -174,10 +177,10 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
             A0 = wave_sum(A0); A1 = wave_sum(A1); A2 = wave_sum(A2);
             ga_acc += P.gz_coef * gz * A0 + (A1 - A0 * A2);
 
-            // weight gradients: gW_enc[c] (lane k) += coef * gpsi[c] * hist_enc[k]
+            // weight gradients: gW_enc[c] (lane k) += coef * gpsi[c] * s_enc[k]
 #pragma unroll
             for (int en = 0; en < NENC; en++) {
-                const float sk = hist[en * HS + lane] * (en == 0 ? P.gw_dist_coef : P.angle_coef);
+                const float sk = take_bin(hist, en * HS + lane) * (en == 0 ? P.gw_dist_coef : P.angle_coef);
 #pragma unroll
                 for (int c = 0; c < DH; c++) gW[en * DH + c] = fmaf(gp[c], sk, gW[en * DH + c]);
             }

@@ -205,7 +205,8 @@ def framed_pe(a_ih, rpos, tvecs, batch, edges, W_k, W_axes, frames, *, K=64, dis
     else:
         wl, wa = windows
     if A > 0:
-        angle_sigma = (angle_wscale / (A - 1)) if cos_abs else (2.0 * angle_wscale / (A - 1))
+        # the reference hands this to its kernels as a float32 scalar (real_space_framed_proj.py:37-40,97)
+        angle_sigma = float(np.float32((angle_wscale / (A - 1)) if cos_abs else (2.0 * angle_wscale / (A - 1))))
     R = translation_ranges(a_ih, rvlen, batch, cutoff_radius, lattice_range, minimum_range)
     sizes = torch.bincount(batch, minlength=tvecs.shape[0]).tolist()
     Dh = W_k.shape[-2] if W_k is not None else (W_axes[0].shape[-2] if W_axes is not None else 0)

@@ -50,5 +50,6 @@ def make_problem(num_crystals=6, atoms_lo=1, atoms_hi=5, len_lo=3.0, len_hi=8.0,
 
 def rel_err(x, ref):
     """max |x-ref| / max |ref| (tensor-scale relative error)."""
+    x, ref = x.detach(), ref.detach()
     scale = ref.abs().max().clamp_min(1e-30)
     return float((x.double().cpu() - ref.double()).abs().max() / scale)

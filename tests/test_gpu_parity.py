@@ -1,0 +1,344 @@
+"""Parity of the HIP kernels (through the C ABI and the autograd.Function boundary) against the CPU
+oracles, on seeded synthetic crystals.  Tolerances (float32 kernels vs float64 oracle, errors
+relative to the largest magnitude of the tensor compared):
+
+  * same truncation windows as the oracle ........ 2e-5 forward, 5e-5 gradients
+  * 5-sigma kernel windows vs full-basis oracle .. 1e-4   (the bar BASELINE.json states)
+  * 4-sigma (reference) windows vs full basis .... 5e-4   (the reference kernels' own truncation,
+                                                           exp(-8) per dropped bin)
+"""
+import math
+
+import pytest
+import torch
+
+import helpers as Hh
+from oracle import c_oracle as CO
+from oracle import torch_oracle as TO
+
+pytestmark = pytest.mark.gpu
+
+CUT = -3.5
+
+
+@pytest.fixture(autouse=True)
+def _defaults():
+    import crystalframer_amd as cf
+    KM = cf.KernelManager
+    saved = (KM.SYMM_BREAK_NOISE, KM.PRUNE_LOG2, KM.WINDOW_MODE, KM.GRAD_COEF_QUIRK, KM.LATTICE_RANGE, KM.MINIMUM_RANGE)
+    KM.SYMM_BREAK_NOISE = 0.0
+    KM.PRUNE_LOG2 = 32.0
+    KM.WINDOW_MODE = 0
+    KM.GRAD_COEF_QUIRK = False
+    KM.LATTICE_RANGE, KM.MINIMUM_RANGE = 2, 2
+    yield
+    (KM.SYMM_BREAK_NOISE, KM.PRUNE_LOG2, KM.WINDOW_MODE, KM.GRAD_COEF_QUIRK, KM.LATTICE_RANGE, KM.MINIMUM_RANGE) = saved
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def g(t):
+    return None if t is None else t.to(dtype=torch.float32, device=dev())
+
+
+def run_pe(P, *, K=64, A=64, cos_abs=0, cd=1.0, ca=1.0, cutoff=CUT, frames=None, need_grad=True):
+    """Call the operator boundary the way the reference layer does; returns outputs and leaves."""
+    import crystalframer_amd as cf
+    a = g(P.a).requires_grad_(need_grad)
+    Wk = g(P.W_k).requires_grad_(need_grad) if K > 0 else None
+    Wax = [g(w).requires_grad_(need_grad) for w in P.W_ax] if (A > 0 and K > 0) else [None] * 3
+    fr = [g(f) for f in (frames or P.frames)] if A > 0 else [None] * 3
+    extra = (g(P.rvlen), cutoff) if cutoff is not None else ()
+    out = cf.RealEncodingWithFramedProjFuncCUDA.apply(
+        a, g(P.rpos), None, g(P.tvecs), P.batch.to(dev()), P.edges.to(dev()), K, Hh.DIST_MAX, 1.0,
+        Wk, Wax[0], Wax[1], Wax[2], fr[0], fr[1], fr[2], A, 4.0, cos_abs, cd, ca, *extra)
+    return out, a, Wk, Wax
+
+
+def oracle_pe(P, *, K=64, A=64, cos_abs=0, cd=1.0, ca=1.0, cutoff=CUT, windows="reference", frames=None,
+              lattice_range=2):
+    a = P.a.clone().requires_grad_(True)
+    Wk = P.W_k.clone().requires_grad_(True) if K > 0 else None
+    Wax = [w.clone().requires_grad_(True) for w in P.W_ax] if (A > 0 and K > 0) else None
+    z, psi = TO.framed_pe(a, P.rpos, P.tvecs, P.batch, P.edges, Wk, Wax, frames or P.frames, K=K, A=A,
+                          cos_abs=cos_abs, c_dist=cd, c_angle=ca, rvlen=P.rvlen, cutoff_radius=cutoff,
+                          windows=windows, lattice_range=lattice_range)
+    return z, psi, a, Wk, Wax
+
+
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("cos_abs", [0, 1])
+@pytest.mark.parametrize("prune", [0.0, 32.0])
+def test_framed_pe_forward_backward_reference_windows(cos_abs, prune):
+    import crystalframer_amd as cf
+    cf.KernelManager.PRUNE_LOG2 = prune
+    P = Hh.make_problem(num_crystals=10, atoms_hi=6, seed=100 + cos_abs)
+    cd, ca = 0.75, 1.25
+    (z, psi), a, Wk, Wax = run_pe(P, cos_abs=cos_abs, cd=cd, ca=ca)
+    zo, psio, ao, Wko, Waxo = oracle_pe(P, cos_abs=cos_abs, cd=cd, ca=ca)
+    assert Hh.rel_err(z, zo.detach()) < 2e-5
+    assert Hh.rel_err(psi, psio.detach()) < 2e-5
+    ((z * g(P.gz)).sum() + (psi * g(P.gpsi)).sum()).backward()
+    ((zo * P.gz).sum() + (psio * P.gpsi).sum()).backward()
+    assert Hh.rel_err(a.grad, ao.grad) < 5e-5
+    assert Hh.rel_err(Wk.grad, Wko.grad) < 5e-5
+    for x, y in zip(Wax, Waxo):
+        assert Hh.rel_err(x.grad, y.grad) < 5e-5
+
+
+def test_framed_pe_matches_c_oracle_in_reference_arithmetic():
+    """Kernel vs the float32 scalar port of the reference kernels (same windows, same ranges)."""
+    P = Hh.make_problem(num_crystals=8, atoms_hi=5, seed=7)
+    (z, psi), *_ = run_pe(P, need_grad=False)
+    p = CO.make_params(cutoff_radius=CUT)
+    zc, psic, _ = CO.pe_forward(p, P.a, P.rpos, P.tvecs, P.rvlen, P.batch, P.edges, P.W_k[0], P.W_ax, P.frames, "f32")
+    assert Hh.rel_err(z, zc) < 2e-5
+    assert Hh.rel_err(psi, psic) < 5e-5
+
+
+def test_wide_windows_match_full_basis_within_1e4():
+    import crystalframer_amd as cf
+    P = Hh.make_problem(num_crystals=10, atoms_hi=6, seed=17)
+    zo, psio, ao, Wko, Waxo = oracle_pe(P, windows="full")
+    ((zo * P.gz).sum() + (psio * P.gpsi).sum()).backward()
+    for mode, tol in ((1, 1e-4), (0, 5e-4)):
+        cf.KernelManager.WINDOW_MODE = mode
+        (z, psi), a, Wk, Wax = run_pe(P)
+        ((z * g(P.gz)).sum() + (psi * g(P.gpsi)).sum()).backward()
+        assert Hh.rel_err(z, zo.detach()) < 2e-5
+        assert Hh.rel_err(psi, psio.detach()) < tol
+        assert Hh.rel_err(a.grad, ao.grad) < tol
+        assert Hh.rel_err(Wk.grad, Wko.grad) < tol
+        for x, y in zip(Wax, Waxo):
+            assert Hh.rel_err(x.grad, y.grad) < tol
+
+
+def test_distance_only_and_z_only_variants():
+    P = Hh.make_problem(num_crystals=8, atoms_hi=5, seed=23)
+    # Crystalformer mode: value_pe_angle_real = 0
+    (z, psi), a, Wk, _ = run_pe(P, A=0)
+    zo, psio, ao, Wko, _ = oracle_pe(P, A=0)
+    ((z * g(P.gz)).sum() + (psi * g(P.gpsi)).sum()).backward()
+    ((zo * P.gz).sum() + (psio * P.gpsi).sum()).backward()
+    assert Hh.rel_err(z, zo.detach()) < 2e-5 and Hh.rel_err(psi, psio.detach()) < 2e-5
+    assert Hh.rel_err(a.grad, ao.grad) < 5e-5 and Hh.rel_err(Wk.grad, Wko.grad) < 5e-5
+    # no value encoding at all: returns a 1-tuple like the reference
+    out, a, _, _ = run_pe(P, K=0, A=0)
+    assert isinstance(out, tuple) and len(out) == 1
+    ao = P.a.clone().requires_grad_(True)
+    zo = TO.lattice_logsumexp(ao, P.rpos, P.tvecs, P.batch, P.edges, rvlen=P.rvlen, cutoff_radius=CUT)
+    (out[0] * g(P.gz)).sum().backward()
+    (zo * P.gz).sum().backward()
+    assert Hh.rel_err(out[0], zo.detach()) < 2e-5
+    assert Hh.rel_err(a.grad, ao.grad) < 5e-5
+
+
+def test_fixed_grid_without_adaptive_cutoff():
+    """cutoff arguments omitted: the fixed (2*LATTICE_RANGE+1)^3 grid of the pure-PyTorch path."""
+    P = Hh.make_problem(num_crystals=8, atoms_hi=5, seed=29)
+    (z, psi), *_ = run_pe(P, cutoff=None, need_grad=False)
+    zo, psio, *_ = oracle_pe(P, cutoff=None)
+    assert Hh.rel_err(z, zo.detach()) < 2e-5 and Hh.rel_err(psi, psio.detach()) < 2e-5
+
+
+def test_gradient_coefficient_quirk_mode():
+    import crystalframer_amd as cf
+    cf.KernelManager.GRAD_COEF_QUIRK = True
+    P = Hh.make_problem(num_crystals=6, atoms_hi=4, seed=31)
+    cd, ca = 0.5, 1.5
+    (z, psi), a, Wk, Wax = run_pe(P, cd=cd, ca=ca)
+    ((z * g(P.gz)).sum() + (psi * g(P.gpsi)).sum()).backward()
+    p = CO.make_params(dist_coef=cd, angle_coef=ca, cutoff_radius=CUT, grad_coef_quirk=True)
+    zc, _, _ = CO.pe_forward(p, P.a, P.rpos, P.tvecs, P.rvlen, P.batch, P.edges, P.W_k[0], P.W_ax, P.frames, "f64")
+    ga, gWd, gWa = CO.pe_backward(p, P.a, P.rpos, P.tvecs, P.rvlen, P.batch, P.edges, P.W_k[0], P.W_ax, P.frames,
+                                  zc, P.gz, P.gpsi, "f64")
+    assert Hh.rel_err(a.grad, ga) < 5e-5
+    assert Hh.rel_err(Wk.grad[0], gWd) < 5e-5
+    for ax in range(3):
+        assert Hh.rel_err(Wax[ax].grad[0], gWa[ax]) < 5e-5
+
+
+def test_small_cells_need_more_translations_than_one_lds_table():
+    """Cells of 1.5-2 angstrom: R up to 4-5, i.e. more than 512 translations (chunked table path)."""
+    P = Hh.make_problem(num_crystals=4, atoms_lo=1, atoms_hi=3, len_lo=1.5, len_hi=2.0, ang_lo=80, ang_hi=100, seed=37)
+    R = TO.translation_ranges(P.a, P.rvlen, P.batch, CUT)
+    assert int((2 * R + 1).prod(-1).max()) > 512
+    (z, psi), a, Wk, Wax = run_pe(P)
+    zo, psio, ao, Wko, Waxo = oracle_pe(P)
+    ((z * g(P.gz)).sum() + (psi * g(P.gpsi)).sum()).backward()
+    ((zo * P.gz).sum() + (psio * P.gpsi).sum()).backward()
+    assert Hh.rel_err(z, zo.detach()) < 2e-5 and Hh.rel_err(psi, psio.detach()) < 2e-5
+    assert Hh.rel_err(a.grad, ao.grad) < 5e-5 and Hh.rel_err(Wk.grad, Wko.grad) < 5e-5
+    f1, f2 = run_frames(P)
+    f1o, f2o, gap1, gap2 = TO.frame_axes_max(P.q, P.k, P.a, P.rpos, P.tvecs, P.batch, P.edges, rvlen=P.rvlen,
+                                             cutoff_radius=CUT, return_gaps=True)
+    check_frames(f1, f2, f1o, f2o, gap1, gap2)
+
+
+def test_one_atom_crystals_and_empty_batch():
+    import crystalframer_amd as cf
+    P = Hh.make_problem(num_crystals=5, atoms_lo=1, atoms_hi=1, seed=41)
+    (z, psi), *_ = run_pe(P, need_grad=False)
+    zo, psio, *_ = oracle_pe(P)
+    assert Hh.rel_err(z, zo.detach()) < 2e-5 and Hh.rel_err(psi, psio.detach()) < 2e-5
+    # empty batch: nothing to do, empty outputs, zero weight gradients
+    d = dev()
+    a = torch.zeros(0, Hh.H, device=d, requires_grad=True)
+    Wk = g(P.W_k).requires_grad_(True)
+    z, psi = cf.RealEncodingWithFramedProjFuncCUDA.apply(
+        a, torch.zeros(0, 3, device=d), None, torch.zeros(0, 3, 3, device=d), torch.zeros(0, dtype=torch.long, device=d),
+        torch.zeros(2, 0, dtype=torch.long, device=d), 64, 14.0, 1.0, Wk, None, None, None, None, None, None,
+        0, 4.0, 0, 1.0, 1.0)
+    assert z.shape == (0, Hh.H) and psi.shape == (0, Hh.H, Hh.DH)
+    (z.sum() + psi.sum()).backward()
+    assert float(Wk.grad.abs().max()) == 0.0
+
+
+# ------------------------------------------------------------------------------------------------
+def run_frames(P, cutoff=CUT, f1_for_second=None):
+    import crystalframer_amd as cf
+    args = (g(P.q), g(P.k), None, g(P.a), g(P.rpos), None, g(P.tvecs), P.batch.to(dev()), P.edges.to(dev()),
+            64, Hh.DIST_MAX, 1.0)
+    extra = (g(P.rvlen), cutoff) if cutoff is not None else ()
+    f1 = cf.ComputeFrame1MaximumMethodCUDA.apply(*args, *extra)
+    f2 = cf.ComputeFrame2MaximumMethodCUDA.apply(*args, f1 if f1_for_second is None else g(f1_for_second), *extra)
+    return f1, f2
+
+
+def check_frames(f1, f2, f1o, f2o, gap1, gap2, min_clear=0.9):
+    """Equal wherever the float64 winner beats its runner-up by more than float32 rounding."""
+    clear1 = gap1 > 1e-4
+    clear2 = clear1 & (gap2 > 1e-4)
+    assert clear2.double().mean() > min_clear
+    assert (f1.cpu().double() - f1o)[clear1].abs().max() < 1e-5
+    assert (f2.cpu().double() - f2o)[clear2].abs().max() < 1e-5
+    n1 = f1.cpu().double().norm(dim=-1)
+    assert (n1 - 1).abs().max() < 1e-5
+
+
+def test_frame_axes_match_oracle():
+    P = Hh.make_problem(num_crystals=12, atoms_hi=6, seed=51)
+    f1o, f2o, gap1, gap2 = TO.frame_axes_max(P.q, P.k, P.a, P.rpos, P.tvecs, P.batch, P.edges, rvlen=P.rvlen,
+                                             cutoff_radius=CUT, return_gaps=True)
+    f1, f2 = run_frames(P)
+    check_frames(f1, f2, f1o, f2o, gap1, gap2)
+    # second axis given the oracle's first axis (decouples the two searches)
+    _, f2b = run_frames(P, f1_for_second=f1o)
+    assert (f2b.cpu().double() - f2o)[gap2 > 1e-4].abs().max() < 1e-5
+
+
+def test_frame_axes_self_edge_tie_rule_single_atom():
+    """One atom per cell: every candidate is a +n/-n pair with exactly equal score; the first image
+    in loop order (the lexicographically smaller translation) must win, as in the C oracle."""
+    P = Hh.make_problem(num_crystals=6, atoms_lo=1, atoms_hi=1, seed=57)
+    f1, f2 = run_frames(P)
+    p = CO.make_params(cutoff_radius=CUT)
+    c1, c2 = CO.frame_axes(p, P.q, P.k, P.a, P.rpos, P.tvecs, P.rvlen, P.batch, P.edges, "f32")
+    assert (f1.cpu() - c1).abs().max() < 1e-5
+    agree = ((f2.cpu() - c2).abs().amax(-1) < 1e-5).float().mean()
+    assert agree > 0.9            # remaining cases: float32 near-ties between different shells
+
+
+def test_frame_noise_keeps_clear_winners():
+    import crystalframer_amd as cf
+    P = Hh.make_problem(num_crystals=10, atoms_lo=2, atoms_hi=6, seed=61)
+    f1o, f2o, gap1, gap2 = TO.frame_axes_max(P.q, P.k, P.a, P.rpos, P.tvecs, P.batch, P.edges, rvlen=P.rvlen,
+                                             cutoff_radius=CUT, return_gaps=True)
+    cf.KernelManager.SYMM_BREAK_NOISE = 1e-5
+    cf.KernelManager.NOISE_SEED = 1234
+    try:
+        f1, f2 = run_frames(P)
+    finally:
+        cf.KernelManager.NOISE_SEED = None
+    # the noise decides the exact +n/-n ties of self images, so a clear winner is fixed up to sign
+    clear = (gap1 > 1e-3) & (gap2 > 1e-3)
+    assert (1 - (f1.cpu().double() * f1o).sum(-1).abs())[clear].max() < 1e-5
+    assert (1 - (f2.cpu().double() * f2o).sum(-1).abs())[clear].max() < 1e-5
+    flipped = ((f1.cpu().double() * f1o).sum(-1) < 0)[clear].double().mean()
+    assert 0.0 < flipped < 0.5    # some ties do go the other way, which zero noise never does
+
+
+# ------------------------------------------------------------------------------------------------
+# size-independent properties at the benchmark's batch shape
+# ------------------------------------------------------------------------------------------------
+def _c2_problem(num_crystals):
+    from crystalframer_amd import synthetic
+    cb = synthetic.make_config("C2", seed=123, num_crystals=num_crystals)
+    gen = torch.Generator().manual_seed(9)
+    P = Hh.Problem()
+    P.batch, P.sizes = cb.batch, cb.sizes.tolist()
+    P.pos, P.tvecs = cb.pos.double(), cb.trans_vec.double()
+    P.edges, P.rpos, recip, _ = TO.geometry(P.pos, P.tvecs, P.sizes)
+    P.rvlen = torch.norm(recip, 2, dim=-1)
+    P.N, P.E = P.pos.shape[0], P.edges.shape[1]
+    P.a = TO.gaussian_coefficient(torch.randn(P.N, Hh.H, generator=gen, dtype=torch.float64))
+    P.q = torch.randn(P.N, Hh.H, Hh.DH, generator=gen, dtype=torch.float64) / 4
+    P.k = torch.randn(P.N, Hh.H, Hh.DH, generator=gen, dtype=torch.float64)
+    P.W_k = torch.randn(1, Hh.H, Hh.DH, 64, generator=gen, dtype=torch.float64) * 0.3
+    P.W_ax = [torch.randn(1, Hh.H, Hh.DH, 64, generator=gen, dtype=torch.float64) * 0.3 for _ in range(3)]
+    f1 = torch.nn.functional.normalize(torch.randn(P.N, Hh.H, 3, generator=gen, dtype=torch.float64), dim=-1)
+    f2 = torch.nn.functional.normalize(torch.randn(P.N, Hh.H, 3, generator=gen, dtype=torch.float64), dim=-1)
+    P.frames = list(TO.orthonormal_frame(f1, f2))
+    return P
+
+
+def test_full_batch_rotation_invariance_and_frame_equivariance():
+    """Batch 256 of the benchmark distribution: rotating every crystal rotates the frames and leaves
+    z and psi unchanged (the SE(3) property the method is built for)."""
+    P = _c2_problem(256)
+    gq = torch.Generator().manual_seed(5)
+    Q, _ = torch.linalg.qr(torch.randn(3, 3, generator=gq, dtype=torch.float64))
+    if torch.det(Q) < 0:
+        Q[:, 0] = -Q[:, 0]
+    f1, f2 = run_frames(P)
+    fr = TO.orthonormal_frame(f1.cpu().double(), f2.cpu().double())
+    (z, psi), *_ = run_pe(P, frames=fr, need_grad=False)
+    assert torch.isfinite(z).all() and torch.isfinite(psi).all()
+    P2 = Hh.Problem()
+    P2.__dict__.update(P.__dict__)
+    P2.rpos, P2.tvecs = P.rpos @ Q.T, P.tvecs @ Q.T
+    g1, g2 = run_frames(P2)
+    same1 = ((f1.cpu().double() @ Q.T - g1.cpu().double()).abs().amax(-1) < 1e-4)
+    same2 = ((f2.cpu().double() @ Q.T - g2.cpu().double()).abs().amax(-1) < 1e-4)
+    assert same1.double().mean() > 0.999 and same2.double().mean() > 0.995   # float32 near-ties aside
+    fr2 = [f @ Q.T for f in fr]
+    (z2, psi2), *_ = run_pe(P2, frames=fr2, need_grad=False)
+    assert Hh.rel_err(z2, z.cpu().double()) < 2e-5
+    assert Hh.rel_err(psi2, psi.cpu().double()) < 1e-4
+    # spot check of the full batch against the oracle on its first crystals
+    nb = 6
+    n_at, n_e = sum(P.sizes[:nb]), sum(s * s for s in P.sizes[:nb])
+    S = Hh.Problem()
+    S.a, S.rpos, S.tvecs, S.batch, S.edges = P.a[:n_at], P.rpos[:n_e], P.tvecs[:nb], P.batch[:n_at], P.edges[:, :n_e]
+    S.rvlen, S.W_k, S.W_ax = P.rvlen[:nb], P.W_k, P.W_ax
+    S.frames = [f[:n_at] for f in fr]
+    zo, psio, *_ = oracle_pe(S)
+    assert Hh.rel_err(z[:n_e], zo.detach()) < 2e-5
+    assert Hh.rel_err(psi[:n_e], psio.detach()) < 5e-5
+
+
+def test_full_batch_atom_permutation_equivariance():
+    """Reversing the atom order inside every crystal permutes z and psi accordingly."""
+    P = _c2_problem(64)
+    (z, psi), *_ = run_pe(P, need_grad=False)
+    perm = []
+    off = 0
+    for n in P.sizes:
+        perm += list(range(off + n - 1, off - 1, -1))
+        off += n
+    perm = torch.tensor(perm)
+    P2 = Hh.Problem()
+    P2.__dict__.update(P.__dict__)
+    P2.pos, P2.a = P.pos[perm], P.a[perm]
+    P2.frames = [f[perm] for f in P.frames]
+    P2.edges, P2.rpos, _, _ = TO.geometry(P2.pos, P.tvecs, P.sizes)
+    (z2, psi2), *_ = run_pe(P2, need_grad=False)
+    # edge (i,j) of the permuted problem is edge (perm[i], perm[j]) of the original one
+    lookup = {}
+    for e in range(P.E):
+        lookup[(int(P.edges[0, e]), int(P.edges[1, e]))] = e
+    src = torch.tensor([lookup[(int(perm[int(P2.edges[0, e])]), int(perm[int(P2.edges[1, e])]))] for e in range(P.E)])
+    assert Hh.rel_err(z2, z.cpu().double()[src]) < 1e-5
+    assert Hh.rel_err(psi2, psi.cpu().double()[src]) < 2e-5
