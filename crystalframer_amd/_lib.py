@@ -41,7 +41,7 @@ class CfhParams(ctypes.Structure):
         ("symm_break_noise", ctypes.c_float),
         ("noise_seed", ctypes.c_uint64),
         ("grad_coef_quirk", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("collect_stats", ctypes.c_int32),
     ]
 
 
@@ -122,8 +122,22 @@ def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        buf[:512].zero_()          # work-queue heads and the statistics block
         _workspaces[key] = buf
     return buf
+
+
+STAT_NAMES = ("fwd_evaluated", "fwd_in_box", "bwd_evaluated", "bwd_in_box", "frame1_scanned",
+              "frame2_scanned", "fwd_pairs", "bwd_pairs")
+
+
+def read_stats(device: torch.device, reset: bool = False) -> dict:
+    """Term counts accumulated by launches made with ``collect_stats`` on this stream (synchronises)."""
+    buf = workspace(device, 512)
+    vals = buf[256:256 + 8 * len(STAT_NAMES)].view(torch.int64).cpu().tolist()
+    if reset:
+        buf[256:512].zero_()
+    return dict(zip(STAT_NAMES, vals))
 
 
 def current_stream_ptr(device: torch.device):

@@ -28,7 +28,8 @@ int fail(int code, const char* fmt, ...) {
 }
 
 constexpr int MAX_HEADS = 64;
-constexpr size_t COUNTER_BYTES = 256;          // MAX_HEADS int32 work-queue heads
+constexpr size_t COUNTER_BYTES = 512;          // MAX_HEADS int32 work-queue heads, then 32 uint64 statistics
+constexpr size_t STATS_OFFSET = 256;
 constexpr int WAVES_PER_SIMD = 3;
 
 __global__ void reset_counters_kernel(int32_t* counters) { counters[threadIdx.x] = 0; }
@@ -150,6 +151,7 @@ void fill_common(cfh::KernelArgs& A, const cfh_params* p, const float* a_ih, con
     A.a_ih = a_ih; A.rpos = rpos; A.tvecs = tvecs; A.rvlen = rvlen;
     A.batch = batch; A.edges = edges; A.e_start = e_start; A.order = order;
     A.counters = reinterpret_cast<int32_t*>(workspace);
+    A.stats = p->collect_stats ? reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(workspace) + STATS_OFFSET) : nullptr;
     A.N = (int32_t)N; A.E = (int32_t)E; A.H = p->num_heads;
     A.cutoff_radius = rvlen ? p->cutoff_radius : 0.0f;
     A.lattice_range = p->lattice_range; A.minimum_range = p->minimum_range;

@@ -61,6 +61,10 @@ __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
         if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
     }
 }
+// slots of KernelArgs::stats
+enum { STAT_FWD_EVAL = 0, STAT_FWD_RAW = 1, STAT_BWD_EVAL = 2, STAT_BWD_RAW = 3, STAT_FRAME1_RAW = 4,
+       STAT_FRAME2_RAW = 5, STAT_FWD_PAIRS = 6, STAT_BWD_PAIRS = 7 };
+
 __device__ __forceinline__ int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ float uniform_f(float v) {
     return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
@@ -227,6 +231,7 @@ struct KernelArgs {
     float* out_z; float* out_psi; float* out_d2min; float* out_frame; float* out_ga;
     float* gw_partial;            // (waves, 4, DH, NBINS) per-wave weight-gradient partials
     int32_t* counters;            // (H) work-queue heads
+    unsigned long long* stats;    // optional running totals (see STAT_* below); never reset by a launch
     int32_t N, E, H;
     float cutoff_radius; int32_t lattice_range, minimum_range;
     float prune_log2;             // <= 0: keep every translation

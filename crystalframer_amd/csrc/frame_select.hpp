@@ -172,6 +172,9 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
             const float inv = d2 > 0.0f ? 1.0f / sqrtf(d2) : 0.0f;
             float* o = P.out_frame + ((size_t)i * H + h) * 3;
             o[0] = bx_ * inv; o[1] = by_ * inv; o[2] = bz_ * inv;
+            if (P.stats)
+                atomicAdd(P.stats + (SECOND ? STAT_FRAME2_RAW : STAT_FRAME1_RAW),
+                          (unsigned long long)bx.T * (unsigned long long)(e1 - e0));
         }
     }
 }

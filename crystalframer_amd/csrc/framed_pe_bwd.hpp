@@ -81,6 +81,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
         const int e0 = uniform_i((int)P.e_start[i]);
         const int e1 = uniform_i((int)P.e_start[i + 1]);
         float ga_acc = 0.0f;
+        unsigned long long n_eval = 0;
 
         for (int e = e0; e < e1; e++) {
             const float rx = uniform_f(P.rpos[(size_t)e * 3 + 0]);
@@ -130,6 +131,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
                     if (keep) list[nkeep + lane_prefix(m)] = (uint16_t)u;
                     nkeep += __popcll(m);
                 }
+                n_eval += (unsigned long long)nkeep;
                 __syncthreads();
                 for (int v0 = 0; v0 < nkeep; v0 += WAVE) {
                     if (v0 + lane < nkeep) {
@@ -185,7 +187,14 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
                 for (int c = 0; c < DH; c++) gW[en * DH + c] = fmaf(gp[c], sk, gW[en * DH + c]);
             }
         }
-        if (lane == 0) P.out_ga[(size_t)i * H + h] = ga_acc;
+        if (lane == 0) {
+            P.out_ga[(size_t)i * H + h] = ga_acc;
+            if (P.stats) {
+                atomicAdd(P.stats + STAT_BWD_EVAL, n_eval);
+                atomicAdd(P.stats + STAT_BWD_RAW, (unsigned long long)bx.T * (unsigned long long)(e1 - e0));
+                atomicAdd(P.stats + STAT_BWD_PAIRS, (unsigned long long)(e1 - e0));
+            }
+        }
     }
 
     // per-wavefront partials of the weight gradients: (wave, enc, c, k)

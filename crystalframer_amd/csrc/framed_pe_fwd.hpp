@@ -83,6 +83,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
         }
         const int e0 = uniform_i((int)P.e_start[i]);
         const int e1 = uniform_i((int)P.e_start[i + 1]);
+        unsigned long long n_eval = 0;
 
         for (int e = e0; e < e1; e++) {
             const float rx = uniform_f(P.rpos[(size_t)e * 3 + 0]);
@@ -151,6 +152,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                     nkeep += __popcll(m);
                 }
                 if (nchunks == 1) S = wave_sum(Sb);
+                n_eval += (unsigned long long)nkeep;
                 const float wfix = FIX_ONE / S;
                 __syncthreads();
                 // ---- pass C: window scatters of the normalised weights
@@ -221,6 +223,11 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                 P.out_z[(size_t)e * H + h] = logf(S) + d2min * a;
                 if (P.out_d2min) P.out_d2min[(size_t)e * H + h] = d2min;
             }
+        }
+        if (P.stats && lane == 0) {
+            atomicAdd(P.stats + STAT_FWD_EVAL, n_eval);
+            atomicAdd(P.stats + STAT_FWD_RAW, (unsigned long long)bx.T * (unsigned long long)(e1 - e0));
+            atomicAdd(P.stats + STAT_FWD_PAIRS, (unsigned long long)(e1 - e0));
         }
     }
 }

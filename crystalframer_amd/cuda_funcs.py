@@ -32,6 +32,8 @@ class KernelManager:
     WINDOW_MODE: int = _lib.CFH_WINDOW_REFERENCE
     PRUNE_LOG2: float = 32.0            # skip translations lighter than 2^-32 of their pair's heaviest
     GRAD_COEF_QUIRK: bool = False
+    COLLECT_STATS: bool = False         # count translations (read with _lib.read_stats)
+    EVENT_LOG = None                    # a list: every library call appends (name, start, end) events
     _compiled_for = None
 
 
@@ -78,10 +80,39 @@ def _params(H: int, Dh: int, K: int, A: int, cos_abs: int, dist_max: float, wsca
     else:
         p.noise_seed = int(KernelManager.NOISE_SEED)
     p.grad_coef_quirk = int(bool(KernelManager.GRAD_COEF_QUIRK))
+    p.collect_stats = int(bool(KernelManager.COLLECT_STATS))
     return p
 
 
+class _timed:
+    """Brackets one library call with HIP events on the current stream when
+    ``KernelManager.EVENT_LOG`` is a list; appends (name, start, end) to it."""
+
+    def __init__(self, name, dev):
+        self.name, self.dev, self.log = name, dev, KernelManager.EVENT_LOG
+
+    def __enter__(self):
+        if self.log is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.end = torch.cuda.Event(enable_timing=True)
+            self.start.record(torch.cuda.current_stream(self.dev))
+        return self
+
+    def __exit__(self, *exc):
+        if self.log is not None:
+            self.end.record(torch.cuda.current_stream(self.dev))
+            self.log.append((self.name, self.start, self.end))
+        return False
+
+
 _edge_cache = {"ref": None, "version": None, "N": None, "val": None}
+
+
+def seed_edge_schedule(edge_ij_e: torch.Tensor, e_start: torch.Tensor, order: torch.Tensor):
+    """Hand over an (e_start, order) pair already known for ``edge_ij_e`` (geometry.py computes it)."""
+    N = e_start.shape[0] - 1
+    _edge_cache.update(ref=weakref.ref(edge_ij_e), version=edge_ij_e._version, N=N,
+                       val=(e_start.contiguous(), order.to(torch.int32).contiguous()))
 
 
 def edge_schedule(edge_ij_e: torch.Tensor, N: int):
@@ -139,7 +170,7 @@ def _frame_call(second: bool, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e
     e_start, order = edge_schedule(edge_ij_e, N)
     out = torch.zeros((N, H, 3), dtype=torch.float32, device=dev)
     p = _params(H, Dh, 0, 0, 0, 1.0, 1.0, 1.0, 1.0, 1.0, cutoff_radius if rv is not None else None)
-    with torch.cuda.device(dev):
+    with torch.cuda.device(dev), _timed("frame_axis2" if second else "frame_axis1", dev):
         need = lib.cfh_workspace_bytes(ctypes.byref(p), N, E)
         ws = _lib.workspace(dev, need)
         st = _lib.current_stream_ptr(dev)
@@ -220,7 +251,7 @@ class RealEncodingWithFramedProjFuncCUDA(torch.autograd.Function):
         v = torch.empty((E, H, Dh), dtype=torch.float32, device=dev) if K > 0 else None
         p = _params(H, Dh, K, A, cos_abs, float(dist_max), wscale, value_pe_angle_scale,
                     length_rbf_mul, angle_rbf_mul, cutoff_radius if rv is not None else None)
-        with torch.cuda.device(dev):
+        with torch.cuda.device(dev), _timed("framed_pe_forward", dev):
             ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
             rc = lib.cfh_framed_pe_forward(
                 ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch),
@@ -251,7 +282,7 @@ class RealEncodingWithFramedProjFuncCUDA(torch.autograd.Function):
         ga = torch.empty((N, H), dtype=torch.float32, device=dev)
         gWd = torch.empty_like(Wd) if Wd is not None else None
         gWa = [torch.empty_like(w) if w is not None else None for w in (W1, W2, W3)]
-        with torch.cuda.device(dev):
+        with torch.cuda.device(dev), _timed("framed_pe_backward", dev):
             ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
             rc = lib.cfh_framed_pe_backward(
                 ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch),
@@ -263,3 +294,52 @@ class RealEncodingWithFramedProjFuncCUDA(torch.autograd.Function):
         gws = [g if g is None else g.reshape(s) for g, s in zip([gWd] + gWa, ctx.w_shapes)]
         return (ga, None, None, None, None, None, None, None, None, gws[0], gws[1], gws[2], gws[3],
                 None, None, None, None, None, None, None, None, None, None)
+
+
+# --------------------------------------------------------------------------------------------------
+# consumers of z and psi.  Interim composites of stock PyTorch device ops with the reference's names
+# and signatures; they run on the HIP device (no CPU path) but are not hand-written kernels yet.
+# --------------------------------------------------------------------------------------------------
+class FusedDotProductAttentionCUDA:
+    """out_i = sum_j softmax_j(q_i.k_j + a_ij) (v_j + b_ij), per head, over the edges of atom i.
+
+    Signature of models/cuda_funcs/fused_dpa.py:17-63 (``que_ihk`` already divided by sqrt(Dh));
+    max-subtracted softmax as in models/kernels/fused_dpa_fwd.cu:46-91.
+    """
+
+    @staticmethod
+    def apply(que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, batch_i, edge_ij_e):
+        _lib.require_gpu(que_ihk, key_ihk, val_ihk)
+        N, H, _ = que_ihk.shape
+        ei, ej = edge_ij_e[0], edge_ij_e[1]
+        logit = (que_ihk[ei] * key_ihk[ej]).sum(-1)
+        if aij_eh is not None:
+            logit = logit + aij_eh
+        idx = ei[:, None].expand(-1, H)
+        mx = torch.full((N, H), -3.0e38, dtype=logit.dtype, device=logit.device)
+        mx = mx.scatter_reduce(0, idx, logit.detach(), reduce="amax", include_self=True)
+        ex = torch.exp(logit - mx[ei])
+        den = torch.zeros((N, H), dtype=logit.dtype, device=logit.device).index_add_(0, ei, ex)
+        prob = ex / den[ei]
+        val = val_ihk[ej]
+        if bij_ehk is not None:
+            val = val + bij_ehk
+        out = torch.zeros_like(val_ihk).index_add_(0, ei, prob[..., None] * val)
+        return out
+
+
+class IrregularMeanCUDA:
+    """Per-crystal mean of per-atom features.  Signature of models/cuda_funcs/irregular_mean.py:19-70."""
+
+    @staticmethod
+    def apply(x_ik, batch_i, sizes):
+        _lib.require_gpu(x_ik)
+        if sizes is None:
+            B = int(batch_i.max().item()) + 1
+            sizes = torch.zeros(B, dtype=torch.long, device=x_ik.device)
+            sizes.scatter_add_(0, batch_i, torch.ones_like(batch_i))
+        B = sizes.shape[0]
+        out = torch.zeros((B,) + tuple(x_ik.shape[1:]), dtype=x_ik.dtype, device=x_ik.device)
+        out.index_add_(0, batch_i, x_ik)
+        shape = [B] + [1] * (x_ik.dim() - 1)
+        return out / sizes.reshape(shape).to(x_ik.dtype)

@@ -1,0 +1,132 @@
+"""Encoder stack around the periodic attention layer.
+
+Counterpart of ``CrystalformerEncoderCUDA`` / ``CrystalformerEncoderLayerCUDA``
+(reference: models/indexed_latticeformer_encoder.py:644-901): same sub-module and parameter names,
+residual blocks without normalisation when T-Fixup is on, T-Fixup rescaling of the value / output /
+feed-forward weights.  The per-batch geometry is prepared once on the device (``geometry.py``)
+instead of in a Python loop over crystals.
+"""
+from __future__ import annotations
+
+from typing import Callable, Optional, Union
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor, nn
+from torch.nn.init import constant_, xavier_uniform_
+
+from . import cuda_funcs, geometry
+from .attention import CrystalformerMultiheadAttentionCUDA
+from .params import LatticeformerParams
+
+
+def _activation(name):
+    if callable(name):
+        return name
+    if name == "relu":
+        return F.relu
+    if name == "gelu":
+        return F.gelu
+    raise RuntimeError(f"activation should be relu/gelu, not {name}")
+
+
+class CrystalformerEncoderLayerCUDA(nn.Module):
+    def __init__(self, d_model: int, nhead: int, dim_feedforward: int = 2048, dropout: float = 0.1,
+                 activation: Union[str, Callable[[Tensor], Tensor]] = F.relu, layer_norm_eps: float = 1e-5,
+                 norm_first: bool = False, no_layer_norm: bool = False,
+                 params: Optional[LatticeformerParams] = None, k_dim: int = 0, v_dim: int = 0) -> None:
+        super().__init__()
+        params = params if params is not None else LatticeformerParams()
+        self.domain = params.domain
+        self.self_attn = CrystalformerMultiheadAttentionCUDA(d_model, nhead, dropout=dropout, kdim=k_dim,
+                                                             vdim=v_dim, params=params)
+        self.linear1 = nn.Linear(d_model, dim_feedforward)
+        self.dropout = nn.Dropout(dropout) if dropout > 0 else nn.Identity()
+        self.linear2 = nn.Linear(dim_feedforward, d_model)
+        self.norm_first = norm_first
+        self.norm1 = nn.LayerNorm(d_model, eps=layer_norm_eps) if not no_layer_norm else nn.Identity()
+        self.norm2 = nn.LayerNorm(d_model, eps=layer_norm_eps) if not no_layer_norm else nn.Identity()
+        self.dropout1 = nn.Dropout(dropout) if dropout > 0 else nn.Identity()
+        self.dropout2 = nn.Dropout(dropout) if dropout > 0 else nn.Identity()
+        self.activation = _activation(activation)
+        xavier_uniform_(self.linear1.weight)
+        xavier_uniform_(self.linear2.weight)
+        constant_(self.linear1.bias, 0)
+        constant_(self.linear2.bias, 0)
+
+    def fixup_initialization(self, num_layers: int):
+        """T-Fixup: scale four weight matrices by 0.67 * L^(-1/4)
+        (reference: models/indexed_latticeformer_encoder.py:820-841)."""
+        s = 0.67 * num_layers ** (-1.0 / 4.0)
+        with torch.no_grad():
+            for w in (self.linear1.weight, self.linear2.weight, self.self_attn.out_proj.weight,
+                      self.self_attn.v_proj_weight):
+                w.mul_(s)
+
+    def _sa_block(self, x, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell, onehot, this_epoch):
+        x = self.self_attn(x, x, x, batch, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs, vcell,
+                           onehot, need_weights=False, this_epoch=this_epoch)[0]
+        return self.dropout1(x)
+
+    def _ff_block(self, x):
+        return self.dropout2(self.linear2(self.dropout(self.activation(self.linear1(x)))))
+
+    def forward(self, src: Tensor, batch: Tensor, edges: Tensor, pos_ij: Tensor = None,
+                dist2_min: Tensor = None, trans: Tensor = None, kr_base: Tensor = None,
+                rvecs: Tensor = None, vcell: Tensor = None, onehot: Tensor = None,
+                this_epoch: int = None) -> Tensor:
+        x = src
+        if self.norm_first:
+            x = x + self._sa_block(self.norm1(x), batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs,
+                                   vcell, onehot, this_epoch)
+            x = x + self._ff_block(self.norm2(x))
+        else:
+            x = self.norm1(x + self._sa_block(x, batch, edges, pos_ij, dist2_min, trans, kr_base, rvecs,
+                                              vcell, onehot, this_epoch))
+            x = self.norm2(x + self._ff_block(x))
+        return x
+
+
+class CrystalformerEncoderCUDA(nn.Module):
+    def __init__(self, d_model: int = 512, nhead: int = 8, num_encoder_layers: int = 6,
+                 dim_feedforward: int = 2048, dropout: float = 0.1,
+                 activation: Union[str, Callable[[Tensor], Tensor]] = F.relu, layer_norm_eps: float = 1e-5,
+                 norm_first: bool = False, t_fixup_init: bool = False, no_layer_norm: bool = False,
+                 lattice_params: Optional[LatticeformerParams] = None, k_dim: int = 0, v_dim: int = 0) -> None:
+        super().__init__()
+        lattice_params = lattice_params if lattice_params is not None else LatticeformerParams()
+        self.lattice_params = lattice_params
+        self.layers = nn.ModuleList([
+            CrystalformerEncoderLayerCUDA(d_model, nhead, dim_feedforward, dropout, activation, layer_norm_eps,
+                                          norm_first, no_layer_norm,
+                                          params=lattice_params.getLayerParameters(i), k_dim=k_dim, v_dim=v_dim)
+            for i in range(num_encoder_layers)])
+        if t_fixup_init:
+            for layer in self.layers:
+                layer.fixup_initialization(num_encoder_layers)
+        self.num_layers = num_encoder_layers
+        self.norm = nn.LayerNorm(d_model, eps=layer_norm_eps) if not no_layer_norm else None
+        self.d_model = d_model
+        self.nhead = nhead
+        P = lattice_params
+        cuda_funcs.compile_kernels(
+            P.lattice_range, nhead, k_dim if k_dim > 0 else d_model // nhead, P.value_pe_dist_real,
+            P.value_pe_angle_real, v_dim if v_dim > 0 else d_model // nhead, P.minimum_range, P.cos_abs,
+            P.value_pe_dist_wscale, P.value_pe_angle_wscale, P.value_pe_dist_coef, P.value_pe_angle_coef,
+            P.symm_break_noise)
+
+    def forward(self, src: Tensor, pos: Tensor, batch: Tensor, trans: Tensor, sizes: Tensor,
+                onehot: Tensor = None, this_epoch: int = None) -> Tensor:
+        """Reference: models/indexed_latticeformer_encoder.py:699-742."""
+        if src.size(-1) != self.d_model:
+            raise RuntimeError("the feature number of src and tgt must be equal to d_model")
+        batch = batch - batch[0]
+        geo = geometry.crystal_geometry(pos, batch, trans, sizes)
+        cuda_funcs.seed_edge_schedule(geo.edges, geo.e_start, geo.order)
+        x = src
+        for layer in self.layers:
+            # rvecs: the lengths of the reciprocal vectors are all the layers use, computed once here
+            x = layer(x, batch, geo.edges, geo.rpos, None, trans, None, geo.rvlen, geo.vcell, onehot, this_epoch)
+        if self.norm is not None:
+            x = self.norm(x)
+        return x

@@ -1,0 +1,88 @@
+"""Crystal property regressor: atom embedding -> periodic-attention encoder -> pooling -> MLP.
+
+Counterpart of ``Latticeformer`` (reference: models/latticeformer.py:32-287) for one GPU: same
+sub-module names (``input_embeddings``, ``encoder``, ``mlp``), same initialisation.  The
+single-process multi-GPU split of the reference (:209-273) is not part of this build.
+"""
+from __future__ import annotations
+
+import copy
+
+import torch
+from torch import nn
+
+from . import cuda_funcs
+from .encoder import CrystalformerEncoderCUDA
+from .params import LatticeformerParams, ModelParams
+
+ATOM_FEAT_DIM = 98
+
+
+def max_pool(x, batch, sizes):
+    B = sizes.shape[0]
+    out = torch.full((B,) + tuple(x.shape[1:]), -float("inf"), dtype=x.dtype, device=x.device)
+    return out.scatter_reduce(0, batch[:, None].expand_as(x), x, reduce="amax", include_self=True)
+
+
+def avr_pool(x, batch, sizes):
+    """Reference: models/pooling.py:19-25."""
+    return cuda_funcs.IrregularMeanCUDA.apply(x, batch, sizes)
+
+
+class Latticeformer(nn.Module):
+    def __init__(self, params: ModelParams = None):
+        super().__init__()
+        params = params if params is not None else ModelParams()
+        self.params = params
+        embedding_dim = copy.deepcopy(list(params.embedding_dim))
+        num_layers, model_dim = params.num_layers, params.model_dim
+        if params.use_cgcnn_feat or params.scale_grad > 0:
+            raise NotImplementedError("use_cgcnn_feat / scale_grad are not implemented")
+        lattice_params = LatticeformerParams().parseFromArgs(params)
+        self.input_embeddings = nn.Linear(ATOM_FEAT_DIM, model_dim, bias=False)
+        emb_scale = model_dim ** (-0.5)
+        if params.t_fixup_init:
+            emb_scale *= (9 * num_layers) ** (-1 / 4)
+        nn.init.normal_(self.input_embeddings.weight, mean=0, std=emb_scale)
+        self.encoder = CrystalformerEncoderCUDA(
+            model_dim, params.head_num, activation=params.t_activation, num_encoder_layers=num_layers,
+            dim_feedforward=params.ff_dim, dropout=params.dropout, t_fixup_init=params.t_fixup_init,
+            no_layer_norm=params.t_fixup_init, lattice_params=lattice_params, k_dim=params.k_dim,
+            v_dim=params.v_dim)
+        norm = {"bn": nn.BatchNorm1d, "ln": nn.LayerNorm, "in": nn.InstanceNorm1d,
+                "id": nn.Identity, "no": nn.Identity}.get(params.norm_type)
+        if norm is None:
+            raise NotImplementedError(f"norm_type: {params.norm_type}")
+        dim_pooled = model_dim
+        self.proj_before_pooling = nn.Identity()
+        if params.pre_pooling_op == "w+bn+relu":
+            dim_pooled = embedding_dim.pop(0)
+            self.proj_before_pooling = nn.Sequential(nn.Linear(model_dim, dim_pooled), norm(dim_pooled), nn.ReLU(True))
+        elif params.pre_pooling_op == "w+relu":
+            dim_pooled = embedding_dim.pop(0)
+            self.proj_before_pooling = nn.Sequential(nn.Linear(model_dim, dim_pooled), nn.ReLU(True))
+        elif params.pre_pooling_op == "relu":
+            self.proj_before_pooling = nn.ReLU(True)
+        elif params.pre_pooling_op != "no":
+            raise NotImplementedError(f"pre_pooling_op: {params.pre_pooling_op}")
+        if params.pooling == "max":
+            self.pooling_layer = max_pool
+        elif params.pooling == "avr":
+            self.pooling_layer = avr_pool
+        else:
+            raise NotImplementedError(f"pooling: {params.pooling}")
+        final_dim = 1 if isinstance(params.targets, str) else len(params.targets)
+        in_dim = [dim_pooled] + embedding_dim[:-1]
+        layers = []
+        for di, do in zip(in_dim, embedding_dim):
+            layers += [nn.Linear(di, do), norm(do), nn.ReLU(True)]
+        layers.append(nn.Linear(embedding_dim[-1], final_dim))
+        self.mlp = nn.Sequential(*layers)
+
+    def forward(self, data, this_epoch=None):
+        """``data`` carries x (N,98), pos (N,3), batch (N), trans_vec (B,3,3), sizes (B)."""
+        x = self.input_embeddings(data.x)
+        x = self.encoder(x, data.pos, data.batch, data.trans_vec, data.sizes, this_epoch=this_epoch)
+        x = self.proj_before_pooling(x)
+        x = self.pooling_layer(x, data.batch, data.sizes)
+        return self.mlp(x)

@@ -42,7 +42,7 @@ enum {
 enum {
     CFH_WINDOW_REFERENCE = 0,  /* +-4 sigma: ceil(8*wscale+1) bins, the reference kernels' rule
                                   (models/cuda_funcs/kernel_manager.py:146-147)                 */
-    CFH_WINDOW_WIDE = 1        /* two more bins on each side; dropped tail < 4e-6 of the peak   */
+    CFH_WINDOW_WIDE = 1        /* +-5 sigma: ceil(10*wscale+1) bins; dropped tail < 4e-6 of the peak */
 };
 
 /*
@@ -74,7 +74,11 @@ typedef struct cfh_params {
     uint64_t noise_seed;     /* seed of that noise                                                */
     int32_t grad_coef_quirk; /* 1: backward scales like the reference (d/dz part by dist_coef,
                                 dW_dist unscaled; real_space_framed_proj.py:183-184); 0: exact    */
-    int32_t reserved;
+    int32_t collect_stats;   /* 1: add term counts to the 32 uint64 totals at workspace+256 (the caller
+                                zeroes them; launches never do): [0] forward translations evaluated,
+                                [1] forward translations in the boxes, [2],[3] same for backward,
+                                [4],[5] translations scanned by the two frame searches, [6],[7] (pair,
+                                head) items of forward / backward                                   */
 } cfh_params;
 
 /* Version of this ABI; a mismatch with CFH_ABI_VERSION means header and library differ. */

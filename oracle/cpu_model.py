@@ -1,0 +1,107 @@
+"""CPU restatement of the CrystalFramer model forward (TEST INFRASTRUCTURE ONLY).
+
+Runs the architecture of the reference (models/latticeformer.py:191-287,
+models/indexed_latticeformer_encoder.py:699-742,848-897,
+models/indexed_lattice_multi_head_attention_cuda.py:869-988) on the CPU with the operators of
+``oracle/torch_oracle.py``, reading the weights from a state dict with the reference's parameter
+names.  It materialises the per-translation tensors like the reference's pure-PyTorch path does, so
+it is also what the benchmark times as its CPU baseline.  Gradients come from autograd.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+import torch.nn.functional as F
+
+from . import torch_oracle as TO
+
+
+def attention_layer(x, sd: Dict[str, torch.Tensor], prefix: str, geo, lp, *, windows="reference",
+                    gauss_scale: Optional[torch.Tensor] = None, frames_override=None, return_aux=False):
+    """One periodic attention layer.  ``geo`` = dict(edges, rpos, tvecs, rvlen, batch); ``lp`` = the
+    layer's LatticeformerParams-like object."""
+    dt = x.dtype
+    w = lambda name: sd[prefix + name].to(dt)
+    H = lp_heads(sd, prefix)
+    N = x.shape[0]
+    kdim = w("q_proj_weight").shape[0]
+    b = w("in_proj_bias")
+    q = F.linear(x, w("q_proj_weight"), b[:kdim]).view(N, H, -1)
+    k = F.linear(x, w("k_proj_weight"), b[kdim:2 * kdim]).view(N, H, -1)
+    v = F.linear(x, w("v_proj_weight"), b[2 * kdim:]).view(N, H, -1)
+    Dh = q.shape[-1]
+    alpha = (q * w("lattice_pos_weights").view(1, H, Dh)).sum(-1)
+    if lp.normalize_gauss:
+        gs = gauss_scale if gauss_scale is not None else sd[prefix + "gauss_scale"]
+        if float(gs[0]) > 0:
+            scale, shift = gs[0].to(dt), gs[1].to(dt)
+        else:
+            scale, shift = 1.0 / alpha.detach().std(), -alpha.detach().mean()
+        alpha = (alpha + shift) * scale
+    a = TO.gaussian_coefficient(alpha, lp.scale_real, lp.gauss_lb_real, lp.positive_func_beta)
+    cutoff = lp.adaptive_cutoff_sigma if lp.adaptive_cutoff_sigma < 0 else (
+        lp.scale_real * lp.gauss_lb_real ** (-0.5) * lp.adaptive_cutoff_sigma if lp.adaptive_cutoff_sigma > 0 else None)
+    rng = dict(rvlen=geo["rvlen"] if cutoff is not None else None, cutoff_radius=cutoff,
+               lattice_range=lp.lattice_range, minimum_range=lp.lattice_range if lp.minimum_range else 0)
+    dist_max = lp.value_pe_dist_max if lp.value_pe_dist_max >= 0 else -lp.value_pe_dist_max * lp.scale_real
+    K, A = lp.value_pe_dist_real, lp.value_pe_angle_real
+    W_k = w("pe_dist_proj") if K > 0 else None
+    W_ax = [w(f"proj_angle{n}") for n in (1, 2, 3)] if (A > 0 and K > 0) else None
+    frames = None
+    if W_ax is not None:
+        if frames_override is not None:
+            frames = frames_override
+        else:
+            qs = (q / math.sqrt(Dh)).detach()
+            f1, f2m = TO.frame_axes_max_vec(qs, k.detach(), a.detach(), geo["rpos"], geo["tvecs"], geo["batch"],
+                                            geo["edges"], **rng)
+            frames = TO.orthonormal_frame(f1, f2m)
+    z, psi = TO.framed_pe(a, geo["rpos"], geo["tvecs"], geo["batch"], geo["edges"], W_k, W_ax, frames,
+                          K=K, dist_max=dist_max, wscale=lp.value_pe_dist_wscale, A=A if W_ax is not None else 0,
+                          angle_wscale=lp.value_pe_angle_wscale, cos_abs=lp.cos_abs,
+                          c_dist=lp.value_pe_dist_coef, c_angle=lp.value_pe_angle_coef, windows=windows, **rng)
+    out, _ = TO.softmax_attention(q / math.sqrt(Dh), k, v, z, psi if K > 0 else None, geo["batch"], geo["edges"])
+    out = F.linear(out.reshape(N, -1), w("out_proj.weight"), w("out_proj.bias"))
+    if return_aux:
+        return out, dict(a=a, z=z, psi=psi, frames=frames, q=q, k=k, v=v)
+    return out
+
+
+def lp_heads(sd, prefix):
+    for name in ("pe_dist_proj", "proj_angle1"):
+        if prefix + name in sd:
+            return sd[prefix + name].shape[1]
+    raise KeyError("cannot infer the number of heads from " + prefix)
+
+
+def model_forward(sd: Dict[str, torch.Tensor], data, mp, *, dtype=torch.float32, windows="reference",
+                  frames_per_layer=None, return_aux=False):
+    """Prediction (B, targets) of the full model for a CrystalBatch-like ``data`` on the CPU."""
+    from crystalframer_amd.params import LatticeformerParams
+    lat = LatticeformerParams().parseFromArgs(mp)
+    pos, tv = data.pos.to(dtype), data.trans_vec.to(dtype)
+    sizes = data.sizes.tolist()
+    edges, rpos, recip, _ = TO.geometry(pos, tv, sizes)
+    geo = dict(edges=edges, rpos=rpos, tvecs=tv, rvlen=torch.norm(recip, 2, dim=-1), batch=data.batch)
+    x = F.linear(data.x.to(dtype), sd["input_embeddings.weight"].to(dtype))
+    auxes = []
+    for li in range(mp.num_layers):
+        lp = lat.getLayerParameters(li)
+        pre = f"encoder.layers.{li}."
+        r = attention_layer(x, sd, pre + "self_attn.", geo, lp, windows=windows,
+                            frames_override=None if frames_per_layer is None else frames_per_layer[li],
+                            return_aux=return_aux)
+        if return_aux:
+            r, aux = r
+            auxes.append(aux)
+        x = x + r
+        hdn = F.relu(F.linear(x, sd[pre + "linear1.weight"].to(dtype), sd[pre + "linear1.bias"].to(dtype)))
+        x = x + F.linear(hdn, sd[pre + "linear2.weight"].to(dtype), sd[pre + "linear2.bias"].to(dtype))
+    pooled = TO.crystal_mean(x, data.batch, len(sizes))
+    hdn = F.relu(F.linear(pooled, sd["mlp.0.weight"].to(dtype), sd["mlp.0.bias"].to(dtype)))
+    out = F.linear(hdn, sd["mlp.3.weight"].to(dtype), sd["mlp.3.bias"].to(dtype))
+    if return_aux:
+        return out, auxes
+    return out

@@ -186,7 +186,7 @@ def _angle_basis(c: torch.Tensor, valid: torch.Tensor, A: int, angle_sigma: floa
 def framed_pe(a_ih, rpos, tvecs, batch, edges, W_k, W_axes, frames, *, K=64, dist_max=14.0,
               wscale=1.0, A=64, angle_wscale=4.0, cos_abs=0, c_dist=1.0, c_angle=1.0,
               rvlen=None, cutoff_radius=None, lattice_range=2, minimum_range=2,
-              windows="reference", return_parts=False):
+              windows="reference", return_parts=False, max_elements=1 << 25):
     """z (E,H) and psi (E,H,Dh) of RealEncodingWithFramedProjFuncCUDA.forward.
 
     models/cuda_funcs/real_space_framed_proj.py:21-120 with the two kernels it launches.
@@ -217,43 +217,52 @@ def framed_pe(a_ih, rpos, tvecs, batch, edges, W_k, W_axes, frames, *, K=64, dis
     for b, nb in enumerate(sizes):
         if nb == 0:
             continue
-        sl_n = slice(n_off, n_off + nb)
-        sl_e = slice(e_off, e_off + nb * nb)
-        Rb = R[sl_n]                                        # (nb,H,3)
-        gi, gf = _grid(Rb.reshape(-1, 3).max(0).values.tolist(), dt)
-        shift = gf @ tvecs[b].to(dt)                        # (T,3): n1*t1 + n2*t2 + n3*t3
-        delta = rpos[sl_e].to(dt)[:, None, :] + shift[None]  # (nb*nb, T, 3)
-        d2 = (delta * delta).sum(-1)                        # (e,T)
-        inbox = (gi.abs()[None, None] <= Rb[:, :, None, :]).all(-1)   # (nb,H,T)
-        inbox_e = inbox.repeat_interleave(nb, dim=0)        # (e,H,T) rows follow i
-        a_e = a_ih[sl_n].repeat_interleave(nb, dim=0)       # (e,H)
-        logit = a_e[:, :, None] * d2[:, None, :]
-        logit = torch.where(inbox_e, logit, torch.full_like(logit, -float("inf")))
-        z = torch.logsumexp(logit, dim=-1)                  # (e,H)
-        p = torch.exp(logit - z[..., None])                 # softmax over translations
-        z_out.append(z)
-        d2min_out.append(torch.where(inbox_e, d2[:, None, :].expand_as(logit),
-                                     torch.full_like(logit, 1e10)).min(-1).values)
-        psi = torch.zeros(nb * nb, H, Dh, dtype=dt)
-        d = torch.sqrt(d2)
-        if W_k is not None and K > 0:
-            g = _length_basis(d, K, dist_max, wscale, wl)    # (e,T,K)
-            s = torch.einsum("eht,etk->ehk", p, g)
-            shat_len.append(s)
-            psi = psi + c_dist * torch.einsum("hck,ehk->ehc", W_k.reshape(H, Dh, K).to(dt), s)
-        if W_axes is not None and A > 0:
-            valid = d2 > 1e-5
-            dsafe = torch.where(valid, d, torch.ones_like(d))
-            s_axes = []
-            for ax in range(3):
-                f = frames[ax][sl_n].to(dt).repeat_interleave(nb, dim=0)     # (e,H,3)
-                cosv = torch.einsum("etx,ehx->eht", delta, f) / dsafe[:, None, :]
-                g = _angle_basis(cosv, valid[:, None, :].expand_as(cosv), A, angle_sigma, cos_abs, wa)
-                s = torch.einsum("eht,ehtm->ehm", p, g)
-                s_axes.append(s)
-                psi = psi + c_angle * torch.einsum("hcm,ehm->ehc", W_axes[ax].reshape(H, Dh, A).to(dt), s)
-            shat_ang.append(torch.stack(s_axes))
-        psi_out.append(psi)
+        Tb = int((2 * R[n_off:n_off + nb].reshape(-1, 3).max(0).values + 1).prod())
+        # rows (query atoms) per block, so that the (pairs, heads, translations, bins) tensors stay small
+        rows = max(1, min(nb, max_elements // max(1, nb * H * Tb * max(K, A, 1))))
+        for r0 in range(0, nb, rows):
+            r1 = min(nb, r0 + rows)
+            nr = r1 - r0
+            sl_n = slice(n_off + r0, n_off + r1)
+            sl_e = slice(e_off + r0 * nb, e_off + r1 * nb)
+            Rb = R[sl_n]                                        # (nr,H,3)
+            gi, gf = _grid(Rb.reshape(-1, 3).max(0).values.tolist(), dt)
+            shift = gf @ tvecs[b].to(dt)                        # (T,3): n1*t1 + n2*t2 + n3*t3
+            delta = rpos[sl_e].to(dt)[:, None, :] + shift[None]  # (nr*nb, T, 3)
+            d2 = (delta * delta).sum(-1)                        # (e,T)
+            inbox = (gi.abs()[None, None] <= Rb[:, :, None, :]).all(-1)   # (nr,H,T)
+            inbox_e = inbox.repeat_interleave(nb, dim=0)        # (e,H,T) rows follow i
+            a_e = a_ih[sl_n].repeat_interleave(nb, dim=0)       # (e,H)
+            logit = a_e[:, :, None] * d2[:, None, :]
+            logit = torch.where(inbox_e, logit, torch.full_like(logit, -float("inf")))
+            z = torch.logsumexp(logit, dim=-1)                  # (e,H)
+            p = torch.exp(logit - z[..., None])                 # softmax over translations
+            z_out.append(z)
+            if return_parts:
+                d2min_out.append(torch.where(inbox_e, d2[:, None, :].expand_as(logit),
+                                             torch.full_like(logit, 1e10)).min(-1).values)
+            psi = torch.zeros(nr * nb, H, Dh, dtype=dt)
+            d = torch.sqrt(d2)
+            if W_k is not None and K > 0:
+                g = _length_basis(d, K, dist_max, wscale, wl)    # (e,T,K)
+                s = torch.einsum("eht,etk->ehk", p, g)
+                if return_parts:
+                    shat_len.append(s)
+                psi = psi + c_dist * torch.einsum("hck,ehk->ehc", W_k.reshape(H, Dh, K).to(dt), s)
+            if W_axes is not None and A > 0:
+                valid = d2 > 1e-5
+                dsafe = torch.where(valid, d, torch.ones_like(d))
+                s_axes = []
+                for ax in range(3):
+                    f = frames[ax][sl_n].to(dt).repeat_interleave(nb, dim=0)     # (e,H,3)
+                    cosv = torch.einsum("etx,ehx->eht", delta, f) / dsafe[:, None, :]
+                    g = _angle_basis(cosv, valid[:, None, :].expand_as(cosv), A, angle_sigma, cos_abs, wa)
+                    s = torch.einsum("eht,ehtm->ehm", p, g)
+                    s_axes.append(s)
+                    psi = psi + c_angle * torch.einsum("hcm,ehm->ehc", W_axes[ax].reshape(H, Dh, A).to(dt), s)
+                if return_parts:
+                    shat_ang.append(torch.stack(s_axes))
+            psi_out.append(psi)
         n_off += nb
         e_off += nb * nb
     z = torch.cat(z_out) if z_out else torch.zeros(0, H, dtype=dt)
@@ -361,6 +370,61 @@ def frame_axes_max(q, k, a_ih, rpos, tvecs, batch, edges, *, rvlen=None, cutoff_
         e_off += nb * nb
     if return_gaps:
         return f1, f2, gap1, gap2
+    return f1, f2
+
+
+def frame_axes_max_vec(q, k, a_ih, rpos, tvecs, batch, edges, *, rvlen=None, cutoff_radius=None,
+                       lattice_range=2, minimum_range=2):
+    """Same result as ``frame_axes_max`` computed with whole-crystal tensor operations (used where
+    the Python loops would be too slow; tests check the two against each other).  ``argmax`` returns
+    the first maximal index, which is the tie rule wanted."""
+    dt = a_ih.dtype
+    N, H = a_ih.shape
+    R = translation_ranges(a_ih, rvlen, batch, cutoff_radius, lattice_range, minimum_range)
+    sizes = torch.bincount(batch, minlength=tvecs.shape[0]).tolist()
+    f1 = torch.zeros(N, H, 3, dtype=dt)
+    f2 = torch.zeros(N, H, 3, dtype=dt)
+    n_off = e_off = 0
+    big = torch.tensor(float("inf"), dtype=dt)
+    for b, nb in enumerate(sizes):
+        if nb == 0:
+            continue
+        sl_n = slice(n_off, n_off + nb)
+        sl_e = slice(e_off, e_off + nb * nb)
+        Rb = R[sl_n]
+        gi, gf = _grid(Rb.reshape(-1, 3).max(0).values.tolist(), dt)
+        T = gi.shape[0]
+        shift = gf @ tvecs[b].to(dt)
+        delta = rpos[sl_e].to(dt)[:, None, :] + shift[None]                 # (e,T,3)
+        d2 = (delta * delta).sum(-1)                                        # (e,T)
+        inbox = (gi.abs()[None, None] <= Rb[:, :, None, :]).all(-1).repeat_interleave(nb, dim=0)  # (e,H,T)
+        ok = inbox & (d2 > 1e-5)[:, None, :]
+        a_e = a_ih[sl_n].repeat_interleave(nb, dim=0)                       # (e,H)
+        js = edges[1, sl_e]
+        i_of_e = edges[0, sl_e]
+        qk = (q[i_of_e].to(dt) * k[js].to(dt)).sum(-1)                      # (e,H)
+        d2m = torch.where(ok, d2[:, None, :].expand(-1, H, -1), big)
+        d2min = d2m.min(-1).values                                          # (e,H)
+        tmin = (d2m == d2min[..., None]).to(torch.int8).argmax(-1)          # first minimum
+        score1 = (qk + a_e * d2min).reshape(nb, nb, H)
+        j1 = score1.argmax(1)                                               # (nb,H) first maximum
+        e1 = torch.arange(nb)[:, None] * nb + j1                            # local edge index
+        v1 = delta[e1, tmin[e1, torch.arange(H)[None, :]]]                  # (nb,H,3)
+        f1b = v1 / v1.norm(dim=-1, keepdim=True)
+        f1[sl_n] = f1b
+        dsafe = torch.sqrt(torch.where(d2 > 1e-5, d2, torch.ones_like(d2)))
+        unit = delta / dsafe[..., None]                                     # (e,T,3)
+        cosv = torch.einsum("etx,ehx->eht", unit, f1b.repeat_interleave(nb, dim=0))
+        val = a_e[..., None] * (d2[:, None, :] - d2min[..., None]) + torch.log(torch.clamp(1 - cosv.abs(), min=1e-5))
+        val = torch.where(ok & (cosv.abs() < 0.9999), val, -big)
+        best_t = (val == val.max(-1, keepdim=True).values).to(torch.int8).argmax(-1)   # (e,H)
+        best_v = val.max(-1).values + a_e * d2min
+        score2 = (qk + best_v).reshape(nb, nb, H)
+        j2 = score2.argmax(1)
+        e2 = torch.arange(nb)[:, None] * nb + j2
+        f2[sl_n] = unit[e2, best_t[e2, torch.arange(H)[None, :]]]
+        n_off += nb
+        e_off += nb * nb
     return f1, f2
 
 
