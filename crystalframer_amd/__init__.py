@@ -9,6 +9,9 @@ from .cuda_funcs import (  # noqa: F401
     CUPY_AVAILABLE,
     ComputeFrame1MaximumMethodCUDA,
     ComputeFrame2MaximumMethodCUDA,
+    ComputeFramesMaximumMethodCUDA,
+    FusedDotProductAttentionCUDA,
+    IrregularMeanCUDA,
     KernelManager,
     RealEncodingWithFramedProjFuncCUDA,
     compile_kernels,
@@ -16,5 +19,6 @@ from .cuda_funcs import (  # noqa: F401
 
 __all__ = [
     "CUPY_AVAILABLE", "ComputeFrame1MaximumMethodCUDA", "ComputeFrame2MaximumMethodCUDA",
+    "ComputeFramesMaximumMethodCUDA", "FusedDotProductAttentionCUDA", "IrregularMeanCUDA",
     "KernelManager", "RealEncodingWithFramedProjFuncCUDA", "compile_kernels",
 ]

@@ -46,7 +46,7 @@ class CfhParams(ctypes.Structure):
 
 
 EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_frame_axis1",
-           "cfh_frame_axis2", "cfh_framed_pe_forward", "cfh_framed_pe_backward")
+           "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_backward")
 
 _lib = None
 _lock = threading.Lock()
@@ -79,6 +79,8 @@ def load():
         lib.cfh_frame_axis1.argtypes = [pp] + [_P] * 10 + [_I64] * 3 + [_P, _P, ctypes.c_size_t, _P]
         lib.cfh_frame_axis2.restype = ctypes.c_int
         lib.cfh_frame_axis2.argtypes = [pp] + [_P] * 11 + [_I64] * 3 + [_P, _P, ctypes.c_size_t, _P]
+        lib.cfh_frame_axes.restype = ctypes.c_int
+        lib.cfh_frame_axes.argtypes = [pp] + [_P] * 10 + [_I64] * 3 + [_P, _P, ctypes.c_size_t, _P]
         lib.cfh_framed_pe_forward.restype = ctypes.c_int
         lib.cfh_framed_pe_forward.argtypes = [pp] + [_P] * 13 + [_I64] * 3 + [_P] * 4 + [ctypes.c_size_t, _P]
         lib.cfh_framed_pe_backward.restype = ctypes.c_int

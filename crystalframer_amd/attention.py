@@ -21,6 +21,9 @@ from . import cuda_funcs
 from .params import LatticeformerParams
 
 
+FUSED_FRAMES = True      # one launch for both axes + orthogonalisation (False: the reference's three steps)
+
+
 def compute_frame_maximum_method_(q, k, v, alpha, pos, dist2_min, tvecs, batch, edges, proj, K: int,
                                   dist_max: float, wscale: float, frame_method: str, this_epoch=None,
                                   rvecs: Optional[Tensor] = None, cutoff: Optional[float] = None):
@@ -33,6 +36,10 @@ def compute_frame_maximum_method_(q, k, v, alpha, pos, dist2_min, tvecs, batch, 
     q = q / math.sqrt(q.shape[-1])
     if frame_method != "max":
         raise NotImplementedError(f"frame_method={frame_method!r}: only 'max' is implemented")
+    if FUSED_FRAMES:
+        frames = cuda_funcs.ComputeFramesMaximumMethodCUDA.apply(
+            q, k, v, alpha, pos, dist2_min, tvecs, batch, edges, K, dist_max, wscale, *adap)
+        return frames[0], frames[1], frames[2]
     frame1 = cuda_funcs.ComputeFrame1MaximumMethodCUDA.apply(
         q, k, v, alpha, pos, dist2_min, tvecs, batch, edges, K, dist_max, wscale, *adap)
     frame2_max = cuda_funcs.ComputeFrame2MaximumMethodCUDA.apply(

@@ -28,11 +28,9 @@ int fail(int code, const char* fmt, ...) {
 }
 
 constexpr int MAX_HEADS = 64;
-constexpr size_t COUNTER_BYTES = 512;          // MAX_HEADS int32 work-queue heads, then 32 uint64 statistics
+constexpr size_t COUNTER_BYTES = 512;          // workspace header: 256 reserved bytes, then 32 uint64 statistics
 constexpr size_t STATS_OFFSET = 256;
 constexpr int WAVES_PER_SIMD = 3;
-
-__global__ void reset_counters_kernel(int32_t* counters) { counters[threadIdx.x] = 0; }
 
 // number of compute units of the current device (cached per device)
 int device_cus() {
@@ -47,7 +45,8 @@ int device_cus() {
     return cus[dev];
 }
 
-// persistent wavefronts to launch: a multiple of H, enough to fill the device, no more than items
+// upper bound of the persistent wavefronts of a launch (sizes the workspace): a multiple of H, no
+// more than there are items
 int launch_waves(int64_t N, int H) {
     int cus = device_cus();
     if (cus <= 0) cus = 256;
@@ -171,10 +170,28 @@ int finish_launch(const char* what) {
     return CFH_OK;
 }
 
+// Wavefronts that are resident at once for this kernel on the current device.  Work is dealt to
+// wavefronts statically, so launching more than fit would run them in a second wave of blocks and
+// double the makespan.
 template <typename Kern>
-int launch_persistent(Kern kern, const cfh::KernelArgs& A, int waves, hipStream_t st, const char* what) {
-    hipLaunchKernelGGL(reset_counters_kernel, dim3(1), dim3(MAX_HEADS), 0, st, A.counters);
-    hipLaunchKernelGGL(kern, dim3(waves), dim3(cfh::WAVE), 0, st, A);
+int resident_waves(Kern kern, int cap, int H) {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, cfh::WAVE, 0) != hipSuccess || per_cu < 1)
+        per_cu = 4;
+    int cus = device_cus();
+    if (cus <= 0) cus = 256;
+    int64_t want = (int64_t)cus * per_cu;
+    if (want > cap) want = cap;
+    want = (want / H) * H;
+    if (want < H) want = H;
+    return (int)want;
+}
+
+// `waves`: in = upper bound, out = wavefronts actually launched
+template <typename Kern>
+int launch_persistent(Kern kern, const cfh::KernelArgs& A, int* waves, hipStream_t st, const char* what) {
+    *waves = resident_waves(kern, *waves, A.H);
+    hipLaunchKernelGGL(kern, dim3(*waves), dim3(cfh::WAVE), 0, st, A);
     return finish_launch(what);
 }
 
@@ -207,8 +224,8 @@ int cfh_frame_axis1(const cfh_params* p, const float* q, const float* k, const f
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.q = q; A.k = k; A.out_frame = frame1;
-    return launch_persistent(cfh::frame_axis_kernel<false>, A, launch_waves(N, p->num_heads),
-                             (hipStream_t)stream, "frame_axis1");
+    int waves = launch_waves(N, p->num_heads);
+    return launch_persistent(cfh::frame_axis_kernel<0>, A, &waves, (hipStream_t)stream, "frame_axis1");
 }
 
 int cfh_frame_axis2(const cfh_params* p, const float* q, const float* k, const float* a_ih,
@@ -225,18 +242,36 @@ int cfh_frame_axis2(const cfh_params* p, const float* q, const float* k, const f
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.q = q; A.k = k; A.frame1 = frame1; A.out_frame = frame2max;
-    return launch_persistent(cfh::frame_axis_kernel<true>, A, launch_waves(N, p->num_heads),
-                             (hipStream_t)stream, "frame_axis2");
+    int waves = launch_waves(N, p->num_heads);
+    return launch_persistent(cfh::frame_axis_kernel<1>, A, &waves, (hipStream_t)stream, "frame_axis2");
+}
+
+int cfh_frame_axes(const cfh_params* p, const float* q, const float* k, const float* a_ih,
+                   const float* rpos, const float* tvecs, const float* rvlen, const int64_t* batch,
+                   const int64_t* edges, const int64_t* e_start, const int32_t* order, int64_t N,
+                   int64_t E, int64_t B, float* frames, void* workspace, size_t workspace_bytes,
+                   void* stream) {
+    int rc = check_params(p);
+    if (rc) return rc;
+    if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
+    if (N == 0) return CFH_OK;
+    if (!q || !k || !frames) return fail(CFH_EINVAL, "q, k and frames must not be NULL");
+    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES))) return rc;
+    cfh::KernelArgs A;
+    fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
+    A.q = q; A.k = k; A.out_frame = frames;
+    int waves = launch_waves(N, p->num_heads);
+    return launch_persistent(cfh::frame_axis_kernel<2>, A, &waves, (hipStream_t)stream, "frame_axes");
 }
 
 #define CFH_DISPATCH_PE(KERNEL, HAS_LEN, HAS_ANG)                                                   \
     do {                                                                                            \
         if (wide) {                                                                                 \
-            if (p->cos_abs) rc = launch_persistent(KERNEL<11, 41, true, HAS_LEN, HAS_ANG>, A, waves, st, what);  \
-            else rc = launch_persistent(KERNEL<11, 41, false, HAS_LEN, HAS_ANG>, A, waves, st, what);            \
+            if (p->cos_abs) rc = launch_persistent(KERNEL<11, 41, true, HAS_LEN, HAS_ANG>, A, &waves, st, what);  \
+            else rc = launch_persistent(KERNEL<11, 41, false, HAS_LEN, HAS_ANG>, A, &waves, st, what);            \
         } else {                                                                                    \
-            if (p->cos_abs) rc = launch_persistent(KERNEL<9, 33, true, HAS_LEN, HAS_ANG>, A, waves, st, what);   \
-            else rc = launch_persistent(KERNEL<9, 33, false, HAS_LEN, HAS_ANG>, A, waves, st, what);             \
+            if (p->cos_abs) rc = launch_persistent(KERNEL<9, 33, true, HAS_LEN, HAS_ANG>, A, &waves, st, what);   \
+            else rc = launch_persistent(KERNEL<9, 33, false, HAS_LEN, HAS_ANG>, A, &waves, st, what);             \
         }                                                                                           \
     } while (0)
 
@@ -264,13 +299,13 @@ int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* r
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.W[0] = W_dist; A.W[1] = W_axis1; A.W[2] = W_axis2; A.W[3] = W_axis3;
     A.frames = frames; A.out_z = z; A.out_psi = psi; A.out_d2min = d2min_out;
-    const int waves = launch_waves(N, p->num_heads);
+    int waves = launch_waves(N, p->num_heads);
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     hipStream_t st = (hipStream_t)stream;
     const char* what = "framed_pe_forward";
     if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_fwd_kernel, true, true);
     else if (has_len) CFH_DISPATCH_PE(cfh::framed_pe_fwd_kernel, true, false);
-    else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, false, false>, A, waves, st, what);
+    else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, false, false>, A, &waves, st, what);
     return rc;
 }
 
@@ -301,7 +336,7 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
         return fail(CFH_EINVAL, "W_axis1..3 and frames must be given together");
     int wl = 0, wa = 0;
     if ((rc = window_widths(p, &wl, &wa))) return rc;
-    const int waves = launch_waves(N, p->num_heads);
+    int waves = launch_waves(N, p->num_heads);
     const size_t need = COUNTER_BYTES + (size_t)waves * 4 * cfh::DH * cfh::NBINS * sizeof(float);
     if ((rc = check_workspace(workspace, workspace_bytes, need))) return rc;
     cfh::KernelArgs A;
@@ -313,13 +348,18 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
     const char* what = "framed_pe_backward";
     if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, true);
     else if (has_len) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, false);
-    else rc = launch_persistent(cfh::framed_pe_bwd_kernel<9, 33, false, false, false>, A, waves, st, what);
+    else rc = launch_persistent(cfh::framed_pe_bwd_kernel<9, 33, false, false, false>, A, &waves, st, what);
     if (rc) return rc;
     if (has_len) {
         const int nenc = has_ang ? 4 : 1;
-        const int total = nenc * p->num_heads * cfh::DH * cfh::NBINS;
-        hipLaunchKernelGGL(cfh::gw_reduce_kernel, dim3((total + 255) / 256), dim3(256), 0, st, A.gw_partial,
-                           waves, p->num_heads, nenc, gW_dist, gW_axis1, gW_axis2, gW_axis3);
+        const int per_enc = p->num_heads * cfh::DH * cfh::NBINS;
+        const int total = nenc * per_enc;
+        const int nslices = 16;
+        hipLaunchKernelGGL(cfh::zero_outputs_kernel, dim3((per_enc + 255) / 256), dim3(256), 0, st, per_enc,
+                           gW_dist, nenc > 1 ? gW_axis1 : nullptr, nenc > 1 ? gW_axis2 : nullptr,
+                           nenc > 1 ? gW_axis3 : nullptr);
+        hipLaunchKernelGGL(cfh::gw_reduce_kernel, dim3((total + 255) / 256, nslices), dim3(256), 0, st,
+                           A.gw_partial, waves, p->num_heads, nenc, nslices, gW_dist, gW_axis1, gW_axis2, gW_axis3);
         rc = finish_launch("gw_reduce");
     }
     return rc;

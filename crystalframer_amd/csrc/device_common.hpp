@@ -154,13 +154,23 @@ __device__ __forceinline__ WindowSeed window_seed(float beta_c, float sig, float
 // a ds_add_f32 costs 190-260 whatever the addresses (the float adder takes the lanes one at a time),
 // so float atomics are not usable in an inner loop.  The quantities accumulated are
 // softmax-normalised weights times Gaussians, so every bin stays within [0, 1]; one unit in the last
-// place is 4.7e-10, finer than a float32 accumulator.  Lanes spread over NREP replicas of the
-// histogram (lane & (NREP-1)), shifted by 4 banks each, which divides same-address collisions of
-// lanes whose windows coincide (clamped windows at the ends of the cosine range).
-constexpr int NREP = 8;
-constexpr int REP_STRIDE = 4 * HS + 4;            // words between replicas: 4 rows + a 4-bank shift
+// place is 4.7e-10, finer than a float32 accumulator.
+//
+// Pairs (i,j) of one (atom, head) item are processed GROUP at a time: the translations that
+// survive pruning are compacted for the whole group into one LDS list (entry = pair-in-group and
+// table index), and the heavy pass runs over that list 64 entries per step, so its lanes stay full
+// although a single pair keeps only ~17 translations on average.  Each pair of the group has its own
+// 4 x 64 histogram; a batch takes every nb-th entry of the list (nb = number of batches), so its
+// lanes come from all pairs of the group, which also spreads the same-address collisions of clamped
+// windows (cosines near +-1 all use the windows [0,W) or [64-W,64)).
+constexpr int GROUP = 8;                           // pairs per group (forward)
+constexpr int GROUP_BWD = 4;                       // pairs per group (backward: also holds G per pair)
+constexpr int GROUP_BITS = 3;
+constexpr int LISTCAP = 1024;                      // list entries (>= TCAP: one pair's chunk always fits)
+constexpr int PAIR_STRIDE = 4 * HS + 4;            // words between the histograms of two pairs (+4 banks)
 constexpr float FIX_ONE = 2147483648.0f;          // 2^31
 constexpr float FIX_INV = 1.0f / 2147483648.0f;
+static_assert(TCAP <= (1 << (16 - GROUP_BITS)) && GROUP <= (1 << GROUP_BITS), "list entry is 16 bits");
 
 template <int W>
 __device__ __forceinline__ void window_scatter(uint32_t* base, const WindowSeed& s, float cc) {
@@ -190,14 +200,10 @@ __device__ __forceinline__ float window_scatter_gather(uint32_t* hbase, const fl
     return acc;
 }
 
-// Sum the NREP replicas of histogram word `idx` (idx < 4*HS), clear them, return the float value.
+// Read histogram word `idx` as a float in [0,1] and clear it.
 __device__ __forceinline__ float take_bin(uint32_t* hist, int idx) {
-    uint32_t s = 0;
-#pragma unroll
-    for (int r = 0; r < NREP; r++) {
-        s += hist[r * REP_STRIDE + idx];
-        hist[r * REP_STRIDE + idx] = 0u;
-    }
+    const uint32_t s = hist[idx];
+    hist[idx] = 0u;
     return (float)s * FIX_INV;
 }
 
@@ -240,18 +246,13 @@ struct KernelArgs {
     BasisConsts bc;
 };
 
-// Next work item of this wavefront's head: one lane takes it from the counter, all lanes get it.
-// The electing lane id passes through an empty asm so that the compiler cannot relate this branch
-// to the `if (lane == 0)` stores at the tail of the persistent loop: when it can, it threads the two
-// branches together across the back edge, lanes 1..63 re-enter the loop apart from lane 0 (reading
-// item 0 from the readfirstlane below), and the wavefront never leaves the loop.
-__device__ __forceinline__ int next_item(int32_t* counter, int lane) {
-    int elect = lane;
-    asm volatile("" : "+v"(elect));
-    int it = 0;
-    if (elect == 0) it = atomicAdd(counter, 1);
-    return uniform_i(it);
-}
+// Work distribution.  Wavefront w (= blockIdx.x) serves head w % H and visits the items
+// w / H, w / H + W, w / H + 2 W, ... of that head, W = gridDim.x / H wavefronts per head.  Items are
+// visited in `order` (atoms by descending neighbour count), so every round hands all wavefronts
+// items of nearly equal cost.  A shared counter per head (one global atomic per item) was measured
+// first: the 19 000 same-address atomics of a launch serialise in L2 and cost more than the work.
+__device__ __forceinline__ int first_item(int H) { return (int)blockIdx.x / H; }
+__device__ __forceinline__ int item_stride(int H) { return (int)gridDim.x / H; }
 
 // Counter-based uniform in [0,1) for the optional tie-breaking noise of the frame search.
 __device__ __forceinline__ float hash_uniform(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {

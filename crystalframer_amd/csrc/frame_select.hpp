@@ -7,10 +7,17 @@
 //  models/kernels/compute_second_frame_each_edge.cu:81-142,
 //  models/cuda_funcs/calc_maximum_frame.py:72-86,146-164).
 //
-// Tie rule with zero noise: per pair the first image in the reference's loop order wins (its
-// strict comparisons), across pairs the lowest edge index wins.  With noise > 0 every candidate's
-// key is perturbed by a counter-based uniform in (-noise/2, noise/2) (the reference draws from
-// cuRAND XORWOW seeded by numpy; its stream cannot be reproduced).
+// Both searches are arg-maxima over (j, n) of one expression -- q_i.k_j + a d^2 for the first axis
+// (for a < 0 the nearest image of a neighbour is also its best), q_i.k_j + a d^2 + log(max(1-|cos|,
+// 1e-5)) for the second -- so every lane keeps a running best over its own translations of every
+// pair and the wavefront reduces once per item.  Tie rule with zero noise: lowest pair index, then
+// first translation in the reference's loop order (what its strict comparisons and the plain
+// arg-max over pairs give).  With noise > 0 every candidate's key is perturbed by a counter-based
+// uniform in (-noise/2, noise/2) (the reference draws from cuRAND XORWOW seeded by numpy; its
+// stream cannot be reproduced).
+//
+// MODE 0: first axis only.  MODE 1: second axis for a given first axis.  MODE 2: both, then
+// Gram-Schmidt and the cross product, written as (3,N,H,3) orthonormal frames.
 #pragma once
 #include "device_common.hpp"
 
@@ -28,17 +35,30 @@ __device__ __forceinline__ void shift_of(int t, const Box& bx, const Lattice& L,
     vz = fmaf(L.t[8], n3, fmaf(L.t[5], n2, L.t[2] * n1));
 }
 
-template <bool SECOND>
+// best candidate of a wavefront: largest score, then lowest pair, then lowest translation
+struct Best { float score; int e; int t; };
+__device__ __forceinline__ void wave_best(Best& b) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float os = __shfl_xor(b.score, o, WAVE);
+        const int oe = __shfl_xor(b.e, o, WAVE);
+        const int ot = __shfl_xor(b.t, o, WAVE);
+        if (os > b.score || (os == b.score && (oe < b.e || (oe == b.e && ot < b.t)))) {
+            b.score = os; b.e = oe; b.t = ot;
+        }
+    }
+}
+
+template <int MODE>
 __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
     __shared__ float4 tab[TCAP];
+    __shared__ float4 pair_rq[WAVE];        // rpos and q.k of up to 64 pairs
     const int lane = threadIdx.x;
     const int H = P.H;
     const int h = blockIdx.x % H;
     const bool noisy = P.noise > 0.0f;
 
-    for (;;) {
-        const int it = next_item(P.counters + h, lane);
-        if (it >= P.N) break;
+    for (int it = first_item(H); it < P.N; it += item_stride(H)) {
         const int i = P.order ? uniform_i(P.order[it]) : it;
         const int b = uniform_i((int)P.batch[i]);
         const float a = uniform_f(P.a_ih[(size_t)i * H + h]);
@@ -56,12 +76,6 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
         float qi[DH];
 #pragma unroll
         for (int c = 0; c < DH; c++) qi[c] = uniform_f(P.q[((size_t)i * H + h) * DH + c]);
-        float f1x = 0.f, f1y = 0.f, f1z = 0.f;
-        if (SECOND) {
-            f1x = uniform_f(P.frame1[((size_t)i * H + h) * 3 + 0]);
-            f1y = uniform_f(P.frame1[((size_t)i * H + h) * 3 + 1]);
-            f1z = uniform_f(P.frame1[((size_t)i * H + h) * 3 + 2]);
-        }
         const int nchunks = (bx.T + TCAP - 1) / TCAP;
         if (nchunks == 1) {
             __syncthreads();
@@ -71,35 +85,39 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
         const int e0 = uniform_i((int)P.e_start[i]);
         const int e1 = uniform_i((int)P.e_start[i + 1]);
 
-        float best_score = -3.0e38f;
-        float bx_ = 0.f, by_ = 0.f, bz_ = 0.f;      // best direction (unnormalised image vector)
+        float f1x = 0.f, f1y = 0.f, f1z = 0.f;     // first axis (input in MODE 1, result otherwise)
+        float f2x = 0.f, f2y = 0.f, f2z = 0.f;     // second axis before orthogonalisation
+        if (MODE == 1) {
+            f1x = uniform_f(P.frame1[((size_t)i * H + h) * 3 + 0]);
+            f1y = uniform_f(P.frame1[((size_t)i * H + h) * 3 + 1]);
+            f1z = uniform_f(P.frame1[((size_t)i * H + h) * 3 + 2]);
+        }
 
-        for (int eb = e0; eb < e1; eb += WAVE) {
-            // q_i . k_j for up to 64 neighbours, one per lane
-            float qk_lane = 0.0f;
-            if (eb + lane < e1) {
-                const int64_t j = P.edges[(size_t)P.E + eb + lane];
-                const float4* kp = reinterpret_cast<const float4*>(P.k + ((size_t)j * H + h) * DH);
+        // pass 0 searches the first axis, pass 1 the second
+        for (int pass = (MODE == 1 ? 1 : 0); pass < (MODE == 0 ? 1 : 2); pass++) {
+            Best best;
+            best.score = -3.0e38f; best.e = 0x7fffffff; best.t = 0x7fffffff;
+            for (int eb = e0; eb < e1; eb += WAVE) {
+                // stage rpos and q_i.k_j of up to 64 pairs, one per lane
+                __syncthreads();
+                if (eb + lane < e1) {
+                    const int e = eb + lane;
+                    const int64_t j = P.edges[(size_t)P.E + e];
+                    const float4* kp = reinterpret_cast<const float4*>(P.k + ((size_t)j * H + h) * DH);
+                    float qk = 0.0f;
 #pragma unroll
-                for (int c4 = 0; c4 < DH / 4; c4++) {
-                    const float4 kv = kp[c4];
-                    qk_lane = fmaf(qi[4 * c4 + 0], kv.x, qk_lane);
-                    qk_lane = fmaf(qi[4 * c4 + 1], kv.y, qk_lane);
-                    qk_lane = fmaf(qi[4 * c4 + 2], kv.z, qk_lane);
-                    qk_lane = fmaf(qi[4 * c4 + 3], kv.w, qk_lane);
+                    for (int c4 = 0; c4 < DH / 4; c4++) {
+                        const float4 kv = kp[c4];
+                        qk = fmaf(qi[4 * c4 + 0], kv.x, qk);
+                        qk = fmaf(qi[4 * c4 + 1], kv.y, qk);
+                        qk = fmaf(qi[4 * c4 + 2], kv.z, qk);
+                        qk = fmaf(qi[4 * c4 + 3], kv.w, qk);
+                    }
+                    pair_rq[lane] = make_float4(P.rpos[(size_t)e * 3 + 0], P.rpos[(size_t)e * 3 + 1],
+                                                P.rpos[(size_t)e * 3 + 2], qk);
                 }
-            }
-            const int ne = min(WAVE, e1 - eb);
-            for (int el = 0; el < ne; el++) {
-                const int e = eb + el;
-                const float qk = __shfl(qk_lane, el, WAVE);
-                const float rx = uniform_f(P.rpos[(size_t)e * 3 + 0]);
-                const float ry = uniform_f(P.rpos[(size_t)e * 3 + 1]);
-                const float rz = uniform_f(P.rpos[(size_t)e * 3 + 2]);
-
-                // ---- nearest image with d^2 > 1e-5 (first in loop order on ties)
-                float bd = 3.0e38f;
-                int bt = 0x7fffffff;
+                __syncthreads();
+                const int ne = min(WAVE, e1 - eb);
                 for (int ch = 0; ch < nchunks; ch++) {
                     const int t0 = ch * TCAP;
                     const int cnt = min(TCAP, bx.T - t0);
@@ -108,73 +126,77 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                         build_shift_table(tab, t0, cnt, bx, L, lane);
                         __syncthreads();
                     }
-                    for (int u = lane; u < cnt; u += WAVE) {
-                        const float4 v = tab[u];
-                        const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
-                        const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
-                        float key = d2;
-                        if (noisy && !SECOND)
-                            key += (hash_uniform(P.seed_lo, P.seed_hi, (uint32_t)(e * H + h), (uint32_t)(t0 + u)) - 0.5f) * P.noise;
-                        if (d2 > 1e-5f && key < bd) { bd = key; bt = t0 + u; }
-                    }
-                }
-                wave_argmin(bd, bt);
-                if (bt == 0x7fffffff) continue;      // no image at all: cannot happen for R >= 1
-
-                if (!SECOND) {
-                    const float score = qk + a * bd;
-                    if (score > best_score) {
-                        best_score = score;
-                        float vx, vy, vz;
-                        shift_of(bt, bx, L, vx, vy, vz);
-                        bx_ = rx + vx; by_ = ry + vy; bz_ = rz + vz;
-                    }
-                } else {
-                    const float d2min = bd;
-                    float bv = -3.0e38f;
-                    int bt2 = 0x7fffffff;
-                    for (int ch = 0; ch < nchunks; ch++) {
-                        const int t0 = ch * TCAP;
-                        const int cnt = min(TCAP, bx.T - t0);
-                        if (nchunks > 1) {
-                            __syncthreads();
-                            build_shift_table(tab, t0, cnt, bx, L, lane);
-                            __syncthreads();
-                        }
+                    for (int el = 0; el < ne; el++) {
+                        const float4 rq = pair_rq[el];
+                        const int e = eb + el;
                         for (int u = lane; u < cnt; u += WAVE) {
                             const float4 v = tab[u];
-                            const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                            const float dx = rq.x + v.x, dy = rq.y + v.y, dz = rq.z + v.z;
                             const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
-                            if (d2 > 1e-5f) {
+                            float d2k = d2;
+                            if (noisy && pass == 0)
+                                d2k += (hash_uniform(P.seed_lo, P.seed_hi, (uint32_t)(e * H + h), (uint32_t)(t0 + u)) - 0.5f) * P.noise;
+                            float score = fmaf(a, d2k, rq.w);
+                            bool ok = d2 > 1e-5f;
+                            if (pass == 1) {
                                 const float rinv = hw_rsq(d2);
                                 const float ac = fabsf((dx * f1x + dy * f1y + dz * f1z) * rinv);
-                                float val = a * (d2 - d2min) + hw_log2(fmaxf(1.0f - ac, 1e-5f)) * LN2;
+                                score += hw_log2(fmaxf(1.0f - ac, 1e-5f)) * LN2;
                                 if (noisy)
-                                    val += (hash_uniform(P.seed_lo, P.seed_hi, (uint32_t)(e * H + h), (uint32_t)(t0 + u)) - 0.5f) * P.noise;
-                                if (ac < 0.9999f && val > bv) { bv = val; bt2 = t0 + u; }
+                                    score += (hash_uniform(P.seed_hi, P.seed_lo, (uint32_t)(e * H + h), (uint32_t)(t0 + u)) - 0.5f) * P.noise;
+                                ok = ok && ac < 0.9999f;
+                            }
+                            // a lane meets its candidates in ascending (e, t) order when the table is
+                            // one chunk: the strict comparison keeps the first; with several chunks the
+                            // explicit (e, t) comparison does
+                            if (ok && (score > best.score ||
+                                       (score == best.score && (e < best.e || (e == best.e && t0 + u < best.t))))) {
+                                best.score = score; best.e = e; best.t = t0 + u;
                             }
                         }
                     }
-                    wave_argmax(bv, bt2);
-                    if (bt2 == 0x7fffffff) continue;  // every image collinear with the first axis
-                    const float score = qk + (bv + a * d2min);
-                    if (score > best_score) {
-                        best_score = score;
-                        float vx, vy, vz;
-                        shift_of(bt2, bx, L, vx, vy, vz);
-                        bx_ = rx + vx; by_ = ry + vy; bz_ = rz + vz;
-                    }
                 }
             }
+            wave_best(best);
+            float vx = 0.f, vy = 0.f, vz = 0.f;
+            if (best.e != 0x7fffffff) {
+                float sx, sy, sz;
+                shift_of(best.t, bx, L, sx, sy, sz);
+                vx = uniform_f(P.rpos[(size_t)best.e * 3 + 0]) + sx;
+                vy = uniform_f(P.rpos[(size_t)best.e * 3 + 1]) + sy;
+                vz = uniform_f(P.rpos[(size_t)best.e * 3 + 2]) + sz;
+                const float inv = 1.0f / sqrtf(vx * vx + vy * vy + vz * vz);
+                vx *= inv; vy *= inv; vz *= inv;
+            }
+            if (pass == 0) { f1x = vx; f1y = vy; f1z = vz; }
+            else { f2x = vx; f2y = vy; f2z = vz; }
         }
+
         if (lane == 0) {
-            const float d2 = bx_ * bx_ + by_ * by_ + bz_ * bz_;
-            const float inv = d2 > 0.0f ? 1.0f / sqrtf(d2) : 0.0f;
-            float* o = P.out_frame + ((size_t)i * H + h) * 3;
-            o[0] = bx_ * inv; o[1] = by_ * inv; o[2] = bz_ * inv;
-            if (P.stats)
-                atomicAdd(P.stats + (SECOND ? STAT_FRAME2_RAW : STAT_FRAME1_RAW),
-                          (unsigned long long)bx.T * (unsigned long long)(e1 - e0));
+            if (MODE == 0 || MODE == 1) {
+                float* o = P.out_frame + ((size_t)i * H + h) * 3;
+                if (MODE == 0) { o[0] = f1x; o[1] = f1y; o[2] = f1z; }
+                else { o[0] = f2x; o[1] = f2y; o[2] = f2z; }
+            } else {
+                // Gram-Schmidt and cross product
+                // (models/indexed_lattice_multi_head_attention_cuda.py:475-481; F.normalize eps 1e-12)
+                const float dot = f1x * f2x + f1y * f2y + f1z * f2z;
+                float gx = f2x - dot * f1x, gy = f2y - dot * f1y, gz = f2z - dot * f1z;
+                const float inv = 1.0f / fmaxf(sqrtf(gx * gx + gy * gy + gz * gz), 1e-12f);
+                gx *= inv; gy *= inv; gz *= inv;
+                const size_t stride = (size_t)P.N * H * 3;
+                float* o = P.out_frame + ((size_t)i * H + h) * 3;
+                o[0] = f1x; o[1] = f1y; o[2] = f1z;
+                o[stride + 0] = gx; o[stride + 1] = gy; o[stride + 2] = gz;
+                o[2 * stride + 0] = f1y * gz - f1z * gy;
+                o[2 * stride + 1] = f1z * gx - f1x * gz;
+                o[2 * stride + 2] = f1x * gy - f1y * gx;
+            }
+            if (P.stats) {
+                const unsigned long long raw = (unsigned long long)bx.T * (unsigned long long)(e1 - e0);
+                if (MODE != 1) atomicAdd(P.stats + STAT_FRAME1_RAW, raw);
+                if (MODE != 0) atomicAdd(P.stats + STAT_FRAME2_RAW, raw);
+            }
         }
     }
 }

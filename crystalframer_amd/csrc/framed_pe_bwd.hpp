@@ -4,12 +4,15 @@
 // (models/kernels/real_enc_frame_proj_bwd_length.cu:100-237, ..._bwd_angle.cu:104-275) and the
 // sums around them (models/cuda_funcs/real_space_framed_proj.py:123-221).
 //
-// With p_n = exp(a d_n^2 - z) (recomputed, never stored), G_enc[k] = coef_enc sum_c W_enc[h,c,k] gpsi[c]
-// and bg_n = sum_enc sum_{k in window} g_k(x_enc,n) G_enc[k]:
-//   ga_ih   = sum_j [ gz sum_n p d^2 + sum_n p d^2 bg - (sum_n p d^2)(sum_n p bg) ]
+// With p_n = exp(a d_n^2 - z) (recomputed, never stored), G_enc[k] = coef_enc sum_c W_enc[h,c,k] gpsi[c],
+// bg_n = sum_enc sum_{k in window} g_k(x_enc,n) G_enc[k] and A0 = sum_n p_n d_n^2:
+//   ga_ih   = sum_j [ gz A0 + sum_n p_n (d_n^2 - A0) bg_n ]          (the reference's covariance form
+//             sum p d^2 bg - (sum p d^2)(sum p bg), written without the cancellation)
 //   gW_enc[h,c,k] = coef_enc sum_e gpsi[e,h,c] sum_n p g_k
-// Lane k of the wavefront keeps W_enc[h,:,k] and the running gW_enc[h,:,k] in registers for the
-// whole launch; partials are written once per wavefront and summed by gw_reduce_kernel, so no
+// Pairs are taken GROUP_BWD at a time: per pair a light sweep gives A0 and compacts the translations
+// that matter into the group's list, the heavy pass (window gather + scatter) runs over the list with
+// full lanes.  Lane k of the wavefront keeps W_enc[h,:,k] and the running gW_enc[h,:,k] in registers
+// for the whole launch; partials are written once per wavefront and summed by gw_reduce_kernel, so no
 // global atomics touch the weight gradients.
 #pragma once
 #include "device_common.hpp"
@@ -19,15 +22,17 @@ namespace cfh {
 template <int WL, int WA, bool COS_ABS, bool HAS_LEN, bool HAS_ANG>
 __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P) {
     __shared__ float4 tab[TCAP];
-    __shared__ uint16_t list[TCAP];
-    __shared__ uint32_t hist[NREP * REP_STRIDE];                  // fixed-point sum_n p g_k per encoder
-    __shared__ __attribute__((aligned(16))) float Gs[4 * HS];     // projected upstream gradient / 2^31
+    __shared__ uint16_t list[LISTCAP];
+    __shared__ uint32_t hist[GROUP_BWD * PAIR_STRIDE];                              // fixed-point sum_n p g_k
+    __shared__ __attribute__((aligned(16))) float Gs[GROUP_BWD * PAIR_STRIDE];      // G / 2^31 per pair
+    __shared__ __attribute__((aligned(16))) float gpS[GROUP_BWD * DH];              // gpsi of the pairs
+    __shared__ float4 pairA[GROUP_BWD];     // rx, ry, rz, A0
+    __shared__ float pairZ[GROUP_BWD];      // z * log2(e)
 
     constexpr int NENC = HAS_ANG ? 4 : (HAS_LEN ? 1 : 0);
     const int lane = threadIdx.x;
     const int H = P.H;
     const int h = blockIdx.x % H;
-    uint32_t* const myhist = hist + (lane & (NREP - 1)) * REP_STRIDE;
 
     // lane k: W_enc[h, c, k] for all (enc, c), and the gradient accumulators of the same shape
     float Wt[NENC > 0 ? NENC * DH : 1];
@@ -42,13 +47,10 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
     const BasisConsts bc = P.bc;
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
 
-    for (int u = lane; u < NREP * REP_STRIDE; u += WAVE) hist[u] = 0u;
-    for (int u = lane; u < 4 * HS; u += WAVE) Gs[u] = 0.0f;
+    for (int u = lane; u < GROUP_BWD * PAIR_STRIDE; u += WAVE) { hist[u] = 0u; Gs[u] = 0.0f; }
     __syncthreads();
 
-    for (;;) {
-        const int it = next_item(P.counters + h, lane);
-        if (it >= P.N) break;
+    for (int it = first_item(H); it < P.N; it += item_stride(H)) {
         const int i = P.order ? uniform_i(P.order[it]) : it;
         const int b = uniform_i((int)P.batch[i]);
         const float a = uniform_f(P.a_ih[(size_t)i * H + h]);
@@ -80,75 +82,37 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
         }
         const int e0 = uniform_i((int)P.e_start[i]);
         const int e1 = uniform_i((int)P.e_start[i + 1]);
-        float ga_acc = 0.0f;
+        float ga_acc = 0.0f;      // uniform part: sum_e gz A0
+        float cov = 0.0f;         // per lane: sum over its terms of p (d^2 - A0) bg
         unsigned long long n_eval = 0;
+        int nlist = 0;
 
-        for (int e = e0; e < e1; e++) {
-            const float rx = uniform_f(P.rpos[(size_t)e * 3 + 0]);
-            const float ry = uniform_f(P.rpos[(size_t)e * 3 + 1]);
-            const float rz = uniform_f(P.rpos[(size_t)e * 3 + 2]);
-            const float z2 = uniform_f(P.z[(size_t)e * H + h]) * LOG2E;
-            const float gz = uniform_f(P.gz[(size_t)e * H + h]);
-
-            // upstream gradient of psi, projected onto the bins:  G_enc[k] (this lane: k = lane)
-            float gp[DH];
-            if (NENC > 0) {
-#pragma unroll
-                for (int c = 0; c < DH; c++) gp[c] = uniform_f(P.gpsi[((size_t)e * H + h) * DH + c]);
-            }
-            __syncthreads();       // previous pair's reads of Gs are done
-#pragma unroll
-            for (int en = 0; en < NENC; en++) {
-                float g = 0.0f;
-#pragma unroll
-                for (int c = 0; c < DH; c++) g = fmaf(Wt[en * DH + c], gp[c], g);
-                Gs[en * HS + lane] = g * ((en == 0 ? P.dist_coef : P.angle_coef) * FIX_INV);
-            }
+        // heavy pass over the current list; the table the entries point into must still be resident
+        auto flush = [&]() {
             __syncthreads();
-
-            float A0 = 0.0f, A1 = 0.0f, A2 = 0.0f;   // sum p d^2, sum p d^2 bg, sum p bg
-            for (int ch = 0; ch < nchunks; ch++) {
-                const int t0 = ch * TCAP;
-                const int cnt = min(TCAP, bx.T - t0);
-                if (nchunks > 1) {
-                    __syncthreads();
-                    build_shift_table(tab, t0, cnt, bx, L, lane);
-                    __syncthreads();
-                }
-                int nkeep = 0;
-                for (int u0 = 0; u0 < cnt; u0 += WAVE) {
-                    const int u = u0 + lane;
-                    bool keep = false;
-                    if (u < cnt) {
-                        const float4 v = tab[u];
-                        const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+            if (NENC > 0) {
+                const int nb = (nlist + WAVE - 1) / WAVE;
+                for (int bt = 0; bt < nb; bt++) {
+                    const int idx = lane * nb + bt;
+                    if (idx < nlist) {
+                        const uint32_t ent = list[idx];
+                        const int el = ent >> (16 - GROUP_BITS);
+                        const float4 v = tab[ent & ((1u << (16 - GROUP_BITS)) - 1u)];
+                        const float4 pa = pairA[el];
+                        const float dx = pa.x + v.x, dy = pa.y + v.y, dz = pa.z + v.z;
                         const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
-                        const float ex = fmaf(a2, d2, -z2);
-                        keep = ex >= prune;
-                        if (!keep) A0 = fmaf(hw_exp2(ex), d2, A0);    // light terms still count in dz/da
-                    }
-                    const uint64_t m = __ballot(keep);
-                    if (keep) list[nkeep + lane_prefix(m)] = (uint16_t)u;
-                    nkeep += __popcll(m);
-                }
-                n_eval += (unsigned long long)nkeep;
-                __syncthreads();
-                for (int v0 = 0; v0 < nkeep; v0 += WAVE) {
-                    if (v0 + lane < nkeep) {
-                        const float4 v = tab[list[v0 + lane]];
-                        const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
-                        const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
-                        const float p = hw_exp2(fmaf(a2, d2, -z2));
-                        const float pf = p * FIX_ONE;
+                        const float pf = hw_exp2(fmaf(a2, d2, -pairZ[el])) * FIX_ONE;
+                        uint32_t* const myhist = hist + el * PAIR_STRIDE;
+                        const float* const myG = Gs + el * PAIR_STRIDE;
                         float pbg = 0.0f;
-                        if (HAS_LEN) {
+                        {
                             const float d = hw_sqrt(d2);
                             const float u = d * bc.inv_interval;
                             int start = (int)(u - bc.start_off);
                             start = max(0, min(start, NBINS - WL));
                             const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
                             const WindowSeed s = window_seed(beta_c, bc.len_step, pf);
-                            pbg += window_scatter_gather<WL>(myhist + start, Gs + start, s, bc.len_cc);
+                            pbg += window_scatter_gather<WL>(myhist + start, myG + start, s, bc.len_cc);
                         }
                         if (HAS_ANG) {
                             if (d2 > 1e-5f) {
@@ -165,30 +129,123 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
                                     const float beta_c = (mu_c - cs) * bc.ang_sigma_inv;
                                     const WindowSeed s = window_seed(beta_c, bc.ang_step, pf);
                                     pbg += window_scatter_gather<WA>(myhist + (ax + 1) * HS + start,
-                                                                     Gs + (ax + 1) * HS + start, s, bc.ang_cc);
+                                                                     myG + (ax + 1) * HS + start, s, bc.ang_cc);
                                 }
                             }
                         }
-                        A0 = fmaf(p, d2, A0);
-                        A1 = fmaf(d2, pbg, A1);
-                        A2 += pbg;
+                        cov = fmaf(d2 - pa.w, pbg, cov);
                     }
                 }
-                __syncthreads();
             }
-            A0 = wave_sum(A0); A1 = wave_sum(A1); A2 = wave_sum(A2);
-            ga_acc += P.gz_coef * gz * A0 + (A1 - A0 * A2);
+            n_eval += (unsigned long long)nlist;
+            nlist = 0;
+            __syncthreads();
+        };
+
+        for (int g0 = e0; g0 < e1; g0 += GROUP_BWD) {
+            const int ng = min(GROUP_BWD, e1 - g0);
+            // stage gpsi of the group's pairs (coalesced: 16 consecutive floats per pair)
+            if (NENC > 0 && lane < ng * DH) gpS[lane] = P.gpsi[((size_t)g0 * H) * DH + (size_t)(lane / DH) * H * DH + (size_t)h * DH + (lane % DH)];
+            __syncthreads();
+
+            for (int el = 0; el < ng; el++) {
+                const int e = g0 + el;
+                const float rx = uniform_f(P.rpos[(size_t)e * 3 + 0]);
+                const float ry = uniform_f(P.rpos[(size_t)e * 3 + 1]);
+                const float rz = uniform_f(P.rpos[(size_t)e * 3 + 2]);
+                const float z2 = uniform_f(P.z[(size_t)e * H + h]) * LOG2E;
+                const float gz = uniform_f(P.gz[(size_t)e * H + h]);
+
+                // upstream gradient of psi projected onto the bins: G_enc[k], this lane: k = lane
+                if (NENC > 0) {
+                    float gp[DH];
+#pragma unroll
+                    for (int c4 = 0; c4 < DH / 4; c4++) {
+                        const float4 t4 = reinterpret_cast<const float4*>(gpS + el * DH)[c4];
+                        gp[4 * c4 + 0] = t4.x; gp[4 * c4 + 1] = t4.y; gp[4 * c4 + 2] = t4.z; gp[4 * c4 + 3] = t4.w;
+                    }
+#pragma unroll
+                    for (int en = 0; en < NENC; en++) {
+                        float g = 0.0f;
+#pragma unroll
+                        for (int c = 0; c < DH; c++) g = fmaf(Wt[en * DH + c], gp[c], g);
+                        Gs[el * PAIR_STRIDE + en * HS + lane] = g * ((en == 0 ? P.dist_coef : P.angle_coef) * FIX_INV);
+                    }
+                }
+
+                // light sweep: A0 = sum_n p d^2 over every translation, compaction of those that matter
+                float A0 = 0.0f;
+                for (int ch = 0; ch < nchunks; ch++) {
+                    const int t0 = ch * TCAP;
+                    const int cnt = min(TCAP, bx.T - t0);
+                    if (nchunks > 1) {
+                        flush();
+                        build_shift_table(tab, t0, cnt, bx, L, lane);
+                        __syncthreads();
+                    }
+                    for (int u = lane; u < cnt; u += WAVE) {
+                        const float4 v = tab[u];
+                        const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                        const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+                        A0 = fmaf(hw_exp2(fmaf(a2, d2, -z2)), d2, A0);
+                    }
+                }
+                A0 = wave_sum(A0);
+                ga_acc = fmaf(P.gz_coef * gz, A0, ga_acc);
+                if (lane == 0) {
+                    pairA[el] = make_float4(rx, ry, rz, A0);
+                    pairZ[el] = z2;
+                }
+                for (int ch = 0; ch < nchunks; ch++) {
+                    const int t0 = ch * TCAP;
+                    const int cnt = min(TCAP, bx.T - t0);
+                    if (nchunks > 1) {
+                        __syncthreads();
+                        build_shift_table(tab, t0, cnt, bx, L, lane);
+                        __syncthreads();
+                    } else if (nlist + cnt > LISTCAP) {
+                        flush();
+                    }
+                    for (int u0 = 0; u0 < cnt; u0 += WAVE) {
+                        const int u = u0 + lane;
+                        bool keep = false;
+                        if (u < cnt) {
+                            const float4 v = tab[u];
+                            const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                            keep = fmaf(a2, fmaf(dx, dx, fmaf(dy, dy, dz * dz)), -z2) >= prune;
+                        }
+                        const uint64_t m = __ballot(keep);
+                        if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((el << (16 - GROUP_BITS)) | u);
+                        nlist += __popcll(m);
+                    }
+                    if (nchunks > 1) flush();
+                }
+            }
+            flush();
 
             // weight gradients: gW_enc[c] (lane k) += coef * gpsi[c] * s_enc[k]
+            if (NENC > 0) {
+                for (int el = 0; el < ng; el++) {
+                    float gp[DH];
 #pragma unroll
-            for (int en = 0; en < NENC; en++) {
-                const float sk = take_bin(hist, en * HS + lane) * (en == 0 ? P.gw_dist_coef : P.angle_coef);
+                    for (int c4 = 0; c4 < DH / 4; c4++) {
+                        const float4 t4 = reinterpret_cast<const float4*>(gpS + el * DH)[c4];
+                        gp[4 * c4 + 0] = t4.x; gp[4 * c4 + 1] = t4.y; gp[4 * c4 + 2] = t4.z; gp[4 * c4 + 3] = t4.w;
+                    }
 #pragma unroll
-                for (int c = 0; c < DH; c++) gW[en * DH + c] = fmaf(gp[c], sk, gW[en * DH + c]);
+                    for (int en = 0; en < NENC; en++) {
+                        const float sk = take_bin(hist + el * PAIR_STRIDE, en * HS + lane) *
+                                         (en == 0 ? P.gw_dist_coef : P.angle_coef);
+#pragma unroll
+                        for (int c = 0; c < DH; c++) gW[en * DH + c] = fmaf(gp[c], sk, gW[en * DH + c]);
+                    }
+                }
             }
+            __syncthreads();               // gpS, pair data and histograms are free again
         }
+        cov = wave_sum(cov);
         if (lane == 0) {
-            P.out_ga[(size_t)i * H + h] = ga_acc;
+            P.out_ga[(size_t)i * H + h] = ga_acc + cov;
             if (P.stats) {
                 atomicAdd(P.stats + STAT_BWD_EVAL, n_eval);
                 atomicAdd(P.stats + STAT_BWD_RAW, (unsigned long long)bx.T * (unsigned long long)(e1 - e0));
@@ -207,10 +264,11 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
     }
 }
 
-// gW_enc[h, c, k] = sum over the wavefronts w of head h (w % H == h) of partial[w, enc, c, k].
+// gW_enc[h, c, k] += sum over a slice of the wavefronts w of head h (w % H == h) of
+// partial[w, enc, c, k]; the outputs are cleared by zero_outputs_kernel first.
 __global__ __launch_bounds__(256) void gw_reduce_kernel(const float* __restrict__ partial, int nwaves,
-                                                        int H, int nenc, float* out0, float* out1,
-                                                        float* out2, float* out3) {
+                                                        int H, int nenc, int nslices, float* out0,
+                                                        float* out1, float* out2, float* out3) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;       // over (enc, h, c, k)
     const int per_enc = H * DH * NBINS;
     if (idx >= nenc * per_enc) return;
@@ -219,9 +277,20 @@ __global__ __launch_bounds__(256) void gw_reduce_kernel(const float* __restrict_
     const int h = rem / (DH * NBINS);
     const int ck = rem % (DH * NBINS);
     float s = 0.0f;
-    for (int w = h; w < nwaves; w += H) s += partial[((size_t)w * 4 + en) * DH * NBINS + ck];
+    for (int w = h + H * blockIdx.y; w < nwaves; w += H * nslices)
+        s += partial[((size_t)w * 4 + en) * DH * NBINS + ck];
     float* out = en == 0 ? out0 : (en == 1 ? out1 : (en == 2 ? out2 : out3));
-    if (out) out[rem] = s;
+    if (out) atomicAdd(out + rem, s);
+}
+
+__global__ __launch_bounds__(256) void zero_outputs_kernel(int n, float* out0, float* out1, float* out2,
+                                                           float* out3) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n) return;
+    if (out0) out0[idx] = 0.0f;
+    if (out1) out1[idx] = 0.0f;
+    if (out2) out2[idx] = 0.0f;
+    if (out3) out3[idx] = 0.0f;
 }
 
 }  // namespace cfh

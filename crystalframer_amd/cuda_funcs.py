@@ -155,8 +155,10 @@ def _proj_weight(W: Optional[torch.Tensor], H: int, what: str) -> Optional[torch
     return _f32c(W)
 
 
-def _frame_call(second: bool, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, frame1, rvlen_n,
+def _frame_call(mode: int, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, frame1, rvlen_n,
                 cutoff_radius):
+    """mode 0: first axis (N,H,3); 1: second axis given the first; 2: orthonormal frames (3,N,H,3)."""
+    second = mode == 1
     _lib.require_gpu(q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e)
     lib = _lib.load()
     N, H = a_ik.shape
@@ -168,13 +170,18 @@ def _frame_call(second: bool, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e
     rv = _f32c(rvlen_n)
     batch, edges = batch_i.contiguous(), edge_ij_e.contiguous()
     e_start, order = edge_schedule(edge_ij_e, N)
-    out = torch.zeros((N, H, 3), dtype=torch.float32, device=dev)
+    out = torch.zeros((3, N, H, 3) if mode == 2 else (N, H, 3), dtype=torch.float32, device=dev)
     p = _params(H, Dh, 0, 0, 0, 1.0, 1.0, 1.0, 1.0, 1.0, cutoff_radius if rv is not None else None)
-    with torch.cuda.device(dev), _timed("frame_axis2" if second else "frame_axis1", dev):
+    with torch.cuda.device(dev), _timed(("frame_axis1", "frame_axis2", "frame_axes")[mode], dev):
         need = lib.cfh_workspace_bytes(ctypes.byref(p), N, E)
         ws = _lib.workspace(dev, need)
         st = _lib.current_stream_ptr(dev)
-        if not second:
+        if mode == 2:
+            rc = lib.cfh_frame_axes(ctypes.byref(p), _lib.ptr(q), _lib.ptr(k), _lib.ptr(a), _lib.ptr(rpos),
+                                    _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges),
+                                    _lib.ptr(e_start), _lib.ptr(order), N, E, tv.shape[0], _lib.ptr(out),
+                                    _lib.ptr(ws), ws.numel(), st)
+        elif not second:
             rc = lib.cfh_frame_axis1(ctypes.byref(p), _lib.ptr(q), _lib.ptr(k), _lib.ptr(a), _lib.ptr(rpos),
                                      _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges),
                                      _lib.ptr(e_start), _lib.ptr(order), N, E, tv.shape[0], _lib.ptr(out),
@@ -185,7 +192,7 @@ def _frame_call(second: bool, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e
                                      _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges),
                                      _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(f1), N, E, tv.shape[0],
                                      _lib.ptr(out), _lib.ptr(ws), ws.numel(), st)
-    _lib.check(rc, "cfh_frame_axis2" if second else "cfh_frame_axis1")
+    _lib.check(rc, ("cfh_frame_axis1", "cfh_frame_axis2", "cfh_frame_axes")[mode])
     return out
 
 
@@ -196,8 +203,10 @@ class ComputeFrame1MaximumMethodCUDA(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max,
                 wscale, rvlen_n=None, cutoff_radius=None):
-        return _frame_call(False, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, None, rvlen_n,
-                           cutoff_radius)
+        out = _frame_call(0, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, None, rvlen_n,
+                          cutoff_radius)
+        ctx.mark_non_differentiable(out)      # the reference returns None for every input gradient
+        return out
 
     @staticmethod
     def backward(ctx, gframevec):
@@ -211,12 +220,44 @@ class ComputeFrame2MaximumMethodCUDA(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max,
                 wscale, frame1, rvlen_n=None, cutoff_radius=None):
-        return _frame_call(True, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, frame1, rvlen_n,
-                           cutoff_radius)
+        out = _frame_call(1, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, frame1, rvlen_n,
+                          cutoff_radius)
+        ctx.mark_non_differentiable(out)
+        return out
 
     @staticmethod
     def backward(ctx, gframevec):
         return (None,) * 15
+
+
+class ComputeFramesMaximumMethodCUDA(torch.autograd.Function):
+    """Orthonormal "max" frames (3,N,H,3) in one launch: both axis searches, Gram-Schmidt and the cross
+    product of compute_frame_maximum_method_ (models/indexed_lattice_multi_head_attention_cuda.py:
+    455-481).  No counterpart class in the reference; same leading arguments as the two above."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max,
+                wscale, rvlen_n=None, cutoff_radius=None):
+        out = _frame_call(2, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, None, rvlen_n,
+                          cutoff_radius)
+        ctx.mark_non_differentiable(out)
+        return out
+
+    @staticmethod
+    def backward(ctx, gframes):
+        return (None,) * 14
+
+
+def _stacked_frames(f1, f2, f3):
+    """(3,N,H,3) contiguous float32 holding the three frames, without a copy when they already are
+    the three slices of one such tensor."""
+    base = f1._base
+    if (base is not None and f2._base is base and f3._base is base and base.dtype == torch.float32
+            and base.is_contiguous() and base.dim() == 4 and base.shape[0] == 3
+            and f1.shape == base.shape[1:] and f1.data_ptr() == base.data_ptr()
+            and f2.data_ptr() == base[1].data_ptr() and f3.data_ptr() == base[2].data_ptr()):
+        return base.detach()
+    return torch.stack([_f32c(f1), _f32c(f2), _f32c(f3)], 0).contiguous()
 
 
 class RealEncodingWithFramedProjFuncCUDA(torch.autograd.Function):
@@ -245,8 +286,7 @@ class RealEncodingWithFramedProjFuncCUDA(torch.autograd.Function):
         rpos, tv, rv = _f32c(rpos_ij_e), _f32c(tvecs_n), _f32c(rvlen_n)
         batch, edges = batch_i.contiguous(), edge_ij_e.contiguous()
         e_start, order = edge_schedule(edge_ij_e, N)
-        frames = torch.stack([_f32c(frame_vec_1), _f32c(frame_vec_2), _f32c(frame_vec_3)], 0).contiguous() \
-            if use_angle else None
+        frames = _stacked_frames(frame_vec_1, frame_vec_2, frame_vec_3) if use_angle else None
         z = torch.empty((E, H), dtype=torch.float32, device=dev)
         v = torch.empty((E, H, Dh), dtype=torch.float32, device=dev) if K > 0 else None
         p = _params(H, Dh, K, A, cos_abs, float(dist_max), wscale, value_pe_angle_scale,

@@ -118,6 +118,18 @@ int cfh_frame_axis2(const cfh_params* p, const float* q, const float* k, const f
                     float* frame2max, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Both searches above in one launch, followed by the orthogonalisation the reference does in PyTorch:
+ * frames (3,N,H,3) = (f1, normalize(f2max - (f1.f2max) f1), f1 x f2).
+ * Replaces compute_frame_maximum_method_ for frame_method "max"
+ * (models/indexed_lattice_multi_head_attention_cuda.py:455-481).
+ */
+int cfh_frame_axes(const cfh_params* p, const float* q, const float* k, const float* a_ih,
+                   const float* rpos, const float* tvecs, const float* rvlen, const int64_t* batch,
+                   const int64_t* edges, const int64_t* e_start, const int32_t* order, int64_t N,
+                   int64_t E, int64_t B, float* frames, void* workspace, size_t workspace_bytes,
+                   void* stream);
+
+/*
  * z (E,H) = log sum_n exp(a_ih*|rpos + n.L|^2) and, when K > 0, the value position encoding
  * psi (E,H,Dh) = dist_coef * W_dist.s_dist + angle_coef * sum_axis W_axis.s_axis, where s are the
  * softmax-over-translations averages of the truncated Gaussian bases of the distance and of the

@@ -1,0 +1,82 @@
+"""End-to-end parity of the model (attention layer, encoder, pooling, head) on the GPU against the
+float64 CPU restatement, forward and parameter gradients."""
+import pytest
+import torch
+
+import helpers as Hh
+from oracle import cpu_model
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(mp, cb, seed=0):
+    import crystalframer_amd as cf
+    from crystalframer_amd import latticeformer
+    KM = cf.KernelManager
+    KM.SYMM_BREAK_NOISE = 0.0
+    dev = torch.device("cuda:0")
+    torch.manual_seed(seed)
+    model = latticeformer.Latticeformer(mp).to(dev)
+    for layer in model.encoder.layers:
+        layer.self_attn.frame_sink = []
+    out = model(cb.to(dev))
+    target = torch.linspace(-1, 1, cb.num_crystals, device=dev)[:, None]
+    loss = torch.nn.functional.mse_loss(out, target)
+    loss.backward()
+    torch.cuda.synchronize()
+    sd = {k: v.detach().cpu().double() for k, v in model.state_dict().items()}
+    leaves = {k: v.clone().requires_grad_("scale" not in k) for k, v in sd.items()}
+    frames = None
+    if mp.value_pe_angle_real > 0:
+        frames = [[f.detach().cpu().double() for f in layer.self_attn.frame_sink[0]] for layer in model.encoder.layers]
+    ref = cpu_model.model_forward(leaves, cb, mp, dtype=torch.float64, frames_per_layer=frames)
+    ref_loss = torch.nn.functional.mse_loss(ref, target.cpu().double())
+    ref_loss.backward()
+    return model, out, ref, leaves
+
+
+@pytest.mark.parametrize("angle_bins", [64, 0])
+def test_model_forward_backward_matches_cpu_oracle(angle_bins):
+    from crystalframer_amd import params, synthetic
+    mp = params.ModelParams(num_layers=2, value_pe_angle_real=angle_bins, symm_break_noise=0.0)
+    cb = synthetic.make_batch(8, atoms="uniform", atoms_lo=1, atoms_hi=6, len_lo=3.0, len_hi=9.0,
+                              ang_lo=65.0, ang_hi=115.0, seed=11)
+    model, out, ref, leaves = _run(mp, cb)
+    assert Hh.rel_err(out, ref) < 1e-4
+    checked = 0
+    for name, p in model.named_parameters():
+        if p.grad is None:
+            continue
+        g_ref = leaves[name].grad
+        assert g_ref is not None, name
+        assert Hh.rel_err(p.grad, g_ref) < 2e-4, name
+        checked += 1
+    assert checked >= 20
+    # the first training-mode forward stored the normalisation of alpha
+    for layer in model.encoder.layers:
+        assert float(layer.self_attn.gauss_scale[0]) > 0
+
+
+def test_model_frames_agree_with_oracle_frames():
+    """The frames the model used are the oracle's wherever the winner is clear."""
+    from crystalframer_amd import params, synthetic
+    from oracle import torch_oracle as TO
+    import math
+    mp = params.ModelParams(num_layers=1, symm_break_noise=0.0)
+    cb = synthetic.make_batch(8, atoms="uniform", atoms_lo=2, atoms_hi=6, len_lo=3.0, len_hi=9.0,
+                              ang_lo=65.0, ang_hi=115.0, seed=13)
+    model, out, ref, leaves = _run(mp, cb)
+    sd = {k: v.detach() for k, v in leaves.items()}
+    lat = params.LatticeformerParams().parseFromArgs(mp).getLayerParameters(0)
+    pos, tv = cb.pos.double(), cb.trans_vec.double()
+    edges, rpos, recip, _ = TO.geometry(pos, tv, cb.sizes.tolist())
+    geo = dict(edges=edges, rpos=rpos, tvecs=tv, rvlen=recip.norm(dim=-1), batch=cb.batch)
+    x = torch.nn.functional.linear(cb.x.double(), sd["input_embeddings.weight"])
+    _, aux = cpu_model.attention_layer(x, sd, "encoder.layers.0.self_attn.", geo, lat, return_aux=True)
+    q = aux["q"] / math.sqrt(16)
+    f1, f2, gap1, gap2 = TO.frame_axes_max(q, aux["k"], aux["a"], rpos, tv, cb.batch, edges, rvlen=geo["rvlen"],
+                                           cutoff_radius=-3.5, return_gaps=True)
+    used = model.encoder.layers[0].self_attn.frame_sink[0]
+    clear = (gap1 > 1e-4) & (gap2 > 1e-4)
+    assert clear.double().mean() > 0.9
+    assert (used[0].cpu().double() - f1)[clear].abs().max() < 1e-4

@@ -342,3 +342,21 @@ def test_full_batch_atom_permutation_equivariance():
     src = torch.tensor([lookup[(int(perm[int(P2.edges[0, e])]), int(perm[int(P2.edges[1, e])]))] for e in range(P.E)])
     assert Hh.rel_err(z2, z.cpu().double()[src]) < 1e-5
     assert Hh.rel_err(psi2, psi.cpu().double()[src]) < 2e-5
+
+
+def test_fused_frames_equal_the_three_step_construction():
+    """cfh_frame_axes (both searches + Gram-Schmidt + cross product in one launch) against the
+    reference's sequence: axis 1, axis 2, PyTorch orthogonalisation."""
+    import crystalframer_amd as cf
+    P = Hh.make_problem(num_crystals=12, atoms_hi=6, seed=67)
+    f1, f2 = run_frames(P)
+    r1, r2, r3 = TO.orthonormal_frame(f1.cpu().double(), f2.cpu().double())
+    args = (g(P.q), g(P.k), None, g(P.a), g(P.rpos), None, g(P.tvecs), P.batch.to(dev()), P.edges.to(dev()),
+            64, Hh.DIST_MAX, 1.0, g(P.rvlen), CUT)
+    fr = cf.ComputeFramesMaximumMethodCUDA.apply(*args)
+    assert fr.shape == (3, P.N, Hh.H, 3)
+    for got, want in zip(fr.cpu().double(), (r1, r2, r3)):
+        assert (got - want).abs().max() < 1e-5
+    M = fr.cpu().double().permute(1, 2, 0, 3)
+    assert (M @ M.transpose(-1, -2) - torch.eye(3, dtype=torch.float64)).abs().max() < 1e-5
+    assert (torch.linalg.det(M) - 1).abs().max() < 1e-5

@@ -13,8 +13,16 @@ import helpers as Hh
 from oracle import c_oracle as CO
 from oracle import torch_oracle as TO
 
-torch.set_default_dtype(torch.float64)
 F64 = torch.float64
+
+
+@pytest.fixture(autouse=True)
+def _float64_default():
+    """These tests build their small tensors in float64; restore the default for other modules."""
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float64)
+    yield
+    torch.set_default_dtype(old)
 
 
 def _one_crystal(lattice, frac):
