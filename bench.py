@@ -123,13 +123,18 @@ def main():
     # ---- a second, instrumented pass over the same steps: HIP events around every library call on
     #      its stream, and term counters; kept out of the timed region so that it cannot perturb it
     KM.EVENT_LOG = []
-    KM.COLLECT_STATS = True
-    _lib.read_stats(dev, reset=True)
     nprof = min(args.steps, 5)
     for _ in range(nprof):
         step()
     torch.cuda.synchronize()
-    log, KM.EVENT_LOG, KM.COLLECT_STATS = KM.EVENT_LOG, None, False
+    log, KM.EVENT_LOG = KM.EVENT_LOG, None
+    # ---- and a third one that counts translations (separately: the counters add a few atomics)
+    KM.COLLECT_STATS = True
+    _lib.read_stats(dev, reset=True)
+    for _ in range(nprof):
+        step()
+    torch.cuda.synchronize()
+    KM.COLLECT_STATS = False
     stats = _lib.read_stats(dev, reset=True)
     per_kernel = {}
     for name, s, e in log:

@@ -58,6 +58,7 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
     const int h = blockIdx.x % H;
     const bool noisy = P.noise > 0.0f;
 
+    unsigned long long st_raw = 0;
     for (int it = first_item(H); it < P.N; it += item_stride(H)) {
         const int i = P.order ? uniform_i(P.order[it]) : it;
         const int b = uniform_i((int)P.batch[i]);
@@ -192,12 +193,12 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                 o[2 * stride + 1] = f1z * gx - f1x * gz;
                 o[2 * stride + 2] = f1x * gy - f1y * gx;
             }
-            if (P.stats) {
-                const unsigned long long raw = (unsigned long long)bx.T * (unsigned long long)(e1 - e0);
-                if (MODE != 1) atomicAdd(P.stats + STAT_FRAME1_RAW, raw);
-                if (MODE != 0) atomicAdd(P.stats + STAT_FRAME2_RAW, raw);
-            }
         }
+        st_raw += (unsigned long long)bx.T * (unsigned long long)(e1 - e0);
+    }
+    if (P.stats && lane == 0) {      // once per wavefront
+        if (MODE != 1) atomicAdd(P.stats + STAT_FRAME1_RAW, st_raw);
+        if (MODE != 0) atomicAdd(P.stats + STAT_FRAME2_RAW, st_raw);
     }
 }
 

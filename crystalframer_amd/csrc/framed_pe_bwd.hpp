@@ -50,6 +50,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
     for (int u = lane; u < GROUP_BWD * PAIR_STRIDE; u += WAVE) { hist[u] = 0u; Gs[u] = 0.0f; }
     __syncthreads();
 
+    unsigned long long st_eval = 0, st_raw = 0, st_pairs = 0;
     for (int it = first_item(H); it < P.N; it += item_stride(H)) {
         const int i = P.order ? uniform_i(P.order[it]) : it;
         const int b = uniform_i((int)P.batch[i]);
@@ -244,14 +245,15 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
             __syncthreads();               // gpS, pair data and histograms are free again
         }
         cov = wave_sum(cov);
-        if (lane == 0) {
-            P.out_ga[(size_t)i * H + h] = ga_acc + cov;
-            if (P.stats) {
-                atomicAdd(P.stats + STAT_BWD_EVAL, n_eval);
-                atomicAdd(P.stats + STAT_BWD_RAW, (unsigned long long)bx.T * (unsigned long long)(e1 - e0));
-                atomicAdd(P.stats + STAT_BWD_PAIRS, (unsigned long long)(e1 - e0));
-            }
-        }
+        if (lane == 0) P.out_ga[(size_t)i * H + h] = ga_acc + cov;
+        st_eval += n_eval;
+        st_raw += (unsigned long long)bx.T * (unsigned long long)(e1 - e0);
+        st_pairs += (unsigned long long)(e1 - e0);
+    }
+    if (P.stats && lane == 0) {      // once per wavefront
+        atomicAdd(P.stats + STAT_BWD_EVAL, st_eval);
+        atomicAdd(P.stats + STAT_BWD_RAW, st_raw);
+        atomicAdd(P.stats + STAT_BWD_PAIRS, st_pairs);
     }
 
     // per-wavefront partials of the weight gradients: (wave, enc, c, k)

@@ -52,6 +52,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
     for (int u = lane; u < GROUP * PAIR_STRIDE; u += WAVE) hist[u] = 0u;
     __syncthreads();
 
+    unsigned long long st_eval = 0, st_raw = 0, st_pairs = 0;
     for (int it = first_item(H); it < P.N; it += item_stride(H)) {
         const int i = P.order ? uniform_i(P.order[it]) : it;
         const int b = uniform_i((int)P.batch[i]);
@@ -259,11 +260,15 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
             }
             __syncthreads();                       // pair data of this group no longer needed
         }
-        if (P.stats && lane == 0) {
-            atomicAdd(P.stats + STAT_FWD_EVAL, n_eval);
-            atomicAdd(P.stats + STAT_FWD_RAW, (unsigned long long)bx.T * (unsigned long long)(e1 - e0));
-            atomicAdd(P.stats + STAT_FWD_PAIRS, (unsigned long long)(e1 - e0));
-        }
+        st_eval += n_eval;
+        st_raw += (unsigned long long)bx.T * (unsigned long long)(e1 - e0);
+        st_pairs += (unsigned long long)(e1 - e0);
+    }
+    // one set of atomics per wavefront (per-item atomics on three shared addresses serialise in L2)
+    if (P.stats && lane == 0) {
+        atomicAdd(P.stats + STAT_FWD_EVAL, st_eval);
+        atomicAdd(P.stats + STAT_FWD_RAW, st_raw);
+        atomicAdd(P.stats + STAT_FWD_PAIRS, st_pairs);
     }
 }
 
