@@ -46,7 +46,9 @@ class CfhParams(ctypes.Structure):
 
 
 EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_frame_axis1",
-           "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_backward")
+           "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_backward",
+           "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
+           "cfh_crystal_mean_forward", "cfh_crystal_mean_backward")
 
 _lib = None
 _lock = threading.Lock()
@@ -85,6 +87,16 @@ def load():
         lib.cfh_framed_pe_forward.argtypes = [pp] + [_P] * 13 + [_I64] * 3 + [_P] * 4 + [ctypes.c_size_t, _P]
         lib.cfh_framed_pe_backward.restype = ctypes.c_int
         lib.cfh_framed_pe_backward.argtypes = [pp] + [_P] * 16 + [_I64] * 3 + [_P] * 6 + [ctypes.c_size_t, _P]
+        lib.cfh_fused_dpa_forward.restype = ctypes.c_int
+        lib.cfh_fused_dpa_forward.argtypes = [_P] * 7 + [_I64] * 4 + [_P] * 3
+        lib.cfh_fused_dpa_backward.restype = ctypes.c_int
+        lib.cfh_fused_dpa_backward.argtypes = [_P] * 10 + [_I64] * 4 + [_P] * 6
+        lib.cfh_pair_layout_check.restype = ctypes.c_int
+        lib.cfh_pair_layout_check.argtypes = [_P, _P, _I64, _I64, _P, _P]
+        lib.cfh_crystal_mean_forward.restype = ctypes.c_int
+        lib.cfh_crystal_mean_forward.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P]
+        lib.cfh_crystal_mean_backward.restype = ctypes.c_int
+        lib.cfh_crystal_mean_backward.argtypes = [_P, _P, _P, _I64, _I64, _I64, _P, _P]
         if lib.cfh_abi_version() != ABI_VERSION:
             raise RuntimeError(f"ABI version {lib.cfh_abi_version()} of {LIB_PATH} != {ABI_VERSION}")
         _lib = lib

@@ -1,5 +1,5 @@
 // C ABI of the gfx950 kernels (see include/crystalframer_hip.h).  Host side: argument checks,
-// constant preparation, work-queue reset and kernel launches.  Nothing here allocates or
+// constant preparation and kernel launches.  Nothing here allocates or
 // synchronises.
 #include "../../include/crystalframer_hip.h"
 
@@ -14,6 +14,7 @@
 #include "frame_select.hpp"
 #include "framed_pe_bwd.hpp"
 #include "framed_pe_fwd.hpp"
+#include "fused_dpa.hpp"
 
 namespace {
 
@@ -325,10 +326,10 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
     hipStream_t st = (hipStream_t)stream;
     const size_t wbytes = (size_t)p->num_heads * cfh::DH * cfh::NBINS * sizeof(float);
     if (N == 0) {     // no atoms: the weight gradients are zero
-        float* outs[4] = {gW_dist, gW_axis1, gW_axis2, gW_axis3};
-        for (float* o : outs)
-            if (o && hipMemsetAsync(o, 0, wbytes, st) != hipSuccess) return fail(CFH_ELAUNCH, "memset of an empty gradient failed");
-        return CFH_OK;
+        const int per_enc = (int)(wbytes / sizeof(float));
+        hipLaunchKernelGGL(cfh::zero_outputs_kernel, dim3((per_enc + 255) / 256), dim3(256), 0, st, per_enc,
+                           gW_dist, gW_axis1, gW_axis2, gW_axis3);
+        return finish_launch("zero_outputs");
     }
     if (!z || !gz || !ga) return fail(CFH_EINVAL, "z, gz and ga must not be NULL");
     if (has_len && !gpsi) return fail(CFH_EINVAL, "gpsi must not be NULL when dist_bins > 0");
@@ -363,6 +364,98 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
         rc = finish_launch("gw_reduce");
     }
     return rc;
+}
+
+namespace {
+int check_dpa(const void* q, const void* k, const void* v, const int64_t* edges, const int64_t* e_start,
+              int64_t N, int64_t H, int64_t Dh, int64_t E) {
+    if (N < 0 || E < 0) return fail(CFH_EINVAL, "negative size N=%lld E=%lld", (long long)N, (long long)E);
+    if (H < 1 || H > MAX_HEADS) return fail(CFH_EINVAL, "H %lld outside 1..%d", (long long)H, MAX_HEADS);
+    if (Dh != cfh::DH) return fail(CFH_EINVAL, "head_dim %lld not compiled (only %d)", (long long)Dh, cfh::DH);
+    if (N > 0x7fffffffLL / 64 || E > 0x7fffffffLL / 64)
+        return fail(CFH_EINVAL, "N=%lld or E=%lld beyond the 32-bit index range of the kernels", (long long)N, (long long)E);
+    if (N > 0 && (!q || !k || !v || !e_start)) return fail(CFH_EINVAL, "q, k, v and e_start must not be NULL");
+    if (E > 0 && !edges) return fail(CFH_EINVAL, "edges must not be NULL");
+    return CFH_OK;
+}
+}  // namespace
+
+int cfh_fused_dpa_forward(const float* q, const float* k, const float* v, const float* aij,
+                          const float* bij, const int64_t* edges, const int64_t* e_start, int64_t N,
+                          int64_t H, int64_t Dh, int64_t E, float* prob, float* out, void* stream) {
+    int rc = check_dpa(q, k, v, edges, e_start, N, H, Dh, E);
+    if (rc) return rc;
+    if (N == 0) return CFH_OK;
+    if (!out || (E > 0 && !prob)) return fail(CFH_EINVAL, "prob and out must not be NULL");
+    cfh::DpaArgs A;
+    std::memset(&A, 0, sizeof(A));
+    A.q = q; A.k = k; A.v = v; A.aij = aij; A.bij = bij; A.edges = edges; A.e_start = e_start;
+    A.prob = prob; A.out = out; A.N = (int32_t)N; A.H = (int32_t)H; A.E = (int32_t)E;
+    const int64_t items = N * H;
+    hipLaunchKernelGGL(cfh::dpa_fwd_kernel, dim3((unsigned)((items + cfh::DPA_WAVES - 1) / cfh::DPA_WAVES)),
+                       dim3(cfh::WAVE * cfh::DPA_WAVES), 0, (hipStream_t)stream, A);
+    return finish_launch("fused_dpa_forward");
+}
+
+int cfh_fused_dpa_backward(const float* q, const float* k, const float* v, const float* aij,
+                           const float* bij, const int64_t* edges, const int64_t* e_start,
+                           const float* prob, const float* out, const float* gout, int64_t N,
+                           int64_t H, int64_t Dh, int64_t E, float* gq, float* gk, float* gv,
+                           float* gaij, float* gbij, void* stream) {
+    int rc = check_dpa(q, k, v, edges, e_start, N, H, Dh, E);
+    if (rc) return rc;
+    if (N == 0) return CFH_OK;
+    if (!out || !gout || !gq || !gk || !gv) return fail(CFH_EINVAL, "out, gout, gq, gk and gv must not be NULL");
+    if (E > 0 && (!prob || !gaij)) return fail(CFH_EINVAL, "prob and gaij must not be NULL");
+    (void)aij;
+    cfh::DpaArgs A;
+    std::memset(&A, 0, sizeof(A));
+    A.q = q; A.k = k; A.v = v; A.bij = bij; A.edges = edges; A.e_start = e_start;
+    A.prob = const_cast<float*>(prob); A.out = const_cast<float*>(out); A.go = gout;
+    A.gq = gq; A.gk = gk; A.gv = gv; A.gaij = gaij; A.gbij = gbij;
+    A.N = (int32_t)N; A.H = (int32_t)H; A.E = (int32_t)E;
+    const int64_t items = N * H;
+    const dim3 grid((unsigned)((items + cfh::DPA_WAVES - 1) / cfh::DPA_WAVES)), block(cfh::WAVE * cfh::DPA_WAVES);
+    hipLaunchKernelGGL(cfh::dpa_bwd_row_kernel, grid, block, 0, (hipStream_t)stream, A);
+    hipLaunchKernelGGL(cfh::dpa_bwd_col_kernel, grid, block, 0, (hipStream_t)stream, A);
+    return finish_launch("fused_dpa_backward");
+}
+
+int cfh_pair_layout_check(const int64_t* edges, const int64_t* e_start, int64_t N, int64_t E,
+                          int32_t* flag, void* stream) {
+    if (!flag) return fail(CFH_EINVAL, "flag must not be NULL");
+    if (N < 0 || E < 0 || N > 0x7fffffffLL / 64 || E > 0x7fffffffLL / 64)
+        return fail(CFH_EINVAL, "N=%lld or E=%lld outside the index range of the kernels", (long long)N, (long long)E);
+    if (N > 0 && (!e_start || (E > 0 && !edges))) return fail(CFH_EINVAL, "edges and e_start must not be NULL");
+    hipLaunchKernelGGL(cfh::set_flag_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, flag, 0);
+    if (N > 0)
+        hipLaunchKernelGGL(cfh::dpa_check_layout_kernel, dim3((unsigned)((N + 255) / 256)), dim3(256), 0,
+                           (hipStream_t)stream, edges, e_start, (int)N, (int)E, flag);
+    return finish_launch("pair_layout_check");
+}
+
+int cfh_crystal_mean_forward(const float* x, const int64_t* atom_start, int64_t N, int64_t B,
+                             int64_t C, float* out, void* stream) {
+    if (N < 0 || B < 0 || C < 0 || C > 0x7fffffffLL || N > 0x7fffffffLL || B > 0x7fffffffLL)
+        return fail(CFH_EINVAL, "sizes N=%lld B=%lld C=%lld out of range", (long long)N, (long long)B, (long long)C);
+    if (B == 0 || C == 0) return CFH_OK;
+    if (!atom_start || !out || (N > 0 && !x)) return fail(CFH_EINVAL, "x, atom_start and out must not be NULL");
+    const int threads = C >= 256 ? 256 : (C >= 128 ? 128 : 64);
+    hipLaunchKernelGGL(cfh::crystal_mean_fwd_kernel, dim3((unsigned)B), dim3(threads), 0, (hipStream_t)stream, x,
+                       atom_start, (int)B, (int)C, out);
+    return finish_launch("crystal_mean_forward");
+}
+
+int cfh_crystal_mean_backward(const float* gout, const int64_t* batch, const int64_t* atom_start,
+                              int64_t N, int64_t B, int64_t C, float* gx, void* stream) {
+    if (N < 0 || B < 0 || C < 0 || C > 0x7fffffffLL || N > 0x7fffffffLL || B > 0x7fffffffLL)
+        return fail(CFH_EINVAL, "sizes N=%lld B=%lld C=%lld out of range", (long long)N, (long long)B, (long long)C);
+    if (N == 0 || C == 0) return CFH_OK;
+    if (!gout || !batch || !atom_start || !gx) return fail(CFH_EINVAL, "gout, batch, atom_start and gx must not be NULL");
+    const size_t total = (size_t)N * (size_t)C;
+    hipLaunchKernelGGL(cfh::crystal_mean_bwd_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, gout, batch, atom_start, (int)N, (int)C, gx);
+    return finish_launch("crystal_mean_backward");
 }
 
 }  // extern "C"

@@ -340,46 +340,121 @@ class RealEncodingWithFramedProjFuncCUDA(torch.autograd.Function):
 # consumers of z and psi.  Interim composites of stock PyTorch device ops with the reference's names
 # and signatures; they run on the HIP device (no CPU path) but are not hand-written kernels yet.
 # --------------------------------------------------------------------------------------------------
-class FusedDotProductAttentionCUDA:
-    """out_i = sum_j softmax_j(q_i.k_j + a_ij) (v_j + b_ij), per head, over the edges of atom i.
+_layout_cache = {"ref": None, "version": None, "ok": None}
 
-    Signature of models/cuda_funcs/fused_dpa.py:17-63 (``que_ihk`` already divided by sqrt(Dh));
-    max-subtracted softmax as in models/kernels/fused_dpa_fwd.cu:46-91.
+
+def declare_complete_blocks(edge_ij_e: torch.Tensor):
+    """Record that ``edge_ij_e`` holds all n x n pairs of every crystal, sorted by i then j (true by
+    construction for geometry.py), which spares the attention backward its one-off layout check."""
+    _layout_cache.update(ref=weakref.ref(edge_ij_e), version=edge_ij_e._version, ok=True)
+
+
+def _require_complete_blocks(edge_ij_e: torch.Tensor, e_start: torch.Tensor, N: int):
+    c = _layout_cache
+    if not (c["ref"] is not None and c["ref"]() is edge_ij_e and c["version"] == edge_ij_e._version):
+        flag = torch.empty(1, dtype=torch.int32, device=edge_ij_e.device)
+        lib = _lib.load()
+        rc = lib.cfh_pair_layout_check(_lib.ptr(edge_ij_e), _lib.ptr(e_start), N, edge_ij_e.shape[1],
+                                       _lib.ptr(flag), _lib.current_stream_ptr(edge_ij_e.device))
+        _lib.check(rc, "cfh_pair_layout_check")
+        c.update(ref=weakref.ref(edge_ij_e), version=edge_ij_e._version, ok=int(flag.item()) == 0)
+    if not c["ok"]:
+        raise ValueError("FusedDotProductAttentionCUDA.backward needs the complete n x n pair block of every "
+                         "crystal, sorted by i then j (the layout the reference's irregular_transpose assumes)")
+
+
+class FusedDotProductAttentionCUDA(torch.autograd.Function):
+    """out_i = sum_j softmax_j(q_i.k_j + a_ij) (v_j + b_ij), per head, over the pairs of atom i.
+
+    Signature and gradients of models/cuda_funcs/fused_dpa.py:17-170 (``que_ihk`` already divided by
+    sqrt(Dh)).
     """
 
     @staticmethod
-    def apply(que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, batch_i, edge_ij_e):
-        _lib.require_gpu(que_ihk, key_ihk, val_ihk)
-        N, H, _ = que_ihk.shape
-        ei, ej = edge_ij_e[0], edge_ij_e[1]
-        logit = (que_ihk[ei] * key_ihk[ej]).sum(-1)
-        if aij_eh is not None:
-            logit = logit + aij_eh
-        idx = ei[:, None].expand(-1, H)
-        mx = torch.full((N, H), -3.0e38, dtype=logit.dtype, device=logit.device)
-        mx = mx.scatter_reduce(0, idx, logit.detach(), reduce="amax", include_self=True)
-        ex = torch.exp(logit - mx[ei])
-        den = torch.zeros((N, H), dtype=logit.dtype, device=logit.device).index_add_(0, ei, ex)
-        prob = ex / den[ei]
-        val = val_ihk[ej]
-        if bij_ehk is not None:
-            val = val + bij_ehk
-        out = torch.zeros_like(val_ihk).index_add_(0, ei, prob[..., None] * val)
-        return out
+    def forward(ctx, que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, batch_i, edge_ij_e):
+        _lib.require_gpu(que_ihk, key_ihk, val_ihk, aij_eh, bij_ehk, edge_ij_e)
+        lib = _lib.load()
+        N, H, K = que_ihk.shape
+        E = edge_ij_e.shape[1]
+        dev = que_ihk.device
+        q, k, v = _f32c(que_ihk), _f32c(key_ihk), _f32c(val_ihk)
+        a, b = _f32c(aij_eh), _f32c(bij_ehk)
+        edge_c = edge_ij_e if edge_ij_e.is_contiguous() else edge_ij_e.contiguous()
+        e_start, _ = edge_schedule(edge_ij_e, N)
+        out = torch.empty((N, H, K), dtype=torch.float32, device=dev)
+        prob = torch.empty((E, H), dtype=torch.float32, device=dev)
+        with _timed("fused_dpa_forward", dev):
+            rc = lib.cfh_fused_dpa_forward(_lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b),
+                                           _lib.ptr(edge_c), _lib.ptr(e_start), N, H, K, E, _lib.ptr(prob),
+                                           _lib.ptr(out), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_fused_dpa_forward")
+        ctx.save_for_backward(q, k, v, a, b, edge_c, e_start, prob, out)
+        ctx.edge_ref = edge_ij_e
+        ctx.in_dtype = que_ihk.dtype
+        return out.to(que_ihk.dtype)
+
+    @staticmethod
+    def backward(ctx, go_ihk):
+        q, k, v, a, b, edge_c, e_start, prob, out = ctx.saved_tensors
+        lib = _lib.load()
+        N, H, K = q.shape
+        E = edge_c.shape[1]
+        dev = q.device
+        _require_complete_blocks(ctx.edge_ref, e_start, N)
+        go = _f32c(go_ihk)
+        gq, gk, gv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        ga = torch.empty((E, H), dtype=torch.float32, device=dev)
+        gb = torch.empty_like(b) if b is not None else None
+        with _timed("fused_dpa_backward", dev):
+            rc = lib.cfh_fused_dpa_backward(_lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b),
+                                            _lib.ptr(edge_c), _lib.ptr(e_start), _lib.ptr(prob), _lib.ptr(out),
+                                            _lib.ptr(go), N, H, K, E, _lib.ptr(gq), _lib.ptr(gk), _lib.ptr(gv),
+                                            _lib.ptr(ga), _lib.ptr(gb), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_fused_dpa_backward")
+        dt = ctx.in_dtype
+        return (gq.to(dt), gk.to(dt), gv.to(dt), ga.to(dt) if a is not None else None,
+                gb.to(dt) if gb is not None else None, None, None)
 
 
-class IrregularMeanCUDA:
+class IrregularMeanCUDA(torch.autograd.Function):
     """Per-crystal mean of per-atom features.  Signature of models/cuda_funcs/irregular_mean.py:19-70."""
 
     @staticmethod
-    def apply(x_ik, batch_i, sizes):
-        _lib.require_gpu(x_ik)
+    def forward(ctx, x_ik, batch_i, sizes):
+        _lib.require_gpu(x_ik, batch_i)
+        lib = _lib.load()
+        dev = x_ik.device
         if sizes is None:
-            B = int(batch_i.max().item()) + 1
-            sizes = torch.zeros(B, dtype=torch.long, device=x_ik.device)
+            B = int(batch_i.max().item()) + 1 if batch_i.numel() else 0
+            sizes = torch.zeros(B, dtype=torch.long, device=dev)
             sizes.scatter_add_(0, batch_i, torch.ones_like(batch_i))
         B = sizes.shape[0]
-        out = torch.zeros((B,) + tuple(x_ik.shape[1:]), dtype=x_ik.dtype, device=x_ik.device)
-        out.index_add_(0, batch_i, x_ik)
-        shape = [B] + [1] * (x_ik.dim() - 1)
-        return out / sizes.reshape(shape).to(x_ik.dtype)
+        N = x_ik.shape[0]
+        C = x_ik[0].numel() if N else int(torch.tensor(x_ik.shape[1:]).prod())
+        atom_start = torch.zeros(B + 1, dtype=torch.long, device=dev)
+        atom_start[1:] = sizes.to(device=dev, dtype=torch.long).cumsum(0)
+        x = _f32c(x_ik)
+        out = torch.empty((B,) + tuple(x_ik.shape[1:]), dtype=torch.float32, device=dev)
+        with _timed("crystal_mean_forward", dev):
+            rc = lib.cfh_crystal_mean_forward(_lib.ptr(x), _lib.ptr(atom_start), N, B, C, _lib.ptr(out),
+                                              _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_crystal_mean_forward")
+        ctx.save_for_backward(batch_i.contiguous(), atom_start)
+        ctx.x_shape, ctx.in_dtype = tuple(x_ik.shape), x_ik.dtype
+        return out.to(x_ik.dtype)
+
+    @staticmethod
+    def backward(ctx, gout):
+        batch_i, atom_start = ctx.saved_tensors
+        lib = _lib.load()
+        dev = gout.device
+        N = ctx.x_shape[0]
+        B = atom_start.shape[0] - 1
+        g = _f32c(gout)
+        C = g[0].numel() if B else 0
+        gx = torch.empty(ctx.x_shape, dtype=torch.float32, device=dev)
+        with _timed("crystal_mean_backward", dev):
+            rc = lib.cfh_crystal_mean_backward(_lib.ptr(g), _lib.ptr(batch_i), _lib.ptr(atom_start), N, B, C,
+                                               _lib.ptr(gx), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_crystal_mean_backward")
+        return gx.to(ctx.in_dtype), None, None

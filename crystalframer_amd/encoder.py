@@ -123,6 +123,7 @@ class CrystalformerEncoderCUDA(nn.Module):
         batch = batch - batch[0]
         geo = geometry.crystal_geometry(pos, batch, trans, sizes)
         cuda_funcs.seed_edge_schedule(geo.edges, geo.e_start, geo.order)
+        cuda_funcs.declare_complete_blocks(geo.edges)
         x = src
         for layer in self.layers:
             # rvecs: the lengths of the reciprocal vectors are all the layers use, computed once here

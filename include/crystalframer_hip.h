@@ -164,6 +164,53 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
                            float* ga, float* gW_dist, float* gW_axis1, float* gW_axis2,
                            float* gW_axis3, void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * Attention over the pairs of each atom: l_e = q_i.k_j + aij_e, p = softmax over the pairs (i,.)
+ * of atom i, out_i = sum_e p_e (v_j + bij_e).  q (already divided by sqrt(Dh)), k, v, out (N,H,Dh);
+ * aij (E,H) or NULL; bij (E,H,Dh) or NULL; prob (E,H) receives the attention weights (the backward
+ * needs them).  Dh = 16.  Needs no workspace.
+ * Replaces FusedDotProductAttentionCUDA.forward: kernel fused_dpa_fwd
+ * (models/cuda_funcs/fused_dpa.py:17-63, models/kernels/fused_dpa_fwd.cu).
+ */
+int cfh_fused_dpa_forward(const float* q, const float* k, const float* v, const float* aij,
+                          const float* bij, const int64_t* edges, const int64_t* e_start, int64_t N,
+                          int64_t H, int64_t Dh, int64_t E, float* prob, float* out, void* stream);
+
+/*
+ * Gradients of the above for upstream gout (N,H,Dh): gq, gk, gv (N,H,Dh), gaij (E,H; always
+ * written, also when aij was NULL) and gbij (E,H,Dh) or NULL.  The pairs must be the complete
+ * n x n block of every crystal with rows and columns in atom order (cfh_pair_layout_check), which
+ * is what lets gk and gv be summed without atomics and without the transposed copies the
+ * reference makes.
+ * Replaces FusedDotProductAttentionCUDA.backward: kernels irregular_transpose, fused_dpa_bwd and
+ * fused_dpa_bwd_q (models/cuda_funcs/fused_dpa.py:65-170).
+ */
+int cfh_fused_dpa_backward(const float* q, const float* k, const float* v, const float* aij,
+                           const float* bij, const int64_t* edges, const int64_t* e_start,
+                           const float* prob, const float* out, const float* gout, int64_t N,
+                           int64_t H, int64_t Dh, int64_t E, float* gq, float* gk, float* gv,
+                           float* gaij, float* gbij, void* stream);
+
+/*
+ * Sets *flag (device memory) to 0 when edges (2,E) / e_start (N+1) hold, for every crystal, all
+ * n x n pairs (i,j) sorted by i then j, to 1 otherwise.  The reference relies on the same layout
+ * without checking it (models/kernels/irregular_transpose.cu).
+ */
+int cfh_pair_layout_check(const int64_t* edges, const int64_t* e_start, int64_t N, int64_t E,
+                          int32_t* flag, void* stream);
+
+/*
+ * Per-crystal mean of per-atom rows: out (B,C) from x (N,C); atom_start (B+1) are the prefix sums
+ * of the crystal sizes (atoms of a crystal are contiguous).  The backward spreads gout (B,C) back:
+ * gx[i] = gout[batch[i]] / size.
+ * Replaces IrregularMeanCUDA: kernels irregular_mean_fwd and the gather of its backward
+ * (models/cuda_funcs/irregular_mean.py:19-70).
+ */
+int cfh_crystal_mean_forward(const float* x, const int64_t* atom_start, int64_t N, int64_t B,
+                             int64_t C, float* out, void* stream);
+int cfh_crystal_mean_backward(const float* gout, const int64_t* batch, const int64_t* atom_start,
+                              int64_t N, int64_t B, int64_t C, float* gx, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,166 @@
+"""Parity of the HIP attention (softmax over the pairs of an atom, with logit and value biases) and
+of the per-crystal mean against the float64 oracles, forward and backward, through the
+autograd.Function boundary (which calls the C ABI).  float32 kernels vs float64 oracle: 2e-5 of the
+largest magnitude forward, 5e-5 for gradients."""
+import pytest
+import torch
+
+import helpers as Hh
+from oracle import c_oracle as CO
+from oracle import torch_oracle as TO
+
+pytestmark = pytest.mark.gpu
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def f32(t):
+    return t.to(dtype=torch.float32, device=dev())
+
+
+def attention_case(P, seed, with_a=True, with_b=True, big_logits=False):
+    g = torch.Generator().manual_seed(seed)
+    z = torch.randn(P.E, Hh.H, generator=g, dtype=torch.float64) * (30.0 if big_logits else 1.0) if with_a else None
+    psi = torch.randn(P.E, Hh.H, Hh.DH, generator=g, dtype=torch.float64) if with_b else None
+    gout = torch.randn(P.N, Hh.H, Hh.DH, generator=g, dtype=torch.float64)
+    return z, psi, gout
+
+
+def run_both(P, z, psi, gout):
+    import crystalframer_amd as cf
+    leaves64 = [t.double().clone().requires_grad_(True) if t is not None else None for t in (P.q, P.k, P.v, z, psi)]
+    out64, prob64 = TO.softmax_attention(*leaves64, P.batch, P.edges)
+    (out64 * gout).sum().backward()
+    leaves = [f32(t).requires_grad_(True) if t is not None else None for t in (P.q, P.k, P.v, z, psi)]
+    out = cf.FusedDotProductAttentionCUDA.apply(*leaves, P.batch.to(dev()), P.edges.to(dev()))
+    (out * f32(gout)).sum().backward()
+    return out64, leaves64, out, leaves
+
+
+@pytest.mark.parametrize("with_a,with_b", [(True, True), (True, False), (False, False)])
+def test_attention_forward_backward(with_a, with_b):
+    P = Hh.make_problem(num_crystals=7, atoms_hi=9, seed=71)
+    z, psi, gout = attention_case(P, 5, with_a, with_b)
+    out64, leaves64, out, leaves = run_both(P, z, psi, gout)
+    assert Hh.rel_err(out.cpu().double(), out64.detach()) < 2e-5
+    for l32, l64, name in zip(leaves, leaves64, "q k v a b".split()):
+        if l64 is None:
+            continue
+        assert Hh.rel_err(l32.grad.cpu().double(), l64.grad) < 5e-5, name
+
+
+def test_attention_matches_c_oracle_and_saves_probabilities():
+    import crystalframer_amd as cf
+    from crystalframer_amd import _lib
+    P = Hh.make_problem(num_crystals=5, atoms_hi=6, seed=72)
+    z, psi, gout = attention_case(P, 6)
+    oc, pc = CO.dpa_forward(P.q, P.k, P.v, z, psi, P.edges, "f64")
+    # straight through the C ABI
+    lib = _lib.load()
+    q, k, v, a, b = (f32(t).contiguous() for t in (P.q, P.k, P.v, z, psi))
+    edges = P.edges.to(dev()).contiguous()
+    e_start, _ = cf.cuda_funcs.edge_schedule(edges, P.N)
+    out = torch.empty_like(v)
+    prob = torch.empty(P.E, Hh.H, device=dev())
+    rc = lib.cfh_fused_dpa_forward(_lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b), _lib.ptr(edges),
+                                   _lib.ptr(e_start), P.N, Hh.H, Hh.DH, P.E, _lib.ptr(prob), _lib.ptr(out),
+                                   _lib.current_stream_ptr(dev()))
+    assert rc == 0
+    assert Hh.rel_err(out.cpu().double(), oc) < 2e-5
+    assert Hh.rel_err(prob.cpu().double(), pc) < 2e-5
+    rowsum = torch.zeros(P.N, Hh.H, device=dev()).index_add_(0, edges[0], prob)
+    assert (rowsum - 1).abs().max() < 1e-5
+
+
+def test_attention_large_logits_and_long_rows():
+    """Rows longer than the 4 pairs in flight and logits of magnitude ~100: the running-maximum
+    softmax must neither overflow nor lose the small terms."""
+    P = Hh.make_problem(num_crystals=3, atoms_lo=17, atoms_hi=23, seed=73)
+    z, psi, gout = attention_case(P, 7, big_logits=True)
+    out64, leaves64, out, leaves = run_both(P, z, psi, gout)
+    assert torch.isfinite(out).all()
+    assert Hh.rel_err(out.cpu().double(), out64.detach()) < 2e-5
+    for l32, l64 in zip(leaves, leaves64):
+        assert Hh.rel_err(l32.grad.cpu().double(), l64.grad) < 5e-5
+
+
+def test_attention_single_atom_crystals_and_empty():
+    import crystalframer_amd as cf
+    P = Hh.make_problem(num_crystals=4, atoms_lo=1, atoms_hi=1, seed=74)
+    z, psi, gout = attention_case(P, 8)
+    out64, leaves64, out, leaves = run_both(P, z, psi, gout)
+    # one pair per atom: probability 1, out = v + b
+    assert Hh.rel_err(out.cpu().double(), (P.v.double() + psi)) < 1e-6
+    assert leaves[3].grad.abs().max() < 1e-5          # p (gp - D) cancels up to rounding
+    q = torch.zeros(0, Hh.H, Hh.DH, device=dev())
+    out = cf.FusedDotProductAttentionCUDA.apply(q, q, q, torch.zeros(0, Hh.H, device=dev()),
+                                                torch.zeros(0, Hh.H, Hh.DH, device=dev()),
+                                                torch.zeros(0, dtype=torch.long, device=dev()),
+                                                torch.zeros(2, 0, dtype=torch.long, device=dev()))
+    assert out.shape == (0, Hh.H, Hh.DH)
+
+
+def test_attention_backward_rejects_incomplete_pair_blocks():
+    import crystalframer_amd as cf
+    P = Hh.make_problem(num_crystals=3, atoms_lo=3, atoms_hi=4, seed=75)
+    keep = torch.ones(P.E, dtype=torch.bool)
+    keep[1] = False                                   # drop one pair: no longer n x n
+    edges = P.edges[:, keep].to(dev()).contiguous()
+    z, psi, gout = attention_case(P, 9)
+    leaves = [f32(t).requires_grad_(True) for t in (P.q, P.k, P.v, z[keep], psi[keep])]
+    out = cf.FusedDotProductAttentionCUDA.apply(*leaves, P.batch.to(dev()), edges)
+    # the forward needs no such layout and still matches
+    o64, _ = TO.softmax_attention(P.q.double(), P.k.double(), P.v.double(), z[keep], psi[keep], P.batch, P.edges[:, keep])
+    assert Hh.rel_err(out.detach().cpu().double(), o64) < 2e-5
+    with pytest.raises(ValueError, match="complete"):
+        out.sum().backward()
+
+
+def test_attention_full_batch_properties():
+    """Batch of 256 crystals: rows sum to one, out is a convex combination (bounded by the values),
+    the value gradients sum to the upstream gradient, and a constant shift of a row's logits changes
+    nothing."""
+    import crystalframer_amd as cf
+    from crystalframer_amd import geometry, synthetic
+    cb = synthetic.make_config("C3", seed=5).to(dev())
+    geo = geometry.crystal_geometry(cb.pos, cb.batch, cb.trans_vec, cb.sizes)
+    N, E, H, D = cb.pos.shape[0], geo.num_edges, 8, 16
+    g = torch.Generator(device="cpu").manual_seed(11)
+    q = (torch.randn(N, H, D, generator=g) / 4).to(dev())
+    k = torch.randn(N, H, D, generator=g).to(dev())
+    v = torch.randn(N, H, D, generator=g).to(dev()).requires_grad_(True)
+    a = torch.randn(E, H, generator=g).to(dev())
+    out = cf.FusedDotProductAttentionCUDA.apply(q, k, v, a, None, cb.batch, geo.edges)
+    vmax = torch.zeros(N, H, D, device=dev()).scatter_reduce(0, geo.edges[0][:, None, None].expand(-1, H, D),
+                                                             v.detach()[geo.edges[1]], reduce="amax", include_self=False)
+    assert (out.detach() <= vmax + 1e-5).all()
+    shift = torch.randn(N, H, generator=g).to(dev()) * 5
+    out2 = cf.FusedDotProductAttentionCUDA.apply(q, k, v, a + shift[geo.edges[0]], None, cb.batch, geo.edges)
+    assert (out2 - out).abs().max() < 2e-5
+    go = torch.randn(N, H, D, generator=g).to(dev())
+    (out * go).sum().backward()
+    # sum_j gv_j = sum_i go_i within each crystal (probabilities of a row sum to one)
+    per_crystal = lambda t: torch.zeros(cb.sizes.shape[0], H, D, device=dev()).index_add_(0, cb.batch, t)
+    assert Hh.rel_err(per_crystal(v.grad).cpu(), per_crystal(go).cpu()) < 1e-5
+
+
+def test_crystal_mean_forward_backward():
+    import crystalframer_amd as cf
+    sizes = torch.tensor([2, 1, 7, 4, 30])
+    batch = torch.repeat_interleave(torch.arange(5), sizes)
+    x64 = torch.randn(int(sizes.sum()), 128, dtype=torch.float64, requires_grad=True)
+    ref = TO.crystal_mean(x64, batch, 5)
+    gout = torch.randn(5, 128, dtype=torch.float64)
+    (ref * gout).sum().backward()
+    x = f32(x64.detach()).requires_grad_(True)
+    out = cf.IrregularMeanCUDA.apply(x, batch.to(dev()), sizes.to(dev()))
+    (out * f32(gout)).sum().backward()
+    assert Hh.rel_err(out.detach().cpu().double(), ref.detach()) < 1e-6
+    assert Hh.rel_err(x.grad.cpu().double(), x64.grad) < 1e-6
+    # sizes derived from batch, odd channel count
+    x3 = torch.randn(int(sizes.sum()), 5, device=dev())
+    out3 = cf.IrregularMeanCUDA.apply(x3, batch.to(dev()), None)
+    ref3 = TO.crystal_mean(x3.cpu().double(), batch, 5)
+    assert Hh.rel_err(out3.cpu().double(), ref3) < 1e-6
