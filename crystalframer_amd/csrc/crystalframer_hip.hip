@@ -29,9 +29,16 @@ int fail(int code, const char* fmt, ...) {
 }
 
 constexpr int MAX_HEADS = 64;
-constexpr size_t COUNTER_BYTES = 512;          // workspace header: 256 reserved bytes, then 32 uint64 statistics
+constexpr size_t QUEUE_OFFSET = 512;           // workspace header: 256 reserved bytes, 32 uint64 statistics, then the work queues
 constexpr size_t STATS_OFFSET = 256;
+constexpr size_t COUNTER_BYTES = QUEUE_OFFSET + (size_t)MAX_HEADS * cfh::NQUEUE * cfh::QSTRIDE * sizeof(int32_t);   // whole header
 constexpr int WAVES_PER_SIMD = 3;
+
+// workspace: header | item records (N, H, REC_WORDS) | per-wavefront weight-gradient partials
+size_t items_bytes(int64_t N, int H) {
+    const size_t raw = (size_t)N * (size_t)H * cfh::REC_WORDS * sizeof(uint32_t);
+    return (raw + 255) & ~(size_t)255;
+}
 
 // number of compute units of the current device (cached per device)
 int device_cus() {
@@ -150,7 +157,8 @@ void fill_common(cfh::KernelArgs& A, const cfh_params* p, const float* a_ih, con
     std::memset(&A, 0, sizeof(A));
     A.a_ih = a_ih; A.rpos = rpos; A.tvecs = tvecs; A.rvlen = rvlen;
     A.batch = batch; A.edges = edges; A.e_start = e_start; A.order = order;
-    A.counters = reinterpret_cast<int32_t*>(workspace);
+    A.counters = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(workspace) + QUEUE_OFFSET);
+    A.items = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(workspace) + COUNTER_BYTES);
     A.stats = p->collect_stats ? reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(workspace) + STATS_OFFSET) : nullptr;
     A.N = (int32_t)N; A.E = (int32_t)E; A.H = p->num_heads;
     A.cutoff_radius = rvlen ? p->cutoff_radius : 0.0f;
@@ -192,6 +200,8 @@ int resident_waves(Kern kern, int cap, int H) {
 template <typename Kern>
 int launch_persistent(Kern kern, const cfh::KernelArgs& A, int* waves, hipStream_t st, const char* what) {
     *waves = resident_waves(kern, *waves, A.H);
+    const int threads = A.N * A.H > A.H * cfh::NQUEUE ? A.N * A.H : A.H * cfh::NQUEUE;
+    hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, A, A.q != nullptr ? 1 : 0);
     hipLaunchKernelGGL(kern, dim3(*waves), dim3(cfh::WAVE), 0, st, A);
     return finish_launch(what);
 }
@@ -208,7 +218,7 @@ size_t cfh_workspace_bytes(const cfh_params* p, int64_t N, int64_t E) {
     (void)E;
     if (check_params(p) != CFH_OK) return 0;
     const int waves = launch_waves(N > 0 ? N : 1, p->num_heads);
-    return COUNTER_BYTES + (size_t)waves * 4 * cfh::DH * cfh::NBINS * sizeof(float);
+    return COUNTER_BYTES + items_bytes(N > 0 ? N : 1, p->num_heads) + (size_t)waves * 4 * cfh::DH * cfh::NBINS * sizeof(float);
 }
 
 int cfh_frame_axis1(const cfh_params* p, const float* q, const float* k, const float* a_ih,
@@ -221,7 +231,7 @@ int cfh_frame_axis1(const cfh_params* p, const float* q, const float* k, const f
     if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
     if (N == 0) return CFH_OK;
     if (!q || !k || !frame1) return fail(CFH_EINVAL, "q, k and frame1 must not be NULL");
-    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES))) return rc;
+    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES + items_bytes(N, p->num_heads)))) return rc;
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.q = q; A.k = k; A.out_frame = frame1;
@@ -239,7 +249,7 @@ int cfh_frame_axis2(const cfh_params* p, const float* q, const float* k, const f
     if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
     if (N == 0) return CFH_OK;
     if (!q || !k || !frame1 || !frame2max) return fail(CFH_EINVAL, "q, k, frame1 and frame2max must not be NULL");
-    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES))) return rc;
+    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES + items_bytes(N, p->num_heads)))) return rc;
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.q = q; A.k = k; A.frame1 = frame1; A.out_frame = frame2max;
@@ -257,7 +267,7 @@ int cfh_frame_axes(const cfh_params* p, const float* q, const float* k, const fl
     if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
     if (N == 0) return CFH_OK;
     if (!q || !k || !frames) return fail(CFH_EINVAL, "q, k and frames must not be NULL");
-    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES))) return rc;
+    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES + items_bytes(N, p->num_heads)))) return rc;
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.q = q; A.k = k; A.out_frame = frames;
@@ -295,7 +305,7 @@ int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* r
         return fail(CFH_EINVAL, "W_axis1..3 and frames must be given together");
     int wl = 0, wa = 0;
     if ((rc = window_widths(p, &wl, &wa))) return rc;
-    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES))) return rc;
+    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES + items_bytes(N, p->num_heads)))) return rc;
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.W[0] = W_dist; A.W[1] = W_axis1; A.W[2] = W_axis2; A.W[3] = W_axis3;
@@ -338,13 +348,13 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
     int wl = 0, wa = 0;
     if ((rc = window_widths(p, &wl, &wa))) return rc;
     int waves = launch_waves(N, p->num_heads);
-    const size_t need = COUNTER_BYTES + (size_t)waves * 4 * cfh::DH * cfh::NBINS * sizeof(float);
+    const size_t need = COUNTER_BYTES + items_bytes(N, p->num_heads) + (size_t)waves * 4 * cfh::DH * cfh::NBINS * sizeof(float);
     if ((rc = check_workspace(workspace, workspace_bytes, need))) return rc;
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.W[0] = W_dist; A.W[1] = W_axis1; A.W[2] = W_axis2; A.W[3] = W_axis3;
     A.frames = frames; A.z = z; A.gz = gz; A.gpsi = gpsi; A.out_ga = ga;
-    A.gw_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + COUNTER_BYTES);
+    A.gw_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + COUNTER_BYTES + items_bytes(N, p->num_heads));
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "framed_pe_backward";
     if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, true);

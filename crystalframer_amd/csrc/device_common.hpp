@@ -43,6 +43,37 @@ __device__ __forceinline__ float wave_min(float v) {
     for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, WAVE));
     return v;
 }
+// ---- reductions over a 16-lane row in DPP (VALU latency only; every lane must be active) --------
+// quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror: after the four steps all
+// 16 lanes of the row hold the reduction of the row.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row_min(float x) {
+    x = fminf(x, dpp_move<0xB1>(x));
+    x = fminf(x, dpp_move<0x4E>(x));
+    x = fminf(x, dpp_move<0x141>(x));
+    x = fminf(x, dpp_move<0x140>(x));
+    return x;
+}
+__device__ __forceinline__ float row_sum(float x) {
+    x += dpp_move<0xB1>(x);
+    x += dpp_move<0x4E>(x);
+    x += dpp_move<0x141>(x);
+    x += dpp_move<0x140>(x);
+    return x;
+}
+
+// Ordering point between the lanes of a ONE-wavefront workgroup that communicate through LDS.  The
+// LDS executes a wavefront's instructions in order, so no hardware barrier and no wait for
+// outstanding global stores is needed -- only the compiler must not move LDS accesses across.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // arg-min over (value, index): smallest value, then smallest index
 __device__ __forceinline__ void wave_argmin(float& v, int& idx) {
 #pragma unroll
@@ -236,7 +267,8 @@ struct KernelArgs {
     // outputs
     float* out_z; float* out_psi; float* out_d2min; float* out_frame; float* out_ga;
     float* gw_partial;            // (waves, 4, DH, NBINS) per-wave weight-gradient partials
-    int32_t* counters;            // (H) work-queue heads
+    int32_t* counters;            // (H, NQUEUE) work-queue heads
+    uint32_t* items;              // (N, H, REC_WORDS) item records of this launch
     unsigned long long* stats;    // optional running totals (see STAT_* below); never reset by a launch
     int32_t N, E, H;
     float cutoff_radius; int32_t lattice_range, minimum_range;
@@ -246,13 +278,114 @@ struct KernelArgs {
     BasisConsts bc;
 };
 
-// Work distribution.  Wavefront w (= blockIdx.x) serves head w % H and visits the items
-// w / H, w / H + W, w / H + 2 W, ... of that head, W = gridDim.x / H wavefronts per head.  Items are
-// visited in `order` (atoms by descending neighbour count), so every round hands all wavefronts
-// items of nearly equal cost.  A shared counter per head (one global atomic per item) was measured
-// first: the 19 000 same-address atomics of a launch serialise in L2 and cost more than the work.
-__device__ __forceinline__ int first_item(int H) { return (int)blockIdx.x / H; }
-__device__ __forceinline__ int item_stride(int H) { return (int)gridDim.x / H; }
+// Work distribution.  Wavefront w (= blockIdx.x) serves head w % H.  The items (atoms, visited in
+// `order`: descending neighbour count, i.e. longest first) of a head are dealt round-robin to NQUEUE
+// queues; a wavefront pops from queue (w / H) % NQUEUE with one global atomic per item and, when
+// that queue is empty, moves to any queue of its head that is not.  Measured alternatives: ONE
+// counter per head serialises its 2 400 same-address atomics (about 100 ns each) and costs more
+// than the work; a static deal leaves the average wavefront idle for 40 % of the launch, and any
+// wavefront that is not resident at launch doubles the makespan.
+constexpr int NQUEUE = 16;
+constexpr int QSTRIDE = 64;        // ints between two queue heads: each in a 256-byte block of its own
+// The lane that issues the atomic is picked through an opaque copy of the lane id: with a visible
+// `lane == 0` test here and another at the end of the caller's loop body the optimiser threads the
+// two branches and lanes 1..63 re-enter the loop on their own.
+__device__ __forceinline__ int queue_ticket(const KernelArgs& P, int h, int q) {
+    int v = 0;
+    int elect = threadIdx.x;
+    asm volatile("" : "+v"(elect));
+    if (elect == 0) v = atomicAdd(P.counters + (h * NQUEUE + q) * QSTRIDE, 1);
+    return v;         // valid in lane 0; not waited for until it is used
+}
+// Next item of head h, or -1 when every queue of the head is empty.  `q` is the queue to try first
+// and is updated.
+__device__ __forceinline__ int queue_pop(const KernelArgs& P, int h, int& q) {
+    for (;;) {
+        const int it = __builtin_amdgcn_readfirstlane(queue_ticket(P, h, q)) * NQUEUE + q;
+        if (it < P.N) return it;
+        bool more = false;
+        if (threadIdx.x < NQUEUE) {
+            const int c = __hip_atomic_load(P.counters + (h * NQUEUE + (int)threadIdx.x) * QSTRIDE, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT);
+            more = c * NQUEUE + (int)threadIdx.x < P.N;
+        }
+        const uint64_t m = __ballot(more);
+        if (m == 0) return -1;
+        q = __builtin_ctzll(m);
+    }
+}
+// Turns a ticket drawn earlier from queue q into an item; falls back to the other queues.
+__device__ __forceinline__ int queue_redeem(const KernelArgs& P, int h, int& q, int ticket) {
+    const int it = __builtin_amdgcn_readfirstlane(ticket) * NQUEUE + q;
+    return it < P.N ? it : queue_pop(P, h, q);
+}
+__device__ __forceinline__ int first_queue(int H) { return ((int)blockIdx.x / H) % NQUEUE; }
+
+// ---- item records ------------------------------------------------------------------------------
+// Everything a wavefront needs to start on item (it, h), gathered by prepare_items_kernel into one
+// 128-byte record so that the main kernels fetch it with ONE coalesced load, issued a whole item
+// ahead (the chain order -> batch -> lattice would be three dependent round trips per item):
+//   word 0 atom i, 1 first pair, 2 number of pairs, 3 R1 | R2 << 8 | R3 << 16, 4 a_ih,
+//   5..13 lattice rows, 14..22 frame axes (frame search: 14..29 the query vector q_ih)
+constexpr int REC_WORDS = 32;
+enum { REC_ATOM = 0, REC_E0 = 1, REC_NPAIRS = 2, REC_BOX = 3, REC_A = 4, REC_LATTICE = 5, REC_FRAMES = 14,
+       REC_QUERY = 14 };
+
+struct Item {
+    int i, e0, npairs;
+    float a;
+    Box bx;
+    Lattice L;
+};
+__device__ __forceinline__ float rec_f(uint32_t rec, int word) {
+    return __int_as_float(__builtin_amdgcn_readlane((int)rec, word));
+}
+__device__ __forceinline__ Item unpack_item(uint32_t rec) {
+    Item t;
+    t.i = __builtin_amdgcn_readlane((int)rec, REC_ATOM);
+    t.e0 = __builtin_amdgcn_readlane((int)rec, REC_E0);
+    t.npairs = __builtin_amdgcn_readlane((int)rec, REC_NPAIRS);
+    const int box = __builtin_amdgcn_readlane((int)rec, REC_BOX);
+    t.bx.R1 = box & 255; t.bx.R2 = (box >> 8) & 255; t.bx.R3 = (box >> 16) & 255;
+    t.bx.s2 = 2 * t.bx.R2 + 1; t.bx.s3 = 2 * t.bx.R3 + 1;
+    t.bx.T = (2 * t.bx.R1 + 1) * t.bx.s2 * t.bx.s3;
+    t.a = rec_f(rec, REC_A);
+#pragma unroll
+    for (int d = 0; d < 9; d++) t.L.t[d] = rec_f(rec, REC_LATTICE + d);
+    return t;
+}
+__device__ __forceinline__ uint32_t load_record(const KernelArgs& P, int it, int h) {
+    return (it >= 0 && threadIdx.x < REC_WORDS) ? P.items[((size_t)it * P.H + h) * REC_WORDS + threadIdx.x] : 0u;
+}
+
+// One thread per (item, head): builds the records and clears the work queues of the launch.
+__global__ __launch_bounds__(256) void prepare_items_kernel(const KernelArgs P, int with_query) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < P.H * NQUEUE) P.counters[idx * QSTRIDE] = 0;
+    if (idx >= P.N * P.H) return;
+    const int it = idx / P.H, h = idx - it * P.H;
+    const int i = P.order ? P.order[it] : it;
+    const int b = (int)P.batch[i];
+    const float a = P.a_ih[(size_t)i * P.H + h];
+    float rvl1 = 0.f, rvl2 = 0.f, rvl3 = 0.f;
+    if (P.rvlen) { rvl1 = P.rvlen[(size_t)b * 3 + 0]; rvl2 = P.rvlen[(size_t)b * 3 + 1]; rvl3 = P.rvlen[(size_t)b * 3 + 2]; }
+    const Box bx = translation_box(a, rvl1, rvl2, rvl3, P.cutoff_radius, P.lattice_range, P.minimum_range);
+    uint32_t* rec = P.items + (size_t)idx * REC_WORDS;
+    const int e0 = (int)P.e_start[i];
+    rec[REC_ATOM] = (uint32_t)i;
+    rec[REC_E0] = (uint32_t)e0;
+    rec[REC_NPAIRS] = (uint32_t)((int)P.e_start[i + 1] - e0);
+    rec[REC_BOX] = (uint32_t)(bx.R1 | (bx.R2 << 8) | (bx.R3 << 16));
+    rec[REC_A] = __float_as_uint(a);
+    for (int d = 0; d < 9; d++) rec[REC_LATTICE + d] = __float_as_uint(P.tvecs[(size_t)b * 9 + d]);
+    if (with_query) {
+        for (int c = 0; c < DH; c++) rec[REC_QUERY + c] = __float_as_uint(P.q[((size_t)i * P.H + h) * DH + c]);
+    } else if (P.frames) {
+        for (int ax = 0; ax < 3; ax++)
+            for (int d = 0; d < 3; d++)
+                rec[REC_FRAMES + ax * 3 + d] = __float_as_uint(P.frames[(((size_t)ax * P.N + i) * P.H + h) * 3 + d]);
+    }
+}
 
 // Counter-based uniform in [0,1) for the optional tie-breaking noise of the frame search.
 __device__ __forceinline__ float hash_uniform(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {

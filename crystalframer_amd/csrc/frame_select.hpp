@@ -59,32 +59,30 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
     const bool noisy = P.noise > 0.0f;
 
     unsigned long long st_raw = 0;
-    for (int it = first_item(H); it < P.N; it += item_stride(H)) {
-        const int i = P.order ? uniform_i(P.order[it]) : it;
-        const int b = uniform_i((int)P.batch[i]);
-        const float a = uniform_f(P.a_ih[(size_t)i * H + h]);
-        Lattice L;
-#pragma unroll
-        for (int d = 0; d < 9; d++) L.t[d] = uniform_f(P.tvecs[(size_t)b * 9 + d]);
-        float rvl1 = 0.f, rvl2 = 0.f, rvl3 = 0.f;
-        if (P.rvlen) {
-            rvl1 = uniform_f(P.rvlen[(size_t)b * 3 + 0]);
-            rvl2 = uniform_f(P.rvlen[(size_t)b * 3 + 1]);
-            rvl3 = uniform_f(P.rvlen[(size_t)b * 3 + 2]);
-        }
-        const Box bx = translation_box(a, rvl1, rvl2, rvl3, P.cutoff_radius, P.lattice_range,
-                                       P.minimum_range);
+    // software pipeline over items: record of item n+1 and queue ticket of item n+2 in flight
+    int queue = first_queue(H);
+    int it_cur = queue_pop(P, h, queue);
+    int it_next = it_cur >= 0 ? queue_pop(P, h, queue) : -1;
+    uint32_t rec_cur = load_record(P, it_cur, h);
+    while (it_cur >= 0) {
+        const int ticket = queue_ticket(P, h, queue);
+        const uint32_t rec_next = load_record(P, it_next, h);
+        const Item item = unpack_item(rec_cur);
+        const int i = item.i;
+        const float a = item.a;
+        const Lattice L = item.L;
+        const Box bx = item.bx;
         float qi[DH];
 #pragma unroll
-        for (int c = 0; c < DH; c++) qi[c] = uniform_f(P.q[((size_t)i * H + h) * DH + c]);
+        for (int c = 0; c < DH; c++) qi[c] = rec_f(rec_cur, REC_QUERY + c);
         const int nchunks = (bx.T + TCAP - 1) / TCAP;
         if (nchunks == 1) {
             __syncthreads();
             build_shift_table(tab, 0, bx.T, bx, L, lane);
             __syncthreads();
         }
-        const int e0 = uniform_i((int)P.e_start[i]);
-        const int e1 = uniform_i((int)P.e_start[i + 1]);
+        const int e0 = item.e0;
+        const int e1 = e0 + item.npairs;
 
         float f1x = 0.f, f1y = 0.f, f1z = 0.f;     // first axis (input in MODE 1, result otherwise)
         float f2x = 0.f, f2y = 0.f, f2z = 0.f;     // second axis before orthogonalisation
@@ -195,6 +193,9 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
             }
         }
         st_raw += (unsigned long long)bx.T * (unsigned long long)(e1 - e0);
+        it_cur = it_next;
+        rec_cur = rec_next;
+        it_next = it_cur >= 0 ? queue_redeem(P, h, queue, ticket) : -1;
     }
     if (P.stats && lane == 0) {      // once per wavefront
         if (MODE != 1) atomicAdd(P.stats + STAT_FRAME1_RAW, st_raw);

@@ -4,35 +4,47 @@
 //  models/cuda_funcs/real_space_framed_proj.py:63-105).
 //
 // Per (atom i, head h) item, pairs e=(i,j) taken GROUP at a time:
-//   per pair, lanes over translations n:
-//     pass A  d2min = min_n |r_ij + n.L|^2                                (6 VALU per translation)
+//   rounds of up to 4 pairs, one pair per 16-lane row, lanes of a row over the translations n:
+//     pass A  d2min = min_n |r_ij + n.L|^2                     (row reduction in DPP, no LDS)
 //     pass B  w_n = 2^(a'(d^2-d2min)); S = sum_n w_n; the translations with w_n >= 2^-prune are
 //             appended (ballot/prefix compaction) to the group's LDS list
 //   per group, lanes over the list:
 //     pass C  p = w/S; scatter p*g_k(d) into the pair's 9-bin distance window and p*g_m(cos(n,f_axis))
 //             into its three 33-bin angle windows (fixed-point LDS adds, Gaussians by recurrence)
-//   per pair:
-//     epilogue lane (enc,c): psi_enc[c] = W_enc[h,c,:] . hist_enc, W rows held in registers;
+//   per 4 pairs of the group:
+//     epilogue psi[pair, c] = sum_enc sum_k W_enc[h,c,k] hist[pair,enc,k] as 64 MFMA 4x4x1 steps:
+//             block (enc, c/4) of the instruction multiplies the 4 channels of its lanes' weight
+//             rows (held in registers for the whole launch) with the bins of 4 pairs;
 //             z = log S + a d2min.
 #pragma once
 #include "device_common.hpp"
 
 namespace cfh {
 
+constexpr int FWD_TCAP = 256;          // translations staged in LDS at a time (4 KB)
+constexpr int FWD_LISTCAP = 512;       // entries of the survivor list (a round that overflows it is repeated)
+constexpr int FWD_SHIFT = 13;          // list entry = pair-in-group << 13 | table index
+constexpr int FWD_ROWS = 4;            // pairs per round, one per 16-lane row
+static_assert(FWD_TCAP <= (1 << FWD_SHIFT) && (GROUP << FWD_SHIFT) <= 65536, "list entry is 16 bits");
+static_assert(GROUP % FWD_ROWS == 0 && WAVE % GROUP == 0, "rounds must not straddle groups or 64-pair rows");
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
 template <int WL, int WA, bool COS_ABS, bool HAS_LEN, bool HAS_ANG>
 __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P) {
-    __shared__ float4 tab[TCAP];
-    __shared__ uint16_t list[LISTCAP];
-    __shared__ uint32_t hist[GROUP * PAIR_STRIDE];
-    __shared__ __attribute__((aligned(16))) float shat[4 * HS];
+    __shared__ float4 tab[FWD_TCAP];
+    __shared__ uint16_t list[FWD_LISTCAP];
+    __shared__ __attribute__((aligned(16))) uint32_t hist[GROUP * PAIR_STRIDE];
     __shared__ float4 pairA[GROUP];        // rx, ry, rz, d2min of the pairs of the group
     __shared__ float2 pairS[GROUP];        // S and 2^31/S
 
     const int lane = threadIdx.x;
     const int H = P.H;
     const int h = blockIdx.x % H;
-    const int enc = lane >> 4;        // 0 = distance, 1..3 = frame axes
-    const int c = lane & 15;          // output channel
+    const int enc = lane >> 4;        // epilogue: 0 = distance, 1..3 = frame axes
+    const int c = lane & 15;          // epilogue: output channel of this lane's weight row
+    const int slot = lane >> 4;       // passes A/B: which pair of the round
+    const int tl = lane & 15;         // passes A/B: position in the row
 
     // this lane's row of the projection weights, W_enc[h, c, 0:64]
     float Wrow[NBINS];
@@ -45,60 +57,59 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
             Wrow[4 * k4 + 0] = v.x; Wrow[4 * k4 + 1] = v.y; Wrow[4 * k4 + 2] = v.z; Wrow[4 * k4 + 3] = v.w;
         }
     }
-    const float enc_coef = (enc == 0) ? P.dist_coef : P.angle_coef;
+    const float enc_scale = ((enc == 0) ? P.dist_coef : P.angle_coef) * FIX_INV;
     const BasisConsts bc = P.bc;
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
 
     for (int u = lane; u < GROUP * PAIR_STRIDE; u += WAVE) hist[u] = 0u;
-    __syncthreads();
+    wave_sync();
 
     unsigned long long st_eval = 0, st_raw = 0, st_pairs = 0;
-    for (int it = first_item(H); it < P.N; it += item_stride(H)) {
-        const int i = P.order ? uniform_i(P.order[it]) : it;
-        const int b = uniform_i((int)P.batch[i]);
-        const float a = uniform_f(P.a_ih[(size_t)i * H + h]);
+    // software pipeline over items: while item n is processed, the record of item n+1 and the
+    // queue ticket of item n+2 are in flight
+    int queue = first_queue(H);
+    int it_cur = queue_pop(P, h, queue);
+    int it_next = it_cur >= 0 ? queue_pop(P, h, queue) : -1;
+    uint32_t rec_cur = load_record(P, it_cur, h);
+    while (it_cur >= 0) {
+        const int ticket = queue_ticket(P, h, queue);
+        const uint32_t rec_next = load_record(P, it_next, h);
+        const Item item = unpack_item(rec_cur);
+        const int i = item.i;
+        const float a = item.a;
         const float a2 = a * LOG2E;
-        Lattice L;
-#pragma unroll
-        for (int d = 0; d < 9; d++) L.t[d] = uniform_f(P.tvecs[(size_t)b * 9 + d]);
-        float rvl1 = 0.f, rvl2 = 0.f, rvl3 = 0.f;
-        if (P.rvlen) {
-            rvl1 = uniform_f(P.rvlen[(size_t)b * 3 + 0]);
-            rvl2 = uniform_f(P.rvlen[(size_t)b * 3 + 1]);
-            rvl3 = uniform_f(P.rvlen[(size_t)b * 3 + 2]);
-        }
-        const Box bx = translation_box(a, rvl1, rvl2, rvl3, P.cutoff_radius, P.lattice_range,
-                                       P.minimum_range);
+        const Lattice L = item.L;
+        const Box bx = item.bx;
         float f[3][3];
         if (HAS_ANG) {
 #pragma unroll
             for (int ax = 0; ax < 3; ax++)
 #pragma unroll
-                for (int d = 0; d < 3; d++)
-                    f[ax][d] = uniform_f(P.frames[(((size_t)ax * P.N + i) * H + h) * 3 + d]);
+                for (int d = 0; d < 3; d++) f[ax][d] = rec_f(rec_cur, REC_FRAMES + ax * 3 + d);
         }
-        const int nchunks = (bx.T + TCAP - 1) / TCAP;
+        const int nchunks = (bx.T + FWD_TCAP - 1) / FWD_TCAP;
         if (nchunks == 1) {
-            __syncthreads();
+            wave_sync();
             build_shift_table(tab, 0, bx.T, bx, L, lane);
-            __syncthreads();
+            wave_sync();
         }
-        const int e0 = uniform_i((int)P.e_start[i]);
-        const int e1 = uniform_i((int)P.e_start[i + 1]);
+        const int e0 = item.e0;
+        const int npairs = item.npairs;
+        const int e1 = e0 + npairs;
         unsigned long long n_eval = 0;
         int nlist = 0;
 
-        // pass C over the current list; the table the entries point into must still be resident
+        // ---- pass C over the current list; the table the entries point into is still resident
         auto flush = [&]() {
-            __syncthreads();                       // list and pair data written
+            wave_sync();                           // list and pair data written
             if (HAS_LEN) {
                 const int nb = (nlist + WAVE - 1) / WAVE;
                 for (int bt = 0; bt < nb; bt++) {
                     const int idx = lane * nb + bt;       // every nb-th entry: lanes spread over the pairs
                     if (idx < nlist) {
                         const uint32_t ent = list[idx];
-                        const int el = ent >> (16 - GROUP_BITS);
-                        const float4 v = tab[ent & ((1u << (16 - GROUP_BITS)) - 1u)];
+                        const int el = ent >> FWD_SHIFT;
+                        const float4 v = tab[ent & ((1u << FWD_SHIFT) - 1u)];
                         const float4 pa = pairA[el];
                         const float dx = pa.x + v.x, dy = pa.y + v.y, dz = pa.z + v.z;
                         const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
@@ -137,132 +148,166 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
             }
             n_eval += (unsigned long long)nlist;
             nlist = 0;
-            __syncthreads();                       // list may be refilled, histograms may be read
+            wave_sync();                           // list may be refilled, histograms may be read
         };
 
-        for (int g0 = e0; g0 < e1; g0 += GROUP) {
-            const int ng = min(GROUP, e1 - g0);
-            for (int el = 0; el < ng; el++) {
-                const int e = g0 + el;
-                const float rx = uniform_f(P.rpos[(size_t)e * 3 + 0]);
-                const float ry = uniform_f(P.rpos[(size_t)e * 3 + 1]);
-                const float rz = uniform_f(P.rpos[(size_t)e * 3 + 2]);
-
-                // ---- pass A: nearest image
-                float d2min = 3.0e38f;
-                for (int ch = 0; ch < nchunks; ch++) {
-                    const int t0 = ch * TCAP;
-                    const int cnt = min(TCAP, bx.T - t0);
-                    if (nchunks > 1) {
-                        flush();
-                        build_shift_table(tab, t0, cnt, bx, L, lane);
-                        __syncthreads();
+        // ---- projection of the histograms of group g0 (ng pairs), stores, histograms cleared
+        auto epilogue = [&](int g0, int ng) {
+            if (HAS_LEN) {
+                const int sub = lane & 3;
+                for (int half = 0; half * 4 < ng; half++) {
+                    const int pl = half * 4 + sub;        // this lane's column of the MFMA: a pair
+                    uint4* hb = reinterpret_cast<uint4*>(hist + pl * PAIR_STRIDE + enc * HS);
+                    v4f acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int k4 = 0; k4 < NBINS / 4; k4++) {
+                        const uint4 hv = hb[k4];
+                        hb[k4] = make_uint4(0u, 0u, 0u, 0u);
+                        acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(Wrow[4 * k4 + 0], (float)hv.x, acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(Wrow[4 * k4 + 1], (float)hv.y, acc1, 0, 0, 0);
+                        acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(Wrow[4 * k4 + 2], (float)hv.z, acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(Wrow[4 * k4 + 3], (float)hv.w, acc1, 0, 0, 0);
                     }
-                    for (int u = lane; u < cnt; u += WAVE) {
+                    float o[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        float x = (acc0[r] + acc1[r]) * enc_scale;
+                        x += __shfl_xor(x, 16, WAVE);
+                        x += __shfl_xor(x, 32, WAVE);
+                        o[r] = x;
+                    }
+                    if (lane < 16 && pl < ng) {
+                        // lane (c/4 = lane>>2, pair = lane&3) holds channels 4*(lane>>2) .. +3
+                        float4* dst = reinterpret_cast<float4*>(P.out_psi + ((size_t)(g0 + pl) * H + h) * DH) + (lane >> 2);
+                        *dst = make_float4(o[0], o[1], o[2], o[3]);
+                    }
+                }
+            }
+            if (lane < ng) {
+                const float4 pa = pairA[lane];
+                P.out_z[(size_t)(g0 + lane) * H + h] = logf(pairS[lane].x) + pa.w * a;
+                if (P.out_d2min) P.out_d2min[(size_t)(g0 + lane) * H + h] = pa.w;
+            }
+            wave_sync();                           // pair data of this group no longer needed
+        };
+
+        // ---- rounds: (pairs el_glob .. el_glob+nslots of the row, chunk ch of the translations)
+        float prx = 0.f, pry = 0.f, prz = 0.f;     // rpos of pair (row base + lane)
+        float rx = 0.f, ry = 0.f, rz = 0.f, d2min = 0.f, S = 0.f;
+        int cur_g0 = -1, cur_ng = 0;
+        int el_glob = 0, ch = 0;
+        int skip = 0;          // survivors of the current round already processed (list overflow)
+        while (true) {
+            const bool done = el_glob >= npairs;
+            const int g0n = done ? -2 : e0 + (el_glob / GROUP) * GROUP;
+            const bool group_change = g0n != cur_g0;
+            if (nlist > 0 && (group_change || nchunks > 1 || skip > 0)) flush();
+            if (group_change && cur_g0 >= 0) epilogue(cur_g0, cur_ng);
+            if (done) break;
+            if (group_change) { cur_g0 = g0n; cur_ng = min(GROUP, e1 - g0n); }
+            if ((el_glob & (WAVE - 1)) == 0 && ch == 0) {      // next 64 pairs of the row
+                const int e = e0 + el_glob + lane;
+                if (e < e1) {
+                    prx = P.rpos[(size_t)e * 3 + 0];
+                    pry = P.rpos[(size_t)e * 3 + 1];
+                    prz = P.rpos[(size_t)e * 3 + 2];
+                }
+            }
+            const int el = (el_glob & (GROUP - 1)) + slot;      // pair-in-group of this row of lanes
+            const bool active = el < cur_ng;
+
+            if (ch == 0) {
+                const int src = (el_glob & (WAVE - 1)) + min(slot, WAVE - 1 - (el_glob & (WAVE - 1)));
+                rx = __shfl(prx, src, WAVE);
+                ry = __shfl(pry, src, WAVE);
+                rz = __shfl(prz, src, WAVE);
+                // ---- pass A: nearest image
+                d2min = 3.0e38f;
+                for (int cc = 0; cc < nchunks; cc++) {
+                    const int t0 = cc * FWD_TCAP;
+                    const int cnt = min(FWD_TCAP, bx.T - t0);
+                    if (nchunks > 1) {
+                        wave_sync();
+                        build_shift_table(tab, t0, cnt, bx, L, lane);
+                        wave_sync();
+                    }
+                    for (int u = tl; u < cnt; u += 16) {
                         const float4 v = tab[u];
                         const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
                         d2min = fminf(d2min, fmaf(dx, dx, fmaf(dy, dy, dz * dz)));
                     }
                 }
-                d2min = wave_min(d2min);
-
+                d2min = row_min(d2min);
                 // ---- the normaliser S when the table does not fit at once (otherwise pass B gives it)
-                float S = 0.0f;
                 if (nchunks > 1) {
-                    for (int ch = 0; ch < nchunks; ch++) {
-                        const int t0 = ch * TCAP;
-                        const int cnt = min(TCAP, bx.T - t0);
-                        __syncthreads();
+                    float Sb = 0.0f;
+                    for (int cc = 0; cc < nchunks; cc++) {
+                        const int t0 = cc * FWD_TCAP;
+                        const int cnt = min(FWD_TCAP, bx.T - t0);
+                        wave_sync();
                         build_shift_table(tab, t0, cnt, bx, L, lane);
-                        __syncthreads();
-                        for (int u = lane; u < cnt; u += WAVE) {
+                        wave_sync();
+                        for (int u = tl; u < cnt; u += 16) {
                             const float4 v = tab[u];
                             const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
-                            S += hw_exp2(a2 * (fmaf(dx, dx, fmaf(dy, dy, dz * dz)) - d2min));
+                            Sb += hw_exp2(a2 * (fmaf(dx, dx, fmaf(dy, dy, dz * dz)) - d2min));
                         }
                     }
-                    S = wave_sum(S);
-                    if (lane == 0) {
+                    S = row_sum(Sb);
+                    if (active && tl == 0) {
                         pairA[el] = make_float4(rx, ry, rz, d2min);
                         pairS[el] = make_float2(S, FIX_ONE / S);
                     }
                 }
+            }
 
-                // ---- pass B: weights, normaliser, compaction of the translations that matter
-                for (int ch = 0; ch < nchunks; ch++) {
-                    const int t0 = ch * TCAP;
-                    const int cnt = min(TCAP, bx.T - t0);
-                    if (nchunks > 1) {
-                        __syncthreads();
-                        build_shift_table(tab, t0, cnt, bx, L, lane);
-                        __syncthreads();
-                    } else if (nlist + cnt > LISTCAP) {
-                        flush();
+            // ---- pass B on chunk ch: weights, normaliser, compaction of the translations that matter
+            {
+                const int t0 = ch * FWD_TCAP;
+                const int cnt = min(FWD_TCAP, bx.T - t0);
+                if (nchunks > 1) {
+                    wave_sync();
+                    build_shift_table(tab, t0, cnt, bx, L, lane);
+                    wave_sync();
+                }
+                float Sb = 0.0f;
+                const int room = FWD_LISTCAP - nlist;
+                int seen = 0;                      // survivors met so far in this round
+                for (int u0 = 0; u0 < cnt; u0 += 16) {
+                    const int u = u0 + tl;
+                    bool keep = false;
+                    if (active && u < cnt) {
+                        const float4 v = tab[u];
+                        const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                        const float ex = a2 * (fmaf(dx, dx, fmaf(dy, dy, dz * dz)) - d2min);
+                        Sb += hw_exp2(ex);
+                        keep = ex >= prune;
                     }
-                    float Sb = 0.0f;
-                    for (int u0 = 0; u0 < cnt; u0 += WAVE) {
-                        const int u = u0 + lane;
-                        bool keep = false;
-                        if (u < cnt) {
-                            const float4 v = tab[u];
-                            const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
-                            const float ex = a2 * (fmaf(dx, dx, fmaf(dy, dy, dz * dz)) - d2min);
-                            Sb += hw_exp2(ex);
-                            keep = ex >= prune;
-                        }
-                        const uint64_t m = __ballot(keep);
-                        if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((el << (16 - GROUP_BITS)) | u);
-                        nlist += __popcll(m);
-                    }
-                    if (nchunks == 1) {
-                        S = wave_sum(Sb);
-                        if (lane == 0) {
-                            pairA[el] = make_float4(rx, ry, rz, d2min);
-                            pairS[el] = make_float2(S, FIX_ONE / S);
-                        }
-                    } else {
-                        flush();       // the entries point into this chunk of the table
+                    const uint64_t m = __ballot(keep);
+                    const int pos = seen + lane_prefix(m) - skip;     // slot after those already done
+                    if (keep && pos >= 0 && pos < room) list[nlist + pos] = (uint16_t)((el << FWD_SHIFT) | u);
+                    seen += __popcll(m);
+                }
+                const int appended = min(seen - skip, room);
+                nlist += appended;
+                skip = (skip + appended < seen) ? skip + appended : 0;   // > 0: repeat the round after a flush
+                if (nchunks == 1) {
+                    S = row_sum(Sb);
+                    if (active && tl == 0) {
+                        pairA[el] = make_float4(rx, ry, rz, d2min);
+                        pairS[el] = make_float2(S, FIX_ONE / S);
                     }
                 }
             }
-            flush();
-
-            // ---- per pair: histogram -> float bins, projection by this lane's weight row, stores
-            for (int el = 0; el < ng; el++) {
-                const int e = g0 + el;
-                if (HAS_LEN) {
-                    for (int u = lane; u < (HAS_ANG ? 4 : 1) * HS; u += WAVE)
-                        shat[u] = take_bin(hist + el * PAIR_STRIDE, u);
-                    __syncthreads();
-                    float acc = 0.0f;
-                    const float4* hrow = reinterpret_cast<const float4*>(shat + enc * HS);
-                    if (HAS_ANG || enc == 0) {
-#pragma unroll
-                        for (int k4 = 0; k4 < NBINS / 4; k4++) {
-                            const float4 hv = hrow[k4];
-                            acc = fmaf(Wrow[4 * k4 + 0], hv.x, acc);
-                            acc = fmaf(Wrow[4 * k4 + 1], hv.y, acc);
-                            acc = fmaf(Wrow[4 * k4 + 2], hv.z, acc);
-                            acc = fmaf(Wrow[4 * k4 + 3], hv.w, acc);
-                        }
-                    }
-                    acc *= enc_coef;
-                    acc += __shfl_xor(acc, 16, WAVE);
-                    acc += __shfl_xor(acc, 32, WAVE);
-                    if (lane < DH) P.out_psi[((size_t)e * H + h) * DH + lane] = acc;
-                    __syncthreads();               // shat is rewritten for the next pair
-                }
-                if (lane == 0) {
-                    const float d2min = pairA[el].w;
-                    P.out_z[(size_t)e * H + h] = logf(pairS[el].x) + d2min * a;
-                    if (P.out_d2min) P.out_d2min[(size_t)e * H + h] = d2min;
-                }
-            }
-            __syncthreads();                       // pair data of this group no longer needed
+            if (skip == 0 && ++ch == nchunks) { ch = 0; el_glob += FWD_ROWS; }
         }
         st_eval += n_eval;
-        st_raw += (unsigned long long)bx.T * (unsigned long long)(e1 - e0);
-        st_pairs += (unsigned long long)(e1 - e0);
+        st_raw += (unsigned long long)bx.T * (unsigned long long)npairs;
+        st_pairs += (unsigned long long)npairs;
+        (void)i;
+        it_cur = it_next;
+        rec_cur = rec_next;
+        it_next = it_cur >= 0 ? queue_redeem(P, h, queue, ticket) : -1;
     }
     // one set of atomics per wavefront (per-item atomics on three shared addresses serialise in L2)
     if (P.stats && lane == 0) {
