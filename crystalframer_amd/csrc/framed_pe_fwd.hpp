@@ -25,6 +25,7 @@ constexpr int FWD_TCAP = 256;          // translations staged in LDS at a time (
 constexpr int FWD_LISTCAP = 512;       // entries of the survivor list (a round that overflows it is repeated)
 constexpr int FWD_SHIFT = 13;          // list entry = pair-in-group << 13 | table index
 constexpr int FWD_ROWS = 4;            // pairs per round, one per 16-lane row
+constexpr int FAST_PER_LANE = 8;       // boxes of up to 128 translations: 8 per lane of a row, kept in registers
 static_assert(FWD_TCAP <= (1 << FWD_SHIFT) && (GROUP << FWD_SHIFT) <= 65536, "list entry is 16 bits");
 static_assert(GROUP % FWD_ROWS == 0 && WAVE % GROUP == 0, "rounds must not straddle groups or 64-pair rows");
 
@@ -154,32 +155,36 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
         // ---- projection of the histograms of group g0 (ng pairs), stores, histograms cleared
         auto epilogue = [&](int g0, int ng) {
             if (HAS_LEN) {
-                const int sub = lane & 3;
+                const int sub = lane & 3;          // A row of this lane: a pair; B column: channel 4 cg + sub
+                const int cg = (lane >> 2) & 3;
                 for (int half = 0; half * 4 < ng; half++) {
-                    const int pl = half * 4 + sub;        // this lane's column of the MFMA: a pair
-                    uint4* hb = reinterpret_cast<uint4*>(hist + pl * PAIR_STRIDE + enc * HS);
+                    // block (enc, cg) supplies the bins 16 cg .. 16 cg + 15 of its encoding; each of the
+                    // four MFMA of a step broadcasts the A operand of one cg to all four blocks of enc
+                    uint4* hb = reinterpret_cast<uint4*>(hist + (half * 4 + sub) * PAIR_STRIDE + enc * HS + 16 * cg);
+                    float hv[16];
+#pragma unroll
+                    for (int k4 = 0; k4 < 4; k4++) {
+                        const uint4 t4 = hb[k4];
+                        hb[k4] = make_uint4(0u, 0u, 0u, 0u);
+                        hv[4 * k4 + 0] = (float)t4.x; hv[4 * k4 + 1] = (float)t4.y;
+                        hv[4 * k4 + 2] = (float)t4.z; hv[4 * k4 + 3] = (float)t4.w;
+                    }
                     v4f acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int k4 = 0; k4 < NBINS / 4; k4++) {
-                        const uint4 hv = hb[k4];
-                        hb[k4] = make_uint4(0u, 0u, 0u, 0u);
-                        acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(Wrow[4 * k4 + 0], (float)hv.x, acc0, 0, 0, 0);
-                        acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(Wrow[4 * k4 + 1], (float)hv.y, acc1, 0, 0, 0);
-                        acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(Wrow[4 * k4 + 2], (float)hv.z, acc0, 0, 0, 0);
-                        acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(Wrow[4 * k4 + 3], (float)hv.w, acc1, 0, 0, 0);
+                    for (int s = 0; s < 16; s++) {
+                        acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(hv[s], Wrow[s], acc0, 2, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(hv[s], Wrow[16 + s], acc1, 2, 1, 0);
+                        acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(hv[s], Wrow[32 + s], acc0, 2, 2, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(hv[s], Wrow[48 + s], acc1, 2, 3, 0);
                     }
-                    float o[4];
+                    // lane (enc, c = lane & 15), component r: pair half*4 + r
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
                         float x = (acc0[r] + acc1[r]) * enc_scale;
                         x += __shfl_xor(x, 16, WAVE);
                         x += __shfl_xor(x, 32, WAVE);
-                        o[r] = x;
-                    }
-                    if (lane < 16 && pl < ng) {
-                        // lane (c/4 = lane>>2, pair = lane&3) holds channels 4*(lane>>2) .. +3
-                        float4* dst = reinterpret_cast<float4*>(P.out_psi + ((size_t)(g0 + pl) * H + h) * DH) + (lane >> 2);
-                        *dst = make_float4(o[0], o[1], o[2], o[3]);
+                        if (lane < DH && half * 4 + r < ng)
+                            P.out_psi[((size_t)(g0 + half * 4 + r) * H + h) * DH + lane] = x;
                     }
                 }
             }
@@ -197,6 +202,10 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
         int cur_g0 = -1, cur_ng = 0;
         int el_glob = 0, ch = 0;
         int skip = 0;          // survivors of the current round already processed (list overflow)
+        const bool fast = bx.T <= 16 * FAST_PER_LANE;      // one slab: distances stay in registers
+        float d2r[FAST_PER_LANE];
+#pragma unroll
+        for (int k = 0; k < FAST_PER_LANE; k++) d2r[k] = 0.0f;
         while (true) {
             const bool done = el_glob >= npairs;
             const int g0n = done ? -2 : e0 + (el_glob / GROUP) * GROUP;
@@ -223,18 +232,30 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                 rz = __shfl(prz, src, WAVE);
                 // ---- pass A: nearest image
                 d2min = 3.0e38f;
-                for (int cc = 0; cc < nchunks; cc++) {
-                    const int t0 = cc * FWD_TCAP;
-                    const int cnt = min(FWD_TCAP, bx.T - t0);
-                    if (nchunks > 1) {
-                        wave_sync();
-                        build_shift_table(tab, t0, cnt, bx, L, lane);
-                        wave_sync();
-                    }
-                    for (int u = tl; u < cnt; u += 16) {
-                        const float4 v = tab[u];
+                if (fast) {
+                    // every lane keeps the squared distances of its 8 translations for pass B
+#pragma unroll
+                    for (int k = 0; k < FAST_PER_LANE; k++) {
+                        const int u = tl + 16 * k;
+                        const float4 v = tab[u];      // beyond T: stale words, masked by the select
                         const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
-                        d2min = fminf(d2min, fmaf(dx, dx, fmaf(dy, dy, dz * dz)));
+                        d2r[k] = (u < bx.T) ? fmaf(dx, dx, fmaf(dy, dy, dz * dz)) : 3.0e38f;
+                        d2min = fminf(d2min, d2r[k]);
+                    }
+                } else {
+                    for (int cc = 0; cc < nchunks; cc++) {
+                        const int t0 = cc * FWD_TCAP;
+                        const int cnt = min(FWD_TCAP, bx.T - t0);
+                        if (nchunks > 1) {
+                            wave_sync();
+                            build_shift_table(tab, t0, cnt, bx, L, lane);
+                            wave_sync();
+                        }
+                        for (int u = tl; u < cnt; u += 16) {
+                            const float4 v = tab[u];
+                            const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                            d2min = fminf(d2min, fmaf(dx, dx, fmaf(dy, dy, dz * dz)));
+                        }
                     }
                 }
                 d2min = row_min(d2min);
@@ -273,20 +294,35 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                 float Sb = 0.0f;
                 const int room = FWD_LISTCAP - nlist;
                 int seen = 0;                      // survivors met so far in this round
-                for (int u0 = 0; u0 < cnt; u0 += 16) {
-                    const int u = u0 + tl;
-                    bool keep = false;
-                    if (active && u < cnt) {
-                        const float4 v = tab[u];
-                        const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
-                        const float ex = a2 * (fmaf(dx, dx, fmaf(dy, dy, dz * dz)) - d2min);
-                        Sb += hw_exp2(ex);
-                        keep = ex >= prune;
+                if (fast) {
+#pragma unroll
+                    for (int k = 0; k < FAST_PER_LANE; k++) {
+                        const int u = tl + 16 * k;
+                        const bool valid = active && u < cnt;
+                        const float ex = a2 * (d2r[k] - d2min);
+                        Sb += valid ? hw_exp2(ex) : 0.0f;
+                        const bool keep = valid && ex >= prune;
+                        const uint64_t m = __ballot(keep);
+                        const int pos = seen + lane_prefix(m) - skip;     // slot after those already done
+                        if (keep && pos >= 0 && pos < room) list[nlist + pos] = (uint16_t)((el << FWD_SHIFT) | u);
+                        seen += __popcll(m);
                     }
-                    const uint64_t m = __ballot(keep);
-                    const int pos = seen + lane_prefix(m) - skip;     // slot after those already done
-                    if (keep && pos >= 0 && pos < room) list[nlist + pos] = (uint16_t)((el << FWD_SHIFT) | u);
-                    seen += __popcll(m);
+                } else {
+                    for (int u0 = 0; u0 < cnt; u0 += 16) {
+                        const int u = u0 + tl;
+                        bool keep = false;
+                        if (active && u < cnt) {
+                            const float4 v = tab[u];
+                            const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                            const float ex = a2 * (fmaf(dx, dx, fmaf(dy, dy, dz * dz)) - d2min);
+                            Sb += hw_exp2(ex);
+                            keep = ex >= prune;
+                        }
+                        const uint64_t m = __ballot(keep);
+                        const int pos = seen + lane_prefix(m) - skip;
+                        if (keep && pos >= 0 && pos < room) list[nlist + pos] = (uint16_t)((el << FWD_SHIFT) | u);
+                        seen += __popcll(m);
+                    }
                 }
                 const int appended = min(seen - skip, room);
                 nlist += appended;
