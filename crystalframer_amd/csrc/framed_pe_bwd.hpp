@@ -289,21 +289,44 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
                 float Ap = 0.0f;
                 const int room = BWD_LISTCAP - nlist;
                 int seen = 0;
-                for (int u0 = 0; u0 < cnt; u0 += 16) {
-                    const int u = u0 + tl;
-                    bool keep = false;
-                    if (active && u < cnt) {
-                        const float4 v = tab[u];
+                if (bx.T <= 128) {
+                    // one slab of 8 translations per lane: all table reads are issued before the arithmetic
+                    float d2r[8];
+#pragma unroll
+                    for (int k = 0; k < 8; k++) {
+                        const float4 v = tab[tl + 16 * k];       // beyond T: stale words, masked below
                         const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
-                        const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
-                        const float ex = fmaf(a2, d2, -z2);
-                        if (nchunks == 1) Ap = fmaf(hw_exp2(ex), d2, Ap);
-                        keep = ex >= prune;
+                        d2r[k] = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
                     }
-                    const uint64_t m = __ballot(keep);
-                    const int pos = seen + lane_prefix(m) - skip;
-                    if (keep && pos >= 0 && pos < room) list[nlist + pos] = (uint16_t)((el << BWD_SHIFT) | u);
-                    seen += __popcll(m);
+#pragma unroll
+                    for (int k = 0; k < 8; k++) {
+                        const int u = tl + 16 * k;
+                        const bool valid = active && u < cnt;
+                        const float ex = fmaf(a2, d2r[k], -z2);
+                        Ap += valid ? hw_exp2(ex) * d2r[k] : 0.0f;
+                        const bool keep = valid && ex >= prune;
+                        const uint64_t m = __ballot(keep);
+                        const int pos = seen + lane_prefix(m) - skip;
+                        if (keep && pos >= 0 && pos < room) list[nlist + pos] = (uint16_t)((el << BWD_SHIFT) | u);
+                        seen += __popcll(m);
+                    }
+                } else {
+                    for (int u0 = 0; u0 < cnt; u0 += 16) {
+                        const int u = u0 + tl;
+                        bool keep = false;
+                        if (active && u < cnt) {
+                            const float4 v = tab[u];
+                            const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                            const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+                            const float ex = fmaf(a2, d2, -z2);
+                            if (nchunks == 1) Ap = fmaf(hw_exp2(ex), d2, Ap);
+                            keep = ex >= prune;
+                        }
+                        const uint64_t m = __ballot(keep);
+                        const int pos = seen + lane_prefix(m) - skip;
+                        if (keep && pos >= 0 && pos < room) list[nlist + pos] = (uint16_t)((el << BWD_SHIFT) | u);
+                        seen += __popcll(m);
+                    }
                 }
                 const int appended = min(seen - skip, room);
                 nlist += appended;

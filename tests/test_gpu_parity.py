@@ -27,7 +27,7 @@ def _defaults():
     KM = cf.KernelManager
     saved = (KM.SYMM_BREAK_NOISE, KM.PRUNE_LOG2, KM.WINDOW_MODE, KM.GRAD_COEF_QUIRK, KM.LATTICE_RANGE, KM.MINIMUM_RANGE)
     KM.SYMM_BREAK_NOISE = 0.0
-    KM.PRUNE_LOG2 = 32.0
+    KM.PRUNE_LOG2 = 24.0
     KM.WINDOW_MODE = 0
     KM.GRAD_COEF_QUIRK = False
     KM.LATTICE_RANGE, KM.MINIMUM_RANGE = 2, 2
@@ -70,7 +70,7 @@ def oracle_pe(P, *, K=64, A=64, cos_abs=0, cd=1.0, ca=1.0, cutoff=CUT, windows="
 
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("cos_abs", [0, 1])
-@pytest.mark.parametrize("prune", [0.0, 32.0])
+@pytest.mark.parametrize("prune", [0.0, 24.0, 32.0])
 def test_framed_pe_forward_backward_reference_windows(cos_abs, prune):
     import crystalframer_amd as cf
     cf.KernelManager.PRUNE_LOG2 = prune
