@@ -45,6 +45,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="launch every kernel from Python instead of replaying the step as one HIP graph")
     ap.add_argument("--cpu-crystals", type=int, default=12, help="crystals of the batch in the CPU sample")
     return ap.parse_args()
 
@@ -97,7 +99,14 @@ def main():
     cb_cpu = synthetic.make_config("C3", seed=123, num_crystals=args.batch)
     cb = cb_cpu.to(dev)
     target = torch.randn(args.batch, 1, generator=torch.Generator().manual_seed(7)).to(dev)
-    opt = torch.optim.AdamW(model.parameters(), lr=5e-4, betas=(0.9, 0.98), weight_decay=1e-5)
+    use_graph = not args.no_graph
+    opt = torch.optim.AdamW(model.parameters(), lr=5e-4, betas=(0.9, 0.98), weight_decay=1e-5,
+                            capturable=use_graph)
+    # the tie-breaking noise of the frame search: seed word on the device, advanced by every call, so
+    # that replays of the captured step draw fresh noise like separate launches do
+    KM.NOISE_SEED = 20240607
+    KM.NOISE_SEED_DEVICE = torch.zeros(1, dtype=torch.int64, device=dev)
+    loss_out = torch.zeros((), device=dev)
 
     def step():
         opt.zero_grad(set_to_none=True)
@@ -105,18 +114,37 @@ def main():
         loss = torch.nn.functional.mse_loss(out, target)
         loss.backward()
         opt.step()
-        return loss
+        loss_out.copy_(loss.detach())
 
-    for _ in range(args.warmup):
-        step()
+    if use_graph:
+        # the whole training step (geometry, 4 layers forward, loss, backward, AdamW) as ONE HIP graph:
+        # the step is ~450 small launches and Python cannot issue them as fast as the GPU retires them
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(max(args.warmup, 3)):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        run_step = graph.replay
+        for _ in range(2):
+            run_step()
+    else:
+        run_step = step
+        for _ in range(args.warmup):
+            step()
     torch.cuda.synchronize()
 
     # ---- timed region: exactly K steps
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        run_step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    final_loss = float(loss_out)
     ms_per_step = dt / args.steps * 1e3
     crystals_per_s = args.batch / (dt / args.steps)
 
@@ -185,7 +213,9 @@ def main():
                    "global_batch": args.batch, "atoms": int(cb.pos.shape[0]),
                    "atom_pairs": int((cb_cpu.sizes ** 2).sum()), "heads": 8, "head_dim": 16,
                    "dist_bins": 64, "angle_bins": 64, "adaptive_cutoff_sigma": -3.5, "prune_log2": KM.PRUNE_LOG2,
-                   "windows": "reference (9/33 bins)", "optimizer": "adamw", "parallelism": "single GPU"},
+                   "windows": "reference (9/33 bins)", "optimizer": "adamw", "parallelism": "single GPU",
+                   "launch": "one HIP graph per step" if use_graph else "eager"},
+        "final_loss": final_loss,
         "roofline": roofline,
         "lattice_terms": terms,
         "kernel_ms": avg_ms, "kernel_launches_per_step": launches, "library_ms_per_step": lib_ms_per_step,

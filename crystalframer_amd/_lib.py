@@ -42,6 +42,7 @@ class CfhParams(ctypes.Structure):
         ("noise_seed", ctypes.c_uint64),
         ("grad_coef_quirk", ctypes.c_int32),
         ("collect_stats", ctypes.c_int32),
+        ("noise_seed_dev", ctypes.c_void_p),
     ]
 
 

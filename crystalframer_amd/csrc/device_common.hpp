@@ -275,6 +275,7 @@ struct KernelArgs {
     float prune_log2;             // <= 0: keep every translation
     float dist_coef, angle_coef, gz_coef, gw_dist_coef;
     float noise; uint32_t seed_lo, seed_hi;
+    const unsigned long long* seed_dev;   // optional device word mixed into the seed
     BasisConsts bc;
 };
 

@@ -12,9 +12,10 @@
 // 1e-5)) for the second -- so every lane keeps a running best over its own translations of every
 // pair and the wavefront reduces once per item.  Tie rule with zero noise: lowest pair index, then
 // first translation in the reference's loop order (what its strict comparisons and the plain
-// arg-max over pairs give).  With noise > 0 every candidate's key is perturbed by a counter-based
-// uniform in (-noise/2, noise/2) (the reference draws from cuRAND XORWOW seeded by numpy; its
-// stream cannot be reproduced).
+// arg-max over pairs give).  With noise > 0 every candidate's key is perturbed by a uniform in
+// (-noise/2, noise/2): a golden-ratio sequence over the translations with a hashed phase per
+// (pair, head, pass, seed) -- three operations per candidate (the reference draws from cuRAND
+// XORWOW seeded by numpy; its stream cannot be reproduced, only its distribution).
 //
 // MODE 0: first axis only.  MODE 1: second axis for a given first axis.  MODE 2: both, then
 // Gram-Schmidt and the cross product, written as (3,N,H,3) orthonormal frames.
@@ -57,6 +58,12 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
     const int H = P.H;
     const int h = blockIdx.x % H;
     const bool noisy = P.noise > 0.0f;
+    uint32_t seed_lo = P.seed_lo, seed_hi = P.seed_hi;
+    if (noisy && P.seed_dev) {
+        const unsigned long long s = *P.seed_dev;
+        seed_lo ^= (uint32_t)s * 0x9E3779B1u;
+        seed_hi += (uint32_t)(s >> 32) ^ ((uint32_t)s * 0x85EBCA77u);
+    }
 
     unsigned long long st_raw = 0;
     // software pipeline over items: record of item n+1 and queue ticket of item n+2 in flight
@@ -128,22 +135,26 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                     for (int el = 0; el < ne; el++) {
                         const float4 rq = pair_rq[el];
                         const int e = eb + el;
+                        // per (pair, head, pass) phase of the tie-breaking noise (uniform: scalar unit)
+                        const float phase = noisy ? hash_uniform(pass ? seed_hi : seed_lo, pass ? seed_lo : seed_hi,
+                                                                 (uint32_t)(e * H + h), (uint32_t)pass) : 0.0f;
                         for (int u = lane; u < cnt; u += WAVE) {
                             const float4 v = tab[u];
                             const float dx = rq.x + v.x, dy = rq.y + v.y, dz = rq.z + v.z;
                             const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
-                            float d2k = d2;
-                            if (noisy && pass == 0)
-                                d2k += (hash_uniform(P.seed_lo, P.seed_hi, (uint32_t)(e * H + h), (uint32_t)(t0 + u)) - 0.5f) * P.noise;
-                            float score = fmaf(a, d2k, rq.w);
+                            float score = fmaf(a, d2, rq.w);
                             bool ok = d2 > 1e-5f;
                             if (pass == 1) {
                                 const float rinv = hw_rsq(d2);
                                 const float ac = fabsf((dx * f1x + dy * f1y + dz * f1z) * rinv);
                                 score += hw_log2(fmaxf(1.0f - ac, 1e-5f)) * LN2;
-                                if (noisy)
-                                    score += (hash_uniform(P.seed_hi, P.seed_lo, (uint32_t)(e * H + h), (uint32_t)(t0 + u)) - 0.5f) * P.noise;
                                 ok = ok && ac < 0.9999f;
+                            }
+                            if (noisy) {
+                                // uniform in [0,1): golden-ratio sequence over the translations, phase per pair
+                                const float un = __builtin_amdgcn_fractf(fmaf((float)(t0 + u), 0.61803399f, phase));
+                                if (pass == 0) score = fmaf(a, d2 + (un - 0.5f) * P.noise, rq.w);
+                                else score += (un - 0.5f) * P.noise;
                             }
                             // a lane meets its candidates in ascending (e, t) order when the table is
                             // one chunk: the strict comparison keeps the first; with several chunks the

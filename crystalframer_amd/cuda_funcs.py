@@ -28,6 +28,10 @@ class KernelManager:
     MINIMUM_RANGE: int = 2
     SYMM_BREAK_NOISE: float = 1e-5
     NOISE_SEED: Optional[int] = None    # None: a fresh seed per call, as the reference draws one
+    # a one-element int64 device tensor: mixed into the seed on the device and advanced after every
+    # frame search, so that replays of a captured HIP graph (where NOISE_SEED is frozen) still draw
+    # fresh noise
+    NOISE_SEED_DEVICE: Optional[torch.Tensor] = None
     # options of this implementation (no reference counterpart)
     WINDOW_MODE: int = _lib.CFH_WINDOW_REFERENCE
     # skip translations lighter than 2^-24 of their pair's heaviest: below the float32 resolution of the
@@ -81,6 +85,8 @@ def _params(H: int, Dh: int, K: int, A: int, cos_abs: int, dist_max: float, wsca
         p.noise_seed = int(torch.randint(0, 2 ** 62, (1,)).item()) if p.symm_break_noise > 0 else 0
     else:
         p.noise_seed = int(KernelManager.NOISE_SEED)
+    sd = KernelManager.NOISE_SEED_DEVICE
+    p.noise_seed_dev = sd.data_ptr() if (sd is not None and p.symm_break_noise > 0) else None
     p.grad_coef_quirk = int(bool(KernelManager.GRAD_COEF_QUIRK))
     p.collect_stats = int(bool(KernelManager.COLLECT_STATS))
     return p
@@ -172,7 +178,7 @@ def _frame_call(mode: int, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, f
     rv = _f32c(rvlen_n)
     batch, edges = batch_i.contiguous(), edge_ij_e.contiguous()
     e_start, order = edge_schedule(edge_ij_e, N)
-    out = torch.zeros((3, N, H, 3) if mode == 2 else (N, H, 3), dtype=torch.float32, device=dev)
+    out = torch.empty((3, N, H, 3) if mode == 2 else (N, H, 3), dtype=torch.float32, device=dev)
     p = _params(H, Dh, 0, 0, 0, 1.0, 1.0, 1.0, 1.0, 1.0, cutoff_radius if rv is not None else None)
     with torch.cuda.device(dev), _timed(("frame_axis1", "frame_axis2", "frame_axes")[mode], dev):
         need = lib.cfh_workspace_bytes(ctypes.byref(p), N, E)
@@ -195,6 +201,8 @@ def _frame_call(mode: int, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, f
                                      _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(f1), N, E, tv.shape[0],
                                      _lib.ptr(out), _lib.ptr(ws), ws.numel(), st)
     _lib.check(rc, ("cfh_frame_axis1", "cfh_frame_axis2", "cfh_frame_axes")[mode])
+    if KernelManager.NOISE_SEED_DEVICE is not None and p.symm_break_noise > 0:
+        KernelManager.NOISE_SEED_DEVICE.add_(1)
     return out
 
 
@@ -433,8 +441,7 @@ class IrregularMeanCUDA(torch.autograd.Function):
         B = sizes.shape[0]
         N = x_ik.shape[0]
         C = x_ik[0].numel() if N else int(torch.tensor(x_ik.shape[1:]).prod())
-        atom_start = torch.zeros(B + 1, dtype=torch.long, device=dev)
-        atom_start[1:] = sizes.to(device=dev, dtype=torch.long).cumsum(0)
+        atom_start = torch.nn.functional.pad(sizes.to(device=dev, dtype=torch.long).cumsum(0), (1, 0))
         x = _f32c(x_ik)
         out = torch.empty((B,) + tuple(x_ik.shape[1:]), dtype=torch.float32, device=dev)
         with _timed("crystal_mean_forward", dev):

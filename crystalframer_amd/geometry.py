@@ -50,7 +50,7 @@ def edge_start_from_edges(edges: torch.Tensor, num_atoms: int) -> torch.Tensor:
 
 
 def crystal_geometry(pos: torch.Tensor, batch: torch.Tensor, trans: torch.Tensor,
-                     sizes: Optional[torch.Tensor] = None) -> CrystalGeometry:
+                     sizes: Optional[torch.Tensor] = None, num_edges: Optional[int] = None) -> CrystalGeometry:
     dev = pos.device
     B = trans.shape[0]
     N = pos.shape[0]
@@ -60,9 +60,11 @@ def crystal_geometry(pos: torch.Tensor, batch: torch.Tensor, trans: torch.Tensor
     sizes = sizes.to(device=dev, dtype=torch.long)
     n_of_atom = sizes[batch]                                   # neighbours per atom
     atom_start = torch.cumsum(sizes, 0) - sizes                # first atom of each crystal
-    e_start = torch.zeros(N + 1, dtype=torch.long, device=dev)
-    torch.cumsum(n_of_atom, 0, out=e_start[1:])
-    E = int(e_start[-1].item()) if N > 0 else 0
+    e_start = torch.nn.functional.pad(torch.cumsum(n_of_atom, 0), (1, 0))
+    if num_edges is not None:
+        E = int(num_edges)
+    else:
+        E = int(e_start[-1].item()) if N > 0 else 0
     i_of_e = torch.repeat_interleave(torch.arange(N, device=dev), n_of_atom, output_size=E)
     j_of_e = atom_start[batch[i_of_e]] + (torch.arange(E, device=dev) - e_start[i_of_e])
     edges = torch.stack([i_of_e, j_of_e]).contiguous()

@@ -22,10 +22,15 @@ class CrystalBatch:
     batch: torch.Tensor      # (N,) int64
     trans_vec: torch.Tensor  # (B, 3, 3) float32
     sizes: torch.Tensor      # (B,) int64
+    num_pairs: int = -1      # sum of sizes^2, known on the host (spares the model a device read); -1: unknown
+
+    def __post_init__(self):
+        if self.num_pairs < 0 and not self.sizes.is_cuda:
+            self.num_pairs = int((self.sizes.long() ** 2).sum())
 
     def to(self, device):
         return CrystalBatch(self.x.to(device), self.pos.to(device), self.batch.to(device),
-                            self.trans_vec.to(device), self.sizes.to(device))
+                            self.trans_vec.to(device), self.sizes.to(device), self.num_pairs)
 
     @property
     def num_crystals(self) -> int:

@@ -80,3 +80,67 @@ def test_model_frames_agree_with_oracle_frames():
     clear = (gap1 > 1e-4) & (gap2 > 1e-4)
     assert clear.double().mean() > 0.9
     assert (used[0].cpu().double() - f1)[clear].abs().max() < 1e-4
+
+
+def test_training_step_as_hip_graph_matches_eager_on_every_replay():
+    """The whole training step (geometry, forward, loss, backward, AdamW) captured as one HIP graph:
+    every replay is compared with an eager twin of the same model, with eager work and
+    synchronisations between the replays."""
+    import crystalframer_amd as cf
+    from crystalframer_amd import latticeformer, params, synthetic
+    KM = cf.KernelManager
+    dev = torch.device("cuda:0")
+    saved = (KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE)
+    mp = params.ModelParams(num_layers=2)
+    cb = synthetic.make_batch(24, atoms="uniform", atoms_lo=1, atoms_hi=9, len_lo=3.0, len_hi=9.0,
+                              ang_lo=65.0, ang_hi=115.0, seed=21).to(dev)
+    assert cb.num_pairs > 0          # host-known pair count: the geometry needs no device read
+    target = torch.linspace(-1, 1, cb.num_crystals, device=dev)[:, None]
+
+    def twin():
+        torch.manual_seed(5)
+        model = latticeformer.Latticeformer(mp).to(dev)
+        model.train()
+        opt = torch.optim.AdamW(model.parameters(), lr=1e-3, capturable=True)
+        seed_word = torch.zeros(1, dtype=torch.int64, device=dev)
+        loss_out = torch.zeros((), device=dev)
+
+        def step():
+            KM.NOISE_SEED_DEVICE = seed_word
+            opt.zero_grad(set_to_none=True)
+            loss = torch.nn.functional.mse_loss(model(cb), target)
+            loss.backward()
+            opt.step()
+            loss_out.copy_(loss.detach())
+        return model, step, loss_out
+
+    try:
+        KM.SYMM_BREAK_NOISE, KM.NOISE_SEED = 1e-5, 99
+        model_e, step_e, loss_e = twin()
+        model_g, step_g, loss_g = twin()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step_g()
+        torch.cuda.current_stream().wait_stream(side)
+        for _ in range(3):
+            step_e()
+        torch.cuda.synchronize()
+        assert abs(float(loss_e) - float(loss_g)) < 1e-4 * abs(float(loss_e))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step_g()
+        junk = torch.randn(512, 512, device=dev)
+        for replay in range(5):
+            step_e()
+            graph.replay()
+            torch.cuda.synchronize()
+            le, lg = float(loss_e), float(loss_g)
+            assert abs(le - lg) < 2e-4 * abs(le), (replay, le, lg)
+            junk = torch.tanh(junk @ junk / 512.0)          # eager work between the replays
+            assert torch.isfinite(junk).all()
+        for (n, pe), (_, pg) in zip(model_e.named_parameters(), model_g.named_parameters()):
+            assert Hh.rel_err(pg, pe.detach().cpu()) < 5e-3, n
+    finally:
+        KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE = saved
