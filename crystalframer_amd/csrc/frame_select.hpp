@@ -83,10 +83,11 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
 #pragma unroll
         for (int c = 0; c < DH; c++) qi[c] = rec_f(rec_cur, REC_QUERY + c);
         const int nchunks = (bx.T + TCAP - 1) / TCAP;
-        if (nchunks == 1) {
-            __syncthreads();
-            build_shift_table(tab, 0, bx.T, bx, L, lane);
-            __syncthreads();
+        float sx[TCAP / WAVE], sy[TCAP / WAVE], sz[TCAP / WAVE];
+#pragma unroll
+        for (int k = 0; k < TCAP / WAVE; k++) {
+            sx[k] = sy[k] = sz[k] = 0.0f;
+            if (nchunks == 1 && k * WAVE < bx.T) shift_of(min(lane + k * WAVE, bx.T - 1), bx, L, sx[k], sy[k], sz[k]);
         }
         const int e0 = item.e0;
         const int e1 = e0 + item.npairs;
@@ -124,44 +125,59 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                 }
                 __syncthreads();
                 const int ne = min(WAVE, e1 - eb);
-                for (int ch = 0; ch < nchunks; ch++) {
-                    const int t0 = ch * TCAP;
-                    const int cnt = min(TCAP, bx.T - t0);
-                    if (nchunks > 1) {
-                        __syncthreads();
-                        build_shift_table(tab, t0, cnt, bx, L, lane);
-                        __syncthreads();
+                // one candidate: pair e shifted by (vx,vy,vz), translation index t
+                auto consider = [&](const float4& rq, float phase, int e, int t, float vx, float vy, float vz) {
+                    const float dx = rq.x + vx, dy = rq.y + vy, dz = rq.z + vz;
+                    const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+                    float score = fmaf(a, d2, rq.w);
+                    bool ok = d2 > 1e-5f;
+                    if (pass == 1) {
+                        const float rinv = hw_rsq(d2);
+                        const float ac = fabsf((dx * f1x + dy * f1y + dz * f1z) * rinv);
+                        score += hw_log2(fmaxf(1.0f - ac, 1e-5f)) * LN2;
+                        ok = ok && ac < 0.9999f;
                     }
+                    if (noisy) {
+                        // uniform in [0,1): golden-ratio sequence over the translations, phase per pair
+                        const float un = __builtin_amdgcn_fractf(fmaf((float)t, 0.61803399f, phase));
+                        if (pass == 0) score = fmaf(a, d2 + (un - 0.5f) * P.noise, rq.w);
+                        else score += (un - 0.5f) * P.noise;
+                    }
+                    // largest score, then lowest pair, then lowest translation
+                    if (ok && (score > best.score ||
+                               (score == best.score && (e < best.e || (e == best.e && t < best.t))))) {
+                        best.score = score; best.e = e; best.t = t;
+                    }
+                };
+                if (nchunks == 1) {
+                    // the shifts of this lane's translations (t = lane + 64 k) stay in registers
                     for (int el = 0; el < ne; el++) {
                         const float4 rq = pair_rq[el];
                         const int e = eb + el;
-                        // per (pair, head, pass) phase of the tie-breaking noise (uniform: scalar unit)
                         const float phase = noisy ? hash_uniform(pass ? seed_hi : seed_lo, pass ? seed_lo : seed_hi,
                                                                  (uint32_t)(e * H + h), (uint32_t)pass) : 0.0f;
-                        for (int u = lane; u < cnt; u += WAVE) {
-                            const float4 v = tab[u];
-                            const float dx = rq.x + v.x, dy = rq.y + v.y, dz = rq.z + v.z;
-                            const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
-                            float score = fmaf(a, d2, rq.w);
-                            bool ok = d2 > 1e-5f;
-                            if (pass == 1) {
-                                const float rinv = hw_rsq(d2);
-                                const float ac = fabsf((dx * f1x + dy * f1y + dz * f1z) * rinv);
-                                score += hw_log2(fmaxf(1.0f - ac, 1e-5f)) * LN2;
-                                ok = ok && ac < 0.9999f;
+#pragma unroll
+                        for (int k = 0; k < TCAP / WAVE; k++)
+                            if (k * WAVE < bx.T) {
+                                const int t = lane + k * WAVE;
+                                if (t < bx.T) consider(rq, phase, e, t, sx[k], sy[k], sz[k]);
                             }
-                            if (noisy) {
-                                // uniform in [0,1): golden-ratio sequence over the translations, phase per pair
-                                const float un = __builtin_amdgcn_fractf(fmaf((float)(t0 + u), 0.61803399f, phase));
-                                if (pass == 0) score = fmaf(a, d2 + (un - 0.5f) * P.noise, rq.w);
-                                else score += (un - 0.5f) * P.noise;
-                            }
-                            // a lane meets its candidates in ascending (e, t) order when the table is
-                            // one chunk: the strict comparison keeps the first; with several chunks the
-                            // explicit (e, t) comparison does
-                            if (ok && (score > best.score ||
-                                       (score == best.score && (e < best.e || (e == best.e && t0 + u < best.t))))) {
-                                best.score = score; best.e = e; best.t = t0 + u;
+                    }
+                } else {
+                    for (int ch = 0; ch < nchunks; ch++) {
+                        const int t0 = ch * TCAP;
+                        const int cnt = min(TCAP, bx.T - t0);
+                        __syncthreads();
+                        build_shift_table(tab, t0, cnt, bx, L, lane);
+                        __syncthreads();
+                        for (int el = 0; el < ne; el++) {
+                            const float4 rq = pair_rq[el];
+                            const int e = eb + el;
+                            const float phase = noisy ? hash_uniform(pass ? seed_hi : seed_lo, pass ? seed_lo : seed_hi,
+                                                                     (uint32_t)(e * H + h), (uint32_t)pass) : 0.0f;
+                            for (int u = lane; u < cnt; u += WAVE) {
+                                const float4 v = tab[u];
+                                consider(rq, phase, e, t0 + u, v.x, v.y, v.z);
                             }
                         }
                     }
