@@ -35,7 +35,12 @@ EPI_FWD = 4 * 2 * 16 * 64              # projection epilogue per (pair, head)
 PEAK_FP32_TFLOPS = 157.3               # published MI355X FP32 vector peak (packed FMA)
 PEAK_FP32_UNPACKED = 78.6              # 256 CU x 64 lanes x 2 flop x 2.4 GHz, packed FP32 not used
 PEAK_TRANS_TOPS = 9.8                  # quarter-rate transcendental unit
-HBM_BYTES_PER_PAIR_HEAD_BWD = 8 + 64 + 4 + 4   # z, gz (4+4), gpsi (64), shares of rpos/a/ga
+# HBM bytes per launch of the dominant kernel on this workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (KiB per dispatch) scaled by what the same counters read for the 256 MiB device copy of --calibrate-copy
+# (FETCH_SIZE reads 128 MiB for it: factor 2.0; WRITE_SIZE reads 256 MiB: factor 1.0); see profiles/.
+# backward: 25 502 KiB x 2.0 fetched + 34 248 KiB written (33.5 MB of that are the per-wavefront partials of
+# the weight gradients).  The forward kernel's fetches were not collected.
+TRAFFIC_BYTES_PER_LAUNCH = {"framed_pe_backward": 87.3e6, "framed_pe_forward": None}
 
 
 def parse():
@@ -45,6 +50,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (reference point for HBM traffic counters)")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying the step as one HIP graph")
     ap.add_argument("--cpu-crystals", type=int, default=12, help="crystals of the batch in the CPU sample")
@@ -151,11 +158,18 @@ def main():
     # ---- a second, instrumented pass over the same steps: HIP events around every library call on
     #      its stream, and term counters; kept out of the timed region so that it cannot perturb it
     KM.EVENT_LOG = []
+    _lib.kernel_timing(True)          # the library's own event bracket around each lattice-sum kernel
     nprof = min(args.steps, 5)
     for _ in range(nprof):
         step()
     torch.cuda.synchronize()
+    _lib.kernel_timing(False)
     log, KM.EVENT_LOG = KM.EVENT_LOG, None
+    kern_ms = {}
+    for what in ("frame_axes", "framed_pe_forward", "framed_pe_backward"):
+        total, count = _lib.read_kernel_timing(what)
+        if count:
+            kern_ms[what] = total / count
     # ---- and a third one that counts translations (separately: the counters add a few atomics)
     KM.COLLECT_STATS = True
     _lib.read_stats(dev, reset=True)
@@ -179,23 +193,25 @@ def main():
     fwd_eval = stats["fwd_evaluated"] / nlaunch_fwd
     fwd_box = stats["fwd_in_box"] / nlaunch_fwd
     fwd_pairs = stats["fwd_pairs"] / nlaunch_fwd
-    t_bwd = avg_ms.get("framed_pe_backward", float("nan")) * 1e-3
-    t_fwd = avg_ms.get("framed_pe_forward", float("nan")) * 1e-3
+    t_bwd = kern_ms.get("framed_pe_backward", float("nan")) * 1e-3
+    t_fwd = kern_ms.get("framed_pe_forward", float("nan")) * 1e-3
     flop_bwd = bwd_eval * F_BWD + bwd_pairs * 2 * EPI_FWD    # terms actually evaluated + epilogues
     flop_fwd = fwd_eval * F_FWD + fwd_pairs * EPI_FWD
     dominant = "framed_pe_backward" if t_bwd >= t_fwd else "framed_pe_forward"
     flop_dom, t_dom, eval_dom = (flop_bwd, t_bwd, bwd_eval) if dominant == "framed_pe_backward" else (flop_fwd, t_fwd, fwd_eval)
     achieved = flop_dom / t_dom / 1e12
     roofline = {
-        "kernel": dominant, "bound": "valu", "achieved": achieved, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-        "frac": achieved / PEAK_FP32_TFLOPS, "traffic": None,
+        "kernel": dominant + "_kernel", "bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS,
+        "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_TFLOPS, "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
+        "bound_detail": "FP32 arithmetic (vector + a little MFMA) against the published 157.3 TFLOP/s; HBM traffic is "
+                        "<1 byte per term; what limits the kernel in practice is LDS atomic throughput",
         "frac_of_unpacked_fp32_peak": achieved / PEAK_FP32_UNPACKED,
         "transcendental_frac": eval_dom * X_TERM / t_dom / 1e12 / PEAK_TRANS_TOPS,
         "avg_launch_ms": t_dom * 1e3,
         "terms_evaluated_per_launch": eval_dom,
         "note": "algorithmic flop of the reference formulation (709 bwd / 488 fwd per term, 109 exp) x terms "
-                "actually evaluated after pruning, + projection epilogues; duration from HIP events around the "
-                "library call on its stream",
+                "actually evaluated after pruning, + projection epilogues; duration from HIP events recorded by "
+                "the library around this kernel alone, on the stream it is launched on",
     }
     terms = {
         "forward_terms_in_box_per_s": fwd_box / t_fwd, "forward_terms_evaluated_per_s": fwd_eval / t_fwd,
@@ -218,8 +234,15 @@ def main():
         "final_loss": final_loss,
         "roofline": roofline,
         "lattice_terms": terms,
-        "kernel_ms": avg_ms, "kernel_launches_per_step": launches, "library_ms_per_step": lib_ms_per_step,
+        "lattice_kernel_ms": kern_ms, "library_call_ms": avg_ms, "library_calls_per_step": launches,
+        "library_ms_per_step": lib_ms_per_step,
     }
+    if args.calibrate_copy:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        result["calibrate_copy_bytes"] = int(src.numel() * 4)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(model, cb_cpu, mp, min(args.cpu_crystals, args.batch))
     print(json.dumps(result))

@@ -49,7 +49,7 @@ class CfhParams(ctypes.Structure):
 EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_frame_axis1",
            "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_backward",
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
-           "cfh_crystal_mean_forward", "cfh_crystal_mean_backward")
+           "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read")
 
 _lib = None
 _lock = threading.Lock()
@@ -98,6 +98,10 @@ def load():
         lib.cfh_crystal_mean_forward.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P]
         lib.cfh_crystal_mean_backward.restype = ctypes.c_int
         lib.cfh_crystal_mean_backward.argtypes = [_P, _P, _P, _I64, _I64, _I64, _P, _P]
+        lib.cfh_timing_enable.restype = ctypes.c_int
+        lib.cfh_timing_enable.argtypes = [ctypes.c_int]
+        lib.cfh_timing_read.restype = ctypes.c_int
+        lib.cfh_timing_read.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_I64)]
         if lib.cfh_abi_version() != ABI_VERSION:
             raise RuntimeError(f"ABI version {lib.cfh_abi_version()} of {LIB_PATH} != {ABI_VERSION}")
         _lib = lib
@@ -157,3 +161,15 @@ def read_stats(device: torch.device, reset: bool = False) -> dict:
 
 def current_stream_ptr(device: torch.device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def kernel_timing(enable: bool):
+    """Switch the library's own HIP-event bracket around its lattice-sum kernels on or off."""
+    check(load().cfh_timing_enable(1 if enable else 0), "cfh_timing_enable")
+
+
+def read_kernel_timing(what: str):
+    """(total milliseconds, launches) of the kernels recorded under ``what`` since the last read."""
+    total, count = ctypes.c_double(0.0), _I64(0)
+    check(load().cfh_timing_read(what.encode(), ctypes.byref(total), ctypes.byref(count)), "cfh_timing_read")
+    return total.value, count.value

@@ -9,6 +9,9 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
 
 #include "device_common.hpp"
 #include "frame_select.hpp"
@@ -197,13 +200,35 @@ int resident_waves(Kern kern, int cap, int H) {
     return (int)want;
 }
 
+// Optional timing of the lattice-sum kernels alone (not the small kernels around them): HIP events
+// on the stream of the launch, kept until cfh_timing_read collects them.
+struct TimedLaunch { std::string what; hipEvent_t start, stop; };
+std::mutex g_timing_mutex;
+bool g_timing_on = false;
+std::vector<TimedLaunch> g_timed;
+
 // `waves`: in = upper bound, out = wavefronts actually launched
 template <typename Kern>
 int launch_persistent(Kern kern, const cfh::KernelArgs& A, int* waves, hipStream_t st, const char* what) {
     *waves = resident_waves(kern, *waves, A.H);
     const int threads = A.N * A.H > A.H * cfh::NQUEUE ? A.N * A.H : A.H * cfh::NQUEUE;
     hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, A, A.q != nullptr ? 1 : 0);
+    bool timed = false;
+    TimedLaunch t;
+    {
+        std::lock_guard<std::mutex> lock(g_timing_mutex);
+        timed = g_timing_on;
+    }
+    if (timed) {
+        t.what = what;
+        timed = hipEventCreate(&t.start) == hipSuccess && hipEventCreate(&t.stop) == hipSuccess &&
+                hipEventRecord(t.start, st) == hipSuccess;
+    }
     hipLaunchKernelGGL(kern, dim3(*waves), dim3(cfh::WAVE), 0, st, A);
+    if (timed && hipEventRecord(t.stop, st) == hipSuccess) {
+        std::lock_guard<std::mutex> lock(g_timing_mutex);
+        g_timed.push_back(t);
+    }
     return finish_launch(what);
 }
 
@@ -214,6 +239,34 @@ extern "C" {
 int cfh_abi_version(void) { return CFH_ABI_VERSION; }
 
 const char* cfh_last_error(void) { return g_err; }
+
+int cfh_timing_enable(int on) {
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    g_timing_on = on != 0;
+    return CFH_OK;
+}
+
+int cfh_timing_read(const char* what, double* total_ms, int64_t* launches) {
+    if (!what || !total_ms || !launches) return fail(CFH_EINVAL, "what, total_ms and launches must not be NULL");
+    std::vector<TimedLaunch> mine, rest;
+    {
+        std::lock_guard<std::mutex> lock(g_timing_mutex);
+        for (const TimedLaunch& t : g_timed) (t.what == what ? mine : rest).push_back(t);
+        g_timed.swap(rest);
+    }
+    *total_ms = 0.0;
+    *launches = 0;
+    for (const TimedLaunch& t : mine) {
+        float ms = 0.0f;
+        if (hipEventSynchronize(t.stop) == hipSuccess && hipEventElapsedTime(&ms, t.start, t.stop) == hipSuccess) {
+            *total_ms += (double)ms;
+            *launches += 1;
+        }
+        (void)hipEventDestroy(t.start);
+        (void)hipEventDestroy(t.stop);
+    }
+    return CFH_OK;
+}
 
 size_t cfh_workspace_bytes(const cfh_params* p, int64_t N, int64_t E) {
     (void)E;

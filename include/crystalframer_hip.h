@@ -90,6 +90,17 @@ int cfh_abi_version(void);
 /* Text of the last error on the calling thread ("" if none). */
 const char* cfh_last_error(void);
 
+/*
+ * Diagnostics with no counterpart in the reference.  After cfh_timing_enable(1) every call of the
+ * frame-search and value-encoding entry points brackets its lattice-sum kernel (that kernel alone,
+ * not the small kernels around it) with HIP events on the stream of the call; cfh_timing_read waits
+ * for the launches recorded under `what` ("frame_axis1", "frame_axis2", "frame_axes",
+ * "framed_pe_forward", "framed_pe_backward"), returns their summed duration and count, and forgets
+ * them.  Not to be enabled while the stream is being captured into a graph.
+ */
+int cfh_timing_enable(int on);
+int cfh_timing_read(const char* what, double* total_ms, int64_t* launches);
+
 /* Bytes of device scratch the four entry points below need for (N atoms, E pairs). */
 size_t cfh_workspace_bytes(const cfh_params* p, int64_t N, int64_t E);
 
