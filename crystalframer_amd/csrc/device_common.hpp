@@ -3,11 +3,13 @@
 // Execution model used by every kernel in this directory:
 //   * a workgroup is ONE 64-lane wavefront that owns one attention head h (= blockIdx.x % H, so
 //     all wavefronts of a head land on the same XCD and share its L2 copy of that head's weights);
-//   * wavefronts are persistent: each pulls (atom i) work items for its head from a per-head
-//     counter in global memory until the counter passes N -- an exit every wavefront reaches;
+//   * wavefronts are persistent: each pops (atom i) work items of its head from one of the head's
+//     queues in global memory until all are empty -- an exit every wavefront reaches;
+//   * what an item needs (box, lattice, frame axes ...) comes as one 128-byte record written by
+//     prepare_items_kernel and fetched one item ahead;
 //   * for an item (i,h) the integer translations n of the box [-R1,R1]x[-R2,R2]x[-R3,R3] are
-//     expanded once into an LDS table of Cartesian shifts n.L (TCAP entries at a time), lanes then
-//     run over table entries, so one pair (i,j) is processed 64 translations per step.
+//     expanded once into an LDS table of Cartesian shifts n.L (a chunk at a time for large boxes);
+//     pairs (i,j) are then processed four at a time, one per 16-lane row, lanes over translations.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
