@@ -52,4 +52,4 @@ def rel_err(x, ref):
     """max |x-ref| / max |ref| (tensor-scale relative error)."""
     x, ref = x.detach(), ref.detach()
     scale = ref.abs().max().clamp_min(1e-30)
-    return float((x.double().cpu() - ref.double()).abs().max() / scale)
+    return float((x.double().cpu() - ref.double().cpu()).abs().max() / scale.cpu())
