@@ -34,17 +34,6 @@ __device__ __forceinline__ float hw_rcp(float x) { return __builtin_amdgcn_rcpf(
 __device__ __forceinline__ float hw_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
 __device__ __forceinline__ float clampf(float x, float lo, float hi) { return fminf(fmaxf(x, lo), hi); }
 
-// ---- wave64 reductions ------------------------------------------------------------------------
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-    return v;
-}
-__device__ __forceinline__ float wave_min(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, WAVE));
-    return v;
-}
 // ---- reductions over a 16-lane row in DPP (VALU latency only; every lane must be active) --------
 // quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror: after the four steps all
 // 16 lanes of the row hold the reduction of the row.
@@ -67,6 +56,32 @@ __device__ __forceinline__ float row_sum(float x) {
     return x;
 }
 
+// ---- reductions over the four rows of a wavefront (same column), gfx950 lane swaps ---------------
+// v_permlane32_swap exchanges the upper half of one register with the lower half of another,
+// v_permlane16_swap the odd rows of one with the even rows of another: applied to two copies of x
+// they hand every lane the two values to combine.  VALU only, no LDS round trip.
+__device__ __forceinline__ void swap32(float x, float& lo, float& hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    lo = __uint_as_float(r[0]); hi = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void swap16(float x, float& even, float& odd) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    even = __uint_as_float(r[0]); odd = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float rows_sum(float x) {      // every lane: sum over lanes c, c+16, c+32, c+48
+    float p, q;
+    swap32(x, p, q); x = p + q;
+    swap16(x, p, q); return p + q;
+}
+__device__ __forceinline__ float rows_min(float x) {
+    float p, q;
+    swap32(x, p, q); x = fminf(p, q);
+    swap16(x, p, q); return fminf(p, q);
+}
+// ---- wave64 reductions: rows in DPP, then across the rows -----------------------------------------
+__device__ __forceinline__ float wave_sum(float v) { return rows_sum(row_sum(v)); }
+__device__ __forceinline__ float wave_min(float v) { return rows_min(row_min(v)); }
+
 // Ordering point between the lanes of a ONE-wavefront workgroup that communicate through LDS.  The
 // LDS executes a wavefront's instructions in order, so no hardware barrier and no wait for
 // outstanding global stores is needed -- only the compiler must not move LDS accesses across.
@@ -76,24 +91,6 @@ __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// arg-min over (value, index): smallest value, then smallest index
-__device__ __forceinline__ void wave_argmin(float& v, int& idx) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        float ov = __shfl_xor(v, o, WAVE);
-        int oi = __shfl_xor(idx, o, WAVE);
-        if (ov < v || (ov == v && oi < idx)) { v = ov; idx = oi; }
-    }
-}
-// arg-max over (value, index): largest value, then smallest index
-__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        float ov = __shfl_xor(v, o, WAVE);
-        int oi = __shfl_xor(idx, o, WAVE);
-        if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
-    }
-}
 // slots of KernelArgs::stats
 enum { STAT_FWD_EVAL = 0, STAT_FWD_RAW = 1, STAT_BWD_EVAL = 2, STAT_BWD_RAW = 3, STAT_FRAME1_RAW = 4,
        STAT_FRAME2_RAW = 5, STAT_FWD_PAIRS = 6, STAT_BWD_PAIRS = 7 };

@@ -38,15 +38,28 @@ __device__ __forceinline__ void shift_of(int t, const Box& bx, const Lattice& L,
 
 // best candidate of a wavefront: largest score, then lowest pair, then lowest translation
 struct Best { float score; int e; int t; };
+__device__ __forceinline__ bool better(float s1, int e1, int t1, float s2, int e2, int t2) {
+    return s1 > s2 || (s1 == s2 && (e1 < e2 || (e1 == e2 && t1 < t2)));
+}
+template <int CTRL>
+__device__ __forceinline__ void best_dpp(Best& b) {
+    const float os = dpp_move<CTRL>(b.score);
+    const int oe = __float_as_int(dpp_move<CTRL>(__int_as_float(b.e)));
+    const int ot = __float_as_int(dpp_move<CTRL>(__int_as_float(b.t)));
+    if (better(os, oe, ot, b.score, b.e, b.t)) { b.score = os; b.e = oe; b.t = ot; }
+}
 __device__ __forceinline__ void wave_best(Best& b) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const float os = __shfl_xor(b.score, o, WAVE);
-        const int oe = __shfl_xor(b.e, o, WAVE);
-        const int ot = __shfl_xor(b.t, o, WAVE);
-        if (os > b.score || (os == b.score && (oe < b.e || (oe == b.e && ot < b.t)))) {
-            b.score = os; b.e = oe; b.t = ot;
-        }
+    best_dpp<0xB1>(b); best_dpp<0x4E>(b); best_dpp<0x141>(b); best_dpp<0x140>(b);     // within the rows
+    float s0, s1, e0, e1, t0, t1;
+    swap32(b.score, s0, s1); swap32(__int_as_float(b.e), e0, e1); swap32(__int_as_float(b.t), t0, t1);
+    {
+        const bool first = !better(s1, __float_as_int(e1), __float_as_int(t1), s0, __float_as_int(e0), __float_as_int(t0));
+        b.score = first ? s0 : s1; b.e = __float_as_int(first ? e0 : e1); b.t = __float_as_int(first ? t0 : t1);
+    }
+    swap16(b.score, s0, s1); swap16(__int_as_float(b.e), e0, e1); swap16(__int_as_float(b.t), t0, t1);
+    {
+        const bool first = !better(s1, __float_as_int(e1), __float_as_int(t1), s0, __float_as_int(e0), __float_as_int(t0));
+        b.score = first ? s0 : s1; b.e = __float_as_int(first ? e0 : e1); b.t = __float_as_int(first ? t0 : t1);
     }
 }
 
@@ -105,9 +118,11 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
             Best best;
             best.score = -3.0e38f; best.e = 0x7fffffff; best.t = 0x7fffffff;
             for (int eb = e0; eb < e1; eb += WAVE) {
-                // stage rpos and q_i.k_j of up to 64 pairs, one per lane
+                // stage rpos and q_i.k_j of up to 64 pairs, one per lane (rows of up to 64 pairs keep
+                // what the first search staged)
+                const bool staged = pass == 1 && MODE == 2 && e1 - e0 <= WAVE;
                 __syncthreads();
-                if (eb + lane < e1) {
+                if (!staged && eb + lane < e1) {
                     const int e = eb + lane;
                     const int64_t j = P.edges[(size_t)P.E + e];
                     const float4* kp = reinterpret_cast<const float4*>(P.k + ((size_t)j * H + h) * DH);

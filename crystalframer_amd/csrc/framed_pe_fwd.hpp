@@ -170,19 +170,18 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                         hv[4 * k4 + 2] = (float)t4.z; hv[4 * k4 + 3] = (float)t4.w;
                     }
                     v4f acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+                    v4f acc2 = {0.f, 0.f, 0.f, 0.f}, acc3 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int s = 0; s < 16; s++) {
                         acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(hv[s], Wrow[s], acc0, 2, 0, 0);
                         acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(hv[s], Wrow[16 + s], acc1, 2, 1, 0);
-                        acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(hv[s], Wrow[32 + s], acc0, 2, 2, 0);
-                        acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(hv[s], Wrow[48 + s], acc1, 2, 3, 0);
+                        acc2 = __builtin_amdgcn_mfma_f32_4x4x1f32(hv[s], Wrow[32 + s], acc2, 2, 2, 0);
+                        acc3 = __builtin_amdgcn_mfma_f32_4x4x1f32(hv[s], Wrow[48 + s], acc3, 2, 3, 0);
                     }
                     // lane (enc, c = lane & 15), component r: pair half*4 + r
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
-                        float x = (acc0[r] + acc1[r]) * enc_scale;
-                        x += __shfl_xor(x, 16, WAVE);
-                        x += __shfl_xor(x, 32, WAVE);
+                        const float x = rows_sum(((acc0[r] + acc1[r]) + (acc2[r] + acc3[r])) * enc_scale);
                         if (lane < DH && half * 4 + r < ng)
                             P.out_psi[((size_t)(g0 + half * 4 + r) * H + h) * DH + lane] = x;
                     }
