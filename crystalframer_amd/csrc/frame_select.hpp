@@ -141,7 +141,9 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                 __syncthreads();
                 const int ne = min(WAVE, e1 - eb);
                 // one candidate: pair e shifted by (vx,vy,vz), translation index t
-                auto consider = [&](const float4& rq, float phase, int e, int t, float vx, float vy, float vz) {
+                // `ordered`: this lane meets its candidates in ascending (pair, translation) order,
+                // so the strict comparison alone keeps the first of equal scores
+                auto consider = [&](bool ordered, const float4& rq, float phase, int e, int t, float vx, float vy, float vz) {
                     const float dx = rq.x + vx, dy = rq.y + vy, dz = rq.z + vz;
                     const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
                     float score = fmaf(a, d2, rq.w);
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                     }
                     // largest score, then lowest pair, then lowest translation
                     if (ok && (score > best.score ||
-                               (score == best.score && (e < best.e || (e == best.e && t < best.t))))) {
+                               (!ordered && score == best.score && (e < best.e || (e == best.e && t < best.t))))) {
                         best.score = score; best.e = e; best.t = t;
                     }
                 };
@@ -175,7 +177,7 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                         for (int k = 0; k < TCAP / WAVE; k++)
                             if (k * WAVE < bx.T) {
                                 const int t = lane + k * WAVE;
-                                if (t < bx.T) consider(rq, phase, e, t, sx[k], sy[k], sz[k]);
+                                if (t < bx.T) consider(true, rq, phase, e, t, sx[k], sy[k], sz[k]);
                             }
                     }
                 } else {
@@ -192,7 +194,7 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                                                                      (uint32_t)(e * H + h), (uint32_t)pass) : 0.0f;
                             for (int u = lane; u < cnt; u += WAVE) {
                                 const float4 v = tab[u];
-                                consider(rq, phase, e, t0 + u, v.x, v.y, v.z);
+                                consider(false, rq, phase, e, t0 + u, v.x, v.y, v.z);
                             }
                         }
                     }
