@@ -49,7 +49,8 @@ class CfhParams(ctypes.Structure):
 EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_frame_axis1",
            "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_backward",
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
-           "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read")
+           "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
+           "cfh_linear_weight_bias_grad")
 
 _lib = None
 _lock = threading.Lock()
@@ -98,6 +99,8 @@ def load():
         lib.cfh_crystal_mean_forward.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P]
         lib.cfh_crystal_mean_backward.restype = ctypes.c_int
         lib.cfh_crystal_mean_backward.argtypes = [_P, _P, _P, _I64, _I64, _I64, _P, _P]
+        lib.cfh_linear_weight_bias_grad.restype = ctypes.c_int
+        lib.cfh_linear_weight_bias_grad.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P, _P]
         lib.cfh_timing_enable.restype = ctypes.c_int
         lib.cfh_timing_enable.argtypes = [ctypes.c_int]
         lib.cfh_timing_read.restype = ctypes.c_int

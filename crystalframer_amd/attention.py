@@ -216,20 +216,20 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
             # arithmetic per output element; forward, input gradient and weight gradient each
             # become one launch instead of three)
             w_in = torch.cat([self.q_proj_weight, self.k_proj_weight, self.v_proj_weight], dim=0)
-            qkv = F.linear(query, w_in, self.in_proj_bias)
+            qkv = cuda_funcs.linear(query, w_in, self.in_proj_bias)
             q, k, v = qkv.split([self.kdim, self.kdim, self.vdim], dim=1)
             q = q.reshape(N, H, -1)
             k = k.reshape(N, H, -1)
             v = v.reshape(N, H, -1)
         else:
-            q = F.linear(query, self.q_proj_weight, bq).view(N, H, -1)
-            k = F.linear(key, self.k_proj_weight, bk).view(key.shape[0], H, -1)
-            v = F.linear(value, self.v_proj_weight, bv).view(value.shape[0], H, -1)
+            q = cuda_funcs.linear(query, self.q_proj_weight, bq).view(N, H, -1)
+            k = cuda_funcs.linear(key, self.k_proj_weight, bk).view(key.shape[0], H, -1)
+            v = cuda_funcs.linear(value, self.v_proj_weight, bv).view(value.shape[0], H, -1)
         a = self.gaussian_coefficient(q)
         z, psi = compute_real_domain_attn_frame_proj(
             q, k, v, batch_q, batch_kv, edges, points, dist2_min, tvecs, rvecs, self.pe_dist_proj,
             self.proj_angle1, self.proj_angle2, self.proj_angle3, a, self.params, this_epoch,
             frame_sink=self.frame_sink)
         out = _scaled_dot_product_attention(q, k, v, batch_q, batch_kv, edges, z, psi)
-        out = self.out_proj(out.reshape(N, H * v.shape[-1]))
+        out = cuda_funcs.linear(out.reshape(N, H * v.shape[-1]), self.out_proj.weight, self.out_proj.bias)
         return out, psi

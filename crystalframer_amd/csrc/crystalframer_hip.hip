@@ -18,6 +18,7 @@
 #include "framed_pe_bwd.hpp"
 #include "framed_pe_fwd.hpp"
 #include "fused_dpa.hpp"
+#include "linear_grad.hpp"
 
 namespace {
 
@@ -520,6 +521,29 @@ int cfh_crystal_mean_backward(const float* gout, const int64_t* batch, const int
     hipLaunchKernelGGL(cfh::crystal_mean_bwd_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, gout, batch, atom_start, (int)N, (int)C, gx);
     return finish_launch("crystal_mean_backward");
+}
+
+int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int64_t I, int64_t O,
+                                float* dW, float* db, void* stream) {
+    if (N < 0 || I < 1 || O < 1 || N > 0x7fffffffLL / 64 || I > 65536 || O > 65536)
+        return fail(CFH_EINVAL, "sizes N=%lld I=%lld O=%lld out of range", (long long)N, (long long)I, (long long)O);
+    if (!dW || (N > 0 && (!x || !dy))) return fail(CFH_EINVAL, "x, dy and dW must not be NULL");
+    hipStream_t st = (hipStream_t)stream;
+    const int nw = (int)(O * I), nb = (int)O;
+    hipLaunchKernelGGL(cfh::zero2_kernel, dim3((nw + 255) / 256), dim3(256), 0, st, dW, nw, db, nb);
+    if (N > 0) {
+        const int bx = (int)((I + 63) / 64), by = (int)((O + 63) / 64);
+        int slices = (512 + bx * by - 1) / (bx * by);
+        const int max_slices = (int)((N + 31) / 32);
+        if (slices > max_slices) slices = max_slices;
+        if (slices < 1) slices = 1;
+        int rows = (int)((N + slices - 1) / slices);
+        rows = (rows + 3) & ~3;
+        slices = (int)((N + rows - 1) / rows);
+        hipLaunchKernelGGL(cfh::linear_wgrad_kernel, dim3(bx, by, slices), dim3(256), 0, st, x, dy, (int)N, (int)I,
+                           (int)O, rows, dW, db);
+    }
+    return finish_launch("linear_weight_bias_grad");
 }
 
 }  // extern "C"

@@ -467,3 +467,42 @@ class IrregularMeanCUDA(torch.autograd.Function):
                                                _lib.ptr(gx), _lib.current_stream_ptr(dev))
         _lib.check(rc, "cfh_crystal_mean_backward")
         return gx.to(ctx.in_dtype), None, None
+
+
+class LinearHIP(torch.autograd.Function):
+    """y = x W^T + b with the weight and bias gradients from one launch of the library
+    (cfh_linear_weight_bias_grad); forward and input gradient are the framework's GEMMs.
+    Same values as torch.nn.functional.linear up to the order of the float32 sums."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return torch.nn.functional.linear(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, weight = ctx.saved_tensors
+        gx = gw = gb = None
+        if ctx.needs_input_grad[0]:
+            gx = gy.matmul(weight)
+        if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
+            lib = _lib.load()
+            O, I = weight.shape
+            x2 = _f32c(x.reshape(-1, I))
+            g2 = _f32c(gy.reshape(-1, O))
+            gw32 = torch.empty((O, I), dtype=torch.float32, device=x.device)
+            gb32 = torch.empty((O,), dtype=torch.float32, device=x.device) if ctx.has_bias else None
+            with _timed("linear_weight_bias_grad", x.device):
+                rc = lib.cfh_linear_weight_bias_grad(_lib.ptr(x2), _lib.ptr(g2), x2.shape[0], I, O, _lib.ptr(gw32),
+                                                     _lib.ptr(gb32), _lib.current_stream_ptr(x.device))
+            _lib.check(rc, "cfh_linear_weight_bias_grad")
+            gw = gw32.to(weight.dtype)
+            gb = gb32.to(weight.dtype) if ctx.has_bias else None
+        return gx, gw, gb
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """torch.nn.functional.linear for device tensors, with the library's weight-gradient kernel."""
+    _lib.require_gpu(x, weight)
+    return LinearHIP.apply(x, weight, bias)

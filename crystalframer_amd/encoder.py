@@ -69,7 +69,8 @@ class CrystalformerEncoderLayerCUDA(nn.Module):
         return self.dropout1(x)
 
     def _ff_block(self, x):
-        return self.dropout2(self.linear2(self.dropout(self.activation(self.linear1(x)))))
+        h = self.activation(cuda_funcs.linear(x, self.linear1.weight, self.linear1.bias))
+        return self.dropout2(cuda_funcs.linear(self.dropout(h), self.linear2.weight, self.linear2.bias))
 
     def forward(self, src: Tensor, batch: Tensor, edges: Tensor, pos_ij: Tensor = None,
                 dist2_min: Tensor = None, trans: Tensor = None, kr_base: Tensor = None,

@@ -81,7 +81,7 @@ class Latticeformer(nn.Module):
 
     def forward(self, data, this_epoch=None):
         """``data`` carries x (N,98), pos (N,3), batch (N), trans_vec (B,3,3), sizes (B)."""
-        x = self.input_embeddings(data.x)
+        x = cuda_funcs.linear(data.x, self.input_embeddings.weight, self.input_embeddings.bias)
         num_pairs = getattr(data, "num_pairs", -1)
         x = self.encoder(x, data.pos, data.batch, data.trans_vec, data.sizes, this_epoch=this_epoch,
                          num_pairs=num_pairs if num_pairs is not None and num_pairs >= 0 else None)

@@ -225,6 +225,17 @@ int cfh_crystal_mean_forward(const float* x, const int64_t* atom_start, int64_t 
 int cfh_crystal_mean_backward(const float* gout, const int64_t* batch, const int64_t* atom_start,
                               int64_t N, int64_t B, int64_t C, float* gx, void* stream);
 
+/*
+ * Weight and bias gradients of a projection y = x W^T + b:  dW (O,I) = dy^T x, db (O) = column sums
+ * of dy (db may be NULL); x (N,I), dy (N,O), row-major.  One launch (plus a clearing kernel) sized
+ * for the shapes of this model, N = atoms in the thousands and I, O in the hundreds, where the
+ * general GEMM plus a separate reduction take 19 + 10 us.  The reference leaves this to
+ * torch.nn.functional.linear's autograd (models/indexed_lattice_multi_head_attention_cuda.py:141,988,
+ * models/indexed_latticeformer_encoder.py:606).
+ */
+int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int64_t I, int64_t O,
+                                float* dW, float* db, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -164,3 +164,29 @@ def test_crystal_mean_forward_backward():
     out3 = cf.IrregularMeanCUDA.apply(x3, batch.to(dev()), None)
     ref3 = TO.crystal_mean(x3.cpu().double(), batch, 5)
     assert Hh.rel_err(out3.cpu().double(), ref3) < 1e-6
+
+
+@pytest.mark.parametrize("N,I,O,bias", [(2372, 128, 384, True), (2372, 512, 128, True), (2372, 98, 128, False),
+                                        (37, 20, 50, True), (1, 16, 16, True), (0, 16, 32, True)])
+def test_linear_weight_and_bias_gradients(N, I, O, bias):
+    """The library's weight/bias gradient kernel against float64 autograd of x W^T + b."""
+    import crystalframer_amd as cf
+    gen = torch.Generator().manual_seed(N + I + O)
+    x64 = torch.randn(N, I, generator=gen, dtype=torch.float64, requires_grad=True)
+    w64 = torch.randn(O, I, generator=gen, dtype=torch.float64, requires_grad=True)
+    b64 = torch.randn(O, generator=gen, dtype=torch.float64, requires_grad=True) if bias else None
+    gy = torch.randn(N, O, generator=gen, dtype=torch.float64)
+    (torch.nn.functional.linear(x64, w64, b64) * gy).sum().backward()
+    x = f32(x64.detach()).requires_grad_(True)
+    w = f32(w64.detach()).requires_grad_(True)
+    b = f32(b64.detach()).requires_grad_(True) if bias else None
+    y = cf.cuda_funcs.linear(x, w, b)
+    (y * f32(gy)).sum().backward()
+    if N > 0:
+        assert Hh.rel_err(y, torch.nn.functional.linear(x64, w64, b64)) < 1e-5
+        assert Hh.rel_err(x.grad, x64.grad) < 1e-5
+        assert Hh.rel_err(w.grad, w64.grad) < 1e-5
+        if bias:
+            assert Hh.rel_err(b.grad, b64.grad) < 1e-5
+    else:
+        assert float(w.grad.abs().max()) == 0.0 and float(b.grad.abs().max()) == 0.0
