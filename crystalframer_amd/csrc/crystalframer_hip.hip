@@ -533,7 +533,7 @@ int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int6
     hipLaunchKernelGGL(cfh::zero2_kernel, dim3((nw + 255) / 256), dim3(256), 0, st, dW, nw, db, nb);
     if (N > 0) {
         const int bx = (int)((I + 63) / 64), by = (int)((O + 63) / 64);
-        int slices = (512 + bx * by - 1) / (bx * by);
+        int slices = (128 + bx * by - 1) / (bx * by);      // about 128 workgroups of 4 wavefronts
         const int max_slices = (int)((N + 31) / 32);
         if (slices > max_slices) slices = max_slices;
         if (slices < 1) slices = 1;

@@ -30,6 +30,7 @@ __global__ __launch_bounds__(256) void linear_wgrad_kernel(const float* __restri
     const bool voa = oa < O, vob = ob < O, via = ia < I, vib = ib < I;
     v4f_l acc00 = {0.f, 0.f, 0.f, 0.f}, acc01 = acc00, acc10 = acc00, acc11 = acc00;
     float bsum_a = 0.f, bsum_b = 0.f;
+#pragma unroll 4
     for (int r = r0 + kk; r < r1 + kk; r += 4) {          // every lane group takes the same number of steps
         const bool vr = r < r1;
         const float ya = (vr && voa) ? dy[(size_t)r * O + oa] : 0.f;
