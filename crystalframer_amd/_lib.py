@@ -86,9 +86,9 @@ def load():
         lib.cfh_frame_axes.restype = ctypes.c_int
         lib.cfh_frame_axes.argtypes = [pp] + [_P] * 10 + [_I64] * 3 + [_P, _P, ctypes.c_size_t, _P]
         lib.cfh_framed_pe_forward.restype = ctypes.c_int
-        lib.cfh_framed_pe_forward.argtypes = [pp] + [_P] * 13 + [_I64] * 3 + [_P] * 4 + [ctypes.c_size_t, _P]
+        lib.cfh_framed_pe_forward.argtypes = [pp] + [_P] * 13 + [_I64] * 3 + [_P] * 5 + [ctypes.c_size_t, _P]
         lib.cfh_framed_pe_backward.restype = ctypes.c_int
-        lib.cfh_framed_pe_backward.argtypes = [pp] + [_P] * 16 + [_I64] * 3 + [_P] * 6 + [ctypes.c_size_t, _P]
+        lib.cfh_framed_pe_backward.argtypes = [pp] + [_P] * 17 + [_I64] * 3 + [_P] * 6 + [ctypes.c_size_t, _P]
         lib.cfh_fused_dpa_forward.restype = ctypes.c_int
         lib.cfh_fused_dpa_forward.argtypes = [_P] * 7 + [_I64] * 4 + [_P] * 3
         lib.cfh_fused_dpa_backward.restype = ctypes.c_int

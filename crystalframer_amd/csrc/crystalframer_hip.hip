@@ -16,6 +16,7 @@
 #include "device_common.hpp"
 #include "frame_select.hpp"
 #include "framed_pe_bwd.hpp"
+#include "framed_pe_bwd_saved.hpp"
 #include "framed_pe_fwd.hpp"
 #include "fused_dpa.hpp"
 #include "linear_grad.hpp"
@@ -346,7 +347,8 @@ int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* r
                           const int64_t* e_start, const int32_t* order, const float* W_dist,
                           const float* W_axis1, const float* W_axis2, const float* W_axis3,
                           const float* frames, int64_t N, int64_t E, int64_t B, float* z, float* psi,
-                          float* d2min_out, void* workspace, size_t workspace_bytes, void* stream) {
+                          float* d2min_out, float* shat_out, void* workspace, size_t workspace_bytes,
+                          void* stream) {
     int rc = check_params(p);
     if (rc) return rc;
     if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
@@ -364,7 +366,7 @@ int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* r
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.W[0] = W_dist; A.W[1] = W_axis1; A.W[2] = W_axis2; A.W[3] = W_axis3;
-    A.frames = frames; A.out_z = z; A.out_psi = psi; A.out_d2min = d2min_out;
+    A.frames = frames; A.out_z = z; A.out_psi = psi; A.out_d2min = d2min_out; A.shat = shat_out;
     int waves = launch_waves(N, p->num_heads);
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     hipStream_t st = (hipStream_t)stream;
@@ -380,7 +382,8 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
                            const int64_t* e_start, const int32_t* order, const float* W_dist,
                            const float* W_axis1, const float* W_axis2, const float* W_axis3,
                            const float* frames, const float* z, const float* gz, const float* gpsi,
-                           int64_t N, int64_t E, int64_t B, float* ga, float* gW_dist, float* gW_axis1,
+                           const float* shat, int64_t N, int64_t E, int64_t B, float* ga, float* gW_dist,
+                           float* gW_axis1,
                            float* gW_axis2, float* gW_axis3, void* workspace, size_t workspace_bytes,
                            void* stream) {
     int rc = check_params(p);
@@ -409,10 +412,14 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.W[0] = W_dist; A.W[1] = W_axis1; A.W[2] = W_axis2; A.W[3] = W_axis3;
     A.frames = frames; A.z = z; A.gz = gz; A.gpsi = gpsi; A.out_ga = ga;
+    A.shat = const_cast<float*>(shat);
     A.gw_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + COUNTER_BYTES + items_bytes(N, p->num_heads));
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "framed_pe_backward";
-    if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, true);
+    if (has_len && shat) {      // the forward kept its histograms: gather-only kernel
+        if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_bwd_saved_kernel, true, true);
+        else CFH_DISPATCH_PE(cfh::framed_pe_bwd_saved_kernel, true, false);
+    } else if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, true);
     else if (has_len) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, false);
     else rc = launch_persistent(cfh::framed_pe_bwd_kernel<9, 33, false, false, false>, A, &waves, st, what);
     if (rc) return rc;
@@ -533,7 +540,7 @@ int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int6
     hipLaunchKernelGGL(cfh::zero2_kernel, dim3((nw + 255) / 256), dim3(256), 0, st, dW, nw, db, nb);
     if (N > 0) {
         const int bx = (int)((I + 63) / 64), by = (int)((O + 63) / 64);
-        int slices = (128 + bx * by - 1) / (bx * by);      // about 128 workgroups of 4 wavefronts
+        int slices = (512 + bx * by - 1) / (bx * by);      // about 512 workgroups of 4 wavefronts
         const int max_slices = (int)((N + 31) / 32);
         if (slices > max_slices) slices = max_slices;
         if (slices < 1) slices = 1;

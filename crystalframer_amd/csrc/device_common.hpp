@@ -230,6 +230,20 @@ __device__ __forceinline__ float window_scatter_gather(uint32_t* hbase, const fl
     return acc;
 }
 
+// sum_m weight*g_m*gbase[m] alone (the histograms come from the forward pass).
+template <int W>
+__device__ __forceinline__ float window_gather(const float* gbase, const WindowSeed& s, float cc) {
+    constexpr int C = W / 2;
+    float acc = s.gc * gbase[C];
+    float g = s.gc, r = s.rr;
+#pragma unroll
+    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); }
+    g = s.gc; r = s.rl;
+#pragma unroll
+    for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); }
+    return acc;
+}
+
 // Read histogram word `idx` as a float in [0,1] and clear it.
 __device__ __forceinline__ float take_bin(uint32_t* hist, int idx) {
     const uint32_t s = hist[idx];
@@ -266,6 +280,8 @@ struct KernelArgs {
     // outputs
     float* out_z; float* out_psi; float* out_d2min; float* out_frame; float* out_ga;
     float* gw_partial;            // (waves, 4, DH, NBINS) per-wave weight-gradient partials
+    float* shat;                  // (E, H, 4, NBINS) window histograms: written by the forward when given,
+                                  // read by the backward that does not rebuild them
     int32_t* counters;            // (H, NQUEUE) work-queue heads
     uint32_t* items;              // (N, H, REC_WORDS) item records of this launch
     unsigned long long* stats;    // optional running totals (see STAT_* below); never reset by a launch

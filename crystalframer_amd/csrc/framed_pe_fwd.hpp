@@ -169,6 +169,15 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                         hv[4 * k4 + 0] = (float)t4.x; hv[4 * k4 + 1] = (float)t4.y;
                         hv[4 * k4 + 2] = (float)t4.z; hv[4 * k4 + 3] = (float)t4.w;
                     }
+                    if (P.shat && half * 4 + sub < ng) {
+                        // keep the histograms for the backward pass: this lane's 16 bins of (pair, enc)
+                        float4* dst = reinterpret_cast<float4*>(
+                            P.shat + (((size_t)(g0 + half * 4 + sub) * H + h) * 4 + enc) * NBINS + 16 * cg);
+#pragma unroll
+                        for (int k4 = 0; k4 < 4; k4++)
+                            dst[k4] = make_float4(hv[4 * k4 + 0] * FIX_INV, hv[4 * k4 + 1] * FIX_INV,
+                                                  hv[4 * k4 + 2] * FIX_INV, hv[4 * k4 + 3] * FIX_INV);
+                    }
                     v4f acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
                     v4f acc2 = {0.f, 0.f, 0.f, 0.f}, acc3 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll

@@ -148,7 +148,10 @@ int cfh_frame_axes(const cfh_params* p, const float* q, const float* k, const fl
  * psi (E,H,Dh) = dist_coef * W_dist.s_dist + angle_coef * sum_axis W_axis.s_axis, where s are the
  * softmax-over-translations averages of the truncated Gaussian bases of the distance and of the
  * cosine to each frame axis.  W_dist (H,Dh,K); W_axis[3] each (H,Dh,A) or all NULL; frames
- * (3,N,H,3) or NULL.  d2min_out (E,H) is optional.
+ * (3,N,H,3) or NULL.  d2min_out (E,H) is optional.  shat_out (E,H,4,64) is optional: when given,
+ * the softmax-averaged basis values s (the window histograms, rows: distance, axis 1..3) are kept
+ * for cfh_framed_pe_backward, which then rebuilds nothing (1 KB per (pair, head) of HBM against
+ * about a third of the backward's time).
  * Replaces RealEncodingWithFramedProjFuncCUDA.forward: kernels real_enc_frame_proj_fwd_length and
  * real_enc_frame_proj_fwd_angle and the sums between them
  * (models/cuda_funcs/real_space_framed_proj.py:21-120).
@@ -158,14 +161,15 @@ int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* r
                           const int64_t* edges, const int64_t* e_start, const int32_t* order,
                           const float* W_dist, const float* W_axis1, const float* W_axis2,
                           const float* W_axis3, const float* frames, int64_t N, int64_t E,
-                          int64_t B, float* z, float* psi, float* d2min_out, void* workspace,
-                          size_t workspace_bytes, void* stream);
+                          int64_t B, float* z, float* psi, float* d2min_out, float* shat_out,
+                          void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Gradients of the above for upstream gz (E,H) and gpsi (E,H,Dh): ga (N,H), gW_dist (H,Dh,K),
  * gW_axis[3] (H,Dh,A).  The per-translation weights are recomputed from z, not stored.  The
  * weight gradients are returned already summed over atoms.  No gradient flows to the frames
- * (the reference returns None for them).
+ * (the reference returns None for them).  `shat` is what the forward wrote to shat_out, or NULL
+ * (the histograms are then rebuilt, as the reference does).
  * Replaces RealEncodingWithFramedProjFuncCUDA.backward: kernels real_enc_frame_proj_bwd_length and
  * real_enc_frame_proj_bwd_angle (models/cuda_funcs/real_space_framed_proj.py:123-221).
  */
@@ -174,9 +178,10 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
                            const int64_t* edges, const int64_t* e_start, const int32_t* order,
                            const float* W_dist, const float* W_axis1, const float* W_axis2,
                            const float* W_axis3, const float* frames, const float* z,
-                           const float* gz, const float* gpsi, int64_t N, int64_t E, int64_t B,
-                           float* ga, float* gW_dist, float* gW_axis1, float* gW_axis2,
-                           float* gW_axis3, void* workspace, size_t workspace_bytes, void* stream);
+                           const float* gz, const float* gpsi, const float* shat, int64_t N,
+                           int64_t E, int64_t B, float* ga, float* gW_dist, float* gW_axis1,
+                           float* gW_axis2, float* gW_axis3, void* workspace, size_t workspace_bytes,
+                           void* stream);
 
 /*
  * Attention over the pairs of each atom: l_e = q_i.k_j + aij_e, p = softmax over the pairs (i,.)

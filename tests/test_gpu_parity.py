@@ -26,6 +26,7 @@ def _defaults():
     import crystalframer_amd as cf
     KM = cf.KernelManager
     saved = (KM.SYMM_BREAK_NOISE, KM.PRUNE_LOG2, KM.WINDOW_MODE, KM.GRAD_COEF_QUIRK, KM.LATTICE_RANGE, KM.MINIMUM_RANGE)
+    saved_hist = KM.SAVE_HISTOGRAMS
     KM.SYMM_BREAK_NOISE = 0.0
     KM.PRUNE_LOG2 = 24.0
     KM.WINDOW_MODE = 0
@@ -33,6 +34,7 @@ def _defaults():
     KM.LATTICE_RANGE, KM.MINIMUM_RANGE = 2, 2
     yield
     (KM.SYMM_BREAK_NOISE, KM.PRUNE_LOG2, KM.WINDOW_MODE, KM.GRAD_COEF_QUIRK, KM.LATTICE_RANGE, KM.MINIMUM_RANGE) = saved
+    KM.SAVE_HISTOGRAMS = saved_hist
 
 
 def dev():
@@ -71,9 +73,13 @@ def oracle_pe(P, *, K=64, A=64, cos_abs=0, cd=1.0, ca=1.0, cutoff=CUT, windows="
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("cos_abs", [0, 1])
 @pytest.mark.parametrize("prune", [0.0, 24.0, 32.0])
-def test_framed_pe_forward_backward_reference_windows(cos_abs, prune):
+@pytest.mark.parametrize("save_histograms", [True, False])
+def test_framed_pe_forward_backward_reference_windows(cos_abs, prune, save_histograms):
+    """Both backward kernels: the one that reads the histograms the forward kept and the one that
+    rebuilds them (the reference's way)."""
     import crystalframer_amd as cf
     cf.KernelManager.PRUNE_LOG2 = prune
+    cf.KernelManager.SAVE_HISTOGRAMS = save_histograms
     P = Hh.make_problem(num_crystals=10, atoms_hi=6, seed=100 + cos_abs)
     cd, ca = 0.75, 1.25
     (z, psi), a, Wk, Wax = run_pe(P, cos_abs=cos_abs, cd=cd, ca=ca)

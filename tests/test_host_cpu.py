@@ -41,7 +41,7 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert b"head_dim" in lib.cfh_last_error()
     p.head_dim = 16
     p.struct_size = 4
-    rc = lib.cfh_framed_pe_forward(ctypes.byref(p), *([None] * 13), 1, 1, 1, None, None, None, None, 0, None)
+    rc = lib.cfh_framed_pe_forward(ctypes.byref(p), *([None] * 13), 1, 1, 1, None, None, None, None, None, 0, None)
     assert rc == -1 and b"struct_size" in lib.cfh_last_error()
 
 
