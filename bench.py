@@ -38,9 +38,11 @@ PEAK_TRANS_TOPS = 9.8                  # quarter-rate transcendental unit
 # HBM bytes per launch of the dominant kernel on this workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch) scaled by what the same counters read for the 256 MiB device copy of --calibrate-copy
 # (FETCH_SIZE reads 128 MiB for it: factor 2.0; WRITE_SIZE reads 256 MiB: factor 1.0); see profiles/.
-# backward: 25 502 KiB x 2.0 fetched + 34 248 KiB written (33.5 MB of that are the per-wavefront partials of
-# the weight gradients).  The forward kernel's fetches were not collected.
-TRAFFIC_BYTES_PER_LAUNCH = {"framed_pe_backward": 87.3e6, "framed_pe_forward": None}
+# With the forward keeping its window histograms for the backward (KernelManager.SAVE_HISTOGRAMS, the default):
+# forward 3 627 KiB x 2.0 fetched + 262 023 KiB written (243.9 MB of that are the histograms, E x H x 4 x 64
+# floats); backward 144 847 KiB x 2.0 fetched (the histograms again) + 34 261 KiB written (33.5 MB of that are
+# the per-wavefront partials of the weight gradients).
+TRAFFIC_BYTES_PER_LAUNCH = {"framed_pe_backward": 331.7e6, "framed_pe_forward": 275.7e6}
 
 
 def parse():
