@@ -50,7 +50,8 @@ EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_fram
            "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_backward",
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
            "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
-           "cfh_linear_weight_bias_grad")
+           "cfh_linear_weight_bias_grad", "cfh_attention_inputs_forward",
+           "cfh_attention_inputs_backward")
 
 _lib = None
 _lock = threading.Lock()
@@ -101,6 +102,12 @@ def load():
         lib.cfh_crystal_mean_backward.argtypes = [_P, _P, _P, _I64, _I64, _I64, _P, _P]
         lib.cfh_linear_weight_bias_grad.restype = ctypes.c_int
         lib.cfh_linear_weight_bias_grad.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P, _P]
+        _F, _I32 = ctypes.c_float, ctypes.c_int32
+        lib.cfh_attention_inputs_forward.restype = ctypes.c_int
+        lib.cfh_attention_inputs_forward.argtypes = [_P, _P, _P, _F, _F, _F, _F, _I64, _I32, _I32, _P, _P, _P, _P, _P]
+        lib.cfh_attention_inputs_backward.restype = ctypes.c_int
+        lib.cfh_attention_inputs_backward.argtypes = [_P, _P, _P, _F, _F, _F, _F, _P, _P, _P, _P, _I64, _I32, _I32,
+                                                      _P, _P, _P]
         lib.cfh_timing_enable.restype = ctypes.c_int
         lib.cfh_timing_enable.argtypes = [ctypes.c_int]
         lib.cfh_timing_read.restype = ctypes.c_int

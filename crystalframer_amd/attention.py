@@ -22,18 +22,22 @@ from .params import LatticeformerParams
 
 
 FUSED_FRAMES = True      # one launch for both axes + orthogonalisation (False: the reference's three steps)
+FUSED_INPUTS = True      # q/k/v split, query scaling and Gaussian coefficient in one launch (False: framework ops)
 
 
 def compute_frame_maximum_method_(q, k, v, alpha, pos, dist2_min, tvecs, batch, edges, proj, K: int,
                                   dist_max: float, wscale: float, frame_method: str, this_epoch=None,
-                                  rvecs: Optional[Tensor] = None, cutoff: Optional[float] = None):
-    """Three orthonormal frame axes per (atom, head).
+                                  rvecs: Optional[Tensor] = None, cutoff: Optional[float] = None,
+                                  q_is_scaled: bool = False):
+    """Three orthonormal frame axes per (atom, head).  ``q_is_scaled``: the query already carries
+    the 1/sqrt(Dh) that the reference applies here.
     Reference: models/indexed_lattice_multi_head_attention_cuda.py:435-493."""
     adap = ()
     if cutoff is not None:
         rvlen = rvecs if rvecs.dim() == 2 else torch.norm(rvecs, 2, dim=-1)
         adap = (rvlen, cutoff)
-    q = q / math.sqrt(q.shape[-1])
+    if not q_is_scaled:
+        q = q / math.sqrt(q.shape[-1])
     if frame_method != "max":
         raise NotImplementedError(f"frame_method={frame_method!r}: only 'max' is implemented")
     if FUSED_FRAMES:
@@ -52,7 +56,8 @@ def compute_frame_maximum_method_(q, k, v, alpha, pos, dist2_min, tvecs, batch, 
 
 def compute_real_domain_attn_frame_proj(q, k, v, batch_q, batch_kv, edges, pos, dist2_min, tvecs, rvecs,
                                         pe_dist_proj, proj_angle1, proj_angle2, proj_angle3, alpha,
-                                        params: LatticeformerParams, this_epoch=None, frame_sink=None):
+                                        params: LatticeformerParams, this_epoch=None, frame_sink=None,
+                                        q_is_scaled: bool = False):
     """z (E,H) and psi (E,H,Dh) for one layer.
     Reference: models/indexed_lattice_multi_head_attention_cuda.py:589-734 (frame_method 'max')."""
     K = params.value_pe_dist_real
@@ -77,7 +82,7 @@ def compute_real_domain_attn_frame_proj(q, k, v, batch_q, batch_kv, edges, pos, 
         # is the angle encoding, so they are skipped here in that case
         f1, f2, f3 = compute_frame_maximum_method_(
             q, k, None, alpha, pos, dist2_min, tvecs, batch_q, edges, pe_dist_proj, K, dist_max, wscale,
-            params.frame_method, this_epoch, *rvlen_args)
+            params.frame_method, this_epoch, *rvlen_args, q_is_scaled=q_is_scaled)
     else:
         f1 = f2 = f3 = None
     if frame_sink is not None:
@@ -93,9 +98,11 @@ def compute_real_domain_attn_frame_proj(q, k, v, batch_q, batch_kv, edges, pos, 
     return out
 
 
-def _scaled_dot_product_attention(q, k, v, batch, batch_kv, edges, attn_weights=None, values=None):
+def _scaled_dot_product_attention(q, k, v, batch, batch_kv, edges, attn_weights=None, values=None,
+                                  q_is_scaled: bool = False):
     """Reference: models/indexed_lattice_multi_head_attention_cuda.py:144-185."""
-    q = q / math.sqrt(q.shape[-1])
+    if not q_is_scaled:
+        q = q / math.sqrt(q.shape[-1])
     return cuda_funcs.FusedDotProductAttentionCUDA.apply(q, k, v, attn_weights, values, batch, edges)
 
 
@@ -172,6 +179,18 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
         self._gauss_ready = None
         return super()._load_from_state_dict(*args, **kwargs)
 
+    def _gauss_constants(self):
+        """(c1, lb, c2) of a = ((1 - lb) elu(c1 alpha') + 1) c2."""
+        P = self.params
+        lb = P.gauss_lb_real
+        return P.positive_func_beta / (1.0 - lb), lb, -0.5 * P.scale_real ** -2
+
+    def _gauss_scale_ready(self) -> bool:
+        """True once gauss_scale holds the normalisation of alpha (one host read, then cached)."""
+        if self._gauss_ready is None:
+            self._gauss_ready = bool(self.gauss_scale[0] > 0)
+        return self._gauss_ready
+
     def gaussian_coefficient(self, q: Tensor) -> Tensor:
         """alpha = q_h . w_h, normalised, mapped to a = [(1-lb) elu(alpha beta/(1-lb)) + 1] (-1/2 r0^-2).
         Reference: models/indexed_lattice_multi_head_attention_cuda.py:896-940."""
@@ -207,6 +226,7 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
             raise NotImplementedError("need_weights=True is not implemented")
         N = query.shape[0]
         H, Dh = self.num_heads, self.head_dim
+        q_is_scaled = False
         if self.in_proj_bias is None:
             bq = bk = bv = None
         else:
@@ -217,19 +237,31 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
             # become one launch instead of three)
             w_in = torch.cat([self.q_proj_weight, self.k_proj_weight, self.v_proj_weight], dim=0)
             qkv = cuda_funcs.linear(query, w_in, self.in_proj_bias)
-            q, k, v = qkv.split([self.kdim, self.kdim, self.vdim], dim=1)
-            q = q.reshape(N, H, -1)
-            k = k.reshape(N, H, -1)
-            v = v.reshape(N, H, -1)
+            fused = (FUSED_INPUTS and self.kdim == self.vdim == H * Dh
+                     and cuda_funcs.AttentionInputsHIP.supported(H, Dh)
+                     and (not self.params.normalize_gauss or self._gauss_scale_ready()))
+            if fused:
+                # split, query scaling and Gaussian coefficient in one launch (one more in backward)
+                c1, lb, c2 = self._gauss_constants()
+                q, k, v, a = cuda_funcs.AttentionInputsHIP.apply(
+                    qkv, self.lattice_pos_weights, self.gauss_scale if self.params.normalize_gauss else None,
+                    H, c1, lb, c2, 1.0 / math.sqrt(Dh))
+                q_is_scaled = True
+            else:
+                q, k, v = qkv.split([self.kdim, self.kdim, self.vdim], dim=1)
+                q = q.reshape(N, H, -1)
+                k = k.reshape(N, H, -1)
+                v = v.reshape(N, H, -1)
         else:
             q = cuda_funcs.linear(query, self.q_proj_weight, bq).view(N, H, -1)
             k = cuda_funcs.linear(key, self.k_proj_weight, bk).view(key.shape[0], H, -1)
             v = cuda_funcs.linear(value, self.v_proj_weight, bv).view(value.shape[0], H, -1)
-        a = self.gaussian_coefficient(q)
+        if not q_is_scaled:
+            a = self.gaussian_coefficient(q)
         z, psi = compute_real_domain_attn_frame_proj(
             q, k, v, batch_q, batch_kv, edges, points, dist2_min, tvecs, rvecs, self.pe_dist_proj,
             self.proj_angle1, self.proj_angle2, self.proj_angle3, a, self.params, this_epoch,
-            frame_sink=self.frame_sink)
-        out = _scaled_dot_product_attention(q, k, v, batch_q, batch_kv, edges, z, psi)
+            frame_sink=self.frame_sink, q_is_scaled=q_is_scaled)
+        out = _scaled_dot_product_attention(q, k, v, batch_q, batch_kv, edges, z, psi, q_is_scaled=q_is_scaled)
         out = cuda_funcs.linear(out.reshape(N, H * v.shape[-1]), self.out_proj.weight, self.out_proj.bias)
         return out, psi

@@ -13,6 +13,7 @@
 #include <string>
 #include <vector>
 
+#include "attention_inputs.hpp"
 #include "device_common.hpp"
 #include "frame_select.hpp"
 #include "framed_pe_bwd.hpp"
@@ -553,4 +554,50 @@ int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int6
     return finish_launch("linear_weight_bias_grad");
 }
 
+static int attention_inputs_args(cfh::AttnInArgs& A, const float* qkv, const float* w, const float* gauss, float c1,
+                                 float lb, float c2, float q_scale, int64_t N, int32_t H, int32_t Dh) {
+    if (Dh != 16 || H < 1 || 256 % (H * Dh) != 0)
+        return fail(CFH_EINVAL, "attention inputs: head_dim must be 16 and 256 a multiple of H*Dh (H=%d Dh=%d)", H, Dh);
+    if (N < 0 || N > 0x7fffffffLL / (3 * H * Dh)) return fail(CFH_EINVAL, "N=%lld out of range", (long long)N);
+    if (N > 0 && (!qkv || !w)) return fail(CFH_EINVAL, "qkv and lattice_w must not be NULL");
+    A = cfh::AttnInArgs{};
+    A.qkv = qkv; A.w = w; A.gauss = gauss; A.N = (int)N; A.HD = H * Dh;
+    A.c1 = c1; A.lb = lb; A.c2 = c2; A.q_scale = q_scale;
+    return CFH_OK;
+}
+
+int cfh_attention_inputs_forward(const float* qkv, const float* lattice_w, const float* gauss_scale_dev,
+                                 float c1, float lb, float c2, float q_scale, int64_t N, int32_t H, int32_t Dh,
+                                 float* qs, float* k, float* v, float* a, void* stream) {
+    cfh::AttnInArgs A;
+    if (int rc = attention_inputs_args(A, qkv, lattice_w, gauss_scale_dev, c1, lb, c2, q_scale, N, H, Dh)) return rc;
+    if (N == 0) return CFH_OK;
+    if (!qs || !k || !v || !a) return fail(CFH_EINVAL, "qs, k, v and a must not be NULL");
+    A.qs = qs; A.k = k; A.v = v; A.a = a;
+    const long total = (long)N * A.HD;
+    hipLaunchKernelGGL(cfh::attention_inputs_fwd_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, A);
+    return finish_launch("attention_inputs_forward");
+}
+
+int cfh_attention_inputs_backward(const float* qkv, const float* lattice_w, const float* gauss_scale_dev,
+                                  float c1, float lb, float c2, float q_scale, const float* gqs, const float* gk,
+                                  const float* gv, const float* ga, int64_t N, int32_t H, int32_t Dh,
+                                  float* gqkv, float* g_lattice_w, void* stream) {
+    cfh::AttnInArgs A;
+    if (int rc = attention_inputs_args(A, qkv, lattice_w, gauss_scale_dev, c1, lb, c2, q_scale, N, H, Dh)) return rc;
+    if (!g_lattice_w || (N > 0 && !gqkv)) return fail(CFH_EINVAL, "gqkv and g_lattice_w must not be NULL");
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(cfh::zero2_kernel, dim3((A.HD + 255) / 256), dim3(256), 0, st, g_lattice_w, A.HD,
+                       (float*)nullptr, 0);
+    if (N > 0) {
+        A.gqs = gqs; A.gk = gk; A.gv = gv; A.ga = ga; A.gqkv = gqkv; A.gw = g_lattice_w;
+        A.rows_per_block = 8 * (256 / A.HD);
+        hipLaunchKernelGGL(cfh::attention_inputs_bwd_kernel, dim3((unsigned)((N + A.rows_per_block - 1) / A.rows_per_block)),
+                           dim3(256), 0, st, A);
+    }
+    return finish_launch("attention_inputs_backward");
+}
+
 }  // extern "C"
+

@@ -508,6 +508,59 @@ class LinearHIP(torch.autograd.Function):
         return gx, gw, gb
 
 
+class AttentionInputsHIP(torch.autograd.Function):
+    """(qs, k, v, a) from the stacked projection output qkv (N, 3 H Dh): query scaled by q_scale,
+    key, value, and the Gaussian coefficient a (N,H) = ((1 - lb) elu(c1 alpha') + 1) c2 with
+    alpha = q_h . lattice_w_h, alpha' = (alpha + gauss_scale[1]) gauss_scale[0] (gauss_scale None:
+    alpha' = alpha; it is treated as a constant).  One launch each way instead of the framework's
+    elementwise chain (reference arithmetic: models/indexed_lattice_multi_head_attention_cuda.py:896-940,
+    query scaling :144-185)."""
+
+    @staticmethod
+    def supported(H: int, Dh: int) -> bool:
+        return Dh == 16 and H >= 1 and 256 % (H * Dh) == 0
+
+    @staticmethod
+    def forward(ctx, qkv, lattice_w, gauss_scale, H, c1, lb, c2, q_scale):
+        _lib.require_gpu(qkv, lattice_w)
+        lib = _lib.load()
+        N = qkv.shape[0]
+        HD = qkv.shape[1] // 3
+        Dh = HD // H
+        qkv = _f32c(qkv)
+        w = _f32c(lattice_w.detach())
+        gs = _f32c(gauss_scale.detach()) if gauss_scale is not None else None
+        qs = torch.empty((N, H, Dh), dtype=torch.float32, device=qkv.device)
+        k = torch.empty_like(qs)
+        v = torch.empty_like(qs)
+        a = torch.empty((N, H), dtype=torch.float32, device=qkv.device)
+        with _timed("attention_inputs_forward", qkv.device):
+            rc = lib.cfh_attention_inputs_forward(_lib.ptr(qkv), _lib.ptr(w), _lib.ptr(gs), c1, lb, c2, q_scale, N, H, Dh,
+                                                  _lib.ptr(qs), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a),
+                                                  _lib.current_stream_ptr(qkv.device))
+        _lib.check(rc, "cfh_attention_inputs_forward")
+        ctx.save_for_backward(qkv, w, gs)
+        ctx.consts = (H, Dh, c1, lb, c2, q_scale)
+        ctx.set_materialize_grads(False)
+        return qs, k, v, a
+
+    @staticmethod
+    def backward(ctx, gqs, gk, gv, ga):
+        qkv, w, gs = ctx.saved_tensors
+        H, Dh, c1, lb, c2, q_scale = ctx.consts
+        lib = _lib.load()
+        N = qkv.shape[0]
+        gqs, gk, gv, ga = (None if g is None else _f32c(g) for g in (gqs, gk, gv, ga))
+        gqkv = torch.empty_like(qkv)
+        gw = torch.empty((H * Dh,), dtype=torch.float32, device=qkv.device)
+        with _timed("attention_inputs_backward", qkv.device):
+            rc = lib.cfh_attention_inputs_backward(_lib.ptr(qkv), _lib.ptr(w), _lib.ptr(gs), c1, lb, c2, q_scale,
+                                                   _lib.ptr(gqs), _lib.ptr(gk), _lib.ptr(gv), _lib.ptr(ga), N, H, Dh,
+                                                   _lib.ptr(gqkv), _lib.ptr(gw), _lib.current_stream_ptr(qkv.device))
+        _lib.check(rc, "cfh_attention_inputs_backward")
+        return gqkv, gw, None, None, None, None, None, None
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """torch.nn.functional.linear for device tensors, with the library's weight-gradient kernel."""
     _lib.require_gpu(x, weight)

@@ -241,6 +241,26 @@ int cfh_crystal_mean_backward(const float* gout, const int64_t* batch, const int
 int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int64_t I, int64_t O,
                                 float* dW, float* db, void* stream);
 
+/*
+ * What lies between the stacked q/k/v projection of a layer and its kernels, one launch each way.
+ * Forward: qkv (N, 3 H Dh), rows = [query | key | value];  qs = query * q_scale, k, v (N,H,Dh) contiguous,
+ *   a (N,H) = ((1 - lb) elu(c1 alpha') + 1) c2  with alpha = query_h . lattice_w_h and
+ *   alpha' = (alpha + gauss_scale_dev[1]) * gauss_scale_dev[0]  (alpha' = alpha when the pointer is NULL).
+ * Backward: gqkv (N, 3 H Dh) = [ga da/dquery + gqs q_scale | gk | gv],  g_lattice_w (H Dh) = sum over atoms
+ *   of ga da/dalpha query;  gqs, gk, gv, ga may each be NULL (zero).  gauss_scale_dev is a constant.
+ * Dh = 16, 256 % (H Dh) == 0.  Replaces the framework arithmetic of
+ * models/indexed_lattice_multi_head_attention_cuda.py:896-940 (gaussian coefficient: c1 = beta / (1 - lb),
+ * c2 = -1/2 scale_real^-2), the query scaling of :144-185 and :455, and the chunk / cat of the
+ * projection output and its gradient (:399-409).
+ */
+int cfh_attention_inputs_forward(const float* qkv, const float* lattice_w, const float* gauss_scale_dev,
+                                 float c1, float lb, float c2, float q_scale, int64_t N, int32_t H, int32_t Dh,
+                                 float* qs, float* k, float* v, float* a, void* stream);
+int cfh_attention_inputs_backward(const float* qkv, const float* lattice_w, const float* gauss_scale_dev,
+                                  float c1, float lb, float c2, float q_scale, const float* gqs, const float* gk,
+                                  const float* gv, const float* ga, int64_t N, int32_t H, int32_t Dh,
+                                  float* gqkv, float* g_lattice_w, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

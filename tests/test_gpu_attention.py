@@ -190,3 +190,45 @@ def test_linear_weight_and_bias_gradients(N, I, O, bias):
             assert Hh.rel_err(b.grad, b64.grad) < 1e-5
     else:
         assert float(w.grad.abs().max()) == 0.0 and float(b.grad.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("N,H,normalised", [(2372, 8, True), (37, 8, False), (5, 2, True), (1, 16, True), (0, 8, True)])
+def test_attention_inputs_split_scale_and_gaussian_coefficient(N, H, normalised):
+    """q/k/v split + query scaling + Gaussian coefficient in one launch against the float64
+    framework arithmetic (alpha = q.w, normalised, elu, affine), forward and gradients."""
+    import math
+    import crystalframer_amd as cf
+    Dh, lb, beta, scale_real = 16, 0.5, 0.1, 1.4
+    c1, c2 = beta / (1.0 - lb), -0.5 * scale_real ** -2
+    gen = torch.Generator().manual_seed(100 + N + H)
+    qkv64 = (torch.randn(N, 3 * H * Dh, generator=gen, dtype=torch.float64) * 3).requires_grad_(True)
+    w64 = torch.randn(H * Dh, generator=gen, dtype=torch.float64, requires_grad=True)
+    gs64 = torch.tensor([0.37, -0.8], dtype=torch.float64) if normalised else None
+    q, k, v = (t.reshape(N, H, Dh) for t in qkv64.split(H * Dh, dim=1))
+    alpha = (q * w64.view(1, H, Dh)).sum(-1)
+    if normalised:
+        alpha = (alpha + gs64[1]) * gs64[0]
+    a64 = ((1.0 - lb) * torch.nn.functional.elu(alpha * c1) + 1.0) * c2
+    qs64 = q / math.sqrt(Dh)
+    g = [torch.randn(t.shape, generator=gen, dtype=torch.float64) for t in (qs64, k, v, a64)]
+    sum((o * gi).sum() for o, gi in zip((qs64, k, v, a64), g)).backward()
+
+    qkv = f32(qkv64.detach()).requires_grad_(True)
+    w = f32(w64.detach()).requires_grad_(True)
+    gs = f32(gs64) if normalised else None
+    outs = cf.cuda_funcs.AttentionInputsHIP.apply(qkv, w, gs, H, c1, lb, c2, 1.0 / math.sqrt(Dh))
+    assert [tuple(o.shape) for o in outs] == [(N, H, Dh)] * 3 + [(N, H)]
+    sum((o * f32(gi)).sum() for o, gi in zip(outs, g)).backward()
+    if N == 0:
+        assert float(w.grad.abs().max()) == 0.0
+        return
+    for o, ref in zip(outs, (qs64, k, v, a64)):
+        assert Hh.rel_err(o.detach(), ref.detach()) < 1e-6
+    assert Hh.rel_err(qkv.grad, qkv64.grad) < 1e-6
+    assert Hh.rel_err(w.grad, w64.grad) < 1e-5
+    # only the value gradient given: the others count as zero
+    qkv.grad = None
+    outs = cf.cuda_funcs.AttentionInputsHIP.apply(qkv, w, gs, H, c1, lb, c2, 1.0 / math.sqrt(Dh))
+    (outs[2] * f32(g[2])).sum().backward()
+    expect = torch.cat([torch.zeros(N, 2 * H * Dh, dtype=torch.float64), g[2].reshape(N, -1)], dim=1)
+    assert Hh.rel_err(qkv.grad, expect) < 1e-6

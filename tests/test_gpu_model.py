@@ -9,7 +9,7 @@ from oracle import cpu_model
 pytestmark = pytest.mark.gpu
 
 
-def _run(mp, cb, seed=0):
+def _run(mp, cb, seed=0, passes=1):
     import crystalframer_amd as cf
     from crystalframer_amd import latticeformer
     KM = cf.KernelManager
@@ -19,10 +19,16 @@ def _run(mp, cb, seed=0):
     model = latticeformer.Latticeformer(mp).to(dev)
     for layer in model.encoder.layers:
         layer.self_attn.frame_sink = []
-    out = model(cb.to(dev))
     target = torch.linspace(-1, 1, cb.num_crystals, device=dev)[:, None]
-    loss = torch.nn.functional.mse_loss(out, target)
-    loss.backward()
+    for _ in range(passes):
+        # the first training-mode pass measures and stores the normalisation of alpha with framework
+        # ops; later passes take the fused split / scaling / Gaussian-coefficient launch
+        model.zero_grad(set_to_none=True)
+        for layer in model.encoder.layers:
+            layer.self_attn.frame_sink.clear()
+        out = model(cb.to(dev))
+        loss = torch.nn.functional.mse_loss(out, target)
+        loss.backward()
     torch.cuda.synchronize()
     sd = {k: v.detach().cpu().double() for k, v in model.state_dict().items()}
     leaves = {k: v.clone().requires_grad_("scale" not in k) for k, v in sd.items()}
@@ -35,13 +41,13 @@ def _run(mp, cb, seed=0):
     return model, out, ref, leaves
 
 
-@pytest.mark.parametrize("angle_bins", [64, 0])
-def test_model_forward_backward_matches_cpu_oracle(angle_bins):
+@pytest.mark.parametrize("angle_bins,passes", [(64, 1), (0, 1), (64, 2)])
+def test_model_forward_backward_matches_cpu_oracle(angle_bins, passes):
     from crystalframer_amd import params, synthetic
     mp = params.ModelParams(num_layers=2, value_pe_angle_real=angle_bins, symm_break_noise=0.0)
     cb = synthetic.make_batch(8, atoms="uniform", atoms_lo=1, atoms_hi=6, len_lo=3.0, len_hi=9.0,
                               ang_lo=65.0, ang_hi=115.0, seed=11)
-    model, out, ref, leaves = _run(mp, cb)
+    model, out, ref, leaves = _run(mp, cb, passes=passes)
     assert Hh.rel_err(out, ref) < 1e-4
     checked = 0
     for name, p in model.named_parameters():
