@@ -17,7 +17,7 @@
 namespace cfh {
 
 constexpr int WAVE = 64;
-constexpr int TCAP = 512;      // translations staged in LDS per pass (8 KB of float4)
+constexpr int TCAP = 256;      // frame search: translations per chunk (4 KB of float4 when staged in LDS)
 constexpr int NBINS = 64;      // distance bins K and angle bins A the kernels are compiled for
 constexpr int DH = 16;         // head dimension the kernels are compiled for
 constexpr int HS = 72;         // padded row stride (floats) of the 4 x 64 histograms in LDS

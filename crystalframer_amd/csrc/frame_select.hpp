@@ -24,13 +24,20 @@
 
 namespace cfh {
 
+// translation index -> box coordinates, t = (i1 s2 + i2) s3 + i3; the quotients by float reciprocal
+// (exact: t + 1/2 over a divisor below 2^10 is never within rounding of an integer)
+__device__ __forceinline__ void box_coords(int t, const Box& bx, float inv_s2, float inv_s3, int& n1, int& n2, int& n3) {
+    const int q = (int)(((float)t + 0.5f) * inv_s3);
+    const int i1 = (int)(((float)q + 0.5f) * inv_s2);
+    n3 = t - q * bx.s3 - bx.R3;
+    n2 = q - i1 * bx.s2 - bx.R2;
+    n1 = i1 - bx.R1;
+}
 __device__ __forceinline__ void shift_of(int t, const Box& bx, const Lattice& L, float& vx, float& vy,
                                          float& vz) {
-    const int i3 = t % bx.s3;
-    const int q = t / bx.s3;
-    const int i2 = q % bx.s2;
-    const int i1 = q / bx.s2;
-    const float n1 = (float)(i1 - bx.R1), n2 = (float)(i2 - bx.R2), n3 = (float)(i3 - bx.R3);
+    int m1, m2, m3;
+    box_coords(t, bx, 1.0f / (float)bx.s2, 1.0f / (float)bx.s3, m1, m2, m3);
+    const float n1 = (float)m1, n2 = (float)m2, n3 = (float)m3;
     vx = fmaf(L.t[6], n3, fmaf(L.t[3], n2, L.t[0] * n1));
     vy = fmaf(L.t[7], n3, fmaf(L.t[4], n2, L.t[1] * n1));
     vz = fmaf(L.t[8], n3, fmaf(L.t[5], n2, L.t[2] * n1));
@@ -67,6 +74,10 @@ template <int MODE>
 __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
     __shared__ float4 tab[TCAP];
     __shared__ float4 pair_rq[WAVE];        // rpos and q.k of up to 64 pairs
+    // one-chunk boxes do not use the table: its memory holds the translation order and per-pair scalars
+    uint16_t* const perm = reinterpret_cast<uint16_t*>(tab);              // [TCAP] position -> translation
+    float* const reach = reinterpret_cast<float*>(tab) + TCAP / 2;        // [WAVE] see the slab skip below
+    float* const phase_of = reach + WAVE;                                 // [WAVE] noise phase of a pair
     const int lane = threadIdx.x;
     const int H = P.H;
     const int h = blockIdx.x % H;
@@ -96,11 +107,53 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
 #pragma unroll
         for (int c = 0; c < DH; c++) qi[c] = rec_f(rec_cur, REC_QUERY + c);
         const int nchunks = (bx.T + TCAP - 1) / TCAP;
-        float sx[TCAP / WAVE], sy[TCAP / WAVE], sz[TCAP / WAVE];
+        // One-chunk boxes (T <= TCAP): the lane keeps the shifts of its translations in registers, slab k
+        // = positions lane + 64 k of an order that puts the 27 translations with every |n_d| <= 1 first
+        // (both groups in the reference's loop order).  The slabs k >= 1 then hold distant translations
+        // only, and a whole (pair, slab) is skipped when its nearest possible image cannot reach the
+        // best score found in slab 0 (smin = smallest shift length of the slab).
+        float sx[TCAP / WAVE], sy[TCAP / WAVE], sz[TCAP / WAVE], smin[TCAP / WAVE];
+        int tt[TCAP / WAVE];
+        if (nchunks == 1) {
+            const float inv_s2 = 1.0f / (float)bx.s2, inv_s3 = 1.0f / (float)bx.s3;
+            const int ncore = min(3, 2 * bx.R1 + 1) * min(3, bx.s2) * min(3, bx.s3);
+            int seen_core = 0, seen_out = 0;
+            wave_sync();                      // the previous item's readers of perm / reach / phase are done
 #pragma unroll
-        for (int k = 0; k < TCAP / WAVE; k++) {
-            sx[k] = sy[k] = sz[k] = 0.0f;
-            if (nchunks == 1 && k * WAVE < bx.T) shift_of(min(lane + k * WAVE, bx.T - 1), bx, L, sx[k], sy[k], sz[k]);
+            for (int k = 0; k < TCAP / WAVE; k++)
+                if (k * WAVE < bx.T) {
+                    const int t = lane + k * WAVE;
+                    int n1, n2, n3;
+                    box_coords(t, bx, inv_s2, inv_s3, n1, n2, n3);
+                    const bool valid = t < bx.T;
+                    const bool core = valid && abs(n1) <= 1 && abs(n2) <= 1 && abs(n3) <= 1;
+                    const uint64_t mc = __ballot(core), mo = __ballot(valid && !core);
+                    if (core) perm[seen_core + lane_prefix(mc)] = (uint16_t)t;
+                    else if (valid) perm[ncore + seen_out + lane_prefix(mo)] = (uint16_t)t;
+                    seen_core += __popcll(mc);
+                    seen_out += __popcll(mo);
+                }
+            wave_sync();
+#pragma unroll
+            for (int k = 0; k < TCAP / WAVE; k++) {
+                sx[k] = sy[k] = sz[k] = 0.0f; smin[k] = 0.0f; tt[k] = 0;
+                if (k * WAVE < bx.T) {
+                    const bool valid = lane + k * WAVE < bx.T;
+                    tt[k] = perm[min(lane + k * WAVE, bx.T - 1)];
+                    int n1, n2, n3;
+                    box_coords(tt[k], bx, inv_s2, inv_s3, n1, n2, n3);
+                    const float f1 = (float)n1, f2 = (float)n2, f3 = (float)n3;
+                    sx[k] = fmaf(L.t[6], f3, fmaf(L.t[3], f2, L.t[0] * f1));
+                    sy[k] = fmaf(L.t[7], f3, fmaf(L.t[4], f2, L.t[1] * f1));
+                    sz[k] = fmaf(L.t[8], f3, fmaf(L.t[5], f2, L.t[2] * f1));
+                    if (k > 0)
+                        smin[k] = uniform_f(wave_min(valid ? sqrtf(fmaf(sx[k], sx[k], fmaf(sy[k], sy[k], sz[k] * sz[k])))
+                                                           : 3.0e38f));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < TCAP / WAVE; k++) { sx[k] = sy[k] = sz[k] = 0.0f; smin[k] = 0.0f; tt[k] = 0; }
         }
         const int e0 = item.e0;
         const int e1 = e0 + item.npairs;
@@ -121,7 +174,7 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                 // stage rpos and q_i.k_j of up to 64 pairs, one per lane (rows of up to 64 pairs keep
                 // what the first search staged)
                 const bool staged = pass == 1 && MODE == 2 && e1 - e0 <= WAVE;
-                __syncthreads();
+                wave_sync();
                 if (!staged && eb + lane < e1) {
                     const int e = eb + lane;
                     const int64_t j = P.edges[(size_t)P.E + e];
@@ -138,7 +191,7 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                     pair_rq[lane] = make_float4(P.rpos[(size_t)e * 3 + 0], P.rpos[(size_t)e * 3 + 1],
                                                 P.rpos[(size_t)e * 3 + 2], qk);
                 }
-                __syncthreads();
+                wave_sync();
                 const int ne = min(WAVE, e1 - eb);
                 // one candidate: pair e shifted by (vx,vy,vz), translation index t
                 // `ordered`: this lane meets its candidates in ascending (pair, translation) order,
@@ -167,26 +220,53 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                     }
                 };
                 if (nchunks == 1) {
-                    // the shifts of this lane's translations (t = lane + 64 k) stay in registers
+                    if (noisy) {
+                        if (lane < ne)
+                            phase_of[lane] = hash_uniform(pass ? seed_hi : seed_lo, pass ? seed_lo : seed_hi,
+                                                          (uint32_t)((eb + lane) * H + h), (uint32_t)pass);
+                        wave_sync();
+                    }
+                    // slab 0: the near translations, one candidate per lane and pair (ascending pairs)
                     for (int el = 0; el < ne; el++) {
                         const float4 rq = pair_rq[el];
-                        const int e = eb + el;
-                        const float phase = noisy ? hash_uniform(pass ? seed_hi : seed_lo, pass ? seed_lo : seed_hi,
-                                                                 (uint32_t)(e * H + h), (uint32_t)pass) : 0.0f;
+                        if (lane < bx.T) consider(true, rq, noisy ? phase_of[el] : 0.0f, eb + el, tt[0], sx[0], sy[0], sz[0]);
+                    }
+                    if (bx.T > WAVE) {
+                        // A candidate at distance d scores at most q.k + a d^2 + margin (the second search
+                        // only subtracts from it; margin = largest noise), and in slab k of pair (i,j)
+                        // d >= smin[k] - |r_ij|.  It can matter only if that reaches the best score so far:
+                        // smin[k] < reach = |r_ij| + sqrt((best - q.k - margin) / a), widened for rounding.
+                        const float glb = -wave_min(-best.score);
+                        const float margin = noisy ? (pass == 0 ? fabsf(a) : 1.0f) * 0.5f * P.noise : 0.0f;
+                        if (lane < ne) {
+                            const float4 rq = pair_rq[lane];
+                            const float r = sqrtf(fmaf(rq.x, rq.x, fmaf(rq.y, rq.y, rq.z * rq.z)));
+                            const float need = (glb - rq.w - margin) / a;
+                            reach[lane] = (a < 0.0f && glb > -1.0e38f)
+                                              ? (r + sqrtf(fmaxf(need, 0.0f))) * 1.0001f + 1.0e-3f : 3.0e38f;
+                        }
+                        wave_sync();
+                        const float my_reach = lane < ne ? reach[lane] : -1.0f;
 #pragma unroll
-                        for (int k = 0; k < TCAP / WAVE; k++)
+                        for (int k = 1; k < TCAP / WAVE; k++)
                             if (k * WAVE < bx.T) {
-                                const int t = lane + k * WAVE;
-                                if (t < bx.T) consider(true, rq, phase, e, t, sx[k], sy[k], sz[k]);
+                                uint64_t live = __ballot(smin[k] < my_reach);      // pairs whose slab k is scanned
+                                const bool mine = lane + k * WAVE < bx.T;
+                                while (live) {
+                                    const int el = __builtin_ctzll(live);
+                                    live &= live - 1;
+                                    const float4 rq = pair_rq[el];
+                                    if (mine) consider(false, rq, noisy ? phase_of[el] : 0.0f, eb + el, tt[k], sx[k], sy[k], sz[k]);
+                                }
                             }
                     }
                 } else {
                     for (int ch = 0; ch < nchunks; ch++) {
                         const int t0 = ch * TCAP;
                         const int cnt = min(TCAP, bx.T - t0);
-                        __syncthreads();
+                        wave_sync();
                         build_shift_table(tab, t0, cnt, bx, L, lane);
-                        __syncthreads();
+                        wave_sync();
                         for (int el = 0; el < ne; el++) {
                             const float4 rq = pair_rq[el];
                             const int e = eb + el;
@@ -205,9 +285,15 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
             if (best.e != 0x7fffffff) {
                 float sx, sy, sz;
                 shift_of(best.t, bx, L, sx, sy, sz);
-                vx = uniform_f(P.rpos[(size_t)best.e * 3 + 0]) + sx;
-                vy = uniform_f(P.rpos[(size_t)best.e * 3 + 1]) + sy;
-                vz = uniform_f(P.rpos[(size_t)best.e * 3 + 2]) + sz;
+                const int eb_last = e0 + ((e1 - e0 - 1) / WAVE) * WAVE;      // pairs still staged in LDS
+                if (best.e >= eb_last) {
+                    const float4 rq = pair_rq[best.e - eb_last];
+                    vx = rq.x + sx; vy = rq.y + sy; vz = rq.z + sz;
+                } else {
+                    vx = uniform_f(P.rpos[(size_t)best.e * 3 + 0]) + sx;
+                    vy = uniform_f(P.rpos[(size_t)best.e * 3 + 1]) + sy;
+                    vz = uniform_f(P.rpos[(size_t)best.e * 3 + 2]) + sz;
+                }
                 const float inv = 1.0f / sqrtf(vx * vx + vy * vy + vz * vz);
                 vx *= inv; vy *= inv; vz *= inv;
             }
