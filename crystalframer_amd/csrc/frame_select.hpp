@@ -107,20 +107,28 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
 #pragma unroll
         for (int c = 0; c < DH; c++) qi[c] = rec_f(rec_cur, REC_QUERY + c);
         const int nchunks = (bx.T + TCAP - 1) / TCAP;
-        // One-chunk boxes (T <= TCAP): the lane keeps the shifts of its translations in registers, slab k
-        // = positions lane + 64 k of an order that puts the 27 translations with every |n_d| <= 1 first
-        // (both groups in the reference's loop order).  The slabs k >= 1 then hold distant translations
-        // only, and a whole (pair, slab) is skipped when its nearest possible image cannot reach the
-        // best score found in slab 0 (smin = smallest shift length of the slab).
-        float sx[TCAP / WAVE], sy[TCAP / WAVE], sz[TCAP / WAVE], smin[TCAP / WAVE];
-        int tt[TCAP / WAVE];
+        // One-chunk boxes (T <= TCAP): the lane keeps the shifts of its translations in registers.  The
+        // translations with every |n_d| <= 1 (the core, at most 27) come first and are searched two pairs
+        // at a time (lanes 0-31 the even pairs of the staged row, lanes 32-63 the odd ones); the others
+        // follow in slabs of 64 (both groups in the reference's loop order).  The slabs hold distant
+        // translations only: a whole (pair, slab) is skipped when its nearest possible image cannot reach
+        // the best score found in the core (smin = smallest shift length of the slab).
+        constexpr int SLABS = TCAP / WAVE;
+        float cx = 0.f, cy = 0.f, cz = 0.f;
+        int ct = 0;
+        float sx[SLABS], sy[SLABS], sz[SLABS], smin[SLABS];
+        int tt[SLABS];
+#pragma unroll
+        for (int k = 0; k < SLABS; k++) { sx[k] = sy[k] = sz[k] = 0.0f; smin[k] = 0.0f; tt[k] = 0; }
+        int ncore = 0, nout = 0;
         if (nchunks == 1) {
             const float inv_s2 = 1.0f / (float)bx.s2, inv_s3 = 1.0f / (float)bx.s3;
-            const int ncore = min(3, 2 * bx.R1 + 1) * min(3, bx.s2) * min(3, bx.s3);
+            ncore = min(3, 2 * bx.R1 + 1) * min(3, bx.s2) * min(3, bx.s3);
+            nout = bx.T - ncore;
             int seen_core = 0, seen_out = 0;
             wave_sync();                      // the previous item's readers of perm / reach / phase are done
 #pragma unroll
-            for (int k = 0; k < TCAP / WAVE; k++)
+            for (int k = 0; k < SLABS; k++)
                 if (k * WAVE < bx.T) {
                     const int t = lane + k * WAVE;
                     int n1, n2, n3;
@@ -134,26 +142,25 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                     seen_out += __popcll(mo);
                 }
             wave_sync();
+            auto shift = [&](int t, float& vx, float& vy, float& vz) {
+                int n1, n2, n3;
+                box_coords(t, bx, inv_s2, inv_s3, n1, n2, n3);
+                const float f1 = (float)n1, f2 = (float)n2, f3 = (float)n3;
+                vx = fmaf(L.t[6], f3, fmaf(L.t[3], f2, L.t[0] * f1));
+                vy = fmaf(L.t[7], f3, fmaf(L.t[4], f2, L.t[1] * f1));
+                vz = fmaf(L.t[8], f3, fmaf(L.t[5], f2, L.t[2] * f1));
+            };
+            ct = perm[min(lane & 31, ncore - 1)];
+            shift(ct, cx, cy, cz);
 #pragma unroll
-            for (int k = 0; k < TCAP / WAVE; k++) {
-                sx[k] = sy[k] = sz[k] = 0.0f; smin[k] = 0.0f; tt[k] = 0;
-                if (k * WAVE < bx.T) {
-                    const bool valid = lane + k * WAVE < bx.T;
-                    tt[k] = perm[min(lane + k * WAVE, bx.T - 1)];
-                    int n1, n2, n3;
-                    box_coords(tt[k], bx, inv_s2, inv_s3, n1, n2, n3);
-                    const float f1 = (float)n1, f2 = (float)n2, f3 = (float)n3;
-                    sx[k] = fmaf(L.t[6], f3, fmaf(L.t[3], f2, L.t[0] * f1));
-                    sy[k] = fmaf(L.t[7], f3, fmaf(L.t[4], f2, L.t[1] * f1));
-                    sz[k] = fmaf(L.t[8], f3, fmaf(L.t[5], f2, L.t[2] * f1));
-                    if (k > 0)
-                        smin[k] = uniform_f(wave_min(valid ? sqrtf(fmaf(sx[k], sx[k], fmaf(sy[k], sy[k], sz[k] * sz[k])))
-                                                           : 3.0e38f));
+            for (int k = 0; k < SLABS; k++)
+                if (k * WAVE < nout) {
+                    const int pos = ncore + lane + k * WAVE;
+                    tt[k] = perm[min(pos, bx.T - 1)];
+                    shift(tt[k], sx[k], sy[k], sz[k]);
+                    smin[k] = uniform_f(wave_min(pos < bx.T ? sqrtf(fmaf(sx[k], sx[k], fmaf(sy[k], sy[k], sz[k] * sz[k])))
+                                                            : 3.0e38f));
                 }
-            }
-        } else {
-#pragma unroll
-            for (int k = 0; k < TCAP / WAVE; k++) { sx[k] = sy[k] = sz[k] = 0.0f; smin[k] = 0.0f; tt[k] = 0; }
         }
         const int e0 = item.e0;
         const int e1 = e0 + item.npairs;
@@ -226,12 +233,20 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                                                           (uint32_t)((eb + lane) * H + h), (uint32_t)pass);
                         wave_sync();
                     }
-                    // slab 0: the near translations, one candidate per lane and pair (ascending pairs)
-                    for (int el = 0; el < ne; el++) {
-                        const float4 rq = pair_rq[el];
-                        if (lane < bx.T) consider(true, rq, noisy ? phase_of[el] : 0.0f, eb + el, tt[0], sx[0], sy[0], sz[0]);
+                    // the core: one candidate per lane and step, two pairs per step (ascending pairs)
+                    {
+                        const int half = lane >> 5;
+                        const bool core_lane = (lane & 31) < ncore;
+#pragma unroll 2
+                        for (int m = 0; 2 * m < ne; m++) {
+                            const int el = 2 * m + half;
+                            const int elc = min(el, ne - 1);
+                            const float4 rq = pair_rq[elc];
+                            const float ph = noisy ? phase_of[elc] : 0.0f;
+                            if (core_lane && el < ne) consider(true, rq, ph, eb + el, ct, cx, cy, cz);
+                        }
                     }
-                    if (bx.T > WAVE) {
+                    if (nout > 0) {
                         // A candidate at distance d scores at most q.k + a d^2 + margin (the second search
                         // only subtracts from it; margin = largest noise), and in slab k of pair (i,j)
                         // d >= smin[k] - |r_ij|.  It can matter only if that reaches the best score so far:
@@ -248,10 +263,10 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                         wave_sync();
                         const float my_reach = lane < ne ? reach[lane] : -1.0f;
 #pragma unroll
-                        for (int k = 1; k < TCAP / WAVE; k++)
-                            if (k * WAVE < bx.T) {
+                        for (int k = 0; k < SLABS; k++)
+                            if (k * WAVE < nout) {
                                 uint64_t live = __ballot(smin[k] < my_reach);      // pairs whose slab k is scanned
-                                const bool mine = lane + k * WAVE < bx.T;
+                                const bool mine = lane + k * WAVE < nout;
                                 while (live) {
                                     const int el = __builtin_ctzll(live);
                                     live &= live - 1;
