@@ -39,6 +39,7 @@ constexpr size_t QUEUE_OFFSET = 512;           // workspace header: 256 reserved
 constexpr size_t STATS_OFFSET = 256;
 constexpr size_t COUNTER_BYTES = QUEUE_OFFSET + (size_t)MAX_HEADS * cfh::NQUEUE * cfh::QSTRIDE * sizeof(int32_t);   // whole header
 constexpr int WAVES_PER_SIMD = 3;
+constexpr int FRAME_WAVES_PER_SIMD = 8;      // the frame search keeps no per-wavefront partials: as many as are resident
 
 // workspace: header | item records (N, H, REC_WORDS) | per-wavefront weight-gradient partials
 size_t items_bytes(int64_t N, int H) {
@@ -61,10 +62,10 @@ int device_cus() {
 
 // upper bound of the persistent wavefronts of a launch (sizes the workspace): a multiple of H, no
 // more than there are items
-int launch_waves(int64_t N, int H) {
+int launch_waves(int64_t N, int H, int per_simd = WAVES_PER_SIMD) {
     int cus = device_cus();
     if (cus <= 0) cus = 256;
-    int64_t want = (int64_t)cus * 4 * WAVES_PER_SIMD;
+    int64_t want = (int64_t)cus * 4 * per_simd;
     want = (want / H) * H;
     if (want < H) want = H;
     const int64_t items = N * H;
@@ -292,7 +293,7 @@ int cfh_frame_axis1(const cfh_params* p, const float* q, const float* k, const f
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.q = q; A.k = k; A.out_frame = frame1;
-    int waves = launch_waves(N, p->num_heads);
+    int waves = launch_waves(N, p->num_heads, FRAME_WAVES_PER_SIMD);
     return launch_persistent(cfh::frame_axis_kernel<0>, A, &waves, (hipStream_t)stream, "frame_axis1");
 }
 
@@ -310,7 +311,7 @@ int cfh_frame_axis2(const cfh_params* p, const float* q, const float* k, const f
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.q = q; A.k = k; A.frame1 = frame1; A.out_frame = frame2max;
-    int waves = launch_waves(N, p->num_heads);
+    int waves = launch_waves(N, p->num_heads, FRAME_WAVES_PER_SIMD);
     return launch_persistent(cfh::frame_axis_kernel<1>, A, &waves, (hipStream_t)stream, "frame_axis2");
 }
 
@@ -328,7 +329,7 @@ int cfh_frame_axes(const cfh_params* p, const float* q, const float* k, const fl
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     A.q = q; A.k = k; A.out_frame = frames;
-    int waves = launch_waves(N, p->num_heads);
+    int waves = launch_waves(N, p->num_heads, FRAME_WAVES_PER_SIMD);
     return launch_persistent(cfh::frame_axis_kernel<2>, A, &waves, (hipStream_t)stream, "frame_axes");
 }
 

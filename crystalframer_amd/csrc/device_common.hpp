@@ -56,6 +56,39 @@ __device__ __forceinline__ float row_sum(float x) {
     return x;
 }
 
+// ---- compaction of flagged translations into the survivor list ------------------------------------
+// Lane (slot, tl) flags in `bits` which of its translations tl + 16 k (k = 0..7) of pair `slot` of the
+// round survive.  The flagged ones of the whole wavefront get consecutive positions (rows in order,
+// lanes of a row in order, a lane's own in ascending k): position - skip is where the entry goes in
+// list[nlist ...), entries before `skip` (already processed) or beyond `room` are left out.  One row
+// scan in DPP, four lane reads and a short loop over the largest number of flags of any lane replace
+// a ballot / prefix / branch per k.  `code` = pair-in-group << shift | tl.  Returns the number of
+// flagged entries of the wavefront.
+template <int CTRL>
+__device__ __forceinline__ int dpp_movei(int x) { return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xf, 0xf, false); }
+__device__ __forceinline__ int append_flagged(uint16_t* list, int nlist, int room, int skip, uint32_t bits,
+                                              int slot, uint32_t code) {
+    const int own = __popc(bits);
+    int x = own;                                  // inclusive prefix within the 16-lane row (row_shr 1, 2, 4, 8)
+    x += dpp_movei<0x111>(x);
+    x += dpp_movei<0x112>(x);
+    x += dpp_movei<0x114>(x);
+    x += dpp_movei<0x118>(x);
+    const int t0 = __builtin_amdgcn_readlane(x, 15), t1 = __builtin_amdgcn_readlane(x, 31);
+    const int t2 = __builtin_amdgcn_readlane(x, 47), t3 = __builtin_amdgcn_readlane(x, 63);
+    const int base = slot == 0 ? 0 : slot == 1 ? t0 : slot == 2 ? t0 + t1 : t0 + t1 + t2;
+    int pos = base + x - own - skip;
+    while (__ballot(bits != 0u)) {
+        if (bits != 0u) {
+            const int k = __builtin_ctz(bits);
+            bits &= bits - 1u;
+            if (pos >= 0 && pos < room) list[nlist + pos] = (uint16_t)(code + 16u * (uint32_t)k);
+            pos++;
+        }
+    }
+    return t0 + t1 + t2 + t3;
+}
+
 // ---- reductions over the four rows of a wavefront (same column), gfx950 lane swaps ---------------
 // v_permlane32_swap exchanges the upper half of one register with the lower half of another,
 // v_permlane16_swap the odd rows of one with the even rows of another: applied to two copies of x

@@ -89,9 +89,16 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                 for (int d = 0; d < 3; d++) f[ax][d] = rec_f(rec_cur, REC_FRAMES + ax * 3 + d);
         }
         const int nchunks = (bx.T + FWD_TCAP - 1) / FWD_TCAP;
+        // boxes of up to 128 translations with a < 0: one slab of 8 per lane, distances stay in
+        // registers between the passes; the table is padded with infinitely distant shifts, whose weight
+        // 2^(a d^2) is exactly zero, so that the slab needs no bounds checks
+        const bool fast = bx.T <= 16 * FAST_PER_LANE && a2 < 0.0f;
         if (nchunks == 1) {
             wave_sync();
             build_shift_table(tab, 0, bx.T, bx, L, lane);
+            if (fast)
+                for (int u = bx.T + lane; u < 16 * FAST_PER_LANE; u += WAVE)
+                    tab[u] = make_float4(__builtin_inff(), 0.0f, 0.0f, 0.0f);
             wave_sync();
         }
         const int e0 = item.e0;
@@ -210,7 +217,6 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
         int cur_g0 = -1, cur_ng = 0;
         int el_glob = 0, ch = 0;
         int skip = 0;          // survivors of the current round already processed (list overflow)
-        const bool fast = bx.T <= 16 * FAST_PER_LANE;      // one slab: distances stay in registers
         float d2r[FAST_PER_LANE];
 #pragma unroll
         for (int k = 0; k < FAST_PER_LANE; k++) d2r[k] = 0.0f;
@@ -244,10 +250,9 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                     // every lane keeps the squared distances of its 8 translations for pass B
 #pragma unroll
                     for (int k = 0; k < FAST_PER_LANE; k++) {
-                        const int u = tl + 16 * k;
-                        const float4 v = tab[u];      // beyond T: stale words, masked by the select
+                        const float4 v = tab[tl + 16 * k];
                         const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
-                        d2r[k] = (u < bx.T) ? fmaf(dx, dx, fmaf(dy, dy, dz * dz)) : 3.0e38f;
+                        d2r[k] = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
                         d2min = fminf(d2min, d2r[k]);
                     }
                 } else {
@@ -303,18 +308,15 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                 const int room = FWD_LISTCAP - nlist;
                 int seen = 0;                      // survivors met so far in this round
                 if (fast) {
+                    uint32_t bits = 0u;
 #pragma unroll
                     for (int k = 0; k < FAST_PER_LANE; k++) {
-                        const int u = tl + 16 * k;
-                        const bool valid = active && u < cnt;
-                        const float ex = a2 * (d2r[k] - d2min);
-                        Sb += valid ? hw_exp2(ex) : 0.0f;
-                        const bool keep = valid && ex >= prune;
-                        const uint64_t m = __ballot(keep);
-                        const int pos = seen + lane_prefix(m) - skip;     // slot after those already done
-                        if (keep && pos >= 0 && pos < room) list[nlist + pos] = (uint16_t)((el << FWD_SHIFT) | u);
-                        seen += __popcll(m);
+                        const float ex = a2 * (d2r[k] - d2min);          // -inf for the padding
+                        Sb += hw_exp2(ex);
+                        bits |= (ex >= prune) ? (1u << k) : 0u;
                     }
+                    if (!active) bits = 0u;
+                    seen = append_flagged(list, nlist, room, skip, bits, slot, (uint32_t)((el << FWD_SHIFT) | tl));
                 } else {
                     for (int u0 = 0; u0 < cnt; u0 += 16) {
                         const int u = u0 + tl;
