@@ -46,11 +46,18 @@ class CfhParams(ctypes.Structure):
     ]
 
 
+class CfhLinearGradJob(ctypes.Structure):
+    """Mirror of ``cfh_linear_grad_job`` in include/crystalframer_hip.h."""
+    _fields_ = [("x", ctypes.c_void_p), ("dy", ctypes.c_void_p), ("dW", ctypes.c_void_p), ("db", ctypes.c_void_p),
+                ("N", ctypes.c_int64), ("I", ctypes.c_int64), ("O", ctypes.c_int64), ("ldx", ctypes.c_int64),
+                ("ldy", ctypes.c_int64)]
+
+
 EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_frame_axis1",
            "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_backward",
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
            "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
-           "cfh_linear_weight_bias_grad", "cfh_attention_inputs_forward",
+           "cfh_linear_weight_bias_grad", "cfh_linear_weight_bias_grad_batch", "cfh_attention_inputs_forward",
            "cfh_attention_inputs_backward")
 
 _lib = None
@@ -102,6 +109,8 @@ def load():
         lib.cfh_crystal_mean_backward.argtypes = [_P, _P, _P, _I64, _I64, _I64, _P, _P]
         lib.cfh_linear_weight_bias_grad.restype = ctypes.c_int
         lib.cfh_linear_weight_bias_grad.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P, _P]
+        lib.cfh_linear_weight_bias_grad_batch.restype = ctypes.c_int
+        lib.cfh_linear_weight_bias_grad_batch.argtypes = [ctypes.POINTER(CfhLinearGradJob), ctypes.c_int32, _P]
         _F, _I32 = ctypes.c_float, ctypes.c_int32
         lib.cfh_attention_inputs_forward.restype = ctypes.c_int
         lib.cfh_attention_inputs_forward.argtypes = [_P, _P, _P, _F, _F, _F, _F, _I64, _I32, _I32, _P, _P, _P, _P, _P]

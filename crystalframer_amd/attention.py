@@ -148,6 +148,7 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
                 if params.value_pe_angle_real > 0 else None
             setattr(self, f"proj_angle{n}", w)
         self._gauss_ready = None      # host-side cache of "gauss_scale[0] > 0"
+        self._in_proj_stack = None    # the storage q/k/v_proj_weight share once they are adjacent
         self.frame_sink = None        # a list: every forward appends its (f1, f2, f3) (diagnostics)
         self._reset_parameters()
 
@@ -178,6 +179,27 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
     def _load_from_state_dict(self, *args, **kwargs):
         self._gauss_ready = None
         return super()._load_from_state_dict(*args, **kwargs)
+
+    def _stacked_in_proj(self) -> Tensor:
+        """The three input-projection weights as one (2 kdim + vdim, E) matrix without a copy per step:
+        the parameters live as adjacent row blocks of one storage.  Re-established here whenever
+        something gave them storages of their own (``.to(device)``, ``load_state_dict(assign=True)``);
+        values, names and shapes of the parameters do not change."""
+        q, k, v = self.q_proj_weight, self.k_proj_weight, self.v_proj_weight
+        st = self._in_proj_stack
+        es = q.element_size()
+        adjacent = (st is not None and st.device == q.device and st.dtype == q.dtype
+                    and q.data_ptr() == st.data_ptr() and k.data_ptr() == q.data_ptr() + q.numel() * es
+                    and v.data_ptr() == k.data_ptr() + k.numel() * es
+                    and q.is_contiguous() and k.is_contiguous() and v.is_contiguous())
+        if not adjacent:
+            with torch.no_grad():
+                st = torch.cat([q.data, k.data, v.data], dim=0)
+                q.data = st[:q.shape[0]]
+                k.data = st[q.shape[0]:q.shape[0] + k.shape[0]]
+                v.data = st[q.shape[0] + k.shape[0]:]
+            self._in_proj_stack = st
+        return st
 
     def _gauss_constants(self):
         """(c1, lb, c2) of a = ((1 - lb) elu(c1 alpha') + 1) c2."""
@@ -235,8 +257,8 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
             # self-attention: the three projections as one GEMM over the stacked weights (same
             # arithmetic per output element; forward, input gradient and weight gradient each
             # become one launch instead of three)
-            w_in = torch.cat([self.q_proj_weight, self.k_proj_weight, self.v_proj_weight], dim=0)
-            qkv = cuda_funcs.linear(query, w_in, self.in_proj_bias)
+            qkv = cuda_funcs.linear(query, (self.q_proj_weight, self.k_proj_weight, self.v_proj_weight),
+                                    self.in_proj_bias, stacked=self._stacked_in_proj())
             fused = (FUSED_INPUTS and self.kdim == self.vdim == H * Dh
                      and cuda_funcs.AttentionInputsHIP.supported(H, Dh)
                      and (not self.params.normalize_gauss or self._gauss_scale_ready()))

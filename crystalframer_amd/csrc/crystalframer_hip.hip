@@ -600,5 +600,49 @@ int cfh_attention_inputs_backward(const float* qkv, const float* lattice_w, cons
     return finish_launch("attention_inputs_backward");
 }
 
+int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t njobs, void* stream) {
+    if (njobs < 0 || (njobs > 0 && !jobs)) return fail(CFH_EINVAL, "jobs is NULL or njobs negative");
+    for (int32_t j = 0; j < njobs; j++) {
+        const cfh_linear_grad_job& J = jobs[j];
+        if (J.N < 0 || J.I < 1 || J.O < 1 || J.N > 0x7fffffffLL / 64 || J.I > 65536 || J.O > 65536 || J.ldx < J.I ||
+            J.ldy < J.O || J.ldx > 0x7fffffffLL || J.ldy > 0x7fffffffLL)
+            return fail(CFH_EINVAL, "job %d: sizes N=%lld I=%lld O=%lld ldx=%lld ldy=%lld out of range", (int)j,
+                        (long long)J.N, (long long)J.I, (long long)J.O, (long long)J.ldx, (long long)J.ldy);
+        if (!J.dW || (J.N > 0 && (!J.x || !J.dy))) return fail(CFH_EINVAL, "job %d: x, dy and dW must not be NULL", (int)j);
+    }
+    hipStream_t st = (hipStream_t)stream;
+    for (int32_t first = 0; first < njobs; first += cfh::WGRAD_MAX_JOBS) {
+        const int32_t last = njobs < first + cfh::WGRAD_MAX_JOBS ? njobs : first + cfh::WGRAD_MAX_JOBS;
+        long tiles = 0;
+        for (int32_t j = first; j < last; j++)
+            if (jobs[j].N > 0) tiles += (long)((jobs[j].I + 63) / 64) * (long)((jobs[j].O + 63) / 64);
+        if (tiles == 0) continue;
+        const int want = (int)((2048 + tiles - 1) / tiles);        // slices of a job: about 2048 workgroups in all
+        cfh::WgradJobs T{};
+        int blocks = 0;
+        for (int32_t j = first; j < last; j++) {
+            const cfh_linear_grad_job& J = jobs[j];
+            if (J.N == 0) continue;
+            cfh::WgradJob& W = T.job[T.njobs++];
+            W.x = J.x; W.dy = J.dy; W.dW = J.dW; W.db = J.db;
+            W.N = (int)J.N; W.I = (int)J.I; W.O = (int)J.O; W.ldx = (int)J.ldx; W.ldy = (int)J.ldy;
+            W.bx = (int)((J.I + 63) / 64); W.by = (int)((J.O + 63) / 64);
+            int slices = want;
+            const int max_slices = (int)((J.N + 31) / 32);
+            if (slices > max_slices) slices = max_slices;
+            if (slices < 1) slices = 1;
+            int rows = (int)((J.N + slices - 1) / slices);
+            rows = (rows + 3) & ~3;
+            slices = (int)((J.N + rows - 1) / rows);
+            W.rows_per_slice = rows;
+            W.block0 = blocks;
+            blocks += W.bx * W.by * slices;
+        }
+        hipLaunchKernelGGL(cfh::linear_wgrad_batch_kernel, dim3(blocks), dim3(256), 0, st, T);
+    }
+    return finish_launch("linear_weight_bias_grad_batch");
+}
+
 }  // extern "C"
+
 

@@ -13,16 +13,17 @@ namespace cfh {
 
 typedef float v4f_l __attribute__((ext_vector_type(4)));
 
-// grid: (ceil(I/64), ceil(O/64), slices), block: 256 threads = 4 wavefronts, wavefront w of a block
-// owns the 32x32 block (o0 + 32 (w/2), i0 + 32 (w%2)).
-__global__ __launch_bounds__(256) void linear_wgrad_kernel(const float* __restrict__ x, const float* __restrict__ dy,
-                                                           int N, int I, int O, int rows_per_slice,
-                                                           float* dW, float* db) {
+// One workgroup's share: 256 threads = 4 wavefronts, wavefront w owns the 32x32 block
+// (64 ty + 32 (w/2), 64 tx + 32 (w%2)) of dW and the rows [slice rows_per_slice, ...) of x and dy
+// (row strides ldx, ldy: dy may be a column slice of a wider matrix).
+__device__ __forceinline__ void wgrad_block(const float* __restrict__ x, const float* __restrict__ dy, int N, int I,
+                                            int O, int ldx, int ldy, int rows_per_slice, int tx, int ty, int slice,
+                                            float* dW, float* db) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int o0 = blockIdx.y * 64 + 32 * (w >> 1);
-    const int i0 = blockIdx.x * 64 + 32 * (w & 1);
+    const int o0 = ty * 64 + 32 * (w >> 1);
+    const int i0 = tx * 64 + 32 * (w & 1);
     if (o0 >= O || i0 >= I) return;
-    const int r0 = blockIdx.z * rows_per_slice;
+    const int r0 = slice * rows_per_slice;
     const int r1 = min(N, r0 + rows_per_slice);
     const int col = lane & 15, kk = lane >> 4;
     const int oa = o0 + col, ob = o0 + 16 + col;          // columns of dY this lane feeds (A operand)
@@ -33,10 +34,10 @@ __global__ __launch_bounds__(256) void linear_wgrad_kernel(const float* __restri
 #pragma unroll 4
     for (int r = r0 + kk; r < r1 + kk; r += 4) {          // every lane group takes the same number of steps
         const bool vr = r < r1;
-        const float ya = (vr && voa) ? dy[(size_t)r * O + oa] : 0.f;
-        const float yb = (vr && vob) ? dy[(size_t)r * O + ob] : 0.f;
-        const float xa = (vr && via) ? x[(size_t)r * I + ia] : 0.f;
-        const float xb = (vr && vib) ? x[(size_t)r * I + ib] : 0.f;
+        const float ya = (vr && voa) ? dy[(size_t)r * ldy + oa] : 0.f;
+        const float yb = (vr && vob) ? dy[(size_t)r * ldy + ob] : 0.f;
+        const float xa = (vr && via) ? x[(size_t)r * ldx + ia] : 0.f;
+        const float xb = (vr && vib) ? x[(size_t)r * ldx + ib] : 0.f;
         acc00 = __builtin_amdgcn_mfma_f32_16x16x4f32(ya, xa, acc00, 0, 0, 0);
         acc01 = __builtin_amdgcn_mfma_f32_16x16x4f32(ya, xb, acc01, 0, 0, 0);
         acc10 = __builtin_amdgcn_mfma_f32_16x16x4f32(yb, xa, acc10, 0, 0, 0);
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(256) void linear_wgrad_kernel(const float* __restri
             if (vib) atomicAdd(dW + (size_t)(o0 + 16 + oo) * I + ib, acc11[c]);
         }
     }
-    if (db && blockIdx.x == 0 && (w & 1) == 0) {          // one column of blocks sums dY over its rows
+    if (db && tx == 0 && (w & 1) == 0) {                  // one column of blocks sums dY over its rows
         bsum_a = rows_sum(bsum_a);
         bsum_b = rows_sum(bsum_b);
         if (kk == 0) {
@@ -64,6 +65,34 @@ __global__ __launch_bounds__(256) void linear_wgrad_kernel(const float* __restri
             if (vob) atomicAdd(db + ob, bsum_b);
         }
     }
+}
+
+// grid: (ceil(I/64), ceil(O/64), slices), block: 256 threads
+__global__ __launch_bounds__(256) void linear_wgrad_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+                                                           int N, int I, int O, int rows_per_slice,
+                                                           float* dW, float* db) {
+    wgrad_block(x, dy, N, I, O, I, O, rows_per_slice, blockIdx.x, blockIdx.y, blockIdx.z, dW, db);
+}
+
+// Several layers' gradients in one launch: the jobs travel in the kernel arguments, workgroup b
+// belongs to the job with block0 <= b < block0 + bx by slices.
+constexpr int WGRAD_MAX_JOBS = 24;
+struct WgradJob {
+    const float* x; const float* dy; float* dW; float* db;
+    int N, I, O, ldx, ldy;
+    int block0, bx, by, rows_per_slice;
+};
+struct WgradJobs { WgradJob job[WGRAD_MAX_JOBS]; int njobs; };
+
+__global__ __launch_bounds__(256) void linear_wgrad_batch_kernel(const WgradJobs T) {
+    int j = 0;
+    for (int t = 1; t < T.njobs; t++)
+        if ((int)blockIdx.x >= T.job[t].block0) j = t;
+    const WgradJob& J = T.job[j];
+    const int b = (int)blockIdx.x - J.block0;
+    const int tiles = J.bx * J.by;
+    const int slice = b / tiles, tile = b - slice * tiles;
+    wgrad_block(J.x, J.dy, J.N, J.I, J.O, J.ldx, J.ldy, J.rows_per_slice, tile % J.bx, tile / J.bx, slice, J.dW, J.db);
 }
 
 __global__ __launch_bounds__(256) void zero2_kernel(float* a, int na, float* b, int nb) {

@@ -41,6 +41,9 @@ class KernelManager:
     # pass, which then gathers only: about a third less backward time for 244 MB per layer at batch 256
     SAVE_HISTOGRAMS: bool = True
     GRAD_COEF_QUIRK: bool = False
+    # weight / bias gradients of the linear layers (leaf parameters): all layers of a backward pass in
+    # one launch when the pass ends, instead of one launch per layer as the gradient is reached
+    DEFER_WEIGHT_GRADS: bool = True
     COLLECT_STATS: bool = False         # count translations (read with _lib.read_stats)
     EVENT_LOG = None                    # a list: every library call appends (name, start, end) events
     _compiled_for = None
@@ -475,37 +478,174 @@ class IrregularMeanCUDA(torch.autograd.Function):
         return gx.to(ctx.in_dtype), None, None
 
 
-class LinearHIP(torch.autograd.Function):
-    """y = x W^T + b with the weight and bias gradients from one launch of the library
-    (cfh_linear_weight_bias_grad); forward and input gradient are the framework's GEMMs.
-    Same values as torch.nn.functional.linear up to the order of the float32 sums."""
+class _DeferredWeightGrads:
+    """Weight and bias gradients of the linear layers of ONE backward pass, computed together.
+
+    LinearHIP.backward hands autograd zero-filled gradient tensors (views of one arena that is cleared
+    by a single fill) and records what has to be added to them; when the pass ends (a callback of the
+    autograd engine) one call of cfh_linear_weight_bias_grad_batch adds x^T dy of every layer.  The
+    gradients are complete when ``backward()`` / ``autograd.grad()`` return.  Only parameters that are
+    leaves take part: nothing else reads their gradient before the pass ends.  If a parameter already
+    had a ``.grad`` (accumulation over several passes), autograd has added the zeros to it at once and
+    the batch call adds into that ``.grad`` instead."""
+    ARENA_FLOATS = 1 << 21
+    pending = []            # (x2, gy2, col0, O, dW_view, db_view, weight, bias, whole bias-gradient view, marks)
+    arena = None
+    arena_off = 0
+    callback_queued = False
+    task_id = -1            # autograd graph task the pending work belongs to
+
+    @classmethod
+    def take(cls, n: int, device) -> torch.Tensor:
+        n_al = (n + 63) & ~63
+        if cls.arena is None or cls.arena.device != device or cls.arena_off + n_al > cls.arena.numel():
+            cls.arena = torch.zeros(max(cls.ARENA_FLOATS, n_al), dtype=torch.float32, device=device)
+            cls.arena_off = 0
+        v = cls.arena[cls.arena_off:cls.arena_off + n]
+        cls.arena_off += n_al
+        return v
 
     @staticmethod
-    def forward(ctx, x, weight, bias):
-        ctx.save_for_backward(x, weight)
-        ctx.has_bias = bias is not None
-        return torch.nn.functional.linear(x, weight, bias)
+    def mark(param):
+        """Identity and version of a parameter's .grad: changes when autograd sets or adds to it."""
+        g = param.grad
+        return None if g is None else (id(g), g._version)
+
+    @classmethod
+    def reset(cls):
+        cls.pending = []
+        cls.arena = None
+        cls.arena_off = 0
+        cls.callback_queued = False
+
+    @classmethod
+    def flush(cls):
+        pending, cls.pending = cls.pending, []
+        cls.arena = None
+        cls.arena_off = 0
+        cls.callback_queued = False
+        if not pending:
+            return
+        lib = _lib.load()
+        dev = pending[0][0].device
+        jobs = (_lib.CfhLinearGradJob * len(pending))()
+        fixups = []
+        for n, (x2, g2, col0, O, dW, db, weight, bias, first, w_mark, b_mark) in enumerate(pending):
+            dst_w, dst_b = dW, db
+            wg = weight.grad
+            if wg is not None and cls.mark(weight) != w_mark and wg.data_ptr() != dW.data_ptr():
+                # .grad was set or updated during this pass, but not by adopting our tensor: autograd
+                # copied or accumulated it (adding our zeros), so the result belongs into .grad
+                if wg.dtype == torch.float32 and wg.is_contiguous() and wg.device == dev:
+                    dst_w = wg
+                else:
+                    fixups.append((wg, dW))
+            if db is not None:
+                bg = bias.grad
+                if bg is not None and cls.mark(bias) != b_mark and bg.data_ptr() != first.data_ptr():
+                    if bg.dtype == torch.float32 and bg.is_contiguous() and bg.device == dev:
+                        dst_b = bg[col0:col0 + O]
+                    elif col0 == 0:
+                        fixups.append((bg, first))
+            J = jobs[n]
+            J.x, J.dy = x2.data_ptr(), g2.data_ptr() + 4 * col0
+            J.dW, J.db = dst_w.data_ptr(), (dst_b.data_ptr() if dst_b is not None else None)
+            J.N, J.I, J.O, J.ldx, J.ldy = x2.shape[0], x2.shape[1], O, x2.stride(0), g2.stride(0)
+        with torch.cuda.device(dev), _timed("linear_weight_bias_grad_batch", dev):
+            rc = lib.cfh_linear_weight_bias_grad_batch(jobs, len(pending), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
+        for grad, part in fixups:
+            grad.add_(part.to(grad.dtype))
+
+
+class LinearHIP(torch.autograd.Function):
+    """y = x W^T + b, W the row-wise stack of ``weights`` (``stacked``: a tensor that already holds
+    that stack, e.g. an alias of the parameters' shared storage; None: concatenated here).  Forward and
+    input gradient are the framework's GEMMs; the weight and bias gradients come from the library: for
+    leaf parameters deferred to one launch per backward pass (see _DeferredWeightGrads), otherwise
+    one launch here.  Same values as torch.nn.functional.linear up to the order of the float32 sums."""
+
+    @staticmethod
+    def forward(ctx, x, bias, stacked, *weights):
+        if stacked is not None:
+            W = stacked
+        elif len(weights) == 1:
+            W = weights[0]
+        else:
+            W = torch.cat(weights, dim=0)
+        ctx.save_for_backward(x, W.detach())
+        ctx.weights = weights
+        ctx.bias = bias
+        return torch.nn.functional.linear(x, W.detach(), None if bias is None else bias.detach())
 
     @staticmethod
     def backward(ctx, gy):
-        x, weight = ctx.saved_tensors
-        gx = gw = gb = None
-        if ctx.needs_input_grad[0]:
-            gx = gy.matmul(weight)
-        if ctx.needs_input_grad[1] or (ctx.has_bias and ctx.needs_input_grad[2]):
+        x, W = ctx.saved_tensors
+        weights, bias = ctx.weights, ctx.bias
+        gx = gy.matmul(W) if ctx.needs_input_grad[0] else None
+        need_w = [ctx.needs_input_grad[3 + n] for n in range(len(weights))]
+        need_b = bias is not None and ctx.needs_input_grad[1]
+        if not (any(need_w) or need_b):
+            return (gx, None, None) + (None,) * len(weights)
+        dev = x.device
+        I = W.shape[1]
+        x2 = _f32c(x.reshape(-1, I))
+        g2 = _f32c(gy.reshape(-1, W.shape[0]))
+        D = _DeferredWeightGrads
+        if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
+            D.reset()                               # left over from a backward pass that raised
+        defer = (KernelManager.DEFER_WEIGHT_GRADS and all(w.is_leaf for w in weights)
+                 and (bias is None or bias.is_leaf) and all(w.dtype == torch.float32 for w in weights))
+        if defer:
+            take = lambda n: D.take(n, dev)
+        else:
+            total = sum(w.numel() for w in weights) + (W.shape[0] if bias is not None else 0)
+            buf = torch.zeros(total, dtype=torch.float32, device=dev)
+            state = [0]
+
+            def take(n):
+                v = buf[state[0]:state[0] + n]
+                state[0] += n
+                return v
+        gb = take(W.shape[0]) if bias is not None else None
+        gws, jobs, col0 = [], [], 0
+        for w in weights:
+            O = w.shape[0]
+            dW = take(O * I).view(O, I)
+            gws.append(dW)
+            jobs.append((x2, g2, col0, O, dW, gb[col0:col0 + O] if gb is not None else None, w, bias, gb,
+                         D.mark(w) if defer else None, D.mark(bias) if defer and bias is not None else None))
+            col0 += O
+        if defer:
+            D.pending.extend(jobs)
+            if not D.callback_queued:
+                torch.autograd.Variable._execution_engine.queue_callback(D.flush)
+                D.callback_queued = True
+                D.task_id = torch._C._current_graph_task_id()
+        else:
             lib = _lib.load()
-            O, I = weight.shape
-            x2 = _f32c(x.reshape(-1, I))
-            g2 = _f32c(gy.reshape(-1, O))
-            gw32 = torch.empty((O, I), dtype=torch.float32, device=x.device)
-            gb32 = torch.empty((O,), dtype=torch.float32, device=x.device) if ctx.has_bias else None
-            with _timed("linear_weight_bias_grad", x.device):
-                rc = lib.cfh_linear_weight_bias_grad(_lib.ptr(x2), _lib.ptr(g2), x2.shape[0], I, O, _lib.ptr(gw32),
-                                                     _lib.ptr(gb32), _lib.current_stream_ptr(x.device))
-            _lib.check(rc, "cfh_linear_weight_bias_grad")
-            gw = gw32.to(weight.dtype)
-            gb = gb32.to(weight.dtype) if ctx.has_bias else None
-        return gx, gw, gb
+            arr = (_lib.CfhLinearGradJob * len(jobs))()
+            for n, (x2_, g2_, c0, O, dW, db, *_) in enumerate(jobs):
+                J = arr[n]
+                J.x, J.dy = x2_.data_ptr(), g2_.data_ptr() + 4 * c0
+                J.dW, J.db = dW.data_ptr(), (db.data_ptr() if db is not None else None)
+                J.N, J.I, J.O, J.ldx, J.ldy = x2_.shape[0], I, O, x2_.stride(0), g2_.stride(0)
+            with torch.cuda.device(dev), _timed("linear_weight_bias_grad", dev):
+                rc = lib.cfh_linear_weight_bias_grad_batch(arr, len(jobs), _lib.current_stream_ptr(dev))
+            _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
+        gws = [g.to(w.dtype) if g.dtype != w.dtype else g for g, w in zip(gws, weights)]
+        gb_out = None if gb is None else (gb if gb.dtype == bias.dtype else gb.to(bias.dtype))
+        return (gx, gb_out, None) + tuple(gws)
+
+
+def linear(x: torch.Tensor, weight, bias: Optional[torch.Tensor] = None,
+           stacked: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """torch.nn.functional.linear for device tensors with the library's weight-gradient kernel.
+    ``weight``: a tensor (O,I), or a sequence of tensors (O_k,I) whose row-wise stack is the weight
+    (``stacked``: that stack if it already exists in memory)."""
+    weights = (weight,) if isinstance(weight, torch.Tensor) else tuple(weight)
+    _lib.require_gpu(x, *weights)
+    return LinearHIP.apply(x, bias, stacked, *weights)
 
 
 class AttentionInputsHIP(torch.autograd.Function):
@@ -560,8 +700,3 @@ class AttentionInputsHIP(torch.autograd.Function):
         _lib.check(rc, "cfh_attention_inputs_backward")
         return gqkv, gw, None, None, None, None, None, None
 
-
-def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """torch.nn.functional.linear for device tensors, with the library's weight-gradient kernel."""
-    _lib.require_gpu(x, weight)
-    return LinearHIP.apply(x, weight, bias)

@@ -242,6 +242,25 @@ int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int6
                                 float* dW, float* db, void* stream);
 
 /*
+ * The same gradients for several layers in one launch, ACCUMULATED into dW and db (the caller has
+ * initialised them: zeros, or gradients to add to).  Each job: x (N,I) with row stride ldx, dy (N,O)
+ * with row stride ldy (so a job may take a column block of a wider dy, e.g. one of the three
+ * stacked input projections), dW (O,I) contiguous, db (O) or NULL.  `jobs` is a host array; it is
+ * copied into the kernel arguments, 24 jobs per launch.  Deferring the weight gradients of a whole
+ * backward pass to one call replaces one launch (plus clearing) per layer -- latency-bound at these
+ * sizes -- by a launch that fills the chip.  No counterpart in the reference (autograd of
+ * torch.nn.functional.linear, one GEMM per layer).
+ */
+typedef struct cfh_linear_grad_job {
+    const float* x;
+    const float* dy;
+    float* dW;
+    float* db;
+    int64_t N, I, O, ldx, ldy;
+} cfh_linear_grad_job;
+int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t njobs, void* stream);
+
+/*
  * What lies between the stacked q/k/v projection of a layer and its kernels, one launch each way.
  * Forward: qkv (N, 3 H Dh), rows = [query | key | value];  qs = query * q_scale, k, v (N,H,Dh) contiguous,
  *   a (N,H) = ((1 - lb) elu(c1 alpha') + 1) c2  with alpha = query_h . lattice_w_h and

@@ -232,3 +232,58 @@ def test_attention_inputs_split_scale_and_gaussian_coefficient(N, H, normalised)
     (outs[2] * f32(g[2])).sum().backward()
     expect = torch.cat([torch.zeros(N, 2 * H * Dh, dtype=torch.float64), g[2].reshape(N, -1)], dim=1)
     assert Hh.rel_err(qkv.grad, expect) < 1e-6
+
+
+def test_linear_deferred_gradients_stacked_accumulated_and_nonleaf():
+    """The deferred weight-gradient launch: several layers in one backward pass (one of them with three
+    stacked weights sharing a bias), a second pass accumulating into existing .grad, a weight that is
+    not a leaf (gradient needed before the pass ends), and torch.autograd.grad instead of backward."""
+    import crystalframer_amd as cf
+    lin = cf.cuda_funcs.linear
+    gen = torch.Generator().manual_seed(9)
+    N = 301
+    mk = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    x64 = mk(N, 48).requires_grad_(True)
+    ws64 = [mk(32, 48).requires_grad_(True), mk(16, 48).requires_grad_(True), mk(64, 48).requires_grad_(True)]
+    b64 = mk(112).requires_grad_(True)
+    w2_64 = mk(40, 112).requires_grad_(True)
+    b2_64 = mk(40).requires_grad_(True)
+    scale64 = torch.tensor(0.7, dtype=torch.float64, requires_grad=True)
+    leaves64 = [x64, *ws64, b64, w2_64, b2_64, scale64]
+
+    def net(x, ws, b, w2, b2, scale, linear, cat):
+        h = torch.tanh(linear(x, cat(ws), b))
+        h = linear(h, w2 * scale, b2)              # a weight that is not a leaf
+        return h.square().sum()
+
+    ref = net(x64, ws64, b64, w2_64, b2_64, scale64, torch.nn.functional.linear, lambda ws: torch.cat(ws, 0))
+    ref.backward()
+    leaves = [f32(t.detach()).requires_grad_(True) for t in leaves64]
+    x, w0, w1, w2s, b, w2, b2, scale = leaves
+
+    def run():
+        return net(x, [w0, w1, w2s], b, w2, b2, scale, lambda xx, ww, bb: lin(xx, ww, bb), lambda ws: tuple(ws))
+
+    run().backward()
+    for t32, t64 in zip(leaves, leaves64):
+        assert Hh.rel_err(t32.grad, t64.grad) < 2e-5
+    # second pass: gradients accumulate into the existing .grad tensors
+    run().backward()
+    for t32, t64 in zip(leaves, leaves64):
+        assert Hh.rel_err(t32.grad, 2 * t64.grad) < 2e-5
+    # autograd.grad returns complete gradients and leaves .grad alone
+    before = w0.grad.clone()
+    g = torch.autograd.grad(run(), [w0, b, w2])
+    assert Hh.rel_err(g[0], ws64[0].grad) < 2e-5 and Hh.rel_err(g[1], b64.grad) < 2e-5 and Hh.rel_err(g[2], w2_64.grad) < 2e-5
+    assert torch.equal(w0.grad, before)
+    # deferral switched off gives the same numbers
+    KM = cf.KernelManager
+    KM.DEFER_WEIGHT_GRADS = False
+    try:
+        for t in leaves:
+            t.grad = None
+        run().backward()
+    finally:
+        KM.DEFER_WEIGHT_GRADS = True
+    for t32, t64 in zip(leaves, leaves64):
+        assert Hh.rel_err(t32.grad, t64.grad) < 2e-5
