@@ -116,7 +116,7 @@ def load():
         lib.cfh_attention_inputs_forward.argtypes = [_P, _P, _P, _F, _F, _F, _F, _I64, _I32, _I32, _P, _P, _P, _P, _P]
         lib.cfh_attention_inputs_backward.restype = ctypes.c_int
         lib.cfh_attention_inputs_backward.argtypes = [_P, _P, _P, _F, _F, _F, _F, _P, _P, _P, _P, _I64, _I32, _I32,
-                                                      _P, _P, _P]
+                                                      _P, _P, _P, ctypes.c_size_t, _P]
         lib.cfh_timing_enable.restype = ctypes.c_int
         lib.cfh_timing_enable.argtypes = [ctypes.c_int]
         lib.cfh_timing_read.restype = ctypes.c_int

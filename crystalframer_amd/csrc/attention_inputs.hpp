@@ -23,8 +23,9 @@ struct AttnInArgs {
     float* k;
     float* v;
     float* a;
-    float* gqkv;               // backward outputs: (N, 3 HD) and (HD), the latter zeroed before the launch
+    float* gqkv;               // backward outputs: (N, 3 HD) and (HD)
     float* gw;
+    float* partial;            // backward scratch: (blocks, HD) per-block sums of the weight gradient
     int N, HD, rows_per_block;
     float c1, lb, c2, q_scale;
 };
@@ -60,7 +61,8 @@ __global__ __launch_bounds__(256) void attention_inputs_fwd_kernel(AttnInArgs P)
 }
 
 // grid: ceil(N / rows_per_block) blocks of 256 threads; 256 % HD == 0.  Thread = (row offset, channel),
-// walks rows_per_block rows in steps of 256 / HD and keeps its channel's weight gradient in a register.
+// walks rows_per_block rows in steps of 256 / HD; the block's sum of the weight gradient goes to
+// partial[block][HD] (no atomics: a second small launch adds the blocks up).
 __global__ __launch_bounds__(256) void attention_inputs_bwd_kernel(AttnInArgs P) {
     const int c = threadIdx.x % P.HD, r = threadIdx.x / P.HD, step = 256 / P.HD;
     const int n0 = blockIdx.x * P.rows_per_block;
@@ -68,22 +70,52 @@ __global__ __launch_bounds__(256) void attention_inputs_bwd_kernel(AttnInArgs P)
     const float wc = P.w[c];
     const int H = P.HD >> 4;
     float gw = 0.0f;
-    for (int nb = n0; nb < n1; nb += step) {          // uniform trip count: row_sum needs every lane
+#pragma unroll 4
+    for (int nb = n0; nb < n0 + P.rows_per_block; nb += step) {   // uniform trip count: row_sum needs every lane
         const int n = nb + r;
         const bool live = n < n1;
         const size_t row = (size_t)(live ? n : n0) * 3 * P.HD;
-        const float q = live ? P.qkv[row + c] : 0.0f;
+        const size_t o = (size_t)(live ? n : n0) * P.HD + c;
+        const float q = P.qkv[row + c];
+        const float ga = P.ga ? P.ga[(size_t)(live ? n : n0) * H + (c >> 4)] : 0.0f;
+        const float gqs = P.gqs ? P.gqs[o] : 0.0f;
+        const float gk = P.gk ? P.gk[o] : 0.0f;
+        const float gv = P.gv ? P.gv[o] : 0.0f;
         float slope;
         gauss_alpha(P, q, wc, slope);
-        if (!live) continue;
-        const size_t o = (size_t)n * P.HD + c;
-        const float galpha = P.ga ? P.ga[(size_t)n * H + (c >> 4)] * slope : 0.0f;
-        gw += galpha * q;
-        P.gqkv[row + c] = galpha * wc + (P.gqs ? P.gqs[o] * P.q_scale : 0.0f);
-        P.gqkv[row + P.HD + c] = P.gk ? P.gk[o] : 0.0f;
-        P.gqkv[row + 2 * P.HD + c] = P.gv ? P.gv[o] : 0.0f;
+        const float galpha = ga * slope;
+        if (live) {
+            gw += galpha * q;
+            P.gqkv[row + c] = galpha * wc + gqs * P.q_scale;
+            P.gqkv[row + P.HD + c] = gk;
+            P.gqkv[row + 2 * P.HD + c] = gv;
+        }
     }
-    atomicAdd(P.gw + c, gw);
+    __shared__ float part[256];
+    part[threadIdx.x] = gw;
+    __syncthreads();
+    if (threadIdx.x < P.HD) {
+        float sum = 0.0f;
+        for (int g = 0; g < step; g++) sum += part[threadIdx.x + g * P.HD];
+        P.partial[(size_t)blockIdx.x * P.HD + threadIdx.x] = sum;
+    }
+}
+
+// gw[c] = sum over blocks of partial[block][c].  grid: ceil(HD / 32) blocks of 1024 threads = 32 groups x 32 channels
+__global__ __launch_bounds__(1024) void attention_inputs_gw_kernel(const float* __restrict__ partial, int nblocks, int HD,
+                                                                   float* __restrict__ gw) {
+    const int c = blockIdx.x * 32 + (threadIdx.x & 31), g = threadIdx.x >> 5;
+    float sum = 0.0f;
+    if (c < HD)
+        for (int b = g; b < nblocks; b += 32) sum += partial[(size_t)b * HD + c];
+    __shared__ float part[1024];
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    if (g == 0 && c < HD) {
+        float total = 0.0f;
+        for (int k = 0; k < 32; k++) total += part[(threadIdx.x & 31) + 32 * k];
+        gw[c] = total;
+    }
 }
 
 }  // namespace cfh

@@ -584,19 +584,22 @@ int cfh_attention_inputs_forward(const float* qkv, const float* lattice_w, const
 int cfh_attention_inputs_backward(const float* qkv, const float* lattice_w, const float* gauss_scale_dev,
                                   float c1, float lb, float c2, float q_scale, const float* gqs, const float* gk,
                                   const float* gv, const float* ga, int64_t N, int32_t H, int32_t Dh,
-                                  float* gqkv, float* g_lattice_w, void* stream) {
+                                  float* gqkv, float* g_lattice_w, void* workspace, size_t workspace_bytes,
+                                  void* stream) {
     cfh::AttnInArgs A;
     if (int rc = attention_inputs_args(A, qkv, lattice_w, gauss_scale_dev, c1, lb, c2, q_scale, N, H, Dh)) return rc;
     if (!g_lattice_w || (N > 0 && !gqkv)) return fail(CFH_EINVAL, "gqkv and g_lattice_w must not be NULL");
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(cfh::zero2_kernel, dim3((A.HD + 255) / 256), dim3(256), 0, st, g_lattice_w, A.HD,
-                       (float*)nullptr, 0);
+    A.rows_per_block = 4 * (256 / A.HD);
+    const int blocks = (int)((N + A.rows_per_block - 1) / A.rows_per_block);
+    if (int rc = check_workspace(workspace, workspace_bytes, (size_t)blocks * A.HD * sizeof(float))) return rc;
     if (N > 0) {
         A.gqs = gqs; A.gk = gk; A.gv = gv; A.ga = ga; A.gqkv = gqkv; A.gw = g_lattice_w;
-        A.rows_per_block = 8 * (256 / A.HD);
-        hipLaunchKernelGGL(cfh::attention_inputs_bwd_kernel, dim3((unsigned)((N + A.rows_per_block - 1) / A.rows_per_block)),
-                           dim3(256), 0, st, A);
+        A.partial = (float*)workspace;
+        hipLaunchKernelGGL(cfh::attention_inputs_bwd_kernel, dim3((unsigned)blocks), dim3(256), 0, st, A);
     }
+    hipLaunchKernelGGL(cfh::attention_inputs_gw_kernel, dim3((A.HD + 31) / 32), dim3(1024), 0, st,
+                       (const float*)workspace, blocks, A.HD, g_lattice_w);
     return finish_launch("attention_inputs_backward");
 }
 

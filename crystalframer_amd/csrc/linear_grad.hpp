@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void linear_wgrad_kernel(const float* __restri
 
 // Several layers' gradients in one launch: the jobs travel in the kernel arguments, workgroup b
 // belongs to the job with block0 <= b < block0 + bx by slices.
-constexpr int WGRAD_MAX_JOBS = 24;
+constexpr int WGRAD_MAX_JOBS = 32;
 struct WgradJob {
     const float* x; const float* dy; float* dW; float* db;
     int N, I, O, ldx, ldy;

@@ -489,9 +489,11 @@ class _DeferredWeightGrads:
     had a ``.grad`` (accumulation over several passes), autograd has added the zeros to it at once and
     the batch call adds into that ``.grad`` instead."""
     ARENA_FLOATS = 1 << 21
-    pending = []            # (x2, gy2, col0, O, dW_view, db_view, weight, bias, whole bias-gradient view, marks)
+    pending = []            # (x2, gy2, col0, O, dW ref, bias-gradient ref, weight, bias, marks)
     arena = None
     arena_off = 0
+    arenas = []             # keeps the gradient memory of the pass alive; the views themselves are NOT kept:
+                            # autograd adopts a gradient tensor as .grad only if nobody else references it
     callback_queued = False
     task_id = -1            # autograd graph task the pending work belongs to
 
@@ -503,6 +505,8 @@ class _DeferredWeightGrads:
             cls.arena_off = 0
         v = cls.arena[cls.arena_off:cls.arena_off + n]
         cls.arena_off += n_al
+        if not cls.arenas or cls.arenas[-1] is not cls.arena:
+            cls.arenas.append(cls.arena)
         return v
 
     @staticmethod
@@ -516,40 +520,47 @@ class _DeferredWeightGrads:
         cls.pending = []
         cls.arena = None
         cls.arena_off = 0
+        cls.arenas = []
         cls.callback_queued = False
 
     @classmethod
     def flush(cls):
         pending, cls.pending = cls.pending, []
+        arenas, cls.arenas = cls.arenas, []
         cls.arena = None
         cls.arena_off = 0
         cls.callback_queued = False
         if not pending:
             return
+
+        def view(ref):           # (arena, offset, count) -> tensor
+            return ref[0][ref[1]:ref[1] + ref[2]]
         lib = _lib.load()
         dev = pending[0][0].device
         jobs = (_lib.CfhLinearGradJob * len(pending))()
         fixups = []
-        for n, (x2, g2, col0, O, dW, db, weight, bias, first, w_mark, b_mark) in enumerate(pending):
-            dst_w, dst_b = dW, db
+        for n, (x2, g2, col0, O, dW, db, weight, bias, w_mark, b_mark) in enumerate(pending):
+            # dW, db: (arena, offset, count) of the zero-filled tensors handed to autograd (db: of the whole bias)
+            dst_w = dW[0].data_ptr() + 4 * dW[1]
+            dst_b = None if db is None else db[0].data_ptr() + 4 * (db[1] + col0)
             wg = weight.grad
-            if wg is not None and cls.mark(weight) != w_mark and wg.data_ptr() != dW.data_ptr():
+            if wg is not None and cls.mark(weight) != w_mark and wg.data_ptr() != dst_w:
                 # .grad was set or updated during this pass, but not by adopting our tensor: autograd
                 # copied or accumulated it (adding our zeros), so the result belongs into .grad
                 if wg.dtype == torch.float32 and wg.is_contiguous() and wg.device == dev:
-                    dst_w = wg
+                    dst_w = wg.data_ptr()
                 else:
-                    fixups.append((wg, dW))
+                    fixups.append((wg, view(dW).view(wg.shape)))
             if db is not None:
                 bg = bias.grad
-                if bg is not None and cls.mark(bias) != b_mark and bg.data_ptr() != first.data_ptr():
+                if bg is not None and cls.mark(bias) != b_mark and bg.data_ptr() != db[0].data_ptr() + 4 * db[1]:
                     if bg.dtype == torch.float32 and bg.is_contiguous() and bg.device == dev:
-                        dst_b = bg[col0:col0 + O]
+                        dst_b = bg.data_ptr() + 4 * col0
                     elif col0 == 0:
-                        fixups.append((bg, first))
+                        fixups.append((bg, view(db)))
             J = jobs[n]
             J.x, J.dy = x2.data_ptr(), g2.data_ptr() + 4 * col0
-            J.dW, J.db = dst_w.data_ptr(), (dst_b.data_ptr() if dst_b is not None else None)
+            J.dW, J.db = dst_w, dst_b
             J.N, J.I, J.O, J.ldx, J.ldy = x2.shape[0], x2.shape[1], O, x2.stride(0), g2.stride(0)
         with torch.cuda.device(dev), _timed("linear_weight_bias_grad_batch", dev):
             rc = lib.cfh_linear_weight_bias_grad_batch(jobs, len(pending), _lib.current_stream_ptr(dev))
@@ -597,7 +608,9 @@ class LinearHIP(torch.autograd.Function):
         defer = (KernelManager.DEFER_WEIGHT_GRADS and all(w.is_leaf for w in weights)
                  and (bias is None or bias.is_leaf) and all(w.dtype == torch.float32 for w in weights))
         if defer:
-            take = lambda n: D.take(n, dev)
+            def take(n):
+                v = D.take(n, dev)
+                return v, (D.arena, D.arena_off - ((n + 63) & ~63), n)
         else:
             total = sum(w.numel() for w in weights) + (W.shape[0] if bias is not None else 0)
             buf = torch.zeros(total, dtype=torch.float32, device=dev)
@@ -606,15 +619,16 @@ class LinearHIP(torch.autograd.Function):
             def take(n):
                 v = buf[state[0]:state[0] + n]
                 state[0] += n
-                return v
-        gb = take(W.shape[0]) if bias is not None else None
+                return v, (buf, state[0] - n, n)
+        gb, gb_ref = take(W.shape[0]) if bias is not None else (None, None)
         gws, jobs, col0 = [], [], 0
         for w in weights:
             O = w.shape[0]
-            dW = take(O * I).view(O, I)
-            gws.append(dW)
-            jobs.append((x2, g2, col0, O, dW, gb[col0:col0 + O] if gb is not None else None, w, bias, gb,
+            dW, dW_ref = take(O * I)
+            gws.append(dW.view(O, I))
+            jobs.append((x2, g2, col0, O, dW_ref, gb_ref, w, bias,
                          D.mark(w) if defer else None, D.mark(bias) if defer and bias is not None else None))
+            del dW
             col0 += O
         if defer:
             D.pending.extend(jobs)
@@ -628,7 +642,8 @@ class LinearHIP(torch.autograd.Function):
             for n, (x2_, g2_, c0, O, dW, db, *_) in enumerate(jobs):
                 J = arr[n]
                 J.x, J.dy = x2_.data_ptr(), g2_.data_ptr() + 4 * c0
-                J.dW, J.db = dW.data_ptr(), (db.data_ptr() if db is not None else None)
+                J.dW = dW[0].data_ptr() + 4 * dW[1]
+                J.db = None if db is None else db[0].data_ptr() + 4 * (db[1] + c0)
                 J.N, J.I, J.O, J.ldx, J.ldy = x2_.shape[0], I, O, x2_.stride(0), g2_.stride(0)
             with torch.cuda.device(dev), _timed("linear_weight_bias_grad", dev):
                 rc = lib.cfh_linear_weight_bias_grad_batch(arr, len(jobs), _lib.current_stream_ptr(dev))
@@ -693,10 +708,13 @@ class AttentionInputsHIP(torch.autograd.Function):
         gqs, gk, gv, ga = (None if g is None else _f32c(g) for g in (gqs, gk, gv, ga))
         gqkv = torch.empty_like(qkv)
         gw = torch.empty((H * Dh,), dtype=torch.float32, device=qkv.device)
+        # scratch of the call: per-block partial sums of the weight gradient (256-byte aligned by the allocator)
+        ws = torch.empty(4 * H * Dh * (N // (4 * (256 // (H * Dh))) + 1), dtype=torch.uint8, device=qkv.device)
         with _timed("attention_inputs_backward", qkv.device):
             rc = lib.cfh_attention_inputs_backward(_lib.ptr(qkv), _lib.ptr(w), _lib.ptr(gs), c1, lb, c2, q_scale,
                                                    _lib.ptr(gqs), _lib.ptr(gk), _lib.ptr(gv), _lib.ptr(ga), N, H, Dh,
-                                                   _lib.ptr(gqkv), _lib.ptr(gw), _lib.current_stream_ptr(qkv.device))
+                                                   _lib.ptr(gqkv), _lib.ptr(gw), _lib.ptr(ws), ws.numel(),
+                                                   _lib.current_stream_ptr(qkv.device))
         _lib.check(rc, "cfh_attention_inputs_backward")
         return gqkv, gw, None, None, None, None, None, None
 

@@ -246,7 +246,7 @@ int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int6
  * initialised them: zeros, or gradients to add to).  Each job: x (N,I) with row stride ldx, dy (N,O)
  * with row stride ldy (so a job may take a column block of a wider dy, e.g. one of the three
  * stacked input projections), dW (O,I) contiguous, db (O) or NULL.  `jobs` is a host array; it is
- * copied into the kernel arguments, 24 jobs per launch.  Deferring the weight gradients of a whole
+ * copied into the kernel arguments, 32 jobs per launch.  Deferring the weight gradients of a whole
  * backward pass to one call replaces one launch (plus clearing) per layer -- latency-bound at these
  * sizes -- by a launch that fills the chip.  No counterpart in the reference (autograd of
  * torch.nn.functional.linear, one GEMM per layer).
@@ -267,6 +267,7 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
  *   alpha' = (alpha + gauss_scale_dev[1]) * gauss_scale_dev[0]  (alpha' = alpha when the pointer is NULL).
  * Backward: gqkv (N, 3 H Dh) = [ga da/dquery + gqs q_scale | gk | gv],  g_lattice_w (H Dh) = sum over atoms
  *   of ga da/dalpha query;  gqs, gk, gv, ga may each be NULL (zero).  gauss_scale_dev is a constant.
+ *   workspace: ceil(N / (4 * (256 / (H Dh)))) * H Dh floats of scratch (per-block partial sums).
  * Dh = 16, 256 % (H Dh) == 0.  Replaces the framework arithmetic of
  * models/indexed_lattice_multi_head_attention_cuda.py:896-940 (gaussian coefficient: c1 = beta / (1 - lb),
  * c2 = -1/2 scale_real^-2), the query scaling of :144-185 and :455, and the chunk / cat of the
@@ -278,7 +279,8 @@ int cfh_attention_inputs_forward(const float* qkv, const float* lattice_w, const
 int cfh_attention_inputs_backward(const float* qkv, const float* lattice_w, const float* gauss_scale_dev,
                                   float c1, float lb, float c2, float q_scale, const float* gqs, const float* gk,
                                   const float* gv, const float* ga, int64_t N, int32_t H, int32_t Dh,
-                                  float* gqkv, float* g_lattice_w, void* stream);
+                                  float* gqkv, float* g_lattice_w, void* workspace, size_t workspace_bytes,
+                                  void* stream);
 
 #ifdef __cplusplus
 }
