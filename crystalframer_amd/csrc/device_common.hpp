@@ -247,6 +247,24 @@ __device__ __forceinline__ void window_scatter(uint32_t* base, const WindowSeed&
     for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; atomicAdd(base + m, (uint32_t)g); }
 }
 
+// The same with the walking order chosen per lane (dir = +1: centre, upwards, then downwards; -1: centre,
+// downwards, then upwards): lanes whose windows coincide (clamped windows of one pair) then add to
+// different words at the same time instead of queueing on one.
+template <int W>
+__device__ __forceinline__ void window_scatter_dir(uint32_t* base, const WindowSeed& s, float cc, int dir) {
+    constexpr int C = W / 2;
+    static_assert(W == 2 * C + 1, "window width must be odd");
+    uint32_t* const centre = base + C;
+    atomicAdd(centre, (uint32_t)s.gc);
+    float g = s.gc, r = dir > 0 ? s.rr : s.rl;
+    uint32_t* p = centre;
+#pragma unroll
+    for (int m = 1; m <= C; m++) { p += dir; g *= r; r *= cc; atomicAdd(p, (uint32_t)g); }
+    g = s.gc; r = dir > 0 ? s.rl : s.rr; p = centre;
+#pragma unroll
+    for (int m = 1; m <= C; m++) { p -= dir; g *= r; r *= cc; atomicAdd(p, (uint32_t)g); }
+}
+
 // Scatter weight*g_m into hbase[m] and return sum_m weight*g_m*gbase[m].
 template <int W>
 __device__ __forceinline__ float window_scatter_gather(uint32_t* hbase, const float* gbase,

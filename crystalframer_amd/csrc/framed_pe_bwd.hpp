@@ -109,7 +109,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
             if (NENC > 0) {
                 const int nb = (nlist + WAVE - 1) / WAVE;
                 for (int bt = 0; bt < nb; bt++) {
-                    const int idx = lane * nb + bt;
+                    const int idx = (((lane & 15) << 2) | (lane >> 4)) * nb + bt;   // neighbours in different rows, as in the forward
                     if (idx < nlist) {
                         const uint32_t ent = list[idx];
                         const int el = ent >> BWD_SHIFT;

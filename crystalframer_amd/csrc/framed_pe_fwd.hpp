@@ -113,7 +113,9 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
             if (HAS_LEN) {
                 const int nb = (nlist + WAVE - 1) / WAVE;
                 for (int bt = 0; bt < nb; bt++) {
-                    const int idx = lane * nb + bt;       // every nb-th entry: lanes spread over the pairs
+                    // every nb-th entry, and neighbouring entries (mostly translations of one pair, which
+                    // often share a clamped window and then add to the same words) in different 16-lane rows
+                    const int idx = (((lane & 15) << 2) | (lane >> 4)) * nb + bt;
                     if (idx < nlist) {
                         const uint32_t ent = list[idx];
                         const int el = ent >> FWD_SHIFT;
@@ -123,6 +125,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                         const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
                         const float w = hw_exp2(a2 * (d2 - pa.w)) * pairS[el].y;
                         uint32_t* const myhist = hist + el * PAIR_STRIDE;
+                        const int dir = ((lane ^ (lane >> 4)) & 1) ? -1 : 1;     // half of the lanes walk their windows the other way round
                         {
                             const float d = hw_sqrt(d2);
                             const float u = d * bc.inv_interval;
@@ -131,7 +134,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                             // bin k has centre (k+1)*interval: scaled offset ((k+1) - u)*len_step
                             const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
                             const WindowSeed s = window_seed(beta_c, bc.len_step, w);
-                            window_scatter<WL>(myhist + start, s, bc.len_cc);
+                            window_scatter_dir<WL>(myhist + start, s, bc.len_cc, dir);
                         }
                         if (HAS_ANG) {
                             if (d2 > 1e-5f) {       // the self image contributes to S only
@@ -147,7 +150,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                                     const float mu_c = bc.ang_mu0 + (float)(start + WA / 2) * bc.ang_interval;
                                     const float beta_c = (mu_c - cs) * bc.ang_sigma_inv;
                                     const WindowSeed s = window_seed(beta_c, bc.ang_step, w);
-                                    window_scatter<WA>(myhist + (ax + 1) * HS + start, s, bc.ang_cc);
+                                    window_scatter_dir<WA>(myhist + (ax + 1) * HS + start, s, bc.ang_cc, dir);
                                 }
                             }
                         }
