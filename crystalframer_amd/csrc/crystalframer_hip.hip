@@ -197,7 +197,6 @@ int resident_waves(Kern kern, int cap, int H) {
         per_cu = 4;
     int cus = device_cus();
     if (cus <= 0) cus = 256;
-    if (const char* e = getenv("CFH_DEBUG_WAVES_PER_CU")) { int v = atoi(e); if (v > 0 && v < per_cu) per_cu = v; }
     int64_t want = (int64_t)cus * per_cu;
     if (want > cap) want = cap;
     want = (want / H) * H;
