@@ -7,14 +7,16 @@
 //   l_e = q_i . k_j + a_e,   p_e = softmax over the pairs e = (i, .) of atom i,
 //   o_i = sum_e p_e (v_j + b_e)
 //
-// One wavefront per (atom, head).  A lane is (slot, channel): 4 pairs are in flight at once, each
-// on 16 lanes that hold one channel of the 16-wide head each.  The forward keeps a running
-// (max, sum, accumulator) per slot and merges the four slots at the end, so a row of any length
-// needs no scratch memory.  The backward is split in a row kernel (gq, ga, gb: everything indexed
-// like the forward) and a column kernel (gk, gv: sums over the pairs (., j) that point AT an atom),
-// which finds the pair (i, j) from the row of i.  Pairs are the complete n x n block of each
-// crystal, rows and columns in atom order -- the layout the reference's transposition kernel
-// assumes as well -- so pair (i, j) sits at e_start[i] + (j - first atom of the crystal).
+// One wavefront per (atom, head).  A lane is (slot, quarter): 16 pairs are in flight at once, each
+// on 4 lanes that hold 4 of the 16 channels of the head each (one 16-byte load per lane and operand;
+// most rows fit one step, so a row costs three dependent memory round trips: its bounds, the
+// neighbour indices, the operands).  Rows of up to 16 pairs are finished in registers; longer rows
+// keep a running (max, sum, accumulator) per slot, merge the slots at the end and rescale the
+// logits they parked in the probability array.  The backward is split in a row kernel (gq, ga, gb:
+// everything indexed like the forward) and a column kernel (gk, gv: sums over the pairs (., j) that
+// point AT an atom), which finds the pair (i, j) from the row of i.  Pairs are the complete n x n
+// block of each crystal, rows and columns in atom order -- the layout the reference's transposition
+// kernel assumes as well -- so pair (i, j) sits at e_start[i] + (j - first atom of the crystal).
 // Every sum is taken in a fixed order: results are bit-reproducible run to run.
 #pragma once
 #include "device_common.hpp"
@@ -41,14 +43,29 @@ struct DpaArgs {
 };
 
 constexpr int DPA_WAVES = 4;     // wavefronts (items) per workgroup
+constexpr int DPA_SLOTS = 16;    // pairs in flight per wavefront
 
-// sum over the 16 lanes of a slot
-__device__ __forceinline__ float slot_sum(float x) {
-    x += __shfl_xor(x, 1, WAVE);
-    x += __shfl_xor(x, 2, WAVE);
-    x += __shfl_xor(x, 4, WAVE);
-    x += __shfl_xor(x, 8, WAVE);
+// sum over the 4 lanes of a slot (quad_perm [1,0,3,2], [2,3,0,1])
+__device__ __forceinline__ float quad_sum(float x) {
+    x += dpp_move<0xB1>(x);
+    x += dpp_move<0x4E>(x);
     return x;
+}
+// sum over the 16 slots, for every quarter: lanes q, q+4, ..., q+60 (row_ror 4, 8, then the four rows)
+__device__ __forceinline__ float slots_sum(float x) {
+    x += dpp_move<0x124>(x);
+    x += dpp_move<0x128>(x);
+    return rows_sum(x);
+}
+__device__ __forceinline__ float4 slots_sum(float4 v) {
+    return make_float4(slots_sum(v.x), slots_sum(v.y), slots_sum(v.z), slots_sum(v.w));
+}
+__device__ __forceinline__ float wave_max(float v) { return -wave_min(-v); }
+__device__ __forceinline__ float dot4(const float4& a, const float4& b) {
+    return fmaf(a.x, b.x, fmaf(a.y, b.y, fmaf(a.z, b.z, a.w * b.w)));
+}
+__device__ __forceinline__ float4 ld4(const float* base, size_t row, int quarter) {
+    return reinterpret_cast<const float4*>(base + row * DH)[quarter];
 }
 
 __global__ __launch_bounds__(WAVE * DPA_WAVES) void dpa_fwd_kernel(const DpaArgs P) {
@@ -57,44 +74,76 @@ __global__ __launch_bounds__(WAVE * DPA_WAVES) void dpa_fwd_kernel(const DpaArgs
     if (item >= P.N * P.H) return;
     const int H = P.H;
     const int i = item / H, h = item - i * H;
-    const int slot = lane >> 4, c = lane & 15;
+    const int slot = lane >> 2, qd = lane & 3;
     const int e0 = (int)P.e_start[i], e1 = (int)P.e_start[i + 1];
-    const float qc = P.q[((size_t)i * H + h) * DH + c];
+    const float4 q4 = ld4(P.q, (size_t)i * H + h, qd);
+    float4* const out4 = reinterpret_cast<float4*>(P.out + ((size_t)i * H + h) * DH) + qd;
 
-    float m = -3.0e38f, s = 0.0f, acc = 0.0f;
-    for (int eb = e0; eb < e1; eb += 4) {
-        const int e = eb + slot;
+    if (e1 - e0 <= DPA_SLOTS) {
+        // the whole row in one step
+        const int e = e0 + slot;
         const bool valid = e < e1;
-        float part = 0.0f, val = 0.0f, bias = 0.0f;
+        float part = 0.0f, bias = 0.0f;
+        float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
         if (valid) {
             const size_t j = (size_t)P.edges[(size_t)P.E + e];
-            part = qc * P.k[(j * H + h) * DH + c];
-            val = P.v[(j * H + h) * DH + c];
-            if (P.bij) val += P.bij[((size_t)e * H + h) * DH + c];
+            part = dot4(q4, ld4(P.k, j * H + h, qd));
+            val = ld4(P.v, j * H + h, qd);
+            if (P.bij) {
+                const float4 b = ld4(P.bij, (size_t)e * H + h, qd);
+                val.x += b.x; val.y += b.y; val.z += b.z; val.w += b.w;
+            }
             if (P.aij) bias = P.aij[(size_t)e * H + h];
         }
-        const float l = slot_sum(part) + bias;
+        const float l = valid ? quad_sum(part) + bias : -3.0e38f;
+        const float M = wave_max(l);
+        const float w = valid ? __expf(l - M) : 0.0f;
+        const float S = wave_sum(w) * 0.25f;              // every slot counted by its 4 lanes
+        const float inv = (S > 0.0f) ? 1.0f / S : 0.0f;
+        const float4 acc = slots_sum(make_float4(w * val.x, w * val.y, w * val.z, w * val.w));
+        if (slot == 0) *out4 = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
+        if (valid && qd == 0) P.prob[(size_t)e * H + h] = w * inv;
+        return;
+    }
+
+    float m = -3.0e38f, s = 0.0f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int eb = e0; eb < e1; eb += DPA_SLOTS) {
+        const int e = eb + slot;
+        const bool valid = e < e1;
+        float part = 0.0f, bias = 0.0f;
+        float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
         if (valid) {
-            if (c == 0) P.prob[(size_t)e * H + h] = l;       // the logit for now
+            const size_t j = (size_t)P.edges[(size_t)P.E + e];
+            part = dot4(q4, ld4(P.k, j * H + h, qd));
+            val = ld4(P.v, j * H + h, qd);
+            if (P.bij) {
+                const float4 b = ld4(P.bij, (size_t)e * H + h, qd);
+                val.x += b.x; val.y += b.y; val.z += b.z; val.w += b.w;
+            }
+            if (P.aij) bias = P.aij[(size_t)e * H + h];
+        }
+        const float l = quad_sum(part) + bias;
+        if (valid) {
+            if (qd == 0) P.prob[(size_t)e * H + h] = l;       // the logit for now
             const float mn = fmaxf(m, l);
             const float sc = __expf(m - mn), w = __expf(l - mn);
             s = s * sc + w;
-            acc = acc * sc + w * val;
+            acc.x = acc.x * sc + w * val.x; acc.y = acc.y * sc + w * val.y;
+            acc.z = acc.z * sc + w * val.z; acc.w = acc.w * sc + w * val.w;
             m = mn;
         }
     }
-    // merge the four slots
-    float M = fmaxf(m, __shfl_xor(m, 16, WAVE));
-    M = fmaxf(M, __shfl_xor(M, 32, WAVE));
+    // merge the slots
+    const float M = wave_max(m);
     const float sc = (s > 0.0f) ? __expf(m - M) : 0.0f;
-    s *= sc; acc *= sc;
-    s += __shfl_xor(s, 16, WAVE); s += __shfl_xor(s, 32, WAVE);
-    acc += __shfl_xor(acc, 16, WAVE); acc += __shfl_xor(acc, 32, WAVE);
-    const float inv = (s > 0.0f) ? 1.0f / s : 0.0f;
-    if (slot == 0) P.out[((size_t)i * H + h) * DH + c] = acc * inv;
+    const float S = wave_sum(s * sc) * 0.25f;
+    const float inv = (S > 0.0f) ? 1.0f / S : 0.0f;
+    acc = slots_sum(make_float4(acc.x * sc, acc.y * sc, acc.z * sc, acc.w * sc));
+    if (slot == 0) *out4 = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
     // logits -> probabilities (each was written by the lane that now reads it)
-    if (c == 0)
-        for (int e = e0 + slot; e < e1; e += 4) {
+    if (qd == 0)
+        for (int e = e0 + slot; e < e1; e += DPA_SLOTS) {
             const size_t o = (size_t)e * H + h;
             P.prob[o] = __expf(P.prob[o] - M) * inv;
         }
@@ -107,66 +156,77 @@ __global__ __launch_bounds__(WAVE * DPA_WAVES) void dpa_bwd_row_kernel(const Dpa
     if (item >= P.N * P.H) return;
     const int H = P.H;
     const int i = item / H, h = item - i * H;
-    const int slot = lane >> 4, c = lane & 15;
+    const int slot = lane >> 2, qd = lane & 3;
     const int e0 = (int)P.e_start[i], e1 = (int)P.e_start[i + 1];
-    const size_t ih = ((size_t)i * H + h) * DH + c;
-    const float goc = P.go[ih];
-    const float D = slot_sum(goc * P.out[ih]);
-    float gq = 0.0f;
-    for (int eb = e0; eb < e1; eb += 4) {
+    const size_t ih = (size_t)i * H + h;
+    const float4 go4 = ld4(P.go, ih, qd);
+    const float D = quad_sum(dot4(go4, ld4(P.out, ih, qd)));
+    float4 gq = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int eb = e0; eb < e1; eb += DPA_SLOTS) {
         const int e = eb + slot;
         const bool valid = e < e1;
-        float part = 0.0f, kc = 0.0f, p = 0.0f;
+        float part = 0.0f, p = 0.0f;
+        float4 k4 = make_float4(0.f, 0.f, 0.f, 0.f);
         if (valid) {
             const size_t j = (size_t)P.edges[(size_t)P.E + e];
-            kc = P.k[(j * H + h) * DH + c];
-            float val = P.v[(j * H + h) * DH + c];
-            if (P.bij) val += P.bij[((size_t)e * H + h) * DH + c];
+            k4 = ld4(P.k, j * H + h, qd);
+            float4 val = ld4(P.v, j * H + h, qd);
+            if (P.bij) {
+                const float4 b = ld4(P.bij, (size_t)e * H + h, qd);
+                val.x += b.x; val.y += b.y; val.z += b.z; val.w += b.w;
+            }
             p = P.prob[(size_t)e * H + h];
-            part = goc * val;
+            part = dot4(go4, val);
         }
-        const float gl = p * (slot_sum(part) - D);
+        const float gl = p * (quad_sum(part) - D);
         if (valid) {
-            if (c == 0) P.gaij[(size_t)e * H + h] = gl;
-            if (P.gbij) P.gbij[((size_t)e * H + h) * DH + c] = p * goc;
-            gq = fmaf(gl, kc, gq);
+            if (qd == 0) P.gaij[(size_t)e * H + h] = gl;
+            if (P.gbij)
+                reinterpret_cast<float4*>(P.gbij + ((size_t)e * H + h) * DH)[qd] =
+                    make_float4(p * go4.x, p * go4.y, p * go4.z, p * go4.w);
+            gq.x = fmaf(gl, k4.x, gq.x); gq.y = fmaf(gl, k4.y, gq.y);
+            gq.z = fmaf(gl, k4.z, gq.z); gq.w = fmaf(gl, k4.w, gq.w);
         }
     }
-    gq += __shfl_xor(gq, 16, WAVE);
-    gq += __shfl_xor(gq, 32, WAVE);
-    if (slot == 0) P.gq[ih] = gq;
+    gq = slots_sum(gq);
+    if (slot == 0) reinterpret_cast<float4*>(P.gq + ih * DH)[qd] = gq;
 }
 
-// gk_j = sum_i gl_(i,j) q_i, gv_j = sum_i p_(i,j) go_i over the atoms i of the crystal of j
+// gk_j = sum_i gl_(i,j) q_i, gv_j = sum_i p_(i,j) go_i over the atoms i of the crystal of j; every
+// row of the crystal's block has n pairs, so pair (i, j) is at (first pair of the crystal) + r n + col
 __global__ __launch_bounds__(WAVE * DPA_WAVES) void dpa_bwd_col_kernel(const DpaArgs P) {
     const int lane = threadIdx.x & (WAVE - 1);
     const int item = blockIdx.x * DPA_WAVES + (threadIdx.x >> 6);
     if (item >= P.N * P.H) return;
     const int H = P.H;
     const int j = item / H, h = item - j * H;
-    const int slot = lane >> 4, c = lane & 15;
+    const int slot = lane >> 2, qd = lane & 3;
     const int e0 = (int)P.e_start[j], n = (int)P.e_start[j + 1] - e0;
-    float gk = 0.0f, gv = 0.0f;
+    float4 gk = make_float4(0.f, 0.f, 0.f, 0.f), gv = gk;
     if (n > 0) {
         const int first = (int)P.edges[(size_t)P.E + e0];      // first atom of the crystal
         const int col = j - first;
-        for (int ib = 0; ib < n; ib += 4) {
+        const size_t eblock = (size_t)e0 - (size_t)col * n;    // first pair of the crystal
+        for (int ib = 0; ib < n; ib += DPA_SLOTS) {
             const int r = ib + slot;
             if (r < n) {
-                const int i = first + r;
-                const size_t e = (size_t)P.e_start[i] + col;
-                const size_t ih = ((size_t)i * H + h) * DH + c;
-                gk = fmaf(P.gaij[e * H + h], P.q[ih], gk);
-                gv = fmaf(P.prob[e * H + h], P.go[ih], gv);
+                const size_t e = eblock + (size_t)r * n + col;
+                const size_t ih = (size_t)(first + r) * H + h;
+                const float gl = P.gaij[e * H + h], p = P.prob[e * H + h];
+                const float4 q4 = ld4(P.q, ih, qd), go4 = ld4(P.go, ih, qd);
+                gk.x = fmaf(gl, q4.x, gk.x); gk.y = fmaf(gl, q4.y, gk.y);
+                gk.z = fmaf(gl, q4.z, gk.z); gk.w = fmaf(gl, q4.w, gk.w);
+                gv.x = fmaf(p, go4.x, gv.x); gv.y = fmaf(p, go4.y, gv.y);
+                gv.z = fmaf(p, go4.z, gv.z); gv.w = fmaf(p, go4.w, gv.w);
             }
         }
     }
-    gk += __shfl_xor(gk, 16, WAVE); gk += __shfl_xor(gk, 32, WAVE);
-    gv += __shfl_xor(gv, 16, WAVE); gv += __shfl_xor(gv, 32, WAVE);
+    gk = slots_sum(gk);
+    gv = slots_sum(gv);
     if (slot == 0) {
-        const size_t jh = ((size_t)j * H + h) * DH + c;
-        P.gk[jh] = gk;
-        P.gv[jh] = gv;
+        const size_t jh = (size_t)j * H + h;
+        reinterpret_cast<float4*>(P.gk + jh * DH)[qd] = gk;
+        reinterpret_cast<float4*>(P.gv + jh * DH)[qd] = gv;
     }
 }
 
