@@ -54,6 +54,7 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (reference point for HBM traffic counters)")
+    ap.add_argument("--no-fused-adamw", action="store_true", help="PyTorch's multi-tensor AdamW instead of the fused kernel")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying the step as one HIP graph")
     ap.add_argument("--cpu-crystals", type=int, default=12, help="crystals of the batch in the CPU sample")
@@ -109,8 +110,9 @@ def main():
     cb = cb_cpu.to(dev)
     target = torch.randn(args.batch, 1, generator=torch.Generator().manual_seed(7)).to(dev)
     use_graph = not args.no_graph
+    # fused=True: PyTorch's single-kernel AdamW (same update rule as the default multi-tensor loop)
     opt = torch.optim.AdamW(model.parameters(), lr=5e-4, betas=(0.9, 0.98), weight_decay=1e-5,
-                            capturable=use_graph)
+                            capturable=use_graph, fused=not args.no_fused_adamw)
     # the tie-breaking noise of the frame search: seed word on the device, advanced by every call, so
     # that replays of the captured step draw fresh noise like separate launches do
     KM.NOISE_SEED = 20240607

@@ -215,7 +215,8 @@ std::vector<TimedLaunch> g_timed;
 template <typename Kern>
 int launch_persistent(Kern kern, const cfh::KernelArgs& A, int* waves, hipStream_t st, const char* what) {
     *waves = resident_waves(kern, *waves, A.H);
-    const int threads = A.N * A.H > A.H * cfh::NQUEUE ? A.N * A.H : A.H * cfh::NQUEUE;
+    int threads = A.N * A.H > A.H * cfh::NQUEUE ? A.N * A.H : A.H * cfh::NQUEUE;
+    if (threads < A.gw_out_n) threads = A.gw_out_n;
     hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, A, A.q != nullptr ? 1 : 0);
     bool timed = false;
     TimedLaunch t;
@@ -416,6 +417,11 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
     A.frames = frames; A.z = z; A.gz = gz; A.gpsi = gpsi; A.out_ga = ga;
     A.shat = const_cast<float*>(shat);
     A.gw_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + COUNTER_BYTES + items_bytes(N, p->num_heads));
+    if (has_len) {      // cleared by the prepare kernel of this launch, added into by gw_reduce_kernel
+        A.gw_out[0] = gW_dist;
+        if (has_ang) { A.gw_out[1] = gW_axis1; A.gw_out[2] = gW_axis2; A.gw_out[3] = gW_axis3; }
+        A.gw_out_n = p->num_heads * cfh::DH * cfh::NBINS;
+    }
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "framed_pe_backward";
     if (has_len && shat) {      // the forward kept its histograms: gather-only kernel
@@ -430,9 +436,6 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
         const int per_enc = p->num_heads * cfh::DH * cfh::NBINS;
         const int total = nenc * per_enc;
         const int nslices = 16;
-        hipLaunchKernelGGL(cfh::zero_outputs_kernel, dim3((per_enc + 255) / 256), dim3(256), 0, st, per_enc,
-                           gW_dist, nenc > 1 ? gW_axis1 : nullptr, nenc > 1 ? gW_axis2 : nullptr,
-                           nenc > 1 ? gW_axis3 : nullptr);
         hipLaunchKernelGGL(cfh::gw_reduce_kernel, dim3((total + 255) / 256, nslices), dim3(256), 0, st,
                            A.gw_partial, waves, p->num_heads, nenc, nslices, gW_dist, gW_axis1, gW_axis2, gW_axis3);
         rc = finish_launch("gw_reduce");

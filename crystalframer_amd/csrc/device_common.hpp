@@ -331,6 +331,8 @@ struct KernelArgs {
     // outputs
     float* out_z; float* out_psi; float* out_d2min; float* out_frame; float* out_ga;
     float* gw_partial;            // (waves, 4, DH, NBINS) per-wave weight-gradient partials
+    float* gw_out[4];             // backward: the (H, DH, NBINS) weight gradients, cleared by prepare_items_kernel
+    int32_t gw_out_n;             // elements of each (0: nothing to clear)
     float* shat;                  // (E, H, 4, NBINS) window histograms: written by the forward when given,
                                   // read by the backward that does not rebuild them
     int32_t* counters;            // (H, NQUEUE) work-queue heads
@@ -425,10 +427,16 @@ __device__ __forceinline__ uint32_t load_record(const KernelArgs& P, int it, int
     return (it >= 0 && threadIdx.x < REC_WORDS) ? P.items[((size_t)it * P.H + h) * REC_WORDS + threadIdx.x] : 0u;
 }
 
-// One thread per (item, head): builds the records and clears the work queues of the launch.
+// One thread per (item, head): builds the records, clears the work queues of the launch and (backward)
+// the weight-gradient outputs that the reduction after the main kernel adds into.
 __global__ __launch_bounds__(256) void prepare_items_kernel(const KernelArgs P, int with_query) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx < P.H * NQUEUE) P.counters[idx * QSTRIDE] = 0;
+    if (idx < P.gw_out_n) {
+#pragma unroll
+        for (int en = 0; en < 4; en++)
+            if (P.gw_out[en]) P.gw_out[en][idx] = 0.0f;
+    }
     if (idx >= P.N * P.H) return;
     const int it = idx / P.H, h = idx - it * P.H;
     const int i = P.order ? P.order[it] : it;
