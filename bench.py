@@ -39,10 +39,10 @@ PEAK_TRANS_TOPS = 9.8                  # quarter-rate transcendental unit
 # (KiB per dispatch) scaled by what the same counters read for the 256 MiB device copy of --calibrate-copy
 # (FETCH_SIZE reads 128 MiB for it: factor 2.0; WRITE_SIZE reads 256 MiB: factor 1.0); see profiles/.
 # With the forward keeping its window histograms for the backward (KernelManager.SAVE_HISTOGRAMS, the default):
-# forward 3 627 KiB x 2.0 fetched + 262 023 KiB written (243.9 MB of that are the histograms, E x H x 4 x 64
-# floats); backward 144 847 KiB x 2.0 fetched (the histograms again) + 34 261 KiB written (33.5 MB of that are
+# forward 3 396 KiB x 2.0 fetched + 261 808 KiB written (243.9 MB of that are the histograms, E x H x 4 x 64
+# floats); backward 144 766 KiB x 2.0 fetched (the histograms again) + 34 258 KiB written (33.5 MB of that are
 # the per-wavefront partials of the weight gradients).
-TRAFFIC_BYTES_PER_LAUNCH = {"framed_pe_backward": 331.7e6, "framed_pe_forward": 275.7e6}
+TRAFFIC_BYTES_PER_LAUNCH = {"framed_pe_backward": 331.6e6, "framed_pe_forward": 275.0e6}
 
 
 def parse():
@@ -207,8 +207,10 @@ def main():
     roofline = {
         "kernel": dominant + "_kernel", "bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS,
         "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_TFLOPS, "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
-        "bound_detail": "FP32 arithmetic (vector + a little MFMA) against the published 157.3 TFLOP/s; HBM traffic is "
-                        "<1 byte per term; what limits the kernel in practice is LDS atomic throughput",
+        "bound_detail": "FP32 arithmetic (vector + a little MFMA) against the published 157.3 TFLOP/s; HBM traffic "
+                        "(the kept window histograms) runs at 15-18 % of the HBM peak; in practice the forward is "
+                        "limited by LDS atomic throughput and bank conflicts, the backward by instruction issue and "
+                        "memory latency at 8 wavefronts per CU",
         "frac_of_unpacked_fp32_peak": achieved / PEAK_FP32_UNPACKED,
         "transcendental_frac": eval_dom * X_TERM / t_dom / 1e12 / PEAK_TRANS_TOPS,
         "avg_launch_ms": t_dom * 1e3,
