@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
@@ -43,6 +43,8 @@ class CfhParams(ctypes.Structure):
         ("grad_coef_quirk", ctypes.c_int32),
         ("collect_stats", ctypes.c_int32),
         ("noise_seed_dev", ctypes.c_void_p),
+        ("noise_seed_advance", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
     ]
 
 

@@ -177,7 +177,9 @@ void fill_common(cfh::KernelArgs& A, const cfh_params* p, const float* a_ih, con
     A.noise = p->symm_break_noise;
     A.seed_lo = (uint32_t)(p->noise_seed & 0xffffffffu);
     A.seed_hi = (uint32_t)(p->noise_seed >> 32);
-    A.seed_dev = reinterpret_cast<const unsigned long long*>(p->noise_seed_dev);
+    A.seed_dev = reinterpret_cast<unsigned long long*>(p->noise_seed_dev);
+    A.seed_snap = reinterpret_cast<unsigned long long*>(workspace);      // first word of the reserved header bytes
+    A.seed_advance = p->noise_seed_advance;
     A.bc = basis_consts(p);
 }
 

@@ -343,7 +343,10 @@ struct KernelArgs {
     float prune_log2;             // <= 0: keep every translation
     float dist_coef, angle_coef, gz_coef, gw_dist_coef;
     float noise; uint32_t seed_lo, seed_hi;
-    const unsigned long long* seed_dev;   // optional device word mixed into the seed
+    unsigned long long* seed_dev;   // optional device word mixed into the seed: prepare_items_kernel copies it
+                                    // to seed_snap (what the frame search reads) and, if seed_advance, adds one
+    unsigned long long* seed_snap;
+    int32_t seed_advance;
     BasisConsts bc;
 };
 
@@ -432,6 +435,11 @@ __device__ __forceinline__ uint32_t load_record(const KernelArgs& P, int it, int
 __global__ __launch_bounds__(256) void prepare_items_kernel(const KernelArgs P, int with_query) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx < P.H * NQUEUE) P.counters[idx * QSTRIDE] = 0;
+    if (idx == 0 && with_query && P.seed_dev) {
+        const unsigned long long s = *P.seed_dev;
+        *P.seed_snap = s;
+        if (P.seed_advance) *P.seed_dev = s + 1ull;
+    }
     if (idx < P.gw_out_n) {
 #pragma unroll
         for (int en = 0; en < 4; en++)

@@ -84,7 +84,7 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
     const bool noisy = P.noise > 0.0f;
     uint32_t seed_lo = P.seed_lo, seed_hi = P.seed_hi;
     if (noisy && P.seed_dev) {
-        const unsigned long long s = *P.seed_dev;
+        const unsigned long long s = *P.seed_snap;
         seed_lo ^= (uint32_t)s * 0x9E3779B1u;
         seed_hi += (uint32_t)(s >> 32) ^ ((uint32_t)s * 0x85EBCA77u);
     }

@@ -93,6 +93,7 @@ def _params(H: int, Dh: int, K: int, A: int, cos_abs: int, dist_max: float, wsca
         p.noise_seed = int(KernelManager.NOISE_SEED)
     sd = KernelManager.NOISE_SEED_DEVICE
     p.noise_seed_dev = sd.data_ptr() if (sd is not None and p.symm_break_noise > 0) else None
+    p.noise_seed_advance = 1          # every frame search advances the device word itself
     p.grad_coef_quirk = int(bool(KernelManager.GRAD_COEF_QUIRK))
     p.collect_stats = int(bool(KernelManager.COLLECT_STATS))
     return p
@@ -207,8 +208,6 @@ def _frame_call(mode: int, q, k, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, f
                                      _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(f1), N, E, tv.shape[0],
                                      _lib.ptr(out), _lib.ptr(ws), ws.numel(), st)
     _lib.check(rc, ("cfh_frame_axis1", "cfh_frame_axis2", "cfh_frame_axes")[mode])
-    if KernelManager.NOISE_SEED_DEVICE is not None and p.symm_break_noise > 0:
-        KernelManager.NOISE_SEED_DEVICE.add_(1)
     return out
 
 
@@ -577,27 +576,42 @@ class LinearHIP(torch.autograd.Function):
     one launch here.  Same values as torch.nn.functional.linear up to the order of the float32 sums."""
 
     @staticmethod
-    def forward(ctx, x, bias, stacked, *weights):
+    def forward(ctx, x, bias, stacked, relu, *weights):
         if stacked is not None:
             W = stacked
         elif len(weights) == 1:
             W = weights[0]
         else:
             W = torch.cat(weights, dim=0)
-        ctx.save_for_backward(x, W.detach())
         ctx.weights = weights
         ctx.bias = bias
+        ctx.relu = bool(relu)
+        if relu:
+            # bias and rectifier in the epilogue of the library GEMM
+            x2 = x.reshape(-1, W.shape[1])
+            if bias is not None:
+                y = torch._addmm_activation(bias.detach(), x2, W.detach().t(), use_gelu=False)
+            else:
+                y = torch.relu(x2.matmul(W.detach().t()))
+            y = y.reshape(*x.shape[:-1], W.shape[0])
+            ctx.save_for_backward(x, W.detach(), y)
+            return y
+        ctx.save_for_backward(x, W.detach())
         return torch.nn.functional.linear(x, W.detach(), None if bias is None else bias.detach())
 
     @staticmethod
     def backward(ctx, gy):
-        x, W = ctx.saved_tensors
+        if ctx.relu:
+            x, W, y = ctx.saved_tensors
+            gy = torch.ops.aten.threshold_backward(gy, y, 0.0)
+        else:
+            x, W = ctx.saved_tensors
         weights, bias = ctx.weights, ctx.bias
         gx = gy.matmul(W) if ctx.needs_input_grad[0] else None
-        need_w = [ctx.needs_input_grad[3 + n] for n in range(len(weights))]
+        need_w = [ctx.needs_input_grad[4 + n] for n in range(len(weights))]
         need_b = bias is not None and ctx.needs_input_grad[1]
         if not (any(need_w) or need_b):
-            return (gx, None, None) + (None,) * len(weights)
+            return (gx, None, None, None) + (None,) * len(weights)
         dev = x.device
         I = W.shape[1]
         x2 = _f32c(x.reshape(-1, I))
@@ -650,17 +664,18 @@ class LinearHIP(torch.autograd.Function):
             _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
         gws = [g.to(w.dtype) if g.dtype != w.dtype else g for g, w in zip(gws, weights)]
         gb_out = None if gb is None else (gb if gb.dtype == bias.dtype else gb.to(bias.dtype))
-        return (gx, gb_out, None) + tuple(gws)
+        return (gx, gb_out, None, None) + tuple(gws)
 
 
 def linear(x: torch.Tensor, weight, bias: Optional[torch.Tensor] = None,
-           stacked: Optional[torch.Tensor] = None) -> torch.Tensor:
+           stacked: Optional[torch.Tensor] = None, relu: bool = False) -> torch.Tensor:
     """torch.nn.functional.linear for device tensors with the library's weight-gradient kernel.
     ``weight``: a tensor (O,I), or a sequence of tensors (O_k,I) whose row-wise stack is the weight
-    (``stacked``: that stack if it already exists in memory)."""
+    (``stacked``: that stack if it already exists in memory); ``relu``: max(0, .) of the result, in
+    the epilogue of the GEMM."""
     weights = (weight,) if isinstance(weight, torch.Tensor) else tuple(weight)
     _lib.require_gpu(x, *weights)
-    return LinearHIP.apply(x, bias, stacked, *weights)
+    return LinearHIP.apply(x, bias, stacked, relu, *weights)
 
 
 class AttentionInputsHIP(torch.autograd.Function):

@@ -69,7 +69,10 @@ class CrystalformerEncoderLayerCUDA(nn.Module):
         return self.dropout1(x)
 
     def _ff_block(self, x):
-        h = self.activation(cuda_funcs.linear(x, self.linear1.weight, self.linear1.bias))
+        if self.activation is F.relu:
+            h = cuda_funcs.linear(x, self.linear1.weight, self.linear1.bias, relu=True)
+        else:
+            h = self.activation(cuda_funcs.linear(x, self.linear1.weight, self.linear1.bias))
         return self.dropout2(cuda_funcs.linear(self.dropout(h), self.linear2.weight, self.linear2.bias))
 
     def forward(self, src: Tensor, batch: Tensor, edges: Tensor, pos_ij: Tensor = None,

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 1
+#define CFH_ABI_VERSION 2
 
 enum {
     CFH_OK = 0,
@@ -79,9 +79,12 @@ typedef struct cfh_params {
                                 [1] forward translations in the boxes, [2],[3] same for backward,
                                 [4],[5] translations scanned by the two frame searches, [6],[7] (pair,
                                 head) items of forward / backward                                   */
-    const uint64_t* noise_seed_dev; /* optional device word mixed into noise_seed when a frame search
+    uint64_t* noise_seed_dev; /* optional device word mixed into noise_seed when a frame search
                                 starts: a caller that replays a captured graph advances it between
                                 replays to draw fresh noise; NULL: noise_seed alone              */
+    int32_t noise_seed_advance; /* 1: every frame search adds one to *noise_seed_dev after reading it
+                                (in its own launch, so a replayed graph needs no extra kernel)   */
+    int32_t reserved0;
 } cfh_params;
 
 /* Version of this ABI; a mismatch with CFH_ABI_VERSION means header and library differ. */

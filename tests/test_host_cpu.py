@@ -28,9 +28,9 @@ def test_library_exports_every_declared_symbol():
 def test_params_struct_matches_header_layout():
     header = open(os.path.join(ROOT, "include", "crystalframer_hip.h")).read()
     body = header[header.index("typedef struct cfh_params"):header.index("} cfh_params;")]
-    fields = re.findall(r"^\s*(?:int32_t|float|uint64_t|const uint64_t\*)\s+([a-z0-9_]+);", body, flags=re.M)
+    fields = re.findall(r"^\s*(?:int32_t|float|uint64_t|uint64_t\*)\s+([a-z0-9_]+);", body, flags=re.M)
     assert fields == [f[0] for f in _lib.CfhParams._fields_]
-    assert ctypes.sizeof(_lib.CfhParams) == 96
+    assert ctypes.sizeof(_lib.CfhParams) == 104
 
 
 def test_argument_errors_are_reported_without_a_gpu():
