@@ -20,6 +20,7 @@
 #include "framed_pe_bwd_saved.hpp"
 #include "framed_pe_fwd.hpp"
 #include "fused_dpa.hpp"
+#include "geometry.hpp"
 #include "linear_grad.hpp"
 
 namespace {
@@ -651,6 +652,32 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
     return finish_launch("linear_weight_bias_grad_batch");
 }
 
+int cfh_crystal_geometry(const float* pos, const int64_t* batch, const float* tvecs, const int64_t* sizes,
+                         int64_t N, int64_t B, int64_t E, int64_t* edges, float* rpos, float* recip,
+                         float* rvlen, float* vcell, int64_t* e_start, int64_t* atom_start, int32_t* order,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+    if (N < 0 || B < 0 || E < 0 || N > 0x7fffffffLL / 64 || B > 0x7fffffffLL / 64)
+        return fail(CFH_EINVAL, "sizes N=%lld B=%lld E=%lld out of range", (long long)N, (long long)B, (long long)E);
+    if (!e_start || !atom_start || (B > 0 && (!tvecs || !sizes || !recip || !rvlen || !vcell)) ||
+        (N > 0 && (!pos || !batch || !order)) || (E > 0 && (!edges || !rpos)))
+        return fail(CFH_EINVAL, "geometry: an input or output pointer is NULL");
+    if (int rc = check_workspace(workspace, workspace_bytes, (size_t)(2 * B + 1) * sizeof(int64_t))) return rc;
+    cfh::GeometryArgs A{};
+    A.pos = pos; A.batch = batch; A.tvecs = tvecs; A.sizes = sizes;
+    A.edges = edges; A.rpos = rpos; A.recip = recip; A.rvlen = rvlen; A.vcell = vcell;
+    A.e_start = e_start; A.order = order; A.atom_start = atom_start;
+    A.pair_start = reinterpret_cast<int64_t*>(workspace);
+    A.order_start = A.pair_start + (B + 1);
+    A.N = (int32_t)N; A.B = (int32_t)B; A.E = E;
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(cfh::geometry_crystals_kernel, dim3(1), dim3(cfh::GEO_THREADS), 0, st, A);
+    hipLaunchKernelGGL(cfh::geometry_atoms_kernel, dim3((unsigned)((N + 256) / 256)), dim3(256), 0, st, A);
+    if (E > 0)
+        hipLaunchKernelGGL(cfh::geometry_pairs_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, A);
+    return finish_launch("crystal_geometry");
+}
+
 }  // extern "C"
+
 
 

@@ -1,0 +1,155 @@
+// Per-batch geometry shared by every layer of a forward pass, in three launches: the pair list of the
+// fully connected crystals (i-major, the complete n x n block of each crystal), the pair vectors, the
+// reciprocal lattice and the work order of the atoms (longest rows first).  The reference builds the
+// same tensors with framework index arithmetic and a Python loop over crystals
+// (models/indexed_latticeformer_encoder.py:15-44,175-245).
+#pragma once
+#include "device_common.hpp"
+
+namespace cfh {
+
+struct GeometryArgs {
+    const float* pos;          // (N, 3)
+    const int64_t* batch;      // (N) crystal of each atom, ascending
+    const float* tvecs;        // (B, 3, 3) lattice rows
+    const int64_t* sizes;      // (B) atoms per crystal
+    int64_t* edges;            // (2, E)
+    float* rpos;               // (E, 3) pos[j] - pos[i]
+    float* recip;              // (B, 3, 3) 2 pi (t_b x t_c) / V, ...
+    float* rvlen;              // (B, 3)
+    float* vcell;              // (B)
+    int64_t* e_start;          // (N + 1)
+    int32_t* order;            // (N) atoms by descending crystal size
+    int64_t* atom_start;       // (B + 1) scratch / output: first atom of each crystal
+    int64_t* pair_start;       // (B + 1) scratch: first pair of each crystal
+    int64_t* order_start;      // (B) scratch: first position of each crystal's atoms in `order`
+    int32_t N, B;
+    int64_t E;
+};
+
+constexpr int GEO_THREADS = 1024;
+constexpr int GEO_KEYS = 2048;      // crystals of GEO_KEYS - 1 atoms or more share the first place of the order
+
+// One workgroup: prefix sums over the crystals, the reciprocal lattice, and where each crystal's atoms
+// go in the work order (descending size; equal sizes in crystal order when B <= GEO_THREADS, in the
+// order their atomics happen to arrive otherwise).
+#pragma clang fp contract(off)      // the framework expressions this replaces round every product and sum
+__global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const GeometryArgs P) {
+    __shared__ long long scan_a[GEO_THREADS], scan_p[GEO_THREADS];
+    __shared__ long long carry_a, carry_p;
+    __shared__ int hist[GEO_KEYS];
+    const int t = threadIdx.x;
+    if (t == 0) { carry_a = 0; carry_p = 0; }
+    __syncthreads();
+    // exclusive prefix sums of n and n^2, GEO_THREADS crystals at a time
+    for (int b0 = 0; b0 < P.B; b0 += GEO_THREADS) {
+        const int b = b0 + t;
+        const long long n = b < P.B ? (long long)P.sizes[b] : 0;
+        scan_a[t] = n; scan_p[t] = n * n;
+        __syncthreads();
+        for (int off = 1; off < GEO_THREADS; off <<= 1) {
+            const long long va = t >= off ? scan_a[t - off] : 0, vp = t >= off ? scan_p[t - off] : 0;
+            __syncthreads();
+            scan_a[t] += va; scan_p[t] += vp;
+            __syncthreads();
+        }
+        if (b < P.B) {
+            P.atom_start[b] = carry_a + scan_a[t] - n;
+            P.pair_start[b] = carry_p + scan_p[t] - n * n;
+        }
+        __syncthreads();
+        if (t == GEO_THREADS - 1) { carry_a += scan_a[t]; carry_p += scan_p[t]; }
+        __syncthreads();
+    }
+    if (t == 0) { P.atom_start[P.B] = carry_a; P.pair_start[P.B] = carry_p; }
+
+    // reciprocal lattice (same operation order as the framework expressions it replaces)
+    for (int b = t; b < P.B; b += GEO_THREADS) {
+        const float* m = P.tvecs + (size_t)b * 9;
+        const float v = m[0] * m[4] * m[8] + m[1] * m[5] * m[6] + m[2] * m[3] * m[7] - m[2] * m[4] * m[6]
+                        - m[0] * m[5] * m[7] - m[1] * m[3] * m[8];
+        const float s = (float)(2.0 * 3.14159265358979323846) / v;
+        P.vcell[b] = v;
+        for (int r = 0; r < 3; r++) {
+            const float* u = m + 3 * ((r + 1) % 3);
+            const float* w = m + 3 * ((r + 2) % 3);
+            const float cx = u[1] * w[2] - u[2] * w[1], cy = u[2] * w[0] - u[0] * w[2], cz = u[0] * w[1] - u[1] * w[0];
+            const float rx = cx * s, ry = cy * s, rz = cz * s;
+            P.recip[(size_t)b * 9 + 3 * r + 0] = rx;
+            P.recip[(size_t)b * 9 + 3 * r + 1] = ry;
+            P.recip[(size_t)b * 9 + 3 * r + 2] = rz;
+            P.rvlen[(size_t)b * 3 + r] = sqrtf(rx * rx + ry * ry + rz * rz);
+        }
+    }
+
+    // work order
+    if (P.B <= GEO_THREADS) {
+        // rank by (size descending, crystal ascending): atoms of the crystals ranked before this one
+        const long long n = t < P.B ? (long long)P.sizes[t] : 0;
+        __syncthreads();
+        scan_a[t] = n;
+        __syncthreads();
+        if (t < P.B) {
+            long long before = 0;
+            for (int c = 0; c < P.B; c++) {
+                const long long m = scan_a[c];
+                if (m > n || (m == n && c < t)) before += m;
+            }
+            P.order_start[t] = before;
+        }
+    } else {
+        for (int k = t; k < GEO_KEYS; k += GEO_THREADS) hist[k] = 0;
+        __syncthreads();
+        for (int b = t; b < P.B; b += GEO_THREADS) {
+            const int n = (int)P.sizes[b];
+            atomicAdd(&hist[min(n, GEO_KEYS - 1)], n);
+        }
+        __syncthreads();
+        // hist[k] <- atoms of the crystals with a larger key (suffix sums, serial over 2048 keys by one wavefront)
+        if (t == 0) {
+            int run = 0;
+            for (int k = GEO_KEYS - 1; k >= 0; k--) { const int h = hist[k]; hist[k] = run; run += h; }
+        }
+        __syncthreads();
+        for (int b = t; b < P.B; b += GEO_THREADS) {
+            const int n = (int)P.sizes[b];
+            P.order_start[b] = atomicAdd(&hist[min(n, GEO_KEYS - 1)], n);
+        }
+    }
+}
+
+// One thread per atom: first pair of its row and its place in the work order.
+__global__ __launch_bounds__(256) void geometry_atoms_kernel(const GeometryArgs P) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i == 0) P.e_start[P.N] = P.pair_start[P.B];
+    if (i >= P.N) return;
+    const int b = (int)P.batch[i];
+    const long long n = (long long)P.sizes[b];
+    const long long local = (long long)i - P.atom_start[b];
+    P.e_start[i] = P.pair_start[b] + local * n;
+    P.order[P.order_start[b] + local] = i;
+}
+
+// One thread per pair: its crystal by bisection of the pairs' prefix sums, then (i, j) and the pair vector.
+__global__ __launch_bounds__(256) void geometry_pairs_kernel(const GeometryArgs P) {
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= P.E || e >= P.pair_start[P.B]) return;      // never beyond the pairs that exist
+    int lo = 0, hi = P.B;                       // pair_start[lo] <= e < pair_start[hi]
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (P.pair_start[mid] <= e) lo = mid; else hi = mid;
+    }
+    const long long n = (long long)P.sizes[lo];
+    if (n <= 0) return;
+    const long long local = e - P.pair_start[lo];
+    const long long il = local / n, jl = local - il * n;
+    const long long a0 = P.atom_start[lo];
+    const long long i = a0 + il, j = a0 + jl;
+    P.edges[e] = i;
+    P.edges[P.E + e] = j;
+    P.rpos[e * 3 + 0] = P.pos[j * 3 + 0] - P.pos[i * 3 + 0];
+    P.rpos[e * 3 + 1] = P.pos[j * 3 + 1] - P.pos[i * 3 + 1];
+    P.rpos[e * 3 + 2] = P.pos[j * 3 + 2] - P.pos[i * 3 + 2];
+}
+
+}  // namespace cfh

@@ -234,6 +234,23 @@ int cfh_crystal_mean_backward(const float* gout, const int64_t* batch, const int
                               int64_t N, int64_t B, int64_t C, float* gx, void* stream);
 
 /*
+ * Geometry of a batch of fully connected crystals, shared by all layers of a forward pass: the pairs
+ * (i, j) of every crystal as the complete n x n block, i-major (edges (2,E) int64), pair vectors
+ * rpos (E,3) = pos[j] - pos[i], reciprocal rows recip (B,3,3) = 2 pi (t_b x t_c) / V etc., their lengths
+ * rvlen (B,3), the signed cell volume vcell (B), e_start (N+1) first pair of each atom, atom_start (B+1)
+ * first atom of each crystal and `order` (N) int32, the atoms by descending crystal size (the order
+ * in which the lattice kernels take their items).  batch (N) ascending, sizes (B) atoms per crystal,
+ * E = sum of sizes^2 (known to the caller; e_start[N] holds what the device counted).  workspace:
+ * (2 B + 1) * 8 bytes.  Three launches.  Replaces the framework arithmetic of
+ * models/indexed_latticeformer_encoder.py:15-44 (compute_lattice_distances_for_cuda) and :175-245
+ * (get_edge_index).
+ */
+int cfh_crystal_geometry(const float* pos, const int64_t* batch, const float* tvecs, const int64_t* sizes,
+                         int64_t N, int64_t B, int64_t E, int64_t* edges, float* rpos, float* recip,
+                         float* rvlen, float* vcell, int64_t* e_start, int64_t* atom_start, int32_t* order,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Weight and bias gradients of a projection y = x W^T + b:  dW (O,I) = dy^T x, db (O) = column sums
  * of dy (db may be NULL); x (N,I), dy (N,O), row-major.  One launch (plus a clearing kernel) sized
  * for the shapes of this model, N = atoms in the thousands and I, O in the hundreds, where the

@@ -133,3 +133,30 @@ def test_large_batch_of_small_cells_distance_encoding_only():
     assert torch.equal(torch.cat([psi1, psi2]), psi)
     assert Hh.rel_err(torch.cat([ga1, ga2]), ga) < 1e-6
     assert Hh.rel_err(gW1 + gW2, gW) < 1e-5
+
+
+@pytest.mark.parametrize("num_crystals,atoms_hi", [(256, 40), (1500, 6), (3, 70), (1, 1)])
+def test_geometry_launches_match_framework_expressions(num_crystals, atoms_hi):
+    """cfh_crystal_geometry against the framework arithmetic it replaces: pairs, offsets and pair
+    vectors exactly, the reciprocal lattice to float32 rounding, the work order as a permutation sorted by
+    crystal size (ties in crystal order up to 1024 crystals, any order beyond)."""
+    from crystalframer_amd import geometry, synthetic
+    cb = synthetic.make_batch(num_crystals, atoms="uniform", atoms_lo=1, atoms_hi=atoms_hi, len_lo=3.0, len_hi=9.0,
+                              ang_lo=65.0, ang_hi=115.0, seed=77).to(dev())
+    geometry.USE_LIBRARY = False
+    try:
+        ref = geometry.crystal_geometry(cb.pos, cb.batch, cb.trans_vec, cb.sizes, cb.num_pairs)
+    finally:
+        geometry.USE_LIBRARY = True
+    got = geometry.crystal_geometry(cb.pos, cb.batch, cb.trans_vec, cb.sizes, cb.num_pairs)
+    assert got.num_edges == ref.num_edges == int((cb.sizes ** 2).sum())
+    for name in ("edges", "e_start", "atom_start", "rpos"):
+        assert torch.equal(getattr(got, name), getattr(ref, name)), name
+    for name in ("vcell", "recip", "rvlen"):          # float32 rounding of the cross products may differ
+        assert Hh.rel_err(getattr(got, name), getattr(ref, name)) < 1e-6, name
+    n_of_atom = cb.sizes.to(dev())[cb.batch]
+    order = got.order.long()
+    assert torch.equal(torch.sort(order).values, torch.arange(order.numel(), device=dev()))
+    assert (n_of_atom[order][:-1] >= n_of_atom[order][1:]).all()
+    if num_crystals <= 1024:
+        assert torch.equal(got.order, ref.order)
