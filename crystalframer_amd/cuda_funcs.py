@@ -130,6 +130,15 @@ def seed_edge_schedule(edge_ij_e: torch.Tensor, e_start: torch.Tensor, order: to
                        val=(e_start.contiguous(), order.to(torch.int32).contiguous()))
 
 
+_atom_start_cache = {"ref": None, "version": None, "val": None}
+
+
+def seed_atom_start(sizes: torch.Tensor, atom_start: torch.Tensor):
+    """Hand over the (B+1) exclusive prefix sums already known for ``sizes`` (geometry.py computes them);
+    the per-crystal mean of the same batch then needs no scan of its own."""
+    _atom_start_cache.update(ref=weakref.ref(sizes), version=sizes._version, val=atom_start)
+
+
 def edge_schedule(edge_ij_e: torch.Tensor, N: int):
     """(e_start (N+1) int64, order (N) int32) for an edge list whose edges are grouped by query atom.
 
@@ -449,7 +458,12 @@ class IrregularMeanCUDA(torch.autograd.Function):
         B = sizes.shape[0]
         N = x_ik.shape[0]
         C = x_ik[0].numel() if N else int(torch.tensor(x_ik.shape[1:]).prod())
-        atom_start = torch.nn.functional.pad(sizes.to(device=dev, dtype=torch.long).cumsum(0), (1, 0))
+        c = _atom_start_cache
+        if (c["ref"] is not None and c["ref"]() is sizes and c["version"] == sizes._version
+                and c["val"].device == dev and c["val"].shape[0] == B + 1):
+            atom_start = c["val"]
+        else:
+            atom_start = torch.nn.functional.pad(sizes.to(device=dev, dtype=torch.long).cumsum(0), (1, 0))
         x = _f32c(x_ik)
         out = torch.empty((B,) + tuple(x_ik.shape[1:]), dtype=torch.float32, device=dev)
         with _timed("crystal_mean_forward", dev):
