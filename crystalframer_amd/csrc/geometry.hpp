@@ -39,15 +39,16 @@ __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const Ge
     __shared__ long long carry_a, carry_p;
     __shared__ int hist[GEO_KEYS];
     const int t = threadIdx.x;
+    const int T = blockDim.x;              // a power of two, 64 .. GEO_THREADS: no more than the crystals need
     if (t == 0) { carry_a = 0; carry_p = 0; }
     __syncthreads();
     // exclusive prefix sums of n and n^2, GEO_THREADS crystals at a time
-    for (int b0 = 0; b0 < P.B; b0 += GEO_THREADS) {
+    for (int b0 = 0; b0 < P.B; b0 += T) {
         const int b = b0 + t;
         const long long n = b < P.B ? (long long)P.sizes[b] : 0;
         scan_a[t] = n; scan_p[t] = n * n;
         __syncthreads();
-        for (int off = 1; off < GEO_THREADS; off <<= 1) {
+        for (int off = 1; off < T; off <<= 1) {
             const long long va = t >= off ? scan_a[t - off] : 0, vp = t >= off ? scan_p[t - off] : 0;
             __syncthreads();
             scan_a[t] += va; scan_p[t] += vp;
@@ -58,13 +59,13 @@ __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const Ge
             P.pair_start[b] = carry_p + scan_p[t] - n * n;
         }
         __syncthreads();
-        if (t == GEO_THREADS - 1) { carry_a += scan_a[t]; carry_p += scan_p[t]; }
+        if (t == T - 1) { carry_a += scan_a[t]; carry_p += scan_p[t]; }
         __syncthreads();
     }
     if (t == 0) { P.atom_start[P.B] = carry_a; P.pair_start[P.B] = carry_p; }
 
     // reciprocal lattice (same operation order as the framework expressions it replaces)
-    for (int b = t; b < P.B; b += GEO_THREADS) {
+    for (int b = t; b < P.B; b += T) {
         const float* m = P.tvecs + (size_t)b * 9;
         const float v = m[0] * m[4] * m[8] + m[1] * m[5] * m[6] + m[2] * m[3] * m[7] - m[2] * m[4] * m[6]
                         - m[0] * m[5] * m[7] - m[1] * m[3] * m[8];
@@ -83,7 +84,7 @@ __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const Ge
     }
 
     // work order
-    if (P.B <= GEO_THREADS) {
+    if (P.B <= T) {
         // rank by (size descending, crystal ascending): atoms of the crystals ranked before this one
         const long long n = t < P.B ? (long long)P.sizes[t] : 0;
         __syncthreads();
@@ -98,9 +99,9 @@ __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const Ge
             P.order_start[t] = before;
         }
     } else {
-        for (int k = t; k < GEO_KEYS; k += GEO_THREADS) hist[k] = 0;
+        for (int k = t; k < GEO_KEYS; k += T) hist[k] = 0;
         __syncthreads();
-        for (int b = t; b < P.B; b += GEO_THREADS) {
+        for (int b = t; b < P.B; b += T) {
             const int n = (int)P.sizes[b];
             atomicAdd(&hist[min(n, GEO_KEYS - 1)], n);
         }
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const Ge
             for (int k = GEO_KEYS - 1; k >= 0; k--) { const int h = hist[k]; hist[k] = run; run += h; }
         }
         __syncthreads();
-        for (int b = t; b < P.B; b += GEO_THREADS) {
+        for (int b = t; b < P.B; b += T) {
             const int n = (int)P.sizes[b];
             P.order_start[b] = atomicAdd(&hist[min(n, GEO_KEYS - 1)], n);
         }
