@@ -278,18 +278,15 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
                         const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
                         d2r[k] = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
                     }
+                    uint32_t bits = 0u;
 #pragma unroll
                     for (int k = 0; k < 8; k++) {
-                        const int u = tl + 16 * k;
-                        const bool valid = active && u < cnt;
+                        const bool valid = active && tl + 16 * k < cnt;
                         const float ex = fmaf(a2, d2r[k], -z2);
                         Ap += valid ? hw_exp2(ex) * d2r[k] : 0.0f;
-                        const bool keep = valid && ex >= prune;
-                        const uint64_t m = __ballot(keep);
-                        const int pos = seen + lane_prefix(m) - skip;
-                        if (keep && pos >= 0 && pos < room) list[nlist + pos] = (uint16_t)((el << BWD_SHIFT) | u);
-                        seen += __popcll(m);
+                        bits |= (valid && ex >= prune) ? (1u << k) : 0u;
                     }
+                    seen = append_flagged(list, nlist, room, skip, bits, slot, (uint32_t)((el << BWD_SHIFT) | tl));
                 } else {
                     for (int u0 = 0; u0 < cnt; u0 += 16) {
                         const int u = u0 + tl;
