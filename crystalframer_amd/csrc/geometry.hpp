@@ -30,9 +30,9 @@ struct GeometryArgs {
 constexpr int GEO_THREADS = 1024;
 constexpr int GEO_KEYS = 2048;      // crystals of GEO_KEYS - 1 atoms or more share the first place of the order
 
-// One workgroup: prefix sums over the crystals, the reciprocal lattice, and where each crystal's atoms
-// go in the work order (descending size; equal sizes in crystal order when B <= GEO_THREADS, in the
-// order their atomics happen to arrive otherwise).
+// Two workgroups.  The second computes the reciprocal lattice; the first the prefix sums over the
+// crystals and where each crystal's atoms go in the work order (descending size; equal sizes in crystal
+// order when B <= its size, in the order their atomics happen to arrive otherwise).
 #pragma clang fp contract(off)      // the framework expressions this replaces round every product and sum
 __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const GeometryArgs P) {
     __shared__ long long scan_a[GEO_THREADS], scan_p[GEO_THREADS];
@@ -40,12 +40,34 @@ __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const Ge
     __shared__ int hist[GEO_KEYS];
     const int t = threadIdx.x;
     const int T = blockDim.x;              // a power of two, 64 .. GEO_THREADS: no more than the crystals need
+    if (blockIdx.x == 1) {
+        // reciprocal lattice (same operation order as the framework expressions it replaces)
+        for (int b = t; b < P.B; b += T) {
+            const float* m = P.tvecs + (size_t)b * 9;
+            const float v = m[0] * m[4] * m[8] + m[1] * m[5] * m[6] + m[2] * m[3] * m[7] - m[2] * m[4] * m[6]
+                            - m[0] * m[5] * m[7] - m[1] * m[3] * m[8];
+            const float s = (float)(2.0 * 3.14159265358979323846) / v;
+            P.vcell[b] = v;
+            for (int r = 0; r < 3; r++) {
+                const float* u = m + 3 * ((r + 1) % 3);
+                const float* w = m + 3 * ((r + 2) % 3);
+                const float cx = u[1] * w[2] - u[2] * w[1], cy = u[2] * w[0] - u[0] * w[2], cz = u[0] * w[1] - u[1] * w[0];
+                const float rx = cx * s, ry = cy * s, rz = cz * s;
+                P.recip[(size_t)b * 9 + 3 * r + 0] = rx;
+                P.recip[(size_t)b * 9 + 3 * r + 1] = ry;
+                P.recip[(size_t)b * 9 + 3 * r + 2] = rz;
+                P.rvlen[(size_t)b * 3 + r] = sqrtf(rx * rx + ry * ry + rz * rz);
+            }
+        }
+        return;
+    }
+    const long long n_first = t < P.B ? (long long)P.sizes[t] : 0;      // the first T sizes: used twice below
     if (t == 0) { carry_a = 0; carry_p = 0; }
     __syncthreads();
     // exclusive prefix sums of n and n^2, GEO_THREADS crystals at a time
     for (int b0 = 0; b0 < P.B; b0 += T) {
         const int b = b0 + t;
-        const long long n = b < P.B ? (long long)P.sizes[b] : 0;
+        const long long n = b0 == 0 ? n_first : (b < P.B ? (long long)P.sizes[b] : 0);
         scan_a[t] = n; scan_p[t] = n * n;
         __syncthreads();
         for (int off = 1; off < T; off <<= 1) {
@@ -64,39 +86,23 @@ __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const Ge
     }
     if (t == 0) { P.atom_start[P.B] = carry_a; P.pair_start[P.B] = carry_p; }
 
-    // reciprocal lattice (same operation order as the framework expressions it replaces)
-    for (int b = t; b < P.B; b += T) {
-        const float* m = P.tvecs + (size_t)b * 9;
-        const float v = m[0] * m[4] * m[8] + m[1] * m[5] * m[6] + m[2] * m[3] * m[7] - m[2] * m[4] * m[6]
-                        - m[0] * m[5] * m[7] - m[1] * m[3] * m[8];
-        const float s = (float)(2.0 * 3.14159265358979323846) / v;
-        P.vcell[b] = v;
-        for (int r = 0; r < 3; r++) {
-            const float* u = m + 3 * ((r + 1) % 3);
-            const float* w = m + 3 * ((r + 2) % 3);
-            const float cx = u[1] * w[2] - u[2] * w[1], cy = u[2] * w[0] - u[0] * w[2], cz = u[0] * w[1] - u[1] * w[0];
-            const float rx = cx * s, ry = cy * s, rz = cz * s;
-            P.recip[(size_t)b * 9 + 3 * r + 0] = rx;
-            P.recip[(size_t)b * 9 + 3 * r + 1] = ry;
-            P.recip[(size_t)b * 9 + 3 * r + 2] = rz;
-            P.rvlen[(size_t)b * 3 + r] = sqrtf(rx * rx + ry * ry + rz * rz);
-        }
-    }
-
     // work order
     if (P.B <= T) {
         // rank by (size descending, crystal ascending): atoms of the crystals ranked before this one
-        const long long n = t < P.B ? (long long)P.sizes[t] : 0;
+        const int n = (int)n_first;
+        int* const sz = reinterpret_cast<int*>(scan_p);
         __syncthreads();
-        scan_a[t] = n;
+        sz[t] = n;
         __syncthreads();
         if (t < P.B) {
-            long long before = 0;
-            for (int c = 0; c < P.B; c++) {
-                const long long m = scan_a[c];
-                if (m > n || (m == n && c < t)) before += m;
+            int before0 = 0, before1 = 0;
+            for (int c = 0; c + 1 < P.B; c += 2) {
+                const int m0 = sz[c], m1 = sz[c + 1];
+                before0 += (m0 > n || (m0 == n && c < t)) ? m0 : 0;
+                before1 += (m1 > n || (m1 == n && c + 1 < t)) ? m1 : 0;
             }
-            P.order_start[t] = before;
+            if (P.B & 1) { const int m = sz[P.B - 1]; before0 += (m > n || (m == n && P.B - 1 < t)) ? m : 0; }
+            P.order_start[t] = (long long)before0 + before1;
         }
     } else {
         for (int k = t; k < GEO_KEYS; k += T) hist[k] = 0;
