@@ -126,3 +126,40 @@ def test_vectorised_frame_oracle_matches_loop_oracle():
     f1, f2 = TO.frame_axes_max(P.q, P.k, P.a, P.rpos, P.tvecs, P.batch, P.edges, rvlen=P.rvlen, cutoff_radius=-3.5)
     g1, g2 = TO.frame_axes_max_vec(P.q, P.k, P.a, P.rpos, P.tvecs, P.batch, P.edges, rvlen=P.rvlen, cutoff_radius=-3.5)
     assert (f1 - g1).abs().max() < 1e-12 and (f2 - g2).abs().max() < 1e-12
+
+
+def test_input_projection_weights_share_one_storage_without_changing_the_parameters():
+    """The attention layer keeps q/k/v_proj_weight as adjacent row blocks of one matrix (the stacked
+    projection then needs no concatenation).  Names, shapes and values stay the reference's; an
+    optimizer step on the three parameters is seen through the stack; moving the module re-establishes it."""
+    from crystalframer_amd import attention, params
+    lat = params.LatticeformerParams()
+    torch.manual_seed(3)
+    m = attention.CrystalformerMultiheadAttentionCUDA(128, 8, params=lat)
+    before = {k: v.clone() for k, v in m.state_dict().items()}
+    st = m._stacked_in_proj()
+    assert st.shape == (384, 128)
+    assert m.q_proj_weight.data_ptr() == st.data_ptr()
+    assert m.k_proj_weight.data_ptr() == st.data_ptr() + 128 * 128 * 4
+    assert m.v_proj_weight.data_ptr() == st.data_ptr() + 2 * 128 * 128 * 4
+    after = m.state_dict()
+    assert list(after.keys()) == list(before.keys())
+    for k in before:
+        assert torch.equal(after[k], before[k]), k
+    assert {n for n, _ in m.named_parameters()} >= {"q_proj_weight", "k_proj_weight", "v_proj_weight"}
+    assert m._stacked_in_proj() is st                      # nothing to redo
+    opt = torch.optim.SGD([m.q_proj_weight, m.k_proj_weight, m.v_proj_weight], lr=0.5)
+    for p in (m.q_proj_weight, m.k_proj_weight, m.v_proj_weight):
+        p.grad = torch.ones_like(p)
+    opt.step()
+    assert torch.equal(st[:128], before["q_proj_weight"] - 0.5)
+    assert torch.equal(st[256:], before["v_proj_weight"] - 0.5)
+    m2 = m.double()                                         # new storages per parameter
+    st2 = m2._stacked_in_proj()
+    assert st2.dtype == torch.float64 and st2 is not st
+    assert torch.equal(st2[128:256], m2.k_proj_weight) and m2.k_proj_weight.data_ptr() == st2.data_ptr() + 128 * 128 * 8
+    sd = {k: v.clone() for k, v in m2.state_dict().items()}
+    m3 = attention.CrystalformerMultiheadAttentionCUDA(128, 8, params=lat).double()
+    m3._stacked_in_proj()
+    m3.load_state_dict(sd)                                  # copies into the shared storage
+    assert torch.equal(m3._stacked_in_proj()[:128], sd["q_proj_weight"])
