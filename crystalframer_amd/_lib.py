@@ -59,7 +59,7 @@ EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_fram
            "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_backward",
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
            "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
-           "cfh_crystal_geometry", "cfh_linear_weight_bias_grad", "cfh_linear_weight_bias_grad_batch", "cfh_attention_inputs_forward",
+           "cfh_crystal_geometry", "cfh_small_linear_forward", "cfh_small_linear_dx", "cfh_linear_weight_bias_grad", "cfh_linear_weight_bias_grad_batch", "cfh_attention_inputs_forward",
            "cfh_attention_inputs_backward")
 
 _lib = None
@@ -111,6 +111,10 @@ def load():
         lib.cfh_crystal_mean_backward.argtypes = [_P, _P, _P, _I64, _I64, _I64, _P, _P]
         lib.cfh_linear_weight_bias_grad.restype = ctypes.c_int
         lib.cfh_linear_weight_bias_grad.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P, _P]
+        lib.cfh_small_linear_forward.restype = ctypes.c_int
+        lib.cfh_small_linear_forward.argtypes = [_P, _P, _P, _I64, _I64, _I64, ctypes.c_int32, _P, _P]
+        lib.cfh_small_linear_dx.restype = ctypes.c_int
+        lib.cfh_small_linear_dx.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P]
         lib.cfh_crystal_geometry.restype = ctypes.c_int
         lib.cfh_crystal_geometry.argtypes = [_P, _P, _P, _P, _I64, _I64, _I64] + [_P] * 8 + [_P, ctypes.c_size_t, _P]
         lib.cfh_linear_weight_bias_grad_batch.restype = ctypes.c_int

@@ -22,6 +22,7 @@
 #include "fused_dpa.hpp"
 #include "geometry.hpp"
 #include "linear_grad.hpp"
+#include "small_gemm.hpp"
 
 namespace {
 
@@ -679,7 +680,31 @@ int cfh_crystal_geometry(const float* pos, const int64_t* batch, const float* tv
     return finish_launch("crystal_geometry");
 }
 
+int cfh_small_linear_forward(const float* x, const float* W, const float* b, int64_t M, int64_t N, int64_t K,
+                             int32_t relu, float* y, void* stream) {
+    if (M < 0 || N < 1 || K < 16 || K % 16 != 0 || M > 0x7fffffffLL / 64 || N > 65536 || K > 65536)
+        return fail(CFH_EINVAL, "small linear forward: M=%lld N=%lld K=%lld (K must be a multiple of 16)", (long long)M,
+                    (long long)N, (long long)K);
+    if (M == 0) return CFH_OK;
+    if (!x || !W || !y || (((uintptr_t)x | (uintptr_t)W) & 15)) return fail(CFH_EINVAL, "x, W, y must not be NULL; x, W 16-byte aligned");
+    hipLaunchKernelGGL(cfh::small_linear_fwd_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((N + 63) / 64)), dim3(256), 0,
+                       (hipStream_t)stream, x, W, b, y, (int)M, (int)N, (int)K, (int)relu);
+    return finish_launch("small_linear_forward");
+}
+
+int cfh_small_linear_dx(const float* dy, const float* W, int64_t M, int64_t N, int64_t K, float* dx, void* stream) {
+    if (M < 0 || K < 1 || N < 16 || N % 16 != 0 || M > 0x7fffffffLL / 64 || N > 65536 || K > 65536)
+        return fail(CFH_EINVAL, "small linear dx: M=%lld N=%lld K=%lld (N must be a multiple of 16)", (long long)M,
+                    (long long)N, (long long)K);
+    if (M == 0) return CFH_OK;
+    if (!dy || !W || !dx || ((uintptr_t)dy & 15)) return fail(CFH_EINVAL, "dy, W, dx must not be NULL; dy 16-byte aligned");
+    hipLaunchKernelGGL(cfh::small_linear_dx_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((K + 63) / 64)), dim3(256), 0,
+                       (hipStream_t)stream, dy, W, dx, (int)M, (int)N, (int)K);
+    return finish_launch("small_linear_dx");
+}
+
 }  // extern "C"
+
 
 
 

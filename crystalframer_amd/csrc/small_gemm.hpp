@@ -1,0 +1,102 @@
+// Projections with FEW rows (the pooled features of a batch: one row per crystal).  The library GEMM
+// the framework calls runs such a product on one or two workgroups (20 us for 256 x 128 x 128); here a
+// wavefront owns a 32x32 block of the result, so even 256 rows give dozens of wavefronts, and bias,
+// rectifier and the layout of the weight (O, I) as torch.nn.Linear stores it are handled in place.
+//   forward   y (M,N) = x (M,K) W^T + b, W (N,K)           (reference: torch.nn.functional.linear)
+//   backward  dx (M,K) = dy (M,N) W
+#pragma once
+#include "device_common.hpp"
+
+namespace cfh {
+
+typedef float v4f_g __attribute__((ext_vector_type(4)));
+
+// lane (kk, col) of a wavefront: A operand A[m = col][k = kk], B operand B[k = kk][n = col]; a 16-wide step
+// of the reduction index is four MFMA 16x16x4 with k = 4 kk + j, j = 0..3, so that a lane reads 4
+// consecutive floats of its row.
+// grid: (ceil(M/64), ceil(N/64)), block 256 = 4 wavefronts, wavefront w: rows 32 (w/2), columns 32 (w%2).
+// K % 16 == 0, rows 16-byte aligned.
+__global__ __launch_bounds__(256) void small_linear_fwd_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                               const float* __restrict__ b, float* __restrict__ y,
+                                                               int M, int N, int K, int relu) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int col = lane & 15, kk = lane >> 4;
+    const int m0 = blockIdx.x * 64 + 32 * (wv >> 1), n0 = blockIdx.y * 64 + 32 * (wv & 1);
+    if (m0 >= M || n0 >= N) return;
+    const int ra = min(m0 + col, M - 1), rb = min(m0 + 16 + col, M - 1);
+    const int ca = min(n0 + col, N - 1), cb = min(n0 + 16 + col, N - 1);
+    const float4* xa = reinterpret_cast<const float4*>(x + (size_t)ra * K) + kk;
+    const float4* xb = reinterpret_cast<const float4*>(x + (size_t)rb * K) + kk;
+    const float4* wa = reinterpret_cast<const float4*>(w + (size_t)ca * K) + kk;
+    const float4* wb = reinterpret_cast<const float4*>(w + (size_t)cb * K) + kk;
+    v4f_g acc00 = {0.f, 0.f, 0.f, 0.f}, acc01 = acc00, acc10 = acc00, acc11 = acc00;
+    const int chunks = K / 16;
+#pragma unroll 4
+    for (int c = 0; c < chunks; c++) {
+        const float4 a0 = xa[4 * c], a1 = xb[4 * c], b0 = wa[4 * c], b1 = wb[4 * c];
+        const float A0[4] = {a0.x, a0.y, a0.z, a0.w}, A1[4] = {a1.x, a1.y, a1.z, a1.w};
+        const float B0[4] = {b0.x, b0.y, b0.z, b0.w}, B1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            acc00 = __builtin_amdgcn_mfma_f32_16x16x4f32(A0[j], B0[j], acc00, 0, 0, 0);
+            acc01 = __builtin_amdgcn_mfma_f32_16x16x4f32(A0[j], B1[j], acc01, 0, 0, 0);
+            acc10 = __builtin_amdgcn_mfma_f32_16x16x4f32(A1[j], B0[j], acc10, 0, 0, 0);
+            acc11 = __builtin_amdgcn_mfma_f32_16x16x4f32(A1[j], B1[j], acc11, 0, 0, 0);
+        }
+    }
+    // accumulator component c of lane (kk, col): row 4 kk + c of the 16x16 block, column col
+    const float ba = b ? b[ca] : 0.f, bb = b ? b[cb] : 0.f;
+    auto put = [&](int r, int n, float v) {
+        if (r < M && n < N) y[(size_t)r * N + n] = relu ? fmaxf(v, 0.f) : v;
+    };
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const int r0 = m0 + 4 * kk + c;
+        put(r0, n0 + col, acc00[c] + ba);
+        put(r0, n0 + 16 + col, acc01[c] + bb);
+        put(r0 + 16, n0 + col, acc10[c] + ba);
+        put(r0 + 16, n0 + 16 + col, acc11[c] + bb);
+    }
+}
+
+// dx (M,K) = dy (M,N) W, W (N,K).  grid: (ceil(M/64), ceil(K/64)); N % 16 == 0, rows of dy 16-byte aligned.
+__global__ __launch_bounds__(256) void small_linear_dx_kernel(const float* __restrict__ dy, const float* __restrict__ w,
+                                                              float* __restrict__ dx, int M, int N, int K) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int col = lane & 15, kk = lane >> 4;
+    const int m0 = blockIdx.x * 64 + 32 * (wv >> 1), k0 = blockIdx.y * 64 + 32 * (wv & 1);
+    if (m0 >= M || k0 >= K) return;
+    const int ra = min(m0 + col, M - 1), rb = min(m0 + 16 + col, M - 1);
+    const int ca = min(k0 + col, K - 1), cb = min(k0 + 16 + col, K - 1);
+    const float4* ya = reinterpret_cast<const float4*>(dy + (size_t)ra * N) + kk;
+    const float4* yb = reinterpret_cast<const float4*>(dy + (size_t)rb * N) + kk;
+    v4f_g acc00 = {0.f, 0.f, 0.f, 0.f}, acc01 = acc00, acc10 = acc00, acc11 = acc00;
+    const int chunks = N / 16;
+#pragma unroll 2
+    for (int c = 0; c < chunks; c++) {
+        const float4 a0 = ya[4 * c], a1 = yb[4 * c];
+        const float A0[4] = {a0.x, a0.y, a0.z, a0.w}, A1[4] = {a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float* wr = w + (size_t)(16 * c + 4 * kk + j) * K;      // row n = 16 c + 4 kk + j of W
+            const float b0 = wr[ca], b1 = wr[cb];
+            acc00 = __builtin_amdgcn_mfma_f32_16x16x4f32(A0[j], b0, acc00, 0, 0, 0);
+            acc01 = __builtin_amdgcn_mfma_f32_16x16x4f32(A0[j], b1, acc01, 0, 0, 0);
+            acc10 = __builtin_amdgcn_mfma_f32_16x16x4f32(A1[j], b0, acc10, 0, 0, 0);
+            acc11 = __builtin_amdgcn_mfma_f32_16x16x4f32(A1[j], b1, acc11, 0, 0, 0);
+        }
+    }
+    auto put = [&](int r, int n, float v) {
+        if (r < M && n < K) dx[(size_t)r * K + n] = v;
+    };
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const int r0 = m0 + 4 * kk + c;
+        put(r0, k0 + col, acc00[c]);
+        put(r0, k0 + 16 + col, acc01[c]);
+        put(r0 + 16, k0 + col, acc10[c]);
+        put(r0 + 16, k0 + 16 + col, acc11[c]);
+    }
+}
+
+}  // namespace cfh

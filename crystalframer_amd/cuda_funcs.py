@@ -589,6 +589,8 @@ class LinearHIP(torch.autograd.Function):
     leaf parameters deferred to one launch per backward pass (see _DeferredWeightGrads), otherwise
     one launch here.  Same values as torch.nn.functional.linear up to the order of the float32 sums."""
 
+    SMALL_ROWS = 512        # up to this many rows the library's small-projection kernels replace the GEMMs
+
     @staticmethod
     def forward(ctx, x, bias, stacked, relu, *weights):
         if stacked is not None:
@@ -600,6 +602,28 @@ class LinearHIP(torch.autograd.Function):
         ctx.weights = weights
         ctx.bias = bias
         ctx.relu = bool(relu)
+        rows = x.numel() // max(W.shape[1], 1)
+        ctx.small = (0 < rows <= LinearHIP.SMALL_ROWS and x.dtype == torch.float32 and W.dtype == torch.float32
+                     and (bias is None or bias.dtype == torch.float32))
+        if ctx.small and W.shape[1] % 16 == 0:
+            # few rows (one per crystal): the library's own kernel, which does not leave the product to
+            # one or two workgroups
+            lib = _lib.load()
+            x2 = _f32c(x.reshape(rows, W.shape[1]))
+            Wc = _f32c(W)
+            bc = None if bias is None else _f32c(bias)
+            y = torch.empty((rows, W.shape[0]), dtype=torch.float32, device=x.device)
+            with torch.cuda.device(x.device), _timed("small_linear_forward", x.device):
+                rc = lib.cfh_small_linear_forward(_lib.ptr(x2), _lib.ptr(Wc), _lib.ptr(bc), rows, W.shape[0], W.shape[1],
+                                                  1 if relu else 0, _lib.ptr(y), _lib.current_stream_ptr(x.device))
+            _lib.check(rc, "cfh_small_linear_forward")
+            if x.dim() != 2:
+                y = y.reshape(*x.shape[:-1], W.shape[0])
+            if relu:
+                ctx.save_for_backward(x, Wc, y)
+            else:
+                ctx.save_for_backward(x, Wc)
+            return y
         if relu:
             # bias and rectifier in the epilogue of the library GEMM
             x2 = x.reshape(-1, W.shape[1])
@@ -607,7 +631,8 @@ class LinearHIP(torch.autograd.Function):
                 y = torch._addmm_activation(bias.detach(), x2, W.detach().t(), use_gelu=False)
             else:
                 y = torch.relu(x2.matmul(W.detach().t()))
-            y = y.reshape(*x.shape[:-1], W.shape[0])
+            if x.dim() != 2:
+                y = y.reshape(*x.shape[:-1], W.shape[0])
             ctx.save_for_backward(x, W.detach(), y)
             return y
         ctx.save_for_backward(x, W.detach())
@@ -621,7 +646,20 @@ class LinearHIP(torch.autograd.Function):
         else:
             x, W = ctx.saved_tensors
         weights, bias = ctx.weights, ctx.bias
-        gx = gy.matmul(W) if ctx.needs_input_grad[0] else None
+        gx = None
+        if ctx.needs_input_grad[0]:
+            if ctx.small and W.shape[0] % 16 == 0 and gy.dtype == torch.float32:
+                lib = _lib.load()
+                rows = gy.numel() // W.shape[0]
+                g2c = _f32c(gy.reshape(rows, W.shape[0]))
+                gx = torch.empty((rows, W.shape[1]), dtype=torch.float32, device=gy.device)
+                with torch.cuda.device(gy.device), _timed("small_linear_dx", gy.device):
+                    rc = lib.cfh_small_linear_dx(_lib.ptr(g2c), _lib.ptr(_f32c(W)), rows, W.shape[0], W.shape[1],
+                                                 _lib.ptr(gx), _lib.current_stream_ptr(gy.device))
+                _lib.check(rc, "cfh_small_linear_dx")
+                gx = gx.reshape(x.shape)
+            else:
+                gx = gy.matmul(W)
         need_w = [ctx.needs_input_grad[4 + n] for n in range(len(weights))]
         need_b = bias is not None and ctx.needs_input_grad[1]
         if not (any(need_w) or need_b):

@@ -29,6 +29,26 @@ def avr_pool(x, batch, sizes):
     return cuda_funcs.IrregularMeanCUDA.apply(x, batch, sizes)
 
 
+def _run_head(module: nn.Module, x: torch.Tensor) -> torch.Tensor:
+    """``module(x)`` for the Identity / Linear / norm / ReLU stacks of the model's head, with every Linear
+    (and a ReLU that follows it directly) going through ``cuda_funcs.linear``: same arithmetic, weight
+    gradients in the batched launch, few-row products in the library's own kernel."""
+    if not isinstance(module, nn.Sequential):
+        return module(x)
+    mods = [m for m in module if not isinstance(m, nn.Identity)]
+    n = 0
+    while n < len(mods):
+        m = mods[n]
+        if isinstance(m, nn.Linear) and x.is_cuda:
+            fuse = n + 1 < len(mods) and isinstance(mods[n + 1], nn.ReLU)
+            x = cuda_funcs.linear(x, m.weight, m.bias, relu=fuse)
+            n += 2 if fuse else 1
+        else:
+            x = m(x)
+            n += 1
+    return x
+
+
 class Latticeformer(nn.Module):
     def __init__(self, params: ModelParams = None):
         super().__init__()
@@ -85,6 +105,6 @@ class Latticeformer(nn.Module):
         num_pairs = getattr(data, "num_pairs", -1)
         x = self.encoder(x, data.pos, data.batch, data.trans_vec, data.sizes, this_epoch=this_epoch,
                          num_pairs=num_pairs if num_pairs is not None and num_pairs >= 0 else None)
-        x = self.proj_before_pooling(x)
+        x = _run_head(self.proj_before_pooling, x)
         x = self.pooling_layer(x, data.batch, data.sizes)
-        return self.mlp(x)
+        return _run_head(self.mlp, x)

@@ -281,6 +281,17 @@ typedef struct cfh_linear_grad_job {
 int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t njobs, void* stream);
 
 /*
+ * Projections with few rows (one per crystal: the head after pooling), where the general GEMM runs on
+ * one or two workgroups:  y (M,N) = x (M,K) W^T + b with W (N,K) as torch.nn.Linear stores it, b (N) or
+ * NULL, relu != 0: max(0, .);  dx (M,K) = dy (M,N) W.  Contiguous float32; K % 16 == 0 for the forward,
+ * N % 16 == 0 for dx.  Replace torch.nn.functional.linear and its input gradient (models/latticeformer.py,
+ * the MLP head after pooling).
+ */
+int cfh_small_linear_forward(const float* x, const float* W, const float* b, int64_t M, int64_t N, int64_t K,
+                             int32_t relu, float* y, void* stream);
+int cfh_small_linear_dx(const float* dy, const float* W, int64_t M, int64_t N, int64_t K, float* dx, void* stream);
+
+/*
  * What lies between the stacked q/k/v projection of a layer and its kernels, one launch each way.
  * Forward: qkv (N, 3 H Dh), rows = [query | key | value];  qs = query * q_scale, k, v (N,H,Dh) contiguous,
  *   a (N,H) = ((1 - lb) elu(c1 alpha') + 1) c2  with alpha = query_h . lattice_w_h and

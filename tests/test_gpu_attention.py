@@ -287,3 +287,38 @@ def test_linear_deferred_gradients_stacked_accumulated_and_nonleaf():
         KM.DEFER_WEIGHT_GRADS = True
     for t32, t64 in zip(leaves, leaves64):
         assert Hh.rel_err(t32.grad, t64.grad) < 2e-5
+
+
+@pytest.mark.parametrize("M,I,O,bias,relu", [(256, 128, 128, True, True), (256, 128, 1, True, False), (37, 48, 20, False, False),
+                                             (512, 64, 96, True, True), (1, 16, 16, True, False)])
+def test_few_row_projection_kernels(M, I, O, bias, relu):
+    """Projections with few rows take the library's own forward / input-gradient kernels: against
+    float64 autograd of relu(x W^T + b)."""
+    import crystalframer_amd as cf
+    gen = torch.Generator().manual_seed(M + I + O)
+    x64 = torch.randn(M, I, generator=gen, dtype=torch.float64, requires_grad=True)
+    w64 = torch.randn(O, I, generator=gen, dtype=torch.float64, requires_grad=True)
+    b64 = torch.randn(O, generator=gen, dtype=torch.float64, requires_grad=True) if bias else None
+    gy = torch.randn(M, O, generator=gen, dtype=torch.float64)
+    y64 = torch.nn.functional.linear(x64, w64, b64)
+    if relu:
+        y64 = torch.relu(y64)
+    (y64 * gy).sum().backward()
+    x = f32(x64.detach()).requires_grad_(True)
+    w = f32(w64.detach()).requires_grad_(True)
+    b = f32(b64.detach()).requires_grad_(True) if bias else None
+    events = []
+    cf.KernelManager.EVENT_LOG = events
+    try:
+        y = cf.cuda_funcs.linear(x, w, b, relu=relu)
+        (y * f32(gy)).sum().backward()
+    finally:
+        cf.KernelManager.EVENT_LOG = None
+    names = {e[0] for e in events}
+    assert "small_linear_forward" in names                      # the library kernels were the ones that ran
+    assert ("small_linear_dx" in names) == (O % 16 == 0)
+    assert Hh.rel_err(y, y64) < 1e-5
+    assert Hh.rel_err(x.grad, x64.grad) < 1e-5
+    assert Hh.rel_err(w.grad, w64.grad) < 1e-5
+    if bias:
+        assert Hh.rel_err(b.grad, b64.grad) < 1e-5
