@@ -163,3 +163,14 @@ def test_input_projection_weights_share_one_storage_without_changing_the_paramet
     m3._stacked_in_proj()
     m3.load_state_dict(sd)                                  # copies into the shared storage
     assert torch.equal(m3._stacked_in_proj()[:128], sd["q_proj_weight"])
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it says so and exits without touching a device."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr
+    assert r.stdout.strip() == ""
