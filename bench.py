@@ -92,7 +92,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (crystals would be sharded "
-              "data-parallel, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+              "data-parallel, whole crystals per GPU, gradients all-reduced); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py needs a HIP device", file=sys.stderr)
