@@ -595,7 +595,7 @@ int cfh_attention_inputs_backward(const float* qkv, const float* lattice_w, cons
                                   void* stream) {
     cfh::AttnInArgs A;
     if (int rc = attention_inputs_args(A, qkv, lattice_w, gauss_scale_dev, c1, lb, c2, q_scale, N, H, Dh)) return rc;
-    if (!g_lattice_w || (N > 0 && !gqkv)) return fail(CFH_EINVAL, "gqkv and g_lattice_w must not be NULL");
+    if (N > 0 && !gqkv) return fail(CFH_EINVAL, "gqkv must not be NULL");
     hipStream_t st = (hipStream_t)stream;
     A.rows_per_block = 4 * (256 / A.HD);
     const int blocks = (int)((N + A.rows_per_block - 1) / A.rows_per_block);
@@ -605,8 +605,9 @@ int cfh_attention_inputs_backward(const float* qkv, const float* lattice_w, cons
         A.partial = (float*)workspace;
         hipLaunchKernelGGL(cfh::attention_inputs_bwd_kernel, dim3((unsigned)blocks), dim3(256), 0, st, A);
     }
-    hipLaunchKernelGGL(cfh::attention_inputs_gw_kernel, dim3((A.HD + 31) / 32), dim3(1024), 0, st,
-                       (const float*)workspace, blocks, A.HD, g_lattice_w);
+    if (g_lattice_w)
+        hipLaunchKernelGGL(cfh::attention_inputs_gw_kernel, dim3((A.HD + 31) / 32), dim3(1024), 0, st,
+                           (const float*)workspace, blocks, A.HD, g_lattice_w);
     return finish_launch("attention_inputs_backward");
 }
 
@@ -618,14 +619,15 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
             J.ldy < J.O || J.ldx > 0x7fffffffLL || J.ldy > 0x7fffffffLL)
             return fail(CFH_EINVAL, "job %d: sizes N=%lld I=%lld O=%lld ldx=%lld ldy=%lld out of range", (int)j,
                         (long long)J.N, (long long)J.I, (long long)J.O, (long long)J.ldx, (long long)J.ldy);
-        if (!J.dW || (J.N > 0 && (!J.x || !J.dy))) return fail(CFH_EINVAL, "job %d: x, dy and dW must not be NULL", (int)j);
+        if ((!J.dW && !J.db) || (J.N > 0 && (!J.dy || (J.dW && !J.x))))
+            return fail(CFH_EINVAL, "job %d: dy, one of dW and db, and x with dW must not be NULL", (int)j);
     }
     hipStream_t st = (hipStream_t)stream;
     for (int32_t first = 0; first < njobs; first += cfh::WGRAD_MAX_JOBS) {
         const int32_t last = njobs < first + cfh::WGRAD_MAX_JOBS ? njobs : first + cfh::WGRAD_MAX_JOBS;
         long tiles = 0;
         for (int32_t j = first; j < last; j++)
-            if (jobs[j].N > 0) tiles += (long)((jobs[j].I + 63) / 64) * (long)((jobs[j].O + 63) / 64);
+            if (jobs[j].N > 0) tiles += (long)(jobs[j].dW ? (jobs[j].I + 63) / 64 : 1) * (long)((jobs[j].O + 63) / 64);
         if (tiles == 0) continue;
         const int want = (int)((2048 + tiles - 1) / tiles);        // slices of a job: about 2048 workgroups in all
         cfh::WgradJobs T{};
@@ -636,7 +638,7 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
             cfh::WgradJob& W = T.job[T.njobs++];
             W.x = J.x; W.dy = J.dy; W.dW = J.dW; W.db = J.db;
             W.N = (int)J.N; W.I = (int)J.I; W.O = (int)J.O; W.ldx = (int)J.ldx; W.ldy = (int)J.ldy;
-            W.bx = (int)((J.I + 63) / 64); W.by = (int)((J.O + 63) / 64);
+            W.bx = J.dW ? (int)((J.I + 63) / 64) : 1; W.by = (int)((J.O + 63) / 64);
             int slices = want;
             const int max_slices = (int)((J.N + 31) / 32);
             if (slices > max_slices) slices = max_slices;

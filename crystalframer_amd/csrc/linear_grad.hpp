@@ -15,7 +15,8 @@ typedef float v4f_l __attribute__((ext_vector_type(4)));
 
 // One workgroup's share: 256 threads = 4 wavefronts, wavefront w owns the 32x32 block
 // (64 ty + 32 (w/2), 64 tx + 32 (w%2)) of dW and the rows [slice rows_per_slice, ...) of x and dy
-// (row strides ldx, ldy: dy may be a column slice of a wider matrix).
+// (row strides ldx, ldy: dy may be a column slice of a wider matrix).  dW == nullptr: only db is
+// computed (x is not read; I = 1).
 __device__ __forceinline__ void wgrad_block(const float* __restrict__ x, const float* __restrict__ dy, int N, int I,
                                             int O, int ldx, int ldy, int rows_per_slice, int tx, int ty, int slice,
                                             float* dW, float* db) {
@@ -28,7 +29,8 @@ __device__ __forceinline__ void wgrad_block(const float* __restrict__ x, const f
     const int col = lane & 15, kk = lane >> 4;
     const int oa = o0 + col, ob = o0 + 16 + col;          // columns of dY this lane feeds (A operand)
     const int ia = i0 + col, ib = i0 + 16 + col;          // columns of X this lane feeds (B operand)
-    const bool voa = oa < O, vob = ob < O, via = ia < I, vib = ib < I;
+    const bool has_w = dW != nullptr;                     // no dW: the column sums of dY alone
+    const bool voa = oa < O, vob = ob < O, via = has_w && ia < I, vib = has_w && ib < I;
     v4f_l acc00 = {0.f, 0.f, 0.f, 0.f}, acc01 = acc00, acc10 = acc00, acc11 = acc00;
     float bsum_a = 0.f, bsum_b = 0.f;
 #pragma unroll 4

@@ -549,14 +549,15 @@ class _DeferredWeightGrads:
         def view(ref):           # (arena, offset, count) -> tensor
             return ref[0][ref[1]:ref[1] + ref[2]]
         lib = _lib.load()
-        dev = pending[0][0].device
+        dev = pending[0][1].device
         jobs = (_lib.CfhLinearGradJob * len(pending))()
         fixups = []
         for n, (x2, g2, col0, O, dW, db, weight, bias, w_mark, b_mark) in enumerate(pending):
             # dW, db: (arena, offset, count) of the zero-filled tensors handed to autograd (db: of the whole bias)
-            dst_w = dW[0].data_ptr() + 4 * dW[1]
+            # (x2 None: a sum over the rows of g2 alone, kept in the bias slots)
+            dst_w = None if dW is None else dW[0].data_ptr() + 4 * dW[1]
             dst_b = None if db is None else db[0].data_ptr() + 4 * (db[1] + col0)
-            wg = weight.grad
+            wg = None if weight is None else weight.grad
             if wg is not None and cls.mark(weight) != w_mark and wg.data_ptr() != dst_w:
                 # .grad was set or updated during this pass, but not by adopting our tensor: autograd
                 # copied or accumulated it (adding our zeros), so the result belongs into .grad
@@ -572,9 +573,12 @@ class _DeferredWeightGrads:
                     elif col0 == 0:
                         fixups.append((bg, view(db)))
             J = jobs[n]
-            J.x, J.dy = x2.data_ptr(), g2.data_ptr() + 4 * col0
+            J.x, J.dy = (None if x2 is None else x2.data_ptr()), g2.data_ptr() + 4 * col0
             J.dW, J.db = dst_w, dst_b
-            J.N, J.I, J.O, J.ldx, J.ldy = x2.shape[0], x2.shape[1], O, x2.stride(0), g2.stride(0)
+            if x2 is None:
+                J.N, J.I, J.O, J.ldx, J.ldy = g2.shape[0], 1, O, 1, g2.stride(0)
+            else:
+                J.N, J.I, J.O, J.ldx, J.ldy = x2.shape[0], x2.shape[1], O, x2.stride(0), g2.stride(0)
         with torch.cuda.device(dev), _timed("linear_weight_bias_grad_batch", dev):
             rc = lib.cfh_linear_weight_bias_grad_batch(jobs, len(pending), _lib.current_stream_ptr(dev))
         _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
@@ -763,6 +767,7 @@ class AttentionInputsHIP(torch.autograd.Function):
         _lib.check(rc, "cfh_attention_inputs_forward")
         ctx.save_for_backward(qkv, w, gs)
         ctx.consts = (H, Dh, c1, lb, c2, q_scale)
+        ctx.w_in = lattice_w
         ctx.set_materialize_grads(False)
         return qs, k, v, a
 
@@ -774,14 +779,32 @@ class AttentionInputsHIP(torch.autograd.Function):
         N = qkv.shape[0]
         gqs, gk, gv, ga = (None if g is None else _f32c(g) for g in (gqs, gk, gv, ga))
         gqkv = torch.empty_like(qkv)
-        gw = torch.empty((H * Dh,), dtype=torch.float32, device=qkv.device)
+        blocks = (N + 4 * (256 // (H * Dh)) - 1) // (4 * (256 // (H * Dh)))
         # scratch of the call: per-block partial sums of the weight gradient (256-byte aligned by the allocator)
-        ws = torch.empty(4 * H * Dh * (N // (4 * (256 // (H * Dh))) + 1), dtype=torch.uint8, device=qkv.device)
+        part = torch.empty((max(blocks, 1), H * Dh), dtype=torch.float32, device=qkv.device)
+        D = _DeferredWeightGrads
+        w_in = ctx.w_in
+        if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
+            D.reset()                               # left over from a backward pass that raised
+        defer = (KernelManager.DEFER_WEIGHT_GRADS and N > 0 and w_in is not None and w_in.is_leaf
+                 and w_in.dtype == torch.float32 and w_in.dim() == 1)
+        if defer:
+            # the column sums of the partials join the weight gradients of the pass in their one launch
+            gw = D.take(H * Dh, qkv.device)
+            gw_ref = (D.arena, D.arena_off - ((H * Dh + 63) & ~63), H * Dh)
+        else:
+            gw = torch.empty((H * Dh,), dtype=torch.float32, device=qkv.device)
         with _timed("attention_inputs_backward", qkv.device):
             rc = lib.cfh_attention_inputs_backward(_lib.ptr(qkv), _lib.ptr(w), _lib.ptr(gs), c1, lb, c2, q_scale,
                                                    _lib.ptr(gqs), _lib.ptr(gk), _lib.ptr(gv), _lib.ptr(ga), N, H, Dh,
-                                                   _lib.ptr(gqkv), _lib.ptr(gw), _lib.ptr(ws), ws.numel(),
-                                                   _lib.current_stream_ptr(qkv.device))
+                                                   _lib.ptr(gqkv), None if defer else _lib.ptr(gw), _lib.ptr(part),
+                                                   4 * part.numel(), _lib.current_stream_ptr(qkv.device))
         _lib.check(rc, "cfh_attention_inputs_backward")
+        if defer:
+            D.pending.append((None, part, 0, H * Dh, None, gw_ref, None, w_in, None, D.mark(w_in)))
+            if not D.callback_queued:
+                torch.autograd.Variable._execution_engine.queue_callback(D.flush)
+                D.callback_queued = True
+                D.task_id = torch._C._current_graph_task_id()
         return gqkv, gw, None, None, None, None, None, None
 

@@ -265,7 +265,9 @@ int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int6
  * The same gradients for several layers in one launch, ACCUMULATED into dW and db (the caller has
  * initialised them: zeros, or gradients to add to).  Each job: x (N,I) with row stride ldx, dy (N,O)
  * with row stride ldy (so a job may take a column block of a wider dy, e.g. one of the three
- * stacked input projections), dW (O,I) contiguous, db (O) or NULL.  `jobs` is a host array; it is
+ * stacked input projections), dW (O,I) contiguous, db (O) or NULL.  A job with dW == NULL adds only the
+ * column sums of dy to db (x is not read, I = ldx = 1): any sum over rows that a backward pass leaves
+ * for its end, e.g. the per-block partials of cfh_attention_inputs_backward.  `jobs` is a host array; it is
  * copied into the kernel arguments, 32 jobs per launch.  Deferring the weight gradients of a whole
  * backward pass to one call replaces one launch (plus clearing) per layer -- latency-bound at these
  * sizes -- by a launch that fills the chip.  No counterpart in the reference (autograd of
@@ -298,7 +300,9 @@ int cfh_small_linear_dx(const float* dy, const float* W, int64_t M, int64_t N, i
  *   alpha' = (alpha + gauss_scale_dev[1]) * gauss_scale_dev[0]  (alpha' = alpha when the pointer is NULL).
  * Backward: gqkv (N, 3 H Dh) = [ga da/dquery + gqs q_scale | gk | gv],  g_lattice_w (H Dh) = sum over atoms
  *   of ga da/dalpha query;  gqs, gk, gv, ga may each be NULL (zero).  gauss_scale_dev is a constant.
- *   workspace: ceil(N / (4 * (256 / (H Dh)))) * H Dh floats of scratch (per-block partial sums).
+ *   workspace: ceil(N / (4 * (256 / (H Dh)))) * H Dh floats, left holding the per-block partial sums of
+ *   g_lattice_w as a (blocks, H Dh) matrix; with g_lattice_w == NULL the launch that adds them up is left
+ *   out and the caller sums the columns itself (a dW == NULL job of cfh_linear_weight_bias_grad_batch).
  * Dh = 16, 256 % (H Dh) == 0.  Replaces the framework arithmetic of
  * models/indexed_lattice_multi_head_attention_cuda.py:896-940 (gaussian coefficient: c1 = beta / (1 - lb),
  * c2 = -1/2 scale_real^-2), the query scaling of :144-185 and :455, and the chunk / cat of the

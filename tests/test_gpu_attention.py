@@ -232,6 +232,48 @@ def test_attention_inputs_split_scale_and_gaussian_coefficient(N, H, normalised)
     (outs[2] * f32(g[2])).sum().backward()
     expect = torch.cat([torch.zeros(N, 2 * H * Dh, dtype=torch.float64), g[2].reshape(N, -1)], dim=1)
     assert Hh.rel_err(qkv.grad, expect) < 1e-6
+    assert Hh.rel_err(w.grad, w64.grad) < 1e-5           # a zero contribution was added to the existing .grad
+    # a second full pass accumulates; the sum of the per-block partials is deferred to the end of the
+    # pass for a leaf weight and made at once otherwise: same numbers
+    outs = cf.cuda_funcs.AttentionInputsHIP.apply(qkv, w, gs, H, c1, lb, c2, 1.0 / math.sqrt(Dh))
+    sum((o * f32(gi)).sum() for o, gi in zip(outs, g)).backward()
+    assert Hh.rel_err(w.grad, 2 * w64.grad) < 1e-5
+    w_mid = w * 1.0                                      # not a leaf
+    outs = cf.cuda_funcs.AttentionInputsHIP.apply(qkv, w_mid, gs, H, c1, lb, c2, 1.0 / math.sqrt(Dh))
+    gw_now, = torch.autograd.grad(sum((o * f32(gi)).sum() for o, gi in zip(outs, g)), [w_mid])
+    assert Hh.rel_err(gw_now, w64.grad) < 1e-5
+    outs = cf.cuda_funcs.AttentionInputsHIP.apply(qkv, w, gs, H, c1, lb, c2, 1.0 / math.sqrt(Dh))
+    gw_leaf, = torch.autograd.grad(sum((o * f32(gi)).sum() for o, gi in zip(outs, g)), [w])
+    assert Hh.rel_err(gw_leaf, w64.grad) < 1e-5
+    assert Hh.rel_err(w.grad, 2 * w64.grad) < 1e-5       # autograd.grad leaves .grad alone
+
+
+def test_weight_gradient_batch_job_without_weight_sums_columns():
+    """A job of the batched weight-gradient launch with dW == NULL adds the column sums of dy to db,
+    next to an ordinary job in the same launch."""
+    import ctypes
+    from crystalframer_amd import _lib
+    lib = _lib.load()
+    gen = torch.Generator().manual_seed(77)
+    part = f32(torch.randn(297, 128, generator=gen, dtype=torch.float64))
+    x = f32(torch.randn(150, 48, generator=gen, dtype=torch.float64))
+    dy = f32(torch.randn(150, 40, generator=gen, dtype=torch.float64))
+    out = torch.full((128,), 0.5, dtype=torch.float32, device=dev())
+    dW = torch.zeros((40, 48), dtype=torch.float32, device=dev())
+    db = torch.zeros((40,), dtype=torch.float32, device=dev())
+    jobs = (_lib.CfhLinearGradJob * 2)()
+    jobs[0].x, jobs[0].dy, jobs[0].dW, jobs[0].db = None, part.data_ptr(), None, out.data_ptr()
+    jobs[0].N, jobs[0].I, jobs[0].O, jobs[0].ldx, jobs[0].ldy = 297, 1, 128, 1, 128
+    jobs[1].x, jobs[1].dy, jobs[1].dW, jobs[1].db = x.data_ptr(), dy.data_ptr(), dW.data_ptr(), db.data_ptr()
+    jobs[1].N, jobs[1].I, jobs[1].O, jobs[1].ldx, jobs[1].ldy = 150, 48, 40, 48, 40
+    _lib.check(lib.cfh_linear_weight_bias_grad_batch(jobs, 2, _lib.current_stream_ptr(part.device)), "batch")
+    torch.cuda.synchronize()
+    assert Hh.rel_err(out, 0.5 + part.double().sum(0)) < 1e-5
+    assert Hh.rel_err(dW, dy.double().t() @ x.double()) < 1e-5
+    assert Hh.rel_err(db, dy.double().sum(0)) < 1e-5
+    # neither output given: refused
+    jobs[0].db = None
+    assert lib.cfh_linear_weight_bias_grad_batch(jobs, 1, _lib.current_stream_ptr(part.device)) != 0
 
 
 def test_linear_deferred_gradients_stacked_accumulated_and_nonleaf():
