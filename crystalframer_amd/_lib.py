@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
@@ -56,7 +56,8 @@ class CfhLinearGradJob(ctypes.Structure):
 
 
 EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_frame_axis1",
-           "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_backward",
+           "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_frame_axes_framed_pe_forward",
+           "cfh_framed_pe_backward",
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
            "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
            "cfh_crystal_geometry", "cfh_small_linear_forward", "cfh_small_linear_dx", "cfh_linear_weight_bias_grad", "cfh_linear_weight_bias_grad_batch", "cfh_attention_inputs_forward",
@@ -97,6 +98,8 @@ def load():
         lib.cfh_frame_axes.argtypes = [pp] + [_P] * 10 + [_I64] * 3 + [_P, _P, ctypes.c_size_t, _P]
         lib.cfh_framed_pe_forward.restype = ctypes.c_int
         lib.cfh_framed_pe_forward.argtypes = [pp] + [_P] * 13 + [_I64] * 3 + [_P] * 5 + [ctypes.c_size_t, _P]
+        lib.cfh_frame_axes_framed_pe_forward.restype = ctypes.c_int
+        lib.cfh_frame_axes_framed_pe_forward.argtypes = [pp] + [_P] * 14 + [_I64] * 3 + [_P] * 6 + [ctypes.c_size_t, _P]
         lib.cfh_framed_pe_backward.restype = ctypes.c_int
         lib.cfh_framed_pe_backward.argtypes = [pp] + [_P] * 17 + [_I64] * 3 + [_P] * 6 + [ctypes.c_size_t, _P]
         lib.cfh_fused_dpa_forward.restype = ctypes.c_int

@@ -22,6 +22,7 @@ from .params import LatticeformerParams
 
 
 FUSED_FRAMES = True      # one launch for both axes + orthogonalisation (False: the reference's three steps)
+FUSED_FRAMES_PE = True   # frame search and lattice sums in one library call (False: two calls, as the reference makes them)
 FUSED_INPUTS = True      # q/k/v split, query scaling and Gaussian coefficient in one launch (False: framework ops)
 
 
@@ -77,6 +78,16 @@ def compute_real_domain_attn_frame_proj(q, k, v, batch_q, batch_kv, edges, pos, 
         rv = adap[0]
         rvlen_args = (rv if rv.dim() == 2 else torch.norm(rv, 2, dim=-1), adap[1])
     use_angle = proj_angle1 is not None and params.value_pe_angle_real > 0
+    if use_angle and FUSED_FRAMES and FUSED_FRAMES_PE and pe_dist_proj is not None and K > 0:
+        # frame search and lattice sums in one library call (they share the per-item records)
+        qs = q if q_is_scaled else q / math.sqrt(q.shape[-1])
+        z, psi, frames = cuda_funcs.RealEncodingWithMaxFramesFuncHIP.apply(
+            qs, k, alpha, pos, dist2_min, tvecs, batch_q, edges, K, dist_max, wscale, pe_dist_proj,
+            proj_angle1, proj_angle2, proj_angle3, params.value_pe_angle_real, params.value_pe_angle_wscale,
+            params.cos_abs, params.value_pe_dist_coef, params.value_pe_angle_coef, *rvlen_args)
+        if frame_sink is not None:
+            frame_sink.append((frames[0], frames[1], frames[2]))
+        return z, psi
     if use_angle:
         # the reference computes the frames even when the angle encoding is off; their only consumer
         # is the angle encoding, so they are skipped here in that case

@@ -39,7 +39,8 @@ int fail(int code, const char* fmt, ...) {
 constexpr int MAX_HEADS = 64;
 constexpr size_t QUEUE_OFFSET = 512;           // workspace header: 256 reserved bytes, 32 uint64 statistics, then the work queues
 constexpr size_t STATS_OFFSET = 256;
-constexpr size_t COUNTER_BYTES = QUEUE_OFFSET + (size_t)MAX_HEADS * cfh::NQUEUE * cfh::QSTRIDE * sizeof(int32_t);   // whole header
+constexpr size_t QUEUE_SET_BYTES = (size_t)MAX_HEADS * cfh::NQUEUE * cfh::QSTRIDE * sizeof(int32_t);
+constexpr size_t COUNTER_BYTES = QUEUE_OFFSET + 2 * QUEUE_SET_BYTES;   // whole header: two sets of work queues
 constexpr int WAVES_PER_SIMD = 3;
 constexpr int FRAME_WAVES_PER_SIMD = 8;      // the frame search keeps no per-wavefront partials: as many as are resident
 
@@ -217,11 +218,14 @@ std::vector<TimedLaunch> g_timed;
 
 // `waves`: in = upper bound, out = wavefronts actually launched
 template <typename Kern>
-int launch_persistent(Kern kern, const cfh::KernelArgs& A, int* waves, hipStream_t st, const char* what) {
+int launch_persistent(Kern kern, const cfh::KernelArgs& A, int* waves, hipStream_t st, const char* what,
+                      bool prepare = true) {
     *waves = resident_waves(kern, *waves, A.H);
-    int threads = A.N * A.H > A.H * cfh::NQUEUE ? A.N * A.H : A.H * cfh::NQUEUE;
-    if (threads < A.gw_out_n) threads = A.gw_out_n;
-    hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, A, A.q != nullptr ? 1 : 0);
+    if (prepare) {
+        int threads = A.N * A.H > A.H * cfh::NQUEUE ? A.N * A.H : A.H * cfh::NQUEUE;
+        if (threads < A.gw_out_n) threads = A.gw_out_n;
+        hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, A, A.q != nullptr ? 1 : 0);
+    }
     bool timed = false;
     TimedLaunch t;
     {
@@ -349,13 +353,16 @@ int cfh_frame_axes(const cfh_params* p, const float* q, const float* k, const fl
         }                                                                                           \
     } while (0)
 
-int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,
-                          const float* rvlen, const int64_t* batch, const int64_t* edges,
-                          const int64_t* e_start, const int32_t* order, const float* W_dist,
-                          const float* W_axis1, const float* W_axis2, const float* W_axis3,
-                          const float* frames, int64_t N, int64_t E, int64_t B, float* z, float* psi,
-                          float* d2min_out, float* shat_out, void* workspace, size_t workspace_bytes,
-                          void* stream) {
+// Forward of the lattice sums; with q and k also the frame search in front of it, whose item records
+// and frames the forward kernel then takes over (one prepare launch for both).
+static int framed_pe_forward_impl(const cfh_params* p, const float* q, const float* k, const float* a_ih,
+                                  const float* rpos, const float* tvecs, const float* rvlen, const int64_t* batch,
+                                  const int64_t* edges, const int64_t* e_start, const int32_t* order,
+                                  const float* W_dist, const float* W_axis1, const float* W_axis2,
+                                  const float* W_axis3, const float* frames_in, float* frames_out, int64_t N,
+                                  int64_t E, int64_t B, float* z, float* psi, float* d2min_out, float* shat_out,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+    const bool search = q != nullptr;
     int rc = check_params(p);
     if (rc) return rc;
     if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
@@ -363,25 +370,73 @@ int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* r
     if (!z) return fail(CFH_EINVAL, "z must not be NULL");
     const bool has_len = p->dist_bins > 0 && W_dist != nullptr;
     const bool has_ang = has_len && p->angle_bins > 0 && W_axis1 != nullptr;
+    const float* frames = search ? frames_out : frames_in;
     if (p->dist_bins > 0 && !W_dist) return fail(CFH_EINVAL, "dist_bins > 0 but W_dist is NULL");
     if (has_len && !psi) return fail(CFH_EINVAL, "psi must not be NULL when dist_bins > 0");
     if (has_ang && (!W_axis2 || !W_axis3 || !frames))
         return fail(CFH_EINVAL, "W_axis1..3 and frames must be given together");
+    if (search && (!k || !frames_out)) return fail(CFH_EINVAL, "q, k and frames must not be NULL");
     int wl = 0, wa = 0;
     if ((rc = window_widths(p, &wl, &wa))) return rc;
     if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES + items_bytes(N, p->num_heads)))) return rc;
+    hipStream_t st = (hipStream_t)stream;
     cfh::KernelArgs A;
     fill_common(A, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
+    if (search) {
+        cfh::KernelArgs F = A;
+        F.q = q; F.k = k; F.out_frame = frames_out;
+        F.counters2 = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(workspace) + QUEUE_OFFSET + QUEUE_SET_BYTES);
+        F.frames_to_records = 1;
+        int fwaves = launch_waves(N, p->num_heads, FRAME_WAVES_PER_SIMD);
+        if ((rc = launch_persistent(cfh::frame_axis_kernel<2>, F, &fwaves, st, "frame_axes"))) return rc;
+        A.counters = F.counters2;
+    }
     A.W[0] = W_dist; A.W[1] = W_axis1; A.W[2] = W_axis2; A.W[3] = W_axis3;
     A.frames = frames; A.out_z = z; A.out_psi = psi; A.out_d2min = d2min_out; A.shat = shat_out;
     int waves = launch_waves(N, p->num_heads);
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
-    hipStream_t st = (hipStream_t)stream;
     const char* what = "framed_pe_forward";
-    if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_fwd_kernel, true, true);
-    else if (has_len) CFH_DISPATCH_PE(cfh::framed_pe_fwd_kernel, true, false);
-    else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, false, false>, A, &waves, st, what);
+    const bool prep = !search;
+#define CFH_DISPATCH_FWD(HAS_LEN, HAS_ANG)                                                                      \
+    do {                                                                                                        \
+        if (wide) {                                                                                             \
+            if (p->cos_abs) rc = launch_persistent(cfh::framed_pe_fwd_kernel<11, 41, true, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep);  \
+            else rc = launch_persistent(cfh::framed_pe_fwd_kernel<11, 41, false, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep);            \
+        } else {                                                                                                \
+            if (p->cos_abs) rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, true, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep);   \
+            else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep);             \
+        }                                                                                                       \
+    } while (0)
+    if (has_ang) CFH_DISPATCH_FWD(true, true);
+    else if (has_len) CFH_DISPATCH_FWD(true, false);
+    else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, false, false>, A, &waves, st, what, prep);
+#undef CFH_DISPATCH_FWD
     return rc;
+}
+
+int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,
+                          const float* rvlen, const int64_t* batch, const int64_t* edges,
+                          const int64_t* e_start, const int32_t* order, const float* W_dist,
+                          const float* W_axis1, const float* W_axis2, const float* W_axis3,
+                          const float* frames, int64_t N, int64_t E, int64_t B, float* z, float* psi,
+                          float* d2min_out, float* shat_out, void* workspace, size_t workspace_bytes,
+                          void* stream) {
+    return framed_pe_forward_impl(p, nullptr, nullptr, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, W_dist,
+                                  W_axis1, W_axis2, W_axis3, frames, nullptr, N, E, B, z, psi, d2min_out, shat_out,
+                                  workspace, workspace_bytes, stream);
+}
+
+int cfh_frame_axes_framed_pe_forward(const cfh_params* p, const float* q, const float* k, const float* a_ih,
+                                     const float* rpos, const float* tvecs, const float* rvlen,
+                                     const int64_t* batch, const int64_t* edges, const int64_t* e_start,
+                                     const int32_t* order, const float* W_dist, const float* W_axis1,
+                                     const float* W_axis2, const float* W_axis3, int64_t N, int64_t E, int64_t B,
+                                     float* frames, float* z, float* psi, float* d2min_out, float* shat_out,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+    if (N > 0 && !q) return fail(CFH_EINVAL, "q, k and frames must not be NULL");
+    return framed_pe_forward_impl(p, q, k, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, W_dist, W_axis1,
+                                  W_axis2, W_axis3, nullptr, frames, N, E, B, z, psi, d2min_out, shat_out, workspace,
+                                  workspace_bytes, stream);
 }
 
 int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,

@@ -336,6 +336,9 @@ struct KernelArgs {
     float* shat;                  // (E, H, 4, NBINS) window histograms: written by the forward when given,
                                   // read by the backward that does not rebuild them
     int32_t* counters;            // (H, NQUEUE) work-queue heads
+    int32_t* counters2;           // optional second set, cleared along with the first: for a second kernel that
+                                  // works through the same item records without a prepare launch of its own
+    int32_t frames_to_records;    // frame search: also store the orthonormal frames into the item records
     uint32_t* items;              // (N, H, REC_WORDS) item records of this launch
     unsigned long long* stats;    // optional running totals (see STAT_* below); never reset by a launch
     int32_t N, E, H;
@@ -434,7 +437,10 @@ __device__ __forceinline__ uint32_t load_record(const KernelArgs& P, int it, int
 // the weight-gradient outputs that the reduction after the main kernel adds into.
 __global__ __launch_bounds__(256) void prepare_items_kernel(const KernelArgs P, int with_query) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx < P.H * NQUEUE) P.counters[idx * QSTRIDE] = 0;
+    if (idx < P.H * NQUEUE) {
+        P.counters[idx * QSTRIDE] = 0;
+        if (P.counters2) P.counters2[idx * QSTRIDE] = 0;
+    }
     if (idx == 0 && with_query && P.seed_dev) {
         const unsigned long long s = *P.seed_dev;
         *P.seed_snap = s;

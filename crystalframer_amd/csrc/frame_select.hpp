@@ -332,9 +332,16 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                 float* o = P.out_frame + ((size_t)i * H + h) * 3;
                 o[0] = f1x; o[1] = f1y; o[2] = f1z;
                 o[stride + 0] = gx; o[stride + 1] = gy; o[stride + 2] = gz;
-                o[2 * stride + 0] = f1y * gz - f1z * gy;
-                o[2 * stride + 1] = f1z * gx - f1x * gz;
-                o[2 * stride + 2] = f1x * gy - f1y * gx;
+                const float hx = f1y * gz - f1z * gy, hy = f1z * gx - f1x * gz, hz = f1x * gy - f1y * gx;
+                o[2 * stride + 0] = hx; o[2 * stride + 1] = hy; o[2 * stride + 2] = hz;
+                if (P.frames_to_records) {
+                    // the record of this item (already in registers) becomes that of the kernel that
+                    // follows: the query makes room for the frames
+                    float* r = reinterpret_cast<float*>(P.items + ((size_t)it_cur * H + h) * REC_WORDS + REC_FRAMES);
+                    r[0] = f1x; r[1] = f1y; r[2] = f1z;
+                    r[3] = gx; r[4] = gy; r[5] = gz;
+                    r[6] = hx; r[7] = hy; r[8] = hz;
+                }
             }
         }
         st_raw += (unsigned long long)bx.T * (unsigned long long)(e1 - e0);

@@ -284,6 +284,91 @@ def _stacked_frames(f1, f2, f3):
     return torch.stack([_f32c(f1), _f32c(f2), _f32c(f3)], 0).contiguous()
 
 
+def _framed_pe_forward(ctx, qk, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, W_k, W_k1,
+                       W_k2, W_k3, frame_vecs, dim_angle_enc, value_pe_angle_scale, cos_abs, length_rbf_mul,
+                       angle_rbf_mul, rvlen_n, cutoff_radius):
+    """Forward of the two classes below.  ``qk``: None (``frame_vecs`` = the three frame tensors), or
+    (q, k): the frames are searched in the same library call.  Returns (z, v or None, frames or None)."""
+    _lib.require_gpu(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e)
+    lib = _lib.load()
+    N, H = a_ik.shape
+    E = edge_ij_e.shape[1]
+    dev = a_ik.device
+    K = int(K) if W_k is not None else 0
+    Wd = _proj_weight(W_k, H, "W_k") if K > 0 else None
+    use_angle = K > 0 and W_k1 is not None and int(dim_angle_enc) > 0
+    A = int(dim_angle_enc) if use_angle else 0
+    Wa = [_proj_weight(w, H, "W_k%d" % (n + 1)) for n, w in enumerate((W_k1, W_k2, W_k3))] if use_angle \
+        else [None, None, None]
+    Dh = Wd.shape[-2] if Wd is not None else 16
+    a = _f32c(a_ik)
+    rpos, tv, rv = _f32c(rpos_ij_e), _f32c(tvecs_n), _f32c(rvlen_n)
+    batch, edges = batch_i.contiguous(), edge_ij_e.contiguous()
+    e_start, order = edge_schedule(edge_ij_e, N)
+    z = torch.empty((E, H), dtype=torch.float32, device=dev)
+    v = torch.empty((E, H, Dh), dtype=torch.float32, device=dev) if K > 0 else None
+    p = _params(H, Dh, K, A, cos_abs, float(dist_max), wscale, value_pe_angle_scale,
+                length_rbf_mul, angle_rbf_mul, cutoff_radius if rv is not None else None)
+    shat = None
+    if KernelManager.SAVE_HISTOGRAMS and K > 0 and any(ctx.needs_input_grad):
+        shat = torch.empty((E, H, 4, K), dtype=torch.float32, device=dev)
+    if qk is None:
+        frames = _stacked_frames(*frame_vecs) if use_angle else None
+        with torch.cuda.device(dev), _timed("framed_pe_forward", dev):
+            ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
+            rc = lib.cfh_framed_pe_forward(
+                ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch),
+                _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd), _lib.ptr(Wa[0]),
+                _lib.ptr(Wa[1]), _lib.ptr(Wa[2]), _lib.ptr(frames), N, E, tv.shape[0], _lib.ptr(z),
+                _lib.ptr(v), None, _lib.ptr(shat), _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_framed_pe_forward")
+    else:
+        _lib.require_gpu(*qk)
+        q, k = _f32c(qk[0]), _f32c(qk[1])
+        frames = torch.empty((3, N, H, 3), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev), _timed("frame_axes_framed_pe_forward", dev):
+            ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
+            rc = lib.cfh_frame_axes_framed_pe_forward(
+                ctypes.byref(p), _lib.ptr(q), _lib.ptr(k), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv),
+                _lib.ptr(batch), _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd), _lib.ptr(Wa[0]),
+                _lib.ptr(Wa[1]), _lib.ptr(Wa[2]), N, E, tv.shape[0], _lib.ptr(frames), _lib.ptr(z), _lib.ptr(v),
+                None, _lib.ptr(shat), _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_frame_axes_framed_pe_forward")
+    ctx.save_for_backward(a, rpos, tv, rv, batch, edges, e_start, order, Wd, Wa[0], Wa[1], Wa[2],
+                          frames if use_angle else None, z, shat)
+    ctx.params = p
+    ctx.w_shapes = [None if w is None else w.shape for w in (W_k, W_k1, W_k2, W_k3)]
+    return z, v, frames
+
+
+def _framed_pe_backward(ctx, gz_ek, gv_ekd):
+    """ga (N,H) and the gradients of the four projection weights (in the shapes they came in)."""
+    a, rpos, tv, rv, batch, edges, e_start, order, Wd, W1, W2, W3, frames, z, shat = ctx.saved_tensors
+    lib = _lib.load()
+    p = ctx.params
+    N, H = a.shape
+    E = edges.shape[1]
+    dev = a.device
+    gz = _f32c(gz_ek) if gz_ek is not None else torch.zeros_like(z)
+    gv = None
+    if Wd is not None:
+        gv = _f32c(gv_ekd) if gv_ekd is not None else torch.zeros((E, H, Wd.shape[-2]), dtype=torch.float32, device=dev)
+    ga = torch.empty((N, H), dtype=torch.float32, device=dev)
+    gWd = torch.empty_like(Wd) if Wd is not None else None
+    gWa = [torch.empty_like(w) if w is not None else None for w in (W1, W2, W3)]
+    with torch.cuda.device(dev), _timed("framed_pe_backward", dev):
+        ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
+        rc = lib.cfh_framed_pe_backward(
+            ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch),
+            _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd), _lib.ptr(W1), _lib.ptr(W2),
+            _lib.ptr(W3), _lib.ptr(frames), _lib.ptr(z), _lib.ptr(gz), _lib.ptr(gv), _lib.ptr(shat), N, E, tv.shape[0],
+            _lib.ptr(ga), _lib.ptr(gWd), _lib.ptr(gWa[0]), _lib.ptr(gWa[1]), _lib.ptr(gWa[2]),
+            _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
+    _lib.check(rc, "cfh_framed_pe_backward")
+    gws = [g if g is None else g.reshape(s) for g, s in zip([gWd] + gWa, ctx.w_shapes)]
+    return ga, gws
+
+
 class RealEncodingWithFramedProjFuncCUDA(torch.autograd.Function):
     """z (E,H) and the framed value position encoding (E,H,Dh).  Signature and return convention of
     models/cuda_funcs/real_space_framed_proj.py:19-221: returns ``(z,)`` when ``K <= 0``, else
@@ -294,73 +379,46 @@ class RealEncodingWithFramedProjFuncCUDA(torch.autograd.Function):
                 W_k, W_k1, W_k2, W_k3, frame_vec_1, frame_vec_2, frame_vec_3, dim_angle_enc,
                 value_pe_angle_scale, cos_abs, length_rbf_mul, angle_rbf_mul, rvlen_n=None,
                 cutoff_radius=None):
-        _lib.require_gpu(a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e)
-        lib = _lib.load()
-        N, H = a_ik.shape
-        E = edge_ij_e.shape[1]
-        dev = a_ik.device
-        K = int(K) if W_k is not None else 0
-        Wd = _proj_weight(W_k, H, "W_k") if K > 0 else None
-        use_angle = K > 0 and W_k1 is not None and int(dim_angle_enc) > 0
-        A = int(dim_angle_enc) if use_angle else 0
-        Wa = [_proj_weight(w, H, "W_k%d" % (n + 1)) for n, w in enumerate((W_k1, W_k2, W_k3))] if use_angle \
-            else [None, None, None]
-        Dh = Wd.shape[-2] if Wd is not None else 16
-        a = _f32c(a_ik)
-        rpos, tv, rv = _f32c(rpos_ij_e), _f32c(tvecs_n), _f32c(rvlen_n)
-        batch, edges = batch_i.contiguous(), edge_ij_e.contiguous()
-        e_start, order = edge_schedule(edge_ij_e, N)
-        frames = _stacked_frames(frame_vec_1, frame_vec_2, frame_vec_3) if use_angle else None
-        z = torch.empty((E, H), dtype=torch.float32, device=dev)
-        v = torch.empty((E, H, Dh), dtype=torch.float32, device=dev) if K > 0 else None
-        p = _params(H, Dh, K, A, cos_abs, float(dist_max), wscale, value_pe_angle_scale,
-                    length_rbf_mul, angle_rbf_mul, cutoff_radius if rv is not None else None)
-        shat = None
-        if KernelManager.SAVE_HISTOGRAMS and K > 0 and any(ctx.needs_input_grad):
-            shat = torch.empty((E, H, 4, K), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev), _timed("framed_pe_forward", dev):
-            ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
-            rc = lib.cfh_framed_pe_forward(
-                ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch),
-                _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd), _lib.ptr(Wa[0]),
-                _lib.ptr(Wa[1]), _lib.ptr(Wa[2]), _lib.ptr(frames), N, E, tv.shape[0], _lib.ptr(z),
-                _lib.ptr(v), None, _lib.ptr(shat), _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
-        _lib.check(rc, "cfh_framed_pe_forward")
-        ctx.save_for_backward(a, rpos, tv, rv, batch, edges, e_start, order, Wd, Wa[0], Wa[1], Wa[2], frames, z, shat)
-        ctx.params = p
-        ctx.w_shapes = [None if w is None else w.shape for w in (W_k, W_k1, W_k2, W_k3)]
-        ctx.n_inputs = 23
-        if K <= 0:
+        z, v, _ = _framed_pe_forward(ctx, None, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale,
+                                     W_k, W_k1, W_k2, W_k3, (frame_vec_1, frame_vec_2, frame_vec_3),
+                                     dim_angle_enc, value_pe_angle_scale, cos_abs, length_rbf_mul, angle_rbf_mul,
+                                     rvlen_n, cutoff_radius)
+        if v is None:
             return z,
         return z, v
 
     @staticmethod
     def backward(ctx, gz_ek, gv_ekd=None):
-        a, rpos, tv, rv, batch, edges, e_start, order, Wd, W1, W2, W3, frames, z, shat = ctx.saved_tensors
-        lib = _lib.load()
-        p = ctx.params
-        N, H = a.shape
-        E = edges.shape[1]
-        dev = a.device
-        gz = _f32c(gz_ek) if gz_ek is not None else torch.zeros_like(z)
-        gv = None
-        if Wd is not None:
-            gv = _f32c(gv_ekd) if gv_ekd is not None else torch.zeros((E, H, Wd.shape[-2]), dtype=torch.float32, device=dev)
-        ga = torch.empty((N, H), dtype=torch.float32, device=dev)
-        gWd = torch.empty_like(Wd) if Wd is not None else None
-        gWa = [torch.empty_like(w) if w is not None else None for w in (W1, W2, W3)]
-        with torch.cuda.device(dev), _timed("framed_pe_backward", dev):
-            ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
-            rc = lib.cfh_framed_pe_backward(
-                ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch),
-                _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd), _lib.ptr(W1), _lib.ptr(W2),
-                _lib.ptr(W3), _lib.ptr(frames), _lib.ptr(z), _lib.ptr(gz), _lib.ptr(gv), _lib.ptr(shat), N, E, tv.shape[0],
-                _lib.ptr(ga), _lib.ptr(gWd), _lib.ptr(gWa[0]), _lib.ptr(gWa[1]), _lib.ptr(gWa[2]),
-                _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
-        _lib.check(rc, "cfh_framed_pe_backward")
-        gws = [g if g is None else g.reshape(s) for g, s in zip([gWd] + gWa, ctx.w_shapes)]
+        ga, gws = _framed_pe_backward(ctx, gz_ek, gv_ekd)
         return (ga, None, None, None, None, None, None, None, None, gws[0], gws[1], gws[2], gws[3],
                 None, None, None, None, None, None, None, None, None, None)
+
+
+class RealEncodingWithMaxFramesFuncHIP(torch.autograd.Function):
+    """The "max" frame search and RealEncodingWithFramedProjFuncCUDA behind it in one library call:
+    (z, v, frames) with frames (3,N,H,3) as ComputeFramesMaximumMethodCUDA returns them (not
+    differentiable).  ``q`` already divided by sqrt(Dh).  The remaining arguments are those of
+    RealEncodingWithFramedProjFuncCUDA without the frames; needs the angle encoding (K > 0 and the three
+    axis projections).  No counterpart class in the reference, which makes the two calls one after the
+    other (models/indexed_lattice_multi_head_attention_cuda.py:666-734)."""
+
+    @staticmethod
+    def forward(ctx, q, k, a_ik, rpos_ij_e, dist2_min_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale,
+                W_k, W_k1, W_k2, W_k3, dim_angle_enc, value_pe_angle_scale, cos_abs, length_rbf_mul,
+                angle_rbf_mul, rvlen_n=None, cutoff_radius=None):
+        if W_k is None or W_k1 is None or int(K) <= 0 or int(dim_angle_enc) <= 0:
+            raise ValueError("RealEncodingWithMaxFramesFuncHIP needs the distance and the angle encoding")
+        z, v, frames = _framed_pe_forward(ctx, (q, k), a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max,
+                                          wscale, W_k, W_k1, W_k2, W_k3, None, dim_angle_enc, value_pe_angle_scale,
+                                          cos_abs, length_rbf_mul, angle_rbf_mul, rvlen_n, cutoff_radius)
+        ctx.mark_non_differentiable(frames)
+        return z, v, frames
+
+    @staticmethod
+    def backward(ctx, gz_ek, gv_ekd=None, gframes=None):
+        ga, gws = _framed_pe_backward(ctx, gz_ek, gv_ekd)
+        return (None, None, ga, None, None, None, None, None, None, None, None, gws[0], gws[1], gws[2], gws[3],
+                None, None, None, None, None, None, None)
 
 
 # --------------------------------------------------------------------------------------------------

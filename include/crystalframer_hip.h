@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 2
+#define CFH_ABI_VERSION 3
 
 enum {
     CFH_OK = 0,
@@ -166,6 +166,22 @@ int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* r
                           const float* W_axis3, const float* frames, int64_t N, int64_t E,
                           int64_t B, float* z, float* psi, float* d2min_out, float* shat_out,
                           void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * cfh_frame_axes followed by cfh_framed_pe_forward with the frames it found, as the attention layer
+ * calls them (models/indexed_lattice_multi_head_attention_cuda.py:666-734: compute_frame_maximum_method_,
+ * then RealEncodingWithFramedProjFuncCUDA.apply): same arguments and results as the two calls (`frames`
+ * (3,N,H,3) is an output here), one launch less -- the per-item records (box, lattice, coefficient) are
+ * built once, the search stores its frames into them and the forward kernel works through them with a
+ * second set of work queues.
+ */
+int cfh_frame_axes_framed_pe_forward(const cfh_params* p, const float* q, const float* k, const float* a_ih,
+                                     const float* rpos, const float* tvecs, const float* rvlen,
+                                     const int64_t* batch, const int64_t* edges, const int64_t* e_start,
+                                     const int32_t* order, const float* W_dist, const float* W_axis1,
+                                     const float* W_axis2, const float* W_axis3, int64_t N, int64_t E,
+                                     int64_t B, float* frames, float* z, float* psi, float* d2min_out,
+                                     float* shat_out, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Gradients of the above for upstream gz (E,H) and gpsi (E,H,Dh): ga (N,H), gW_dist (H,Dh,K),

@@ -366,3 +366,59 @@ def test_fused_frames_equal_the_three_step_construction():
     M = fr.cpu().double().permute(1, 2, 0, 3)
     assert (M @ M.transpose(-1, -2) - torch.eye(3, dtype=torch.float64)).abs().max() < 1e-5
     assert (torch.linalg.det(M) - 1).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("noise", [0.0, 1e-5])
+def test_frames_and_lattice_sums_in_one_call_equal_the_two_calls(noise):
+    """cfh_frame_axes_framed_pe_forward (frame search, then the forward working through the same
+    item records) against cfh_frame_axes followed by cfh_framed_pe_forward: same kernels on the same
+    numbers, so frames, z, psi and the gradients are equal bit for bit (the weight gradients up to
+    the order of the float sums).  A one-atom problem and the empty batch pass through as well."""
+    import crystalframer_amd as cf
+    KM = cf.KernelManager
+    saved = (KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE)
+    KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE = noise, 1234, None
+    try:
+        for P in (Hh.make_problem(num_crystals=12, atoms_hi=6, seed=83),
+                  Hh.make_problem(num_crystals=3, atoms_lo=1, atoms_hi=1, seed=84)):
+            leaves = []
+            outs = []
+            for fused in (False, True):
+                a = g(P.a).requires_grad_(True)
+                Wk = g(P.W_k).requires_grad_(True)
+                Wax = [g(w).requires_grad_(True) for w in P.W_ax]
+                geo = (g(P.rpos), None, g(P.tvecs), P.batch.to(dev()), P.edges.to(dev()), 64, Hh.DIST_MAX, 1.0)
+                tail = (64, 4.0, 0, 1.0, 1.0, g(P.rvlen), CUT)
+                if fused:
+                    z, psi, fr = cf.cuda_funcs.RealEncodingWithMaxFramesFuncHIP.apply(
+                        g(P.q), g(P.k), a, *geo, Wk, *Wax, *tail)
+                    assert not fr.requires_grad
+                else:
+                    fr = cf.ComputeFramesMaximumMethodCUDA.apply(g(P.q), g(P.k), None, a.detach(), *geo[:-3], 64,
+                                                                 Hh.DIST_MAX, 1.0, g(P.rvlen), CUT)
+                    z, psi = cf.RealEncodingWithFramedProjFuncCUDA.apply(a, *geo, Wk, *Wax, fr[0], fr[1], fr[2], *tail)
+                gen = torch.Generator().manual_seed(5)
+                gz = g(torch.randn(z.shape, generator=gen, dtype=torch.float64))
+                gp = g(torch.randn(psi.shape, generator=gen, dtype=torch.float64))
+                ((z * gz).sum() + (psi * gp).sum()).backward()
+                outs.append((fr, z, psi))
+                leaves.append((a, Wk, *Wax))
+            for x, y in zip(outs[0], outs[1]):
+                assert x.shape == y.shape and torch.equal(x, y)
+            assert torch.equal(leaves[0][0].grad, leaves[1][0].grad)
+            for x, y in zip(leaves[0][1:], leaves[1][1:]):
+                assert Hh.rel_err(y.grad, x.grad.double()) < 1e-6
+        # empty batch: empty outputs, zero weight gradients
+        d = dev()
+        Wk = g(P.W_k).requires_grad_(True)
+        Wax = [g(w).requires_grad_(True) for w in P.W_ax]
+        a = torch.zeros(0, Hh.H, device=d, requires_grad=True)
+        z, psi, fr = cf.cuda_funcs.RealEncodingWithMaxFramesFuncHIP.apply(
+            torch.zeros(0, Hh.H, Hh.DH, device=d), torch.zeros(0, Hh.H, Hh.DH, device=d), a, torch.zeros(0, 3, device=d),
+            None, torch.zeros(0, 3, 3, device=d), torch.zeros(0, dtype=torch.long, device=d),
+            torch.zeros(2, 0, dtype=torch.long, device=d), 64, Hh.DIST_MAX, 1.0, Wk, *Wax, 64, 4.0, 0, 1.0, 1.0)
+        assert z.shape == (0, Hh.H) and psi.shape == (0, Hh.H, Hh.DH) and fr.shape == (3, 0, Hh.H, 3)
+        (z.sum() + psi.sum()).backward()
+        assert float(Wk.grad.abs().max()) == 0.0 and float(Wax[2].grad.abs().max()) == 0.0
+    finally:
+        KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE = saved
