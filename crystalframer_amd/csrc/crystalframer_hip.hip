@@ -684,7 +684,8 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
         for (int32_t j = first; j < last; j++)
             if (jobs[j].N > 0) tiles += (long)(jobs[j].dW ? (jobs[j].I + 63) / 64 : 1) * (long)((jobs[j].O + 63) / 64);
         if (tiles == 0) continue;
-        const int want = (int)((2048 + tiles - 1) / tiles);        // slices of a job: about 2048 workgroups in all
+        const int want = (int)(1900 / tiles > 0 ? 1900 / tiles : 1);   // slices of a job: the workgroups stay below the 2048 that are resident at once
+                                                                        // (a few more would run as a second round and double the time)
         cfh::WgradJobs T{};
         int blocks = 0;
         for (int32_t j = first; j < last; j++) {
