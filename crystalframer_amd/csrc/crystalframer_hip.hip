@@ -23,6 +23,7 @@
 #include "geometry.hpp"
 #include "linear_grad.hpp"
 #include "small_gemm.hpp"
+#include "layer_bridge.hpp"
 
 namespace {
 
@@ -709,6 +710,44 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
         hipLaunchKernelGGL(cfh::linear_wgrad_batch_kernel, dim3(blocks), dim3(256), 0, st, T);
     }
     return finish_launch("linear_weight_bias_grad_batch");
+}
+
+int cfh_layer_bridge_forward(const float* attn, const float* x_res, int64_t N, int32_t D, int32_t F, const float* Wo,
+                             const float* bo, const float* W1, const float* b1, const float* W2, const float* b2,
+                             const float* Wqkv, const float* bqkv, const float* lattice_w,
+                             const float* gauss_scale_dev, float c1, float lb, float c2, float q_scale, int32_t H,
+                             float* x1, float* h, float* x2, float* qkv, float* qs, float* k, float* v, float* a,
+                             void* stream) {
+    if (N < 0 || N > 0x7fffffffLL / 1024 || D < 128 || F < 128 || D % 128 != 0 || F % 128 != 0 || D > 65536 || F > 65536)
+        return fail(CFH_EINVAL, "layer bridge: N=%lld, D=%d and F=%d must be multiples of 128", (long long)N, (int)D, (int)F);
+    if (H < 1 || H * cfh::DH != D || cfh::BR_ROWS * H > 64 * cfh::BR_WAVES)
+        return fail(CFH_EINVAL, "layer bridge: D=%d must be 16 x H=%d, H at most %d", (int)D, (int)H, 64 * cfh::BR_WAVES / cfh::BR_ROWS);
+    if (N == 0) return CFH_OK;
+    if (!attn || !x_res || !Wo || !W1 || !W2 || !x1 || !h || !x2)
+        return fail(CFH_EINVAL, "layer bridge: attn, x_res, the weights and x1, h, x2 must not be NULL");
+    if (Wqkv && (!lattice_w || !qkv || !qs || !k || !v || !a))
+        return fail(CFH_EINVAL, "layer bridge: with Wqkv, lattice_w and qkv, qs, k, v, a must not be NULL");
+    const int wide = F > 3 * D ? F : 3 * D;
+    const size_t lds = (size_t)cfh::BR_ROWS * (2 * (D + cfh::BR_PAD) + wide + cfh::BR_PAD) * sizeof(float);
+    if (lds > 160 * 1024) return fail(CFH_EINVAL, "layer bridge: D=%d, F=%d need %zu bytes of LDS", (int)D, (int)F, lds);
+    static int lds_set[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(CFH_ELAUNCH, "layer bridge: no current device");
+    if (lds_set[dev] < (int)lds) {
+        if (hipFuncSetAttribute((const void*)cfh::layer_bridge_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess)
+            return fail(CFH_ELAUNCH, "layer bridge: %zu bytes of LDS refused", lds);
+        lds_set[dev] = (int)lds;
+    }
+    cfh::BridgeArgs A{};
+    A.attn = attn; A.xres = x_res; A.Wo = Wo; A.bo = bo; A.W1 = W1; A.b1 = b1; A.W2 = W2; A.b2 = b2;
+    A.Wq = Wqkv; A.bq = bqkv; A.lattice_w = lattice_w; A.gauss = gauss_scale_dev;
+    A.x1 = x1; A.h = h; A.x2 = x2; A.qkv = qkv; A.qs = qs; A.k = k; A.v = v; A.a = a;
+    A.N = (int)N; A.D = D; A.F = F; A.H = H;
+    A.c1 = c1; A.lb = lb; A.c2 = c2; A.q_scale = q_scale;
+    hipLaunchKernelGGL(cfh::layer_bridge_fwd_kernel, dim3((unsigned)((N + cfh::BR_ROWS - 1) / cfh::BR_ROWS)),
+                       dim3(64 * cfh::BR_WAVES), lds, (hipStream_t)stream, A);
+    return finish_launch("layer_bridge_forward");
 }
 
 int cfh_crystal_geometry(const float* pos, const int64_t* batch, const float* tvecs, const int64_t* sizes,

@@ -1,0 +1,156 @@
+// The projections between the attention cores of two consecutive encoder layers, which act on every atom
+// (row) separately, in one launch:
+//     x1  = x_res + attn Wo^T + bo              (output projection of the attention + residual)
+//     h   = relu(x1 W1^T + b1)                  (feed-forward, first half)
+//     x2  = x1 + h W2^T + b2                    (second half + residual: the layer's output)
+//     qkv = x2 Wqkv^T + bqkv                    (stacked input projection of the NEXT layer, optional)
+//     qs, k, v, a = split / scaled query / Gaussian coefficient of qkv (see attention_inputs.hpp)
+// The reference runs them as separate framework calls (models/indexed_lattice_multi_head_attention_cuda.py:
+// 399-409 and the out_proj behind :734, models/indexed_latticeformer_encoder.py:606-648 with post-norm
+// switched off), here 4 library GEMMs, 2 additions and the attention-input launch per layer, each a
+// few microseconds of work behind a launch.  A workgroup takes 16 rows -- the M of v_mfma_f32_16x16x4 --
+// through the whole chain with the activations in LDS; its wavefronts share the output columns of a
+// stage, 16 at a time, and stream the weights from the L2.  Every intermediate is also written out:
+// the backward pass needs all of them.
+#pragma once
+#include "device_common.hpp"
+
+namespace cfh {
+
+typedef float v4f_b2 __attribute__((ext_vector_type(4)));
+constexpr int BR_ROWS = 16;       // rows (atoms) per workgroup
+constexpr int BR_WAVES = 8;
+constexpr int BR_PAD = 4;         // floats of padding per LDS row
+
+struct BridgeArgs {
+    const float* attn; const float* xres;         // (N, D)
+    const float* Wo; const float* bo;             // (D, D), (D)        biases may be null
+    const float* W1; const float* b1;             // (F, D), (F)
+    const float* W2; const float* b2;             // (D, F), (D)
+    const float* Wq; const float* bq;             // (3 D, D), (3 D); Wq null: the chain ends with x2
+    const float* lattice_w; const float* gauss;   // (D); device {scale, shift} or null
+    float* x1; float* h; float* x2; float* qkv;   // (N, D), (N, F), (N, D), (N, 3 D)
+    float* qs; float* k; float* v; float* a;      // (N, D) x 3, (N, H)
+    int N, D, F, H;
+    float c1, lb, c2, q_scale;
+};
+
+// out[m][n] = act(sum_k in[m][k] W[n][k] + b[n] + res[m][n]) for the 16 rows of the block and the T column
+// tiles (of 16) wave, wave + 4, ... from tile t0 on.  in: LDS [16][K + BR_PAD]; out_lds: LDS [16][O + BR_PAD]
+// or null; out_g / res: global rows r0.., row stride O; res_lds: LDS [16][O + BR_PAD] or null.  U: steps of 16
+// along K whose loads are in flight.
+template <bool RELU, int T, int U>
+__device__ __forceinline__ void bridge_tiles(const float* in, int K, const float* __restrict__ W,
+                                             const float* __restrict__ b, int O, const float* __restrict__ res,
+                                             const float* res_lds, int r0, int nrows, float* out_lds,
+                                             float* __restrict__ out_g, int t0) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 15, kk = lane >> 4;
+    const int ldin = K + BR_PAD, ldout = O + BR_PAD;
+    const float* const arow = in + col * ldin + 4 * kk;
+    const float* const wrow = W + (size_t)(16 * (t0 + wave) + col) * K + 4 * kk;      // tile tt: + 64 tt K
+    v4f_b2 acc[T];
+#pragma unroll
+    for (int tt = 0; tt < T; tt++) acc[tt] = v4f_b2{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += 16 * U) {
+        float4 a4[U], w4[U][T];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            a4[u] = *reinterpret_cast<const float4*>(arow + k0 + 16 * u);
+#pragma unroll
+            for (int tt = 0; tt < T; tt++)
+                w4[u][tt] = *reinterpret_cast<const float4*>(wrow + (size_t)16 * BR_WAVES * tt * K + k0 + 16 * u);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int tt = 0; tt < T; tt++) {
+                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u].x, w4[u][tt].x, acc[tt], 0, 0, 0);
+                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u].y, w4[u][tt].y, acc[tt], 0, 0, 0);
+                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u].z, w4[u][tt].z, acc[tt], 0, 0, 0);
+                acc[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u].w, w4[u][tt].w, acc[tt], 0, 0, 0);
+            }
+    }
+#pragma unroll
+    for (int tt = 0; tt < T; tt++) {
+        const int n = 16 * (t0 + wave + BR_WAVES * tt) + col;
+        const float bias = b ? b[n] : 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int m = 4 * kk + c;
+            float val = acc[tt][c] + bias;
+            if (res && m < nrows) val += res[(size_t)(r0 + m) * O + n];
+            if (res_lds) val += res_lds[m * ldout + n];
+            if (RELU) val = fmaxf(val, 0.f);
+            if (out_lds) out_lds[m * ldout + n] = val;
+            if (m < nrows) out_g[(size_t)(r0 + m) * O + n] = val;
+        }
+    }
+}
+
+// All O columns (O a multiple of 64: whole tiles for each of the four wavefronts; K a multiple of 64).
+template <bool RELU>
+__device__ __forceinline__ void bridge_stage(const float* in, int K, const float* __restrict__ W,
+                                             const float* __restrict__ b, int O, const float* __restrict__ res,
+                                             const float* res_lds, int r0, int nrows, float* out_lds,
+                                             float* __restrict__ out_g) {
+    int t0 = 0;
+    int left = O / (16 * BR_WAVES);     // tiles per wavefront still to do
+    while (left >= 4) { bridge_tiles<RELU, 4, 2>(in, K, W, b, O, res, res_lds, r0, nrows, out_lds, out_g, t0); t0 += 4 * BR_WAVES; left -= 4; }
+    if (left >= 2) { bridge_tiles<RELU, 2, 4>(in, K, W, b, O, res, res_lds, r0, nrows, out_lds, out_g, t0); t0 += 2 * BR_WAVES; left -= 2; }
+    if (left >= 1) { bridge_tiles<RELU, 1, 8>(in, K, W, b, O, res, res_lds, r0, nrows, out_lds, out_g, t0); }
+}
+
+// grid: ceil(N / 16) workgroups of 512 threads; dynamic LDS: 16 (2 (D + 4) + max(F, 3 D) + 4) floats.
+// D, F multiples of 128; D = 16 H.
+__global__ __launch_bounds__(64 * BR_WAVES) void layer_bridge_fwd_kernel(const BridgeArgs P) {
+    extern __shared__ __attribute__((aligned(16))) float bridge_lds[];
+    const int D = P.D, F = P.F, Q = 3 * D;
+    float* const s_a = bridge_lds;                            // [16][D+4]  attention output, later x2
+    float* const s_b = s_a + BR_ROWS * (D + BR_PAD);          // [16][D+4]  x1
+    float* const s_c = s_b + BR_ROWS * (D + BR_PAD);          // [16][F+4]  h, later [16][3D+4] qkv
+    const int r0 = blockIdx.x * BR_ROWS;
+    const int nrows = min(BR_ROWS, P.N - r0);
+    for (int idx = threadIdx.x * 4; idx < BR_ROWS * D; idx += 64 * BR_WAVES * 4) {
+        const int m = idx / D, c = idx - m * D;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (m < nrows) v = *reinterpret_cast<const float4*>(P.attn + (size_t)(r0 + m) * D + c);
+        *reinterpret_cast<float4*>(s_a + m * (D + BR_PAD) + c) = v;
+    }
+    __syncthreads();
+    bridge_stage<false>(s_a, D, P.Wo, P.bo, D, P.xres, nullptr, r0, nrows, s_b, P.x1);
+    __syncthreads();
+    bridge_stage<true>(s_b, D, P.W1, P.b1, F, nullptr, nullptr, r0, nrows, s_c, P.h);
+    __syncthreads();
+    bridge_stage<false>(s_c, F, P.W2, P.b2, D, nullptr, s_b, r0, nrows, s_a, P.x2);
+    if (!P.Wq) return;
+    __syncthreads();
+    bridge_stage<false>(s_a, D, P.Wq, P.bq, Q, nullptr, nullptr, r0, nrows, s_c, P.qkv);
+    __syncthreads();
+    // split of qkv, query scaling
+    const int ldq = Q + BR_PAD;
+    for (int idx = threadIdx.x * 4; idx < BR_ROWS * Q; idx += 64 * BR_WAVES * 4) {
+        const int m = idx / Q, c = idx - m * Q;
+        if (m >= nrows) break;
+        float4 val = *reinterpret_cast<const float4*>(s_c + m * ldq + c);
+        const int part = c / D, cc = c - part * D;
+        float* dst = part == 0 ? P.qs : (part == 1 ? P.k : P.v);
+        if (part == 0) { val.x *= P.q_scale; val.y *= P.q_scale; val.z *= P.q_scale; val.w *= P.q_scale; }
+        *reinterpret_cast<float4*>(dst + (size_t)(r0 + m) * D + cc) = val;
+    }
+    // Gaussian coefficient of every (row, head)
+    if ((int)threadIdx.x < BR_ROWS * P.H) {
+        const int m = threadIdx.x / P.H, hh = threadIdx.x - m * P.H;
+        if (m < nrows) {
+            float alpha = 0.0f;
+#pragma unroll
+            for (int d = 0; d < DH; d++) alpha = fmaf(s_c[m * ldq + hh * DH + d], P.lattice_w[hh * DH + d], alpha);
+            if (P.gauss) alpha = (alpha + P.gauss[1]) * P.gauss[0];
+            const float u = alpha * P.c1;
+            const float e = u > 0.0f ? u : expm1f(u);
+            P.a[(size_t)(r0 + m) * P.H + hh] = ((1.0f - P.lb) * e + 1.0f) * P.c2;
+        }
+    }
+}
+
+}  // namespace cfh

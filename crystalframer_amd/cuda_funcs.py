@@ -644,6 +644,68 @@ class _DeferredWeightGrads:
             grad.add_(part.to(grad.dtype))
 
 
+def _linear_param_grads(x2, g2, weights, bias):
+    """Gradients of y = x2 W^T + b (W the row-wise stack of ``weights``) for upstream g2: a list of
+    weight gradients and the bias gradient (None without a bias).  For float32 leaf parameters the
+    tensors returned are zero-filled views of the pass's gradient arena and the products are made by
+    ONE library launch when the backward pass ends (see _DeferredWeightGrads); otherwise one launch
+    here."""
+    dev = x2.device
+    I = x2.shape[1]
+    O_all = g2.shape[1]
+    x2 = _f32c(x2)
+    g2 = _f32c(g2)
+    D = _DeferredWeightGrads
+    if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
+        D.reset()                               # left over from a backward pass that raised
+    defer = (KernelManager.DEFER_WEIGHT_GRADS and all(w.is_leaf for w in weights)
+             and (bias is None or bias.is_leaf) and all(w.dtype == torch.float32 for w in weights))
+    if defer:
+        def take(n):
+            v = D.take(n, dev)
+            return v, (D.arena, D.arena_off - ((n + 63) & ~63), n)
+    else:
+        total = sum(w.numel() for w in weights) + (O_all if bias is not None else 0)
+        buf = torch.zeros(total, dtype=torch.float32, device=dev)
+        state = [0]
+
+        def take(n):
+            v = buf[state[0]:state[0] + n]
+            state[0] += n
+            return v, (buf, state[0] - n, n)
+    gb, gb_ref = take(O_all) if bias is not None else (None, None)
+    gws, jobs, col0 = [], [], 0
+    for w in weights:
+        O = w.shape[0]
+        dW, dW_ref = take(O * I)
+        gws.append(dW.view(O, I))
+        jobs.append((x2, g2, col0, O, dW_ref, gb_ref, w, bias,
+                     D.mark(w) if defer else None, D.mark(bias) if defer and bias is not None else None))
+        del dW
+        col0 += O
+    if defer:
+        D.pending.extend(jobs)
+        if not D.callback_queued:
+            torch.autograd.Variable._execution_engine.queue_callback(D.flush)
+            D.callback_queued = True
+            D.task_id = torch._C._current_graph_task_id()
+    else:
+        lib = _lib.load()
+        arr = (_lib.CfhLinearGradJob * len(jobs))()
+        for n, (x2_, g2_, c0, O, dW, db, *_) in enumerate(jobs):
+            J = arr[n]
+            J.x, J.dy = x2_.data_ptr(), g2_.data_ptr() + 4 * c0
+            J.dW = dW[0].data_ptr() + 4 * dW[1]
+            J.db = None if db is None else db[0].data_ptr() + 4 * (db[1] + c0)
+            J.N, J.I, J.O, J.ldx, J.ldy = x2_.shape[0], I, O, x2_.stride(0), g2_.stride(0)
+        with torch.cuda.device(dev), _timed("linear_weight_bias_grad", dev):
+            rc = lib.cfh_linear_weight_bias_grad_batch(arr, len(jobs), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
+    gws = [g.to(w.dtype) if g.dtype != w.dtype else g for g, w in zip(gws, weights)]
+    gb_out = None if gb is None else (gb if gb.dtype == bias.dtype else gb.to(bias.dtype))
+    return gws, gb_out
+
+
 class LinearHIP(torch.autograd.Function):
     """y = x W^T + b, W the row-wise stack of ``weights`` (``stacked``: a tensor that already holds
     that stack, e.g. an alias of the parameters' shared storage; None: concatenated here).  Forward and
@@ -726,59 +788,8 @@ class LinearHIP(torch.autograd.Function):
         need_b = bias is not None and ctx.needs_input_grad[1]
         if not (any(need_w) or need_b):
             return (gx, None, None, None) + (None,) * len(weights)
-        dev = x.device
-        I = W.shape[1]
-        x2 = _f32c(x.reshape(-1, I))
-        g2 = _f32c(gy.reshape(-1, W.shape[0]))
-        D = _DeferredWeightGrads
-        if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
-            D.reset()                               # left over from a backward pass that raised
-        defer = (KernelManager.DEFER_WEIGHT_GRADS and all(w.is_leaf for w in weights)
-                 and (bias is None or bias.is_leaf) and all(w.dtype == torch.float32 for w in weights))
-        if defer:
-            def take(n):
-                v = D.take(n, dev)
-                return v, (D.arena, D.arena_off - ((n + 63) & ~63), n)
-        else:
-            total = sum(w.numel() for w in weights) + (W.shape[0] if bias is not None else 0)
-            buf = torch.zeros(total, dtype=torch.float32, device=dev)
-            state = [0]
-
-            def take(n):
-                v = buf[state[0]:state[0] + n]
-                state[0] += n
-                return v, (buf, state[0] - n, n)
-        gb, gb_ref = take(W.shape[0]) if bias is not None else (None, None)
-        gws, jobs, col0 = [], [], 0
-        for w in weights:
-            O = w.shape[0]
-            dW, dW_ref = take(O * I)
-            gws.append(dW.view(O, I))
-            jobs.append((x2, g2, col0, O, dW_ref, gb_ref, w, bias,
-                         D.mark(w) if defer else None, D.mark(bias) if defer and bias is not None else None))
-            del dW
-            col0 += O
-        if defer:
-            D.pending.extend(jobs)
-            if not D.callback_queued:
-                torch.autograd.Variable._execution_engine.queue_callback(D.flush)
-                D.callback_queued = True
-                D.task_id = torch._C._current_graph_task_id()
-        else:
-            lib = _lib.load()
-            arr = (_lib.CfhLinearGradJob * len(jobs))()
-            for n, (x2_, g2_, c0, O, dW, db, *_) in enumerate(jobs):
-                J = arr[n]
-                J.x, J.dy = x2_.data_ptr(), g2_.data_ptr() + 4 * c0
-                J.dW = dW[0].data_ptr() + 4 * dW[1]
-                J.db = None if db is None else db[0].data_ptr() + 4 * (db[1] + c0)
-                J.N, J.I, J.O, J.ldx, J.ldy = x2_.shape[0], I, O, x2_.stride(0), g2_.stride(0)
-            with torch.cuda.device(dev), _timed("linear_weight_bias_grad", dev):
-                rc = lib.cfh_linear_weight_bias_grad_batch(arr, len(jobs), _lib.current_stream_ptr(dev))
-            _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
-        gws = [g.to(w.dtype) if g.dtype != w.dtype else g for g, w in zip(gws, weights)]
-        gb_out = None if gb is None else (gb if gb.dtype == bias.dtype else gb.to(bias.dtype))
-        return (gx, gb_out, None, None) + tuple(gws)
+        gws, gb = _linear_param_grads(x.reshape(-1, W.shape[1]), gy.reshape(-1, W.shape[0]), weights, bias)
+        return (gx, gb, None, None) + tuple(gws)
 
 
 def linear(x: torch.Tensor, weight, bias: Optional[torch.Tensor] = None,
@@ -790,6 +801,44 @@ def linear(x: torch.Tensor, weight, bias: Optional[torch.Tensor] = None,
     weights = (weight,) if isinstance(weight, torch.Tensor) else tuple(weight)
     _lib.require_gpu(x, *weights)
     return LinearHIP.apply(x, bias, stacked, relu, *weights)
+
+
+def _attention_inputs_grads(qkv, w, gs, consts, w_in, gqs, gk, gv, ga):
+    """Backward of the attention inputs (see AttentionInputsHIP): the gradient of the stacked projection
+    output and of the lattice weights ``w_in`` (for a float32 leaf: a zero-filled view of the pass's
+    gradient arena, completed when the backward pass ends)."""
+    H, Dh, c1, lb, c2, q_scale = consts
+    lib = _lib.load()
+    N = qkv.shape[0]
+    gqs, gk, gv, ga = (None if g is None else _f32c(g) for g in (gqs, gk, gv, ga))
+    gqkv = torch.empty_like(qkv)
+    blocks = (N + 4 * (256 // (H * Dh)) - 1) // (4 * (256 // (H * Dh)))
+    # scratch of the call: per-block partial sums of the weight gradient (256-byte aligned by the allocator)
+    part = torch.empty((max(blocks, 1), H * Dh), dtype=torch.float32, device=qkv.device)
+    D = _DeferredWeightGrads
+    if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
+        D.reset()                               # left over from a backward pass that raised
+    defer = (KernelManager.DEFER_WEIGHT_GRADS and N > 0 and w_in is not None and w_in.is_leaf
+             and w_in.dtype == torch.float32 and w_in.dim() == 1)
+    if defer:
+        # the column sums of the partials join the weight gradients of the pass in their one launch
+        gw = D.take(H * Dh, qkv.device)
+        gw_ref = (D.arena, D.arena_off - ((H * Dh + 63) & ~63), H * Dh)
+    else:
+        gw = torch.empty((H * Dh,), dtype=torch.float32, device=qkv.device)
+    with _timed("attention_inputs_backward", qkv.device):
+        rc = lib.cfh_attention_inputs_backward(_lib.ptr(qkv), _lib.ptr(w), _lib.ptr(gs), c1, lb, c2, q_scale,
+                                               _lib.ptr(gqs), _lib.ptr(gk), _lib.ptr(gv), _lib.ptr(ga), N, H, Dh,
+                                               _lib.ptr(gqkv), None if defer else _lib.ptr(gw), _lib.ptr(part),
+                                               4 * part.numel(), _lib.current_stream_ptr(qkv.device))
+    _lib.check(rc, "cfh_attention_inputs_backward")
+    if defer:
+        D.pending.append((None, part, 0, H * Dh, None, gw_ref, None, w_in, None, D.mark(w_in)))
+        if not D.callback_queued:
+            torch.autograd.Variable._execution_engine.queue_callback(D.flush)
+            D.callback_queued = True
+            D.task_id = torch._C._current_graph_task_id()
+    return gqkv, gw
 
 
 class AttentionInputsHIP(torch.autograd.Function):
@@ -832,37 +881,93 @@ class AttentionInputsHIP(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gqs, gk, gv, ga):
         qkv, w, gs = ctx.saved_tensors
-        H, Dh, c1, lb, c2, q_scale = ctx.consts
-        lib = _lib.load()
-        N = qkv.shape[0]
-        gqs, gk, gv, ga = (None if g is None else _f32c(g) for g in (gqs, gk, gv, ga))
-        gqkv = torch.empty_like(qkv)
-        blocks = (N + 4 * (256 // (H * Dh)) - 1) // (4 * (256 // (H * Dh)))
-        # scratch of the call: per-block partial sums of the weight gradient (256-byte aligned by the allocator)
-        part = torch.empty((max(blocks, 1), H * Dh), dtype=torch.float32, device=qkv.device)
-        D = _DeferredWeightGrads
-        w_in = ctx.w_in
-        if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
-            D.reset()                               # left over from a backward pass that raised
-        defer = (KernelManager.DEFER_WEIGHT_GRADS and N > 0 and w_in is not None and w_in.is_leaf
-                 and w_in.dtype == torch.float32 and w_in.dim() == 1)
-        if defer:
-            # the column sums of the partials join the weight gradients of the pass in their one launch
-            gw = D.take(H * Dh, qkv.device)
-            gw_ref = (D.arena, D.arena_off - ((H * Dh + 63) & ~63), H * Dh)
-        else:
-            gw = torch.empty((H * Dh,), dtype=torch.float32, device=qkv.device)
-        with _timed("attention_inputs_backward", qkv.device):
-            rc = lib.cfh_attention_inputs_backward(_lib.ptr(qkv), _lib.ptr(w), _lib.ptr(gs), c1, lb, c2, q_scale,
-                                                   _lib.ptr(gqs), _lib.ptr(gk), _lib.ptr(gv), _lib.ptr(ga), N, H, Dh,
-                                                   _lib.ptr(gqkv), None if defer else _lib.ptr(gw), _lib.ptr(part),
-                                                   4 * part.numel(), _lib.current_stream_ptr(qkv.device))
-        _lib.check(rc, "cfh_attention_inputs_backward")
-        if defer:
-            D.pending.append((None, part, 0, H * Dh, None, gw_ref, None, w_in, None, D.mark(w_in)))
-            if not D.callback_queued:
-                torch.autograd.Variable._execution_engine.queue_callback(D.flush)
-                D.callback_queued = True
-                D.task_id = torch._C._current_graph_task_id()
+        gqkv, gw = _attention_inputs_grads(qkv, w, gs, ctx.consts, ctx.w_in, gqs, gk, gv, ga)
         return gqkv, gw, None, None, None, None, None, None
+
+
+class LayerBridgeHIP(torch.autograd.Function):
+    """Everything between the attention cores of two consecutive encoder layers in one launch (forward):
+
+        x1 = x_res + attn Wo^T + bo,   h = relu(x1 W1^T + b1),   x2 = x1 + h W2^T + b2,
+
+    and, when the weights of a next layer are given, qkv = x2 Wqkv^T + b_in and (qs, k, v, a) as
+    AttentionInputsHIP makes them.  Returns ``(x2,)`` or ``(x2, qs, k, v, a)``.  ``stacked``: the three
+    input-projection weights as one (3D, D) tensor if they share a storage, else None.  The backward
+    pass uses the framework's GEMMs for the input gradients (the residual additions ride on them),
+    the attention-inputs kernel, and the deferred weight-gradient launch.  For a layer without layer
+    norm and dropout and with the ReLU activation; no counterpart class in the reference
+    (models/indexed_latticeformer_encoder.py:606-648, models/indexed_lattice_multi_head_attention_cuda.py:
+    399-409, 734, 896-940)."""
+
+    @staticmethod
+    def supported(D: int, F: int, H: int) -> bool:
+        wide = max(F, 3 * D)
+        return (D % 128 == 0 and F % 128 == 0 and D == 16 * H and H <= 32
+                and 16 * (2 * (D + 4) + wide + 4) * 4 <= 160 * 1024)
+
+    @staticmethod
+    def forward(ctx, attn, x_res, Wo, bo, W1, b1, W2, b2, stacked, in_bias, lattice_w, gauss_scale, H, c1, lb,
+                c2, q_scale, *qkv_weights):
+        _lib.require_gpu(attn, x_res, Wo, W1, W2)
+        lib = _lib.load()
+        dev = attn.device
+        N, D = attn.shape
+        F = W1.shape[0]
+        Dh = D // H
+        has_next = len(qkv_weights) > 0
+        attn_c, xres_c = _f32c(attn), _f32c(x_res)
+        Wo_c, W1_c, W2_c = _f32c(Wo.detach()), _f32c(W1.detach()), _f32c(W2.detach())
+        bo_c, b1_c, b2_c = (None if b is None else _f32c(b.detach()) for b in (bo, b1, b2))
+        x1 = torch.empty((N, D), dtype=torch.float32, device=dev)
+        h = torch.empty((N, F), dtype=torch.float32, device=dev)
+        x2 = torch.empty((N, D), dtype=torch.float32, device=dev)
+        Wq = bq = w = gs = qkv = qs = k = v = a = None
+        if has_next:
+            Wq = _f32c((stacked if stacked is not None else torch.cat(qkv_weights, dim=0)).detach())
+            bq = None if in_bias is None else _f32c(in_bias.detach())
+            w = _f32c(lattice_w.detach())
+            gs = _f32c(gauss_scale.detach()) if gauss_scale is not None else None
+            qkv = torch.empty((N, 3 * D), dtype=torch.float32, device=dev)
+            qs = torch.empty((N, H, Dh), dtype=torch.float32, device=dev)
+            k = torch.empty_like(qs)
+            v = torch.empty_like(qs)
+            a = torch.empty((N, H), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev), _timed("layer_bridge_forward", dev):
+            rc = lib.cfh_layer_bridge_forward(
+                _lib.ptr(attn_c), _lib.ptr(xres_c), N, D, F, _lib.ptr(Wo_c), _lib.ptr(bo_c), _lib.ptr(W1_c),
+                _lib.ptr(b1_c), _lib.ptr(W2_c), _lib.ptr(b2_c), _lib.ptr(Wq), _lib.ptr(bq), _lib.ptr(w), _lib.ptr(gs),
+                float(c1), float(lb), float(c2), float(q_scale), H, _lib.ptr(x1), _lib.ptr(h), _lib.ptr(x2),
+                _lib.ptr(qkv), _lib.ptr(qs), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_layer_bridge_forward")
+        ctx.save_for_backward(attn_c, x1, h, x2, qkv, Wo_c, W1_c, W2_c, Wq, w, gs)
+        ctx.params = (Wo, bo, W1, b1, W2, b2, tuple(qkv_weights), in_bias, lattice_w)
+        ctx.consts = (H, Dh, c1, lb, c2, q_scale)
+        ctx.set_materialize_grads(False)
+        if has_next:
+            return x2, qs, k, v, a
+        return x2,
+
+    @staticmethod
+    def backward(ctx, g_x2, g_qs=None, g_k=None, g_v=None, g_a=None):
+        attn, x1, h, x2, qkv, Wo_c, W1_c, W2_c, Wq, w, gs = ctx.saved_tensors
+        Wo, bo, W1, b1, W2, b2, qkv_weights, in_bias, lattice_w = ctx.params
+        n_fixed = 17
+        g2 = None if g_x2 is None else _f32c(g_x2)
+        g_in_bias = g_lw = None
+        g_qkv_w = [None] * len(qkv_weights)
+        if qkv_weights and any(g is not None for g in (g_qs, g_k, g_v, g_a)):
+            gqkv, g_lw = _attention_inputs_grads(qkv, w, gs, ctx.consts, lattice_w, g_qs, g_k, g_v, g_a)
+            g2 = gqkv.matmul(Wq) if g2 is None else torch.addmm(g2, gqkv, Wq)      # the residual rides on the GEMM
+            g_qkv_w, g_in_bias = _linear_param_grads(x2, gqkv, qkv_weights, in_bias)
+        if g2 is None:
+            return (None,) * (n_fixed + len(qkv_weights))
+        gh = torch.ops.aten.threshold_backward(g2.matmul(W2_c), h, 0.0)
+        g1 = torch.addmm(g2, gh, W1_c)
+        g_attn = g1.matmul(Wo_c)
+        (gW2,), gb2 = _linear_param_grads(h, g2, (W2,), b2)
+        (gW1,), gb1 = _linear_param_grads(x1, gh, (W1,), b1)
+        (gWo,), gbo = _linear_param_grads(attn, g1, (Wo,), bo)
+        return (g_attn, g1, gWo, gbo, gW1, gb1, gW2, gb2, None, g_in_bias, g_lw, None, None, None, None, None, None,
+                *g_qkv_w)
+
 

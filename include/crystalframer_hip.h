@@ -310,6 +310,28 @@ int cfh_small_linear_forward(const float* x, const float* W, const float* b, int
 int cfh_small_linear_dx(const float* dy, const float* W, int64_t M, int64_t N, int64_t K, float* dx, void* stream);
 
 /*
+ * The projections between the attention cores of two consecutive encoder layers, which act on every atom
+ * separately, in one launch (forward):
+ *   x1 (N,D) = x_res + attn Wo^T + bo;  h (N,F) = relu(x1 W1^T + b1);  x2 (N,D) = x1 + h W2^T + b2;
+ *   with Wqkv (3D,D): qkv (N,3D) = x2 Wqkv^T + bqkv and qs, k, v, a as cfh_attention_inputs_forward makes
+ *   them from qkv (Wqkv NULL: the chain ends with x2 and the last eight outputs are not touched).
+ * Weights as torch.nn.Linear stores them, biases may be NULL; D = 16 H and F multiples of 128.  Every
+ * intermediate is an output because the backward pass (framework GEMMs and the entry points above) needs
+ * it.  Replaces, for a layer without layer norm and dropout and with the ReLU activation, the out_proj of
+ * the attention and the residual (models/indexed_lattice_multi_head_attention_cuda.py:734,
+ * models/indexed_latticeformer_encoder.py:639-648), the feed-forward block (:606, :644-648) and the
+ * input projection, query scaling and Gaussian coefficient of the next layer
+ * (models/indexed_lattice_multi_head_attention_cuda.py:399-409, :896-940): seven launches of the framework
+ * per layer in the reference's formulation.
+ */
+int cfh_layer_bridge_forward(const float* attn, const float* x_res, int64_t N, int32_t D, int32_t F, const float* Wo,
+                             const float* bo, const float* W1, const float* b1, const float* W2, const float* b2,
+                             const float* Wqkv, const float* bqkv, const float* lattice_w,
+                             const float* gauss_scale_dev, float c1, float lb, float c2, float q_scale, int32_t H,
+                             float* x1, float* h, float* x2, float* qkv, float* qs, float* k, float* v, float* a,
+                             void* stream);
+
+/*
  * What lies between the stacked q/k/v projection of a layer and its kernels, one launch each way.
  * Forward: qkv (N, 3 H Dh), rows = [query | key | value];  qs = query * q_scale, k, v (N,H,Dh) contiguous,
  *   a (N,H) = ((1 - lb) elu(c1 alpha') + 1) c2  with alpha = query_h . lattice_w_h and

@@ -364,3 +364,78 @@ def test_few_row_projection_kernels(M, I, O, bias, relu):
     assert Hh.rel_err(w.grad, w64.grad) < 1e-5
     if bias:
         assert Hh.rel_err(b.grad, b64.grad) < 1e-5
+
+
+@pytest.mark.parametrize("N,has_next,normalised,with_bias", [(301, True, True, True), (16, True, False, False),
+                                                              (77, False, False, True), (0, True, True, True)])
+def test_layer_bridge_matches_framework_chain(N, has_next, normalised, with_bias):
+    """Output projection + residual, feed-forward block + residual, next layer's input projection and
+    attention inputs in one launch, against float64 autograd of the same chain; the backward pass
+    (framework GEMMs + deferred weight gradients) gives every gradient, also when accumulated into
+    existing .grad tensors by a second pass."""
+    import math
+    import crystalframer_amd as cf
+    D, F, H, Dh, lb, beta, scale_real = 128, 256, 8, 16, 0.5, 0.1, 1.4
+    c1, c2 = beta / (1.0 - lb), -0.5 * scale_real ** -2
+    gen = torch.Generator().manual_seed(300 + N)
+    mk = lambda *shape, s=1.0: torch.randn(*shape, generator=gen, dtype=torch.float64) * s
+    t64 = dict(attn=mk(N, D), xres=mk(N, D), Wo=mk(D, D, s=D ** -0.5), W1=mk(F, D, s=D ** -0.5), W2=mk(D, F, s=F ** -0.5),
+               Wq=mk(D, D, s=D ** -0.5), Wk=mk(D, D, s=D ** -0.5), Wv=mk(D, D, s=D ** -0.5), lw=mk(D, s=0.25))
+    if with_bias:
+        t64.update(bo=mk(D), b1=mk(F), b2=mk(D), bin=mk(3 * D))
+    for t in t64.values():
+        t.requires_grad_(True)
+    gs64 = torch.tensor([0.37, -0.8], dtype=torch.float64) if normalised else None
+
+    def chain(t, lin, relu, gs):
+        x1 = t["xres"] + lin(t["attn"], t["Wo"], t.get("bo"))
+        hh = relu(lin(x1, t["W1"], t.get("b1")))
+        x2 = x1 + lin(hh, t["W2"], t.get("b2"))
+        if not has_next:
+            return (x2,)
+        qkv = lin(x2, torch.cat([t["Wq"], t["Wk"], t["Wv"]], 0), t.get("bin"))
+        q, k, v = (p.reshape(N, H, Dh) for p in qkv.split(D, dim=1))
+        alpha = (q * t["lw"].view(1, H, Dh)).sum(-1)
+        if gs is not None:
+            alpha = (alpha + gs[1]) * gs[0]
+        a = ((1.0 - lb) * torch.nn.functional.elu(alpha * c1) + 1.0) * c2
+        return x2, q / math.sqrt(Dh), k, v, a
+
+    ref = chain(t64, torch.nn.functional.linear, torch.relu, gs64)
+    g = [torch.randn(o.shape, generator=gen, dtype=torch.float64) for o in ref]
+    sum((o * gi).sum() for o, gi in zip(ref, g)).backward()
+
+    t32 = {n: f32(t.detach()).requires_grad_(True) for n, t in t64.items()}
+    gs = f32(gs64) if normalised else None
+
+    def run():
+        extra = (t32["Wq"], t32["Wk"], t32["Wv"]) if has_next else ()
+        return cf.cuda_funcs.LayerBridgeHIP.apply(
+            t32["attn"], t32["xres"], t32["Wo"], t32.get("bo"), t32["W1"], t32.get("b1"), t32["W2"], t32.get("b2"),
+            None, t32.get("bin") if has_next else None, t32["lw"] if has_next else None, gs if has_next else None,
+            H, c1, lb, c2, 1.0 / math.sqrt(Dh), *extra)
+
+    outs = run()
+    assert len(outs) == len(ref)
+    for o, r in zip(outs, ref):
+        assert o.shape == r.shape
+        if N:
+            assert Hh.rel_err(o.detach(), r.detach()) < 2e-6
+    sum((o * f32(gi)).sum() for o, gi in zip(outs, g)).backward()
+    used = [n for n in t64 if has_next or n not in ("Wq", "Wk", "Wv", "lw", "bin")]
+    for n in used:
+        if N == 0:
+            assert t32[n].grad is None or float(t32[n].grad.abs().sum()) == 0.0
+        else:
+            assert Hh.rel_err(t32[n].grad, t64[n].grad) < 2e-5, n
+    if N == 0:
+        return
+    outs = run()                                         # second pass: accumulation
+    sum((o * f32(gi)).sum() for o, gi in zip(outs, g)).backward()
+    for n in used:
+        assert Hh.rel_err(t32[n].grad, 2 * t64[n].grad) < 2e-5, n
+    # only the layer output is used downstream
+    for t in t32.values():
+        t.grad = None
+    (run()[0] * f32(g[0])).sum().backward()
+    assert t32["attn"].grad is not None and t32["W2"].grad is not None
