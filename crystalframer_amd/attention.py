@@ -291,10 +291,46 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
             v = cuda_funcs.linear(value, self.v_proj_weight, bv).view(value.shape[0], H, -1)
         if not q_is_scaled:
             a = self.gaussian_coefficient(q)
+        out, psi = self.attention_core(q, k, v, a, batch_q, batch_kv, edges, points, dist2_min, tvecs, rvecs,
+                                       this_epoch, q_is_scaled)
+        out = cuda_funcs.linear(out, self.out_proj.weight, self.out_proj.bias)
+        return out, psi
+
+    def attention_core(self, q: Tensor, k: Tensor, v: Tensor, a: Tensor, batch_q: Tensor, batch_kv: Tensor,
+                       edges: Tensor, points: Tensor, dist2_min: Optional[Tensor], tvecs: Tensor,
+                       rvecs: Optional[Tensor], this_epoch: Optional[int], q_is_scaled: bool):
+        """Frames, lattice sums and the softmax attention for projected q, k, v (N,H,Dh) and Gaussian
+        coefficients a (N,H): the heads' outputs side by side (N, H Dv), before the output projection,
+        and psi."""
         z, psi = compute_real_domain_attn_frame_proj(
             q, k, v, batch_q, batch_kv, edges, points, dist2_min, tvecs, rvecs, self.pe_dist_proj,
             self.proj_angle1, self.proj_angle2, self.proj_angle3, a, self.params, this_epoch,
             frame_sink=self.frame_sink, q_is_scaled=q_is_scaled)
         out = _scaled_dot_product_attention(q, k, v, batch_q, batch_kv, edges, z, psi, q_is_scaled=q_is_scaled)
-        out = cuda_funcs.linear(out.reshape(N, H * v.shape[-1]), self.out_proj.weight, self.out_proj.bias)
-        return out, psi
+        return out.reshape(q.shape[0], self.num_heads * v.shape[-1]), psi
+
+    def fused_inputs_ready(self) -> bool:
+        """True when the input projection can be followed by the fused split / scaling / Gaussian
+        coefficient (AttentionInputsHIP, or the last stage of LayerBridgeHIP)."""
+        H, Dh = self.num_heads, self.head_dim
+        return (FUSED_INPUTS and self.kdim == self.vdim == H * Dh
+                and cuda_funcs.AttentionInputsHIP.supported(H, Dh)
+                and (not self.params.normalize_gauss or self._gauss_scale_ready()))
+
+    def bridge_arguments(self):
+        """What LayerBridgeHIP needs of this layer as the NEXT one: (stacked weight, in_proj_bias,
+        lattice_pos_weights, gauss_scale or None, H, c1, lb, c2, q_scale, (q, k, v weights))."""
+        c1, lb, c2 = self._gauss_constants()
+        return (self._stacked_in_proj(), self.in_proj_bias, self.lattice_pos_weights,
+                self.gauss_scale if self.params.normalize_gauss else None, self.num_heads, c1, lb, c2,
+                1.0 / math.sqrt(self.head_dim), (self.q_proj_weight, self.k_proj_weight, self.v_proj_weight))
+
+    def project_inputs(self, x: Tensor):
+        """(qs, k, v, a) of self-attention on x with the fused path (requires fused_inputs_ready())."""
+        H, Dh = self.num_heads, self.head_dim
+        qkv = cuda_funcs.linear(x, (self.q_proj_weight, self.k_proj_weight, self.v_proj_weight),
+                                self.in_proj_bias, stacked=self._stacked_in_proj())
+        c1, lb, c2 = self._gauss_constants()
+        return cuda_funcs.AttentionInputsHIP.apply(
+            qkv, self.lattice_pos_weights, self.gauss_scale if self.params.normalize_gauss else None,
+            H, c1, lb, c2, 1.0 / math.sqrt(Dh))

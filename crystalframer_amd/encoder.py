@@ -20,6 +20,11 @@ from .attention import CrystalformerMultiheadAttentionCUDA
 from .params import LatticeformerParams
 
 
+# Between the attention cores of consecutive layers everything acts on single atoms: one launch per layer
+# (cuda_funcs.LayerBridgeHIP) when the layers have no layer norm, no active dropout and the ReLU activation.
+FUSED_LAYER_BRIDGE = True
+
+
 def _activation(name):
     if callable(name):
         return name
@@ -119,6 +124,43 @@ class CrystalformerEncoderCUDA(nn.Module):
             P.value_pe_dist_wscale, P.value_pe_angle_wscale, P.value_pe_dist_coef, P.value_pe_angle_coef,
             P.symm_break_noise)
 
+    def _bridge_ready(self, x: Tensor) -> bool:
+        if not (FUSED_LAYER_BRIDGE and x.is_cuda and x.dtype == torch.float32 and x.dim() == 2):
+            return False
+        for layer in self.layers:
+            at = layer.self_attn
+            idle = lambda m: isinstance(m, nn.Identity) or not self.training or getattr(m, "p", 0.0) == 0.0
+            if not (isinstance(layer.norm1, nn.Identity) and isinstance(layer.norm2, nn.Identity)
+                    and layer.activation is F.relu and idle(layer.dropout) and idle(layer.dropout1)
+                    and idle(layer.dropout2) and at.fused_inputs_ready() and at.vdim == self.d_model
+                    and cuda_funcs.LayerBridgeHIP.supported(self.d_model, layer.linear1.out_features, at.num_heads)
+                    and layer.linear1.weight.dtype == torch.float32):
+                return False
+        return True
+
+    def _forward_bridged(self, x: Tensor, batch: Tensor, geo, trans: Tensor, this_epoch) -> Tensor:
+        """The layers as: input projection of the first, then per layer the attention core and ONE launch
+        for all that follows it up to the next core (same arithmetic as the modules' own forward)."""
+        layers = self.layers
+        q, k, v, a = layers[0].self_attn.project_inputs(x)
+        for n, layer in enumerate(layers):
+            at = layer.self_attn
+            core, _ = at.attention_core(q, k, v, a, batch, batch, geo.edges, geo.rpos, None, trans, geo.rvlen,
+                                        this_epoch, True)
+            if n + 1 < len(layers):
+                stacked, in_bias, lw, gs, H, c1, lb, c2, q_scale, qkv_w = layers[n + 1].self_attn.bridge_arguments()
+            else:
+                stacked = in_bias = lw = gs = None
+                H, (c1, lb, c2), q_scale, qkv_w = at.num_heads, at._gauss_constants(), 1.0, ()
+            out = cuda_funcs.LayerBridgeHIP.apply(
+                core, x, at.out_proj.weight, at.out_proj.bias, layer.linear1.weight, layer.linear1.bias,
+                layer.linear2.weight, layer.linear2.bias, stacked, in_bias, lw, gs, H, c1, lb, c2, q_scale, *qkv_w)
+            if n + 1 < len(layers):
+                x, q, k, v, a = out
+            else:
+                x, = out
+        return x
+
     def forward(self, src: Tensor, pos: Tensor, batch: Tensor, trans: Tensor, sizes: Tensor,
                 onehot: Tensor = None, this_epoch: int = None, num_pairs: int = None) -> Tensor:
         """Reference: models/indexed_latticeformer_encoder.py:699-742.  ``num_pairs`` (sum of
@@ -133,9 +175,12 @@ class CrystalformerEncoderCUDA(nn.Module):
         if geo.atom_start is not None and sizes is not None:
             cuda_funcs.seed_atom_start(sizes, geo.atom_start)
         x = src
-        for layer in self.layers:
-            # rvecs: the lengths of the reciprocal vectors are all the layers use, computed once here
-            x = layer(x, batch, geo.edges, geo.rpos, None, trans, None, geo.rvlen, geo.vcell, onehot, this_epoch)
+        if self._bridge_ready(x):
+            x = self._forward_bridged(x, batch, geo, trans, this_epoch)
+        else:
+            for layer in self.layers:
+                # rvecs: the lengths of the reciprocal vectors are all the layers use, computed once here
+                x = layer(x, batch, geo.edges, geo.rpos, None, trans, None, geo.rvlen, geo.vcell, onehot, this_epoch)
         if self.norm is not None:
             x = self.norm(x)
         return x
