@@ -61,7 +61,7 @@ EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_fram
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
            "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
            "cfh_crystal_geometry", "cfh_small_linear_forward", "cfh_small_linear_dx", "cfh_linear_weight_bias_grad", "cfh_linear_weight_bias_grad_batch", "cfh_attention_inputs_forward",
-           "cfh_attention_inputs_backward", "cfh_layer_bridge_forward")
+           "cfh_attention_inputs_backward", "cfh_layer_bridge_forward", "cfh_layer_bridge_backward")
 
 _lib = None
 _lock = threading.Lock()
@@ -103,6 +103,8 @@ def load():
         lib.cfh_layer_bridge_forward.restype = ctypes.c_int
         lib.cfh_layer_bridge_forward.argtypes = ([_P, _P, _I64, ctypes.c_int32, ctypes.c_int32] + [_P] * 10
                                                  + [ctypes.c_float] * 4 + [ctypes.c_int32] + [_P] * 9)
+        lib.cfh_layer_bridge_backward.restype = ctypes.c_int
+        lib.cfh_layer_bridge_backward.argtypes = [_P] * 7 + [_I64, ctypes.c_int32, ctypes.c_int32] + [_P] * 5
         lib.cfh_framed_pe_backward.restype = ctypes.c_int
         lib.cfh_framed_pe_backward.argtypes = [pp] + [_P] * 17 + [_I64] * 3 + [_P] * 6 + [ctypes.c_size_t, _P]
         lib.cfh_fused_dpa_forward.restype = ctypes.c_int

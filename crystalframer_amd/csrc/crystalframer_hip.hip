@@ -750,6 +750,34 @@ int cfh_layer_bridge_forward(const float* attn, const float* x_res, int64_t N, i
     return finish_launch("layer_bridge_forward");
 }
 
+int cfh_layer_bridge_backward(const float* g_x2, const float* gqkv, const float* h, const float* Wqkv,
+                              const float* W2, const float* W1, const float* Wo, int64_t N, int32_t D, int32_t F,
+                              float* g2, float* gh, float* g1, float* g_attn, void* stream) {
+    if (N < 0 || N > 0x7fffffffLL / 1024 || D < 128 || F < 128 || D % 128 != 0 || F % 128 != 0 || D > 65536 || F > 65536)
+        return fail(CFH_EINVAL, "layer bridge: N=%lld, D=%d and F=%d must be multiples of 128", (long long)N, (int)D, (int)F);
+    if (N == 0) return CFH_OK;
+    if (!h || !W2 || !W1 || !Wo || !gh || !g1 || !g_attn || (gqkv && (!Wqkv || !g2)))
+        return fail(CFH_EINVAL, "layer bridge backward: h, the weights and gh, g1, g_attn (with gqkv: Wqkv and g2) must not be NULL");
+    const size_t lds = cfh::bridge_bwd_lds_floats(D, F) * sizeof(float);
+    if (lds > 160 * 1024) return fail(CFH_EINVAL, "layer bridge backward: D=%d, F=%d need %zu bytes of LDS", (int)D, (int)F, lds);
+    static int lds_set[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(CFH_ELAUNCH, "layer bridge: no current device");
+    if (lds_set[dev] < (int)lds) {
+        if (hipFuncSetAttribute((const void*)cfh::layer_bridge_bwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess)
+            return fail(CFH_ELAUNCH, "layer bridge backward: %zu bytes of LDS refused", lds);
+        lds_set[dev] = (int)lds;
+    }
+    cfh::BridgeBwdArgs A{};
+    A.g_x2 = g_x2; A.gqkv = gqkv; A.h = h; A.Wq = Wqkv; A.W2 = W2; A.W1 = W1; A.Wo = Wo;
+    A.g2 = g2; A.gh = gh; A.g1 = g1; A.g_attn = g_attn;
+    A.N = (int)N; A.D = D; A.F = F;
+    hipLaunchKernelGGL(cfh::layer_bridge_bwd_kernel, dim3((unsigned)((N + cfh::BR_ROWS - 1) / cfh::BR_ROWS)),
+                       dim3(64 * cfh::BR_WAVES), lds, (hipStream_t)stream, A);
+    return finish_launch("layer_bridge_backward");
+}
+
 int cfh_crystal_geometry(const float* pos, const int64_t* batch, const float* tvecs, const int64_t* sizes,
                          int64_t N, int64_t B, int64_t E, int64_t* edges, float* rpos, float* recip,
                          float* rvlen, float* vcell, int64_t* e_start, int64_t* atom_start, int32_t* order,

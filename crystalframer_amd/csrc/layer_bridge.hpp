@@ -153,4 +153,156 @@ __global__ __launch_bounds__(64 * BR_WAVES) void layer_bridge_fwd_kernel(const B
     }
 }
 
+
+// ---- backward: the input gradients of the same chain ------------------------------------------------
+//     g2 = g_x2 + gqkv Wqkv;   gh = (g2 W2) [h > 0];   g1 = g2 + gh W1;   g_attn = g1 Wo
+// (weights as stored, (out, in) row-major, so these are products with W itself: row k of W is
+// contiguous along the output column n).  Every intermediate is written out: the weight-gradient
+// launch at the end of the backward pass multiplies them with the saved activations.
+struct BridgeBwdArgs {
+    const float* g_x2;            // (N, D) or null (zero)
+    const float* gqkv;            // (N, 3 D) or null: no next layer, g2 = g_x2 (g2 is then not written)
+    const float* h;               // (N, F) forward activations (the rectifier's mask)
+    const float* Wq; const float* W2; const float* W1; const float* Wo;     // (3D, D), (D, F), (F, D), (D, D)
+    float* g2; float* gh; float* g1; float* g_attn;                         // (N, D), (N, F), (N, D), (N, D)
+    int N, D, F;
+};
+
+// Partial products of one stage: out[m][n] += sum over this wavefront's share of k of in[m][k] W[k][n].
+// The 8 wavefronts split the work as (group of 64 output columns) x (slice of K); a lane's float4 of W holds
+// the columns n0 + 4 col .. + 3 of one row k, which feed four accumulators (column n0 + 4 col + tt), and
+// the four steps of a chunk of 16 k take k = k0 + 4 kk + t (the float4 of the LDS operand holds the same four).
+// part: LDS [slices][16][O + BR_PAD].
+__device__ __forceinline__ void bridge_bwd_products(const float* in, int K, const float* __restrict__ W, int O,
+                                                    float* part) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 15, kk = lane >> 4;
+    const int ngroups = O >> 6;
+    const int slices = ngroups >= BR_WAVES ? 1 : BR_WAVES / ngroups;
+    const int ldin = K + BR_PAD, ldp = O + BR_PAD;
+    const int klen = K / slices;                      // a multiple of 32: K is a multiple of 128, slices <= 4
+    for (int unit = wave; unit < ngroups * slices; unit += BR_WAVES) {
+        const int grp = unit / slices, sl = unit - grp * slices;
+        const int n0 = 64 * grp, kbeg = sl * klen;
+        v4f_b2 acc[4];
+#pragma unroll
+        for (int tt = 0; tt < 4; tt++) acc[tt] = v4f_b2{0.f, 0.f, 0.f, 0.f};
+        const float* const arow = in + col * ldin + kbeg + 4 * kk;
+        const float* const wbase = W + (size_t)(kbeg + 4 * kk) * O + n0 + 4 * col;
+        for (int k0 = 0; k0 < klen; k0 += 32) {
+            float4 a4[2], w4[2][4];
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                a4[u] = *reinterpret_cast<const float4*>(arow + k0 + 16 * u);
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    w4[u][t] = *reinterpret_cast<const float4*>(wbase + (size_t)(k0 + 16 * u + t) * O);
+            }
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const float av[4] = {a4[u].x, a4[u].y, a4[u].z, a4[u].w};
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[t], w4[u][t].x, acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[t], w4[u][t].y, acc[1], 0, 0, 0);
+                    acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[t], w4[u][t].z, acc[2], 0, 0, 0);
+                    acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[t], w4[u][t].w, acc[3], 0, 0, 0);
+                }
+            }
+        }
+        float* const dst = part + (size_t)sl * BR_ROWS * ldp + n0 + 4 * col;
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+            *reinterpret_cast<float4*>(dst + (4 * kk + c) * ldp) = make_float4(acc[0][c], acc[1][c], acc[2][c], acc[3][c]);
+    }
+}
+
+// out[m][n] = sum over the slices of part + add (global rows r0.., or LDS, or nothing), times [mask > 0]
+// when a mask is given; to LDS (optional) and to global memory.
+__device__ __forceinline__ void bridge_bwd_finish(const float* part, int O, const float* __restrict__ add_g,
+                                                  const float* add_lds, const float* __restrict__ mask_g, int r0,
+                                                  int nrows, float* out_lds, float* __restrict__ out_g) {
+    const int ngroups = O >> 6;
+    const int slices = ngroups >= BR_WAVES ? 1 : BR_WAVES / ngroups;
+    const int ldp = O + BR_PAD;
+    for (int idx = threadIdx.x * 4; idx < BR_ROWS * O; idx += 64 * BR_WAVES * 4) {
+        const int m = idx / O, n = idx - m * O;
+        float4 v = *reinterpret_cast<const float4*>(part + m * ldp + n);
+        for (int sl = 1; sl < slices; sl++) {
+            const float4 p = *reinterpret_cast<const float4*>(part + ((size_t)sl * BR_ROWS + m) * ldp + n);
+            v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+        }
+        const bool live = m < nrows;
+        const size_t g = (size_t)(r0 + m) * O + n;
+        if (add_g && live) {
+            const float4 p = *reinterpret_cast<const float4*>(add_g + g);
+            v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+        }
+        if (add_lds) {
+            const float4 p = *reinterpret_cast<const float4*>(add_lds + m * ldp + n);
+            v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+        }
+        if (mask_g) {
+            float4 hm = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (live) hm = *reinterpret_cast<const float4*>(mask_g + g);
+            v.x = hm.x > 0.f ? v.x : 0.f; v.y = hm.y > 0.f ? v.y : 0.f;
+            v.z = hm.z > 0.f ? v.z : 0.f; v.w = hm.w > 0.f ? v.w : 0.f;
+        }
+        if (out_lds) *reinterpret_cast<float4*>(out_lds + m * ldp + n) = v;
+        if (live) *reinterpret_cast<float4*>(out_g + g) = v;
+    }
+}
+
+// LDS floats the backward kernel needs
+__host__ __device__ inline size_t bridge_bwd_lds_floats(int D, int F) {
+    const int sl_d = (D >> 6) >= BR_WAVES ? 1 : BR_WAVES / (D >> 6);
+    const int sl_f = (F >> 6) >= BR_WAVES ? 1 : BR_WAVES / (F >> 6);
+    const size_t part_d = (size_t)sl_d * BR_ROWS * (D + BR_PAD), part_f = (size_t)sl_f * BR_ROWS * (F + BR_PAD);
+    return (size_t)BR_ROWS * ((3 * D + BR_PAD) + 2 * (D + BR_PAD) + (F + BR_PAD)) + (part_d > part_f ? part_d : part_f);
+}
+
+// grid: ceil(N / 16) workgroups of 512 threads; dynamic LDS: bridge_bwd_lds_floats(D, F) floats.
+__global__ __launch_bounds__(64 * BR_WAVES) void layer_bridge_bwd_kernel(const BridgeBwdArgs P) {
+    extern __shared__ __attribute__((aligned(16))) float bridge_lds[];
+    const int D = P.D, F = P.F, Q = 3 * D;
+    float* const s_q = bridge_lds;                            // [16][3D+4] gqkv
+    float* const s_g2 = s_q + BR_ROWS * (Q + BR_PAD);         // [16][D+4]
+    float* const s_g1 = s_g2 + BR_ROWS * (D + BR_PAD);        // [16][D+4]
+    float* const s_gh = s_g1 + BR_ROWS * (D + BR_PAD);        // [16][F+4]
+    float* const part = s_gh + BR_ROWS * (F + BR_PAD);
+    const int r0 = blockIdx.x * BR_ROWS;
+    const int nrows = min(BR_ROWS, P.N - r0);
+    if (P.gqkv) {
+        for (int idx = threadIdx.x * 4; idx < BR_ROWS * Q; idx += 64 * BR_WAVES * 4) {
+            const int m = idx / Q, c = idx - m * Q;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m < nrows) v = *reinterpret_cast<const float4*>(P.gqkv + (size_t)(r0 + m) * Q + c);
+            *reinterpret_cast<float4*>(s_q + m * (Q + BR_PAD) + c) = v;
+        }
+        __syncthreads();
+        bridge_bwd_products(s_q, Q, P.Wq, D, part);
+        __syncthreads();
+        bridge_bwd_finish(part, D, P.g_x2, nullptr, nullptr, r0, nrows, s_g2, P.g2);
+    } else {
+        for (int idx = threadIdx.x * 4; idx < BR_ROWS * D; idx += 64 * BR_WAVES * 4) {
+            const int m = idx / D, c = idx - m * D;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m < nrows && P.g_x2) v = *reinterpret_cast<const float4*>(P.g_x2 + (size_t)(r0 + m) * D + c);
+            *reinterpret_cast<float4*>(s_g2 + m * (D + BR_PAD) + c) = v;
+        }
+    }
+    __syncthreads();
+    bridge_bwd_products(s_g2, D, P.W2, F, part);
+    __syncthreads();
+    bridge_bwd_finish(part, F, nullptr, nullptr, P.h, r0, nrows, s_gh, P.gh);
+    __syncthreads();
+    bridge_bwd_products(s_gh, F, P.W1, D, part);
+    __syncthreads();
+    bridge_bwd_finish(part, D, nullptr, s_g2, nullptr, r0, nrows, s_g1, P.g1);
+    __syncthreads();
+    bridge_bwd_products(s_g1, D, P.Wo, D, part);
+    __syncthreads();
+    bridge_bwd_finish(part, D, nullptr, nullptr, nullptr, r0, nrows, nullptr, P.g_attn);
+}
+
 }  // namespace cfh

@@ -899,6 +899,14 @@ class LayerBridgeHIP(torch.autograd.Function):
     (models/indexed_latticeformer_encoder.py:606-648, models/indexed_lattice_multi_head_attention_cuda.py:
     399-409, 734, 896-940)."""
 
+    FUSED_BACKWARD = True     # the four input-gradient products in one launch too (False: framework GEMMs)
+
+    @staticmethod
+    def backward_supported(D: int, F: int) -> bool:
+        sl = lambda O: 1 if O // 64 >= 8 else 8 // (O // 64)
+        part = max(sl(D) * 16 * (D + 4), sl(F) * 16 * (F + 4))
+        return (16 * ((3 * D + 4) + 2 * (D + 4) + (F + 4)) + part) * 4 <= 160 * 1024
+
     @staticmethod
     def supported(D: int, F: int, H: int) -> bool:
         wide = max(F, 3 * D)
@@ -953,17 +961,35 @@ class LayerBridgeHIP(torch.autograd.Function):
         Wo, bo, W1, b1, W2, b2, qkv_weights, in_bias, lattice_w = ctx.params
         n_fixed = 17
         g2 = None if g_x2 is None else _f32c(g_x2)
-        g_in_bias = g_lw = None
+        g_in_bias = g_lw = gqkv = None
         g_qkv_w = [None] * len(qkv_weights)
         if qkv_weights and any(g is not None for g in (g_qs, g_k, g_v, g_a)):
             gqkv, g_lw = _attention_inputs_grads(qkv, w, gs, ctx.consts, lattice_w, g_qs, g_k, g_v, g_a)
-            g2 = gqkv.matmul(Wq) if g2 is None else torch.addmm(g2, gqkv, Wq)      # the residual rides on the GEMM
             g_qkv_w, g_in_bias = _linear_param_grads(x2, gqkv, qkv_weights, in_bias)
-        if g2 is None:
+        if g2 is None and gqkv is None:
             return (None,) * (n_fixed + len(qkv_weights))
-        gh = torch.ops.aten.threshold_backward(g2.matmul(W2_c), h, 0.0)
-        g1 = torch.addmm(g2, gh, W1_c)
-        g_attn = g1.matmul(Wo_c)
+        N, D = attn.shape
+        F = W1_c.shape[0]
+        dev = attn.device
+        if LayerBridgeHIP.FUSED_BACKWARD and LayerBridgeHIP.backward_supported(D, F):
+            lib = _lib.load()
+            g2_out = torch.empty((N, D), dtype=torch.float32, device=dev) if gqkv is not None else None
+            gh = torch.empty((N, F), dtype=torch.float32, device=dev)
+            g1 = torch.empty((N, D), dtype=torch.float32, device=dev)
+            g_attn = torch.empty((N, D), dtype=torch.float32, device=dev)
+            with torch.cuda.device(dev), _timed("layer_bridge_backward", dev):
+                rc = lib.cfh_layer_bridge_backward(_lib.ptr(g2), _lib.ptr(gqkv), _lib.ptr(h), _lib.ptr(Wq), _lib.ptr(W2_c),
+                                                   _lib.ptr(W1_c), _lib.ptr(Wo_c), N, D, F, _lib.ptr(g2_out), _lib.ptr(gh),
+                                                   _lib.ptr(g1), _lib.ptr(g_attn), _lib.current_stream_ptr(dev))
+            _lib.check(rc, "cfh_layer_bridge_backward")
+            if gqkv is not None:
+                g2 = g2_out
+        else:
+            if gqkv is not None:
+                g2 = gqkv.matmul(Wq) if g2 is None else torch.addmm(g2, gqkv, Wq)
+            gh = torch.ops.aten.threshold_backward(g2.matmul(W2_c), h, 0.0)
+            g1 = torch.addmm(g2, gh, W1_c)
+            g_attn = g1.matmul(Wo_c)
         (gW2,), gb2 = _linear_param_grads(h, g2, (W2,), b2)
         (gW1,), gb1 = _linear_param_grads(x1, gh, (W1,), b1)
         (gWo,), gbo = _linear_param_grads(attn, g1, (Wo,), bo)

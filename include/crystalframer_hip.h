@@ -332,6 +332,21 @@ int cfh_layer_bridge_forward(const float* attn, const float* x_res, int64_t N, i
                              void* stream);
 
 /*
+ * Input gradients of the chain of cfh_layer_bridge_forward in one launch:
+ *   g2 (N,D) = g_x2 + gqkv Wqkv;  gh (N,F) = (g2 W2) where h > 0, else 0;  g1 (N,D) = g2 + gh W1  (the
+ *   gradient of x_res and of x1);  g_attn (N,D) = g1 Wo.
+ * g_x2 may be NULL (zero).  gqkv NULL (no next layer): g2 = g_x2 and g2 is not written.  gqkv is what
+ * cfh_attention_inputs_backward returns.  All four results are outputs because the weight gradients are
+ * their products with the saved activations (cfh_linear_weight_bias_grad_batch: dWqkv = gqkv^T x2,
+ * dW2 = g2^T h, dW1 = gh^T x1, dWo = g1^T attn).  D, F multiples of 128; returns CFH_EINVAL when D and F
+ * need more LDS than a CU has (the caller then uses GEMMs).  Replaces the framework's autograd of the same
+ * modules (eight launches per layer).
+ */
+int cfh_layer_bridge_backward(const float* g_x2, const float* gqkv, const float* h, const float* Wqkv,
+                              const float* W2, const float* W1, const float* Wo, int64_t N, int32_t D, int32_t F,
+                              float* g2, float* gh, float* g1, float* g_attn, void* stream);
+
+/*
  * What lies between the stacked q/k/v projection of a layer and its kernels, one launch each way.
  * Forward: qkv (N, 3 H Dh), rows = [query | key | value];  qs = query * q_scale, k, v (N,H,Dh) contiguous,
  *   a (N,H) = ((1 - lb) elu(c1 alpha') + 1) c2  with alpha = query_h . lattice_w_h and

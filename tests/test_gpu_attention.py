@@ -439,3 +439,15 @@ def test_layer_bridge_matches_framework_chain(N, has_next, normalised, with_bias
         t.grad = None
     (run()[0] * f32(g[0])).sum().backward()
     assert t32["attn"].grad is not None and t32["W2"].grad is not None
+    # the input gradients by framework GEMMs instead of the one launch: same numbers
+    LB = cf.cuda_funcs.LayerBridgeHIP
+    LB.FUSED_BACKWARD = False
+    try:
+        for t in t32.values():
+            t.grad = None
+        outs = run()
+        sum((o * f32(gi)).sum() for o, gi in zip(outs, g)).backward()
+    finally:
+        LB.FUSED_BACKWARD = True
+    for n in used:
+        assert Hh.rel_err(t32[n].grad, t64[n].grad) < 2e-5, n
