@@ -412,6 +412,7 @@ class RealEncodingWithMaxFramesFuncHIP(torch.autograd.Function):
                                           wscale, W_k, W_k1, W_k2, W_k3, None, dim_angle_enc, value_pe_angle_scale,
                                           cos_abs, length_rbf_mul, angle_rbf_mul, rvlen_n, cutoff_radius)
         ctx.mark_non_differentiable(frames)
+        ctx.set_materialize_grads(False)       # no zero tensor per pass for the gradient of the frames
         return z, v, frames
 
     @staticmethod
