@@ -190,7 +190,7 @@ def main():
     lib_ms_per_step = sum(sum(v) for v in per_kernel.values()) / nprof
 
     nlaunch_bwd = max(1, len(per_kernel.get("framed_pe_backward", [])))
-    nlaunch_fwd = max(1, len(per_kernel.get("framed_pe_forward", [])))
+    nlaunch_fwd = max(1, len(per_kernel.get("framed_pe_forward", [])) + len(per_kernel.get("frame_axes_framed_pe_forward", [])))
     bwd_eval = stats["bwd_evaluated"] / nlaunch_bwd          # terms evaluated per launch
     bwd_box = stats["bwd_in_box"] / nlaunch_bwd              # terms in the reference's boxes per launch
     bwd_pairs = stats["bwd_pairs"] / nlaunch_bwd
