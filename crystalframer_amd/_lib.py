@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
@@ -46,6 +46,15 @@ class CfhParams(ctypes.Structure):
         ("noise_seed_advance", ctypes.c_int32),
         ("reserved0", ctypes.c_int32),
     ]
+
+
+class CfhAttentionInputsGrad(ctypes.Structure):
+    """cfh_attention_inputs_grad of the C header."""
+    _fields_ = [("qkv", ctypes.c_void_p), ("lattice_w", ctypes.c_void_p), ("gauss_scale_dev", ctypes.c_void_p),
+                ("gqs", ctypes.c_void_p), ("gk", ctypes.c_void_p), ("gv", ctypes.c_void_p), ("ga", ctypes.c_void_p),
+                ("gqkv", ctypes.c_void_p), ("gw_partial", ctypes.c_void_p),
+                ("c1", ctypes.c_float), ("lb", ctypes.c_float), ("c2", ctypes.c_float), ("q_scale", ctypes.c_float),
+                ("H", ctypes.c_int32), ("reserved0", ctypes.c_int32)]
 
 
 class CfhLinearGradJob(ctypes.Structure):
@@ -104,7 +113,7 @@ def load():
         lib.cfh_layer_bridge_forward.argtypes = ([_P, _P, _I64, ctypes.c_int32, ctypes.c_int32] + [_P] * 10
                                                  + [ctypes.c_float] * 4 + [ctypes.c_int32] + [_P] * 9)
         lib.cfh_layer_bridge_backward.restype = ctypes.c_int
-        lib.cfh_layer_bridge_backward.argtypes = [_P] * 7 + [_I64, ctypes.c_int32, ctypes.c_int32] + [_P] * 5
+        lib.cfh_layer_bridge_backward.argtypes = [_P] * 7 + [_I64, ctypes.c_int32, ctypes.c_int32] + [_P] * 6
         lib.cfh_framed_pe_backward.restype = ctypes.c_int
         lib.cfh_framed_pe_backward.argtypes = [pp] + [_P] * 17 + [_I64] * 3 + [_P] * 6 + [ctypes.c_size_t, _P]
         lib.cfh_fused_dpa_forward.restype = ctypes.c_int

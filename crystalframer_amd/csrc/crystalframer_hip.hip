@@ -752,12 +752,17 @@ int cfh_layer_bridge_forward(const float* attn, const float* x_res, int64_t N, i
 
 int cfh_layer_bridge_backward(const float* g_x2, const float* gqkv, const float* h, const float* Wqkv,
                               const float* W2, const float* W1, const float* Wo, int64_t N, int32_t D, int32_t F,
-                              float* g2, float* gh, float* g1, float* g_attn, void* stream) {
+                              float* g2, float* gh, float* g1, float* g_attn, const cfh_attention_inputs_grad* ai,
+                              void* stream) {
     if (N < 0 || N > 0x7fffffffLL / 1024 || D < 128 || F < 128 || D % 128 != 0 || F % 128 != 0 || D > 65536 || F > 65536)
         return fail(CFH_EINVAL, "layer bridge: N=%lld, D=%d and F=%d must be multiples of 128", (long long)N, (int)D, (int)F);
     if (N == 0) return CFH_OK;
-    if (!h || !W2 || !W1 || !Wo || !gh || !g1 || !g_attn || (gqkv && (!Wqkv || !g2)))
+    if (!h || !W2 || !W1 || !Wo || !gh || !g1 || !g_attn || ((gqkv || ai) && (!Wqkv || !g2)))
         return fail(CFH_EINVAL, "layer bridge backward: h, the weights and gh, g1, g_attn (with gqkv: Wqkv and g2) must not be NULL");
+    if (ai && (gqkv || !ai->qkv || !ai->lattice_w || !ai->gqkv || !ai->gw_partial || ai->H < 1 || ai->H * cfh::DH != D ||
+               cfh::BR_ROWS * ai->H > 64 * cfh::BR_WAVES))
+        return fail(CFH_EINVAL, "layer bridge backward: attention-input gradients need qkv, lattice_w, gqkv, gw_partial, "
+                                "D = 16 H, and no gqkv argument");
     const size_t lds = cfh::bridge_bwd_lds_floats(D, F) * sizeof(float);
     if (lds > 160 * 1024) return fail(CFH_EINVAL, "layer bridge backward: D=%d, F=%d need %zu bytes of LDS", (int)D, (int)F, lds);
     static int lds_set[64] = {0};
@@ -773,6 +778,12 @@ int cfh_layer_bridge_backward(const float* g_x2, const float* gqkv, const float*
     A.g_x2 = g_x2; A.gqkv = gqkv; A.h = h; A.Wq = Wqkv; A.W2 = W2; A.W1 = W1; A.Wo = Wo;
     A.g2 = g2; A.gh = gh; A.g1 = g1; A.g_attn = g_attn;
     A.N = (int)N; A.D = D; A.F = F;
+    if (ai) {
+        A.ai_qkv = ai->qkv; A.ai_w = ai->lattice_w; A.ai_gauss = ai->gauss_scale_dev;
+        A.ai_gqs = ai->gqs; A.ai_gk = ai->gk; A.ai_gv = ai->gv; A.ai_ga = ai->ga;
+        A.gqkv_out = ai->gqkv; A.gw_partial = ai->gw_partial; A.H = ai->H;
+        A.c1 = ai->c1; A.lb = ai->lb; A.c2 = ai->c2; A.q_scale = ai->q_scale;
+    }
     hipLaunchKernelGGL(cfh::layer_bridge_bwd_kernel, dim3((unsigned)((N + cfh::BR_ROWS - 1) / cfh::BR_ROWS)),
                        dim3(64 * cfh::BR_WAVES), lds, (hipStream_t)stream, A);
     return finish_launch("layer_bridge_backward");

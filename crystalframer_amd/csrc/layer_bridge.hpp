@@ -166,6 +166,15 @@ struct BridgeBwdArgs {
     const float* Wq; const float* W2; const float* W1; const float* Wo;     // (3D, D), (D, F), (F, D), (D, D)
     float* g2; float* gh; float* g1; float* g_attn;                         // (N, D), (N, F), (N, D), (N, D)
     int N, D, F;
+    // optional: gqkv is not given but made here from the gradients of the attention inputs (the backward of
+    // attention_inputs.hpp for the 16 rows of the block), written to gqkv_out for the weight-gradient launch
+    const float* ai_qkv;          // (N, 3 D) forward projection output; null: gqkv above is used
+    const float* ai_w; const float* ai_gauss;
+    const float* ai_gqs; const float* ai_gk; const float* ai_gv; const float* ai_ga;    // each may be null (zero)
+    float* gqkv_out;              // (N, 3 D)
+    float* gw_partial;            // (blocks, D): this block's sum over its rows of the lattice-weight gradient
+    int H;
+    float c1, lb, c2, q_scale;
 };
 
 // Partial products of one stage: out[m][n] += sum over this wavefront's share of k of in[m][k] W[k][n].
@@ -272,7 +281,62 @@ __global__ __launch_bounds__(64 * BR_WAVES) void layer_bridge_bwd_kernel(const B
     float* const part = s_gh + BR_ROWS * (F + BR_PAD);
     const int r0 = blockIdx.x * BR_ROWS;
     const int nrows = min(BR_ROWS, P.N - r0);
-    if (P.gqkv) {
+    if (P.ai_qkv) {
+        // gradient of the stacked projection output from the gradients of (qs, k, v, a)
+        const int ldd = D + BR_PAD;
+        float* const s_qf = s_g1;                 // [16][D+4] the forward query rows (s_g1 is free until later)
+        float* const s_ga = part;                 // [16][H]   ga da/dalpha
+        for (int idx = threadIdx.x * 4; idx < BR_ROWS * D; idx += 64 * BR_WAVES * 4) {
+            const int m = idx / D, c = idx - m * D;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m < nrows) v = *reinterpret_cast<const float4*>(P.ai_qkv + (size_t)(r0 + m) * Q + c);
+            *reinterpret_cast<float4*>(s_qf + m * ldd + c) = v;
+        }
+        __syncthreads();
+        if ((int)threadIdx.x < BR_ROWS * P.H) {
+            const int m = threadIdx.x / P.H, hh = threadIdx.x - m * P.H;
+            float galpha = 0.0f;
+            if (m < nrows && P.ai_ga) {
+                float alpha = 0.0f, scale = 1.0f;
+#pragma unroll
+                for (int d = 0; d < DH; d++) alpha = fmaf(s_qf[m * ldd + hh * DH + d], P.ai_w[hh * DH + d], alpha);
+                if (P.ai_gauss) { scale = P.ai_gauss[0]; alpha = (alpha + P.ai_gauss[1]) * scale; }
+                const float u = alpha * P.c1;
+                const float e = u > 0.0f ? u : expm1f(u);
+                const float slope = (u > 0.0f ? 1.0f : e + 1.0f) * P.c1 * scale * (1.0f - P.lb) * P.c2;
+                galpha = P.ai_ga[(size_t)(r0 + m) * P.H + hh] * slope;
+            }
+            s_ga[m * P.H + hh] = galpha;
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x * 4; idx < BR_ROWS * Q; idx += 64 * BR_WAVES * 4) {
+            const int m = idx / Q, c = idx - m * Q;
+            const int which = c / D, cc = c - which * D;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m < nrows) {
+                const float* up = which == 0 ? P.ai_gqs : (which == 1 ? P.ai_gk : P.ai_gv);
+                if (up) v = *reinterpret_cast<const float4*>(up + (size_t)(r0 + m) * D + cc);
+                if (which == 0) {
+                    const float ga = s_ga[m * P.H + (cc >> 4)];
+                    const float4 w4 = *reinterpret_cast<const float4*>(P.ai_w + cc);
+                    v.x = fmaf(ga, w4.x, v.x * P.q_scale); v.y = fmaf(ga, w4.y, v.y * P.q_scale);
+                    v.z = fmaf(ga, w4.z, v.z * P.q_scale); v.w = fmaf(ga, w4.w, v.w * P.q_scale);
+                }
+                *reinterpret_cast<float4*>(P.gqkv_out + (size_t)(r0 + m) * Q + c) = v;
+            }
+            *reinterpret_cast<float4*>(s_q + m * (Q + BR_PAD) + c) = v;
+        }
+        for (int c = threadIdx.x; c < D; c += 64 * BR_WAVES) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int m = 0; m < BR_ROWS; m++) sum = fmaf(s_ga[m * P.H + (c >> 4)], s_qf[m * ldd + c], sum);
+            P.gw_partial[(size_t)blockIdx.x * D + c] = sum;
+        }
+        __syncthreads();
+        bridge_bwd_products(s_q, Q, P.Wq, D, part);
+        __syncthreads();
+        bridge_bwd_finish(part, D, P.g_x2, nullptr, nullptr, r0, nrows, s_g2, P.g2);
+    } else if (P.gqkv) {
         for (int idx = threadIdx.x * 4; idx < BR_ROWS * Q; idx += 64 * BR_WAVES * 4) {
             const int m = idx / Q, c = idx - m * Q;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);

@@ -804,6 +804,27 @@ def linear(x: torch.Tensor, weight, bias: Optional[torch.Tensor] = None,
     return LinearHIP.apply(x, bias, stacked, relu, *weights)
 
 
+def _column_sum_grad(part, param):
+    """Gradient of ``param`` (1-D, n elements) as the column sums of ``part`` (rows, n): for a float32 leaf a
+    zero-filled view of the pass's gradient arena, filled by the weight-gradient launch at the end of the
+    backward pass; otherwise summed at once."""
+    n = part.shape[1]
+    D = _DeferredWeightGrads
+    if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
+        D.reset()                               # left over from a backward pass that raised
+    if not (KernelManager.DEFER_WEIGHT_GRADS and part.shape[0] > 0 and param is not None and param.is_leaf
+            and param.dtype == torch.float32 and param.dim() == 1):
+        return part.sum(0)
+    g = D.take(n, part.device)
+    ref = (D.arena, D.arena_off - ((n + 63) & ~63), n)
+    D.pending.append((None, part, 0, n, None, ref, None, param, None, D.mark(param)))
+    if not D.callback_queued:
+        torch.autograd.Variable._execution_engine.queue_callback(D.flush)
+        D.callback_queued = True
+        D.task_id = torch._C._current_graph_task_id()
+    return g
+
+
 def _attention_inputs_grads(qkv, w, gs, consts, w_in, gqs, gk, gv, ga):
     """Backward of the attention inputs (see AttentionInputsHIP): the gradient of the stacked projection
     output and of the lattice weights ``w_in`` (for a float32 leaf: a zero-filled view of the pass's
@@ -964,33 +985,51 @@ class LayerBridgeHIP(torch.autograd.Function):
         g2 = None if g_x2 is None else _f32c(g_x2)
         g_in_bias = g_lw = gqkv = None
         g_qkv_w = [None] * len(qkv_weights)
-        if qkv_weights and any(g is not None for g in (g_qs, g_k, g_v, g_a)):
-            gqkv, g_lw = _attention_inputs_grads(qkv, w, gs, ctx.consts, lattice_w, g_qs, g_k, g_v, g_a)
-            g_qkv_w, g_in_bias = _linear_param_grads(x2, gqkv, qkv_weights, in_bias)
-        if g2 is None and gqkv is None:
-            return (None,) * (n_fixed + len(qkv_weights))
         N, D = attn.shape
         F = W1_c.shape[0]
         dev = attn.device
-        if LayerBridgeHIP.FUSED_BACKWARD and LayerBridgeHIP.backward_supported(D, F):
+        fused = LayerBridgeHIP.FUSED_BACKWARD and LayerBridgeHIP.backward_supported(D, F)
+        with_inputs = bool(qkv_weights) and any(g is not None for g in (g_qs, g_k, g_v, g_a))
+        if with_inputs and not fused:
+            gqkv, g_lw = _attention_inputs_grads(qkv, w, gs, ctx.consts, lattice_w, g_qs, g_k, g_v, g_a)
+        if g2 is None and not with_inputs:
+            return (None,) * (n_fixed + len(qkv_weights))
+        if fused:
             lib = _lib.load()
-            g2_out = torch.empty((N, D), dtype=torch.float32, device=dev) if gqkv is not None else None
+            ai = None
+            keep = ()
+            if with_inputs:
+                # the backward of the attention inputs is made by the same launch
+                H, Dh, c1, lb, c2, q_scale = ctx.consts
+                gqkv = torch.empty((N, 3 * D), dtype=torch.float32, device=dev)
+                part = torch.empty(((N + 15) // 16, D), dtype=torch.float32, device=dev)
+                keep = tuple(None if g is None else _f32c(g) for g in (g_qs, g_k, g_v, g_a))
+                adr = lambda t: None if t is None else t.data_ptr()
+                ai = _lib.CfhAttentionInputsGrad(
+                    adr(qkv), adr(w), adr(gs), adr(keep[0]), adr(keep[1]), adr(keep[2]), adr(keep[3]), adr(gqkv),
+                    adr(part), float(c1), float(lb), float(c2), float(q_scale), H, 0)
+            g2_out = torch.empty((N, D), dtype=torch.float32, device=dev) if with_inputs else None
             gh = torch.empty((N, F), dtype=torch.float32, device=dev)
             g1 = torch.empty((N, D), dtype=torch.float32, device=dev)
             g_attn = torch.empty((N, D), dtype=torch.float32, device=dev)
             with torch.cuda.device(dev), _timed("layer_bridge_backward", dev):
-                rc = lib.cfh_layer_bridge_backward(_lib.ptr(g2), _lib.ptr(gqkv), _lib.ptr(h), _lib.ptr(Wq), _lib.ptr(W2_c),
+                rc = lib.cfh_layer_bridge_backward(_lib.ptr(g2), None, _lib.ptr(h), _lib.ptr(Wq), _lib.ptr(W2_c),
                                                    _lib.ptr(W1_c), _lib.ptr(Wo_c), N, D, F, _lib.ptr(g2_out), _lib.ptr(gh),
-                                                   _lib.ptr(g1), _lib.ptr(g_attn), _lib.current_stream_ptr(dev))
+                                                   _lib.ptr(g1), _lib.ptr(g_attn),
+                                                   None if ai is None else ctypes.byref(ai), _lib.current_stream_ptr(dev))
             _lib.check(rc, "cfh_layer_bridge_backward")
-            if gqkv is not None:
+            del keep
+            if with_inputs:
                 g2 = g2_out
+                g_lw = _column_sum_grad(part, lattice_w) if N > 0 else torch.zeros_like(w)
         else:
             if gqkv is not None:
                 g2 = gqkv.matmul(Wq) if g2 is None else torch.addmm(g2, gqkv, Wq)
             gh = torch.ops.aten.threshold_backward(g2.matmul(W2_c), h, 0.0)
             g1 = torch.addmm(g2, gh, W1_c)
             g_attn = g1.matmul(Wo_c)
+        if with_inputs:
+            g_qkv_w, g_in_bias = _linear_param_grads(x2, gqkv, qkv_weights, in_bias)
         (gW2,), gb2 = _linear_param_grads(h, g2, (W2,), b2)
         (gW1,), gb1 = _linear_param_grads(x1, gh, (W1,), b1)
         (gWo,), gbo = _linear_param_grads(attn, g1, (Wo,), bo)

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 3
+#define CFH_ABI_VERSION 4
 
 enum {
     CFH_OK = 0,
@@ -336,15 +336,32 @@ int cfh_layer_bridge_forward(const float* attn, const float* x_res, int64_t N, i
  *   g2 (N,D) = g_x2 + gqkv Wqkv;  gh (N,F) = (g2 W2) where h > 0, else 0;  g1 (N,D) = g2 + gh W1  (the
  *   gradient of x_res and of x1);  g_attn (N,D) = g1 Wo.
  * g_x2 may be NULL (zero).  gqkv NULL (no next layer): g2 = g_x2 and g2 is not written.  gqkv is what
- * cfh_attention_inputs_backward returns.  All four results are outputs because the weight gradients are
+ * cfh_attention_inputs_backward returns; with `ai` given instead (gqkv NULL), that backward is made here as
+ * well, from the gradients of (qs, k, v, a), and gqkv is an output.  All four results are outputs because the weight gradients are
  * their products with the saved activations (cfh_linear_weight_bias_grad_batch: dWqkv = gqkv^T x2,
  * dW2 = g2^T h, dW1 = gh^T x1, dWo = g1^T attn).  D, F multiples of 128; returns CFH_EINVAL when D and F
  * need more LDS than a CU has (the caller then uses GEMMs).  Replaces the framework's autograd of the same
  * modules (eight launches per layer).
  */
+typedef struct cfh_attention_inputs_grad {
+    const float* qkv;              /* (N, 3D) the forward's stacked projection output */
+    const float* lattice_w;        /* (D) */
+    const float* gauss_scale_dev;  /* device {scale, shift} or NULL */
+    const float* gqs;              /* upstream gradients of qs, k, v (N,D) and a (N,H); each may be NULL (zero) */
+    const float* gk;
+    const float* gv;
+    const float* ga;
+    float* gqkv;                   /* out (N, 3D): what cfh_attention_inputs_backward would return */
+    float* gw_partial;             /* out (ceil(N/16), D): per-block sums of the lattice-weight gradient; their
+                                      column sums are that gradient (a dW == NULL job of the batched launch) */
+    float c1, lb, c2, q_scale;
+    int32_t H;
+    int32_t reserved0;
+} cfh_attention_inputs_grad;
 int cfh_layer_bridge_backward(const float* g_x2, const float* gqkv, const float* h, const float* Wqkv,
                               const float* W2, const float* W1, const float* Wo, int64_t N, int32_t D, int32_t F,
-                              float* g2, float* gh, float* g1, float* g_attn, void* stream);
+                              float* g2, float* gh, float* g1, float* g_attn, const cfh_attention_inputs_grad* ai,
+                              void* stream);
 
 /*
  * What lies between the stacked q/k/v projection of a layer and its kernels, one launch each way.
