@@ -226,7 +226,7 @@ def main():
     }
 
     result = {
-        "metric": "crystals/s fwd+bwd, 4-layer max-frame, batch 256",
+        "metric": f"crystals/s fwd+bwd, 4-layer max-frame, batch {args.batch}",
         "value": crystals_per_s, "unit": "crystals/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
