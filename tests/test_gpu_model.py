@@ -150,3 +150,42 @@ def test_training_step_as_hip_graph_matches_eager_on_every_replay():
             assert Hh.rel_err(pg, pe.detach().cpu()) < 5e-3, n
     finally:
         KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE = saved
+
+
+def test_bridged_encoder_equals_the_modules_own_forward():
+    """The encoder as attention cores joined by the layer bridge against the same model run module by
+    module (out_proj, residual, feed-forward block, next input projection as separate calls): outputs and
+    gradients agree to float32 rounding, in training mode and under no_grad in eval mode."""
+    import crystalframer_amd as cf
+    from crystalframer_amd import encoder, latticeformer, params, synthetic
+    cf.KernelManager.SYMM_BREAK_NOISE = 0.0
+    dev = torch.device("cuda:0")
+    mp = params.ModelParams(num_layers=3, symm_break_noise=0.0)
+    cb = synthetic.make_batch(9, atoms="uniform", atoms_lo=1, atoms_hi=7, len_lo=3.0, len_hi=9.0,
+                              ang_lo=65.0, ang_hi=115.0, seed=17).to(dev)
+    torch.manual_seed(3)
+    model = latticeformer.Latticeformer(mp).to(dev)
+    model.train()
+    model(cb).sum().backward()          # first pass: stores the normalisation of alpha (module path)
+    assert model.encoder._bridge_ready(torch.zeros(1, mp.model_dim, device=dev))
+    results = []
+    for bridged in (True, False):
+        encoder.FUSED_LAYER_BRIDGE = bridged
+        try:
+            model.zero_grad(set_to_none=True)
+            out = model(cb)
+            (out.square().sum()).backward()
+            grads = {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None}
+            model.eval()
+            with torch.no_grad():
+                out_eval = model(cb)
+            model.train()
+        finally:
+            encoder.FUSED_LAYER_BRIDGE = True
+        results.append((out.detach(), out_eval, grads))
+    (o1, e1, g1), (o2, e2, g2) = results
+    assert Hh.rel_err(o1, o2.double()) < 1e-5 and Hh.rel_err(e1, e2.double()) < 1e-5
+    assert Hh.rel_err(e1, o1.double()) < 1e-5          # no dropout: eval equals training output
+    assert g1.keys() == g2.keys() and len(g1) >= 30
+    for n in g1:
+        assert Hh.rel_err(g1[n], g2[n].double()) < 1e-4, n
