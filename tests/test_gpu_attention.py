@@ -451,3 +451,15 @@ def test_layer_bridge_matches_framework_chain(N, has_next, normalised, with_bias
         LB.FUSED_BACKWARD = True
     for n in used:
         assert Hh.rel_err(t32[n].grad, t64[n].grad) < 2e-5, n
+    # weight gradients made at once instead of at the end of the pass: same numbers
+    KM = cf.KernelManager
+    KM.DEFER_WEIGHT_GRADS = False
+    try:
+        for t in t32.values():
+            t.grad = None
+        outs = run()
+        sum((o * f32(gi)).sum() for o, gi in zip(outs, g)).backward()
+    finally:
+        KM.DEFER_WEIGHT_GRADS = True
+    for n in used:
+        assert Hh.rel_err(t32[n].grad, t64[n].grad) < 2e-5, n
