@@ -807,9 +807,7 @@ int cfh_crystal_geometry(const float* pos, const int64_t* batch, const float* tv
     A.order_start = A.pair_start + (B + 1);
     A.N = (int32_t)N; A.B = (int32_t)B; A.E = E;
     hipStream_t st = (hipStream_t)stream;
-    int threads = 64;
-    while (threads < cfh::GEO_THREADS && threads < B) threads <<= 1;
-    hipLaunchKernelGGL(cfh::geometry_crystals_kernel, dim3(2), dim3(threads), 0, st, A);
+    hipLaunchKernelGGL(cfh::geometry_crystals_kernel, dim3(2), dim3(cfh::GEO_THREADS), 0, st, A);
     hipLaunchKernelGGL(cfh::geometry_atoms_kernel, dim3((unsigned)((N + 256) / 256)), dim3(256), 0, st, A);
     if (E > 0)
         hipLaunchKernelGGL(cfh::geometry_pairs_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, A);

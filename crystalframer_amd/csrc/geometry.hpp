@@ -39,7 +39,7 @@ __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const Ge
     __shared__ long long carry_a, carry_p;
     __shared__ int hist[GEO_KEYS];
     const int t = threadIdx.x;
-    const int T = blockDim.x;              // a power of two, 64 .. GEO_THREADS: no more than the crystals need
+    const int T = blockDim.x;              // GEO_THREADS
     if (blockIdx.x == 1) {
         // reciprocal lattice (same operation order as the framework expressions it replaces)
         for (int b = t; b < P.B; b += T) {
@@ -64,46 +64,62 @@ __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const Ge
     const long long n_first = t < P.B ? (long long)P.sizes[t] : 0;      // the first T sizes: used twice below
     if (t == 0) { carry_a = 0; carry_p = 0; }
     __syncthreads();
-    // exclusive prefix sums of n and n^2, GEO_THREADS crystals at a time
+    // exclusive prefix sums of n and n^2, T crystals at a time: a shuffle scan inside every wavefront, then
+    // the totals of the wavefronts before this one
+    const int wv = t >> 6, ln = t & 63, nwv = T >> 6;
     for (int b0 = 0; b0 < P.B; b0 += T) {
         const int b = b0 + t;
         const long long n = b0 == 0 ? n_first : (b < P.B ? (long long)P.sizes[b] : 0);
-        scan_a[t] = n; scan_p[t] = n * n;
-        __syncthreads();
-        for (int off = 1; off < T; off <<= 1) {
-            const long long va = t >= off ? scan_a[t - off] : 0, vp = t >= off ? scan_p[t - off] : 0;
-            __syncthreads();
-            scan_a[t] += va; scan_p[t] += vp;
-            __syncthreads();
+        long long va = n, vp = n * n;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const long long ta = __shfl_up(va, off, 64), tp = __shfl_up(vp, off, 64);
+            if (ln >= off) { va += ta; vp += tp; }
         }
+        if (ln == 63) { scan_a[wv] = va; scan_p[wv] = vp; }
+        __syncthreads();
+        long long base_a = carry_a, base_p = carry_p;
+        for (int w = 0; w < wv; w++) { base_a += scan_a[w]; base_p += scan_p[w]; }
         if (b < P.B) {
-            P.atom_start[b] = carry_a + scan_a[t] - n;
-            P.pair_start[b] = carry_p + scan_p[t] - n * n;
+            P.atom_start[b] = base_a + va - n;
+            P.pair_start[b] = base_p + vp - n * n;
         }
         __syncthreads();
-        if (t == T - 1) { carry_a += scan_a[t]; carry_p += scan_p[t]; }
+        if (t == T - 1) { carry_a = base_a + va; carry_p = base_p + vp; }
         __syncthreads();
     }
+    (void)nwv;
     if (t == 0) { P.atom_start[P.B] = carry_a; P.pair_start[P.B] = carry_p; }
 
     // work order
     if (P.B <= T) {
-        // rank by (size descending, crystal ascending): atoms of the crystals ranked before this one
-        const int n = (int)n_first;
+        // rank by (size descending, crystal ascending): atoms of the crystals ranked before this one; the
+        // candidates of a crystal are shared by T / (power of two >= B) threads
         int* const sz = reinterpret_cast<int*>(scan_p);
+        int* const before = sz + GEO_THREADS;
         __syncthreads();
-        sz[t] = n;
+        sz[t] = (int)n_first;
+        before[t] = 0;
         __syncthreads();
-        if (t < P.B) {
-            int before0 = 0, before1 = 0;
-            for (int c = 0; c + 1 < P.B; c += 2) {
+        int bp = 64;
+        while (bp < P.B) bp <<= 1;
+        const int parts = T / bp, part = t / bp, bb = t - part * bp;
+        if (bb < P.B && part < parts) {
+            const int n = sz[bb];
+            const int span = (P.B + parts - 1) / parts;
+            const int c0 = part * span, c1 = min(P.B, c0 + span);
+            int acc0 = 0, acc1 = 0;
+            int c = c0;
+            for (; c + 1 < c1; c += 2) {
                 const int m0 = sz[c], m1 = sz[c + 1];
-                before0 += (m0 > n || (m0 == n && c < t)) ? m0 : 0;
-                before1 += (m1 > n || (m1 == n && c + 1 < t)) ? m1 : 0;
+                acc0 += (m0 > n || (m0 == n && c < bb)) ? m0 : 0;
+                acc1 += (m1 > n || (m1 == n && c + 1 < bb)) ? m1 : 0;
             }
-            if (P.B & 1) { const int m = sz[P.B - 1]; before0 += (m > n || (m == n && P.B - 1 < t)) ? m : 0; }
-            P.order_start[t] = (long long)before0 + before1;
+            if (c < c1) { const int m = sz[c]; acc0 += (m > n || (m == n && c < bb)) ? m : 0; }
+            atomicAdd(&before[bb], acc0 + acc1);
         }
+        __syncthreads();
+        if (t < P.B) P.order_start[t] = (long long)before[t];
     } else {
         for (int k = t; k < GEO_KEYS; k += T) hist[k] = 0;
         __syncthreads();
