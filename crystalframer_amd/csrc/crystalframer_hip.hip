@@ -827,11 +827,16 @@ int cfh_small_linear_forward(const float* x, const float* W, const float* b, int
 }
 
 int cfh_small_linear_dx(const float* dy, const float* W, int64_t M, int64_t N, int64_t K, float* dx, void* stream) {
-    if (M < 0 || K < 1 || N < 16 || N % 16 != 0 || M > 0x7fffffffLL / 64 || N > 65536 || K > 65536)
-        return fail(CFH_EINVAL, "small linear dx: M=%lld N=%lld K=%lld (N must be a multiple of 16)", (long long)M,
-                    (long long)N, (long long)K);
+    if (M < 0 || K < 1 || N < 1 || M > 0x7fffffffLL / 64 || N > 65536 || K > 65536)
+        return fail(CFH_EINVAL, "small linear dx: M=%lld N=%lld K=%lld out of range", (long long)M, (long long)N, (long long)K);
     if (M == 0) return CFH_OK;
-    if (!dy || !W || !dx || ((uintptr_t)dy & 15)) return fail(CFH_EINVAL, "dy, W, dx must not be NULL; dy 16-byte aligned");
+    if (!dy || !W || !dx) return fail(CFH_EINVAL, "dy, W, dx must not be NULL");
+    if (N % 16 != 0 || ((uintptr_t)dy & 15)) {
+        if (N > 64) return fail(CFH_EINVAL, "small linear dx: N=%lld must be a multiple of 16 (with dy 16-byte aligned) or at most 64", (long long)N);
+        hipLaunchKernelGGL(cfh::small_linear_dx_narrow_kernel, dim3((unsigned)((M * K + 255) / 256)), dim3(256), 0,
+                           (hipStream_t)stream, dy, W, dx, (int)M, (int)N, (int)K);
+        return finish_launch("small_linear_dx");
+    }
     hipLaunchKernelGGL(cfh::small_linear_dx_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((K + 63) / 64)), dim3(256), 0,
                        (hipStream_t)stream, dy, W, dx, (int)M, (int)N, (int)K);
     return finish_launch("small_linear_dx");

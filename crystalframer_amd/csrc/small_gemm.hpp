@@ -99,4 +99,16 @@ __global__ __launch_bounds__(256) void small_linear_dx_kernel(const float* __res
     }
 }
 
+// The same for a few output features (N not a multiple of 16, e.g. the single regression target): one thread per
+// element of dx, the N terms in a loop.  grid: ceil(M K / 256) blocks of 256 threads.
+__global__ __launch_bounds__(256) void small_linear_dx_narrow_kernel(const float* __restrict__ dy, const float* __restrict__ w,
+                                                                     float* __restrict__ dx, int M, int N, int K) {
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long)M * K) return;
+    const int m = (int)(idx / K), k = (int)(idx - (long)m * K);
+    float acc = 0.0f;
+    for (int n = 0; n < N; n++) acc = fmaf(dy[(size_t)m * N + n], w[(size_t)n * K + k], acc);
+    dx[idx] = acc;
+}
+
 }  // namespace cfh

@@ -773,7 +773,7 @@ class LinearHIP(torch.autograd.Function):
         weights, bias = ctx.weights, ctx.bias
         gx = None
         if ctx.needs_input_grad[0]:
-            if ctx.small and W.shape[0] % 16 == 0 and gy.dtype == torch.float32:
+            if ctx.small and (W.shape[0] % 16 == 0 or W.shape[0] <= 64) and gy.dtype == torch.float32:
                 lib = _lib.load()
                 rows = gy.numel() // W.shape[0]
                 g2c = _f32c(gy.reshape(rows, W.shape[0]))

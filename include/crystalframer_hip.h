@@ -301,8 +301,9 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
 /*
  * Projections with few rows (one per crystal: the head after pooling), where the general GEMM runs on
  * one or two workgroups:  y (M,N) = x (M,K) W^T + b with W (N,K) as torch.nn.Linear stores it, b (N) or
- * NULL, relu != 0: max(0, .);  dx (M,K) = dy (M,N) W.  Contiguous float32; K % 16 == 0 for the forward,
- * N % 16 == 0 for dx.  Replace torch.nn.functional.linear and its input gradient (models/latticeformer.py,
+ * NULL, relu != 0: max(0, .);  dx (M,K) = dy (M,N) W.  Contiguous float32; K % 16 == 0 for the forward;
+ * for dx N % 16 == 0, or N <= 64 (a plain loop: the single regression target).  Replace
+ * torch.nn.functional.linear and its input gradient (models/latticeformer.py,
  * the MLP head after pooling).
  */
 int cfh_small_linear_forward(const float* x, const float* W, const float* b, int64_t M, int64_t N, int64_t K,

@@ -358,7 +358,7 @@ def test_few_row_projection_kernels(M, I, O, bias, relu):
         cf.KernelManager.EVENT_LOG = None
     names = {e[0] for e in events}
     assert "small_linear_forward" in names                      # the library kernels were the ones that ran
-    assert ("small_linear_dx" in names) == (O % 16 == 0)
+    assert "small_linear_dx" in names                           # few output features take the plain-loop kernel
     assert Hh.rel_err(y, y64) < 1e-5
     assert Hh.rel_err(x.grad, x64.grad) < 1e-5
     assert Hh.rel_err(w.grad, w64.grad) < 1e-5
