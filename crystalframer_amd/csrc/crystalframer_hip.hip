@@ -577,6 +577,11 @@ int cfh_crystal_mean_forward(const float* x, const int64_t* atom_start, int64_t 
         return fail(CFH_EINVAL, "sizes N=%lld B=%lld C=%lld out of range", (long long)N, (long long)B, (long long)C);
     if (B == 0 || C == 0) return CFH_OK;
     if (!atom_start || !out || (N > 0 && !x)) return fail(CFH_EINVAL, "x, atom_start and out must not be NULL");
+    if (C % 4 == 0 && C <= 1024 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+        hipLaunchKernelGGL(cfh::crystal_mean_fwd_vec_kernel, dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream, x,
+                           atom_start, (int)B, (int)C, out);
+        return finish_launch("crystal_mean_forward");
+    }
     const int threads = C >= 256 ? 256 : (C >= 128 ? 128 : 64);
     hipLaunchKernelGGL(cfh::crystal_mean_fwd_kernel, dim3((unsigned)B), dim3(threads), 0, (hipStream_t)stream, x,
                        atom_start, (int)B, (int)C, out);

@@ -262,6 +262,34 @@ __global__ void crystal_mean_fwd_kernel(const float* x, const int64_t* atom_star
     }
 }
 
+// The same for rows of C = 4 Q floats, Q <= 256, 16-byte aligned: a block of 256 threads per crystal, thread =
+// (slice of the atoms, four channels as one 16-byte load), the 256 / Q slices added up in LDS in a fixed order.
+__global__ __launch_bounds__(256) void crystal_mean_fwd_vec_kernel(const float* x, const int64_t* atom_start, int B,
+                                                                   int C, float* out) {
+    __shared__ float4 part[256];
+    const int b = blockIdx.x;
+    const int Q = C >> 2, S = 256 / Q;
+    const int q = threadIdx.x % Q, sl = threadIdx.x / Q;
+    const int64_t s = atom_start[b], t = atom_start[b + 1];
+    const float4* const x4 = reinterpret_cast<const float4*>(x);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (sl < S)
+        for (int64_t i = s + sl; i < t; i += S) {
+            const float4 v = x4[(size_t)i * Q + q];
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+    part[threadIdx.x] = acc;
+    __syncthreads();
+    if (threadIdx.x < Q) {
+        for (int k = 1; k < S; k++) {
+            const float4 v = part[k * Q + q];
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+        const float inv = t > s ? 1.0f / (float)(t - s) : 0.0f;
+        reinterpret_cast<float4*>(out)[(size_t)b * Q + q] = make_float4(acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv);
+    }
+}
+
 // gx[i, c] = gout[batch[i], c] / size of the crystal
 __global__ void crystal_mean_bwd_kernel(const float* gout, const int64_t* batch, const int64_t* atom_start,
                                         int N, int C, float* gx) {

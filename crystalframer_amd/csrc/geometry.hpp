@@ -128,10 +128,26 @@ __global__ __launch_bounds__(GEO_THREADS) void geometry_crystals_kernel(const Ge
             atomicAdd(&hist[min(n, GEO_KEYS - 1)], n);
         }
         __syncthreads();
-        // hist[k] <- atoms of the crystals with a larger key (suffix sums, serial over 2048 keys by one wavefront)
-        if (t == 0) {
-            int run = 0;
-            for (int k = GEO_KEYS - 1; k >= 0; k--) { const int h = hist[k]; hist[k] = run; run += h; }
+        // hist[k] <- atoms of the crystals with a larger key: exclusive sums from the top key downwards, two
+        // keys per thread, a shuffle scan inside every wavefront and the totals of the wavefronts before it
+        static_assert(GEO_KEYS == 2 * GEO_THREADS, "two keys per thread");
+        {
+            int* const wave_total = reinterpret_cast<int*>(scan_a);
+            const int k0 = GEO_KEYS - 1 - 2 * t;
+            const int h0 = hist[k0], h1 = hist[k0 - 1];
+            int incl = h0 + h1;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int up = __shfl_up(incl, off, 64);
+                if (ln >= off) incl += up;
+            }
+            if (ln == 63) wave_total[wv] = incl;
+            __syncthreads();
+            int base = 0;
+            for (int w = 0; w < wv; w++) base += wave_total[w];
+            const int excl = base + incl - (h0 + h1);
+            hist[k0] = excl;
+            hist[k0 - 1] = excl + h0;
         }
         __syncthreads();
         for (int b = t; b < P.B; b += T) {

@@ -164,6 +164,14 @@ def test_crystal_mean_forward_backward():
     out3 = cf.IrregularMeanCUDA.apply(x3, batch.to(dev()), None)
     ref3 = TO.crystal_mean(x3.cpu().double(), batch, 5)
     assert Hh.rel_err(out3.cpu().double(), ref3) < 1e-6
+    # rows of three 16-byte quads (the slices of a block do not fill it), a long crystal, an empty one
+    sizes12 = torch.tensor([199, 0, 1, 64])
+    batch12 = torch.repeat_interleave(torch.arange(4), sizes12)
+    x12 = torch.randn(int(sizes12.sum()), 12, device=dev())
+    out12 = cf.IrregularMeanCUDA.apply(x12, batch12.to(dev()), sizes12.to(dev()))
+    ref12 = torch.stack([x12[batch12.to(dev()) == b].cpu().double().mean(0) if sizes12[b] > 0
+                         else torch.zeros(12, dtype=torch.float64) for b in range(4)])
+    assert Hh.rel_err(out12.cpu().double(), ref12) < 1e-6
 
 
 @pytest.mark.parametrize("N,I,O,bias", [(2372, 128, 384, True), (2372, 512, 128, True), (2372, 98, 128, False),
