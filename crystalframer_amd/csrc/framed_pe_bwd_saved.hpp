@@ -141,8 +141,9 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
                     const float4 gq = reinterpret_cast<const float4*>(gpT)[p * 4 + sub];   // gpsi[p][4 cq + sub]
                     const float* sp = P.shat + (((size_t)(g0 + p) * H + h) * 4) * NBINS + lane;
                     float sk[NENC > 0 ? NENC : 1];
+                    // read once: streaming loads, so that the L2 keeps what is used again
 #pragma unroll
-                    for (int en = 0; en < NENC; en++) sk[en] = sp[en * NBINS];
+                    for (int en = 0; en < NENC; en++) sk[en] = __builtin_nontemporal_load(sp + en * NBINS);
 #pragma unroll
                     for (int en = 0; en < NENC; en++) {
                         gWacc[en * 4 + 0] = __builtin_amdgcn_mfma_f32_4x4x1f32(sk[en], gq.x, gWacc[en * 4 + 0], 0, 0, 0);
