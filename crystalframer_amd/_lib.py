@@ -14,10 +14,11 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
+FLAG_SINGLE_STREAM = 1      # cfh_params.flags: CFH_FLAG_SINGLE_STREAM
 
 
 class CfhParams(ctypes.Structure):
@@ -44,7 +45,7 @@ class CfhParams(ctypes.Structure):
         ("collect_stats", ctypes.c_int32),
         ("noise_seed_dev", ctypes.c_void_p),
         ("noise_seed_advance", ctypes.c_int32),
-        ("reserved0", ctypes.c_int32),
+        ("flags", ctypes.c_int32),
     ]
 
 

@@ -64,6 +64,31 @@ int device_cus() {
     return cus[dev];
 }
 
+// A second stream per device (default priority) with the two events that fork it from and join it to the
+// stream of a call; created by the first call that uses it on the device.  The mutex orders whole
+// fork .. join sequences of calls from different threads.
+struct SideStream { hipStream_t stream = nullptr; hipEvent_t fork = nullptr, join = nullptr; };
+std::mutex g_side_mutex;
+SideStream* side_stream() {
+    static SideStream side[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    SideStream& s = side[dev];
+    if (!s.stream) {
+        hipStream_t st = nullptr;
+        hipEvent_t f = nullptr, j = nullptr;
+        if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) return nullptr;
+        if (hipEventCreateWithFlags(&f, hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&j, hipEventDisableTiming) != hipSuccess) {
+            if (f) (void)hipEventDestroy(f);
+            (void)hipStreamDestroy(st);
+            return nullptr;
+        }
+        s.fork = f; s.join = j; s.stream = st;
+    }
+    return &s;
+}
+
 // upper bound of the persistent wavefronts of a launch (sizes the workspace): a multiple of H, no
 // more than there are items
 int launch_waves(int64_t N, int H, int per_simd = WAVES_PER_SIMD) {
@@ -354,6 +379,17 @@ int cfh_frame_axes(const cfh_params* p, const float* q, const float* k, const fl
         }                                                                                           \
     } while (0)
 
+#define CFH_DISPATCH_PE_NOGW(KERNEL, HAS_ANG)                                                       \
+    do {                                                                                            \
+        if (wide) {                                                                                 \
+            if (p->cos_abs) rc = launch_persistent(KERNEL<11, 41, true, true, HAS_ANG, false>, A, &waves, st, what);  \
+            else rc = launch_persistent(KERNEL<11, 41, false, true, HAS_ANG, false>, A, &waves, st, what);            \
+        } else {                                                                                    \
+            if (p->cos_abs) rc = launch_persistent(KERNEL<9, 33, true, true, HAS_ANG, false>, A, &waves, st, what);   \
+            else rc = launch_persistent(KERNEL<9, 33, false, true, HAS_ANG, false>, A, &waves, st, what);             \
+        }                                                                                           \
+    } while (0)
+
 // Forward of the lattice sums; with q and k also the frame search in front of it, whose item records
 // and frames the forward kernel then takes over (one prepare launch for both).
 static int framed_pe_forward_impl(const cfh_params* p, const float* q, const float* k, const float* a_ih,
@@ -484,7 +520,53 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
     }
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "framed_pe_backward";
-    if (has_len && shat) {      // the forward kept its histograms: gather-only kernel
+    if (has_len && shat && !(p->flags & CFH_FLAG_SINGLE_STREAM)) {
+        // The forward kept its histograms and the weight gradients need nothing else: they are summed by a
+        // streaming kernel of their own on a second stream while the gather-only kernel, free of their
+        // accumulators, computes the gradient of a on this one.
+        std::lock_guard<std::mutex> lock(g_side_mutex);
+        SideStream* side = side_stream();
+        if (!side) return fail(CFH_ELAUNCH, "second stream for the weight gradients could not be created");
+        int cus = device_cus();
+        if (cus <= 0) cus = 256;
+        const int nslices = (cus * 4 + p->num_heads - 1) / p->num_heads;       // one wavefront per SIMD
+        int gw_waves = nslices * p->num_heads;
+        if ((size_t)gw_waves > (size_t)waves) {      // the workspace is sized for `waves` partials
+            gw_waves = (waves / p->num_heads) * p->num_heads;
+        }
+        const int gw_slices = gw_waves / p->num_heads;
+        // the kernels of this stream first, so that their wavefronts are resident when the others arrive
+        if (hipEventRecord(side->fork, st) != hipSuccess)
+            return fail(CFH_ELAUNCH, "fork to the second stream failed: %s", hipGetErrorString(hipGetLastError()));
+        A.gw_out_n = 0;         // the weight gradients are cleared on the second stream
+        if (has_ang) CFH_DISPATCH_PE_NOGW(cfh::framed_pe_bwd_saved_kernel, true);
+        else CFH_DISPATCH_PE_NOGW(cfh::framed_pe_bwd_saved_kernel, false);
+        // second stream: clear, partial sums per wavefront, their sum; it waits for nothing but the inputs
+        const int nenc = has_ang ? 4 : 1;
+        const int per_enc = p->num_heads * cfh::DH * cfh::NBINS;
+        int rc2 = CFH_OK;
+        if (hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
+            rc2 = fail(CFH_ELAUNCH, "fork to the second stream failed: %s", hipGetErrorString(hipGetLastError()));
+        if (!rc2) {
+            hipLaunchKernelGGL(cfh::zero_outputs_kernel, dim3((per_enc + 255) / 256), dim3(256), 0, side->stream, per_enc,
+                               gW_dist, gW_axis1, gW_axis2, gW_axis3);
+            if (has_ang)
+                hipLaunchKernelGGL(cfh::gw_from_histograms_kernel<true>, dim3(gw_waves), dim3(cfh::WAVE), 0, side->stream,
+                                   shat, gpsi, (int)E, p->num_heads, gw_slices, A.gw_dist_coef, A.angle_coef, A.gw_partial);
+            else
+                hipLaunchKernelGGL(cfh::gw_from_histograms_kernel<false>, dim3(gw_waves), dim3(cfh::WAVE), 0, side->stream,
+                                   shat, gpsi, (int)E, p->num_heads, gw_slices, A.gw_dist_coef, A.angle_coef, A.gw_partial);
+            const int rslices = 16;
+            hipLaunchKernelGGL(cfh::gw_reduce_kernel, dim3((nenc * per_enc + 255) / 256, rslices), dim3(256), 0, side->stream,
+                               A.gw_partial, gw_waves, p->num_heads, nenc, rslices, gW_dist, gW_axis1, gW_axis2, gW_axis3);
+            rc2 = finish_launch("gw_from_histograms");
+            // the join is enqueued whatever happened in between: a stream that was pulled into a capture must
+            // come back to the capturing stream
+            if ((hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(st, side->join, 0) != hipSuccess) && !rc2)
+                rc2 = fail(CFH_ELAUNCH, "join of the second stream failed");
+        }
+        return rc ? rc : rc2;
+    } else if (has_len && shat) {      // the forward kept its histograms: gather-only kernel
         if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_bwd_saved_kernel, true, true);
         else CFH_DISPATCH_PE(cfh::framed_pe_bwd_saved_kernel, true, false);
     } else if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, true);

@@ -12,7 +12,9 @@ namespace cfh {
 
 constexpr int GROUP_SAVED = 8;         // pairs per group: two rounds of four rows
 
-template <int WL, int WA, bool COS_ABS, bool HAS_LEN, bool HAS_ANG>
+// WITH_GW = false leaves the weight gradients to gw_from_histograms_kernel below (launched beside this
+// kernel on a second stream): no accumulators, no histogram reads, no partials written here.
+template <int WL, int WA, bool COS_ABS, bool HAS_LEN, bool HAS_ANG, bool WITH_GW = true>
 __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelArgs P) {
     __shared__ float4 tab[BWD_TCAP];
     __shared__ uint16_t list[BWD_LISTCAP];
@@ -33,13 +35,15 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
 
     // lane k: W_enc[h, c, k] for all (enc, c); accumulators of the weight gradients
     float Wt[NENC > 0 ? NENC * DH : 1];
-    v4f_b gWacc[NENC > 0 ? NENC * 4 : 1];
+    v4f_b gWacc[(NENC > 0 && WITH_GW) ? NENC * 4 : 1];
 #pragma unroll
     for (int en = 0; en < NENC; en++) {
 #pragma unroll
         for (int c = 0; c < DH; c++) Wt[en * DH + c] = P.W[en][((size_t)h * DH + c) * NBINS + lane];
+        if constexpr (WITH_GW) {
 #pragma unroll
-        for (int cq = 0; cq < 4; cq++) gWacc[en * 4 + cq] = v4f_b{0.f, 0.f, 0.f, 0.f};
+            for (int cq = 0; cq < 4; cq++) gWacc[en * 4 + cq] = v4f_b{0.f, 0.f, 0.f, 0.f};
+        }
     }
     const BasisConsts bc = P.bc;
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
@@ -136,7 +140,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
 
         // ---- weight gradients of the ng pairs of the finished group, histograms from the forward pass
         auto gw_update = [&](int g0, int ng) {
-            if (NENC > 0) {
+            if constexpr (NENC > 0 && WITH_GW) {
                 for (int p = 0; p < ng; p++) {
                     const float4 gq = reinterpret_cast<const float4*>(gpT)[p * 4 + sub];   // gpsi[p][4 cq + sub]
                     const float* sp = P.shat + (((size_t)(g0 + p) * H + h) * 4) * NBINS + lane;
@@ -340,7 +344,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
 
     // per-wavefront partials of the weight gradients, (wave, enc, c, k): accumulator (enc, cq),
     // lane (blk, sub), component r is gW_enc[c = 4 cq + sub][k = 4 blk + r]
-    if (NENC > 0) {
+    if constexpr (NENC > 0 && WITH_GW) {
         float* dst = P.gw_partial + (size_t)blockIdx.x * 4 * DH * NBINS;
 #pragma unroll
         for (int en = 0; en < NENC; en++) {
@@ -351,6 +355,64 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
                 *reinterpret_cast<float4*>(dst + (en * DH + 4 * cq + sub) * NBINS + 4 * blk) =
                     make_float4(acc[0] * sc, acc[1] * sc, acc[2] * sc, acc[3] * sc);
             }
+        }
+    }
+}
+
+// The weight gradients from the kept histograms alone,
+//     gW_enc[h, c, k] = sum over the pairs e of gpsi[e, h, c] shat[e, h, enc, k],
+// a stream of 1 KB + 64 B per (pair, head) with nothing else to compute: launched on a second stream beside
+// framed_pe_bwd_saved_kernel<..., false>, whose wavefronts leave a quarter of the registers of every SIMD
+// free, it overlaps its memory traffic with their arithmetic.  Workgroup w (one wavefront) serves head
+// w % H and the pairs of slice w / H; lane = bin for the histogram operand, 4 pairs in flight; partials
+// in the layout gw_reduce_kernel sums.  grid: H * nslices.
+constexpr int GWH_UNROLL = 4;
+template <bool HAS_ANG>
+__global__ __launch_bounds__(WAVE) void gw_from_histograms_kernel(const float* __restrict__ shat,
+                                                                  const float* __restrict__ gpsi, int E, int H,
+                                                                  int nslices, float dist_scale, float angle_scale,
+                                                                  float* __restrict__ partial) {
+    constexpr int NENC = HAS_ANG ? 4 : 1;
+    const int lane = threadIdx.x;
+    const int sub = lane & 3, blk = lane >> 2;
+    const int h = blockIdx.x % H, slice = blockIdx.x / H;
+    const int per = (E + nslices - 1) / nslices;
+    const int e0 = min(E, slice * per), e1 = min(E, e0 + per);
+    v4f_b acc[NENC * 4];
+#pragma unroll
+    for (int u = 0; u < NENC * 4; u++) acc[u] = v4f_b{0.f, 0.f, 0.f, 0.f};
+    for (int e = e0; e < e1; e += GWH_UNROLL) {
+        float sk[GWH_UNROLL][NENC];
+        float gq[GWH_UNROLL][4];
+#pragma unroll
+        for (int u = 0; u < GWH_UNROLL; u++) {
+            const bool live = e + u < e1;
+            const size_t row = (size_t)(live ? e + u : e) * H + h;
+            const float* sp = shat + row * 4 * NBINS + lane;
+            const float* gp = gpsi + row * DH + sub;
+#pragma unroll
+            for (int en = 0; en < NENC; en++) sk[u][en] = live ? __builtin_nontemporal_load(sp + en * NBINS) : 0.0f;
+#pragma unroll
+            for (int cq = 0; cq < 4; cq++) gq[u][cq] = live ? gp[4 * cq] : 0.0f;      // gpsi[e][4 cq + sub]
+        }
+#pragma unroll
+        for (int u = 0; u < GWH_UNROLL; u++)
+#pragma unroll
+            for (int en = 0; en < NENC; en++)
+#pragma unroll
+                for (int cq = 0; cq < 4; cq++)
+                    acc[en * 4 + cq] = __builtin_amdgcn_mfma_f32_4x4x1f32(sk[u][en], gq[u][cq], acc[en * 4 + cq], 0, 0, 0);
+    }
+    // accumulator (enc, cq), lane (blk, sub), component r is gW_enc[c = 4 cq + sub][k = 4 blk + r]
+    float* dst = partial + (size_t)blockIdx.x * 4 * DH * NBINS;
+#pragma unroll
+    for (int en = 0; en < NENC; en++) {
+        const float sc = en == 0 ? dist_scale : angle_scale;
+#pragma unroll
+        for (int cq = 0; cq < 4; cq++) {
+            const v4f_b a = acc[en * 4 + cq];
+            *reinterpret_cast<float4*>(dst + (en * DH + 4 * cq + sub) * NBINS + 4 * blk) =
+                make_float4(a[0] * sc, a[1] * sc, a[2] * sc, a[3] * sc);
         }
     }
 }

@@ -40,6 +40,9 @@ class KernelManager:
     # keep the forward's window histograms (E,H,4,64 float32, 1 KB per (pair, head)) for the backward
     # pass, which then gathers only: about a third less backward time for 244 MB per layer at batch 256
     SAVE_HISTOGRAMS: bool = True
+    # with the histograms kept: their weight gradients in a streaming kernel on a second stream of the
+    # library beside the gather-only backward kernel (False: one kernel on the caller's stream)
+    SECOND_STREAM: bool = True
     GRAD_COEF_QUIRK: bool = False
     # weight / bias gradients of the linear layers (leaf parameters): all layers of a backward pass in
     # one launch when the pass ends, instead of one launch per layer as the gradient is reached
@@ -96,6 +99,7 @@ def _params(H: int, Dh: int, K: int, A: int, cos_abs: int, dist_max: float, wsca
     p.noise_seed_advance = 1          # every frame search advances the device word itself
     p.grad_coef_quirk = int(bool(KernelManager.GRAD_COEF_QUIRK))
     p.collect_stats = int(bool(KernelManager.COLLECT_STATS))
+    p.flags = 0 if KernelManager.SECOND_STREAM else _lib.FLAG_SINGLE_STREAM
     return p
 
 

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 4
+#define CFH_ABI_VERSION 5
 
 enum {
     CFH_OK = 0,
@@ -84,8 +84,15 @@ typedef struct cfh_params {
                                 replays to draw fresh noise; NULL: noise_seed alone              */
     int32_t noise_seed_advance; /* 1: every frame search adds one to *noise_seed_dev after reading it
                                 (in its own launch, so a replayed graph needs no extra kernel)   */
-    int32_t reserved0;
+    int32_t flags;           /* CFH_FLAG_* bits                                                   */
 } cfh_params;
+
+/* cfh_params.flags: with the histograms kept by the forward, cfh_framed_pe_backward sums the weight
+ * gradients in a kernel of its own on a second stream of the library (forked from and joined to the
+ * stream of the call by events, so the call stays ordered and capturable; the first such call on a
+ * device creates the stream and should not be made under capture).  This bit keeps everything in one
+ * kernel on the stream of the call instead. */
+#define CFH_FLAG_SINGLE_STREAM 1
 
 /* Version of this ABI; a mismatch with CFH_ABI_VERSION means header and library differ. */
 int cfh_abi_version(void);

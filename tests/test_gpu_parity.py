@@ -26,7 +26,7 @@ def _defaults():
     import crystalframer_amd as cf
     KM = cf.KernelManager
     saved = (KM.SYMM_BREAK_NOISE, KM.PRUNE_LOG2, KM.WINDOW_MODE, KM.GRAD_COEF_QUIRK, KM.LATTICE_RANGE, KM.MINIMUM_RANGE)
-    saved_hist = KM.SAVE_HISTOGRAMS
+    saved_hist, saved_second = KM.SAVE_HISTOGRAMS, KM.SECOND_STREAM
     KM.SYMM_BREAK_NOISE = 0.0
     KM.PRUNE_LOG2 = 24.0
     KM.WINDOW_MODE = 0
@@ -34,7 +34,7 @@ def _defaults():
     KM.LATTICE_RANGE, KM.MINIMUM_RANGE = 2, 2
     yield
     (KM.SYMM_BREAK_NOISE, KM.PRUNE_LOG2, KM.WINDOW_MODE, KM.GRAD_COEF_QUIRK, KM.LATTICE_RANGE, KM.MINIMUM_RANGE) = saved
-    KM.SAVE_HISTOGRAMS = saved_hist
+    KM.SAVE_HISTOGRAMS, KM.SECOND_STREAM = saved_hist, saved_second
 
 
 def dev():
@@ -92,6 +92,26 @@ def test_framed_pe_forward_backward_reference_windows(cos_abs, prune, save_histo
     assert Hh.rel_err(Wk.grad, Wko.grad) < 5e-5
     for x, y in zip(Wax, Waxo):
         assert Hh.rel_err(x.grad, y.grad) < 5e-5
+
+
+@pytest.mark.parametrize("angle_bins", [64, 0])
+def test_weight_gradients_on_the_second_stream_equal_the_single_kernel(angle_bins):
+    """With the histograms kept, the weight gradients come from a kernel of their own on the library's
+    second stream; one kernel on the caller's stream (cfh_params.flags) must give the same gradients."""
+    import crystalframer_amd as cf
+    P = Hh.make_problem(num_crystals=24, atoms_hi=9, seed=61)
+    res = []
+    for second in (True, False, True):
+        cf.KernelManager.SECOND_STREAM = second
+        (z, psi), a, Wk, Wax = run_pe(P, A=angle_bins)
+        (z * g(P.gz)).sum().add((psi * g(P.gpsi)).sum()).backward()
+        torch.cuda.synchronize()
+        res.append([a.grad.clone(), Wk.grad.clone()] + [w.grad.clone() for w in Wax if w is not None])
+    for x, y, x2 in zip(*res):
+        assert torch.isfinite(x).all()
+        assert Hh.rel_err(x, y) < 1e-5
+        assert Hh.rel_err(x, x2) < 1e-6      # (the partial sums are added by float atomics: order may differ)
+    assert torch.equal(res[0][0], res[1][0])     # the gradient of a is the same arithmetic in both
 
 
 def test_framed_pe_matches_c_oracle_in_reference_arithmetic():
