@@ -14,11 +14,12 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
 FLAG_SINGLE_STREAM = 1      # cfh_params.flags: CFH_FLAG_SINGLE_STREAM
+FLAG_DEFER_JOIN = 2         # cfh_params.flags: CFH_FLAG_DEFER_JOIN
 
 
 class CfhParams(ctypes.Structure):
@@ -71,7 +72,8 @@ EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_fram
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
            "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
            "cfh_crystal_geometry", "cfh_small_linear_forward", "cfh_small_linear_dx", "cfh_linear_weight_bias_grad", "cfh_linear_weight_bias_grad_batch", "cfh_attention_inputs_forward",
-           "cfh_attention_inputs_backward", "cfh_layer_bridge_forward", "cfh_layer_bridge_backward")
+           "cfh_attention_inputs_backward", "cfh_layer_bridge_forward", "cfh_layer_bridge_backward",
+           "cfh_second_stream_fork", "cfh_second_stream_get", "cfh_second_stream_join")
 
 _lib = None
 _lock = threading.Lock()
@@ -147,6 +149,12 @@ def load():
         lib.cfh_timing_enable.argtypes = [ctypes.c_int]
         lib.cfh_timing_read.restype = ctypes.c_int
         lib.cfh_timing_read.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_I64)]
+        lib.cfh_second_stream_fork.restype = ctypes.c_int
+        lib.cfh_second_stream_fork.argtypes = [_P, ctypes.POINTER(_P)]
+        lib.cfh_second_stream_get.restype = ctypes.c_int
+        lib.cfh_second_stream_get.argtypes = [ctypes.POINTER(_P)]
+        lib.cfh_second_stream_join.restype = ctypes.c_int
+        lib.cfh_second_stream_join.argtypes = [_P]
         if lib.cfh_abi_version() != ABI_VERSION:
             raise RuntimeError(f"ABI version {lib.cfh_abi_version()} of {LIB_PATH} != {ABI_VERSION}")
         _lib = lib

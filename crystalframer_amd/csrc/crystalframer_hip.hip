@@ -279,6 +279,37 @@ int cfh_abi_version(void) { return CFH_ABI_VERSION; }
 
 const char* cfh_last_error(void) { return g_err; }
 
+int cfh_second_stream_fork(void* stream, void** second) {
+    if (!second) return fail(CFH_EINVAL, "second must not be NULL");
+    std::lock_guard<std::mutex> lock(g_side_mutex);
+    SideStream* side = side_stream();
+    if (!side) return fail(CFH_ELAUNCH, "second stream could not be created");
+    if (hipEventRecord(side->fork, (hipStream_t)stream) != hipSuccess ||
+        hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
+        return fail(CFH_ELAUNCH, "fork to the second stream failed: %s", hipGetErrorString(hipGetLastError()));
+    *second = (void*)side->stream;
+    return CFH_OK;
+}
+
+int cfh_second_stream_get(void** second) {
+    if (!second) return fail(CFH_EINVAL, "second must not be NULL");
+    std::lock_guard<std::mutex> lock(g_side_mutex);
+    SideStream* side = side_stream();
+    if (!side) return fail(CFH_ELAUNCH, "second stream could not be created");
+    *second = (void*)side->stream;
+    return CFH_OK;
+}
+
+int cfh_second_stream_join(void* stream) {
+    std::lock_guard<std::mutex> lock(g_side_mutex);
+    SideStream* side = side_stream();
+    if (!side) return fail(CFH_ELAUNCH, "second stream could not be created");
+    if (hipEventRecord(side->join, side->stream) != hipSuccess ||
+        hipStreamWaitEvent((hipStream_t)stream, side->join, 0) != hipSuccess)
+        return fail(CFH_ELAUNCH, "join of the second stream failed: %s", hipGetErrorString(hipGetLastError()));
+    return CFH_OK;
+}
+
 int cfh_timing_enable(int on) {
     std::lock_guard<std::mutex> lock(g_timing_mutex);
     g_timing_on = on != 0;
@@ -562,7 +593,8 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
             rc2 = finish_launch("gw_from_histograms");
             // the join is enqueued whatever happened in between: a stream that was pulled into a capture must
             // come back to the capturing stream
-            if ((hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(st, side->join, 0) != hipSuccess) && !rc2)
+            if (!(p->flags & CFH_FLAG_DEFER_JOIN) &&
+                (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(st, side->join, 0) != hipSuccess) && !rc2)
                 rc2 = fail(CFH_ELAUNCH, "join of the second stream failed");
         }
         return rc ? rc : rc2;

@@ -360,15 +360,37 @@ def _framed_pe_backward(ctx, gz_ek, gv_ekd):
     ga = torch.empty((N, H), dtype=torch.float32, device=dev)
     gWd = torch.empty_like(Wd) if Wd is not None else None
     gWa = [torch.empty_like(w) if w is not None else None for w in (W1, W2, W3)]
-    with torch.cuda.device(dev), _timed("framed_pe_backward", dev):
-        ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
-        rc = lib.cfh_framed_pe_backward(
-            ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch),
-            _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd), _lib.ptr(W1), _lib.ptr(W2),
-            _lib.ptr(W3), _lib.ptr(frames), _lib.ptr(z), _lib.ptr(gz), _lib.ptr(gv), _lib.ptr(shat), N, E, tv.shape[0],
-            _lib.ptr(ga), _lib.ptr(gWd), _lib.ptr(gWa[0]), _lib.ptr(gWa[1]), _lib.ptr(gWa[2]),
-            _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
+    # The library runs this backward as a gather-only kernel here and a streaming kernel on its second stream.
+    # The weight gradients of the linear layers collected so far (those of the layers behind this one) go to
+    # that stream as well, behind the library's kernel, instead of waiting for the end of the pass; the join
+    # is then made here.
+    D = _DeferredWeightGrads
+    second = (shat is not None and N > 0 and not (p.flags & _lib.FLAG_SINGLE_STREAM) and bool(D.pending)
+              and D.task_id == torch._C._current_graph_task_id())
+    flags = p.flags
+    held = None
+    with torch.cuda.device(dev):
+        try:
+            if second:
+                p.flags = flags | _lib.FLAG_DEFER_JOIN
+            with _timed("framed_pe_backward", dev):
+                ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
+                rc = lib.cfh_framed_pe_backward(
+                    ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch),
+                    _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd), _lib.ptr(W1), _lib.ptr(W2),
+                    _lib.ptr(W3), _lib.ptr(frames), _lib.ptr(z), _lib.ptr(gz), _lib.ptr(gv), _lib.ptr(shat), N, E,
+                    tv.shape[0], _lib.ptr(ga), _lib.ptr(gWd), _lib.ptr(gWa[0]), _lib.ptr(gWa[1]), _lib.ptr(gWa[2]),
+                    _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
+            if second and rc == 0:
+                held = D.flush(second_stream=True)
+        finally:
+            p.flags = flags
+            if second:
+                rcj = lib.cfh_second_stream_join(_lib.current_stream_ptr(dev))
     _lib.check(rc, "cfh_framed_pe_backward")
+    if second:
+        _lib.check(rcj, "cfh_second_stream_join")
+    del held                # what the second stream read is ordered before everything that follows on this one
     gws = [g if g is None else g.reshape(s) for g, s in zip([gWd] + gWa, ctx.w_shapes)]
     return ga, gws
 
@@ -600,14 +622,20 @@ class _DeferredWeightGrads:
         cls.callback_queued = False
 
     @classmethod
-    def flush(cls):
+    def flush(cls, second_stream=False):
+        """All pending products in one launch.  ``second_stream``: now, on the library's second stream behind
+        what a cfh_framed_pe_backward call that has just been made (with its join deferred) put there, beside
+        that call's kernel on the current stream; the caller joins and keeps the list returned here -- the
+        tensors the launch reads -- until then; the arena and the callback of the end of the pass stay as
+        they are for the layers still to come."""
         pending, cls.pending = cls.pending, []
-        arenas, cls.arenas = cls.arenas, []
-        cls.arena = None
-        cls.arena_off = 0
-        cls.callback_queued = False
+        if not second_stream:
+            arenas, cls.arenas = cls.arenas, []
+            cls.arena = None
+            cls.arena_off = 0
+            cls.callback_queued = False
         if not pending:
-            return
+            return None
 
         def view(ref):           # (arena, offset, count) -> tensor
             return ref[0][ref[1]:ref[1] + ref[2]]
@@ -642,11 +670,24 @@ class _DeferredWeightGrads:
                 J.N, J.I, J.O, J.ldx, J.ldy = g2.shape[0], 1, O, 1, g2.stride(0)
             else:
                 J.N, J.I, J.O, J.ldx, J.ldy = x2.shape[0], x2.shape[1], O, x2.stride(0), g2.stride(0)
+        if second_stream:
+            if fixups:                   # these need framework kernels on the current stream: at the end of the pass
+                cls.pending = pending + cls.pending
+                return None
+            with torch.cuda.device(dev):
+                side = ctypes.c_void_p()
+                # no new fork: the stream was forked when the library call began, and what these jobs read
+                # was complete before that
+                _lib.check(lib.cfh_second_stream_get(ctypes.byref(side)), "cfh_second_stream_get")
+                rc = lib.cfh_linear_weight_bias_grad_batch(jobs, len(pending), side)
+            _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
+            return pending
         with torch.cuda.device(dev), _timed("linear_weight_bias_grad_batch", dev):
             rc = lib.cfh_linear_weight_bias_grad_batch(jobs, len(pending), _lib.current_stream_ptr(dev))
         _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
         for grad, part in fixups:
             grad.add_(part.to(grad.dtype))
+        return None
 
 
 def _linear_param_grads(x2, g2, weights, bias):

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 5
+#define CFH_ABI_VERSION 6
 
 enum {
     CFH_OK = 0,
@@ -93,6 +93,23 @@ typedef struct cfh_params {
  * device creates the stream and should not be made under capture).  This bit keeps everything in one
  * kernel on the stream of the call instead. */
 #define CFH_FLAG_SINGLE_STREAM 1
+/* cfh_framed_pe_backward leaves its second stream unjoined when it returns (only where it uses that stream):
+ * the caller adds work of its own behind the library's with cfh_second_stream_fork and then MUST call
+ * cfh_second_stream_join(stream); until then the weight gradients of the call are not ordered on `stream`. */
+#define CFH_FLAG_DEFER_JOIN 2
+
+/*
+ * The library's second stream of the current device, for a caller that has work of its own to run beside
+ * the gather-only kernel of cfh_framed_pe_backward (the Python mirror sends the weight gradients of the
+ * linear layers collected so far).  cfh_second_stream_fork makes that stream wait for everything enqueued
+ * on `stream` so far and returns it in *second; what the caller enqueues there must be joined before
+ * `stream` (or the host) relies on it, by cfh_second_stream_join(stream).  Memory the enqueued work touches
+ * must stay allocated until then.  One thread per device at a time.  No counterpart in the reference.
+ */
+int cfh_second_stream_fork(void* stream, void** second);
+/* The same stream without making it wait: for work that may run as soon as what is already on it is done. */
+int cfh_second_stream_get(void** second);
+int cfh_second_stream_join(void* stream);
 
 /* Version of this ABI; a mismatch with CFH_ABI_VERSION means header and library differ. */
 int cfh_abi_version(void);
