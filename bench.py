@@ -39,10 +39,11 @@ PEAK_TRANS_TOPS = 9.8                  # quarter-rate transcendental unit
 # (KiB per dispatch) scaled by what the same counters read for the 256 MiB device copy of --calibrate-copy
 # (FETCH_SIZE reads 128 MiB for it: factor 2.0; WRITE_SIZE reads 256 MiB: factor 1.0); see profiles/.
 # With the forward keeping its window histograms for the backward (KernelManager.SAVE_HISTOGRAMS, the default):
-# forward 3 396 KiB x 2.0 fetched + 261 808 KiB written (243.9 MB of that are the histograms, E x H x 4 x 64
-# floats); backward 144 766 KiB x 2.0 fetched (the histograms again) + 34 258 KiB written (33.5 MB of that are
-# the per-wavefront partials of the weight gradients).
-TRAFFIC_BYTES_PER_LAUNCH = {"framed_pe_backward": 331.6e6, "framed_pe_forward": 275.0e6}
+# forward 3 398 KiB x 2.0 fetched + 261 810 KiB written (243.9 MB of that are the histograms, E x H x 4 x 64
+# floats); backward: the gather-only kernel 25 477 KiB x 2.0 fetched and under 2 MB written, the weight-gradient
+# kernel beside it on the second stream 133 999 KiB x 2.0 fetched (the histograms again) + 16 384 KiB written (its
+# per-wavefront partials).
+TRAFFIC_BYTES_PER_LAUNCH = {"framed_pe_backward": 52.2e6 + 291.2e6, "framed_pe_forward": 275.0e6}
 
 
 def parse():
@@ -209,8 +210,16 @@ def main():
         "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_TFLOPS, "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
         "bound_detail": "FP32 arithmetic (vector + a little MFMA) against the published 157.3 TFLOP/s; HBM traffic "
                         "(the kept window histograms) runs at 15-18 % of the HBM peak; in practice the forward is "
-                        "limited by LDS atomic throughput and bank conflicts, the backward by instruction issue and "
-                        "memory latency at 8 wavefronts per CU",
+                        "limited by LDS atomic throughput and bank conflicts, the backward (a gather-only kernel "
+                        "with the weight-gradient kernel beside it on a second stream) by instruction issue",
+        "both_kernels": {
+            "framed_pe_forward": {"achieved": flop_fwd / t_fwd / 1e12, "frac": flop_fwd / t_fwd / 1e12 / PEAK_FP32_TFLOPS,
+                                  "avg_launch_ms": t_fwd * 1e3},
+            # the gather-only kernel's duration; the weight-gradient kernel (its share of the flop: one projection
+            # epilogue per (pair, head)) runs inside that time on the second stream
+            "framed_pe_backward": {"achieved": flop_bwd / t_bwd / 1e12, "frac": flop_bwd / t_bwd / 1e12 / PEAK_FP32_TFLOPS,
+                                   "avg_launch_ms": t_bwd * 1e3},
+        },
         "frac_of_unpacked_fp32_peak": achieved / PEAK_FP32_UNPACKED,
         "transcendental_frac": eval_dom * X_TERM / t_dom / 1e12 / PEAK_TRANS_TOPS,
         "avg_launch_ms": t_dom * 1e3,
