@@ -94,8 +94,9 @@ typedef struct cfh_params {
  * kernel on the stream of the call instead. */
 #define CFH_FLAG_SINGLE_STREAM 1
 /* cfh_framed_pe_backward leaves its second stream unjoined when it returns (only where it uses that stream):
- * the caller adds work of its own behind the library's with cfh_second_stream_fork and then MUST call
- * cfh_second_stream_join(stream); until then the weight gradients of the call are not ordered on `stream`. */
+ * the caller adds work of its own behind the library's (cfh_second_stream_get; work whose inputs were
+ * complete on `stream` before the call) and then MUST call cfh_second_stream_join(stream); until then the
+ * weight gradients of the call are not ordered on `stream`. */
 #define CFH_FLAG_DEFER_JOIN 2
 
 /*
