@@ -174,6 +174,28 @@ def test_crystal_mean_forward_backward():
     assert Hh.rel_err(out12.cpu().double(), ref12) < 1e-6
 
 
+def test_second_stream_fork_and_join_order_a_library_call():
+    """Work put on the library's second stream between fork and join is ordered like work on the caller's."""
+    import ctypes
+    from crystalframer_amd import _lib
+    lib = _lib.load()
+    sizes = torch.tensor([3, 5, 1, 40])
+    start = torch.nn.functional.pad(torch.cumsum(sizes, 0), (1, 0)).to(dev())
+    x = torch.randn(int(sizes.sum()), 128, device=dev())
+    out = torch.full((4, 128), float("nan"), device=dev())
+    x2 = x * 2.0                                        # produced on the caller's stream before the fork
+    cur = _lib.current_stream_ptr(dev())
+    side, side2 = ctypes.c_void_p(), ctypes.c_void_p()
+    _lib.check(lib.cfh_second_stream_fork(cur, ctypes.byref(side)), "fork")
+    _lib.check(lib.cfh_second_stream_get(ctypes.byref(side2)), "get")
+    assert side.value is not None and side.value == side2.value and side.value != (cur.value or 0)
+    _lib.check(lib.cfh_crystal_mean_forward(_lib.ptr(x2), _lib.ptr(start), x.shape[0], 4, 128, _lib.ptr(out), side), "mean")
+    _lib.check(lib.cfh_second_stream_join(cur), "join")
+    res = out + 0.0                                     # consumer on the caller's stream after the join
+    ref = torch.stack([x2[start[b]:start[b + 1]].mean(0) for b in range(4)])
+    assert Hh.rel_err(res, ref) < 1e-6
+
+
 @pytest.mark.parametrize("N,I,O,bias", [(2372, 128, 384, True), (2372, 512, 128, True), (2372, 98, 128, False),
                                         (37, 20, 50, True), (1, 16, 16, True), (0, 16, 32, True)])
 def test_linear_weight_and_bias_gradients(N, I, O, bias):
