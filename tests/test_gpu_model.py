@@ -189,3 +189,39 @@ def test_bridged_encoder_equals_the_modules_own_forward():
     assert g1.keys() == g2.keys() and len(g1) >= 30
     for n in g1:
         assert Hh.rel_err(g1[n], g2[n].double()) < 1e-4, n
+
+
+def test_gradients_accumulate_over_two_passes_and_match_the_single_stream_path():
+    """Weight gradients that leave for the second stream in the middle of the backward pass (those of the
+    layers behind a lattice backward) must end up where autograd accumulates: a second pass without
+    zero_grad doubles every gradient, and the pass with everything on one stream gives the same values."""
+    import crystalframer_amd as cf
+    from crystalframer_amd import latticeformer, params, synthetic
+    KM = cf.KernelManager
+    saved = (KM.SYMM_BREAK_NOISE, KM.SECOND_STREAM)
+    KM.SYMM_BREAK_NOISE = 0.0
+    dev = torch.device("cuda:0")
+    mp = params.ModelParams(num_layers=3, symm_break_noise=0.0)
+    cb = synthetic.make_batch(12, atoms="uniform", atoms_lo=1, atoms_hi=8, len_lo=3.0, len_hi=9.0,
+                              ang_lo=65.0, ang_hi=115.0, seed=23).to(dev)
+    torch.manual_seed(5)
+    model = latticeformer.Latticeformer(mp).to(dev)
+    model.train()
+    model(cb).sum().backward()          # stores the normalisation of alpha
+    try:
+        grads = {}
+        for second in (True, False):
+            KM.SECOND_STREAM = second
+            model.zero_grad(set_to_none=True)
+            model(cb).square().sum().backward()
+            once = {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None}
+            model(cb).square().sum().backward()          # accumulates into the existing .grad
+            twice = {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None}
+            assert once.keys() == twice.keys() and len(once) >= 30
+            for n in once:
+                assert Hh.rel_err(twice[n], 2.0 * once[n].double()) < 2e-5, (second, n)
+            grads[second] = once
+        for n in grads[True]:
+            assert Hh.rel_err(grads[True][n], grads[False][n].double()) < 2e-5, n
+    finally:
+        KM.SYMM_BREAK_NOISE, KM.SECOND_STREAM = saved
