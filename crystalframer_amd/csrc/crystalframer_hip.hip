@@ -75,13 +75,20 @@ SideStream* side_stream() {
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
     SideStream& s = side[dev];
     if (!s.stream) {
+        // the first call may come while the caller's stream is being captured: creating a stream and events
+        // does not touch the capture, which the relaxed mode lets this thread say
+        hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+        const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
         hipStream_t st = nullptr;
         hipEvent_t f = nullptr, j = nullptr;
-        if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess) return nullptr;
-        if (hipEventCreateWithFlags(&f, hipEventDisableTiming) != hipSuccess ||
-            hipEventCreateWithFlags(&j, hipEventDisableTiming) != hipSuccess) {
+        bool ok = hipStreamCreateWithFlags(&st, hipStreamNonBlocking) == hipSuccess;
+        ok = ok && hipEventCreateWithFlags(&f, hipEventDisableTiming) == hipSuccess &&
+             hipEventCreateWithFlags(&j, hipEventDisableTiming) == hipSuccess;
+        if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&mode);      // back to the caller's mode
+        if (!ok) {
             if (f) (void)hipEventDestroy(f);
-            (void)hipStreamDestroy(st);
+            if (st) (void)hipStreamDestroy(st);
+            (void)hipGetLastError();
             return nullptr;
         }
         s.fork = f; s.join = j; s.stream = st;

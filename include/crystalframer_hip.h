@@ -90,8 +90,8 @@ typedef struct cfh_params {
 /* cfh_params.flags: with the histograms kept by the forward, cfh_framed_pe_backward sums the weight
  * gradients in a kernel of its own on a second stream of the library (forked from and joined to the
  * stream of the call by events, so the call stays ordered and capturable; the first such call on a
- * device creates the stream and should not be made under capture).  This bit keeps everything in one
- * kernel on the stream of the call instead. */
+ * device creates the stream, under capture too).  This bit keeps everything in one kernel on the stream
+ * of the call instead. */
 #define CFH_FLAG_SINGLE_STREAM 1
 /* cfh_framed_pe_backward leaves its second stream unjoined when it returns (only where it uses that stream):
  * the caller adds work of its own behind the library's (cfh_second_stream_get; work whose inputs were

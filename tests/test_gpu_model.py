@@ -225,3 +225,57 @@ def test_gradients_accumulate_over_two_passes_and_match_the_single_stream_path()
             assert Hh.rel_err(grads[True][n], grads[False][n].double()) < 2e-5, n
     finally:
         KM.SYMM_BREAK_NOISE, KM.SECOND_STREAM = saved
+
+
+_CAPTURE_FIRST = r'''
+import sys, torch
+sys.path.insert(0, "tests"); sys.path.insert(0, ".")
+import helpers as Hh
+import crystalframer_amd as cf
+from crystalframer_amd import cuda_funcs
+cf.KernelManager.SYMM_BREAK_NOISE = 0.0
+dev = torch.device("cuda:0")
+P = Hh.make_problem(num_crystals=6, atoms_hi=5, seed=3)
+g = lambda t: t.to(dtype=torch.float32, device=dev)
+a = g(P.a).requires_grad_(True)
+Wk = g(P.W_k).requires_grad_(True)
+Wax = [g(w).requires_grad_(True) for w in P.W_ax]
+fr = [g(f) for f in P.frames]
+rpos, tv, rv, batch, edges = g(P.rpos), g(P.tvecs), g(P.rvlen), P.batch.to(dev), P.edges.to(dev)
+gz, gpsi = g(P.gz), g(P.gpsi)
+cuda_funcs.edge_schedule(edges, P.N)          # framework arithmetic only: no library call so far
+torch.cuda.synchronize()
+
+def run():
+    z, psi = cf.RealEncodingWithFramedProjFuncCUDA.apply(
+        a, rpos, None, tv, batch, edges, 64, 14.0, 1.0, Wk, Wax[0], Wax[1], Wax[2], fr[0], fr[1], fr[2],
+        64, 4.0, 0, 1.0, 1.0, rv, -3.5)
+    return torch.autograd.grad([z, psi], [a, Wk] + Wax, [gz, gpsi])
+
+side = torch.cuda.Stream()
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.stream(side):
+    with torch.cuda.graph(graph, stream=side):      # the library's first calls of this process are captured
+        out = run()
+for _ in range(2):
+    graph.replay()
+torch.cuda.synchronize()
+captured = [o.clone() for o in out]
+eager = run()
+torch.cuda.synchronize()
+for c, e in zip(captured, eager):
+    assert torch.isfinite(c).all()
+    err = float((c - e).abs().max() / e.abs().max().clamp_min(1e-30))
+    assert err < 1e-5, err
+print("CAPTURE-FIRST-OK")
+'''
+
+
+def test_the_first_backward_of_a_process_can_be_captured():
+    """The library creates its second stream on first use; that first use may be under graph capture."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "-c", _CAPTURE_FIRST], cwd=root, capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0 and "CAPTURE-FIRST-OK" in res.stdout, res.stdout[-2000:] + res.stderr[-4000:]
