@@ -3,7 +3,7 @@
 
 One "step" is one training step (forward, MSE loss, backward, AdamW update) of the 4-layer
 CrystalFramer max-frame model over one batch of 256 synthetic crystals that is already resident in
-HBM (configuration C3 of BASELINE.json; fp32, random-init weights).  Prints ONE JSON line with
+HBM (configuration C3: the 4-layer max-frame model at batch 256; fp32, random-init weights).  Prints ONE JSON line with
 crystals/s, the roofline figures of the dominant kernel measured with HIP events inside the timed
 steps, and the CPU baseline (the PyTorch restatement of the reference's pure-PyTorch formulation,
 timed on the host cores on a bounded sample of the same batch).

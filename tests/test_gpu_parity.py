@@ -3,7 +3,7 @@ oracles, on seeded synthetic crystals.  Tolerances (float32 kernels vs float64 o
 relative to the largest magnitude of the tensor compared):
 
   * same truncation windows as the oracle ........ 2e-5 forward, 5e-5 gradients
-  * 5-sigma kernel windows vs full-basis oracle .. 1e-4   (the bar BASELINE.json states)
+  * 5-sigma kernel windows vs full-basis oracle .. 1e-4   (the bar set for this path)
   * 4-sigma (reference) windows vs full basis .... 5e-4   (the reference kernels' own truncation,
                                                            exp(-8) per dropped bin)
 """
