@@ -130,7 +130,7 @@ def main():
 
     if use_graph:
         # the whole training step (geometry, 4 layers forward, loss, backward, AdamW) as ONE HIP graph:
-        # the step is ~450 small launches and Python cannot issue them as fast as the GPU retires them
+        # Python cannot issue the step's launches as fast as the GPU retires them
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -139,7 +139,7 @@ def main():
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with torch.cuda.graph(graph, stream=side):      # the stream of the warm-up: its library workspace is reused
             step()
         run_step = graph.replay
         for _ in range(2):
