@@ -162,13 +162,16 @@ class CrystalformerEncoderCUDA(nn.Module):
         return x
 
     def forward(self, src: Tensor, pos: Tensor, batch: Tensor, trans: Tensor, sizes: Tensor,
-                onehot: Tensor = None, this_epoch: int = None, num_pairs: int = None) -> Tensor:
+                onehot: Tensor = None, this_epoch: int = None, num_pairs: int = None,
+                batch_zero_based: bool = False) -> Tensor:
         """Reference: models/indexed_latticeformer_encoder.py:699-742.  ``num_pairs`` (sum of
         sizes^2) may be given when the caller knows it on the host: the geometry then needs no
-        device-to-host read, which also makes the whole forward pass capturable in a HIP graph."""
+        device-to-host read, which also makes the whole forward pass capturable in a HIP graph.
+        ``batch_zero_based``: the crystal indices are known to start at 0 (the reference subtracts batch[0])."""
         if src.size(-1) != self.d_model:
             raise RuntimeError("the feature number of src and tgt must be equal to d_model")
-        batch = batch - batch[0]
+        if not batch_zero_based:           # the caller may know that the crystal indices start at 0
+            batch = batch - batch[0]
         geo = geometry.crystal_geometry(pos, batch, trans, sizes, num_edges=num_pairs)
         cuda_funcs.seed_edge_schedule(geo.edges, geo.e_start, geo.order)
         cuda_funcs.declare_complete_blocks(geo.edges)

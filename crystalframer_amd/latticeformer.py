@@ -104,7 +104,8 @@ class Latticeformer(nn.Module):
         x = cuda_funcs.linear(data.x, self.input_embeddings.weight, self.input_embeddings.bias)
         num_pairs = getattr(data, "num_pairs", -1)
         x = self.encoder(x, data.pos, data.batch, data.trans_vec, data.sizes, this_epoch=this_epoch,
-                         num_pairs=num_pairs if num_pairs is not None and num_pairs >= 0 else None)
+                         num_pairs=num_pairs if num_pairs is not None and num_pairs >= 0 else None,
+                         batch_zero_based=bool(getattr(data, "zero_based", False)))
         x = _run_head(self.proj_before_pooling, x)
         x = self.pooling_layer(x, data.batch, data.sizes)
         return _run_head(self.mlp, x)

@@ -23,6 +23,7 @@ class CrystalBatch:
     trans_vec: torch.Tensor  # (B, 3, 3) float32
     sizes: torch.Tensor      # (B,) int64
     num_pairs: int = -1      # sum of sizes^2, known on the host (spares the model a device read); -1: unknown
+    zero_based: bool = False  # the caller knows that batch[0] == 0 (spares the model the subtraction of batch[0])
 
     def __post_init__(self):
         if self.num_pairs < 0 and not self.sizes.is_cuda:
@@ -30,7 +31,7 @@ class CrystalBatch:
 
     def to(self, device):
         return CrystalBatch(self.x.to(device), self.pos.to(device), self.batch.to(device),
-                            self.trans_vec.to(device), self.sizes.to(device), self.num_pairs)
+                            self.trans_vec.to(device), self.sizes.to(device), self.num_pairs, self.zero_based)
 
     @property
     def num_crystals(self) -> int:
@@ -84,7 +85,7 @@ def make_batch(num_crystals: int, *, atoms: str, atoms_lo: int, atoms_hi: int,
     species = torch.randint(1, species_hi + 1, (N,), generator=g)
     x = torch.zeros(N, ATOM_FEAT_DIM, dtype=torch.float32)
     x[torch.arange(N), species] = 1.0
-    return CrystalBatch(x, pos.float(), batch, trans.float(), sizes)
+    return CrystalBatch(x, pos.float(), batch, trans.float(), sizes, zero_based=True)
 
 
 # The five benchmark configurations (batch shape only; the model settings live with the caller).

@@ -279,3 +279,25 @@ def test_the_first_backward_of_a_process_can_be_captured():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     res = subprocess.run([sys.executable, "-c", _CAPTURE_FIRST], cwd=root, capture_output=True, text=True, timeout=110)
     assert res.returncode == 0 and "CAPTURE-FIRST-OK" in res.stdout, res.stdout[-2000:] + res.stderr[-4000:]
+
+
+def test_crystal_indices_with_an_offset_give_the_same_output():
+    """The reference subtracts batch[0] (a chunk of a split batch does not start at 0); a batch that is known
+    to start at 0 skips that subtraction."""
+    from crystalframer_amd import latticeformer, params, synthetic
+    dev = torch.device("cuda:0")
+    mp = params.ModelParams(num_layers=2, symm_break_noise=0.0)
+    cb = synthetic.make_batch(7, atoms="uniform", atoms_lo=1, atoms_hi=6, len_lo=3.0, len_hi=9.0,
+                              ang_lo=65.0, ang_hi=115.0, seed=31)
+    assert cb.zero_based
+    torch.manual_seed(1)
+    model = latticeformer.Latticeformer(mp).to(dev)
+    model.train()
+    model(cb.to(dev))
+    model.eval()
+    with torch.no_grad():
+        ref = model(cb.to(dev))
+        shifted = synthetic.CrystalBatch(cb.x, cb.pos, cb.batch + 5, cb.trans_vec, cb.sizes).to(dev)
+        assert not shifted.zero_based
+        out = model(shifted)
+    assert torch.equal(out, ref)
