@@ -362,36 +362,42 @@ struct KernelArgs {
 // wavefront that is not resident at launch doubles the makespan.
 constexpr int NQUEUE = 16;
 constexpr int QSTRIDE = 64;        // ints between two queue heads: each in a 256-byte block of its own
-// The lane that issues the atomic is picked through an opaque copy of the lane id: with a visible
-// `lane == 0` test here and another at the end of the caller's loop body the optimiser threads the
-// two branches and lanes 1..63 re-enter the loop on their own.
-__device__ __forceinline__ int queue_ticket(const KernelArgs& P, int h, int q) {
+// Uniformity by construction.  The wave-level operations of the persistent loops (readfirstlane, ballot,
+// DPP) must be reached by all 64 lanes together in every iteration.  The one place where a single lane
+// acts for the wavefront -- the atomic that draws a ticket -- is therefore a function of its own that is
+// never inlined: its lane-0 branch opens and closes inside that function, so the loop bodies that call it
+// contain no branch on the lane id that an optimiser could merge with another one (a visible `lane == 0`
+// test at the queue fetch and another at the stores at the end of a loop body once let the compiler thread
+// the two across the back edge, and lanes 1..63 went round the loop apart from lane 0).  Everything that
+// steers the loops -- the item index, "no more items" -- is a readfirstlane / ballot result, the same in
+// every lane.  The price: the wait for the atomic's result sits at the end of the function instead of at
+// the first use of the ticket (about a microsecond per item, hidden by the other wavefronts of the SIMD).
+__device__ __attribute__((noinline)) int queue_draw(int32_t* head) {
     int v = 0;
-    int elect = threadIdx.x;
-    asm volatile("" : "+v"(elect));
-    if (elect == 0) v = atomicAdd(P.counters + (h * NQUEUE + q) * QSTRIDE, 1);
-    return v;         // valid in lane 0; not waited for until it is used
+    if (threadIdx.x == 0) v = atomicAdd(head, 1);
+    return __builtin_amdgcn_readfirstlane(v);
+}
+__device__ __forceinline__ int queue_ticket(const KernelArgs& P, int h, int q) {
+    return queue_draw(P.counters + (h * NQUEUE + q) * QSTRIDE);      // the same value in every lane
 }
 // Next item of head h, or -1 when every queue of the head is empty.  `q` is the queue to try first
 // and is updated.
 __device__ __forceinline__ int queue_pop(const KernelArgs& P, int h, int& q) {
     for (;;) {
-        const int it = __builtin_amdgcn_readfirstlane(queue_ticket(P, h, q)) * NQUEUE + q;
+        const int it = queue_ticket(P, h, q) * NQUEUE + q;
         if (it < P.N) return it;
-        bool more = false;
-        if (threadIdx.x < NQUEUE) {
-            const int c = __hip_atomic_load(P.counters + (h * NQUEUE + (int)threadIdx.x) * QSTRIDE, __ATOMIC_RELAXED,
-                                            __HIP_MEMORY_SCOPE_AGENT);
-            more = c * NQUEUE + (int)threadIdx.x < P.N;
-        }
-        const uint64_t m = __ballot(more);
+        // all lanes load (lanes >= NQUEUE a copy of queue 0): no lane-dependent branch in front of the ballot
+        const int ql = (int)threadIdx.x & (NQUEUE - 1);
+        const int c = __hip_atomic_load(P.counters + (h * NQUEUE + ql) * QSTRIDE, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+        const uint64_t m = __ballot(c * NQUEUE + ql < P.N) & ((1ull << NQUEUE) - 1ull);
         if (m == 0) return -1;
         q = __builtin_ctzll(m);
     }
 }
 // Turns a ticket drawn earlier from queue q into an item; falls back to the other queues.
 __device__ __forceinline__ int queue_redeem(const KernelArgs& P, int h, int& q, int ticket) {
-    const int it = __builtin_amdgcn_readfirstlane(ticket) * NQUEUE + q;
+    const int it = ticket * NQUEUE + q;
     return it < P.N ? it : queue_pop(P, h, q);
 }
 __device__ __forceinline__ int first_queue(int H) { return ((int)blockIdx.x / H) % NQUEUE; }

@@ -53,3 +53,50 @@ def rel_err(x, ref):
     x, ref = x.detach(), ref.detach()
     scale = ref.abs().max().clamp_min(1e-30)
     return float((x.double().cpu() - ref.double().cpu()).abs().max() / scale.cpu())
+
+
+def elem_err(x, ref, rtol=1e-4, atol_frac=1e-6):
+    """Elementwise error in units of the allowance rtol*|ref| + atol_frac*max|ref|: the largest value of
+    |x-ref| / (rtol*|ref| + atol_frac*max|ref|) over the tensor.  <= 1 means that every element is within
+    ``rtol`` of its own reference value (small elements are given the absolute floor, a fraction
+    ``atol_frac`` of the tensor's largest magnitude)."""
+    x, ref = x.detach().double().cpu(), ref.detach().double().cpu()
+    if ref.numel() == 0:
+        return 0.0
+    allow = rtol * ref.abs() + atol_frac * ref.abs().max().clamp_min(1e-30)
+    return float(((x - ref).abs() / allow).max())
+
+
+def problem_from_batch(cb, seed=9, w_scale=0.3):
+    """Random attention operands (float64, CPU) for the crystals of a CrystalBatch."""
+    gen = torch.Generator().manual_seed(seed)
+    P = Problem()
+    P.batch, P.sizes = cb.batch, cb.sizes.tolist()
+    P.pos, P.tvecs = cb.pos.double(), cb.trans_vec.double()
+    P.edges, P.rpos, recip, P.vcell = TO.geometry(P.pos, P.tvecs, P.sizes)
+    P.rvlen = torch.norm(recip, 2, dim=-1)
+    P.N, P.E = P.pos.shape[0], P.edges.shape[1]
+    P.a = TO.gaussian_coefficient(torch.randn(P.N, H, generator=gen, dtype=torch.float64)).float().double()
+    P.q = (torch.randn(P.N, H, DH, generator=gen, dtype=torch.float64) / 4).float().double()
+    P.k = torch.randn(P.N, H, DH, generator=gen, dtype=torch.float64).float().double()
+    P.v = torch.randn(P.N, H, DH, generator=gen, dtype=torch.float64).float().double()
+    P.W_k = (torch.randn(1, H, DH, K, generator=gen, dtype=torch.float64) * w_scale).float().double()
+    P.W_ax = [(torch.randn(1, H, DH, A, generator=gen, dtype=torch.float64) * w_scale).float().double()
+              for _ in range(3)]
+    f1 = torch.nn.functional.normalize(torch.randn(P.N, H, 3, generator=gen, dtype=torch.float64), dim=-1)
+    f2 = torch.nn.functional.normalize(torch.randn(P.N, H, 3, generator=gen, dtype=torch.float64), dim=-1)
+    P.frames = [f.float().double() for f in TO.orthonormal_frame(f1, f2)]
+    return P
+
+
+def first_crystals(P, nb):
+    """The sub-problem made of the first ``nb`` crystals of P (operands sliced, weights shared)."""
+    n_at, n_e = sum(P.sizes[:nb]), sum(s * s for s in P.sizes[:nb])
+    S = Problem()
+    S.sizes = P.sizes[:nb]
+    S.N, S.E = n_at, n_e
+    S.a, S.q, S.k, S.v = P.a[:n_at], P.q[:n_at], P.k[:n_at], P.v[:n_at]
+    S.rpos, S.tvecs, S.batch, S.edges = P.rpos[:n_e], P.tvecs[:nb], P.batch[:n_at], P.edges[:, :n_e]
+    S.rvlen, S.W_k, S.W_ax = P.rvlen[:nb], P.W_k, P.W_ax
+    S.frames = [f[:n_at] for f in P.frames]
+    return S

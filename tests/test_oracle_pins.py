@@ -394,3 +394,33 @@ def test_crystal_mean():
     assert (CO.crystal_mean(x, sizes, "f64") - ref).abs().max() < 1e-14
     batch = torch.repeat_interleave(torch.arange(3), torch.tensor(sizes))
     assert (TO.crystal_mean(x, batch, 3) - ref).abs().max() < 1e-14
+
+
+# ------------------------------------------------------------------------------------------------
+# alpha -> a
+# ------------------------------------------------------------------------------------------------
+def test_gaussian_coefficient_closed_form_facts():
+    """What the formula a = [(1-lb) elu(alpha beta/(1-lb)) + 1] (-1/2 r0^-2) fixes without restating it:
+    its value at 0, its limit for alpha -> -inf (the lower bound lb of the positive function), its slope
+    for alpha > 0, and that value and slope are continuous at 0."""
+    r0, lb, beta = 1.4, 0.5, 0.1
+    c2 = -0.5 / (r0 * r0)                                  # -0.25510...
+    f = lambda x: float(TO.gaussian_coefficient(torch.tensor([x], dtype=torch.float64), r0, lb, beta))
+    assert abs(f(0.0) - c2) < 1e-15
+    assert abs(c2 - (-0.25510204081632654)) < 1e-15
+    assert abs(f(-1e4) - lb * c2) < 1e-15                  # -> lb (-1/2 r0^-2) = -0.12755...
+    assert abs(lb * c2 - (-0.12755102040816327)) < 1e-15
+    # linear with slope beta (-1/2 r0^-2) on the positive side
+    assert abs((f(7.0) - f(3.0)) / 4.0 - beta * c2) < 1e-15
+    assert abs(f(5.0) - (1.0 + beta * 5.0) * c2) < 1e-15
+    # C^1 at 0: one-sided difference quotients agree with the slope beta c2
+    h = 1e-6
+    assert abs((f(h) - f(0.0)) / h - beta * c2) < 1e-9
+    assert abs((f(0.0) - f(-h)) / h - beta * c2) < 1e-6
+    # monotone: a larger alpha gives a sharper Gaussian (more negative a), always below lb c2
+    xs = torch.linspace(-50, 50, 2001, dtype=torch.float64)
+    a = TO.gaussian_coefficient(xs, r0, lb, beta)
+    assert bool((a[1:] < a[:-1]).all()) and float(a.max()) < lb * c2 + 1e-12
+    # other constants: the limit and the slope follow lb and beta
+    a2 = TO.gaussian_coefficient(torch.tensor([-1e4, 2.0], dtype=torch.float64), 2.0, 0.25, 0.3)
+    assert abs(float(a2[0]) - 0.25 * (-0.125)) < 1e-15 and abs(float(a2[1]) - 1.6 * (-0.125)) < 1e-15
