@@ -67,7 +67,7 @@ class CfhLinearGradJob(ctypes.Structure):
 
 
 EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_frame_axis1",
-           "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_frame_axes_framed_pe_forward",
+           "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_forward_static", "cfh_frame_axes_framed_pe_forward",
            "cfh_framed_pe_backward",
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
            "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
@@ -110,6 +110,8 @@ def load():
         lib.cfh_frame_axes.argtypes = [pp] + [_P] * 10 + [_I64] * 3 + [_P, _P, ctypes.c_size_t, _P]
         lib.cfh_framed_pe_forward.restype = ctypes.c_int
         lib.cfh_framed_pe_forward.argtypes = [pp] + [_P] * 13 + [_I64] * 3 + [_P] * 5 + [ctypes.c_size_t, _P]
+        lib.cfh_framed_pe_forward_static.restype = ctypes.c_int
+        lib.cfh_framed_pe_forward_static.argtypes = [pp] + [_P] * 13 + [_I64] * 3 + [_P] * 4 + [_P]
         lib.cfh_frame_axes_framed_pe_forward.restype = ctypes.c_int
         lib.cfh_frame_axes_framed_pe_forward.argtypes = [pp] + [_P] * 14 + [_I64] * 3 + [_P] * 6 + [ctypes.c_size_t, _P]
         lib.cfh_layer_bridge_forward.restype = ctypes.c_int

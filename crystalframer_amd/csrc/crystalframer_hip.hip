@@ -501,6 +501,65 @@ int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* r
                                   workspace, workspace_bytes, stream);
 }
 
+// ---- the forward of the lattice sums with its scratch in a file-scope device array ---------------------------
+// For callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid
+// hipMalloc).  What cfh_framed_pe_forward takes through its workspace argument -- work-queue heads and one
+// 128-byte record per (atom, head) -- lives in `scratch` below, which every GPU the library runs on holds until
+// the process ends.  In host code the array's name is only a stand-in: the address the kernels get is asked for
+// once per device with hipGetSymbolAddress and kept.
+constexpr size_t STATIC_SCRATCH_BYTES = COUNTER_BYTES + (size_t)CFH_STATIC_MAX_ITEMS * cfh::REC_WORDS * sizeof(uint32_t);
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+namespace {
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[64] = {nullptr};
+// device address of `scratch` on the current device (nullptr: failure, message set)
+void* static_scratch() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        fail(CFH_EDEVICE, "no current HIP device");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        // the first call on a device may come while the caller's stream is being captured: looking up a symbol
+        // enqueues nothing, which the relaxed mode lets this thread say
+        hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+        const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&mode);
+        if (e != hipSuccess || !ptr) {
+            fail(CFH_EDEVICE, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+int cfh_framed_pe_forward_static(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,
+                                 const float* rvlen, const int64_t* batch, const int64_t* edges,
+                                 const int64_t* e_start, const int32_t* order, const float* W_dist,
+                                 const float* W_axis1, const float* W_axis2, const float* W_axis3,
+                                 const float* frames, int64_t N, int64_t E, int64_t B, float* z, float* psi,
+                                 float* d2min_out, float* shat_out, void* stream) {
+    int rc = check_params(p);
+    if (rc) return rc;
+    if (N < 0) return fail(CFH_EINVAL, "negative size N=%lld", (long long)N);
+    if (N * (int64_t)p->num_heads > (int64_t)CFH_STATIC_MAX_ITEMS)
+        return fail(CFH_EINVAL, "N * num_heads = %lld exceeds the %d (atom, head) items the static scratch holds; "
+                    "use cfh_framed_pe_forward with a workspace", (long long)(N * p->num_heads), CFH_STATIC_MAX_ITEMS);
+    if (p->collect_stats) return fail(CFH_EINVAL, "collect_stats is not available with the static scratch");
+    void* ptr = static_scratch();
+    if (!ptr) return CFH_EDEVICE;
+    // the work-queue heads are cleared by the prepare kernel of every launch; nothing else must start at zero
+    return framed_pe_forward_impl(p, nullptr, nullptr, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, W_dist,
+                                  W_axis1, W_axis2, W_axis3, frames, nullptr, N, E, B, z, psi, d2min_out, shat_out,
+                                  ptr, STATIC_SCRATCH_BYTES, stream);
+}
+
 int cfh_frame_axes_framed_pe_forward(const cfh_params* p, const float* q, const float* k, const float* a_ih,
                                      const float* rpos, const float* tvecs, const float* rvlen,
                                      const int64_t* batch, const int64_t* edges, const int64_t* e_start,

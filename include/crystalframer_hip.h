@@ -193,6 +193,25 @@ int cfh_framed_pe_forward(const cfh_params* p, const float* a_ih, const float* r
                           void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * cfh_framed_pe_forward without the workspace argument: the scratch of its kernels (work-queue heads and the
+ * per-(atom, head) records) is a file-scope device array of the library, CFH_STATIC_MAX_ITEMS records plus the
+ * queue heads (about 8.5 MB, held by every GPU the library has run on until the process ends).  It has no
+ * counterpart in the reference: it is for callers that cannot allocate device memory or hand over a workspace --
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The call allocates
+ * nothing.  Same arguments, results and errors as cfh_framed_pe_forward otherwise; N * num_heads beyond
+ * CFH_STATIC_MAX_ITEMS and collect_stats return CFH_EINVAL.  All calls on one GPU share the one array: calls
+ * that overlap on a GPU (two streams, two threads) race; calls on one stream are ordered and safe.
+ */
+#define CFH_STATIC_MAX_ITEMS 65536
+int cfh_framed_pe_forward_static(const cfh_params* p, const float* a_ih, const float* rpos,
+                                 const float* tvecs, const float* rvlen, const int64_t* batch,
+                                 const int64_t* edges, const int64_t* e_start, const int32_t* order,
+                                 const float* W_dist, const float* W_axis1, const float* W_axis2,
+                                 const float* W_axis3, const float* frames, int64_t N, int64_t E,
+                                 int64_t B, float* z, float* psi, float* d2min_out, float* shat_out,
+                                 void* stream);
+
+/*
  * cfh_frame_axes followed by cfh_framed_pe_forward with the frames it found, as the attention layer
  * calls them (models/indexed_lattice_multi_head_attention_cuda.py:666-734: compute_frame_maximum_method_,
  * then RealEncodingWithFramedProjFuncCUDA.apply): same arguments and results as the two calls (`frames`
