@@ -585,7 +585,11 @@ class _DeferredWeightGrads:
     gradients are complete when ``backward()`` / ``autograd.grad()`` return.  Only parameters that are
     leaves take part: nothing else reads their gradient before the pass ends.  If a parameter already
     had a ``.grad`` (accumulation over several passes), autograd has added the zeros to it at once and
-    the batch call adds into that ``.grad`` instead."""
+    the batch call adds into that ``.grad`` instead.  A parameter with tensor hooks or post-accumulate hooks, or
+    a pass with create_graph, is not deferred (``deferrable``): its products are made at once.  The batched
+    kernel adds its row slices with float atomics, so the last bits of the weight gradients depend on the order
+    in which the workgroups arrive: equal inputs give gradients equal to about 1e-7 relative, not bit for bit
+    (``KernelManager.DEFER_WEIGHT_GRADS = False`` does not change that; the kernel is the same)."""
     ARENA_FLOATS = 1 << 21
     pending = []            # (x2, gy2, col0, O, dW ref, bias-gradient ref, weight, bias, marks)
     arena = None
@@ -609,9 +613,34 @@ class _DeferredWeightGrads:
 
     @staticmethod
     def mark(param):
-        """Identity and version of a parameter's .grad: changes when autograd sets or adds to it."""
+        """The parameter's .grad tensor itself (kept alive, so that its identity cannot be reused by another
+        tensor) and its version: ``changed`` tells whether autograd has set or added to .grad since."""
         g = param.grad
-        return None if g is None else (id(g), g._version)
+        return None if g is None else (g, g._version)
+
+    @staticmethod
+    def changed(param, mark) -> bool:
+        g = param.grad
+        if g is None or mark is None:
+            return (g is None) != (mark is None)
+        return g is not mark[0] or g._version != mark[1]
+
+    @staticmethod
+    def deferrable(*params) -> bool:
+        """Deferring hands autograd zero-filled tensors that are completed when the pass ends.  That is only
+        sound if nothing looks at a parameter's gradient before then: a float32 leaf without tensor hooks and
+        without post-accumulate hooks (optimizer-in-backward, clipping in hooks), in a pass that does not
+        build a graph of the backward itself (create_graph)."""
+        if not KernelManager.DEFER_WEIGHT_GRADS or torch.is_grad_enabled():
+            return False
+        for w in params:
+            if w is None:
+                continue
+            if not (w.is_leaf and w.dtype == torch.float32):
+                return False
+            if getattr(w, "_backward_hooks", None) or getattr(w, "_post_accumulate_grad_hooks", None):
+                return False
+        return True
 
     @classmethod
     def reset(cls):
@@ -649,7 +678,7 @@ class _DeferredWeightGrads:
             dst_w = None if dW is None else dW[0].data_ptr() + 4 * dW[1]
             dst_b = None if db is None else db[0].data_ptr() + 4 * (db[1] + col0)
             wg = None if weight is None else weight.grad
-            if wg is not None and cls.mark(weight) != w_mark and wg.data_ptr() != dst_w:
+            if wg is not None and cls.changed(weight, w_mark) and wg.data_ptr() != dst_w:
                 # .grad was set or updated during this pass, but not by adopting our tensor: autograd
                 # copied or accumulated it (adding our zeros), so the result belongs into .grad
                 if wg.dtype == torch.float32 and wg.is_contiguous() and wg.device == dev:
@@ -658,7 +687,7 @@ class _DeferredWeightGrads:
                     fixups.append((wg, view(dW).view(wg.shape)))
             if db is not None:
                 bg = bias.grad
-                if bg is not None and cls.mark(bias) != b_mark and bg.data_ptr() != db[0].data_ptr() + 4 * db[1]:
+                if bg is not None and cls.changed(bias, b_mark) and bg.data_ptr() != db[0].data_ptr() + 4 * db[1]:
                     if bg.dtype == torch.float32 and bg.is_contiguous() and bg.device == dev:
                         dst_b = bg.data_ptr() + 4 * col0
                     elif col0 == 0:
@@ -704,8 +733,7 @@ def _linear_param_grads(x2, g2, weights, bias):
     D = _DeferredWeightGrads
     if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
         D.reset()                               # left over from a backward pass that raised
-    defer = (KernelManager.DEFER_WEIGHT_GRADS and all(w.is_leaf for w in weights)
-             and (bias is None or bias.is_leaf) and all(w.dtype == torch.float32 for w in weights))
+    defer = D.deferrable(*weights, bias) and (bias is None or bias.dtype == torch.float32)
     if defer:
         def take(n):
             v = D.take(n, dev)
@@ -857,8 +885,7 @@ def _column_sum_grad(part, param):
     D = _DeferredWeightGrads
     if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
         D.reset()                               # left over from a backward pass that raised
-    if not (KernelManager.DEFER_WEIGHT_GRADS and part.shape[0] > 0 and param is not None and param.is_leaf
-            and param.dtype == torch.float32 and param.dim() == 1):
+    if not (part.shape[0] > 0 and param is not None and param.dim() == 1 and D.deferrable(param)):
         return part.sum(0)
     g = D.take(n, part.device)
     ref = (D.arena, D.arena_off - ((n + 63) & ~63), n)
@@ -885,8 +912,7 @@ def _attention_inputs_grads(qkv, w, gs, consts, w_in, gqs, gk, gv, ga):
     D = _DeferredWeightGrads
     if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
         D.reset()                               # left over from a backward pass that raised
-    defer = (KernelManager.DEFER_WEIGHT_GRADS and N > 0 and w_in is not None and w_in.is_leaf
-             and w_in.dtype == torch.float32 and w_in.dim() == 1)
+    defer = N > 0 and w_in is not None and w_in.dim() == 1 and D.deferrable(w_in)
     if defer:
         # the column sums of the partials join the weight gradients of the pass in their one launch
         gw = D.take(H * Dh, qkv.device)

@@ -62,7 +62,9 @@ def test_c1_one_layer_forward_operators_against_full_basis(window_mode, tol):
                             cutoff_radius=None, lattice_range=2, windows="full")
     oo, _ = TO.softmax_attention(P.q, P.k, P.v, zo, psio, P.batch, P.edges)
     assert Hh.rel_err(z, zo) < 2e-5 and Hh.elem_err(z, zo, rtol=1e-4) <= 1.0
-    assert Hh.rel_err(psi, psio) < tol and Hh.elem_err(psi, psio, rtol=tol, atol_frac=tol * 1e-1) <= 1.0
+    assert Hh.rel_err(psi, psio) < tol
+    if window_mode == 1:     # (the 4-sigma truncation is an absolute error of exp(-8) per dropped bin: no elementwise bound)
+        assert Hh.elem_err(psi, psio, rtol=1e-4, atol_frac=1e-5) <= 1.0
     assert Hh.rel_err(out, oo) < tol
 
 
