@@ -187,6 +187,7 @@ def require_gpu(*tensors: torch.Tensor):
 
 
 _workspaces = {}
+_superseded = []      # outgrown workspaces, kept for captured graphs that still point at them
 
 
 def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
@@ -195,6 +196,10 @@ def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            # a HIP graph captured on this stream holds the address of the buffer it was given: a superseded
+            # buffer stays allocated, so that replays keep writing into memory that is still theirs
+            _superseded.append(buf)
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         buf[:512].zero_()          # work-queue heads and the statistics block
         _workspaces[key] = buf
@@ -212,6 +217,17 @@ def read_stats(device: torch.device, reset: bool = False) -> dict:
     if reset:
         buf[256:512].zero_()
     return dict(zip(STAT_NAMES, vals))
+
+
+def read_status(device: torch.device, reset: bool = False) -> int:
+    """Status word of this stream's workspace (synchronises): 1 when a launch had to cut a translation box
+    back to the largest half-width the kernels sum (32), i.e. where the result differs from the reference's
+    box rule; 0 otherwise."""
+    buf = workspace(device, 512)
+    val = int(buf[16:20].view(torch.int32).cpu()[0])
+    if reset:
+        buf[16:20].zero_()
+    return val
 
 
 def current_stream_ptr(device: torch.device):

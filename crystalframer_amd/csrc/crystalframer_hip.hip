@@ -40,6 +40,7 @@ int fail(int code, const char* fmt, ...) {
 constexpr int MAX_HEADS = 64;
 constexpr size_t QUEUE_OFFSET = 512;           // workspace header: 256 reserved bytes, 32 uint64 statistics, then the work queues
 constexpr size_t STATS_OFFSET = 256;
+constexpr size_t STATUS_OFFSET = 16;          // int32 status word (box cut back to the largest half-width)
 constexpr size_t QUEUE_SET_BYTES = (size_t)MAX_HEADS * cfh::NQUEUE * cfh::QSTRIDE * sizeof(int32_t);
 constexpr size_t COUNTER_BYTES = QUEUE_OFFSET + 2 * QUEUE_SET_BYTES;   // whole header: two sets of work queues
 constexpr int WAVES_PER_SIMD = 3;
@@ -215,6 +216,7 @@ void fill_common(cfh::KernelArgs& A, const cfh_params* p, const float* a_ih, con
     A.seed_hi = (uint32_t)(p->noise_seed >> 32);
     A.seed_dev = reinterpret_cast<unsigned long long*>(p->noise_seed_dev);
     A.seed_snap = reinterpret_cast<unsigned long long*>(workspace);      // first word of the reserved header bytes
+    A.status = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(workspace) + STATUS_OFFSET);
     A.seed_advance = p->noise_seed_advance;
     A.bc = basis_consts(p);
 }

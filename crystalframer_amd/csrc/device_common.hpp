@@ -141,16 +141,18 @@ struct Box {
     int R1, R2, R3;   // half-widths
     int s2, s3;       // 2*R2+1, 2*R3+1
     int T;            // number of translations
+    int over;         // 1: a half-width was cut back to RMAX
 };
 
 // Half-widths of the translation box.  Same operation order as the reference kernels
 // (models/kernels/real_enc_frame_proj_fwd_length.cu:59-86): float32 up to (cutoff+0.01f)*rvl,
 // double division by 2.0*CUDART_PI_F, ceil; no fused multiply-add.
 #pragma clang fp contract(off)
-__device__ __forceinline__ int half_width(float c1, float rvl, int minimum_range) {
+__device__ __forceinline__ int half_width(float c1, float rvl, int minimum_range, int& over) {
     const float prod = c1 * rvl;
     const double v = (double)prod / (2.0 * (double)3.14159274101257324f);
     int r = (v > 0.0 && v < (double)RMAX) ? (int)ceil(v) : (v >= (double)RMAX ? RMAX : 0);
+    if (v > (double)RMAX) over = 1;          // the rule asks for more than the kernels sum: reported, not silent
     if (minimum_range > 0) r = max(r, minimum_range);
     return min(r, RMAX);
 }
@@ -159,13 +161,14 @@ __device__ __forceinline__ Box translation_box(float a, float rvl1, float rvl2, 
                                                int minimum_range) {
     Box b;
     b.R1 = b.R2 = b.R3 = lattice_range;
+    b.over = 0;
     if (cutoff_radius != 0.0f) {
         float cut = cutoff_radius;
         if (cut < 0.0f) cut = __fsqrt_rn(__fdiv_rn(-0.5f, a)) * (-cut);
         const float c1 = cut + 0.01f;
-        b.R1 = half_width(c1, rvl1, minimum_range);
-        b.R2 = half_width(c1, rvl2, minimum_range);
-        b.R3 = half_width(c1, rvl3, minimum_range);
+        b.R1 = half_width(c1, rvl1, minimum_range, b.over);
+        b.R2 = half_width(c1, rvl2, minimum_range, b.over);
+        b.R3 = half_width(c1, rvl3, minimum_range, b.over);
     }
     b.s2 = 2 * b.R2 + 1; b.s3 = 2 * b.R3 + 1;
     b.T = (2 * b.R1 + 1) * b.s2 * b.s3;
@@ -341,6 +344,7 @@ struct KernelArgs {
     int32_t frames_to_records;    // frame search: also store the orthonormal frames into the item records
     uint32_t* items;              // (N, H, REC_WORDS) item records of this launch
     unsigned long long* stats;    // optional running totals (see STAT_* below); never reset by a launch
+    int32_t* status;              // word of the workspace header: set to 1 when a box was cut back to RMAX (never cleared)
     int32_t N, E, H;
     float cutoff_radius; int32_t lattice_range, minimum_range;
     float prune_log2;             // <= 0: keep every translation
@@ -430,6 +434,7 @@ __device__ __forceinline__ Item unpack_item(uint32_t rec) {
     t.bx.R1 = box & 255; t.bx.R2 = (box >> 8) & 255; t.bx.R3 = (box >> 16) & 255;
     t.bx.s2 = 2 * t.bx.R2 + 1; t.bx.s3 = 2 * t.bx.R3 + 1;
     t.bx.T = (2 * t.bx.R1 + 1) * t.bx.s2 * t.bx.s3;
+    t.bx.over = 0;
     t.a = rec_f(rec, REC_A);
 #pragma unroll
     for (int d = 0; d < 9; d++) t.L.t[d] = rec_f(rec, REC_LATTICE + d);
@@ -465,6 +470,7 @@ __global__ __launch_bounds__(256) void prepare_items_kernel(const KernelArgs P, 
     float rvl1 = 0.f, rvl2 = 0.f, rvl3 = 0.f;
     if (P.rvlen) { rvl1 = P.rvlen[(size_t)b * 3 + 0]; rvl2 = P.rvlen[(size_t)b * 3 + 1]; rvl3 = P.rvlen[(size_t)b * 3 + 2]; }
     const Box bx = translation_box(a, rvl1, rvl2, rvl3, P.cutoff_radius, P.lattice_range, P.minimum_range);
+    if (bx.over && P.status) *P.status = 1;
     uint32_t* rec = P.items + (size_t)idx * REC_WORDS;
     const int e0 = (int)P.e_start[i];
     rec[REC_ATOM] = (uint32_t)i;

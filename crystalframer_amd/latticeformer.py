@@ -19,9 +19,14 @@ ATOM_FEAT_DIM = 98
 
 
 def max_pool(x, batch, sizes):
+    """Per-crystal maximum (reference: models/pooling.py:13-16, which splits by ``sizes``).  The crystal
+    indices in ``batch`` need not start at 0 (the encoder accepts such batches as well)."""
     B = sizes.shape[0]
     out = torch.full((B,) + tuple(x.shape[1:]), -float("inf"), dtype=x.dtype, device=x.device)
-    return out.scatter_reduce(0, batch[:, None].expand_as(x), x, reduce="amax", include_self=True)
+    if batch.numel() == 0:
+        return out
+    idx = (batch - batch[0]).reshape((-1,) + (1,) * (x.dim() - 1)).expand_as(x)
+    return out.scatter_reduce(0, idx, x, reduce="amax", include_self=True)
 
 
 def avr_pool(x, batch, sizes):

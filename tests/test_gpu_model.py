@@ -301,3 +301,80 @@ def test_crystal_indices_with_an_offset_give_the_same_output():
         assert not shifted.zero_based
         out = model(shifted)
     assert torch.equal(out, ref)
+
+
+def test_hooked_parameter_and_reused_weight_get_complete_gradients():
+    """Deferred weight gradients must not be visible as zeros: a parameter with a tensor hook or a
+    post-accumulate hook is not deferred (its hook sees the finished gradient), and a weight used by two
+    projections of one pass receives the sum of both products."""
+    import crystalframer_amd as cf
+    dev = torch.device("cuda:0")
+    gen = torch.Generator().manual_seed(3)
+    x1 = torch.randn(300, 128, generator=gen).to(dev)
+    x2 = torch.randn(300, 128, generator=gen).to(dev)
+    W0 = torch.randn(64, 128, generator=gen)
+    b0 = torch.randn(64, generator=gen)
+    gy = torch.randn(300, 64, generator=gen).to(dev)
+
+    def reference():
+        W = W0.double().requires_grad_(True)
+        b = b0.double().requires_grad_(True)
+        y = torch.nn.functional.linear(x1.cpu().double(), W, b) + 2.0 * torch.nn.functional.linear(x2.cpu().double(), W, b)
+        (y * gy.cpu().double()).sum().backward()
+        return W.grad, b.grad
+
+    gW_ref, gb_ref = reference()
+    for kind in ("plain", "tensor_hook", "post_accumulate_hook"):
+        W = W0.to(dev).requires_grad_(True)
+        b = b0.to(dev).requires_grad_(True)
+        seen = {}
+        if kind == "tensor_hook":
+            W.register_hook(lambda g: seen.setdefault("calls", []).append(g.detach().clone()))
+        elif kind == "post_accumulate_hook":
+            W.register_post_accumulate_grad_hook(lambda p: seen.setdefault("calls", []).append(p.grad.detach().clone()))
+        y = cf.cuda_funcs.linear(x1, W, b) + 2.0 * cf.cuda_funcs.linear(x2, W, b)
+        (y * gy).sum().backward()
+        torch.cuda.synchronize()
+        assert Hh.rel_err(W.grad, gW_ref) < 1e-5, kind
+        assert Hh.rel_err(b.grad, gb_ref) < 1e-5, kind
+        if kind == "tensor_hook":
+            # the engine sums the two uses before it calls the hook: what the hook sees is the gradient
+            assert len(seen["calls"]) == 1
+            assert Hh.rel_err(seen["calls"][0], gW_ref) < 1e-5
+        if kind == "post_accumulate_hook":
+            assert Hh.rel_err(seen["calls"][-1], gW_ref) < 1e-5
+
+
+def test_max_pooling_with_crystal_indices_that_do_not_start_at_zero():
+    from crystalframer_amd import latticeformer
+    dev = torch.device("cuda:0")
+    sizes = torch.tensor([3, 1, 4, 2])
+    x = torch.randn(10, 7, device=dev)
+    batch = torch.repeat_interleave(torch.arange(4), sizes).to(dev) + 5
+    got = latticeformer.max_pool(x, batch, sizes.to(dev))
+    want = torch.stack([c.max(0).values for c in torch.split_with_sizes(x, sizes.tolist())])
+    assert torch.equal(got, want)
+
+
+def test_status_word_reports_a_box_cut_back_to_the_largest_half_width():
+    """A Gaussian so wide that the box rule asks for more than 32 cells along an axis: the kernels sum the
+    clamped box and say so in the status word of the workspace (0 for ordinary inputs)."""
+    import crystalframer_amd as cf
+    from crystalframer_amd import _lib
+    dev = torch.device("cuda:0")
+    P = Hh.make_problem(num_crystals=2, atoms_lo=1, atoms_hi=2, len_lo=2.0, len_hi=2.5, seed=5)
+    g = lambda t: t.to(dtype=torch.float32, device=dev)
+
+    def run(a):
+        out = cf.RealEncodingWithFramedProjFuncCUDA.apply(
+            g(a), g(P.rpos), None, g(P.tvecs), P.batch.to(dev), P.edges.to(dev), 0, 14.0, 1.0, None, None, None, None,
+            None, None, None, 0, 4.0, 0, 1.0, 1.0, g(P.rvlen), -3.5)
+        torch.cuda.synchronize()
+        return out[0]
+
+    _lib.read_status(dev, reset=True)
+    z = run(P.a)
+    assert torch.isfinite(z).all() and _lib.read_status(dev) == 0
+    z = run(torch.full_like(P.a, -1e-3))        # sigma = 22 angstrom in 2 angstrom cells: half-width ~ 39
+    assert torch.isfinite(z).all() and _lib.read_status(dev, reset=True) == 1
+    assert _lib.read_status(dev) == 0
