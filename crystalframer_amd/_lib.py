@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
@@ -73,7 +73,9 @@ EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_fram
            "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
            "cfh_crystal_geometry", "cfh_small_linear_forward", "cfh_small_linear_dx", "cfh_linear_weight_bias_grad", "cfh_linear_weight_bias_grad_batch", "cfh_attention_inputs_forward",
            "cfh_attention_inputs_backward", "cfh_layer_bridge_forward", "cfh_layer_bridge_backward",
-           "cfh_second_stream_fork", "cfh_second_stream_get", "cfh_second_stream_join")
+           "cfh_second_stream_fork", "cfh_second_stream_get", "cfh_second_stream_join",
+           "cfh_fused_core_workspace_bytes", "cfh_fused_core_hist_words", "cfh_fused_core_forward",
+           "cfh_fused_core_backward")
 
 _lib = None
 _lock = threading.Lock()
@@ -147,6 +149,15 @@ def load():
         lib.cfh_attention_inputs_backward.restype = ctypes.c_int
         lib.cfh_attention_inputs_backward.argtypes = [_P, _P, _P, _F, _F, _F, _F, _P, _P, _P, _P, _I64, _I32, _I32,
                                                       _P, _P, _P, ctypes.c_size_t, _P]
+        lib.cfh_fused_core_workspace_bytes.restype = ctypes.c_size_t
+        lib.cfh_fused_core_workspace_bytes.argtypes = [pp, _I64, _I64, _I64, ctypes.c_int32]
+        lib.cfh_fused_core_hist_words.restype = ctypes.c_int32
+        lib.cfh_fused_core_hist_words.argtypes = [pp]
+        lib.cfh_fused_core_forward.restype = ctypes.c_int
+        lib.cfh_fused_core_forward.argtypes = ([pp] + [_P] * 15 + [_I64] * 3 + [_P, ctypes.c_int32] + [_P] * 4
+                                               + [_P, ctypes.c_size_t, _P])
+        lib.cfh_fused_core_backward.restype = ctypes.c_int
+        lib.cfh_fused_core_backward.argtypes = ([pp] + [_P] * 21 + [_I64] * 3 + [_P] * 9 + [_P, ctypes.c_size_t, _P])
         lib.cfh_timing_enable.restype = ctypes.c_int
         lib.cfh_timing_enable.argtypes = [ctypes.c_int]
         lib.cfh_timing_read.restype = ctypes.c_int
@@ -207,7 +218,7 @@ def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
 
 
 STAT_NAMES = ("fwd_evaluated", "fwd_in_box", "bwd_evaluated", "bwd_in_box", "frame1_scanned",
-              "frame2_scanned", "fwd_pairs", "bwd_pairs")
+              "frame2_scanned", "fwd_pairs", "bwd_pairs", "fwd_visited")
 
 
 def read_stats(device: torch.device, reset: bool = False) -> dict:

@@ -20,6 +20,7 @@
 #include "framed_pe_bwd_saved.hpp"
 #include "framed_pe_fwd.hpp"
 #include "fused_dpa.hpp"
+#include "fused_core.hpp"
 #include "geometry.hpp"
 #include "linear_grad.hpp"
 #include "small_gemm.hpp"
@@ -1027,6 +1028,243 @@ int cfh_small_linear_dx(const float* dy, const float* W, int64_t M, int64_t N, i
     hipLaunchKernelGGL(cfh::small_linear_dx_kernel, dim3((unsigned)((M + 63) / 64), (unsigned)((K + 63) / 64)), dim3(256), 0,
                        (hipStream_t)stream, dy, W, dx, (int)M, (int)N, (int)K);
     return finish_launch("small_linear_dx");
+}
+
+
+}  // extern "C"
+
+// ---- fused attention core ----------------------------------------------------------------------------------------
+namespace {
+struct CoreLayout {
+    size_t items, sorted, wcat, gwcat, G, total;
+    int hw;
+};
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+CoreLayout core_layout(const cfh_params* p, int64_t N, int64_t B, bool backward) {
+    CoreLayout L;
+    L.hw = p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
+    size_t off = COUNTER_BYTES;
+    L.items = off; off += items_bytes(N > 0 ? N : 1, p->num_heads);
+    L.sorted = off; off += align256((size_t)(B > 0 ? B : 1) * cfh::FC_TCAP * sizeof(float4));
+    L.wcat = off; off += align256((size_t)p->num_heads * cfh::DH * L.hw * sizeof(float));
+    L.gwcat = off; if (backward) off += align256((size_t)p->num_heads * cfh::DH * L.hw * sizeof(float));
+    L.G = off; if (backward) off += align256((size_t)(N > 0 ? N : 1) * p->num_heads * L.hw * sizeof(float));
+    L.total = off;
+    return L;
+}
+int check_core_params(const cfh_params* p) {
+    int rc = check_params(p);
+    if (rc) return rc;
+    if (p->dist_bins != cfh::NBINS) return fail(CFH_EINVAL, "fused core: dist_bins must be %d", cfh::NBINS);
+    if (p->dist_wscale != 1.0f) return fail(CFH_EINVAL, "fused core: only dist_wscale 1.0 is compiled");
+    if (p->grad_coef_quirk) return fail(CFH_EINVAL, "fused core: grad_coef_quirk is not available (exact gradients only)");
+    if (p->angle_bins > 0 && p->angle_wscale < 3.0f)
+        return fail(CFH_EINVAL, "fused core: angle_wscale %g < 3: the moment expansion of the angle basis (6 terms) "
+                    "is not accurate enough; use the two-step operators", (double)p->angle_wscale);
+    return CFH_OK;
+}
+// the kernels' launch-wide arguments that both directions share
+void fill_core(cfh::CoreArgs& C, const cfh_params* p, const CoreLayout& L, const float* qs, const float* k, const float* v,
+               bool has_rvlen, void* workspace) {
+    C.qs = qs; C.k = k; C.v = v;
+    const bool adaptive = has_rvlen && p->cutoff_radius != 0.0f;
+    const int R0 = adaptive ? p->minimum_range : p->lattice_range;
+    const bool tables = p->prune_log2 > 0.0f && R0 >= 1 && (2 * R0 + 1) * (2 * R0 + 1) * (2 * R0 + 1) <= cfh::FC_TCAP;
+    C.sorted_tab = tables ? reinterpret_cast<const float4*>(reinterpret_cast<char*>(workspace) + L.sorted) : nullptr;
+    C.table_R = tables ? R0 : 0;
+    C.skip_log2 = p->prune_log2 > 0.0f ? (p->prune_log2 + 8.0f > 32.0f ? p->prune_log2 + 8.0f : 32.0f) : 0.0f;
+}
+template <typename Kern>
+int launch_core(Kern kern, const cfh::CoreArgs& C, int cap, hipStream_t st, const char* what) {
+    const int waves = resident_waves(kern, cap, C.K.H);
+    bool timed = false;
+    TimedLaunch t;
+    {
+        std::lock_guard<std::mutex> lock(g_timing_mutex);
+        timed = g_timing_on;
+    }
+    if (timed) {
+        t.what = what;
+        timed = hipEventCreate(&t.start) == hipSuccess && hipEventCreate(&t.stop) == hipSuccess &&
+                hipEventRecord(t.start, st) == hipSuccess;
+    }
+    hipLaunchKernelGGL(kern, dim3(waves), dim3(cfh::WAVE), 0, st, C);
+    if (timed && hipEventRecord(t.stop, st) == hipSuccess) {
+        std::lock_guard<std::mutex> lock(g_timing_mutex);
+        g_timed.push_back(t);
+    }
+    return finish_launch(what);
+}
+constexpr int CORE_WAVES_PER_SIMD = 6;
+}  // namespace
+
+extern "C" {
+
+size_t cfh_fused_core_workspace_bytes(const cfh_params* p, int64_t N, int64_t E, int64_t B, int32_t backward) {
+    (void)E;
+    if (check_core_params(p) != CFH_OK) return 0;
+    return core_layout(p, N, B, backward != 0).total;
+}
+
+int32_t cfh_fused_core_hist_words(const cfh_params* p) {
+    if (check_core_params(p) != CFH_OK) return 0;
+    return p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
+}
+
+int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k, const float* v, const float* a_ih,
+                           const float* rpos, const float* tvecs, const float* rvlen, const int64_t* batch,
+                           const int64_t* edges, const int64_t* e_start, const int32_t* order, const float* W_dist,
+                           const float* W_axis1, const float* W_axis2, const float* W_axis3, int64_t N, int64_t E,
+                           int64_t B, float* frames, int32_t search_frames, float* z, float* prob, float* hist,
+                           float* out, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_core_params(p);
+    if (rc) return rc;
+    if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
+    if (N == 0) return CFH_OK;
+    const bool has_ang = p->angle_bins > 0;
+    if (!qs || !k || !v || !W_dist || !z || !prob || !hist || !out)
+        return fail(CFH_EINVAL, "qs, k, v, W_dist, z, prob, hist and out must not be NULL");
+    if (has_ang && (!W_axis1 || !W_axis2 || !W_axis3 || !frames))
+        return fail(CFH_EINVAL, "the angle encoding needs W_axis1..3 and frames");
+    const CoreLayout L = core_layout(p, N, B, false);
+    if ((rc = check_workspace(workspace, workspace_bytes, L.total))) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    char* ws = reinterpret_cast<char*>(workspace);
+    cfh::CoreArgs C;
+    std::memset(&C, 0, sizeof(C));
+    fill_common(C.K, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
+    fill_core(C, p, L, qs, k, v, rvlen != nullptr, workspace);
+    const bool search = has_ang && search_frames != 0;
+    if (search) {
+        // records with the query, frame search through the first set of queues; it leaves the frames in the records
+        cfh::KernelArgs F = C.K;
+        F.q = qs; F.k = k; F.out_frame = frames;
+        F.counters2 = reinterpret_cast<int32_t*>(ws + QUEUE_OFFSET + QUEUE_SET_BYTES);
+        F.frames_to_records = 1;
+        int fwaves = launch_waves(N, p->num_heads, FRAME_WAVES_PER_SIMD);
+        if ((rc = launch_persistent(cfh::frame_axis_kernel<2>, F, &fwaves, st, "frame_axes"))) return rc;
+        C.K.counters = F.counters2;
+    } else {
+        C.K.frames = has_ang ? frames : nullptr;
+        const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
+                                                                                          : p->num_heads * cfh::NQUEUE);
+        hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, C.K, 0);
+    }
+    if (C.sorted_tab)
+        hipLaunchKernelGGL(cfh::sorted_shifts_kernel, dim3((unsigned)B), dim3(cfh::FC_TCAP), 0, st, tvecs, C.table_R,
+                           reinterpret_cast<float4*>(ws + L.sorted));
+    float* wcat = reinterpret_cast<float*>(ws + L.wcat);
+    hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, W_dist, W_axis1, W_axis2,
+                       W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat);
+    C.out = out; C.prob = prob; C.z = z; C.hist = hist;
+    const int cap = launch_waves(N, p->num_heads, CORE_WAVES_PER_SIMD);
+    const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+    const char* what = "fused_core_forward";
+#define CFH_CORE_DISPATCH(KERNEL)                                                                         \
+    do {                                                                                                  \
+        if (has_ang) {                                                                                    \
+            if (wide) rc = p->cos_abs ? launch_core(KERNEL<11, true, true>, C, cap, st, what)             \
+                                      : launch_core(KERNEL<11, true, false>, C, cap, st, what);           \
+            else rc = p->cos_abs ? launch_core(KERNEL<9, true, true>, C, cap, st, what)                   \
+                                 : launch_core(KERNEL<9, true, false>, C, cap, st, what);                 \
+        } else {                                                                                          \
+            rc = wide ? launch_core(KERNEL<11, false, false>, C, cap, st, what)                           \
+                      : launch_core(KERNEL<9, false, false>, C, cap, st, what);                           \
+        }                                                                                                 \
+    } while (0)
+    CFH_CORE_DISPATCH(cfh::fused_core_fwd_kernel);
+    if (rc) return rc;
+    hipLaunchKernelGGL(cfh::core_project_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads), dim3(cfh::WAVE), 0, st,
+                       hist, wcat, out, (int)N, p->num_heads, L.hw);
+    return finish_launch("fused_core_project");
+}
+
+int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k, const float* v, const float* a_ih,
+                            const float* rpos, const float* tvecs, const float* rvlen, const int64_t* batch,
+                            const int64_t* edges, const int64_t* e_start, const int32_t* order, const float* W_dist,
+                            const float* W_axis1, const float* W_axis2, const float* W_axis3, const float* frames,
+                            const float* z, const float* prob, const float* hist, const float* out, const float* gout,
+                            int64_t N, int64_t E, int64_t B, float* gq, float* gk, float* gv, float* ga, float* glogit,
+                            float* gW_dist, float* gW_axis1, float* gW_axis2, float* gW_axis3, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+    int rc = check_core_params(p);
+    if (rc) return rc;
+    if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const bool has_ang = p->angle_bins > 0;
+    const int per_enc = p->num_heads * cfh::DH * cfh::NBINS;
+    if (N == 0) {
+        hipLaunchKernelGGL(cfh::zero_outputs_kernel, dim3((per_enc + 255) / 256), dim3(256), 0, st, per_enc, gW_dist,
+                           gW_axis1, gW_axis2, gW_axis3);
+        return finish_launch("zero_outputs");
+    }
+    if (!qs || !k || !v || !W_dist || !z || !prob || !hist || !out || !gout || !gq || !gk || !gv || !ga || !glogit)
+        return fail(CFH_EINVAL, "fused core backward: a required pointer is NULL");
+    if (has_ang && (!W_axis1 || !W_axis2 || !W_axis3 || !frames))
+        return fail(CFH_EINVAL, "the angle encoding needs W_axis1..3 and frames");
+    const CoreLayout L = core_layout(p, N, B, true);
+    if ((rc = check_workspace(workspace, workspace_bytes, L.total))) return rc;
+    char* ws = reinterpret_cast<char*>(workspace);
+    float* wcat = reinterpret_cast<float*>(ws + L.wcat);
+    float* gwcat = reinterpret_cast<float*>(ws + L.gwcat);
+    float* G = reinterpret_cast<float*>(ws + L.G);
+    cfh::CoreArgs C;
+    std::memset(&C, 0, sizeof(C));
+    fill_common(C.K, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
+    fill_core(C, p, L, qs, k, v, rvlen != nullptr, workspace);
+    C.K.frames = has_ang ? frames : nullptr;
+    C.K.out_ga = ga;
+    C.z = const_cast<float*>(z); C.prob = const_cast<float*>(prob);
+    C.go = gout; C.outv = out; C.G = G; C.gq = gq; C.glogit = glogit;
+    // Wcat, G = Wcat^T go per item, records, tables
+    hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, W_dist, W_axis1, W_axis2,
+                       W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat);
+    hipLaunchKernelGGL(cfh::core_gbuild_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads), dim3(cfh::WAVE), 0, st,
+                       gout, wcat, G, (int)N, p->num_heads, L.hw);
+    {
+        const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
+                                                                                          : p->num_heads * cfh::NQUEUE);
+        hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, C.K, 0);
+    }
+    if (C.sorted_tab)
+        hipLaunchKernelGGL(cfh::sorted_shifts_kernel, dim3((unsigned)B), dim3(cfh::FC_TCAP), 0, st, tvecs, C.table_R,
+                           reinterpret_cast<float4*>(ws + L.sorted));
+    const int nw = p->num_heads * cfh::DH * L.hw;
+    hipLaunchKernelGGL(cfh::core_zero_kernel, dim3((nw + 255) / 256), dim3(256), 0, st, gwcat, nw);
+    const int cap = launch_waves(N, p->num_heads, CORE_WAVES_PER_SIMD);
+    const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+    const char* what = "fused_core_backward";
+    CFH_CORE_DISPATCH(cfh::fused_core_bwd_kernel);
+#undef CFH_CORE_DISPATCH
+    if (rc) return rc;
+    // gk, gv: sums over the pairs that point at an atom
+    {
+        cfh::DpaArgs A;
+        std::memset(&A, 0, sizeof(A));
+        A.q = qs; A.k = k; A.v = v; A.edges = edges; A.e_start = e_start;
+        A.prob = const_cast<float*>(prob); A.go = gout; A.gk = gk; A.gv = gv; A.gaij = glogit;
+        A.N = (int32_t)N; A.H = p->num_heads; A.E = (int32_t)E;
+        const int64_t items = N * p->num_heads;
+        hipLaunchKernelGGL(cfh::dpa_bwd_col_kernel, dim3((unsigned)((items + cfh::DPA_WAVES - 1) / cfh::DPA_WAVES)),
+                           dim3(cfh::WAVE * cfh::DPA_WAVES), 0, st, A);
+    }
+    // weight gradients: gwcat = sum_i go_i (x) hist_i, then back through the moment matrices
+    {
+        int cus = device_cus();
+        if (cus <= 0) cus = 256;
+        const int blocks_per_slice = (L.hw / 64) * p->num_heads;
+        int nslices = (cus * 4 + blocks_per_slice - 1) / blocks_per_slice;
+        if (nslices < 1) nslices = 1;
+        int per_slice = (int)((N + nslices - 1) / nslices);
+        per_slice = (per_slice + 15) & ~15;
+        nslices = (int)((N + per_slice - 1) / per_slice);
+        hipLaunchKernelGGL(cfh::core_gwcat_kernel, dim3(L.hw / 64, p->num_heads, nslices), dim3(cfh::WAVE), 0, st, gout, hist,
+                           gwcat, (int)N, p->num_heads, L.hw, per_slice);
+        hipLaunchKernelGGL(cfh::core_gw_finish_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, gwcat, L.hw,
+                           p->dist_coef, p->angle_coef, p->angle_wscale, gW_dist, gW_axis1,
+                           gW_axis2, gW_axis3);
+    }
+    return finish_launch("fused_core_backward");
 }
 
 }  // extern "C"

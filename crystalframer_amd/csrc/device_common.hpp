@@ -126,7 +126,7 @@ __device__ __forceinline__ void wave_sync() {
 
 // slots of KernelArgs::stats
 enum { STAT_FWD_EVAL = 0, STAT_FWD_RAW = 1, STAT_BWD_EVAL = 2, STAT_BWD_RAW = 3, STAT_FRAME1_RAW = 4,
-       STAT_FRAME2_RAW = 5, STAT_FWD_PAIRS = 6, STAT_BWD_PAIRS = 7 };
+       STAT_FRAME2_RAW = 5, STAT_FWD_PAIRS = 6, STAT_BWD_PAIRS = 7, STAT_FWD_SEEN = 8 };
 
 __device__ __forceinline__ int uniform_i(int v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ float uniform_f(float v) {
@@ -411,7 +411,8 @@ __device__ __forceinline__ int first_queue(int H) { return ((int)blockIdx.x / H)
 // 128-byte record so that the main kernels fetch it with ONE coalesced load, issued a whole item
 // ahead (the chain order -> batch -> lattice would be three dependent round trips per item):
 //   word 0 atom i, 1 first pair, 2 number of pairs, 3 R1 | R2 << 8 | R3 << 16, 4 a_ih,
-//   5..13 lattice rows, 14..22 frame axes (frame search: 14..29 the query vector q_ih)
+//   5..13 lattice rows, 14..22 frame axes (frame search: 14..29 the query vector q_ih),
+//   30 first neighbour atom (the pairs of an atom point at consecutive atoms), 31 crystal
 constexpr int REC_WORDS = 32;
 enum { REC_ATOM = 0, REC_E0 = 1, REC_NPAIRS = 2, REC_BOX = 3, REC_A = 4, REC_LATTICE = 5, REC_FRAMES = 14,
        REC_QUERY = 14 };
@@ -479,6 +480,8 @@ __global__ __launch_bounds__(256) void prepare_items_kernel(const KernelArgs P, 
     rec[REC_BOX] = (uint32_t)(bx.R1 | (bx.R2 << 8) | (bx.R3 << 16));
     rec[REC_A] = __float_as_uint(a);
     for (int d = 0; d < 9; d++) rec[REC_LATTICE + d] = __float_as_uint(P.tvecs[(size_t)b * 9 + d]);
+    rec[30] = (uint32_t)(P.e_start[i + 1] > e0 ? (int)P.edges[(size_t)P.E + e0] : i);      // first neighbour atom
+    rec[31] = (uint32_t)b;                                                                  // crystal
     if (with_query) {
         for (int c = 0; c < DH; c++) rec[REC_QUERY + c] = __float_as_uint(P.q[((size_t)i * P.H + h) * DH + c]);
     } else if (P.frames) {

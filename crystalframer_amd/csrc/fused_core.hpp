@@ -1,0 +1,840 @@
+// Fused attention core: lattice sums, softmax over the pairs of an atom and the value encoding in ONE pass per
+// (atom i, head h), with ONE histogram per (atom, head) instead of one per (pair, head).
+//
+// The attention output is linear in the value encoding,
+//     out_i = sum_j P_ij (v_j + psi_ij),   psi_ij = W . shat_ij,   shat_ij = sum_n p_n b(image n of pair ij),
+// so  sum_j P_ij psi_ij = W . T_i  with  T_i = sum_j sum_n P_ij p_n b(.): the per-image basis values can be
+// scattered, weighted by P_ij p_n, into one histogram per item, and the projection W is applied once per item by
+// a small MFMA product afterwards.  psi (E,H,16) and the per-pair histograms never exist.  The softmax weights
+// P_ij are not known before all pairs of the row have been seen, so the pass keeps a running maximum of the
+// logits (q_i.k_j + z_ij) and rescales histogram, value accumulator and denominator when it grows (online
+// softmax).  What the reference computes in five kernels and a tensor sum
+// (models/kernels/real_enc_frame_proj_fwd_length.cu, ..._fwd_angle.cu, fused_dpa_fwd.cu;
+//  models/cuda_funcs/real_space_framed_proj.py:21-120, fused_dpa.py:17-63) is one kernel plus the projection here.
+//
+// Two further changes of formulation (same mathematics, different arithmetic):
+//   * sorted translations.  For the usual box (half-width 2 = 125 translations) a table of the box's shifts
+//     sorted by length is made once per crystal.  An image at shift s of a pair at r lies at distance
+//     >= |s| - |r|, so the nearest image of a pair is found in the prefix |s| <= 2|r| and every image whose
+//     weight can reach 2^-skip of the heaviest one in the prefix |s| <= |r| + sqrt(d2min + skip/(-a log2 e)):
+//     the two light sweeps read a fraction of the box instead of all of it twice.
+//   * angle encoding by local moments.  The Gaussian basis of the cosine has sigma = wscale bins (4), so around
+//     the bin m* nearest to x the value of every basis function is a short power series in the offset
+//     eps = 2 (u - m*) in [-1,1] (u = x in bin units):
+//         exp(-((m - u)/ws)^2 / 2) = sum_o eps^o D_o(m - m*),  D_o(d) = exp(-(d/ws)^2/2) He_o(d/ws) / (o! (2 ws)^o)
+//     (generating function of the Hermite polynomials; truncated after NORD = 6 terms the error is below 1e-7 of
+//     the peak).  A term therefore adds NORD moments w eps^o at ONE bin per axis instead of a 33-bin window, and
+//     the constant matrices D_o are folded into the projection weights (core_wcat_kernel).  This is the FULL
+//     basis (no +-4 sigma truncation), i.e. the pure-PyTorch formulation of the reference
+//     (models/indexed_lattice_multi_head_attention.py:580-588) rather than the windowed one of its CUDA kernels.
+//     The distance basis (sigma = 1 bin) keeps its truncated window.
+//
+// Histogram of an item ("hist", HW words): [0,64) distance bins, then for axis ax and order o the 64 moment bins
+// at 64 + (ax NORD + o) 64.  It is accumulated in LDS as signed 32-bit fixed point (round to nearest) in units of
+// 2^30 / npairs relative to the heaviest pair of the row so far, and written out normalised as float32.
+#pragma once
+#include "device_common.hpp"
+
+namespace cfh {
+
+constexpr int FC_TCAP = 128;                    // translations per table chunk (the sorted table of the usual box fits)
+constexpr int FC_GROUP = 8;                     // pairs per group: one per 8-lane row
+constexpr int FC_LISTCAP = FC_GROUP * FC_TCAP;  // a group's survivors always fit: no overflow handling
+constexpr int FC_SHIFT = 7;                     // list entry = pair-in-group << 7 | table index
+constexpr int NORD = 6;                         // moments per axis
+constexpr int HW_DIST = NBINS;
+constexpr int HW_ANG = NBINS * (1 + 3 * NORD);  // 1216 words per (atom, head) with the angle encoding
+constexpr int REC_J0 = 30;                      // item record: first neighbour atom (pairs of an atom are j0, j0+1, ...)
+constexpr int REC_CRYSTAL = 31;                 // item record: crystal of the atom
+static_assert(FC_TCAP == (1 << FC_SHIFT) && (FC_GROUP << FC_SHIFT) <= 65536, "list entry is 16 bits");
+
+typedef float v4f_c __attribute__((ext_vector_type(4)));
+
+struct CoreArgs {
+    KernelArgs K;                 // geometry, work queues, item records, basis constants
+    const float* qs;              // (N,H,16) query, already divided by sqrt(16)
+    const float* k;               // (N,H,16)
+    const float* v;               // (N,H,16)
+    const float4* sorted_tab;     // (B, FC_TCAP) shifts of the usual box sorted by length, w = length; or null
+    int32_t table_R;              // half-width that table was made for
+    float skip_log2;              // images lighter than 2^-skip of the heaviest of their pair are not visited (<= 0: all are)
+    // forward results
+    float* out;                   // (N,H,16) sum_j P_ij v_j (core_project_kernel adds W . hist)
+    float* prob;                  // (E,H) P_ij
+    float* z;                     // (E,H)
+    float* hist;                  // (N,H,hw)
+    // backward operands and results
+    const float* go;              // (N,H,16) upstream gradient of out
+    const float* outv;            // (N,H,16) the forward's final out
+    const float* G;               // (N,H,hw) Wcat^T go per item
+    float* gq;                    // (N,H,16)
+    float* glogit;                // (E,H) gradient of the logits (the column kernel turns it into gk)
+};
+
+// ---- reductions over an 8-lane row (half of a DPP row) -------------------------------------------------------
+__device__ __forceinline__ float half_sum(float x) {
+    x += dpp_move<0xB1>(x); x += dpp_move<0x4E>(x); x += dpp_move<0x141>(x); return x;
+}
+__device__ __forceinline__ float half_min(float x) {
+    x = fminf(x, dpp_move<0xB1>(x)); x = fminf(x, dpp_move<0x4E>(x)); x = fminf(x, dpp_move<0x141>(x)); return x;
+}
+__device__ __forceinline__ float wave_maxf(float v) { return -wave_min(-v); }
+// sum over the 8 rows for every position in the row: lanes s, s+8, ..., s+56
+__device__ __forceinline__ float rows8_sum(float x) {
+    x += dpp_move<0x128>(x);          // row_ror 8: the other half of the 16-lane row
+    return rows_sum(x);
+}
+__device__ __forceinline__ int rint_i(float x) { return (int)__builtin_rintf(x); }
+
+// ---- sorted shifts of the usual box, one table per crystal ---------------------------------------------------
+// block = crystal, 128 threads; entry = (shift, |shift|), ascending length (ties: loop order); entries beyond the
+// box: length +inf.
+__global__ __launch_bounds__(FC_TCAP) void sorted_shifts_kernel(const float* __restrict__ tvecs, int R0, float4* __restrict__ out) {
+    __shared__ float key[FC_TCAP];
+    const int b = blockIdx.x, t = threadIdx.x;
+    const int s = 2 * R0 + 1, T0 = s * s * s;
+    float4 v = make_float4(0.f, 0.f, 0.f, __builtin_inff());
+    if (t < T0) {
+        const float* L = tvecs + (size_t)b * 9;
+        const float n3 = (float)(t % s - R0), n2 = (float)((t / s) % s - R0), n1 = (float)(t / (s * s) - R0);
+        v.x = fmaf(L[6], n3, fmaf(L[3], n2, L[0] * n1));
+        v.y = fmaf(L[7], n3, fmaf(L[4], n2, L[1] * n1));
+        v.z = fmaf(L[8], n3, fmaf(L[5], n2, L[2] * n1));
+        v.w = sqrtf(fmaf(v.x, v.x, fmaf(v.y, v.y, v.z * v.z)));
+    }
+    key[t] = v.w;
+    __syncthreads();
+    int rank = 0;
+    for (int u = 0; u < FC_TCAP; u++) {
+        const float ku = key[u];
+        rank += (ku < v.w || (ku == v.w && u < t)) ? 1 : 0;
+    }
+    out[(size_t)b * FC_TCAP + rank] = v;
+}
+
+// ---- projection weights with the moment matrices folded in ---------------------------------------------------
+// D_o(d) = exp(-(d/ws)^2/2) He_o(d/ws) / (o! (2 ws)^o)
+__device__ __forceinline__ float moment_matrix(int o, float d, float ws) {
+    const float y = d / ws;
+    float h0 = 1.0f, h1 = y;           // probabilists' Hermite polynomials
+    float he = o == 0 ? h0 : h1;
+    for (int n = 1; n < o; n++) { const float h2 = y * h1 - (float)n * h0; h0 = h1; h1 = h2; he = h2; }
+    float coef = 1.0f;
+    for (int n = 1; n <= o; n++) coef /= (float)n * 2.0f * ws;
+    return __expf(-0.5f * y * y) * he * coef;
+}
+// table of D_o(d) for d = -63 .. 63 in LDS, made by the 256 threads of a block: dtab[o * 128 + d + 63]
+__device__ __forceinline__ void build_moment_table(float* dtab, float ws) {
+    for (int u = threadIdx.x; u < NORD * 128; u += 256) {
+        const int o = u >> 7, d = (u & 127) - 63;
+        dtab[u] = (u & 127) < 127 ? moment_matrix(o, (float)d, ws) : 0.0f;
+    }
+    __syncthreads();
+}
+// wcat (H,16,hw): [0,64) dist_coef W_dist;  64 + (ax NORD + o) 64 + m': angle_coef sum_m W_ax[c,m] D_o(m - m').
+// grid: H*16 blocks (h, c), 256 threads over the words.
+__global__ __launch_bounds__(256) void core_wcat_kernel(const float* __restrict__ Wd, const float* __restrict__ W1,
+                                                        const float* __restrict__ W2, const float* __restrict__ W3,
+                                                        int hw, float dist_coef, float angle_coef, float ws,
+                                                        float* __restrict__ wcat) {
+    __shared__ float row[3][NBINS];
+    __shared__ float dtab[NORD * 128];
+    const int hc = blockIdx.x;
+    if (hw > HW_DIST) {
+        for (int u = threadIdx.x; u < 3 * NBINS; u += 256) {
+            const float* W = u < NBINS ? W1 : (u < 2 * NBINS ? W2 : W3);
+            row[u / NBINS][u % NBINS] = W[(size_t)hc * NBINS + (u % NBINS)];
+        }
+        build_moment_table(dtab, ws);
+    }
+    for (int w = threadIdx.x; w < hw; w += 256) {
+        float val;
+        if (w < HW_DIST) val = dist_coef * Wd[(size_t)hc * NBINS + w];
+        else {
+            const int u = w - HW_DIST, ax = u / (NORD * NBINS), o = (u / NBINS) % NORD, mp = u % NBINS;
+            const float* dt = dtab + o * 128 + 63 - mp;
+            float acc = 0.0f;
+#pragma unroll 8
+            for (int m = 0; m < NBINS; m++) acc = fmaf(row[ax][m], dt[m], acc);
+            val = angle_coef * acc;
+        }
+        wcat[(size_t)hc * hw + w] = val;
+    }
+}
+// The way back: gW_dist = dist_coef gwcat[.., 0:64];  gW_ax[c,m] = angle_coef sum_{o,m'} gwcat[.., ax,o,m'] D_o(m - m').
+// grid: H*16 blocks, 256 threads = (enc 0..3, bin m).
+__global__ __launch_bounds__(256) void core_gw_finish_kernel(const float* __restrict__ gwcat, int hw, float dist_coef,
+                                                             float angle_coef, float ws, float* __restrict__ gWd,
+                                                             float* __restrict__ gW1, float* __restrict__ gW2,
+                                                             float* __restrict__ gW3) {
+    __shared__ float dtab[NORD * 128];
+    __shared__ float grow[3 * NORD * NBINS];
+    const int hc = blockIdx.x, enc = threadIdx.x >> 6, m = threadIdx.x & 63;
+    const float* g = gwcat + (size_t)hc * hw;
+    if (hw > HW_DIST) {
+        for (int u = threadIdx.x; u < 3 * NORD * NBINS; u += 256) grow[u] = g[HW_DIST + u];
+        build_moment_table(dtab, ws);
+    }
+    if (enc == 0) {
+        if (gWd) gWd[(size_t)hc * NBINS + m] = dist_coef * g[m];
+        return;
+    }
+    if (hw <= HW_DIST) return;
+    float* dst = enc == 1 ? gW1 : (enc == 2 ? gW2 : gW3);
+    if (!dst) return;
+    float acc = 0.0f;
+    for (int o = 0; o < NORD; o++) {
+        const float* gr = grow + ((enc - 1) * NORD + o) * NBINS;
+        const float* dt = dtab + o * 128 + 63 + m;
+#pragma unroll 8
+        for (int mp = 0; mp < NBINS; mp++) acc = fmaf(gr[mp], dt[-mp], acc);
+    }
+    dst[(size_t)hc * NBINS + m] = angle_coef * acc;
+}
+
+// ---- distance window with round-to-nearest fixed-point adds ---------------------------------------------------
+template <int W>
+__device__ __forceinline__ void window_scatter_rn(int32_t* base, const WindowSeed& s, float cc) {
+    constexpr int C = W / 2;
+    atomicAdd(base + C, rint_i(s.gc));
+    float g = s.gc, r = s.rr;
+#pragma unroll
+    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; atomicAdd(base + m, rint_i(g)); }
+    g = s.gc; r = s.rl;
+#pragma unroll
+    for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; atomicAdd(base + m, rint_i(g)); }
+}
+
+// ---- shared pieces of the two main kernels ---------------------------------------------------------------------
+struct CoreItem {
+    Item item;
+    int j0, crystal;
+    bool sorted;
+    int nchunks;
+};
+__device__ __forceinline__ CoreItem core_unpack(const CoreArgs& C, uint32_t rec, bool want_sorted) {
+    CoreItem ci;
+    ci.item = unpack_item(rec);
+    ci.j0 = __builtin_amdgcn_readlane((int)rec, REC_J0);
+    ci.crystal = __builtin_amdgcn_readlane((int)rec, REC_CRYSTAL);
+    const Box& bx = ci.item.bx;
+    ci.sorted = want_sorted && C.sorted_tab != nullptr && bx.R1 == C.table_R && bx.R2 == C.table_R &&
+                bx.R3 == C.table_R && ci.item.a < 0.0f && C.skip_log2 > 0.0f;
+    ci.nchunks = ci.sorted ? 1 : (bx.T + FC_TCAP - 1) / FC_TCAP;
+    return ci;
+}
+// table of the item's first (or only) chunk
+__device__ __forceinline__ void core_load_table(const CoreArgs& C, const CoreItem& ci, float4* tab, int lane) {
+    if (ci.sorted) {
+        for (int u = lane; u < FC_TCAP; u += WAVE) tab[u] = C.sorted_tab[(size_t)ci.crystal * FC_TCAP + u];
+    } else if (ci.nchunks == 1) {
+        build_shift_table(tab, 0, ci.item.bx.T, ci.item.bx, ci.item.L, lane);
+    }
+}
+
+// =================================================================================================================
+// forward
+// =================================================================================================================
+template <int WL, bool HAS_ANG, bool COS_ABS>
+__global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) {
+    constexpr int HWK = HAS_ANG ? HW_ANG : HW_DIST;
+    __shared__ float4 tab[FC_TCAP];
+    __shared__ uint16_t list[FC_LISTCAP];
+    __shared__ int32_t hist[HWK];
+    __shared__ float4 pairA[FC_GROUP];      // rx, ry, rz, d2min
+    __shared__ float pairC[FC_GROUP];       // exp(logit - running max) / S in fixed-point units
+
+    const KernelArgs& P = C.K;
+    const int lane = threadIdx.x;
+    const int H = P.H;
+    const int h = blockIdx.x % H;
+    const int pr = lane >> 3;          // pair of the group served by this 8-lane row
+    const int sub = lane & 7;          // position in the row
+    const BasisConsts bc = P.bc;
+    const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
+    const float INF = __builtin_inff();
+
+    for (int u = lane; u < HWK; u += WAVE) hist[u] = 0;
+    wave_sync();
+
+    unsigned long long st_eval = 0, st_raw = 0, st_pairs = 0, st_seen = 0;
+    int queue = first_queue(H);
+    int it_cur = queue_pop(P, h, queue);
+    int it_next = it_cur >= 0 ? queue_pop(P, h, queue) : -1;
+    uint32_t rec_cur = load_record(P, it_cur, h);
+    while (it_cur >= 0) {
+        const int ticket = queue_ticket(P, h, queue);
+        const uint32_t rec_next = load_record(P, it_next, h);
+        const CoreItem ci = core_unpack(C, rec_cur, true);
+        const int i = ci.item.i;
+        const float a = ci.item.a;
+        const float a2 = a * LOG2E;
+        const Lattice L = ci.item.L;
+        const Box bx = ci.item.bx;
+        const bool sorted = ci.sorted;
+        const int nchunks = ci.nchunks;
+        float f[3][3];
+        if (HAS_ANG) {
+#pragma unroll
+            for (int ax = 0; ax < 3; ax++)
+#pragma unroll
+                for (int d = 0; d < 3; d++) f[ax][d] = rec_f(rec_cur, REC_FRAMES + ax * 3 + d);
+        }
+        const int e0 = ci.item.e0, npairs = ci.item.npairs;
+        wave_sync();                          // the previous item's readers of the table are done
+        core_load_table(C, ci, tab, lane);
+        wave_sync();
+        const size_t ih = (size_t)i * H + h;
+        const float2 q2 = *reinterpret_cast<const float2*>(C.qs + ih * DH + 2 * sub);
+        const float fixs = 1073741824.0f / (float)max(npairs, 1);      // 2^30 / npairs: sums of weights <= 1 each fit
+        const float cutS = (C.skip_log2 > 0.0f && a2 < 0.0f) ? C.skip_log2 / (-a2) : INF;
+        float m_run = -INF;                   // running maximum of the logits (wave-uniform)
+        float Dl = 0.0f;                      // this lane's share of the softmax denominator
+        float2 accv = make_float2(0.f, 0.f);  // sum_j exp(logit_j - m_run) v_j, channels 2 sub, 2 sub + 1
+        unsigned long long n_eval = 0, n_seen = 0;      // wave-uniform counts
+
+        // operands of the pair served by this row, fetched one group ahead
+        float nrx = 0.f, nry = 0.f, nrz = 0.f;
+        float2 nk2 = make_float2(0.f, 0.f), nv2 = nk2;
+        auto fetch = [&](int g0) {
+            const int el = g0 + pr;
+            if (el < npairs) {
+                const size_t e = (size_t)(e0 + el);
+                const size_t jh = ((size_t)(ci.j0 + el) * H + h) * DH + 2 * sub;
+                nrx = P.rpos[e * 3 + 0]; nry = P.rpos[e * 3 + 1]; nrz = P.rpos[e * 3 + 2];
+                nk2 = *reinterpret_cast<const float2*>(C.k + jh);
+                nv2 = *reinterpret_cast<const float2*>(C.v + jh);
+            }
+        };
+        fetch(0);
+
+        // one sweep of this row's pair over the table(s): fn(inside, table index, d^2)
+        auto sweep = [&](bool active, float rx, float ry, float rz, float reach, auto&& fn) {
+            for (int ch = 0; ch < nchunks; ch++) {
+                const int t0c = ch * FC_TCAP;
+                const int cnt = sorted ? bx.T : min(FC_TCAP, bx.T - t0c);
+                if (nchunks > 1) {
+                    wave_sync();
+                    build_shift_table(tab, t0c, cnt, bx, L, lane);
+                    wave_sync();
+                }
+                for (int t0 = 0; t0 < cnt; t0 += FC_GROUP) {
+                    const int t = t0 + sub;
+                    const float4 v = tab[min(t, cnt - 1)];
+                    const bool in = active && t < cnt && v.w <= reach;
+                    const uint64_t inm = __ballot(in);
+                    if (sorted && inm == 0) break;               // every row is past its reach (lengths ascend)
+                    const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                    fn(in, t, fmaf(dx, dx, fmaf(dy, dy, dz * dz)), __popcll(inm));
+                }
+            }
+        };
+
+        // scatter of the current list (entries point into the resident table)
+        auto heavy = [&](int nlist) {
+            for (int base = 0; base < nlist; base += WAVE) {
+                const int idx = base + lane;
+                if (idx < nlist) {
+                    const uint32_t ent = list[idx];
+                    const int pp = ent >> FC_SHIFT;
+                    const float4 v = tab[ent & (FC_TCAP - 1)];
+                    const float4 pa = pairA[pp];
+                    const float dx = pa.x + v.x, dy = pa.y + v.y, dz = pa.z + v.z;
+                    const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+                    const float w = hw_exp2(a2 * (d2 - pa.w)) * pairC[pp];
+                    {
+                        const float d = hw_sqrt(d2);
+                        const float u = d * bc.inv_interval;
+                        int start = (int)(u - bc.start_off);          // truncation toward zero
+                        start = max(0, min(start, NBINS - WL));
+                        const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
+                        const WindowSeed s = window_seed(beta_c, bc.len_step, w);
+                        window_scatter_rn<WL>(hist + start, s, bc.len_cc);
+                    }
+                    if (HAS_ANG) {
+                        if (d2 > 1e-5f) {       // the self image contributes to S and the distance encoding only
+                            const float rinv = hw_rsq(d2);
+#pragma unroll
+                            for (int ax = 0; ax < 3; ax++) {
+                                float cs = (dx * f[ax][0] + dy * f[ax][1] + dz * f[ax][2]) * rinv;
+                                if (COS_ABS) cs = fabsf(cs);
+                                const float uu = (cs - bc.ang_mu0) * bc.ang_inv_interval;      // in bin units
+                                const float mf = clampf(__builtin_rintf(uu), 0.0f, (float)(NBINS - 1));
+                                const float eps = 2.0f * (uu - mf);
+                                int32_t* hb = hist + HW_DIST + ax * NORD * NBINS + (int)mf;
+                                float val = w;
+                                atomicAdd(hb, rint_i(val));
+#pragma unroll
+                                for (int o = 1; o < NORD; o++) { val *= eps; atomicAdd(hb + o * NBINS, rint_i(val)); }
+                            }
+                        }
+                    }
+                }
+            }
+            n_eval += (unsigned long long)nlist;
+        };
+
+        for (int g0 = 0; g0 < npairs; g0 += FC_GROUP) {
+            const float rx = nrx, ry = nry, rz = nrz;
+            const float2 k2 = nk2, v2 = nv2;
+            if (g0 + FC_GROUP < npairs) fetch(g0 + FC_GROUP);
+            const bool active = g0 + pr < npairs;
+            const float rn = hw_sqrt(fmaf(rx, rx, fmaf(ry, ry, rz * rz)));
+
+            // ---- pass A: nearest image
+            float d2min = 3.0e38f;
+            sweep(active, rx, ry, rz, sorted ? fmaf(2.0002f, rn, 1e-4f) : INF,
+                  [&](bool in, int, float d2, int cnt_in) { d2min = in ? fminf(d2min, d2) : d2min; n_seen += cnt_in; });
+            d2min = half_min(d2min);
+
+            // ---- pass B: weights, normaliser and (one-chunk tables) the survivors
+            const float reachB = sorted ? fmaf(1.0001f, rn + hw_sqrt(d2min + cutS), 1e-4f) : INF;
+            float Sb = 0.0f;
+            int nlist = 0;
+            sweep(active, rx, ry, rz, reachB, [&](bool in, int t, float d2, int cnt_in) {
+                const float ex = a2 * (d2 - d2min);
+                Sb += in ? hw_exp2(ex) : 0.0f;
+                n_seen += cnt_in;
+                if (nchunks == 1) {
+                    const bool keep = in && ex >= prune;
+                    const uint64_t m = __ballot(keep);
+                    if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
+                    nlist += __popcll(m);
+                }
+            });
+            const float S = half_sum(Sb);
+
+            // ---- logits, running softmax
+            const float qk = half_sum(fmaf(q2.x, k2.x, q2.y * k2.y));
+            const float z = fmaf(hw_log2(S), LN2, a * d2min);
+            const float logit = active ? qk + z : -INF;
+            const float gmax = uniform_f(wave_maxf(logit));
+            if (gmax > m_run) {
+                if (m_run > -INF) {
+                    const float fac = hw_exp2((m_run - gmax) * LOG2E);
+                    for (int u = lane; u < HWK; u += WAVE) hist[u] = rint_i((float)hist[u] * fac);
+                    accv.x *= fac; accv.y *= fac; Dl *= fac;
+                }
+                m_run = gmax;
+            }
+            const float ew = active ? hw_exp2((logit - m_run) * LOG2E) : 0.0f;
+            accv.x = fmaf(ew, v2.x, accv.x);
+            accv.y = fmaf(ew, v2.y, accv.y);
+            if (sub == 0 && active) {
+                const size_t eh = (size_t)(e0 + g0 + pr) * H + h;
+                pairA[pr] = make_float4(rx, ry, rz, d2min);
+                pairC[pr] = ew / S * fixs;
+                C.z[eh] = z;
+                C.prob[eh] = logit;              // the logit for now; normalised when the row is complete
+                Dl += ew;
+            }
+            wave_sync();
+
+            // ---- heavy pass
+            if (nchunks == 1) heavy(nlist);
+            else {
+                for (int ch = 0; ch < nchunks; ch++) {
+                    const int t0c = ch * FC_TCAP;
+                    const int cnt = min(FC_TCAP, bx.T - t0c);
+                    wave_sync();
+                    build_shift_table(tab, t0c, cnt, bx, L, lane);
+                    wave_sync();
+                    int nl = 0;
+                    for (int t0 = 0; t0 < cnt; t0 += FC_GROUP) {
+                        const int t = t0 + sub;
+                        const float4 v = tab[min(t, cnt - 1)];
+                        const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                        const float ex = a2 * (fmaf(dx, dx, fmaf(dy, dy, dz * dz)) - d2min);
+                        const bool keep = active && t < cnt && ex >= prune;
+                        const uint64_t m = __ballot(keep);
+                        if (keep) list[nl + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
+                        nl += __popcll(m);
+                    }
+                    wave_sync();
+                    heavy(nl);
+                }
+            }
+            wave_sync();                      // list, pair data and (several chunks) the table may be rewritten
+        }
+
+        // ---- the row is complete: normalise and write
+        const float D = uniform_f(wave_sum(Dl));
+        const float inv = D > 0.0f ? 1.0f / D : 0.0f;
+        {
+            const float ox = rows8_sum(accv.x) * inv, oy = rows8_sum(accv.y) * inv;
+            if (lane < FC_GROUP) *reinterpret_cast<float2*>(C.out + ih * DH + 2 * sub) = make_float2(ox, oy);
+        }
+        {
+            const float sc = inv / fixs;
+            float* dst = C.hist + ih * HWK;
+            for (int u = lane; u < HWK; u += WAVE) {
+                dst[u] = (float)hist[u] * sc;
+                hist[u] = 0;
+            }
+        }
+        for (int g0 = 0; g0 < npairs; g0 += FC_GROUP) {          // logits -> probabilities (same lane wrote them)
+            if (sub == 0 && g0 + pr < npairs) {
+                const size_t eh = (size_t)(e0 + g0 + pr) * H + h;
+                C.prob[eh] = hw_exp2((C.prob[eh] - m_run) * LOG2E) * inv;
+            }
+        }
+        st_eval += n_eval;
+        st_seen += n_seen;
+        st_raw += (unsigned long long)bx.T * (unsigned long long)npairs;
+        st_pairs += (unsigned long long)npairs;
+        it_cur = it_next;
+        rec_cur = rec_next;
+        it_next = it_cur >= 0 ? queue_redeem(P, h, queue, ticket) : -1;
+    }
+    if (P.stats && lane == 0) {         // one set of atomics per wavefront
+        atomicAdd(P.stats + STAT_FWD_EVAL, st_eval);
+        atomicAdd(P.stats + STAT_FWD_RAW, st_raw);
+        atomicAdd(P.stats + STAT_FWD_PAIRS, st_pairs);
+        atomicAdd(P.stats + STAT_FWD_SEEN, st_seen);
+    }
+}
+
+// out (N,H,16) += Wcat_h (16, hw) . hist (N,H,hw): one wavefront per (16 atoms, head); MFMA 16x16x4, a lane owns 16
+// consecutive words of each 64-word step of the reduction index (64-byte loads of its row).  grid (ceil(N/16), H).
+__global__ __launch_bounds__(WAVE) void core_project_kernel(const float* __restrict__ hist, const float* __restrict__ wcat,
+                                                            float* __restrict__ out, int N, int H, int hw) {
+    const int lane = threadIdx.x, col = lane & 15, kk = lane >> 4;
+    const int h = blockIdx.y, i0 = blockIdx.x * 16;
+    const int row = min(i0 + col, N - 1);
+    const float4* ap = reinterpret_cast<const float4*>(hist + ((size_t)row * H + h) * hw) + 4 * kk;
+    const float4* bp = reinterpret_cast<const float4*>(wcat + ((size_t)h * DH + col) * hw) + 4 * kk;
+    v4f_c acc = {0.f, 0.f, 0.f, 0.f};
+    const int steps = hw / 64;
+#pragma unroll 2
+    for (int s = 0; s < steps; s++) {
+        float4 a4[4], b4[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) { a4[u] = ap[16 * s + u]; b4[u] = bp[16 * s + u]; }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u].x, b4[u].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u].y, b4[u].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u].z, b4[u].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u].w, b4[u].w, acc, 0, 0, 0);
+        }
+    }
+    // component r of lane (kk, col): atom 4 kk + r of the tile, channel col
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int it = i0 + 4 * kk + r;
+        if (it < N) out[((size_t)it * H + h) * DH + col] += acc[r];
+    }
+}
+
+// G (N,H,hw) = go (N,H,16) . Wcat_h (16, hw): wavefront per (16 atoms, head); per 64-word block four MFMA tiles whose
+// columns are interleaved (tile t, column c <-> word 4 c + t) so that a lane stores 16 consecutive bytes.
+// grid (ceil(N/16), H).
+__global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restrict__ go, const float* __restrict__ wcat,
+                                                           float* __restrict__ G, int N, int H, int hw) {
+    const int lane = threadIdx.x, col = lane & 15, kk = lane >> 4;
+    const int h = blockIdx.y, i0 = blockIdx.x * 16;
+    const int row = min(i0 + col, N - 1);
+    const float4 a4 = reinterpret_cast<const float4*>(go + ((size_t)row * H + h) * DH)[kk];      // channels 4 kk ..
+    const float A[4] = {a4.x, a4.y, a4.z, a4.w};
+    for (int w0 = 0; w0 < hw; w0 += 64) {
+        float4 b4[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            b4[j] = *reinterpret_cast<const float4*>(wcat + ((size_t)h * DH + 4 * kk + j) * hw + w0 + 4 * col);
+        v4f_c acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) acc[t] = v4f_c{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[j], b4[j].x, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[j], b4[j].y, acc[1], 0, 0, 0);
+            acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[j], b4[j].z, acc[2], 0, 0, 0);
+            acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(A[j], b4[j].w, acc[3], 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int it = i0 + 4 * kk + r;
+            if (it < N)
+                *reinterpret_cast<float4*>(G + ((size_t)it * H + h) * hw + w0 + 4 * col) =
+                    make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+        }
+    }
+}
+
+// gwcat (H,16,hw) += sum over a slice of the atoms of go (.,h,16) (x) hist (.,h,hw): wavefront per (head, 64-word
+// block, slice); four MFMA tiles with interleaved columns as above; float atomics into the cleared result.
+// grid (hw/64, H, nslices).
+__global__ __launch_bounds__(WAVE) void core_gwcat_kernel(const float* __restrict__ go, const float* __restrict__ hist,
+                                                          float* __restrict__ gwcat, int N, int H, int hw, int per_slice) {
+    const int lane = threadIdx.x, col = lane & 15, kk = lane >> 4;
+    const int w0 = blockIdx.x * 64, h = blockIdx.y;
+    const int i_begin = blockIdx.z * per_slice, i_end = min(N, i_begin + per_slice);
+    v4f_c acc[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) acc[t] = v4f_c{0.f, 0.f, 0.f, 0.f};
+    for (int ib = i_begin; ib < i_end; ib += 16) {
+        float av[4];
+        float4 bv[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int it = ib + 4 * j + kk;
+            const bool live = it < i_end;
+            const size_t base = ((size_t)(live ? it : i_begin) * H + h);
+            av[j] = live ? go[base * DH + col] : 0.0f;
+            bv[j] = live ? *reinterpret_cast<const float4*>(hist + base * hw + w0 + 4 * col) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j].x, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j].y, acc[1], 0, 0, 0);
+            acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j].z, acc[2], 0, 0, 0);
+            acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j].w, acc[3], 0, 0, 0);
+        }
+    }
+    // component r of tile t, lane (kk, col): channel 4 kk + r, word w0 + 4 col + t
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+            atomicAdd(gwcat + ((size_t)h * DH + 4 * kk + r) * hw + w0 + 4 * col + t, acc[t][r]);
+}
+
+__global__ void core_zero_kernel(float* p, int n) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < n) p[idx] = 0.0f;
+}
+
+// =================================================================================================================
+// backward
+// =================================================================================================================
+// Per item: G = Wcat^T go (made by core_gbuild_kernel) in LDS; for every image n of pair j with probability
+// p_n = exp(a d^2 - z) the value bg_n = sum_k b_k(d_n) G_k + sum_axis sum_o eps^o G'_(axis,o,m*) is gathered, and
+//     go . psi_ij          = sum_n p_n bg_n                                   (per pair, fixed-point LDS sums)
+//     gl_ij = dL/dlogit_ij = P_ij (go . v_j + go . psi_ij - go . out_i)
+//     ga_ih                = sum_j P_ij [(go . v_j - go . out_i) A0_j + sum_n p_n d_n^2 bg_n],  A0_j = sum_n p_n d_n^2
+//     gq_i                 = sum_j gl_ij k_j
+// (the terms A0_j (go . psi_ij) of dL/dz and of the covariance form cancel).  gk and gv are sums over the pairs that
+// point AT an atom and are left to the column kernel of the attention backward (from gl and P).
+template <int WL, bool HAS_ANG, bool COS_ABS>
+__global__ __launch_bounds__(WAVE) void fused_core_bwd_kernel(const CoreArgs C) {
+    constexpr int HWK = HAS_ANG ? HW_ANG : HW_DIST;
+    __shared__ float4 tab[FC_TCAP];
+    __shared__ uint16_t list[FC_LISTCAP];
+    __shared__ float Gs[HWK];
+    __shared__ float4 pairA[FC_GROUP];      // rx, ry, rz, z log2(e)
+    __shared__ float pairP[FC_GROUP];       // P_ij
+    __shared__ int32_t pairB[FC_GROUP];     // sum_n P_ij p_n bg_n in fixed point
+
+    const KernelArgs& P = C.K;
+    const int lane = threadIdx.x;
+    const int H = P.H;
+    const int h = blockIdx.x % H;
+    const int pr = lane >> 3, sub = lane & 7;
+    const BasisConsts bc = P.bc;
+    const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
+    const float INF = __builtin_inff();
+
+    unsigned long long st_eval = 0, st_raw = 0, st_pairs = 0;
+    int queue = first_queue(H);
+    int it_cur = queue_pop(P, h, queue);
+    int it_next = it_cur >= 0 ? queue_pop(P, h, queue) : -1;
+    uint32_t rec_cur = load_record(P, it_cur, h);
+    while (it_cur >= 0) {
+        const int ticket = queue_ticket(P, h, queue);
+        const uint32_t rec_next = load_record(P, it_next, h);
+        const CoreItem ci = core_unpack(C, rec_cur, true);
+        const int i = ci.item.i;
+        const float a2 = ci.item.a * LOG2E;
+        const Lattice L = ci.item.L;
+        const Box bx = ci.item.bx;
+        const bool sorted = ci.sorted;
+        const int nchunks = ci.nchunks;
+        float f[3][3];
+        if (HAS_ANG) {
+#pragma unroll
+            for (int ax = 0; ax < 3; ax++)
+#pragma unroll
+                for (int d = 0; d < 3; d++) f[ax][d] = rec_f(rec_cur, REC_FRAMES + ax * 3 + d);
+        }
+        const int e0 = ci.item.e0, npairs = ci.item.npairs;
+        const size_t ih = (size_t)i * H + h;
+        wave_sync();
+        core_load_table(C, ci, tab, lane);
+        float gabs = 0.0f;
+        {
+            const float* src = C.G + ih * HWK;
+            for (int u = lane; u < HWK; u += WAVE) { const float g = src[u]; Gs[u] = g; gabs += fabsf(g); }
+        }
+        const float2 go2 = *reinterpret_cast<const float2*>(C.go + ih * DH + 2 * sub);
+        const float2 ov2 = *reinterpret_cast<const float2*>(C.outv + ih * DH + 2 * sub);
+        const float c0 = half_sum(fmaf(go2.x, ov2.x, go2.y * ov2.y));          // go . out_i
+        const float gnorm = uniform_f(wave_sum(gabs));                          // |bg| <= sum |G|
+        const float bscale = 1073741824.0f / fmaxf(gnorm, 1e-30f);
+        const float binv = fmaxf(gnorm, 1e-30f) * (1.0f / 1073741824.0f);
+        wave_sync();
+        float cov = 0.0f;
+        float2 gq2 = make_float2(0.f, 0.f);
+        unsigned long long n_eval = 0;
+
+        float nrx = 0.f, nry = 0.f, nrz = 0.f, nz = 0.f, npb = 0.f;
+        float2 nk2 = make_float2(0.f, 0.f), nv2 = nk2;
+        auto fetch = [&](int g0) {
+            const int el = g0 + pr;
+            if (el < npairs) {
+                const size_t e = (size_t)(e0 + el);
+                const size_t jh = ((size_t)(ci.j0 + el) * H + h) * DH + 2 * sub;
+                nrx = P.rpos[e * 3 + 0]; nry = P.rpos[e * 3 + 1]; nrz = P.rpos[e * 3 + 2];
+                nz = C.z[e * H + h]; npb = C.prob[e * H + h];
+                nk2 = *reinterpret_cast<const float2*>(C.k + jh);
+                nv2 = *reinterpret_cast<const float2*>(C.v + jh);
+            }
+        };
+        fetch(0);
+
+        auto heavy = [&](int nlist) {
+            for (int base = 0; base < nlist; base += WAVE) {
+                const int idx = base + lane;
+                if (idx < nlist) {
+                    const uint32_t ent = list[idx];
+                    const int pp = ent >> FC_SHIFT;
+                    const float4 v = tab[ent & (FC_TCAP - 1)];
+                    const float4 pa = pairA[pp];
+                    const float dx = pa.x + v.x, dy = pa.y + v.y, dz = pa.z + v.z;
+                    const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+                    const float om = hw_exp2(fmaf(a2, d2, -pa.w)) * pairP[pp];       // P_ij p_n
+                    float bg;
+                    {
+                        const float d = hw_sqrt(d2);
+                        const float u = d * bc.inv_interval;
+                        int start = (int)(u - bc.start_off);
+                        start = max(0, min(start, NBINS - WL));
+                        const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
+                        const WindowSeed s = window_seed(beta_c, bc.len_step, 1.0f);
+                        bg = window_gather<WL>(Gs + start, s, bc.len_cc);
+                    }
+                    if (HAS_ANG) {
+                        if (d2 > 1e-5f) {
+                            const float rinv = hw_rsq(d2);
+#pragma unroll
+                            for (int ax = 0; ax < 3; ax++) {
+                                float cs = (dx * f[ax][0] + dy * f[ax][1] + dz * f[ax][2]) * rinv;
+                                if (COS_ABS) cs = fabsf(cs);
+                                const float uu = (cs - bc.ang_mu0) * bc.ang_inv_interval;
+                                const float mf = clampf(__builtin_rintf(uu), 0.0f, (float)(NBINS - 1));
+                                const float eps = 2.0f * (uu - mf);
+                                const float* gb = Gs + HW_DIST + ax * NORD * NBINS + (int)mf;
+                                float pw = eps, part = gb[0];
+#pragma unroll
+                                for (int o = 1; o < NORD; o++) { part = fmaf(pw, gb[o * NBINS], part); pw *= eps; }
+                                bg += part;
+                            }
+                        }
+                    }
+                    const float ob = om * bg;
+                    cov = fmaf(ob, d2, cov);
+                    atomicAdd(pairB + pp, rint_i(ob * bscale));
+                }
+            }
+            n_eval += (unsigned long long)nlist;
+        };
+
+        for (int g0 = 0; g0 < npairs; g0 += FC_GROUP) {
+            const float rx = nrx, ry = nry, rz = nrz;
+            const float z2 = nz * LOG2E, pij = npb;
+            const float2 k2 = nk2, v2 = nv2;
+            if (g0 + FC_GROUP < npairs) fetch(g0 + FC_GROUP);
+            const bool active = g0 + pr < npairs;
+            const float rn = hw_sqrt(fmaf(rx, rx, fmaf(ry, ry, rz * rz)));
+            // images with a d^2 log2 e - z2 >= -skip: d^2 <= (z2 - skip) / (a log2 e)
+            const float dmax2 = (C.skip_log2 > 0.0f && a2 < 0.0f) ? fmaxf((z2 - C.skip_log2) / a2, 0.0f) : INF;
+            const float reach = sorted ? fmaf(1.0001f, rn + hw_sqrt(dmax2), 1e-4f) : INF;
+            if (lane < FC_GROUP) pairB[lane] = 0;
+            if (sub == 0 && active) {
+                pairA[pr] = make_float4(rx, ry, rz, z2);
+                pairP[pr] = pij;
+            }
+            float Ap = 0.0f;
+            int nlist = 0;
+            for (int ch = 0; ch < nchunks; ch++) {
+                const int t0c = ch * FC_TCAP;
+                const int cnt = sorted ? bx.T : min(FC_TCAP, bx.T - t0c);
+                if (nchunks > 1) {
+                    wave_sync();
+                    build_shift_table(tab, t0c, cnt, bx, L, lane);
+                    wave_sync();
+                }
+                for (int t0 = 0; t0 < cnt; t0 += FC_GROUP) {
+                    const int t = t0 + sub;
+                    const float4 v = tab[min(t, cnt - 1)];
+                    const bool in = active && t < cnt && v.w <= reach;
+                    if (sorted && __ballot(in) == 0) break;
+                    const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                    const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+                    const float ex = fmaf(a2, d2, -z2);
+                    Ap += in ? hw_exp2(ex) * d2 : 0.0f;
+                    if (nchunks == 1) {
+                        const bool keep = in && ex >= prune;
+                        const uint64_t m = __ballot(keep);
+                        if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
+                        nlist += __popcll(m);
+                    }
+                }
+            }
+            const float A0 = half_sum(Ap);
+            wave_sync();
+            if (nchunks == 1) heavy(nlist);
+            else {
+                for (int ch = 0; ch < nchunks; ch++) {
+                    const int t0c = ch * FC_TCAP;
+                    const int cnt = min(FC_TCAP, bx.T - t0c);
+                    wave_sync();
+                    build_shift_table(tab, t0c, cnt, bx, L, lane);
+                    wave_sync();
+                    int nl = 0;
+                    for (int t0 = 0; t0 < cnt; t0 += FC_GROUP) {
+                        const int t = t0 + sub;
+                        const float4 v = tab[min(t, cnt - 1)];
+                        const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                        const float ex = fmaf(a2, fmaf(dx, dx, fmaf(dy, dy, dz * dz)), -z2);
+                        const bool keep = active && t < cnt && ex >= prune;
+                        const uint64_t m = __ballot(keep);
+                        if (keep) list[nl + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
+                        nl += __popcll(m);
+                    }
+                    wave_sync();
+                    heavy(nl);
+                }
+            }
+            wave_sync();
+            const float gov = half_sum(fmaf(go2.x, v2.x, go2.y * v2.y));          // go . v_j
+            const float B1 = (float)pairB[pr] * binv;                             // P_ij (go . psi_ij)
+            const float gl = active ? fmaf(pij, gov - c0, B1) : 0.0f;
+            gq2.x = fmaf(gl, k2.x, gq2.x);
+            gq2.y = fmaf(gl, k2.y, gq2.y);
+            if (sub == 0 && active) {
+                C.glogit[(size_t)(e0 + g0 + pr) * H + h] = gl;
+                cov = fmaf(pij * (gov - c0), A0, cov);
+            }
+            wave_sync();                      // pair data, sums and list may be rewritten
+        }
+        cov = wave_sum(cov);
+        {
+            const float gx = rows8_sum(gq2.x), gy = rows8_sum(gq2.y);
+            if (lane < FC_GROUP) *reinterpret_cast<float2*>(C.gq + ih * DH + 2 * sub) = make_float2(gx, gy);
+        }
+        if (lane == 0) P.out_ga[ih] = cov;
+        st_eval += n_eval;
+        st_raw += (unsigned long long)bx.T * (unsigned long long)npairs;
+        st_pairs += (unsigned long long)npairs;
+        it_cur = it_next;
+        rec_cur = rec_next;
+        it_next = it_cur >= 0 ? queue_redeem(P, h, queue, ticket) : -1;
+    }
+    if (P.stats && lane == 0) {
+        atomicAdd(P.stats + STAT_BWD_EVAL, st_eval);
+        atomicAdd(P.stats + STAT_BWD_RAW, st_raw);
+        atomicAdd(P.stats + STAT_BWD_PAIRS, st_pairs);
+    }
+}
+
+}  // namespace cfh

@@ -528,6 +528,113 @@ class FusedDotProductAttentionCUDA(torch.autograd.Function):
                 gb.to(dt) if gb is not None else None, None, None)
 
 
+class PeriodicAttentionCoreHIP(torch.autograd.Function):
+    """The attention core of a layer in one library call:
+
+        out_i = sum_j P_ij (v_j + psi_ij),   P_i. = softmax_j (qs_i . k_j + z_ij)
+
+    with z and psi the lattice sums of RealEncodingWithFramedProjFuncCUDA and, when ``frames`` is None and the
+    angle encoding is on, the "max" frames searched in the same call.  Returns ``(out (N,H,Dh), frames (3,N,H,3)
+    or None)``; gradients flow to qs, k, v, a_ik and the four projection weights.  ``qs`` is the query already
+    divided by sqrt(Dh).  Same result as RealEncodingWithMaxFramesFuncHIP followed by FusedDotProductAttentionCUDA
+    (the reference's sequence, models/indexed_lattice_multi_head_attention_cuda.py:589-734 and :144-185), computed
+    with one histogram per (atom, head) instead of one per (pair, head): psi (E,H,Dh) is never formed.  The angle
+    encoding uses the full Gaussian basis (no +-4 sigma window; a 6-term series around the nearest bin), the
+    distance encoding the window of ``KernelManager.WINDOW_MODE``.  No counterpart class in the reference."""
+
+    @staticmethod
+    def supported(K, dim_angle_enc, wscale, angle_wscale, W_k, W_k1) -> bool:
+        if W_k is None or int(K) != 64 or float(wscale) != 1.0 or KernelManager.GRAD_COEF_QUIRK:
+            return False
+        if W_k.dim() == 4 and W_k.shape[0] != 1:
+            return False
+        A = int(dim_angle_enc) if W_k1 is not None else 0
+        return A == 0 or (A == 64 and float(angle_wscale) >= 3.0)
+
+    @staticmethod
+    def forward(ctx, qs, k, v, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, W_k, W_k1, W_k2,
+                W_k3, dim_angle_enc, value_pe_angle_scale, cos_abs, length_rbf_mul, angle_rbf_mul, rvlen_n=None,
+                cutoff_radius=None, frames=None):
+        _lib.require_gpu(qs, k, v, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e)
+        lib = _lib.load()
+        N, H = a_ik.shape
+        E = edge_ij_e.shape[1]
+        dev = a_ik.device
+        use_angle = W_k1 is not None and int(dim_angle_enc) > 0
+        A = int(dim_angle_enc) if use_angle else 0
+        Wd = _proj_weight(W_k, H, "W_k")
+        Wa = [_proj_weight(w, H, "W_k%d" % (n + 1)) for n, w in enumerate((W_k1, W_k2, W_k3))] if use_angle \
+            else [None, None, None]
+        Dh = Wd.shape[-2]
+        q_, k_, v_, a = _f32c(qs), _f32c(k), _f32c(v), _f32c(a_ik)
+        rpos, tv, rv = _f32c(rpos_ij_e), _f32c(tvecs_n), _f32c(rvlen_n)
+        batch, edges = batch_i.contiguous(), edge_ij_e.contiguous()
+        e_start, order = edge_schedule(edge_ij_e, N)
+        _require_complete_blocks(edge_ij_e, e_start, N)
+        p = _params(H, Dh, int(K), A, cos_abs, float(dist_max), wscale, value_pe_angle_scale, length_rbf_mul,
+                    angle_rbf_mul, cutoff_radius if rv is not None else None)
+        hw = int(lib.cfh_fused_core_hist_words(ctypes.byref(p)))
+        if hw <= 0:
+            _lib.check(-1, "cfh_fused_core_hist_words")
+        search = use_angle and frames is None
+        if use_angle:
+            fr = torch.empty((3, N, H, 3), dtype=torch.float32, device=dev) if search else _f32c(frames)
+        else:
+            fr = None
+        z = torch.empty((E, H), dtype=torch.float32, device=dev)
+        prob = torch.empty((E, H), dtype=torch.float32, device=dev)
+        hist = torch.empty((N, H, hw), dtype=torch.float32, device=dev)
+        out = torch.empty((N, H, Dh), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev), _timed("fused_core_forward", dev):
+            ws = _lib.workspace(dev, lib.cfh_fused_core_workspace_bytes(ctypes.byref(p), N, E, tv.shape[0], 0))
+            rc = lib.cfh_fused_core_forward(
+                ctypes.byref(p), _lib.ptr(q_), _lib.ptr(k_), _lib.ptr(v_), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv),
+                _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd),
+                _lib.ptr(Wa[0]), _lib.ptr(Wa[1]), _lib.ptr(Wa[2]), N, E, tv.shape[0], _lib.ptr(fr), 1 if search else 0,
+                _lib.ptr(z), _lib.ptr(prob), _lib.ptr(hist), _lib.ptr(out), _lib.ptr(ws), ws.numel(),
+                _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_fused_core_forward")
+        ctx.save_for_backward(q_, k_, v_, a, rpos, tv, rv, batch, edges, e_start, order, Wd, Wa[0], Wa[1], Wa[2], fr,
+                              z, prob, hist, out)
+        ctx.params = p
+        ctx.w_shapes = [None if w is None else w.shape for w in (W_k, W_k1, W_k2, W_k3)]
+        ctx.in_dtype = qs.dtype
+        if fr is not None:
+            ctx.mark_non_differentiable(fr)
+        ctx.set_materialize_grads(False)
+        return out, fr
+
+    @staticmethod
+    def backward(ctx, gout, gframes=None):
+        (q_, k_, v_, a, rpos, tv, rv, batch, edges, e_start, order, Wd, W1, W2, W3, fr, z, prob, hist,
+         out) = ctx.saved_tensors
+        lib = _lib.load()
+        p = ctx.params
+        N, H = a.shape
+        E = edges.shape[1]
+        dev = a.device
+        go = _f32c(gout) if gout is not None else torch.zeros_like(out)
+        gq, gk, gv = torch.empty_like(q_), torch.empty_like(k_), torch.empty_like(v_)
+        ga = torch.empty((N, H), dtype=torch.float32, device=dev)
+        glogit = torch.empty((E, H), dtype=torch.float32, device=dev)
+        gWd = torch.empty_like(Wd)
+        gWa = [torch.empty_like(w) if w is not None else None for w in (W1, W2, W3)]
+        with torch.cuda.device(dev), _timed("fused_core_backward", dev):
+            ws = _lib.workspace(dev, lib.cfh_fused_core_workspace_bytes(ctypes.byref(p), N, E, tv.shape[0], 1))
+            rc = lib.cfh_fused_core_backward(
+                ctypes.byref(p), _lib.ptr(q_), _lib.ptr(k_), _lib.ptr(v_), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv),
+                _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd),
+                _lib.ptr(W1), _lib.ptr(W2), _lib.ptr(W3), _lib.ptr(fr), _lib.ptr(z), _lib.ptr(prob), _lib.ptr(hist),
+                _lib.ptr(out), _lib.ptr(go), N, E, tv.shape[0], _lib.ptr(gq), _lib.ptr(gk), _lib.ptr(gv), _lib.ptr(ga),
+                _lib.ptr(glogit), _lib.ptr(gWd), _lib.ptr(gWa[0]), _lib.ptr(gWa[1]), _lib.ptr(gWa[2]), _lib.ptr(ws),
+                ws.numel(), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_fused_core_backward")
+        gws = [g if g is None else g.reshape(s) for g, s in zip([gWd] + gWa, ctx.w_shapes)]
+        dt = ctx.in_dtype
+        return (gq.to(dt), gk.to(dt), gv.to(dt), ga, None, None, None, None, None, None, None, gws[0], gws[1], gws[2],
+                gws[3], None, None, None, None, None, None, None, None)
+
+
 class IrregularMeanCUDA(torch.autograd.Function):
     """Per-crystal mean of per-atom features.  Signature of models/cuda_funcs/irregular_mean.py:19-70."""
 

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 6
+#define CFH_ABI_VERSION 7
 
 enum {
     CFH_OK = 0,
@@ -276,6 +276,51 @@ int cfh_fused_dpa_backward(const float* q, const float* k, const float* v, const
                            const float* prob, const float* out, const float* gout, int64_t N,
                            int64_t H, int64_t Dh, int64_t E, float* gq, float* gk, float* gv,
                            float* gaij, float* gbij, void* stream);
+
+/*
+ * The attention core of a layer in one call: lattice sums, softmax over the pairs of every atom and the value
+ * encoding, with the "max" frame search in front when search_frames != 0 (frames (3,N,H,3) is then an output,
+ * else an input; unused without the angle encoding):
+ *     out_i = sum_j P_ij (v_j + psi_ij),  P_i. = softmax_j (qs_i . k_j + z_ij),
+ * i.e. cfh_frame_axes, cfh_framed_pe_forward and cfh_fused_dpa_forward composed
+ * (models/indexed_lattice_multi_head_attention_cuda.py:589-734 and :144-185; models/cuda_funcs/fused_dpa.py:17-63),
+ * computed differently: because out is linear in psi = W . s, the basis values of all images of all pairs of an
+ * atom are scattered, weighted by P_ij p_n, into ONE histogram per (atom, head), which is projected once.
+ * psi (E,H,Dh) and the per-pair histograms are never formed.  The distance basis keeps the truncated window of
+ * window_mode; the angle basis is the FULL Gaussian basis (no truncation: the pure-PyTorch formulation,
+ * models/indexed_lattice_multi_head_attention.py:580-588), evaluated as a 6-term series around the nearest bin
+ * (error < 1e-7 of a basis function's peak for angle_wscale 4; angle_wscale < 3 returns CFH_EINVAL).
+ * Needs dist_bins = 64, dist_wscale = 1, angle_bins 0 or 64, and the pairs as the complete n x n block of every
+ * crystal (cfh_pair_layout_check).  qs = query / sqrt(Dh).
+ * Results kept for the backward: z (E,H), prob (E,H) = P, hist (N,H,words) the normalised histograms
+ * (words = cfh_fused_core_hist_words: 64 distance bins, then per axis and order 64 moment bins), out (N,H,Dh).
+ * workspace: cfh_fused_core_workspace_bytes(p, N, E, B, 0).
+ */
+size_t cfh_fused_core_workspace_bytes(const cfh_params* p, int64_t N, int64_t E, int64_t B, int32_t backward);
+int32_t cfh_fused_core_hist_words(const cfh_params* p);
+int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k, const float* v, const float* a_ih,
+                           const float* rpos, const float* tvecs, const float* rvlen, const int64_t* batch,
+                           const int64_t* edges, const int64_t* e_start, const int32_t* order, const float* W_dist,
+                           const float* W_axis1, const float* W_axis2, const float* W_axis3, int64_t N, int64_t E,
+                           int64_t B, float* frames, int32_t search_frames, float* z, float* prob, float* hist,
+                           float* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Gradients of the above for upstream gout (N,H,Dh): gq (of qs), gk, gv (N,H,Dh), ga (N,H), the four weight
+ * gradients (H,Dh,64) summed over atoms; glogit (E,H) is scratch the caller provides (the gradient of the logits).
+ * No gradient flows to the frames.  What FusedDotProductAttentionCUDA.backward and
+ * RealEncodingWithFramedProjFuncCUDA.backward compute together (models/cuda_funcs/fused_dpa.py:65-170,
+ * real_space_framed_proj.py:123-221); the weight gradients add their atoms with float atomics.
+ * workspace: cfh_fused_core_workspace_bytes(p, N, E, B, 1).
+ */
+int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k, const float* v, const float* a_ih,
+                            const float* rpos, const float* tvecs, const float* rvlen, const int64_t* batch,
+                            const int64_t* edges, const int64_t* e_start, const int32_t* order, const float* W_dist,
+                            const float* W_axis1, const float* W_axis2, const float* W_axis3, const float* frames,
+                            const float* z, const float* prob, const float* hist, const float* out, const float* gout,
+                            int64_t N, int64_t E, int64_t B, float* gq, float* gk, float* gv, float* ga, float* glogit,
+                            float* gW_dist, float* gW_axis1, float* gW_axis2, float* gW_axis3, void* workspace,
+                            size_t workspace_bytes, void* stream);
 
 /*
  * Sets *flag (device memory) to 0 when edges (2,E) / e_start (N+1) hold, for every crystal, all

@@ -1,0 +1,211 @@
+"""The fused attention core (cfh_fused_core_forward / backward through PeriodicAttentionCoreHIP) against the
+float64 oracle composition  TO.framed_pe -> TO.softmax_attention  (autograd for every gradient), and against the
+two-step operators of the library.  The fused core sums the same translation sets and uses the same distance
+windows as the two-step path; its angle encoding is the FULL Gaussian basis (a 6-term series around the nearest
+bin), so the oracle runs with windows = (9, None): 9-bin distance window, untruncated angle basis.
+
+Tolerances (relative to the largest magnitude of the tensor): 2e-5 forward, 1e-4 gradients."""
+import math
+
+import pytest
+import torch
+
+import helpers as Hh
+from oracle import torch_oracle as TO
+
+pytestmark = pytest.mark.gpu
+
+CUT = -3.5
+
+
+@pytest.fixture(autouse=True)
+def _defaults():
+    import crystalframer_amd as cf
+    KM = cf.KernelManager
+    names = ("SYMM_BREAK_NOISE", "PRUNE_LOG2", "WINDOW_MODE", "GRAD_COEF_QUIRK", "LATTICE_RANGE", "MINIMUM_RANGE",
+             "SAVE_HISTOGRAMS", "SECOND_STREAM", "NOISE_SEED", "NOISE_SEED_DEVICE")
+    saved = {n: getattr(KM, n) for n in names}
+    KM.SYMM_BREAK_NOISE, KM.PRUNE_LOG2, KM.WINDOW_MODE, KM.GRAD_COEF_QUIRK = 0.0, 24.0, 0, False
+    KM.LATTICE_RANGE, KM.MINIMUM_RANGE = 2, 2
+    yield
+    for n, v in saved.items():
+        setattr(KM, n, v)
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def g(t):
+    return None if t is None else t.to(dtype=torch.float32, device=dev())
+
+
+def run_core(P, *, A=64, cos_abs=0, cd=1.0, ca=1.0, cutoff=CUT, frames="given", need_grad=True):
+    from crystalframer_amd import cuda_funcs as F
+    leaves = dict(q=g(P.q), k=g(P.k), v=g(P.v), a=g(P.a), Wk=g(P.W_k))
+    if A > 0:
+        for n in range(3):
+            leaves["W%d" % (n + 1)] = g(P.W_ax[n])
+    for t in leaves.values():
+        t.requires_grad_(need_grad)
+    Wax = [leaves.get("W%d" % n) for n in (1, 2, 3)]
+    fr = None
+    if A > 0 and frames == "given":
+        fr = torch.stack([g(f) for f in P.frames], 0)
+    extra = (g(P.rvlen), cutoff) if cutoff is not None else (None, None)
+    out, fr_out = F.PeriodicAttentionCoreHIP.apply(
+        leaves["q"], leaves["k"], leaves["v"], leaves["a"], g(P.rpos), g(P.tvecs), P.batch.to(dev()), P.edges.to(dev()),
+        64, Hh.DIST_MAX, 1.0, leaves["Wk"], Wax[0], Wax[1], Wax[2], A, 4.0, cos_abs, cd, ca, extra[0], extra[1], fr)
+    return out, fr_out, leaves
+
+
+def oracle_core(P, *, A=64, cos_abs=0, cd=1.0, ca=1.0, cutoff=CUT, frames=None, wl=9):
+    leaves = dict(q=P.q.clone(), k=P.k.clone(), v=P.v.clone(), a=P.a.clone(), Wk=P.W_k.clone())
+    if A > 0:
+        for n in range(3):
+            leaves["W%d" % (n + 1)] = P.W_ax[n].clone()
+    for t in leaves.values():
+        t.requires_grad_(True)
+    Wax = [leaves["W%d" % n] for n in (1, 2, 3)] if A > 0 else None
+    z, psi = TO.framed_pe(leaves["a"], P.rpos, P.tvecs, P.batch, P.edges, leaves["Wk"], Wax, frames or P.frames, K=64,
+                          A=A, cos_abs=cos_abs, c_dist=cd, c_angle=ca, rvlen=P.rvlen, cutoff_radius=cutoff,
+                          windows=(wl, None))
+    out, prob = TO.softmax_attention(leaves["q"], leaves["k"], leaves["v"], z, psi, P.batch, P.edges)
+    return out, leaves
+
+
+def compare(P, gout, out, leaves, oo, oleaves, ftol=2e-5, gtol=1e-4):
+    assert torch.isfinite(out).all()
+    assert Hh.rel_err(out, oo) < ftol
+    (out * g(gout)).sum().backward()
+    (oo * gout).sum().backward()
+    for name, t in leaves.items():
+        assert t.grad is not None and torch.isfinite(t.grad).all(), name
+        ref = oleaves[name].grad
+        if float(ref.abs().max()) < 1e-12:        # e.g. the query gradient of a one-pair row: exactly zero
+            assert float(t.grad.abs().max()) < 1e-5, name
+        else:
+            assert Hh.rel_err(t.grad, ref) < gtol, name
+
+
+def _gout(P, seed=77):
+    gen = torch.Generator().manual_seed(seed)
+    return torch.randn(P.N, Hh.H, Hh.DH, generator=gen, dtype=torch.float64)
+
+
+@pytest.mark.parametrize("cos_abs", [0, 1])
+@pytest.mark.parametrize("prune", [24.0, 0.0])
+def test_fused_core_matches_oracle_composition(cos_abs, prune):
+    """prune 24: sorted tables and skipped prefixes; prune 0: every translation of every box is evaluated."""
+    import crystalframer_amd as cf
+    cf.KernelManager.PRUNE_LOG2 = prune
+    P = Hh.make_problem(num_crystals=10, atoms_hi=6, seed=200 + cos_abs)
+    cd, ca = 0.75, 1.25
+    out, _, leaves = run_core(P, cos_abs=cos_abs, cd=cd, ca=ca)
+    oo, oleaves = oracle_core(P, cos_abs=cos_abs, cd=cd, ca=ca)
+    compare(P, _gout(P), out, leaves, oo, oleaves)
+
+
+def test_fused_core_distance_encoding_only():
+    P = Hh.make_problem(num_crystals=8, atoms_hi=7, seed=211)
+    out, fr, leaves = run_core(P, A=0)
+    assert fr is None
+    oo, oleaves = oracle_core(P, A=0)
+    compare(P, _gout(P), out, leaves, oo, oleaves)
+
+
+def test_fused_core_fixed_box_and_wide_distance_window():
+    import crystalframer_amd as cf
+    cf.KernelManager.WINDOW_MODE = 1
+    P = Hh.make_problem(num_crystals=8, atoms_hi=5, seed=213)
+    out, _, leaves = run_core(P, cutoff=None)
+    oo, oleaves = oracle_core(P, cutoff=None, wl=11)
+    compare(P, _gout(P), out, leaves, oo, oleaves)
+    # and against the untruncated distance basis: the bar of 1e-4
+    leaves2 = {k: v.clone().requires_grad_(True) for k, v in dict(q=P.q, k=P.k, v=P.v, a=P.a, Wk=P.W_k).items()}
+    z, psi = TO.framed_pe(leaves2["a"], P.rpos, P.tvecs, P.batch, P.edges, leaves2["Wk"], P.W_ax, P.frames,
+                          cutoff_radius=None, windows="full")
+    of, _ = TO.softmax_attention(leaves2["q"], leaves2["k"], leaves2["v"], z, psi, P.batch, P.edges)
+    assert Hh.rel_err(out, of) < 1e-4
+
+
+def test_fused_core_small_cells_with_boxes_of_several_chunks():
+    """Cells of 1.5-2 angstrom: boxes of more than 512 translations (tables rebuilt chunk by chunk)."""
+    P = Hh.make_problem(num_crystals=4, atoms_lo=1, atoms_hi=3, len_lo=1.5, len_hi=2.0, ang_lo=80, ang_hi=100, seed=37)
+    R = TO.translation_ranges(P.a, P.rvlen, P.batch, CUT)
+    assert int((2 * R + 1).prod(-1).max()) > 512
+    out, _, leaves = run_core(P)
+    oo, oleaves = oracle_core(P)
+    compare(P, _gout(P), out, leaves, oo, oleaves)
+
+
+def test_fused_core_mixed_boxes_and_long_rows():
+    """Crystals of up to 40 atoms (rows of several groups, the running softmax rescales) with cell sizes that
+    mix the usual box with larger ones."""
+    P = Hh.make_problem(num_crystals=5, atoms_lo=20, atoms_hi=40, len_lo=2.5, len_hi=9.0, seed=219)
+    P.q = P.q * 4.0          # sharper attention: larger changes of the running maximum
+    out, _, leaves = run_core(P)
+    oo, oleaves = oracle_core(P)
+    compare(P, _gout(P), out, leaves, oo, oleaves, gtol=2e-4)
+
+
+def test_fused_core_with_frame_search_equals_two_step_path():
+    """frames=None: the search runs in the same call; its frames are those of ComputeFramesMaximumMethodCUDA
+    bit for bit, and out equals the two-step operators with those frames up to the truncation of their angle
+    windows (5-sigma windows: 1e-4)."""
+    import crystalframer_amd as cf
+    cf.KernelManager.WINDOW_MODE = 1
+    P = Hh.make_problem(num_crystals=12, atoms_hi=6, seed=83)
+    out, fr, leaves = run_core(P, frames="search")
+    ref_fr = cf.ComputeFramesMaximumMethodCUDA.apply(g(P.q), g(P.k), None, g(P.a), g(P.rpos), None, g(P.tvecs),
+                                                     P.batch.to(dev()), P.edges.to(dev()), 64, Hh.DIST_MAX, 1.0,
+                                                     g(P.rvlen), CUT)
+    assert torch.equal(fr, ref_fr)
+    z, psi = cf.RealEncodingWithFramedProjFuncCUDA.apply(
+        g(P.a), g(P.rpos), None, g(P.tvecs), P.batch.to(dev()), P.edges.to(dev()), 64, Hh.DIST_MAX, 1.0, g(P.W_k),
+        g(P.W_ax[0]), g(P.W_ax[1]), g(P.W_ax[2]), fr[0], fr[1], fr[2], 64, 4.0, 0, 1.0, 1.0, g(P.rvlen), CUT)
+    two = cf.FusedDotProductAttentionCUDA.apply(g(P.q), g(P.k), g(P.v), z, psi, P.batch.to(dev()), P.edges.to(dev()))
+    assert Hh.rel_err(out, two.double().cpu()) < 1e-4
+    oo, oleaves = oracle_core(P, frames=[f.double().cpu() for f in fr], wl=11)
+    compare(P, _gout(P), out, leaves, oo, oleaves)
+
+
+def test_fused_core_one_atom_crystals_and_empty_batch():
+    from crystalframer_amd import cuda_funcs as F
+    P = Hh.make_problem(num_crystals=5, atoms_lo=1, atoms_hi=1, seed=41)
+    out, _, leaves = run_core(P)
+    oo, oleaves = oracle_core(P)
+    compare(P, _gout(P), out, leaves, oo, oleaves)
+    d = dev()
+    Wk = g(P.W_k).requires_grad_(True)
+    Wax = [g(w).requires_grad_(True) for w in P.W_ax]
+    a = torch.zeros(0, Hh.H, device=d, requires_grad=True)
+    e3 = torch.zeros(0, Hh.H, Hh.DH, device=d)
+    out, fr = F.PeriodicAttentionCoreHIP.apply(
+        e3, e3, e3, a, torch.zeros(0, 3, device=d), torch.zeros(0, 3, 3, device=d),
+        torch.zeros(0, dtype=torch.long, device=d), torch.zeros(2, 0, dtype=torch.long, device=d), 64, Hh.DIST_MAX, 1.0,
+        Wk, *Wax, 64, 4.0, 0, 1.0, 1.0)
+    assert out.shape == (0, Hh.H, Hh.DH) and fr.shape == (3, 0, Hh.H, 3)
+    out.sum().backward()
+    assert float(Wk.grad.abs().max()) == 0.0 and float(Wax[1].grad.abs().max()) == 0.0
+
+
+def test_fused_core_at_batch_256_against_oracle_on_first_crystals():
+    """The benchmark's batch: the core on all 256 crystals; the upstream gradient is zero outside the first 6
+    crystals, so every gradient can be compared with the oracle run on those crystals alone."""
+    from crystalframer_amd import synthetic
+    P = Hh.problem_from_batch(synthetic.make_config("C2"), seed=9)
+    S = Hh.first_crystals(P, 6)
+    gout = torch.zeros(P.N, Hh.H, Hh.DH, dtype=torch.float64)
+    gout[:S.N] = _gout(S, seed=5)
+    out, _, leaves = run_core(P)
+    oo, oleaves = oracle_core(S)
+    assert torch.isfinite(out).all()
+    assert Hh.rel_err(out[:S.N], oo) < 2e-5 and Hh.elem_err(out[:S.N], oo, atol_frac=1e-5) <= 1.0
+    (out * g(gout)).sum().backward()
+    (oo * gout[:S.N]).sum().backward()
+    for name in ("q", "k", "v", "a"):
+        assert Hh.rel_err(leaves[name].grad[:S.N], oleaves[name].grad) < 1e-4, name
+        assert float(leaves[name].grad[S.N:].abs().max()) == 0.0, name
+    for name in ("Wk", "W1", "W2", "W3"):
+        assert Hh.rel_err(leaves[name].grad, oleaves[name].grad) < 1e-4, name
