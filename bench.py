@@ -171,7 +171,7 @@ def main():
     _lib.kernel_timing(False)
     log, KM.EVENT_LOG = KM.EVENT_LOG, None
     kern_ms = {}
-    for what in ("frame_axes", "framed_pe_forward", "framed_pe_backward"):
+    for what in ("frame_axes", "framed_pe_forward", "framed_pe_backward", "fused_core_forward", "fused_core_backward"):
         total, count = _lib.read_kernel_timing(what)
         if count:
             kern_ms[what] = total / count
@@ -190,8 +190,13 @@ def main():
     launches = {k: len(v) // nprof for k, v in per_kernel.items()}
     lib_ms_per_step = sum(sum(v) for v in per_kernel.values()) / nprof
 
-    nlaunch_bwd = max(1, len(per_kernel.get("framed_pe_backward", [])))
-    nlaunch_fwd = max(1, len(per_kernel.get("framed_pe_forward", [])) + len(per_kernel.get("frame_axes_framed_pe_forward", [])))
+    fused = "fused_core_forward" in kern_ms
+    if fused:
+        kern_ms["framed_pe_forward"] = kern_ms["fused_core_forward"]
+        kern_ms["framed_pe_backward"] = kern_ms["fused_core_backward"]
+    nlaunch_bwd = max(1, len(per_kernel.get("framed_pe_backward", [])) + len(per_kernel.get("fused_core_backward", [])))
+    nlaunch_fwd = max(1, len(per_kernel.get("framed_pe_forward", [])) + len(per_kernel.get("frame_axes_framed_pe_forward", []))
+                      + len(per_kernel.get("fused_core_forward", [])))
     bwd_eval = stats["bwd_evaluated"] / nlaunch_bwd          # terms evaluated per launch
     bwd_box = stats["bwd_in_box"] / nlaunch_bwd              # terms in the reference's boxes per launch
     bwd_pairs = stats["bwd_pairs"] / nlaunch_bwd

@@ -224,10 +224,13 @@ STAT_NAMES = ("fwd_evaluated", "fwd_in_box", "bwd_evaluated", "bwd_in_box", "fra
 def read_stats(device: torch.device, reset: bool = False) -> dict:
     """Term counts accumulated by launches made with ``collect_stats`` on this stream (synchronises)."""
     buf = workspace(device, 512)
-    vals = buf[256:256 + 8 * len(STAT_NAMES)].view(torch.int64).cpu().tolist()
+    vals = buf[256:512].view(torch.int64).cpu().tolist()
     if reset:
         buf[256:512].zero_()
-    return dict(zip(STAT_NAMES, vals))
+    out = dict(zip(STAT_NAMES, vals))
+    if any(vals[16:24]):        # cycle counts of a diagnostics build (phase timing of the fused forward kernel)
+        out["phase_cycles"] = vals[16:24]
+    return out
 
 
 def read_status(device: torch.device, reset: bool = False) -> int:

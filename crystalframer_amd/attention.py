@@ -24,6 +24,8 @@ from .params import LatticeformerParams
 FUSED_FRAMES = True      # one launch for both axes + orthogonalisation (False: the reference's three steps)
 FUSED_FRAMES_PE = True   # frame search and lattice sums in one library call (False: two calls, as the reference makes them)
 FUSED_INPUTS = True      # q/k/v split, query scaling and Gaussian coefficient in one launch (False: framework ops)
+FUSED_CORE = True        # frames, lattice sums and softmax attention in one library call with one histogram per
+                         # (atom, head) (cuda_funcs.PeriodicAttentionCoreHIP); False: the reference's sequence of operators
 
 
 def compute_frame_maximum_method_(q, k, v, alpha, pos, dist2_min, tvecs, batch, edges, proj, K: int,
@@ -302,6 +304,29 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
         """Frames, lattice sums and the softmax attention for projected q, k, v (N,H,Dh) and Gaussian
         coefficients a (N,H): the heads' outputs side by side (N, H Dv), before the output projection,
         and psi."""
+        P = self.params
+        if (FUSED_CORE and q.is_cuda and P.frame_method == "max" and batch_q is batch_kv and self.pe_dist_proj is not None
+                and cuda_funcs.PeriodicAttentionCoreHIP.supported(
+                    P.value_pe_dist_real, P.value_pe_angle_real, P.value_pe_dist_wscale, P.value_pe_angle_wscale,
+                    self.pe_dist_proj, self.proj_angle1)):
+            # one library call: frame search, lattice sums, softmax over the pairs, value encoding through one
+            # histogram per (atom, head); psi is never formed
+            dist_max = P.value_pe_dist_max if P.value_pe_dist_max >= 0 else -P.value_pe_dist_max * P.scale_real
+            rvlen = cutoff = None
+            if P.adaptive_cutoff_sigma != 0:
+                rvlen = rvecs if rvecs.dim() == 2 else torch.norm(rvecs, 2, dim=-1)
+                cutoff = (P.adaptive_cutoff_sigma if P.adaptive_cutoff_sigma < 0
+                          else P.scale_real * P.gauss_lb_real ** (-0.5) * P.adaptive_cutoff_sigma)
+            qs = q if q_is_scaled else q / math.sqrt(q.shape[-1])
+            use_angle = self.proj_angle1 is not None and P.value_pe_angle_real > 0
+            out, frames = cuda_funcs.PeriodicAttentionCoreHIP.apply(
+                qs, k, v, a, points, tvecs, batch_q, edges, P.value_pe_dist_real, dist_max, P.value_pe_dist_wscale,
+                self.pe_dist_proj, self.proj_angle1 if use_angle else None, self.proj_angle2 if use_angle else None,
+                self.proj_angle3 if use_angle else None, P.value_pe_angle_real, P.value_pe_angle_wscale, P.cos_abs,
+                P.value_pe_dist_coef, P.value_pe_angle_coef, rvlen, cutoff, None)
+            if self.frame_sink is not None:
+                self.frame_sink.append((None, None, None) if frames is None else (frames[0], frames[1], frames[2]))
+            return out.reshape(q.shape[0], self.num_heads * v.shape[-1]), None
         z, psi = compute_real_domain_attn_frame_proj(
             q, k, v, batch_q, batch_kv, edges, points, dist2_min, tvecs, rvecs, self.pe_dist_proj,
             self.proj_angle1, self.proj_angle2, self.proj_angle3, a, self.params, this_epoch,

@@ -34,7 +34,9 @@ def build_library(verbose: bool = True) -> str:
     """Compile csrc/crystalframer_hip.hip -> libcrystalframer_hip.so (always recompiles)."""
     src = os.path.join(CSRC, "crystalframer_hip.hip")
     tmp = LIB_PATH + ".tmp"
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-o", tmp, src]
+    # CFH_EXTRA_HIPCC_FLAGS: extra flags for diagnostics builds (e.g. -DCFH_PHASE_TIMING)
+    extra = os.environ.get("CFH_EXTRA_HIPCC_FLAGS", "").split()
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra, "-o", tmp, src]
     if verbose:
         print("[crystalframer_amd] " + " ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

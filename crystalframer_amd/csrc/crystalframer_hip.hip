@@ -1059,7 +1059,7 @@ int check_core_params(const cfh_params* p) {
     if (p->dist_wscale != 1.0f) return fail(CFH_EINVAL, "fused core: only dist_wscale 1.0 is compiled");
     if (p->grad_coef_quirk) return fail(CFH_EINVAL, "fused core: grad_coef_quirk is not available (exact gradients only)");
     if (p->angle_bins > 0 && p->angle_wscale < 3.0f)
-        return fail(CFH_EINVAL, "fused core: angle_wscale %g < 3: the moment expansion of the angle basis (6 terms) "
+        return fail(CFH_EINVAL, "fused core: angle_wscale %g < 3: the moment expansion of the angle basis (5 terms) "
                     "is not accurate enough; use the two-step operators", (double)p->angle_wscale);
     return CFH_OK;
 }
@@ -1174,8 +1174,8 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     } while (0)
     CFH_CORE_DISPATCH(cfh::fused_core_fwd_kernel);
     if (rc) return rc;
-    hipLaunchKernelGGL(cfh::core_project_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads), dim3(cfh::WAVE), 0, st,
-                       hist, wcat, out, (int)N, p->num_heads, L.hw);
+    hipLaunchKernelGGL(cfh::core_project_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads),
+                       dim3(cfh::WAVE * cfh::PROJ_WAVES), 0, st, hist, wcat, out, (int)N, p->num_heads, L.hw);
     return finish_launch("fused_core_project");
 }
 
@@ -1219,8 +1219,8 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
     // Wcat, G = Wcat^T go per item, records, tables
     hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, W_dist, W_axis1, W_axis2,
                        W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat);
-    hipLaunchKernelGGL(cfh::core_gbuild_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads), dim3(cfh::WAVE), 0, st,
-                       gout, wcat, G, (int)N, p->num_heads, L.hw);
+    hipLaunchKernelGGL(cfh::core_gbuild_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads, L.hw / 64), dim3(cfh::WAVE), 0,
+                       st, gout, wcat, G, (int)N, p->num_heads, L.hw);
     {
         const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
                                                                                           : p->num_heads * cfh::NQUEUE);
@@ -1253,7 +1253,7 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         int cus = device_cus();
         if (cus <= 0) cus = 256;
         const int blocks_per_slice = (L.hw / 64) * p->num_heads;
-        int nslices = (cus * 4 + blocks_per_slice - 1) / blocks_per_slice;
+        int nslices = (cus * 4 + blocks_per_slice - 1) / blocks_per_slice;      // about one wavefront per SIMD
         if (nslices < 1) nslices = 1;
         int per_slice = (int)((N + nslices - 1) / nslices);
         per_slice = (per_slice + 15) & ~15;

@@ -22,8 +22,8 @@
 //     the bin m* nearest to x the value of every basis function is a short power series in the offset
 //     eps = 2 (u - m*) in [-1,1] (u = x in bin units):
 //         exp(-((m - u)/ws)^2 / 2) = sum_o eps^o D_o(m - m*),  D_o(d) = exp(-(d/ws)^2/2) He_o(d/ws) / (o! (2 ws)^o)
-//     (generating function of the Hermite polynomials; truncated after NORD = 6 terms the error is below 1e-7 of
-//     the peak).  A term therefore adds NORD moments w eps^o at ONE bin per axis instead of a 33-bin window, and
+//     (generating function of the Hermite polynomials; truncated after NORD = 5 terms the error is below 2e-6 of
+//     the peak, 6 terms: 1e-7).  A term therefore adds NORD moments w eps^o at ONE bin per axis instead of a 33-bin window, and
 //     the constant matrices D_o are folded into the projection weights (core_wcat_kernel).  This is the FULL
 //     basis (no +-4 sigma truncation), i.e. the pure-PyTorch formulation of the reference
 //     (models/indexed_lattice_multi_head_attention.py:580-588) rather than the windowed one of its CUDA kernels.
@@ -41,14 +41,30 @@ constexpr int FC_TCAP = 128;                    // translations per table chunk 
 constexpr int FC_GROUP = 8;                     // pairs per group: one per 8-lane row
 constexpr int FC_LISTCAP = FC_GROUP * FC_TCAP;  // a group's survivors always fit: no overflow handling
 constexpr int FC_SHIFT = 7;                     // list entry = pair-in-group << 7 | table index
-constexpr int NORD = 6;                         // moments per axis
+#ifndef CFH_NORD
+#define CFH_NORD 5
+#endif
+constexpr int NORD = CFH_NORD;                  // moments per axis
+constexpr int FC_LOGCAP = 256;                  // logits of a row kept in LDS until the row is complete
 constexpr int HW_DIST = NBINS;
-constexpr int HW_ANG = NBINS * (1 + 3 * NORD);  // 1216 words per (atom, head) with the angle encoding
+constexpr int HW_ANG = NBINS * (1 + 3 * NORD);  // 1024 words per (atom, head) with the angle encoding
 constexpr int REC_J0 = 30;                      // item record: first neighbour atom (pairs of an atom are j0, j0+1, ...)
 constexpr int REC_CRYSTAL = 31;                 // item record: crystal of the atom
 static_assert(FC_TCAP == (1 << FC_SHIFT) && (FC_GROUP << FC_SHIFT) <= 65536, "list entry is 16 bits");
 
 typedef float v4f_c __attribute__((ext_vector_type(4)));
+
+// Optional phase timing (compile with -DCFH_PHASE_TIMING; diagnostics builds only): cycles per phase of the forward
+// kernel, summed over the wavefronts, in the statistics slots 16..23.
+#ifdef CFH_PHASE_TIMING
+#define CFH_PH_DECL unsigned long long ph_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long ph_last = __builtin_amdgcn_s_memtime(); int ph_cur = 0;
+#define CFH_PH(n) do { const unsigned long long ph_t = __builtin_amdgcn_s_memtime(); ph_acc[ph_cur] += ph_t - ph_last; ph_last = ph_t; ph_cur = (n); } while (0)
+#define CFH_PH_FLUSH(stats) do { CFH_PH(0); if ((stats) && threadIdx.x == 0) for (int u = 0; u < 8; u++) atomicAdd((stats) + 16 + u, ph_acc[u]); } while (0)
+#else
+#define CFH_PH_DECL
+#define CFH_PH(n) do { } while (0)
+#define CFH_PH_FLUSH(stats) do { } while (0)
+#endif
 
 struct CoreArgs {
     KernelArgs K;                 // geometry, work queues, item records, basis constants
@@ -232,6 +248,54 @@ __device__ __forceinline__ void core_load_table(const CoreArgs& C, const CoreIte
     }
 }
 
+// Operands of an item that do not depend on the item before it, fetched a whole item ahead: the two table entries
+// of this lane (sorted table of the item's crystal), the lane's two query channels, and the operands of the pair
+// of the first group that this lane's row serves.
+struct CorePrefetch {
+    float4 t0, t1;
+    float2 q2;
+    float rx, ry, rz;
+    float2 k2, v2;
+};
+__device__ __forceinline__ CorePrefetch core_prefetch(const CoreArgs& C, uint32_t rec, int it, int h, int lane) {
+    CorePrefetch pf;
+    pf.t0 = pf.t1 = make_float4(0.f, 0.f, 0.f, 0.f);
+    pf.q2 = pf.k2 = pf.v2 = make_float2(0.f, 0.f);
+    pf.rx = pf.ry = pf.rz = 0.f;
+    if (it < 0) return pf;
+    const KernelArgs& P = C.K;
+    const int H = P.H;
+    const int i = __builtin_amdgcn_readlane((int)rec, REC_ATOM);
+    const int e0 = __builtin_amdgcn_readlane((int)rec, REC_E0);
+    const int npairs = __builtin_amdgcn_readlane((int)rec, REC_NPAIRS);
+    const int j0 = __builtin_amdgcn_readlane((int)rec, REC_J0);
+    const int crystal = __builtin_amdgcn_readlane((int)rec, REC_CRYSTAL);
+    const int pr = lane >> 3, sub = lane & 7;
+    if (C.sorted_tab) {
+        const float4* src = C.sorted_tab + (size_t)crystal * FC_TCAP;
+        pf.t0 = src[lane];
+        pf.t1 = src[lane + WAVE];
+    }
+    pf.q2 = *reinterpret_cast<const float2*>(C.qs + ((size_t)i * H + h) * DH + 2 * sub);
+    if (pr < npairs) {
+        const size_t e = (size_t)(e0 + pr);
+        const size_t jh = ((size_t)(j0 + pr) * H + h) * DH + 2 * sub;
+        pf.rx = P.rpos[e * 3 + 0]; pf.ry = P.rpos[e * 3 + 1]; pf.rz = P.rpos[e * 3 + 2];
+        pf.k2 = *reinterpret_cast<const float2*>(C.k + jh);
+        pf.v2 = *reinterpret_cast<const float2*>(C.v + jh);
+    }
+    return pf;
+}
+// the item's table from what was prefetched (sorted) or built in place (one chunk)
+__device__ __forceinline__ void core_store_table(const CoreItem& ci, const CorePrefetch& pf, float4* tab, int lane) {
+    if (ci.sorted) {
+        tab[lane] = pf.t0;
+        tab[lane + WAVE] = pf.t1;
+    } else if (ci.nchunks == 1) {
+        build_shift_table(tab, 0, ci.item.bx.T, ci.item.bx, ci.item.L, lane);
+    }
+}
+
 // =================================================================================================================
 // forward
 // =================================================================================================================
@@ -243,6 +307,7 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
     __shared__ int32_t hist[HWK];
     __shared__ float4 pairA[FC_GROUP];      // rx, ry, rz, d2min
     __shared__ float pairC[FC_GROUP];       // exp(logit - running max) / S in fixed-point units
+    __shared__ float logit_s[FC_LOGCAP];    // logits of the row (rows of more pairs park them in the probability array)
 
     const KernelArgs& P = C.K;
     const int lane = threadIdx.x;
@@ -258,13 +323,28 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
     wave_sync();
 
     unsigned long long st_eval = 0, st_raw = 0, st_pairs = 0, st_seen = 0;
+    CFH_PH_DECL
     int queue = first_queue(H);
     int it_cur = queue_pop(P, h, queue);
     int it_next = it_cur >= 0 ? queue_pop(P, h, queue) : -1;
     uint32_t rec_cur = load_record(P, it_cur, h);
+    CorePrefetch pf = core_prefetch(C, rec_cur, it_cur, h, lane);
     while (it_cur >= 0) {
-        const int ticket = queue_ticket(P, h, queue);
+        CFH_PH(6);
         const uint32_t rec_next = load_record(P, it_next, h);
+        int ticket = 0;
+        CorePrefetch pf_next = pf;
+        bool drawn = false;
+        // The ticket of the item after next is drawn, and the operands of the next item are requested, after the
+        // sweeps of the first group: the function that draws the ticket starts by waiting for everything this
+        // wavefront has in flight, and by then the stores of the previous item have been acknowledged, while the
+        // rest of this item is enough for the requested operands to land.
+        auto draw_and_prefetch = [&]() {
+            ticket = queue_ticket(P, h, queue);
+            pf_next = core_prefetch(C, rec_next, it_next, h, lane);
+            drawn = true;
+        };
+        CFH_PH(0);
         const CoreItem ci = core_unpack(C, rec_cur, true);
         const int i = ci.item.i;
         const float a = ci.item.a;
@@ -282,10 +362,10 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
         }
         const int e0 = ci.item.e0, npairs = ci.item.npairs;
         wave_sync();                          // the previous item's readers of the table are done
-        core_load_table(C, ci, tab, lane);
+        core_store_table(ci, pf, tab, lane);
         wave_sync();
         const size_t ih = (size_t)i * H + h;
-        const float2 q2 = *reinterpret_cast<const float2*>(C.qs + ih * DH + 2 * sub);
+        const float2 q2 = pf.q2;
         const float fixs = 1073741824.0f / (float)max(npairs, 1);      // 2^30 / npairs: sums of weights <= 1 each fit
         const float cutS = (C.skip_log2 > 0.0f && a2 < 0.0f) ? C.skip_log2 / (-a2) : INF;
         float m_run = -INF;                   // running maximum of the logits (wave-uniform)
@@ -293,9 +373,9 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
         float2 accv = make_float2(0.f, 0.f);  // sum_j exp(logit_j - m_run) v_j, channels 2 sub, 2 sub + 1
         unsigned long long n_eval = 0, n_seen = 0;      // wave-uniform counts
 
-        // operands of the pair served by this row, fetched one group ahead
-        float nrx = 0.f, nry = 0.f, nrz = 0.f;
-        float2 nk2 = make_float2(0.f, 0.f), nv2 = nk2;
+        // operands of the pair served by this row, fetched one group ahead (the first group: with the item)
+        float nrx = pf.rx, nry = pf.ry, nrz = pf.rz;
+        float2 nk2 = pf.k2, nv2 = pf.v2;
         auto fetch = [&](int g0) {
             const int el = g0 + pr;
             if (el < npairs) {
@@ -306,7 +386,6 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
                 nv2 = *reinterpret_cast<const float2*>(C.v + jh);
             }
         };
-        fetch(0);
 
         // one sweep of this row's pair over the table(s): fn(inside, table index, d^2)
         auto sweep = [&](bool active, float rx, float ry, float rz, float reach, auto&& fn) {
@@ -318,14 +397,16 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
                     build_shift_table(tab, t0c, cnt, bx, L, lane);
                     wave_sync();
                 }
+                float4 v = tab[min(sub, cnt - 1)];
                 for (int t0 = 0; t0 < cnt; t0 += FC_GROUP) {
                     const int t = t0 + sub;
-                    const float4 v = tab[min(t, cnt - 1)];
+                    const float4 vn = tab[min(t + FC_GROUP, cnt - 1)];      // the next step's entry, in flight meanwhile
                     const bool in = active && t < cnt && v.w <= reach;
                     const uint64_t inm = __ballot(in);
                     if (sorted && inm == 0) break;               // every row is past its reach (lengths ascend)
                     const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
                     fn(in, t, fmaf(dx, dx, fmaf(dy, dy, dz * dz)), __popcll(inm));
+                    v = vn;
                 }
             }
         };
@@ -349,7 +430,11 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
                         start = max(0, min(start, NBINS - WL));
                         const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
                         const WindowSeed s = window_seed(beta_c, bc.len_step, w);
+#ifndef CFH_EXP_NOCONFLICT
                         window_scatter_rn<WL>(hist + start, s, bc.len_cc);
+#else
+                        window_scatter_rn<WL>(hist + (start & 0) + lane, s, bc.len_cc);
+#endif
                     }
                     if (HAS_ANG) {
                         if (d2 > 1e-5f) {       // the self image contributes to S and the distance encoding only
@@ -361,7 +446,11 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
                                 const float uu = (cs - bc.ang_mu0) * bc.ang_inv_interval;      // in bin units
                                 const float mf = clampf(__builtin_rintf(uu), 0.0f, (float)(NBINS - 1));
                                 const float eps = 2.0f * (uu - mf);
+#ifndef CFH_EXP_NOCONFLICT
                                 int32_t* hb = hist + HW_DIST + ax * NORD * NBINS + (int)mf;
+#else
+                                int32_t* hb = hist + HW_DIST + ax * NORD * NBINS + ((int)mf & 0) + lane;
+#endif
                                 float val = w;
                                 atomicAdd(hb, rint_i(val));
 #pragma unroll
@@ -382,12 +471,14 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
             const float rn = hw_sqrt(fmaf(rx, rx, fmaf(ry, ry, rz * rz)));
 
             // ---- pass A: nearest image
+            CFH_PH(1);
             float d2min = 3.0e38f;
             sweep(active, rx, ry, rz, sorted ? fmaf(2.0002f, rn, 1e-4f) : INF,
                   [&](bool in, int, float d2, int cnt_in) { d2min = in ? fminf(d2min, d2) : d2min; n_seen += cnt_in; });
             d2min = half_min(d2min);
 
             // ---- pass B: weights, normaliser and (one-chunk tables) the survivors
+            CFH_PH(2);
             const float reachB = sorted ? fmaf(1.0001f, rn + hw_sqrt(d2min + cutS), 1e-4f) : INF;
             float Sb = 0.0f;
             int nlist = 0;
@@ -403,8 +494,10 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
                 }
             });
             const float S = half_sum(Sb);
+            if (g0 == 0) { CFH_PH(6); draw_and_prefetch(); }
 
             // ---- logits, running softmax
+            CFH_PH(3);
             const float qk = half_sum(fmaf(q2.x, k2.x, q2.y * k2.y));
             const float z = fmaf(hw_log2(S), LN2, a * d2min);
             const float logit = active ? qk + z : -INF;
@@ -423,14 +516,18 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
             if (sub == 0 && active) {
                 const size_t eh = (size_t)(e0 + g0 + pr) * H + h;
                 pairA[pr] = make_float4(rx, ry, rz, d2min);
-                pairC[pr] = ew / S * fixs;
+                pairC[pr] = ew * hw_rcp(S) * fixs;
+#ifndef CFH_EXP_NOZ
                 C.z[eh] = z;
-                C.prob[eh] = logit;              // the logit for now; normalised when the row is complete
+#endif
+                if (npairs <= FC_LOGCAP) logit_s[g0 + pr] = logit;
+                else C.prob[eh] = logit;         // the logit for now; normalised when the row is complete
                 Dl += ew;
             }
             wave_sync();
 
             // ---- heavy pass
+            CFH_PH(4);
             if (nchunks == 1) heavy(nlist);
             else {
                 for (int ch = 0; ch < nchunks; ch++) {
@@ -455,29 +552,53 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
                 }
             }
             wave_sync();                      // list, pair data and (several chunks) the table may be rewritten
+            CFH_PH(3);
         }
 
         // ---- the row is complete: normalise and write
+        CFH_PH(5);
+        if (!drawn) draw_and_prefetch();      // (an atom without pairs)
+        // what was requested for the next item is taken over before this item's stores are issued: a wait for it
+        // afterwards would also wait for those stores
+        pf = pf_next;
+        asm volatile("" :: "v"(pf.t0.x), "v"(pf.t1.x), "v"(pf.q2.x), "v"(pf.rx), "v"(pf.k2.x), "v"(pf.v2.x));
+        CFH_PH(7);
         const float D = uniform_f(wave_sum(Dl));
-        const float inv = D > 0.0f ? 1.0f / D : 0.0f;
+        const float inv = D > 0.0f ? hw_rcp(D) : 0.0f;
         {
             const float ox = rows8_sum(accv.x) * inv, oy = rows8_sum(accv.y) * inv;
             if (lane < FC_GROUP) *reinterpret_cast<float2*>(C.out + ih * DH + 2 * sub) = make_float2(ox, oy);
         }
         {
-            const float sc = inv / fixs;
-            float* dst = C.hist + ih * HWK;
-            for (int u = lane; u < HWK; u += WAVE) {
-                dst[u] = (float)hist[u] * sc;
-                hist[u] = 0;
+            // all reads first (one LDS round trip instead of one per word), then clear and store
+            constexpr int NW = HWK / WAVE;
+            const float sc = inv * (float)max(npairs, 1) * (1.0f / 1073741824.0f);
+            float* dst = C.hist + ih * HWK + lane;
+            int32_t hv[NW];
+#pragma unroll
+            for (int u = 0; u < NW; u++) hv[u] = hist[lane + WAVE * u];
+#pragma unroll
+            for (int u = 0; u < NW; u++) {
+                hist[lane + WAVE * u] = 0;
+#ifndef CFH_EXP_NOHIST
+                dst[WAVE * u] = (float)hv[u] * sc;
+#else
+                if (hv[u] == 0x7fffffff) dst[WAVE * u] = (float)hv[u] * sc;
+#endif
             }
         }
-        for (int g0 = 0; g0 < npairs; g0 += FC_GROUP) {          // logits -> probabilities (same lane wrote them)
-            if (sub == 0 && g0 + pr < npairs) {
-                const size_t eh = (size_t)(e0 + g0 + pr) * H + h;
-                C.prob[eh] = hw_exp2((C.prob[eh] - m_run) * LOG2E) * inv;
+        if (npairs <= FC_LOGCAP) {                               // logits -> probabilities
+            for (int el = lane; el < npairs; el += WAVE)
+                C.prob[(size_t)(e0 + el) * H + h] = hw_exp2((logit_s[el] - m_run) * LOG2E) * inv;
+        } else {
+            for (int g0 = 0; g0 < npairs; g0 += FC_GROUP) {      // each was written by the lane that now reads it
+                if (sub == 0 && g0 + pr < npairs) {
+                    const size_t eh = (size_t)(e0 + g0 + pr) * H + h;
+                    C.prob[eh] = hw_exp2((C.prob[eh] - m_run) * LOG2E) * inv;
+                }
             }
         }
+        CFH_PH(6);
         st_eval += n_eval;
         st_seen += n_seen;
         st_raw += (unsigned long long)bx.T * (unsigned long long)npairs;
@@ -486,6 +607,7 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
         rec_cur = rec_next;
         it_next = it_cur >= 0 ? queue_redeem(P, h, queue, ticket) : -1;
     }
+    CFH_PH_FLUSH(P.stats);
     if (P.stats && lane == 0) {         // one set of atomics per wavefront
         atomicAdd(P.stats + STAT_FWD_EVAL, st_eval);
         atomicAdd(P.stats + STAT_FWD_RAW, st_raw);
@@ -494,19 +616,25 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
     }
 }
 
-// out (N,H,16) += Wcat_h (16, hw) . hist (N,H,hw): one wavefront per (16 atoms, head); MFMA 16x16x4, a lane owns 16
-// consecutive words of each 64-word step of the reduction index (64-byte loads of its row).  grid (ceil(N/16), H).
-__global__ __launch_bounds__(WAVE) void core_project_kernel(const float* __restrict__ hist, const float* __restrict__ wcat,
-                                                            float* __restrict__ out, int N, int H, int hw) {
-    const int lane = threadIdx.x, col = lane & 15, kk = lane >> 4;
+// out (N,H,16) += Wcat_h (16, hw) . hist (N,H,hw): one workgroup of PROJ_WAVES wavefronts per (16 atoms, head); each
+// wavefront takes a slice of the reduction index through MFMA 16x16x4 (a lane owns 16 consecutive words of each
+// 64-word step: 64-byte loads of its row), the slices meet in LDS and are added in a fixed order by the first
+// wavefront (no atomics: the result does not depend on timing).  grid (ceil(N/16), H), block 64 * PROJ_WAVES.
+constexpr int PROJ_WAVES = 4;
+__global__ __launch_bounds__(WAVE * PROJ_WAVES) void core_project_kernel(const float* __restrict__ hist,
+                                                                         const float* __restrict__ wcat,
+                                                                         float* __restrict__ out, int N, int H, int hw) {
+    __shared__ float part[PROJ_WAVES][4][WAVE];
+    const int lane = threadIdx.x & (WAVE - 1), wv = threadIdx.x >> 6, col = lane & 15, kk = lane >> 4;
     const int h = blockIdx.y, i0 = blockIdx.x * 16;
     const int row = min(i0 + col, N - 1);
     const float4* ap = reinterpret_cast<const float4*>(hist + ((size_t)row * H + h) * hw) + 4 * kk;
     const float4* bp = reinterpret_cast<const float4*>(wcat + ((size_t)h * DH + col) * hw) + 4 * kk;
     v4f_c acc = {0.f, 0.f, 0.f, 0.f};
-    const int steps = hw / 64;
+    const int steps = hw / 64, per = (steps + PROJ_WAVES - 1) / PROJ_WAVES;
+    const int s_begin = wv * per, s_end = min(steps, s_begin + per);
 #pragma unroll 2
-    for (int s = 0; s < steps; s++) {
+    for (int s = s_begin; s < s_end; s++) {
         float4 a4[4], b4[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) { a4[u] = ap[16 * s + u]; b4[u] = bp[16 * s + u]; }
@@ -518,17 +646,24 @@ __global__ __launch_bounds__(WAVE) void core_project_kernel(const float* __restr
             acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u].w, b4[u].w, acc, 0, 0, 0);
         }
     }
+#pragma unroll
+    for (int r = 0; r < 4; r++) part[wv][r][lane] = acc[r];
+    __syncthreads();
+    if (wv != 0) return;
     // component r of lane (kk, col): atom 4 kk + r of the tile, channel col
 #pragma unroll
     for (int r = 0; r < 4; r++) {
+        float sum = part[0][r][lane];
+#pragma unroll
+        for (int w = 1; w < PROJ_WAVES; w++) sum += part[w][r][lane];
         const int it = i0 + 4 * kk + r;
-        if (it < N) out[((size_t)it * H + h) * DH + col] += acc[r];
+        if (it < N) out[((size_t)it * H + h) * DH + col] += sum;
     }
 }
 
-// G (N,H,hw) = go (N,H,16) . Wcat_h (16, hw): wavefront per (16 atoms, head); per 64-word block four MFMA tiles whose
+// G (N,H,hw) = go (N,H,16) . Wcat_h (16, hw): wavefront per (16 atoms, head, 64-word block); four MFMA tiles whose
 // columns are interleaved (tile t, column c <-> word 4 c + t) so that a lane stores 16 consecutive bytes.
-// grid (ceil(N/16), H).
+// grid (ceil(N/16), H, hw/64).
 __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restrict__ go, const float* __restrict__ wcat,
                                                            float* __restrict__ G, int N, int H, int hw) {
     const int lane = threadIdx.x, col = lane & 15, kk = lane >> 4;
@@ -536,7 +671,8 @@ __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restri
     const int row = min(i0 + col, N - 1);
     const float4 a4 = reinterpret_cast<const float4*>(go + ((size_t)row * H + h) * DH)[kk];      // channels 4 kk ..
     const float A[4] = {a4.x, a4.y, a4.z, a4.w};
-    for (int w0 = 0; w0 < hw; w0 += 64) {
+    {
+        const int w0 = blockIdx.z * 64;
         float4 b4[4];
 #pragma unroll
         for (int j = 0; j < 4; j++)

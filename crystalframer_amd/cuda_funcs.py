@@ -539,7 +539,7 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
     divided by sqrt(Dh).  Same result as RealEncodingWithMaxFramesFuncHIP followed by FusedDotProductAttentionCUDA
     (the reference's sequence, models/indexed_lattice_multi_head_attention_cuda.py:589-734 and :144-185), computed
     with one histogram per (atom, head) instead of one per (pair, head): psi (E,H,Dh) is never formed.  The angle
-    encoding uses the full Gaussian basis (no +-4 sigma window; a 6-term series around the nearest bin), the
+    encoding uses the full Gaussian basis (no +-4 sigma window; a 5-term series around the nearest bin), the
     distance encoding the window of ``KernelManager.WINDOW_MODE``.  No counterpart class in the reference."""
 
     @staticmethod

@@ -288,8 +288,8 @@ int cfh_fused_dpa_backward(const float* q, const float* k, const float* v, const
  * atom are scattered, weighted by P_ij p_n, into ONE histogram per (atom, head), which is projected once.
  * psi (E,H,Dh) and the per-pair histograms are never formed.  The distance basis keeps the truncated window of
  * window_mode; the angle basis is the FULL Gaussian basis (no truncation: the pure-PyTorch formulation,
- * models/indexed_lattice_multi_head_attention.py:580-588), evaluated as a 6-term series around the nearest bin
- * (error < 1e-7 of a basis function's peak for angle_wscale 4; angle_wscale < 3 returns CFH_EINVAL).
+ * models/indexed_lattice_multi_head_attention.py:580-588), evaluated as a 5-term series around the nearest bin
+ * (error < 2e-6 of a basis function's peak for angle_wscale 4; angle_wscale < 3 returns CFH_EINVAL).
  * Needs dist_bins = 64, dist_wscale = 1, angle_bins 0 or 64, and the pairs as the complete n x n block of every
  * crystal (cfh_pair_layout_check).  qs = query / sqrt(Dh).
  * Results kept for the backward: z (E,H), prob (E,H) = P, hist (N,H,words) the normalised histograms

@@ -127,7 +127,7 @@ def test_c2_backward_at_batch_256_against_oracle_on_first_crystals(second_stream
 
 
 # ------------------------------------------------------------------------------------------------ C3
-def test_c3_four_layer_model_at_batch_256_against_cpu_model_on_first_crystals():
+def test_c3_four_layer_model_at_batch_256_against_cpu_model_on_first_crystals(core_mode):
     """The workload bench.py times.  Crystals do not interact once the normalisation of alpha is stored, so
     the first 12 rows of the batch-256 output, and the parameter gradients of a loss on those rows, must be
     what the float64 CPU model gives for those 12 crystals alone (with the frames the GPU chose, so that
@@ -158,7 +158,7 @@ def test_c3_four_layer_model_at_batch_256_against_cpu_model_on_first_crystals():
     frames = [[f.detach().cpu().double()[:n_at] for f in layer.self_attn.frame_sink[0]]
               for layer in model.encoder.layers]
     sub = synthetic.CrystalBatch(cb.x[:n_at], cb.pos[:n_at], cb.batch[:n_at], cb.trans_vec[:nb], cb.sizes[:nb])
-    ref = cpu_model.model_forward(leaves, sub, mp, dtype=torch.float64, frames_per_layer=frames)
+    ref = cpu_model.model_forward(leaves, sub, mp, dtype=torch.float64, frames_per_layer=frames, windows=core_mode)
     torch.nn.functional.mse_loss(ref, target.cpu().double()).backward()
     assert Hh.rel_err(out[:nb], ref) < 1e-4
     checked = 0

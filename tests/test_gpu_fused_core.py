@@ -1,7 +1,7 @@
 """The fused attention core (cfh_fused_core_forward / backward through PeriodicAttentionCoreHIP) against the
 float64 oracle composition  TO.framed_pe -> TO.softmax_attention  (autograd for every gradient), and against the
 two-step operators of the library.  The fused core sums the same translation sets and uses the same distance
-windows as the two-step path; its angle encoding is the FULL Gaussian basis (a 6-term series around the nearest
+windows as the two-step path; its angle encoding is the FULL Gaussian basis (a 5-term series around the nearest
 bin), so the oracle runs with windows = (9, None): 9-bin distance window, untruncated angle basis.
 
 Tolerances (relative to the largest magnitude of the tensor): 2e-5 forward, 1e-4 gradients."""

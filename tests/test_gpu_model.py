@@ -9,7 +9,7 @@ from oracle import cpu_model
 pytestmark = pytest.mark.gpu
 
 
-def _run(mp, cb, seed=0, passes=1):
+def _run(mp, cb, seed=0, passes=1, windows="reference"):
     import crystalframer_amd as cf
     from crystalframer_amd import latticeformer
     KM = cf.KernelManager
@@ -35,19 +35,19 @@ def _run(mp, cb, seed=0, passes=1):
     frames = None
     if mp.value_pe_angle_real > 0:
         frames = [[f.detach().cpu().double() for f in layer.self_attn.frame_sink[0]] for layer in model.encoder.layers]
-    ref = cpu_model.model_forward(leaves, cb, mp, dtype=torch.float64, frames_per_layer=frames)
+    ref = cpu_model.model_forward(leaves, cb, mp, dtype=torch.float64, frames_per_layer=frames, windows=windows)
     ref_loss = torch.nn.functional.mse_loss(ref, target.cpu().double())
     ref_loss.backward()
     return model, out, ref, leaves
 
 
 @pytest.mark.parametrize("angle_bins,passes", [(64, 1), (0, 1), (64, 2)])
-def test_model_forward_backward_matches_cpu_oracle(angle_bins, passes):
+def test_model_forward_backward_matches_cpu_oracle(angle_bins, passes, core_mode):
     from crystalframer_amd import params, synthetic
     mp = params.ModelParams(num_layers=2, value_pe_angle_real=angle_bins, symm_break_noise=0.0)
     cb = synthetic.make_batch(8, atoms="uniform", atoms_lo=1, atoms_hi=6, len_lo=3.0, len_hi=9.0,
                               ang_lo=65.0, ang_hi=115.0, seed=11)
-    model, out, ref, leaves = _run(mp, cb, passes=passes)
+    model, out, ref, leaves = _run(mp, cb, passes=passes, windows=core_mode)
     assert Hh.rel_err(out, ref) < 1e-4
     checked = 0
     for name, p in model.named_parameters():
@@ -63,7 +63,7 @@ def test_model_forward_backward_matches_cpu_oracle(angle_bins, passes):
         assert float(layer.self_attn.gauss_scale[0]) > 0
 
 
-def test_model_frames_agree_with_oracle_frames():
+def test_model_frames_agree_with_oracle_frames(core_mode):
     """The frames the model used are the oracle's wherever the winner is clear."""
     from crystalframer_amd import params, synthetic
     from oracle import torch_oracle as TO
@@ -71,7 +71,7 @@ def test_model_frames_agree_with_oracle_frames():
     mp = params.ModelParams(num_layers=1, symm_break_noise=0.0)
     cb = synthetic.make_batch(8, atoms="uniform", atoms_lo=2, atoms_hi=6, len_lo=3.0, len_hi=9.0,
                               ang_lo=65.0, ang_hi=115.0, seed=13)
-    model, out, ref, leaves = _run(mp, cb)
+    model, out, ref, leaves = _run(mp, cb, windows=core_mode)
     sd = {k: v.detach() for k, v in leaves.items()}
     lat = params.LatticeformerParams().parseFromArgs(mp).getLayerParameters(0)
     pos, tv = cb.pos.double(), cb.trans_vec.double()
