@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
@@ -57,6 +57,13 @@ class CfhAttentionInputsGrad(ctypes.Structure):
                 ("gqkv", ctypes.c_void_p), ("gw_partial", ctypes.c_void_p),
                 ("c1", ctypes.c_float), ("lb", ctypes.c_float), ("c2", ctypes.c_float), ("q_scale", ctypes.c_float),
                 ("H", ctypes.c_int32), ("reserved0", ctypes.c_int32)]
+
+
+class CfhCoreCache(ctypes.Structure):
+    """Mirror of ``cfh_core_cache`` in include/crystalframer_hip.h."""
+    _fields_ = [("shift_table", ctypes.c_void_p), ("wcat", ctypes.c_void_p), ("records", ctypes.c_void_p),
+                ("shift_table_ready", ctypes.c_int32), ("wcat_ready", ctypes.c_int32),
+                ("records_ready", ctypes.c_int32), ("reserved0", ctypes.c_int32)]
 
 
 class CfhLinearGradJob(ctypes.Structure):
@@ -154,10 +161,12 @@ def load():
         lib.cfh_fused_core_hist_words.restype = ctypes.c_int32
         lib.cfh_fused_core_hist_words.argtypes = [pp]
         lib.cfh_fused_core_forward.restype = ctypes.c_int
+        pc = ctypes.POINTER(CfhCoreCache)
         lib.cfh_fused_core_forward.argtypes = ([pp] + [_P] * 15 + [_I64] * 3 + [_P, ctypes.c_int32] + [_P] * 4
-                                               + [_P, ctypes.c_size_t, _P])
+                                               + [pc, _P, ctypes.c_size_t, _P])
         lib.cfh_fused_core_backward.restype = ctypes.c_int
-        lib.cfh_fused_core_backward.argtypes = ([pp] + [_P] * 21 + [_I64] * 3 + [_P] * 9 + [_P, ctypes.c_size_t, _P])
+        lib.cfh_fused_core_backward.argtypes = ([pp] + [_P] * 21 + [_I64] * 3 + [_P] * 9
+                                                + [pc, _P, ctypes.c_size_t, _P])
         lib.cfh_timing_enable.restype = ctypes.c_int
         lib.cfh_timing_enable.argtypes = [ctypes.c_int]
         lib.cfh_timing_read.restype = ctypes.c_int

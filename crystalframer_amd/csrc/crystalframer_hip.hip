@@ -1063,16 +1063,37 @@ int check_core_params(const cfh_params* p) {
                     "is not accurate enough; use the two-step operators", (double)p->angle_wscale);
     return CFH_OK;
 }
-// the kernels' launch-wide arguments that both directions share
-void fill_core(cfh::CoreArgs& C, const cfh_params* p, const CoreLayout& L, const float* qs, const float* k, const float* v,
-               bool has_rvlen, void* workspace) {
+// the kernels' launch-wide arguments that both directions share; buffers of the caller's cache replace the
+// workspace regions of the same content
+struct CoreBuffers {
+    float4* table;       // sorted shifts (null: not used by this launch)
+    bool table_ready;
+    float* wcat;
+    bool wcat_ready;
+    bool records_ready;
+};
+CoreBuffers fill_core(cfh::CoreArgs& C, const cfh_params* p, const CoreLayout& L, const float* qs, const float* k,
+                      const float* v, bool has_rvlen, const cfh_core_cache* cache, void* workspace) {
+    char* ws = reinterpret_cast<char*>(workspace);
     C.qs = qs; C.k = k; C.v = v;
     const bool adaptive = has_rvlen && p->cutoff_radius != 0.0f;
     const int R0 = adaptive ? p->minimum_range : p->lattice_range;
     const bool tables = p->prune_log2 > 0.0f && R0 >= 1 && (2 * R0 + 1) * (2 * R0 + 1) * (2 * R0 + 1) <= cfh::FC_TCAP;
-    C.sorted_tab = tables ? reinterpret_cast<const float4*>(reinterpret_cast<char*>(workspace) + L.sorted) : nullptr;
+    CoreBuffers b;
+    b.table = nullptr; b.table_ready = false;
+    if (tables) {
+        const bool own = cache && cache->shift_table;
+        b.table = own ? reinterpret_cast<float4*>(cache->shift_table) : reinterpret_cast<float4*>(ws + L.sorted);
+        b.table_ready = own && cache->shift_table_ready != 0;
+    }
+    b.wcat = (cache && cache->wcat) ? cache->wcat : reinterpret_cast<float*>(ws + L.wcat);
+    b.wcat_ready = cache && cache->wcat && cache->wcat_ready != 0;
+    b.records_ready = cache && cache->records && cache->records_ready != 0;
+    if (cache && cache->records) C.K.items = cache->records;
+    C.sorted_tab = b.table;
     C.table_R = tables ? R0 : 0;
     C.skip_log2 = p->prune_log2 > 0.0f ? (p->prune_log2 + 8.0f > 32.0f ? p->prune_log2 + 8.0f : 32.0f) : 0.0f;
+    return b;
 }
 template <typename Kern>
 int launch_core(Kern kern, const cfh::CoreArgs& C, int cap, hipStream_t st, const char* what) {
@@ -1116,7 +1137,8 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
                            const int64_t* edges, const int64_t* e_start, const int32_t* order, const float* W_dist,
                            const float* W_axis1, const float* W_axis2, const float* W_axis3, int64_t N, int64_t E,
                            int64_t B, float* frames, int32_t search_frames, float* z, float* prob, float* hist,
-                           float* out, void* workspace, size_t workspace_bytes, void* stream) {
+                           float* out, const cfh_core_cache* cache, void* workspace, size_t workspace_bytes,
+                           void* stream) {
     int rc = check_core_params(p);
     if (rc) return rc;
     if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
@@ -1133,7 +1155,7 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     cfh::CoreArgs C;
     std::memset(&C, 0, sizeof(C));
     fill_common(C.K, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
-    fill_core(C, p, L, qs, k, v, rvlen != nullptr, workspace);
+    const CoreBuffers buf = fill_core(C, p, L, qs, k, v, rvlen != nullptr, cache, workspace);
     const bool search = has_ang && search_frames != 0;
     if (search) {
         // records with the query, frame search through the first set of queues; it leaves the frames in the records
@@ -1150,10 +1172,10 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
                                                                                           : p->num_heads * cfh::NQUEUE);
         hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, C.K, 0);
     }
-    if (C.sorted_tab)
+    if (buf.table && !buf.table_ready)
         hipLaunchKernelGGL(cfh::sorted_shifts_kernel, dim3((unsigned)B), dim3(cfh::FC_TCAP), 0, st, tvecs, C.table_R,
-                           reinterpret_cast<float4*>(ws + L.sorted));
-    float* wcat = reinterpret_cast<float*>(ws + L.wcat);
+                           buf.table);
+    float* wcat = buf.wcat;
     hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, W_dist, W_axis1, W_axis2,
                        W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat);
     C.out = out; C.prob = prob; C.z = z; C.hist = hist;
@@ -1185,8 +1207,8 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
                             const float* W_axis1, const float* W_axis2, const float* W_axis3, const float* frames,
                             const float* z, const float* prob, const float* hist, const float* out, const float* gout,
                             int64_t N, int64_t E, int64_t B, float* gq, float* gk, float* gv, float* ga, float* glogit,
-                            float* gW_dist, float* gW_axis1, float* gW_axis2, float* gW_axis3, void* workspace,
-                            size_t workspace_bytes, void* stream) {
+                            float* gW_dist, float* gW_axis1, float* gW_axis2, float* gW_axis3,
+                            const cfh_core_cache* cache, void* workspace, size_t workspace_bytes, void* stream) {
     int rc = check_core_params(p);
     if (rc) return rc;
     if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
@@ -1205,51 +1227,35 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
     const CoreLayout L = core_layout(p, N, B, true);
     if ((rc = check_workspace(workspace, workspace_bytes, L.total))) return rc;
     char* ws = reinterpret_cast<char*>(workspace);
-    float* wcat = reinterpret_cast<float*>(ws + L.wcat);
     float* gwcat = reinterpret_cast<float*>(ws + L.gwcat);
     float* G = reinterpret_cast<float*>(ws + L.G);
     cfh::CoreArgs C;
     std::memset(&C, 0, sizeof(C));
     fill_common(C.K, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
-    fill_core(C, p, L, qs, k, v, rvlen != nullptr, workspace);
+    const CoreBuffers buf = fill_core(C, p, L, qs, k, v, rvlen != nullptr, cache, workspace);
+    float* wcat = buf.wcat;
     C.K.frames = has_ang ? frames : nullptr;
     C.K.out_ga = ga;
     C.z = const_cast<float*>(z); C.prob = const_cast<float*>(prob);
     C.go = gout; C.outv = out; C.G = G; C.gq = gq; C.glogit = glogit;
-    // Wcat, G = Wcat^T go per item, records, tables
-    hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, W_dist, W_axis1, W_axis2,
-                       W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat);
-    hipLaunchKernelGGL(cfh::core_gbuild_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads, L.hw / 64), dim3(cfh::WAVE), 0,
-                       st, gout, wcat, G, (int)N, p->num_heads, L.hw);
-    {
-        const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
-                                                                                          : p->num_heads * cfh::NQUEUE);
-        hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, C.K, 0);
+
+    // ---- weight gradients: gwcat = sum_i go_i (x) hist_i, then back through the moment matrices.  They read
+    //      nothing that this call makes, so they go to the second stream, beside the kernels below.
+    const bool two = !(p->flags & CFH_FLAG_SINGLE_STREAM);
+    std::unique_lock<std::mutex> side_lock(g_side_mutex, std::defer_lock);
+    SideStream* side = nullptr;
+    hipStream_t st_w = st;
+    if (two) {
+        side_lock.lock();
+        side = side_stream();
+        if (!side) return fail(CFH_ELAUNCH, "second stream for the weight gradients could not be created");
+        if (hipEventRecord(side->fork, st) != hipSuccess || hipStreamWaitEvent(side->stream, side->fork, 0) != hipSuccess)
+            return fail(CFH_ELAUNCH, "fork to the second stream failed: %s", hipGetErrorString(hipGetLastError()));
+        st_w = side->stream;
     }
-    if (C.sorted_tab)
-        hipLaunchKernelGGL(cfh::sorted_shifts_kernel, dim3((unsigned)B), dim3(cfh::FC_TCAP), 0, st, tvecs, C.table_R,
-                           reinterpret_cast<float4*>(ws + L.sorted));
-    const int nw = p->num_heads * cfh::DH * L.hw;
-    hipLaunchKernelGGL(cfh::core_zero_kernel, dim3((nw + 255) / 256), dim3(256), 0, st, gwcat, nw);
-    const int cap = launch_waves(N, p->num_heads, CORE_WAVES_PER_SIMD);
-    const bool wide = p->window_mode == CFH_WINDOW_WIDE;
-    const char* what = "fused_core_backward";
-    CFH_CORE_DISPATCH(cfh::fused_core_bwd_kernel);
-#undef CFH_CORE_DISPATCH
-    if (rc) return rc;
-    // gk, gv: sums over the pairs that point at an atom
-    {
-        cfh::DpaArgs A;
-        std::memset(&A, 0, sizeof(A));
-        A.q = qs; A.k = k; A.v = v; A.edges = edges; A.e_start = e_start;
-        A.prob = const_cast<float*>(prob); A.go = gout; A.gk = gk; A.gv = gv; A.gaij = glogit;
-        A.N = (int32_t)N; A.H = p->num_heads; A.E = (int32_t)E;
-        const int64_t items = N * p->num_heads;
-        hipLaunchKernelGGL(cfh::dpa_bwd_col_kernel, dim3((unsigned)((items + cfh::DPA_WAVES - 1) / cfh::DPA_WAVES)),
-                           dim3(cfh::WAVE * cfh::DPA_WAVES), 0, st, A);
-    }
-    // weight gradients: gwcat = sum_i go_i (x) hist_i, then back through the moment matrices
-    {
+    auto weight_gradients = [&]() {
+        const int nw = p->num_heads * cfh::DH * L.hw;
+        hipLaunchKernelGGL(cfh::core_zero_kernel, dim3((nw + 255) / 256), dim3(256), 0, st_w, gwcat, nw);
         int cus = device_cus();
         if (cus <= 0) cus = 256;
         const int blocks_per_slice = (L.hw / 64) * p->num_heads;
@@ -1258,13 +1264,54 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         int per_slice = (int)((N + nslices - 1) / nslices);
         per_slice = (per_slice + 15) & ~15;
         nslices = (int)((N + per_slice - 1) / per_slice);
-        hipLaunchKernelGGL(cfh::core_gwcat_kernel, dim3(L.hw / 64, p->num_heads, nslices), dim3(cfh::WAVE), 0, st, gout, hist,
-                           gwcat, (int)N, p->num_heads, L.hw, per_slice);
-        hipLaunchKernelGGL(cfh::core_gw_finish_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, gwcat, L.hw,
-                           p->dist_coef, p->angle_coef, p->angle_wscale, gW_dist, gW_axis1,
-                           gW_axis2, gW_axis3);
+        hipLaunchKernelGGL(cfh::core_gwcat_kernel, dim3(L.hw / 64, p->num_heads, nslices), dim3(cfh::WAVE), 0, st_w, gout,
+                           hist, gwcat, (int)N, p->num_heads, L.hw, per_slice);
+        hipLaunchKernelGGL(cfh::core_gw_finish_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st_w, gwcat, L.hw,
+                           p->dist_coef, p->angle_coef, p->angle_wscale, gW_dist, gW_axis1, gW_axis2, gW_axis3);
+        return finish_launch("fused_core_weight_gradients");
+    };
+    int rc_w = CFH_OK;
+    if (two) rc_w = weight_gradients();
+
+    // ---- this stream: Wcat, G = Wcat^T go per item, records, tables, the main kernel, gk and gv
+    if (!buf.wcat_ready)
+        hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, W_dist, W_axis1,
+                           W_axis2, W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat);
+    // (with records kept from the forward the work queues are all that is left to prepare: gbuild clears them)
+    hipLaunchKernelGGL(cfh::core_gbuild_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads, L.hw / 64), dim3(cfh::WAVE), 0,
+                       st, gout, wcat, G, (int)N, p->num_heads, L.hw, buf.records_ready ? C.K.counters : nullptr);
+    if (!buf.records_ready) {
+        const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
+                                                                                          : p->num_heads * cfh::NQUEUE);
+        hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, C.K, 0);
     }
-    return finish_launch("fused_core_backward");
+    if (buf.table && !buf.table_ready)
+        hipLaunchKernelGGL(cfh::sorted_shifts_kernel, dim3((unsigned)B), dim3(cfh::FC_TCAP), 0, st, tvecs, C.table_R,
+                           buf.table);
+    const int cap = launch_waves(N, p->num_heads, CORE_WAVES_PER_SIMD);
+    const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+    const char* what = "fused_core_backward";
+    CFH_CORE_DISPATCH(cfh::fused_core_bwd_kernel);
+#undef CFH_CORE_DISPATCH
+    if (!rc) {
+        // gk, gv: sums over the pairs that point at an atom
+        cfh::DpaArgs A;
+        std::memset(&A, 0, sizeof(A));
+        A.q = qs; A.k = k; A.v = v; A.edges = edges; A.e_start = e_start;
+        A.prob = const_cast<float*>(prob); A.go = gout; A.gk = gk; A.gv = gv; A.gaij = glogit;
+        A.N = (int32_t)N; A.H = p->num_heads; A.E = (int32_t)E;
+        const int64_t items = N * p->num_heads;
+        hipLaunchKernelGGL(cfh::dpa_bwd_col_kernel, dim3((unsigned)((items + cfh::DPA_WAVES - 1) / cfh::DPA_WAVES)),
+                           dim3(cfh::WAVE * cfh::DPA_WAVES), 0, st, A);
+        rc = finish_launch("fused_core_backward");
+    }
+    if (!two) rc_w = weight_gradients();
+    // the join is enqueued whatever happened in between: a stream that was pulled into a capture must come back
+    if (two && !(p->flags & CFH_FLAG_DEFER_JOIN) &&
+        (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(st, side->join, 0) != hipSuccess) &&
+        !rc && !rc_w)
+        rc_w = fail(CFH_ELAUNCH, "join of the second stream failed");
+    return rc ? rc : rc_w;
 }
 
 }  // extern "C"

@@ -663,11 +663,14 @@ __global__ __launch_bounds__(WAVE * PROJ_WAVES) void core_project_kernel(const f
 
 // G (N,H,hw) = go (N,H,16) . Wcat_h (16, hw): wavefront per (16 atoms, head, 64-word block); four MFMA tiles whose
 // columns are interleaved (tile t, column c <-> word 4 c + t) so that a lane stores 16 consecutive bytes.
-// grid (ceil(N/16), H, hw/64).
+// grid (ceil(N/16), H, hw/64).  `queues`: optional work-queue heads to clear (when no prepare launch does).
 __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restrict__ go, const float* __restrict__ wcat,
-                                                           float* __restrict__ G, int N, int H, int hw) {
+                                                           float* __restrict__ G, int N, int H, int hw,
+                                                           int32_t* __restrict__ queues) {
     const int lane = threadIdx.x, col = lane & 15, kk = lane >> 4;
     const int h = blockIdx.y, i0 = blockIdx.x * 16;
+    if (queues && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0)      // work queues of the launch that follows
+        for (int u = lane; u < H * NQUEUE; u += WAVE) queues[u * QSTRIDE] = 0;
     const int row = min(i0 + col, N - 1);
     const float4 a4 = reinterpret_cast<const float4*>(go + ((size_t)row * H + h) * DH)[kk];      // channels 4 kk ..
     const float A[4] = {a4.x, a4.y, a4.z, a4.w};

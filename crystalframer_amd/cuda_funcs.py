@@ -135,6 +135,28 @@ def seed_edge_schedule(edge_ij_e: torch.Tensor, e_start: torch.Tensor, order: to
 
 
 _atom_start_cache = {"ref": None, "version": None, "val": None}
+_shift_table_cache = {"ref": None, "version": None, "table": None, "key": None}
+
+
+def declare_shift_tables(tvecs_n: torch.Tensor):
+    """Announce the lattice tensor that the layers of a forward pass share (the encoder does, once per pass): the
+    first fused attention core of the pass fills a table of every crystal's translations sorted by length, the
+    later ones and the backward pass read it instead of making it again."""
+    _shift_table_cache.update(ref=weakref.ref(tvecs_n), version=tvecs_n._version, table=None, key=None)
+
+
+def _shift_table_for(tvecs_n: torch.Tensor, tv: torch.Tensor, key):
+    """(table (B,128,4), ready) for a fused-core call on lattices ``tv``."""
+    c = _shift_table_cache
+    fresh = lambda: torch.empty((max(tv.shape[0], 1), 128, 4), dtype=torch.float32, device=tv.device)
+    if (c["ref"] is not None and c["ref"]() is tvecs_n and c["version"] == tvecs_n._version
+            and tv.data_ptr() == tvecs_n.data_ptr()):
+        if c["table"] is not None and c["key"] == key:
+            return c["table"], 1
+        table = fresh()
+        c.update(table=table, key=key)
+        return table, 0
+    return fresh(), 0
 
 
 def seed_atom_start(sizes: torch.Tensor, atom_start: torch.Tensor):
@@ -585,17 +607,23 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
         prob = torch.empty((E, H), dtype=torch.float32, device=dev)
         hist = torch.empty((N, H, hw), dtype=torch.float32, device=dev)
         out = torch.empty((N, H, Dh), dtype=torch.float32, device=dev)
+        # kept for the backward (and, the table, for the other layers of the pass): sorted translations of every
+        # crystal, projection weights with the moment matrices folded in, item records
+        table, table_ready = _shift_table_for(tvecs_n, tv, (p.lattice_range, p.minimum_range, p.cutoff_radius != 0.0))
+        wcat = torch.empty((H, Dh, hw), dtype=torch.float32, device=dev)
+        records = torch.empty((max(N, 1), H, 32), dtype=torch.int32, device=dev)
+        cache = _lib.CfhCoreCache(table.data_ptr(), wcat.data_ptr(), records.data_ptr(), table_ready, 0, 0, 0)
         with torch.cuda.device(dev), _timed("fused_core_forward", dev):
             ws = _lib.workspace(dev, lib.cfh_fused_core_workspace_bytes(ctypes.byref(p), N, E, tv.shape[0], 0))
             rc = lib.cfh_fused_core_forward(
                 ctypes.byref(p), _lib.ptr(q_), _lib.ptr(k_), _lib.ptr(v_), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv),
                 _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd),
                 _lib.ptr(Wa[0]), _lib.ptr(Wa[1]), _lib.ptr(Wa[2]), N, E, tv.shape[0], _lib.ptr(fr), 1 if search else 0,
-                _lib.ptr(z), _lib.ptr(prob), _lib.ptr(hist), _lib.ptr(out), _lib.ptr(ws), ws.numel(),
+                _lib.ptr(z), _lib.ptr(prob), _lib.ptr(hist), _lib.ptr(out), ctypes.byref(cache), _lib.ptr(ws), ws.numel(),
                 _lib.current_stream_ptr(dev))
         _lib.check(rc, "cfh_fused_core_forward")
         ctx.save_for_backward(q_, k_, v_, a, rpos, tv, rv, batch, edges, e_start, order, Wd, Wa[0], Wa[1], Wa[2], fr,
-                              z, prob, hist, out)
+                              z, prob, hist, out, table, wcat, records)
         ctx.params = p
         ctx.w_shapes = [None if w is None else w.shape for w in (W_k, W_k1, W_k2, W_k3)]
         ctx.in_dtype = qs.dtype
@@ -607,7 +635,7 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
     @staticmethod
     def backward(ctx, gout, gframes=None):
         (q_, k_, v_, a, rpos, tv, rv, batch, edges, e_start, order, Wd, W1, W2, W3, fr, z, prob, hist,
-         out) = ctx.saved_tensors
+         out, table, wcat, records) = ctx.saved_tensors
         lib = _lib.load()
         p = ctx.params
         N, H = a.shape
@@ -619,16 +647,39 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
         glogit = torch.empty((E, H), dtype=torch.float32, device=dev)
         gWd = torch.empty_like(Wd)
         gWa = [torch.empty_like(w) if w is not None else None for w in (W1, W2, W3)]
-        with torch.cuda.device(dev), _timed("fused_core_backward", dev):
-            ws = _lib.workspace(dev, lib.cfh_fused_core_workspace_bytes(ctypes.byref(p), N, E, tv.shape[0], 1))
-            rc = lib.cfh_fused_core_backward(
-                ctypes.byref(p), _lib.ptr(q_), _lib.ptr(k_), _lib.ptr(v_), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv),
-                _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(Wd),
-                _lib.ptr(W1), _lib.ptr(W2), _lib.ptr(W3), _lib.ptr(fr), _lib.ptr(z), _lib.ptr(prob), _lib.ptr(hist),
-                _lib.ptr(out), _lib.ptr(go), N, E, tv.shape[0], _lib.ptr(gq), _lib.ptr(gk), _lib.ptr(gv), _lib.ptr(ga),
-                _lib.ptr(glogit), _lib.ptr(gWd), _lib.ptr(gWa[0]), _lib.ptr(gWa[1]), _lib.ptr(gWa[2]), _lib.ptr(ws),
-                ws.numel(), _lib.current_stream_ptr(dev))
+        cache = _lib.CfhCoreCache(table.data_ptr(), wcat.data_ptr(), records.data_ptr(), 1, 1, 1, 0)
+        # The library makes the weight gradients of the value encoding on its second stream, beside its main
+        # kernel.  The weight gradients of the linear layers collected so far (those of the layers behind this one)
+        # go to that stream as well instead of waiting for the end of the pass; the join is then made here.
+        D = _DeferredWeightGrads
+        second = (N > 0 and not (p.flags & _lib.FLAG_SINGLE_STREAM) and bool(D.pending)
+                  and D.task_id == torch._C._current_graph_task_id())
+        flags = p.flags
+        held = None
+        rcj = 0
+        with torch.cuda.device(dev):
+            try:
+                if second:
+                    p.flags = flags | _lib.FLAG_DEFER_JOIN
+                with _timed("fused_core_backward", dev):
+                    ws = _lib.workspace(dev, lib.cfh_fused_core_workspace_bytes(ctypes.byref(p), N, E, tv.shape[0], 1))
+                    rc = lib.cfh_fused_core_backward(
+                        ctypes.byref(p), _lib.ptr(q_), _lib.ptr(k_), _lib.ptr(v_), _lib.ptr(a), _lib.ptr(rpos),
+                        _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order),
+                        _lib.ptr(Wd), _lib.ptr(W1), _lib.ptr(W2), _lib.ptr(W3), _lib.ptr(fr), _lib.ptr(z), _lib.ptr(prob),
+                        _lib.ptr(hist), _lib.ptr(out), _lib.ptr(go), N, E, tv.shape[0], _lib.ptr(gq), _lib.ptr(gk),
+                        _lib.ptr(gv), _lib.ptr(ga), _lib.ptr(glogit), _lib.ptr(gWd), _lib.ptr(gWa[0]), _lib.ptr(gWa[1]),
+                        _lib.ptr(gWa[2]), ctypes.byref(cache), _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
+                if second and rc == 0:
+                    held = D.flush(second_stream=True)
+            finally:
+                p.flags = flags
+                if second:
+                    rcj = lib.cfh_second_stream_join(_lib.current_stream_ptr(dev))
         _lib.check(rc, "cfh_fused_core_backward")
+        if second:
+            _lib.check(rcj, "cfh_second_stream_join")
+        del held            # what the second stream read is ordered before everything that follows on this one
         gws = [g if g is None else g.reshape(s) for g, s in zip([gWd] + gWa, ctx.w_shapes)]
         dt = ctx.in_dtype
         return (gq.to(dt), gk.to(dt), gv.to(dt), ga, None, None, None, None, None, None, None, gws[0], gws[1], gws[2],

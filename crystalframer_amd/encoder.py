@@ -175,6 +175,7 @@ class CrystalformerEncoderCUDA(nn.Module):
         geo = geometry.crystal_geometry(pos, batch, trans, sizes, num_edges=num_pairs)
         cuda_funcs.seed_edge_schedule(geo.edges, geo.e_start, geo.order)
         cuda_funcs.declare_complete_blocks(geo.edges)
+        cuda_funcs.declare_shift_tables(trans)
         if geo.atom_start is not None and sizes is not None:
             cuda_funcs.seed_atom_start(sizes, geo.atom_start)
         x = src

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 7
+#define CFH_ABI_VERSION 8
 
 enum {
     CFH_OK = 0,
@@ -295,7 +295,29 @@ int cfh_fused_dpa_backward(const float* q, const float* k, const float* v, const
  * Results kept for the backward: z (E,H), prob (E,H) = P, hist (N,H,words) the normalised histograms
  * (words = cfh_fused_core_hist_words: 64 distance bins, then per axis and order 64 moment bins), out (N,H,Dh).
  * workspace: cfh_fused_core_workspace_bytes(p, N, E, B, 0).
+ *
+ * cache (may be NULL, as may every pointer in it): buffers the caller keeps so that later calls need not make
+ * them again.  Without them the library makes each in its workspace on every call.
+ *   shift_table (B,128,4)   the shifts of the (2R+1)^3 box of every crystal sorted by length (R = minimum_range with
+ *                           the adaptive cutoff, else lattice_range; used when that box has at most 128 shifts and
+ *                           prune_log2 > 0).  It depends on tvecs and R only: with shift_table_ready != 0 the call
+ *                           reads it (filled by an earlier call, forward or backward, with the same tvecs and
+ *                           params), else it fills it.
+ *   wcat (H,Dh,words)       the projection weights with the moment matrices folded in; the forward writes it, the
+ *                           backward reads it when wcat_ready != 0 (same weights as in the forward) or makes it.
+ *   records (N,H,32)        the item records of the launch (box, lattice and frames of every (atom, head)); the
+ *                           forward writes them, the backward reads them when records_ready != 0 or makes them.
  */
+typedef struct cfh_core_cache {
+    float* shift_table;
+    float* wcat;
+    uint32_t* records;
+    int32_t shift_table_ready;
+    int32_t wcat_ready;
+    int32_t records_ready;
+    int32_t reserved0;
+} cfh_core_cache;
+
 size_t cfh_fused_core_workspace_bytes(const cfh_params* p, int64_t N, int64_t E, int64_t B, int32_t backward);
 int32_t cfh_fused_core_hist_words(const cfh_params* p);
 int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k, const float* v, const float* a_ih,
@@ -303,7 +325,8 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
                            const int64_t* edges, const int64_t* e_start, const int32_t* order, const float* W_dist,
                            const float* W_axis1, const float* W_axis2, const float* W_axis3, int64_t N, int64_t E,
                            int64_t B, float* frames, int32_t search_frames, float* z, float* prob, float* hist,
-                           float* out, void* workspace, size_t workspace_bytes, void* stream);
+                           float* out, const cfh_core_cache* cache, void* workspace, size_t workspace_bytes,
+                           void* stream);
 
 /*
  * Gradients of the above for upstream gout (N,H,Dh): gq (of qs), gk, gv (N,H,Dh), ga (N,H), the four weight
@@ -311,7 +334,11 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
  * No gradient flows to the frames.  What FusedDotProductAttentionCUDA.backward and
  * RealEncodingWithFramedProjFuncCUDA.backward compute together (models/cuda_funcs/fused_dpa.py:65-170,
  * real_space_framed_proj.py:123-221); the weight gradients add their atoms with float atomics.
- * workspace: cfh_fused_core_workspace_bytes(p, N, E, B, 1).
+ * The weight gradients need only gout and the histograms of the forward: they are made on the library's second
+ * stream beside the main kernel (forked from and joined to `stream` inside the call) unless
+ * p->flags has CFH_FLAG_SINGLE_STREAM; with CFH_FLAG_DEFER_JOIN the caller joins (cfh_second_stream_join).
+ * workspace: cfh_fused_core_workspace_bytes(p, N, E, B, 1).  cache: as for the forward (read when the ready words
+ * say so).
  */
 int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k, const float* v, const float* a_ih,
                             const float* rpos, const float* tvecs, const float* rvlen, const int64_t* batch,
@@ -319,8 +346,8 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
                             const float* W_axis1, const float* W_axis2, const float* W_axis3, const float* frames,
                             const float* z, const float* prob, const float* hist, const float* out, const float* gout,
                             int64_t N, int64_t E, int64_t B, float* gq, float* gk, float* gv, float* ga, float* glogit,
-                            float* gW_dist, float* gW_axis1, float* gW_axis2, float* gW_axis3, void* workspace,
-                            size_t workspace_bytes, void* stream);
+                            float* gW_dist, float* gW_axis1, float* gW_axis2, float* gW_axis3,
+                            const cfh_core_cache* cache, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Sets *flag (device memory) to 0 when edges (2,E) / e_start (N+1) hold, for every crystal, all
