@@ -21,6 +21,7 @@
 #include "framed_pe_fwd.hpp"
 #include "fused_dpa.hpp"
 #include "fused_core.hpp"
+#include "frame_select_sorted.hpp"
 #include "geometry.hpp"
 #include "linear_grad.hpp"
 #include "small_gemm.hpp"
@@ -1078,7 +1079,7 @@ CoreBuffers fill_core(cfh::CoreArgs& C, const cfh_params* p, const CoreLayout& L
     C.qs = qs; C.k = k; C.v = v;
     const bool adaptive = has_rvlen && p->cutoff_radius != 0.0f;
     const int R0 = adaptive ? p->minimum_range : p->lattice_range;
-    const bool tables = p->prune_log2 > 0.0f && R0 >= 1 && (2 * R0 + 1) * (2 * R0 + 1) * (2 * R0 + 1) <= cfh::FC_TCAP;
+    const bool tables = R0 >= 1 && (2 * R0 + 1) * (2 * R0 + 1) * (2 * R0 + 1) <= cfh::FC_TCAP;
     CoreBuffers b;
     b.table = nullptr; b.table_ready = false;
     if (tables) {
@@ -1095,9 +1096,10 @@ CoreBuffers fill_core(cfh::CoreArgs& C, const cfh_params* p, const CoreLayout& L
     C.skip_log2 = p->prune_log2 > 0.0f ? (p->prune_log2 + 8.0f > 32.0f ? p->prune_log2 + 8.0f : 32.0f) : 0.0f;
     return b;
 }
+// one wavefront (= workgroup) per (item, head); the hardware deals them to the compute units as slots free up
 template <typename Kern>
-int launch_core(Kern kern, const cfh::CoreArgs& C, int cap, hipStream_t st, const char* what) {
-    const int waves = resident_waves(kern, cap, C.K.H);
+int launch_core(Kern kern, const cfh::CoreArgs& C, hipStream_t st, const char* what) {
+    const unsigned blocks = (unsigned)C.K.N * (unsigned)C.K.H;
     bool timed = false;
     TimedLaunch t;
     {
@@ -1109,14 +1111,13 @@ int launch_core(Kern kern, const cfh::CoreArgs& C, int cap, hipStream_t st, cons
         timed = hipEventCreate(&t.start) == hipSuccess && hipEventCreate(&t.stop) == hipSuccess &&
                 hipEventRecord(t.start, st) == hipSuccess;
     }
-    hipLaunchKernelGGL(kern, dim3(waves), dim3(cfh::WAVE), 0, st, C);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(cfh::WAVE), 0, st, C);
     if (timed && hipEventRecord(t.stop, st) == hipSuccess) {
         std::lock_guard<std::mutex> lock(g_timing_mutex);
         g_timed.push_back(t);
     }
     return finish_launch(what);
 }
-constexpr int CORE_WAVES_PER_SIMD = 6;
 }  // namespace
 
 extern "C" {
@@ -1157,41 +1158,43 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     fill_common(C.K, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     const CoreBuffers buf = fill_core(C, p, L, qs, k, v, rvlen != nullptr, cache, workspace);
     const bool search = has_ang && search_frames != 0;
-    if (search) {
-        // records with the query, frame search through the first set of queues; it leaves the frames in the records
-        cfh::KernelArgs F = C.K;
-        F.q = qs; F.k = k; F.out_frame = frames;
-        F.counters2 = reinterpret_cast<int32_t*>(ws + QUEUE_OFFSET + QUEUE_SET_BYTES);
-        F.frames_to_records = 1;
-        int fwaves = launch_waves(N, p->num_heads, FRAME_WAVES_PER_SIMD);
-        if ((rc = launch_persistent(cfh::frame_axis_kernel<2>, F, &fwaves, st, "frame_axes"))) return rc;
-        C.K.counters = F.counters2;
-    } else {
-        C.K.frames = has_ang ? frames : nullptr;
-        const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
-                                                                                          : p->num_heads * cfh::NQUEUE);
-        hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, C.K, 0);
-    }
     if (buf.table && !buf.table_ready)
         hipLaunchKernelGGL(cfh::sorted_shifts_kernel, dim3((unsigned)B), dim3(cfh::FC_TCAP), 0, st, tvecs, C.table_R,
                            buf.table);
+    {
+        const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
+                                                                                          : p->num_heads * cfh::NQUEUE);
+        if (search) {
+            // records with the query, frame search through the first set of queues; it leaves the frames in the
+            // records and the main kernel takes the second set of queues
+            cfh::CoreArgs F = C;
+            F.K.q = qs; F.K.k = k; F.K.out_frame = frames;
+            F.K.counters2 = reinterpret_cast<int32_t*>(ws + QUEUE_OFFSET + QUEUE_SET_BYTES);
+            F.K.frames_to_records = 1;
+            hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, F.K, 1);
+            if ((rc = launch_core(cfh::frame_axes_sorted_kernel, F, st, "frame_axes"))) return rc;
+            C.K.counters = F.K.counters2;
+        } else {
+            C.K.frames = has_ang ? frames : nullptr;
+            hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, C.K, 0);
+        }
+    }
     float* wcat = buf.wcat;
     hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, W_dist, W_axis1, W_axis2,
                        W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat);
     C.out = out; C.prob = prob; C.z = z; C.hist = hist;
-    const int cap = launch_waves(N, p->num_heads, CORE_WAVES_PER_SIMD);
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "fused_core_forward";
 #define CFH_CORE_DISPATCH(KERNEL)                                                                         \
     do {                                                                                                  \
         if (has_ang) {                                                                                    \
-            if (wide) rc = p->cos_abs ? launch_core(KERNEL<11, true, true>, C, cap, st, what)             \
-                                      : launch_core(KERNEL<11, true, false>, C, cap, st, what);           \
-            else rc = p->cos_abs ? launch_core(KERNEL<9, true, true>, C, cap, st, what)                   \
-                                 : launch_core(KERNEL<9, true, false>, C, cap, st, what);                 \
+            if (wide) rc = p->cos_abs ? launch_core(KERNEL<11, true, true>, C, st, what)             \
+                                      : launch_core(KERNEL<11, true, false>, C, st, what);           \
+            else rc = p->cos_abs ? launch_core(KERNEL<9, true, true>, C, st, what)                   \
+                                 : launch_core(KERNEL<9, true, false>, C, st, what);                 \
         } else {                                                                                          \
-            rc = wide ? launch_core(KERNEL<11, false, false>, C, cap, st, what)                           \
-                      : launch_core(KERNEL<9, false, false>, C, cap, st, what);                           \
+            rc = wide ? launch_core(KERNEL<11, false, false>, C, st, what)                           \
+                      : launch_core(KERNEL<9, false, false>, C, st, what);                           \
         }                                                                                                 \
     } while (0)
     CFH_CORE_DISPATCH(cfh::fused_core_fwd_kernel);
@@ -1288,7 +1291,6 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
     if (buf.table && !buf.table_ready)
         hipLaunchKernelGGL(cfh::sorted_shifts_kernel, dim3((unsigned)B), dim3(cfh::FC_TCAP), 0, st, tvecs, C.table_R,
                            buf.table);
-    const int cap = launch_waves(N, p->num_heads, CORE_WAVES_PER_SIMD);
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "fused_core_backward";
     CFH_CORE_DISPATCH(cfh::fused_core_bwd_kernel);

@@ -104,7 +104,9 @@ __device__ __forceinline__ int rint_i(float x) { return (int)__builtin_rintf(x);
 
 // ---- sorted shifts of the usual box, one table per crystal ---------------------------------------------------
 // block = crystal, 128 threads; entry = (shift, |shift|), ascending length (ties: loop order); entries beyond the
-// box: length +inf.
+// box: length +inf.  The low 7 bits of the length hold the translation's index in the reference's loop order (the
+// frame search breaks ties by it): the length is rounded down by at most 2^-16 of itself, which the margins of every
+// reach test cover.
 __global__ __launch_bounds__(FC_TCAP) void sorted_shifts_kernel(const float* __restrict__ tvecs, int R0, float4* __restrict__ out) {
     __shared__ float key[FC_TCAP];
     const int b = blockIdx.x, t = threadIdx.x;
@@ -125,6 +127,7 @@ __global__ __launch_bounds__(FC_TCAP) void sorted_shifts_kernel(const float* __r
         const float ku = key[u];
         rank += (ku < v.w || (ku == v.w && u < t)) ? 1 : 0;
     }
+    if (t < T0) v.w = __uint_as_float((__float_as_uint(v.w) & ~(uint32_t)(FC_TCAP - 1)) | (uint32_t)t);
     out[(size_t)b * FC_TCAP + rank] = v;
 }
 
@@ -319,31 +322,15 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
     const float INF = __builtin_inff();
 
+    const int it_cur = (int)blockIdx.x / H;      // items in descending order of their pair count: the long ones start first
+    if (it_cur >= P.N) return;
     for (int u = lane; u < HWK; u += WAVE) hist[u] = 0;
     wave_sync();
 
-    unsigned long long st_eval = 0, st_raw = 0, st_pairs = 0, st_seen = 0;
     CFH_PH_DECL
-    int queue = first_queue(H);
-    int it_cur = queue_pop(P, h, queue);
-    int it_next = it_cur >= 0 ? queue_pop(P, h, queue) : -1;
-    uint32_t rec_cur = load_record(P, it_cur, h);
-    CorePrefetch pf = core_prefetch(C, rec_cur, it_cur, h, lane);
-    while (it_cur >= 0) {
-        CFH_PH(6);
-        const uint32_t rec_next = load_record(P, it_next, h);
-        int ticket = 0;
-        CorePrefetch pf_next = pf;
-        bool drawn = false;
-        // The ticket of the item after next is drawn, and the operands of the next item are requested, after the
-        // sweeps of the first group: the function that draws the ticket starts by waiting for everything this
-        // wavefront has in flight, and by then the stores of the previous item have been acknowledged, while the
-        // rest of this item is enough for the requested operands to land.
-        auto draw_and_prefetch = [&]() {
-            ticket = queue_ticket(P, h, queue);
-            pf_next = core_prefetch(C, rec_next, it_next, h, lane);
-            drawn = true;
-        };
+    {
+        const uint32_t rec_cur = load_record(P, it_cur, h);
+        const CorePrefetch pf = core_prefetch(C, rec_cur, it_cur, h, lane);
         CFH_PH(0);
         const CoreItem ci = core_unpack(C, rec_cur, true);
         const int i = ci.item.i;
@@ -494,7 +481,6 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
                 }
             });
             const float S = half_sum(Sb);
-            if (g0 == 0) { CFH_PH(6); draw_and_prefetch(); }
 
             // ---- logits, running softmax
             CFH_PH(3);
@@ -556,12 +542,6 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
         }
 
         // ---- the row is complete: normalise and write
-        CFH_PH(5);
-        if (!drawn) draw_and_prefetch();      // (an atom without pairs)
-        // what was requested for the next item is taken over before this item's stores are issued: a wait for it
-        // afterwards would also wait for those stores
-        pf = pf_next;
-        asm volatile("" :: "v"(pf.t0.x), "v"(pf.t1.x), "v"(pf.q2.x), "v"(pf.rx), "v"(pf.k2.x), "v"(pf.v2.x));
         CFH_PH(7);
         const float D = uniform_f(wave_sum(Dl));
         const float inv = D > 0.0f ? hw_rcp(D) : 0.0f;
@@ -578,14 +558,7 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
 #pragma unroll
             for (int u = 0; u < NW; u++) hv[u] = hist[lane + WAVE * u];
 #pragma unroll
-            for (int u = 0; u < NW; u++) {
-                hist[lane + WAVE * u] = 0;
-#ifndef CFH_EXP_NOHIST
-                dst[WAVE * u] = (float)hv[u] * sc;
-#else
-                if (hv[u] == 0x7fffffff) dst[WAVE * u] = (float)hv[u] * sc;
-#endif
-            }
+            for (int u = 0; u < NW; u++) dst[WAVE * u] = (float)hv[u] * sc;
         }
         if (npairs <= FC_LOGCAP) {                               // logits -> probabilities
             for (int el = lane; el < npairs; el += WAVE)
@@ -598,21 +571,13 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
                 }
             }
         }
-        CFH_PH(6);
-        st_eval += n_eval;
-        st_seen += n_seen;
-        st_raw += (unsigned long long)bx.T * (unsigned long long)npairs;
-        st_pairs += (unsigned long long)npairs;
-        it_cur = it_next;
-        rec_cur = rec_next;
-        it_next = it_cur >= 0 ? queue_redeem(P, h, queue, ticket) : -1;
-    }
-    CFH_PH_FLUSH(P.stats);
-    if (P.stats && lane == 0) {         // one set of atomics per wavefront
-        atomicAdd(P.stats + STAT_FWD_EVAL, st_eval);
-        atomicAdd(P.stats + STAT_FWD_RAW, st_raw);
-        atomicAdd(P.stats + STAT_FWD_PAIRS, st_pairs);
-        atomicAdd(P.stats + STAT_FWD_SEEN, st_seen);
+        CFH_PH_FLUSH(P.stats);
+        if (P.stats && lane == 0) {
+            atomicAdd(P.stats + STAT_FWD_EVAL, n_eval);
+            atomicAdd(P.stats + STAT_FWD_RAW, (unsigned long long)bx.T * (unsigned long long)npairs);
+            atomicAdd(P.stats + STAT_FWD_PAIRS, (unsigned long long)npairs);
+            atomicAdd(P.stats + STAT_FWD_SEEN, n_seen);
+        }
     }
 }
 
@@ -773,14 +738,10 @@ __global__ __launch_bounds__(WAVE) void fused_core_bwd_kernel(const CoreArgs C) 
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
     const float INF = __builtin_inff();
 
-    unsigned long long st_eval = 0, st_raw = 0, st_pairs = 0;
-    int queue = first_queue(H);
-    int it_cur = queue_pop(P, h, queue);
-    int it_next = it_cur >= 0 ? queue_pop(P, h, queue) : -1;
-    uint32_t rec_cur = load_record(P, it_cur, h);
-    while (it_cur >= 0) {
-        const int ticket = queue_ticket(P, h, queue);
-        const uint32_t rec_next = load_record(P, it_next, h);
+    const int it_cur = (int)blockIdx.x / H;      // one wavefront per item, long items first
+    if (it_cur >= P.N) return;
+    {
+        const uint32_t rec_cur = load_record(P, it_cur, h);
         const CoreItem ci = core_unpack(C, rec_cur, true);
         const int i = ci.item.i;
         const float a2 = ci.item.a * LOG2E;
@@ -797,7 +758,6 @@ __global__ __launch_bounds__(WAVE) void fused_core_bwd_kernel(const CoreArgs C) 
         }
         const int e0 = ci.item.e0, npairs = ci.item.npairs;
         const size_t ih = (size_t)i * H + h;
-        wave_sync();
         core_load_table(C, ci, tab, lane);
         float gabs = 0.0f;
         {
@@ -962,17 +922,11 @@ __global__ __launch_bounds__(WAVE) void fused_core_bwd_kernel(const CoreArgs C) 
             if (lane < FC_GROUP) *reinterpret_cast<float2*>(C.gq + ih * DH + 2 * sub) = make_float2(gx, gy);
         }
         if (lane == 0) P.out_ga[ih] = cov;
-        st_eval += n_eval;
-        st_raw += (unsigned long long)bx.T * (unsigned long long)npairs;
-        st_pairs += (unsigned long long)npairs;
-        it_cur = it_next;
-        rec_cur = rec_next;
-        it_next = it_cur >= 0 ? queue_redeem(P, h, queue, ticket) : -1;
-    }
-    if (P.stats && lane == 0) {
-        atomicAdd(P.stats + STAT_BWD_EVAL, st_eval);
-        atomicAdd(P.stats + STAT_BWD_RAW, st_raw);
-        atomicAdd(P.stats + STAT_BWD_PAIRS, st_pairs);
+        if (P.stats && lane == 0) {
+            atomicAdd(P.stats + STAT_BWD_EVAL, n_eval);
+            atomicAdd(P.stats + STAT_BWD_RAW, (unsigned long long)bx.T * (unsigned long long)npairs);
+            atomicAdd(P.stats + STAT_BWD_PAIRS, (unsigned long long)npairs);
+        }
     }
 }
 

@@ -170,6 +170,52 @@ def test_fused_core_with_frame_search_equals_two_step_path():
     compare(P, _gout(P), out, leaves, oo, oleaves)
 
 
+def _frames_both_ways(P, cutoff=CUT):
+    """Frames of the fused core's own search (translations sorted by length, bounded prefixes) and of
+    ComputeFramesMaximumMethodCUDA (whole boxes, slabs skipped): two searches written independently."""
+    import crystalframer_amd as cf
+    _, fr, _ = run_core(P, frames="search", need_grad=False, cutoff=cutoff)
+    extra = (g(P.rvlen), cutoff) if cutoff is not None else ()
+    ref = cf.ComputeFramesMaximumMethodCUDA.apply(g(P.q), g(P.k), None, g(P.a), g(P.rpos), None, g(P.tvecs),
+                                                  P.batch.to(dev()), P.edges.to(dev()), 64, Hh.DIST_MAX, 1.0, *extra)
+    return fr, ref
+
+
+@pytest.mark.parametrize("noise", [0.0, 1e-5, 1e-2])
+def test_sorted_frame_search_equals_the_box_search_at_batch_256(noise):
+    """Both searches take the arg-max of the same scores with the same tie rule and, for a given seed, the same
+    noise, so the frames are equal bit for bit -- if the bounded prefixes of the sorted search never lose the winner."""
+    import crystalframer_amd as cf
+    from crystalframer_amd import synthetic
+    KM = cf.KernelManager
+    KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE = noise, 1234567, None
+    P = Hh.problem_from_batch(synthetic.make_config("C2"), seed=9)
+    fr, ref = _frames_both_ways(P)
+    assert torch.equal(fr, ref)
+    n = fr.norm(dim=-1)
+    assert float((n - 1).abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("noise", [0.0, 1e-5])
+def test_sorted_frame_search_mixed_boxes_fixed_box_and_long_rows(noise):
+    """Small cells (boxes wider than the table's: whole-box scan in chunks), the fixed box without a cutoff, rows
+    of more pairs than are staged at once, one-atom crystals (only self images: exact +-n ties)."""
+    import crystalframer_amd as cf
+    KM = cf.KernelManager
+    KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE = noise, 99, None
+    P = Hh.make_problem(num_crystals=6, atoms_lo=2, atoms_hi=12, len_lo=2.5, len_hi=7.0, seed=301)
+    fr, ref = _frames_both_ways(P)
+    assert torch.equal(fr, ref)
+    fr, ref = _frames_both_ways(P, cutoff=None)
+    assert torch.equal(fr, ref)
+    P = Hh.make_problem(num_crystals=1, atoms_lo=300, atoms_hi=300, len_lo=14.0, len_hi=16.0, seed=302)
+    fr, ref = _frames_both_ways(P)
+    assert torch.equal(fr, ref)
+    P = Hh.make_problem(num_crystals=7, atoms_lo=1, atoms_hi=1, seed=303)
+    fr, ref = _frames_both_ways(P)
+    assert torch.equal(fr, ref)
+
+
 def test_fused_core_one_atom_crystals_and_empty_batch():
     from crystalframer_amd import cuda_funcs as F
     P = Hh.make_problem(num_crystals=5, atoms_lo=1, atoms_hi=1, seed=41)
