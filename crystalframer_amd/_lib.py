@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
@@ -61,7 +61,8 @@ class CfhAttentionInputsGrad(ctypes.Structure):
 
 class CfhCoreCache(ctypes.Structure):
     """Mirror of ``cfh_core_cache`` in include/crystalframer_hip.h."""
-    _fields_ = [("shift_table", ctypes.c_void_p), ("wcat", ctypes.c_void_p), ("records", ctypes.c_void_p),
+    _fields_ = [("shift_table", ctypes.c_void_p), ("pair_near", ctypes.c_void_p), ("wcat", ctypes.c_void_p),
+                ("records", ctypes.c_void_p),
                 ("shift_table_ready", ctypes.c_int32), ("wcat_ready", ctypes.c_int32),
                 ("records_ready", ctypes.c_int32), ("reserved0", ctypes.c_int32)]
 

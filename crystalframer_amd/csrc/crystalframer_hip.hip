@@ -1037,16 +1037,17 @@ int cfh_small_linear_dx(const float* dy, const float* W, int64_t M, int64_t N, i
 // ---- fused attention core ----------------------------------------------------------------------------------------
 namespace {
 struct CoreLayout {
-    size_t items, sorted, wcat, gwcat, G, total;
+    size_t items, sorted, near, wcat, gwcat, G, total;
     int hw;
 };
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-CoreLayout core_layout(const cfh_params* p, int64_t N, int64_t B, bool backward) {
+CoreLayout core_layout(const cfh_params* p, int64_t N, int64_t E, int64_t B, bool backward) {
     CoreLayout L;
     L.hw = p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
     size_t off = COUNTER_BYTES;
     L.items = off; off += items_bytes(N > 0 ? N : 1, p->num_heads);
     L.sorted = off; off += align256((size_t)(B > 0 ? B : 1) * cfh::FC_TCAP * sizeof(float4));
+    L.near = off; if (!backward) off += align256((size_t)(E > 0 ? E : 1) * sizeof(float2));
     L.wcat = off; off += align256((size_t)p->num_heads * cfh::DH * L.hw * sizeof(float));
     L.gwcat = off; if (backward) off += align256((size_t)p->num_heads * cfh::DH * L.hw * sizeof(float));
     L.G = off; if (backward) off += align256((size_t)(N > 0 ? N : 1) * p->num_heads * L.hw * sizeof(float));
@@ -1068,6 +1069,7 @@ int check_core_params(const cfh_params* p) {
 // workspace regions of the same content
 struct CoreBuffers {
     float4* table;       // sorted shifts (null: not used by this launch)
+    float2* near;        // nearest images per pair (forward only; made with the table)
     bool table_ready;
     float* wcat;
     bool wcat_ready;
@@ -1081,11 +1083,14 @@ CoreBuffers fill_core(cfh::CoreArgs& C, const cfh_params* p, const CoreLayout& L
     const int R0 = adaptive ? p->minimum_range : p->lattice_range;
     const bool tables = R0 >= 1 && (2 * R0 + 1) * (2 * R0 + 1) * (2 * R0 + 1) <= cfh::FC_TCAP;
     CoreBuffers b;
-    b.table = nullptr; b.table_ready = false;
+    b.table = nullptr; b.near = nullptr; b.table_ready = false;
     if (tables) {
         const bool own = cache && cache->shift_table;
         b.table = own ? reinterpret_cast<float4*>(cache->shift_table) : reinterpret_cast<float4*>(ws + L.sorted);
         b.table_ready = own && cache->shift_table_ready != 0;
+        // the per-pair minima travel with the table: the caller's when it keeps both, else (forward) the workspace's
+        if (own && cache->pair_near) b.near = reinterpret_cast<float2*>(cache->pair_near);
+        else if (!own && L.near != L.wcat) b.near = reinterpret_cast<float2*>(ws + L.near);
     }
     b.wcat = (cache && cache->wcat) ? cache->wcat : reinterpret_cast<float*>(ws + L.wcat);
     b.wcat_ready = cache && cache->wcat && cache->wcat_ready != 0;
@@ -1123,9 +1128,8 @@ int launch_core(Kern kern, const cfh::CoreArgs& C, hipStream_t st, const char* w
 extern "C" {
 
 size_t cfh_fused_core_workspace_bytes(const cfh_params* p, int64_t N, int64_t E, int64_t B, int32_t backward) {
-    (void)E;
     if (check_core_params(p) != CFH_OK) return 0;
-    return core_layout(p, N, B, backward != 0).total;
+    return core_layout(p, N, E, B, backward != 0).total;
 }
 
 int32_t cfh_fused_core_hist_words(const cfh_params* p) {
@@ -1149,7 +1153,7 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
         return fail(CFH_EINVAL, "qs, k, v, W_dist, z, prob, hist and out must not be NULL");
     if (has_ang && (!W_axis1 || !W_axis2 || !W_axis3 || !frames))
         return fail(CFH_EINVAL, "the angle encoding needs W_axis1..3 and frames");
-    const CoreLayout L = core_layout(p, N, B, false);
+    const CoreLayout L = core_layout(p, N, E, B, false);
     if ((rc = check_workspace(workspace, workspace_bytes, L.total))) return rc;
     hipStream_t st = (hipStream_t)stream;
     char* ws = reinterpret_cast<char*>(workspace);
@@ -1158,9 +1162,16 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     fill_common(C.K, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
     const CoreBuffers buf = fill_core(C, p, L, qs, k, v, rvlen != nullptr, cache, workspace);
     const bool search = has_ang && search_frames != 0;
-    if (buf.table && !buf.table_ready)
+    if (buf.table && !buf.table_ready) {
         hipLaunchKernelGGL(cfh::sorted_shifts_kernel, dim3((unsigned)B), dim3(cfh::FC_TCAP), 0, st, tvecs, C.table_R,
                            buf.table);
+        if (buf.near && E > 0) {
+            const int s0 = 2 * C.table_R + 1;
+            hipLaunchKernelGGL(cfh::pair_nearest_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, rpos, edges,
+                               batch, buf.table, s0 * s0 * s0, (int)E, buf.near);
+        }
+    }
+    C.pair_near = buf.near;
     {
         const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
                                                                                           : p->num_heads * cfh::NQUEUE);
@@ -1227,7 +1238,7 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         return fail(CFH_EINVAL, "fused core backward: a required pointer is NULL");
     if (has_ang && (!W_axis1 || !W_axis2 || !W_axis3 || !frames))
         return fail(CFH_EINVAL, "the angle encoding needs W_axis1..3 and frames");
-    const CoreLayout L = core_layout(p, N, B, true);
+    const CoreLayout L = core_layout(p, N, E, B, true);
     if ((rc = check_workspace(workspace, workspace_bytes, L.total))) return rc;
     char* ws = reinterpret_cast<char*>(workspace);
     float* gwcat = reinterpret_cast<float*>(ws + L.gwcat);

@@ -105,6 +105,7 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
         wave_sync();
         const float s1 = sorted ? tab[1].w : 0.0f;      // shortest non-zero shift (entry 0 is the zero shift)
 
+        float dvalid = -1.0f;                           // this lane's pair: d^2 of its nearest valid image, when known
         float f1x = 0.f, f1y = 0.f, f1z = 0.f;          // first axis
         float f2x = 0.f, f2y = 0.f, f2z = 0.f;          // second axis before orthogonalisation
         unsigned long long n_seen = 0;
@@ -121,6 +122,7 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
                     // stage rpos and q_i.k_j of the pairs, one per lane (a row that fits stays staged for all sweeps;
                     // the pairs of an atom point at consecutive atoms)
                     float4 rq = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (sw == 0 && C.pair_near && sorted && lane < npc) dvalid = C.pair_near[e0 + pb + lane].y;
                     if (npairs > WAVE || (pass == 0 && sw == 0)) {
                         if (lane < npc) {
                             const int e = e0 + pb + lane;
@@ -148,7 +150,10 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
                         const float r2 = fmaf(rq.x, rq.x, fmaf(rq.y, rq.y, rq.z * rq.z));
                         const float r = hw_sqrt(r2);
                         if (sw == 0) {
-                            reach = fmaf(1.0001f, fmaf(2.0f, r, (r2 > 1e-5f ? 0.0f : s1) + sq_nz), 1e-3f);
+                            // nearest valid image at distance d: every candidate within the noise of it has
+                            // |s| <= |r| + sqrt(d^2 + noise); without the batch's table of d: d <= |r| (+ |s_1|)
+                            reach = dvalid >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(dvalid + nz), 1e-3f)
+                                                   : fmaf(1.0001f, fmaf(2.0f, r, (r2 > 1e-5f ? 0.0f : s1) + sq_nz), 1e-3f);
                         } else if (bound > -1.0e38f) {
                             const float need = (bound - rq.w - 0.5f * nz) / a;
                             reach = need >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(need), 1e-3f) : -1.0f;

@@ -72,6 +72,8 @@ struct CoreArgs {
     const float* k;               // (N,H,16)
     const float* v;               // (N,H,16)
     const float4* sorted_tab;     // (B, FC_TCAP) shifts of the usual box sorted by length, w = length; or null
+    const float2* pair_near;      // (E) per pair over that box: smallest d^2 of all images, of the images with
+                                  // d^2 > 1e-5 (what the frame search may point at); or null
     int32_t table_R;              // half-width that table was made for
     float skip_log2;              // images lighter than 2^-skip of the heaviest of their pair are not visited (<= 0: all are)
     // forward results
@@ -129,6 +131,33 @@ __global__ __launch_bounds__(FC_TCAP) void sorted_shifts_kernel(const float* __r
     }
     if (t < T0) v.w = __uint_as_float((__float_as_uint(v.w) & ~(uint32_t)(FC_TCAP - 1)) | (uint32_t)t);
     out[(size_t)b * FC_TCAP + rank] = v;
+}
+
+// Per pair, over the usual box of its crystal: the smallest squared distance of all images and of the images with
+// d^2 > 1e-5.  Both depend on the geometry alone, not on the head or the layer, so they are made once per batch:
+// the lattice sums of an item with the usual box then need no sweep for the nearest image, and the frame search
+// knows how far into the sorted table a pair's best first-axis candidate can sit.  Thread per pair; the sorted
+// order ends the loop once |s| - |r| exceeds the larger of the two minima.  Same arithmetic for d^2 as the sweeps.
+__global__ __launch_bounds__(256) void pair_nearest_kernel(const float* __restrict__ rpos, const int64_t* __restrict__ edges,
+                                                           const int64_t* __restrict__ batch,
+                                                           const float4* __restrict__ sorted_tab, int T0, int E,
+                                                           float2* __restrict__ out) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= E) return;
+    const int b = (int)batch[edges[e]];
+    const float4* tab = sorted_tab + (size_t)b * FC_TCAP;
+    const float rx = rpos[(size_t)e * 3 + 0], ry = rpos[(size_t)e * 3 + 1], rz = rpos[(size_t)e * 3 + 2];
+    const float r = sqrtf(fmaf(rx, rx, fmaf(ry, ry, rz * rz)));
+    float dall = 3.0e38f, dval = 3.0e38f;
+    for (int t = 0; t < T0; t++) {
+        const float4 v = tab[t];
+        if (dval < 1.0e38f && v.w > fmaf(1.0001f, r + sqrtf(dval), 1e-3f)) break;
+        const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+        const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+        dall = fminf(dall, d2);
+        if (d2 > 1e-5f) dval = fminf(dval, d2);
+    }
+    out[e] = make_float2(dall, dval);
 }
 
 // ---- projection weights with the moment matrices folded in ---------------------------------------------------
@@ -259,12 +288,14 @@ struct CorePrefetch {
     float2 q2;
     float rx, ry, rz;
     float2 k2, v2;
+    float near;       // smallest d^2 over the images of that pair (when the batch's table of them is given)
 };
 __device__ __forceinline__ CorePrefetch core_prefetch(const CoreArgs& C, uint32_t rec, int it, int h, int lane) {
     CorePrefetch pf;
     pf.t0 = pf.t1 = make_float4(0.f, 0.f, 0.f, 0.f);
     pf.q2 = pf.k2 = pf.v2 = make_float2(0.f, 0.f);
     pf.rx = pf.ry = pf.rz = 0.f;
+    pf.near = 3.0e38f;
     if (it < 0) return pf;
     const KernelArgs& P = C.K;
     const int H = P.H;
@@ -286,6 +317,7 @@ __device__ __forceinline__ CorePrefetch core_prefetch(const CoreArgs& C, uint32_
         pf.rx = P.rpos[e * 3 + 0]; pf.ry = P.rpos[e * 3 + 1]; pf.rz = P.rpos[e * 3 + 2];
         pf.k2 = *reinterpret_cast<const float2*>(C.k + jh);
         pf.v2 = *reinterpret_cast<const float2*>(C.v + jh);
+        if (C.pair_near) pf.near = C.pair_near[e].x;
     }
     return pf;
 }
@@ -361,8 +393,9 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
         unsigned long long n_eval = 0, n_seen = 0;      // wave-uniform counts
 
         // operands of the pair served by this row, fetched one group ahead (the first group: with the item)
-        float nrx = pf.rx, nry = pf.ry, nrz = pf.rz;
+        float nrx = pf.rx, nry = pf.ry, nrz = pf.rz, nnear = pf.near;
         float2 nk2 = pf.k2, nv2 = pf.v2;
+        const bool near_known = sorted && C.pair_near != nullptr;      // the nearest image of every pair comes with the batch
         auto fetch = [&](int g0) {
             const int el = g0 + pr;
             if (el < npairs) {
@@ -371,6 +404,7 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
                 nrx = P.rpos[e * 3 + 0]; nry = P.rpos[e * 3 + 1]; nrz = P.rpos[e * 3 + 2];
                 nk2 = *reinterpret_cast<const float2*>(C.k + jh);
                 nv2 = *reinterpret_cast<const float2*>(C.v + jh);
+                if (near_known) nnear = C.pair_near[e].x;
             }
         };
 
@@ -453,16 +487,19 @@ __global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) 
         for (int g0 = 0; g0 < npairs; g0 += FC_GROUP) {
             const float rx = nrx, ry = nry, rz = nrz;
             const float2 k2 = nk2, v2 = nv2;
+            float d2min = nnear;
             if (g0 + FC_GROUP < npairs) fetch(g0 + FC_GROUP);
             const bool active = g0 + pr < npairs;
             const float rn = hw_sqrt(fmaf(rx, rx, fmaf(ry, ry, rz * rz)));
 
-            // ---- pass A: nearest image
+            // ---- pass A: nearest image (known beforehand for the usual box)
             CFH_PH(1);
-            float d2min = 3.0e38f;
-            sweep(active, rx, ry, rz, sorted ? fmaf(2.0002f, rn, 1e-4f) : INF,
-                  [&](bool in, int, float d2, int cnt_in) { d2min = in ? fminf(d2min, d2) : d2min; n_seen += cnt_in; });
-            d2min = half_min(d2min);
+            if (!near_known) {
+                d2min = 3.0e38f;
+                sweep(active, rx, ry, rz, sorted ? fmaf(2.0002f, rn, 1e-4f) : INF,
+                      [&](bool in, int, float d2, int cnt_in) { d2min = in ? fminf(d2min, d2) : d2min; n_seen += cnt_in; });
+                d2min = half_min(d2min);
+            }
 
             // ---- pass B: weights, normaliser and (one-chunk tables) the survivors
             CFH_PH(2);

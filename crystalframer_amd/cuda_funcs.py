@@ -145,10 +145,13 @@ def declare_shift_tables(tvecs_n: torch.Tensor):
     _shift_table_cache.update(ref=weakref.ref(tvecs_n), version=tvecs_n._version, table=None, key=None)
 
 
-def _shift_table_for(tvecs_n: torch.Tensor, tv: torch.Tensor, key):
-    """(table (B,128,4), ready) for a fused-core call on lattices ``tv``."""
+def _shift_table_for(tvecs_n: torch.Tensor, tv: torch.Tensor, key, E: int):
+    """(table, ready) for a fused-core call on lattices ``tv``: one buffer holding the sorted translations of every
+    crystal (B,128,4) and, behind them, the nearest-image distances of every pair (E,2)."""
     c = _shift_table_cache
-    fresh = lambda: torch.empty((max(tv.shape[0], 1), 128, 4), dtype=torch.float32, device=tv.device)
+    nb = max(tv.shape[0], 1) * 512
+    fresh = lambda: torch.empty(nb + 2 * max(E, 1), dtype=torch.float32, device=tv.device)
+    key = key + (E,)
     if (c["ref"] is not None and c["ref"]() is tvecs_n and c["version"] == tvecs_n._version
             and tv.data_ptr() == tvecs_n.data_ptr()):
         if c["table"] is not None and c["key"] == key:
@@ -609,10 +612,12 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
         out = torch.empty((N, H, Dh), dtype=torch.float32, device=dev)
         # kept for the backward (and, the table, for the other layers of the pass): sorted translations of every
         # crystal, projection weights with the moment matrices folded in, item records
-        table, table_ready = _shift_table_for(tvecs_n, tv, (p.lattice_range, p.minimum_range, p.cutoff_radius != 0.0))
+        table, table_ready = _shift_table_for(tvecs_n, tv, (p.lattice_range, p.minimum_range, p.cutoff_radius != 0.0,
+                                                            rpos.data_ptr()), E)
+        near_ptr = table.data_ptr() + 4 * 512 * max(tv.shape[0], 1)
         wcat = torch.empty((H, Dh, hw), dtype=torch.float32, device=dev)
         records = torch.empty((max(N, 1), H, 32), dtype=torch.int32, device=dev)
-        cache = _lib.CfhCoreCache(table.data_ptr(), wcat.data_ptr(), records.data_ptr(), table_ready, 0, 0, 0)
+        cache = _lib.CfhCoreCache(table.data_ptr(), near_ptr, wcat.data_ptr(), records.data_ptr(), table_ready, 0, 0, 0)
         with torch.cuda.device(dev), _timed("fused_core_forward", dev):
             ws = _lib.workspace(dev, lib.cfh_fused_core_workspace_bytes(ctypes.byref(p), N, E, tv.shape[0], 0))
             rc = lib.cfh_fused_core_forward(
@@ -647,7 +652,7 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
         glogit = torch.empty((E, H), dtype=torch.float32, device=dev)
         gWd = torch.empty_like(Wd)
         gWa = [torch.empty_like(w) if w is not None else None for w in (W1, W2, W3)]
-        cache = _lib.CfhCoreCache(table.data_ptr(), wcat.data_ptr(), records.data_ptr(), 1, 1, 1, 0)
+        cache = _lib.CfhCoreCache(table.data_ptr(), None, wcat.data_ptr(), records.data_ptr(), 1, 1, 1, 0)
         # The library makes the weight gradients of the value encoding on its second stream, beside its main
         # kernel.  The weight gradients of the linear layers collected so far (those of the layers behind this one)
         # go to that stream as well instead of waiting for the end of the pass; the join is then made here.

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 8
+#define CFH_ABI_VERSION 9
 
 enum {
     CFH_OK = 0,
@@ -303,6 +303,11 @@ int cfh_fused_dpa_backward(const float* q, const float* k, const float* v, const
  *                           prune_log2 > 0).  It depends on tvecs and R only: with shift_table_ready != 0 the call
  *                           reads it (filled by an earlier call, forward or backward, with the same tvecs and
  *                           params), else it fills it.
+ *   pair_near (E,2)         per pair over that box: the smallest squared distance of all images and of the images
+ *                           with d^2 > 1e-5 (geometry alone: made once per batch, together with shift_table and
+ *                           under the same ready word; the lattice sums then skip their sweep for the nearest
+ *                           image and the frame search reads shorter prefixes of the table).  Only the forward
+ *                           uses it; without it the forward makes it in its workspace.
  *   wcat (H,Dh,words)       the projection weights with the moment matrices folded in; the forward writes it, the
  *                           backward reads it when wcat_ready != 0 (same weights as in the forward) or makes it.
  *   records (N,H,32)        the item records of the launch (box, lattice and frames of every (atom, head)); the
@@ -310,6 +315,7 @@ int cfh_fused_dpa_backward(const float* q, const float* k, const float* v, const
  */
 typedef struct cfh_core_cache {
     float* shift_table;
+    float* pair_near;
     float* wcat;
     uint32_t* records;
     int32_t shift_table_ready;
