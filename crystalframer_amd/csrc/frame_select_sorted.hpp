@@ -167,8 +167,11 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
                             build_shift_table_indexed(tab, t0c, cnt, bx, L, lane);
                         }
                         wave_sync();              // pq, the table; the readers of pstart are done
+                        // the bound sweep of the second axis looks at the candidates of the first axis' sweep: when
+                        // the row is staged as a whole their list is still there
+                        const bool relist = !(pass == 1 && sw == 0 && sorted && npairs <= WAVE);
                         int mine = cnt;           // candidates of this lane's pair: entries with length <= reach
-                        if (sorted) {
+                        if (sorted && relist) {
                             int lo = 0, hi = FC_TCAP;
 #pragma unroll
                             for (int s = 0; s < 8; s++) {      // the count is one of 0 .. 128: eight halvings
@@ -179,13 +182,19 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
                             }
                             mine = min(lo, cnt);
                         }
-                        if (lane >= npc) mine = 0;
-                        const int incl = wave_scan_incl(mine);
-                        const int total = __builtin_amdgcn_readlane(incl, WAVE - 1);
-                        pstart[lane] = incl - mine;
-                        if (lane == 0) pstart[WAVE] = total;
-                        wave_sync();
+                        int total;
+                        if (relist) {
+                            if (lane >= npc) mine = 0;
+                            const int incl = wave_scan_incl(mine);
+                            total = __builtin_amdgcn_readlane(incl, WAVE - 1);
+                            pstart[lane] = incl - mine;
+                            if (lane == 0) pstart[WAVE] = total;
+                            wave_sync();
+                        } else {
+                            total = uniform_i(pstart[WAVE]);
+                        }
                         n_seen += (unsigned long long)total;
+
                         for (int base = 0; base < total; base += WAVE) {
                             const int c = base + lane;
                             const bool in = c < total;
@@ -231,9 +240,14 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
             if (best.e != 0x7fffffff) {
                 float sx, sy, sz;
                 shift_of(best.t, bx, L, sx, sy, sz);
-                vx = uniform_f(P.rpos[(size_t)best.e * 3 + 0]) + sx;
-                vy = uniform_f(P.rpos[(size_t)best.e * 3 + 1]) + sy;
-                vz = uniform_f(P.rpos[(size_t)best.e * 3 + 2]) + sz;
+                if (npairs <= WAVE) {                 // the row is still staged
+                    const float4 rq = pq[best.e - e0];
+                    vx = rq.x + sx; vy = rq.y + sy; vz = rq.z + sz;
+                } else {
+                    vx = uniform_f(P.rpos[(size_t)best.e * 3 + 0]) + sx;
+                    vy = uniform_f(P.rpos[(size_t)best.e * 3 + 1]) + sy;
+                    vz = uniform_f(P.rpos[(size_t)best.e * 3 + 2]) + sz;
+                }
                 const float inv = 1.0f / sqrtf(vx * vx + vy * vy + vz * vz);
                 vx *= inv; vy *= inv; vz *= inv;
             }
