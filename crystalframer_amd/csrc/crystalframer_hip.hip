@@ -112,6 +112,14 @@ int launch_waves(int64_t N, int H, int per_simd = WAVES_PER_SIMD) {
     return (int)want;
 }
 
+// The 16-bin angle basis of the reference's lightweight setting (train_jarvis_time.sh: value_pe_angle_real 16).  Its
+// window (ANGLE_RANGE = ceil(8 wscale + 1) >= 9) leaves at most 7 bins out, so the reference evaluates the whole
+// basis (models/kernels/real_enc_frame_proj_fwd_angle.cu:154,168-175: the windowed branch needs more than 8).  The
+// kernels here are compiled for rows of 64 bins: the 16 bins are run as ONE 17-bin window that always starts at bin
+// 0 (bin 16 is a padding bin), with the weights copied into zero-padded rows of 64.
+constexpr int SMALL_ANGLE_BINS = 16;
+constexpr int SMALL_ANGLE_WINDOW = 17;
+
 int check_params(const cfh_params* p) {
     if (!p) return fail(CFH_EINVAL, "params is NULL");
     if (p->struct_size != (int32_t)sizeof(cfh_params))
@@ -122,8 +130,10 @@ int check_params(const cfh_params* p) {
     if (p->head_dim != cfh::DH) return fail(CFH_EINVAL, "head_dim %d not compiled (only %d)", p->head_dim, cfh::DH);
     if (p->dist_bins != 0 && p->dist_bins != cfh::NBINS)
         return fail(CFH_EINVAL, "dist_bins %d not compiled (0 or %d)", p->dist_bins, cfh::NBINS);
-    if (p->angle_bins != 0 && p->angle_bins != cfh::NBINS)
-        return fail(CFH_EINVAL, "angle_bins %d not compiled (0 or %d)", p->angle_bins, cfh::NBINS);
+    if (p->angle_bins != 0 && p->angle_bins != cfh::NBINS && p->angle_bins != SMALL_ANGLE_BINS)
+        return fail(CFH_EINVAL, "angle_bins %d not compiled (0, %d or %d)", p->angle_bins, SMALL_ANGLE_BINS, cfh::NBINS);
+    if (p->angle_bins == SMALL_ANGLE_BINS && !(p->angle_wscale >= 1.0f))
+        return fail(CFH_EINVAL, "angle_bins %d needs angle_wscale >= 1", SMALL_ANGLE_BINS);
     if (p->angle_bins != 0 && p->dist_bins == 0)
         return fail(CFH_EINVAL, "angle encoding requires the distance encoding (dist_bins > 0)");
     if (p->lattice_range < 0 || p->lattice_range > cfh::RMAX)
@@ -141,6 +151,7 @@ int window_widths(const cfh_params* p, int* wl, int* wa) {
     *wl = (int)std::ceil(2.0 * (double)p->dist_wscale * cut + 1.0);
     *wa = (int)std::ceil(2.0 * (double)p->angle_wscale * cut + 1.0);
     const int want_l = cut == 4 ? 9 : 11, want_a = cut == 4 ? 33 : 41;
+    if (p->angle_bins == SMALL_ANGLE_BINS) *wa = want_a;      // the whole basis whatever the scale
     if (p->dist_bins > 0 && *wl != want_l)
         return fail(CFH_EINVAL, "dist_wscale %g gives a %d-bin window; only wscale 1.0 (%d bins) is compiled",
                     (double)p->dist_wscale, *wl, want_l);
@@ -176,6 +187,7 @@ cfh::BasisConsts basis_consts(const cfh_params* p) {
         bc.ang_step = (float)(interval * sinv);
         bc.ang_cc = (float)std::exp2(-2.0 * interval * sinv * interval * sinv);
         bc.ang_mu0 = p->cos_abs ? 0.0f : -1.0f;
+        bc.ang_end_max = A == SMALL_ANGLE_BINS ? (float)SMALL_ANGLE_WINDOW : (float)A;
     }
     return bc;
 }
@@ -349,11 +361,21 @@ int cfh_timing_read(const char* what, double* total_ms, int64_t* launches) {
     return CFH_OK;
 }
 
+}  // extern "C"
+namespace {
+// workspace of the lattice-sum calls: header | item records | per-wavefront weight-gradient partials | six padded
+// (H, Dh, 64) rows for the 16-bin angle basis (three weights, three gradients)
+size_t padded_offset(const cfh_params* p, int64_t N) {
+    const int waves = launch_waves(N > 0 ? N : 1, p->num_heads);
+    return COUNTER_BYTES + items_bytes(N > 0 ? N : 1, p->num_heads) + (size_t)waves * 4 * cfh::DH * cfh::NBINS * sizeof(float);
+}
+}  // namespace
+extern "C" {
+
 size_t cfh_workspace_bytes(const cfh_params* p, int64_t N, int64_t E) {
     (void)E;
     if (check_params(p) != CFH_OK) return 0;
-    const int waves = launch_waves(N > 0 ? N : 1, p->num_heads);
-    return COUNTER_BYTES + items_bytes(N > 0 ? N : 1, p->num_heads) + (size_t)waves * 4 * cfh::DH * cfh::NBINS * sizeof(float);
+    return padded_offset(p, N) + 6 * (size_t)p->num_heads * cfh::DH * cfh::NBINS * sizeof(float);
 }
 
 int cfh_frame_axis1(const cfh_params* p, const float* q, const float* k, const float* a_ih,
@@ -471,6 +493,15 @@ static int framed_pe_forward_impl(const cfh_params* p, const float* q, const flo
         A.counters = F.counters2;
     }
     A.W[0] = W_dist; A.W[1] = W_axis1; A.W[2] = W_axis2; A.W[3] = W_axis3;
+    if (has_ang && p->angle_bins == SMALL_ANGLE_BINS) {      // the 16-bin basis runs on zero-padded copies of its weights
+        const int rows = p->num_heads * cfh::DH, per = rows * cfh::NBINS;
+        const size_t off = padded_offset(p, N);
+        if ((rc = check_workspace(workspace, workspace_bytes, off + 3 * (size_t)per * sizeof(float)))) return rc;
+        float* padded = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + off);
+        hipLaunchKernelGGL(cfh::pad_bins_kernel, dim3((3 * per + 255) / 256), dim3(256), 0, st, W_axis1, W_axis2, W_axis3, rows,
+                           SMALL_ANGLE_BINS, padded);
+        A.W[1] = padded; A.W[2] = padded + per; A.W[3] = padded + 2 * per;
+    }
     A.frames = frames; A.out_z = z; A.out_psi = psi; A.out_d2min = d2min_out; A.shat = shat_out;
     int waves = launch_waves(N, p->num_heads);
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
@@ -486,7 +517,15 @@ static int framed_pe_forward_impl(const cfh_params* p, const float* q, const flo
             else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep);             \
         }                                                                                                       \
     } while (0)
-    if (has_ang) CFH_DISPATCH_FWD(true, true);
+    if (has_ang && p->angle_bins == SMALL_ANGLE_BINS) {
+        if (wide) {
+            if (p->cos_abs) rc = launch_persistent(cfh::framed_pe_fwd_kernel<11, SMALL_ANGLE_WINDOW, true, true, true>, A, &waves, st, what, prep);
+            else rc = launch_persistent(cfh::framed_pe_fwd_kernel<11, SMALL_ANGLE_WINDOW, false, true, true>, A, &waves, st, what, prep);
+        } else {
+            if (p->cos_abs) rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, SMALL_ANGLE_WINDOW, true, true, true>, A, &waves, st, what, prep);
+            else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, SMALL_ANGLE_WINDOW, false, true, true>, A, &waves, st, what, prep);
+        }
+    } else if (has_ang) CFH_DISPATCH_FWD(true, true);
     else if (has_len) CFH_DISPATCH_FWD(true, false);
     else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, false, false>, A, &waves, st, what, prep);
 #undef CFH_DISPATCH_FWD
@@ -556,6 +595,8 @@ int cfh_framed_pe_forward_static(const cfh_params* p, const float* a_ih, const f
         return fail(CFH_EINVAL, "N * num_heads = %lld exceeds the %d (atom, head) items the static scratch holds; "
                     "use cfh_framed_pe_forward with a workspace", (long long)(N * p->num_heads), CFH_STATIC_MAX_ITEMS);
     if (p->collect_stats) return fail(CFH_EINVAL, "collect_stats is not available with the static scratch");
+    if (p->angle_bins == SMALL_ANGLE_BINS && W_axis1)
+        return fail(CFH_EINVAL, "the 16-bin angle basis needs workspace for padded weights: use cfh_framed_pe_forward");
     void* ptr = static_scratch();
     if (!ptr) return CFH_EDEVICE;
     // the work-queue heads are cleared by the prepare kernel of every launch; nothing else must start at zero
@@ -577,7 +618,7 @@ int cfh_frame_axes_framed_pe_forward(const cfh_params* p, const float* q, const 
                                   workspace_bytes, stream);
 }
 
-int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,
+static int framed_pe_backward_impl(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,
                            const float* rvlen, const int64_t* batch, const int64_t* edges,
                            const int64_t* e_start, const int32_t* order, const float* W_dist,
                            const float* W_axis1, const float* W_axis2, const float* W_axis3,
@@ -621,7 +662,7 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
     }
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "framed_pe_backward";
-    if (has_len && shat && !(p->flags & CFH_FLAG_SINGLE_STREAM)) {
+    if (has_len && shat && !(p->flags & CFH_FLAG_SINGLE_STREAM) && p->angle_bins != SMALL_ANGLE_BINS) {
         // The forward kept its histograms and the weight gradients need nothing else: they are summed by a
         // streaming kernel of their own on a second stream while the gather-only kernel, free of their
         // accumulators, computes the gradient of a on this one.
@@ -668,6 +709,20 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
                 rc2 = fail(CFH_ELAUNCH, "join of the second stream failed");
         }
         return rc ? rc : rc2;
+    } else if (has_ang && p->angle_bins == SMALL_ANGLE_BINS) {
+#define CFH_DISPATCH_SMALL(KERNEL)                                                                                   \
+    do {                                                                                                             \
+        if (wide) {                                                                                                  \
+            if (p->cos_abs) rc = launch_persistent(KERNEL<11, SMALL_ANGLE_WINDOW, true, true, true>, A, &waves, st, what);   \
+            else rc = launch_persistent(KERNEL<11, SMALL_ANGLE_WINDOW, false, true, true>, A, &waves, st, what);             \
+        } else {                                                                                                     \
+            if (p->cos_abs) rc = launch_persistent(KERNEL<9, SMALL_ANGLE_WINDOW, true, true, true>, A, &waves, st, what);    \
+            else rc = launch_persistent(KERNEL<9, SMALL_ANGLE_WINDOW, false, true, true>, A, &waves, st, what);              \
+        }                                                                                                            \
+    } while (0)
+        if (shat) CFH_DISPATCH_SMALL(cfh::framed_pe_bwd_saved_kernel);
+        else CFH_DISPATCH_SMALL(cfh::framed_pe_bwd_kernel);
+#undef CFH_DISPATCH_SMALL
     } else if (has_len && shat) {      // the forward kept its histograms: gather-only kernel
         if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_bwd_saved_kernel, true, true);
         else CFH_DISPATCH_PE(cfh::framed_pe_bwd_saved_kernel, true, false);
@@ -685,6 +740,49 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
         rc = finish_launch("gw_reduce");
     }
     return rc;
+}
+
+int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,
+                           const float* rvlen, const int64_t* batch, const int64_t* edges,
+                           const int64_t* e_start, const int32_t* order, const float* W_dist,
+                           const float* W_axis1, const float* W_axis2, const float* W_axis3,
+                           const float* frames, const float* z, const float* gz, const float* gpsi,
+                           const float* shat, int64_t N, int64_t E, int64_t B, float* ga, float* gW_dist,
+                           float* gW_axis1, float* gW_axis2, float* gW_axis3, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+    int rc = check_params(p);
+    if (rc) return rc;
+    const bool small = p->angle_bins == SMALL_ANGLE_BINS && p->dist_bins > 0 && W_dist && W_axis1;
+    if (!small)
+        return framed_pe_backward_impl(p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, W_dist, W_axis1, W_axis2,
+                                       W_axis3, frames, z, gz, gpsi, shat, N, E, B, ga, gW_dist, gW_axis1, gW_axis2,
+                                       gW_axis3, workspace, workspace_bytes, stream);
+    // The 16-bin angle basis: zero-padded copies of the weights in, padded gradient rows out (all on this stream).
+    if (!W_axis2 || !W_axis3) return fail(CFH_EINVAL, "W_axis1..3 must be given together");
+    hipStream_t st = (hipStream_t)stream;
+    const int rows = p->num_heads * cfh::DH, per = rows * cfh::NBINS, per_small = rows * SMALL_ANGLE_BINS;
+    if (N <= 0) {
+        hipLaunchKernelGGL(cfh::zero_outputs_kernel, dim3((per + 255) / 256), dim3(256), 0, st, per, gW_dist, nullptr,
+                           nullptr, nullptr);
+        hipLaunchKernelGGL(cfh::zero_outputs_kernel, dim3((per_small + 255) / 256), dim3(256), 0, st, per_small, gW_axis1,
+                           gW_axis2, gW_axis3, nullptr);
+        return finish_launch("zero_outputs");
+    }
+    const size_t off = padded_offset(p, N);
+    if ((rc = check_workspace(workspace, workspace_bytes, off + 6 * (size_t)per * sizeof(float)))) return rc;
+    float* padded = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + off);
+    float* gpad = padded + 3 * per;
+    hipLaunchKernelGGL(cfh::pad_bins_kernel, dim3((3 * per + 255) / 256), dim3(256), 0, st, W_axis1, W_axis2, W_axis3, rows,
+                       SMALL_ANGLE_BINS, padded);
+    cfh_params q = *p;
+    q.flags |= CFH_FLAG_SINGLE_STREAM;
+    rc = framed_pe_backward_impl(&q, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, W_dist, padded, padded + per,
+                                 padded + 2 * per, frames, z, gz, gpsi, shat, N, E, B, ga, gW_dist, gpad, gpad + per,
+                                 gpad + 2 * per, workspace, workspace_bytes, stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL(cfh::unpad_bins_kernel, dim3((3 * per_small + 255) / 256), dim3(256), 0, st, gpad, rows,
+                       SMALL_ANGLE_BINS, gW_axis1, gW_axis2, gW_axis3);
+    return finish_launch("framed_pe_backward (16-bin angle basis)");
 }
 
 namespace {

@@ -320,6 +320,7 @@ struct BasisConsts {
     float ang_step;          // ang_interval*ang_sigma_inv
     float ang_cc;            // 2^(-2 ang_step^2)
     float ang_mu0;           // centre of bin 0: -1 (cos_abs: 0)
+    float ang_end_max;       // largest window end: the number of angle bins (a 16-bin basis: its 17-bin window, see basis_consts)
 };
 
 // Launch-wide arguments (by value in the kernarg segment).

@@ -138,7 +138,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
                                     float cs = (dx * f[ax][0] + dy * f[ax][1] + dz * f[ax][2]) * rinv;
                                     if (COS_ABS) cs = fabsf(cs);
                                     int end = (int)fminf((cs + bc.ang_end_off) * bc.ang_inv_interval + 1.0f,
-                                                         (float)NBINS);
+                                                         bc.ang_end_max);
                                     end = max(end, WA);
                                     const int start = end - WA;
                                     const float mu_c = bc.ang_mu0 + (float)(start + WA / 2) * bc.ang_interval;
@@ -404,6 +404,28 @@ __global__ __launch_bounds__(256) void zero_outputs_kernel(int n, float* out0, f
     if (out1) out1[idx] = 0.0f;
     if (out2) out2[idx] = 0.0f;
     if (out3) out3[idx] = 0.0f;
+}
+
+// Rows of `bins` values <-> zero-padded rows of NBINS (the kernels are compiled for rows of NBINS bins; a basis of
+// fewer bins runs on padded copies of its weights, and its weight gradients are taken back from padded rows).
+// in/out: three tensors of `rows` rows each; thread per padded element.
+__global__ __launch_bounds__(256) void pad_bins_kernel(const float* __restrict__ w1, const float* __restrict__ w2,
+                                                       const float* __restrict__ w3, int rows, int bins,
+                                                       float* __restrict__ padded) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= 3 * rows * NBINS) return;
+    const int k = idx % NBINS, r = (idx / NBINS) % rows, en = idx / (NBINS * rows);
+    const float* w = en == 0 ? w1 : (en == 1 ? w2 : w3);
+    padded[idx] = k < bins ? w[(size_t)r * bins + k] : 0.0f;
+}
+__global__ __launch_bounds__(256) void unpad_bins_kernel(const float* __restrict__ padded, int rows, int bins,
+                                                         float* __restrict__ g1, float* __restrict__ g2,
+                                                         float* __restrict__ g3) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= 3 * rows * bins) return;
+    const int k = idx % bins, r = (idx / bins) % rows, en = idx / (bins * rows);
+    float* g = en == 0 ? g1 : (en == 1 ? g2 : g3);
+    if (g) g[(size_t)r * bins + k] = padded[((size_t)en * rows + r) * NBINS + k];
 }
 
 }  // namespace cfh

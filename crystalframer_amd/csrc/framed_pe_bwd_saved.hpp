@@ -119,7 +119,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
                                     float cs = (dx * f[ax][0] + dy * f[ax][1] + dz * f[ax][2]) * rinv;
                                     if (COS_ABS) cs = fabsf(cs);
                                     int end = (int)fminf((cs + bc.ang_end_off) * bc.ang_inv_interval + 1.0f,
-                                                         (float)NBINS);
+                                                         bc.ang_end_max);
                                     end = max(end, WA);
                                     const int start = end - WA;
                                     const float mu_c = bc.ang_mu0 + (float)(start + WA / 2) * bc.ang_interval;

@@ -144,7 +144,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                                     float cs = (dx * f[ax][0] + dy * f[ax][1] + dz * f[ax][2]) * rinv;
                                     if (COS_ABS) cs = fabsf(cs);
                                     int end = (int)fminf((cs + bc.ang_end_off) * bc.ang_inv_interval + 1.0f,
-                                                         (float)NBINS);
+                                                         bc.ang_end_max);
                                     end = max(end, WA);
                                     const int start = end - WA;
                                     const float mu_c = bc.ang_mu0 + (float)(start + WA / 2) * bc.ang_interval;

@@ -61,13 +61,17 @@ def compile_kernels(lattice_range: int, head_num: int, key_head_dim: int, value_
     the compiled instantiations."""
     if key_head_dim != 16 or value_head_dim != 16:
         raise NotImplementedError(f"head dims ({key_head_dim},{value_head_dim}): only 16 is compiled")
-    if value_pe_dim not in (0, 64) or dim_angle_enc not in (0, 64):
+    if value_pe_dim not in (0, 64) or dim_angle_enc not in (0, 16, 64):
         raise NotImplementedError(f"value_pe_dist_real={value_pe_dim}, value_pe_angle_real={dim_angle_enc}: "
-                                  "only 0 or 64 bins are compiled")
+                                  "compiled are 0 or 64 distance bins and 0, 16 or 64 angle bins")
     if value_pe_dim > 0 and float(value_pe_dist_wscale) != 1.0:
         raise NotImplementedError("value_pe_dist_wscale: only 1.0 is compiled")
-    if dim_angle_enc > 0 and float(value_pe_angle_wscale) != 4.0:
-        raise NotImplementedError("value_pe_angle_wscale: only 4.0 is compiled")
+    if dim_angle_enc == 64 and float(value_pe_angle_wscale) != 4.0:
+        raise NotImplementedError("value_pe_angle_wscale: only 4.0 is compiled for 64 angle bins")
+    if dim_angle_enc == 16 and float(value_pe_angle_wscale) < 1.0:
+        # the 16-bin basis of the reference's lightweight setting (train_jarvis_time.sh:40-57) is evaluated whole,
+        # as the reference does for it (its window leaves at most 7 bins out)
+        raise NotImplementedError("value_pe_angle_wscale: at least 1.0 for 16 angle bins")
     KernelManager.LATTICE_RANGE = int(lattice_range)
     KernelManager.MINIMUM_RANGE = int(lattice_range) if set_minimum_range else 0
     KernelManager.SYMM_BREAK_NOISE = float(symm_break_noise)

@@ -61,8 +61,15 @@ def test_compile_kernels_validates_constants():
     assert cuda_funcs.KernelManager.LATTICE_RANGE == 3 and cuda_funcs.KernelManager.MINIMUM_RANGE == 0
     with pytest.raises(NotImplementedError):
         cuda_funcs.compile_kernels(2, 8, 32, 64, 64, 32, True, 0, 1.0, 4.0, 1.0, 1.0, 1e-5)
+    # the 16-bin angle basis of the lightweight setting (train_jarvis_time.sh:40-57) and the default's scale with it
+    cuda_funcs.compile_kernels(2, 8, 16, 64, 16, 16, True, 0, 1.0, 1.0, 1.5, 6.0, 1e-5)
+    cuda_funcs.compile_kernels(2, 8, 16, 64, 16, 16, True, 1, 1.0, 4.0, 1.0, 1.0, 1e-5)
     with pytest.raises(NotImplementedError):
-        cuda_funcs.compile_kernels(2, 8, 16, 64, 16, 16, True, 0, 1.0, 1.0, 1.0, 1.0, 1e-5)
+        cuda_funcs.compile_kernels(2, 8, 16, 64, 32, 16, True, 0, 1.0, 4.0, 1.0, 1.0, 1e-5)      # 32 angle bins
+    with pytest.raises(NotImplementedError):
+        cuda_funcs.compile_kernels(2, 8, 16, 64, 64, 16, True, 0, 1.0, 1.0, 1.0, 1.0, 1e-5)      # 64 bins, scale 1
+    with pytest.raises(NotImplementedError):
+        cuda_funcs.compile_kernels(2, 8, 16, 64, 16, 16, True, 0, 1.0, 0.5, 1.0, 1.0, 1e-5)      # 16 bins, scale < 1
     cuda_funcs.compile_kernels(2, 8, 16, 64, 64, 16, True, 0, 1.0, 4.0, 1.0, 1.0, 1e-5)
 
 
