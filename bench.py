@@ -4,11 +4,11 @@
 One "step" is one training step (forward, MSE loss, backward, AdamW update) of the 4-layer
 CrystalFramer max-frame model over one batch of 256 synthetic crystals that is already resident in
 HBM (configuration C3: the 4-layer max-frame model at batch 256; fp32, random-init weights).  Prints ONE JSON line with
-crystals/s, the roofline figures of the dominant kernel measured with HIP events inside the timed
-steps, and the CPU baseline (the PyTorch restatement of the reference's pure-PyTorch formulation,
-timed on the host cores on a bounded sample of the same batch).
+crystals/s, the roofline figures of the dominant kernel measured with HIP events inside the library,
+the other large configurations (C2, C4, C5) timed the same way, and the CPU baseline (the PyTorch restatement of
+the reference's pure-PyTorch formulation, timed on the host cores on a bounded sample of the same batch).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-other-configs]
 """
 from __future__ import annotations
 
@@ -29,21 +29,18 @@ sys.path.insert(0, ROOT)
 WL, WA = 9, 33
 F_FWD = 56 + 4 * WL + 12 * WA          # 488 flop per term
 F_BWD = 61 + 6 * WL + 18 * WA          # 709 flop per term
+F_FWD_DIST = 23 + 3 + 3 + 4 * WL       # distance encoding alone (no cosines, one window): 65 flop per term
 X_TERM = 1 + WL + 3 * WA               # 109 exp per term, forward and backward alike
-F_FRAME = 87                           # three frame-search sweeps
-EPI_FWD = 4 * 2 * 16 * 64              # projection epilogue per (pair, head)
+EPI_FWD = 4 * 2 * 16 * 64              # projection epilogue per (pair, head), four encodings
+EPI_FWD_DIST = 2 * 16 * 64             # one encoding
 PEAK_FP32_TFLOPS = 157.3               # published MI355X FP32 vector peak (packed FMA)
 PEAK_FP32_UNPACKED = 78.6              # 256 CU x 64 lanes x 2 flop x 2.4 GHz, packed FP32 not used
 PEAK_TRANS_TOPS = 9.8                  # quarter-rate transcendental unit
-# HBM bytes per launch of the dominant kernel on this workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch) scaled by what the same counters read for the 256 MiB device copy of --calibrate-copy
-# (FETCH_SIZE reads 128 MiB for it: factor 2.0; WRITE_SIZE reads 256 MiB: factor 1.0); see profiles/.
-# With the forward keeping its window histograms for the backward (KernelManager.SAVE_HISTOGRAMS, the default):
-# forward 3 398 KiB x 2.0 fetched + 261 810 KiB written (243.9 MB of that are the histograms, E x H x 4 x 64
-# floats); backward: the gather-only kernel 25 477 KiB x 2.0 fetched and under 2 MB written, the weight-gradient
-# kernel beside it on the second stream 133 999 KiB x 2.0 fetched (the histograms again) + 16 384 KiB written (its
-# per-wavefront partials).
-TRAFFIC_BYTES_PER_LAUNCH = {"framed_pe_backward": 52.2e6 + 291.2e6, "framed_pe_forward": 275.0e6}
+# HBM bytes per launch on the headline workload (batch 256, 64 + 64 bins, fused attention core), from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for the 256 MiB device copy of
+# --calibrate-copy; the figures and the commands are in TRAFFIC_SOURCE.  Other batch sizes or settings: null.
+TRAFFIC_SOURCE = "profiles/fused_core_hbm_traffic_C3.md"
+TRAFFIC_BYTES_PER_LAUNCH = {"fused_core_forward": None, "fused_core_backward": None, "frame_axes": None}
 
 
 def parse():
@@ -53,17 +50,26 @@ def parse():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the timed runs of C2, C4 and C5")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (reference point for HBM traffic counters)")
     ap.add_argument("--no-fused-adamw", action="store_true", help="PyTorch's multi-tensor AdamW instead of the fused kernel")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch every kernel from Python instead of replaying the step as one HIP graph")
-    ap.add_argument("--cpu-crystals", type=int, default=12, help="crystals of the batch in the CPU sample")
+    ap.add_argument("--two-step-core", action="store_true",
+                    help="the reference's sequence of operators (lattice sums, then softmax attention) instead of "
+                         "the fused attention core")
+    ap.add_argument("--no-stats", action="store_true",
+                    help="skip the passes that count lattice terms (their counters add atomics to the kernels, which a "
+                         "profile of the kernels should not see); the roofline object is then null")
+    ap.add_argument("--cpu-crystals", type=int, default=32, help="crystals of the batch in the CPU sample")
+    ap.add_argument("--cpu-repeats", type=int, default=5, help="timed repetitions of the CPU sample (median)")
     return ap.parse_args()
 
 
-def cpu_baseline(model, cb, mp, ncrys: int):
-    """Forward + backward of the same model on the first ``ncrys`` crystals with the CPU oracle."""
+def cpu_baseline(model, cb, mp, ncrys: int, repeats: int):
+    """Forward + backward of the same model on the first ``ncrys`` crystals with the CPU oracle in the
+    pure-PyTorch formulation of the reference (untruncated Gaussian bases)."""
     from oracle import cpu_model
     from crystalframer_amd.synthetic import CrystalBatch
     nat = int(cb.sizes[:ncrys].sum())
@@ -74,19 +80,155 @@ def cpu_baseline(model, cb, mp, ncrys: int):
     torch.set_num_threads(cores)
     target = torch.zeros(ncrys, 1)
     times = []
-    for rep in range(3):
+    for rep in range(repeats + 1):
         leaves = {k: v.clone().requires_grad_(v.dtype.is_floating_point and "scale" not in k) for k, v in sd.items()}
         t0 = time.perf_counter()
-        out = cpu_model.model_forward(leaves, sample, mp, dtype=torch.float32)
+        out = cpu_model.model_forward(leaves, sample, mp, dtype=torch.float32, windows="full")
         loss = torch.nn.functional.mse_loss(out, target)
         loss.backward()
         times.append(time.perf_counter() - t0)
-    t = sorted(times[1:])[len(times[1:]) // 2] if len(times) > 1 else times[0]
+    t = sorted(times[1:])[len(times[1:]) // 2]
     pairs = int((sample.sizes ** 2).sum())
+    pairs_per_crystal_batch = float((cb.sizes.double() ** 2).mean())
     return {"value": ncrys / t, "unit": "crystals/s", "cores": cores, "kind": "port",
-            "sample": f"first {ncrys} crystals of the batch ({nat} atoms, {pairs} atom pairs), 4-layer fwd+bwd, "
-                      f"fp32 PyTorch restatement of the pure-PyTorch formulation, median of {len(times) - 1} after 1 warm-up",
+            "sample": f"first {ncrys} crystals of the batch ({nat} atoms, {pairs} atom pairs = {pairs / ncrys:.0f} per "
+                      f"crystal; the whole batch has {pairs_per_crystal_batch:.0f} per crystal), 4-layer fwd+bwd, fp32 "
+                      f"PyTorch restatement of the pure-PyTorch formulation (full Gaussian bases), median of "
+                      f"{repeats} after 1 warm-up",
             "seconds_per_step": t}
+
+
+def graphed(fn, warmup: int):
+    """Capture ``fn`` (after ``warmup`` eager runs on the capture stream) and return the replay callable."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(max(warmup, 3)):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):      # the stream of the warm-up: its library workspace is reused
+        fn()
+    for _ in range(2):
+        graph.replay()
+    torch.cuda.synchronize()
+    return graph.replay
+
+
+def timed(run, steps: int) -> float:
+    """Seconds per call of ``run`` over exactly ``steps`` calls, device idle before and after."""
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+KERNELS = ("frame_axes", "framed_pe_forward", "framed_pe_backward", "fused_core_forward", "fused_core_backward")
+
+
+def instrumented(fn, nprof: int, dev, count_terms: bool = True):
+    """Run ``fn`` eagerly ``nprof`` times with the library's own HIP events around its lattice kernels and around
+    every library call, then ``nprof`` times with the term counters.  Kept out of every timed region."""
+    import crystalframer_amd as cf
+    from crystalframer_amd import _lib
+    KM = cf.KernelManager
+    for what in KERNELS:                    # drop what earlier runs recorded
+        _lib.read_kernel_timing(what)
+    KM.EVENT_LOG = []
+    _lib.kernel_timing(True)
+    for _ in range(nprof):
+        fn()
+    torch.cuda.synchronize()
+    _lib.kernel_timing(False)
+    log, KM.EVENT_LOG = KM.EVENT_LOG, None
+    kern_ms, kern_launches = {}, {}
+    for what in KERNELS:
+        total, count = _lib.read_kernel_timing(what)
+        if count:
+            kern_ms[what] = total / count
+            kern_launches[what] = count // nprof
+    stats = None
+    if count_terms:
+        KM.COLLECT_STATS = True
+        _lib.read_stats(dev, reset=True)
+        for _ in range(nprof):
+            fn()
+        torch.cuda.synchronize()
+        KM.COLLECT_STATS = False
+        stats = {k: v / nprof for k, v in _lib.read_stats(dev, reset=True).items() if not isinstance(v, list)}
+    calls = {}
+    for name, s, e in log:
+        calls.setdefault(name, []).append(s.elapsed_time(e))
+    return kern_ms, kern_launches, stats, calls
+
+
+def lattice_roofline(kern_ms, kern_launches, stats, angle: bool):
+    """Algorithmic flop of the reference formulation for the terms actually evaluated, per launch of the forward and
+    of the backward lattice-sum kernel, over the kernel's own duration."""
+    fwd = "fused_core_forward" if "fused_core_forward" in kern_ms else "framed_pe_forward"
+    bwd = "fused_core_backward" if "fused_core_backward" in kern_ms else "framed_pe_backward"
+    f_fwd, epi = (F_FWD, EPI_FWD) if angle else (F_FWD_DIST, EPI_FWD_DIST)
+    out = {}
+    if fwd in kern_ms:
+        n = max(1, kern_launches[fwd])
+        t = kern_ms[fwd] * 1e-3
+        flop = stats["fwd_evaluated"] / n * f_fwd + stats["fwd_pairs"] / n * epi
+        out["forward"] = {"kernel": fwd + "_kernel", "avg_launch_ms": kern_ms[fwd], "achieved": flop / t / 1e12,
+                          "frac": flop / t / 1e12 / PEAK_FP32_TFLOPS, "terms_evaluated_per_launch": stats["fwd_evaluated"] / n,
+                          "terms_in_box_per_launch": stats["fwd_in_box"] / n, "flop_per_launch": flop}
+    if bwd in kern_ms and angle:
+        n = max(1, kern_launches[bwd])
+        t = kern_ms[bwd] * 1e-3
+        flop = stats["bwd_evaluated"] / n * F_BWD + stats["bwd_pairs"] / n * 2 * EPI_FWD
+        out["backward"] = {"kernel": bwd + "_kernel", "avg_launch_ms": kern_ms[bwd], "achieved": flop / t / 1e12,
+                           "frac": flop / t / 1e12 / PEAK_FP32_TFLOPS, "terms_evaluated_per_launch": stats["bwd_evaluated"] / n,
+                           "terms_in_box_per_launch": stats["bwd_in_box"] / n, "flop_per_launch": flop}
+    return out
+
+
+def other_config(name: str, dev, *, layers: int, backward: bool, angle_bins: int, steps: int):
+    """One of the large configurations beside the headline one: the step as one HIP graph, timed by the host clock
+    around ``steps`` replays; then the lattice kernels' own durations and term counts from instrumented eager runs."""
+    from crystalframer_amd import latticeformer, params, synthetic
+    torch.manual_seed(11)
+    mp = params.ModelParams(num_layers=layers, value_pe_angle_real=angle_bins)
+    model = latticeformer.Latticeformer(mp).to(dev)
+    cb_cpu = synthetic.make_config(name, seed=123)
+    cb = cb_cpu.to(dev)
+    model.train()
+    with torch.no_grad():
+        model(cb)               # the first training-mode pass measures and stores the normalisation of alpha
+    model.train(backward)
+    B = cb_cpu.num_crystals
+    target = torch.randn(B, 1, generator=torch.Generator().manual_seed(7)).to(dev)
+    sink = torch.zeros((), device=dev)
+
+    if backward:
+        def fn():
+            model.zero_grad(set_to_none=True)
+            loss = torch.nn.functional.mse_loss(model(cb), target)
+            loss.backward()
+            sink.copy_(loss.detach())
+    else:
+        def fn():
+            with torch.no_grad():
+                sink.copy_(model(cb).sum())
+    run = graphed(fn, 2)
+    sec = timed(run, steps)
+    kern_ms, kern_launches, stats, _ = instrumented(fn, 2, dev)
+    roof = lattice_roofline(kern_ms, kern_launches, stats, angle_bins > 0)
+    slow = max(roof.values(), key=lambda r: r["avg_launch_ms"]) if roof else None
+    return {"workload": f"{name}: {B} crystals, {int(cb_cpu.pos.shape[0])} atoms, {int((cb_cpu.sizes ** 2).sum())} atom pairs; "
+                        f"{layers}-layer max-frame model ({'64 + %d bins' % angle_bins if angle_bins else '64 distance bins, no angle encoding'}), "
+                        f"{'forward + backward' if backward else 'forward only'}, one HIP graph per pass",
+            "ms": sec * 1e3, "crystals_per_s": B / sec, "steps": steps,
+            "lattice_kernel_ms": kern_ms,
+            "lattice_kernel_frac": {k: r["frac"] for k, r in roof.items()},
+            "slowest_lattice_kernel": None if slow is None else {"kernel": slow["kernel"], "frac": slow["frac"],
+                                                                 "achieved_tflops": slow["achieved"]}}
 
 
 def main():
@@ -99,8 +241,10 @@ def main():
         print("bench.py needs a HIP device", file=sys.stderr)
         sys.exit(2)
     import crystalframer_amd as cf
-    from crystalframer_amd import _lib, latticeformer, params, synthetic
+    from crystalframer_amd import attention, latticeformer, params, synthetic
     KM = cf.KernelManager
+    if args.two_step_core:
+        attention.FUSED_CORE = False
 
     dev = torch.device("cuda:0")
     torch.manual_seed(123)
@@ -131,19 +275,7 @@ def main():
     if use_graph:
         # the whole training step (geometry, 4 layers forward, loss, backward, AdamW) as ONE HIP graph:
         # Python cannot issue the step's launches as fast as the GPU retires them
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(max(args.warmup, 3)):
-                step()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):      # the stream of the warm-up: its library workspace is reused
-            step()
-        run_step = graph.replay
-        for _ in range(2):
-            run_step()
+        run_step = graphed(step, args.warmup)
     else:
         run_step = step
         for _ in range(args.warmup):
@@ -160,84 +292,55 @@ def main():
     ms_per_step = dt / args.steps * 1e3
     crystals_per_s = args.batch / (dt / args.steps)
 
-    # ---- a second, instrumented pass over the same steps: HIP events around every library call on
-    #      its stream, and term counters; kept out of the timed region so that it cannot perturb it
-    KM.EVENT_LOG = []
-    _lib.kernel_timing(True)          # the library's own event bracket around each lattice-sum kernel
+    # ---- instrumented passes over the same step, outside the timed region
     nprof = min(args.steps, 5)
-    for _ in range(nprof):
-        step()
-    torch.cuda.synchronize()
-    _lib.kernel_timing(False)
-    log, KM.EVENT_LOG = KM.EVENT_LOG, None
-    kern_ms = {}
-    for what in ("frame_axes", "framed_pe_forward", "framed_pe_backward", "fused_core_forward", "fused_core_backward"):
-        total, count = _lib.read_kernel_timing(what)
-        if count:
-            kern_ms[what] = total / count
-    # ---- and a third one that counts translations (separately: the counters add a few atomics)
-    KM.COLLECT_STATS = True
-    _lib.read_stats(dev, reset=True)
-    for _ in range(nprof):
-        step()
-    torch.cuda.synchronize()
-    KM.COLLECT_STATS = False
-    stats = _lib.read_stats(dev, reset=True)
-    per_kernel = {}
-    for name, s, e in log:
-        per_kernel.setdefault(name, []).append(s.elapsed_time(e))
-    avg_ms = {k: sum(v) / len(v) for k, v in per_kernel.items()}
-    launches = {k: len(v) // nprof for k, v in per_kernel.items()}
-    lib_ms_per_step = sum(sum(v) for v in per_kernel.values()) / nprof
-
+    kern_ms, kern_launches, stats, calls = instrumented(step, nprof, dev, count_terms=not args.no_stats)
+    avg_ms = {k: sum(v) / len(v) for k, v in calls.items()}
+    launches = {k: len(v) // nprof for k, v in calls.items()}
+    lib_ms_per_step = sum(sum(v) for v in calls.values()) / nprof
+    if args.calibrate_copy:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+    if stats is None:
+        print(json.dumps({"metric": f"crystals/s fwd+bwd, 4-layer max-frame, batch {args.batch}", "value": crystals_per_s,
+                          "unit": "crystals/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                          "ms_per_step": ms_per_step, "higher_is_better": True, "roofline": None,
+                          "lattice_kernel_ms": kern_ms, "library_call_ms": avg_ms}))
+        return
+    roof = lattice_roofline(kern_ms, kern_launches, stats, True)
+    dom = max(roof.values(), key=lambda r: r["avg_launch_ms"])
     fused = "fused_core_forward" in kern_ms
-    if fused:
-        kern_ms["framed_pe_forward"] = kern_ms["fused_core_forward"]
-        kern_ms["framed_pe_backward"] = kern_ms["fused_core_backward"]
-    nlaunch_bwd = max(1, len(per_kernel.get("framed_pe_backward", [])) + len(per_kernel.get("fused_core_backward", [])))
-    nlaunch_fwd = max(1, len(per_kernel.get("framed_pe_forward", [])) + len(per_kernel.get("frame_axes_framed_pe_forward", []))
-                      + len(per_kernel.get("fused_core_forward", [])))
-    bwd_eval = stats["bwd_evaluated"] / nlaunch_bwd          # terms evaluated per launch
-    bwd_box = stats["bwd_in_box"] / nlaunch_bwd              # terms in the reference's boxes per launch
-    bwd_pairs = stats["bwd_pairs"] / nlaunch_bwd
-    fwd_eval = stats["fwd_evaluated"] / nlaunch_fwd
-    fwd_box = stats["fwd_in_box"] / nlaunch_fwd
-    fwd_pairs = stats["fwd_pairs"] / nlaunch_fwd
-    t_bwd = kern_ms.get("framed_pe_backward", float("nan")) * 1e-3
-    t_fwd = kern_ms.get("framed_pe_forward", float("nan")) * 1e-3
-    flop_bwd = bwd_eval * F_BWD + bwd_pairs * 2 * EPI_FWD    # terms actually evaluated + epilogues
-    flop_fwd = fwd_eval * F_FWD + fwd_pairs * EPI_FWD
-    dominant = "framed_pe_backward" if t_bwd >= t_fwd else "framed_pe_forward"
-    flop_dom, t_dom, eval_dom = (flop_bwd, t_bwd, bwd_eval) if dominant == "framed_pe_backward" else (flop_fwd, t_fwd, fwd_eval)
-    achieved = flop_dom / t_dom / 1e12
+    traffic = TRAFFIC_BYTES_PER_LAUNCH.get(dom["kernel"][:-len("_kernel")]) if (args.batch == 256 and fused) else None
     roofline = {
-        "kernel": dominant + "_kernel", "bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS,
-        "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_TFLOPS, "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
-        "bound_detail": "FP32 arithmetic (vector + a little MFMA) against the published 157.3 TFLOP/s; HBM traffic "
-                        "(the kept window histograms) runs at 15-18 % of the HBM peak; in practice the forward is "
-                        "limited by LDS atomic throughput and bank conflicts, the backward (a gather-only kernel "
-                        "with the weight-gradient kernel beside it on a second stream) by instruction issue",
-        "both_kernels": {
-            "framed_pe_forward": {"achieved": flop_fwd / t_fwd / 1e12, "frac": flop_fwd / t_fwd / 1e12 / PEAK_FP32_TFLOPS,
-                                  "avg_launch_ms": t_fwd * 1e3},
-            # the gather-only kernel's duration; the weight-gradient kernel (its share of the flop: one projection
-            # epilogue per (pair, head)) runs inside that time on the second stream
-            "framed_pe_backward": {"achieved": flop_bwd / t_bwd / 1e12, "frac": flop_bwd / t_bwd / 1e12 / PEAK_FP32_TFLOPS,
-                                   "avg_launch_ms": t_bwd * 1e3},
-        },
-        "frac_of_unpacked_fp32_peak": achieved / PEAK_FP32_UNPACKED,
-        "transcendental_frac": eval_dom * X_TERM / t_dom / 1e12 / PEAK_TRANS_TOPS,
-        "avg_launch_ms": t_dom * 1e3,
-        "terms_evaluated_per_launch": eval_dom,
+        "kernel": dom["kernel"], "bound": "valu-issue/latency",
+        "achieved": dom["achieved"], "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac"], "traffic": traffic,
+        "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
+        "bound_detail": "ALGORITHMIC FP32 flop of the reference formulation (what its kernels would execute for the terms "
+                        "this kernel evaluates) against the published 157.3 TFLOP/s vector peak.  The kernel does not "
+                        "execute that many: the angle encoding is scattered as 5 local moments per axis instead of a "
+                        "33-bin window and the projection runs once per (atom, head) in a separate MFMA kernel.  What "
+                        "binds it is instruction issue and latency of small work items (one wavefront per (atom, "
+                        "head), 12.5 pairs on average): vector ALU busy about half of the time, HBM far from its peak",
+        "both_kernels": {k: {"kernel": r["kernel"], "achieved": r["achieved"], "frac": r["frac"],
+                             "avg_launch_ms": r["avg_launch_ms"]} for k, r in roof.items()},
+        "frac_of_unpacked_fp32_peak": dom["achieved"] / PEAK_FP32_UNPACKED,
+        "transcendental_frac": dom["terms_evaluated_per_launch"] * X_TERM / (dom["avg_launch_ms"] * 1e-3) / 1e12 / PEAK_TRANS_TOPS,
+        "avg_launch_ms": dom["avg_launch_ms"],
+        "terms_evaluated_per_launch": dom["terms_evaluated_per_launch"],
         "note": "algorithmic flop of the reference formulation (709 bwd / 488 fwd per term, 109 exp) x terms "
-                "actually evaluated after pruning, + projection epilogues; duration from HIP events recorded by "
-                "the library around this kernel alone, on the stream it is launched on",
+                "actually evaluated after pruning, + one projection epilogue per (pair, head) and encoding (two for the "
+                "backward); duration from HIP events recorded by the library around this kernel alone, on the stream it "
+                "is launched on",
     }
-    terms = {
-        "forward_terms_in_box_per_s": fwd_box / t_fwd, "forward_terms_evaluated_per_s": fwd_eval / t_fwd,
-        "backward_terms_in_box_per_s": bwd_box / t_bwd, "backward_terms_evaluated_per_s": bwd_eval / t_bwd,
-        "evaluated_fraction": fwd_eval / max(1.0, fwd_box),
-    }
+    terms = {}
+    for k, r in roof.items():
+        t = r["avg_launch_ms"] * 1e-3
+        terms[k + "_terms_in_box_per_s"] = r["terms_in_box_per_launch"] / t
+        terms[k + "_terms_evaluated_per_s"] = r["terms_evaluated_per_launch"] / t
+    if "forward" in roof:
+        terms["evaluated_fraction"] = roof["forward"]["terms_evaluated_per_launch"] / max(1.0, roof["forward"]["terms_in_box_per_launch"])
 
     result = {
         "metric": f"crystals/s fwd+bwd, 4-layer max-frame, batch {args.batch}",
@@ -249,7 +352,9 @@ def main():
                    "global_batch": args.batch, "atoms": int(cb.pos.shape[0]),
                    "atom_pairs": int((cb_cpu.sizes ** 2).sum()), "heads": 8, "head_dim": 16,
                    "dist_bins": 64, "angle_bins": 64, "adaptive_cutoff_sigma": -3.5, "prune_log2": KM.PRUNE_LOG2,
-                   "windows": "reference (9/33 bins)", "optimizer": "adamw", "parallelism": "single GPU",
+                   "attention_core": "fused (one histogram per (atom, head))" if fused else "two-step (reference's operators)",
+                   "windows": "distance 9 bins, angle basis untruncated" if fused else "reference (9/33 bins)",
+                   "optimizer": "adamw", "parallelism": "single GPU",
                    "launch": "one HIP graph per step" if use_graph else "eager"},
         "final_loss": final_loss,
         "roofline": roofline,
@@ -258,13 +363,18 @@ def main():
         "library_ms_per_step": lib_ms_per_step,
     }
     if args.calibrate_copy:
-        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
         result["calibrate_copy_bytes"] = int(src.numel() * 4)
+    if not args.no_other_configs:
+        # the other large configurations, each timed by this process's clock around graph replays
+        del opt
+        other = {}
+        other["C2"] = other_config("C2", dev, layers=1, backward=True, angle_bins=64, steps=20)
+        other["C4"] = other_config("C4", dev, layers=1, backward=True, angle_bins=64, steps=10)
+        other["C5"] = other_config("C5", dev, layers=4, backward=False, angle_bins=64, steps=10)
+        other["C5_no_angle"] = other_config("C5", dev, layers=4, backward=False, angle_bins=0, steps=10)
+        result["other_configs"] = other
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(model, cb_cpu, mp, min(args.cpu_crystals, args.batch))
+        result["cpu_baseline"] = cpu_baseline(model, cb_cpu, mp, min(args.cpu_crystals, args.batch), args.cpu_repeats)
     print(json.dumps(result))
 
 
