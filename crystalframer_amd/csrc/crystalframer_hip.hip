@@ -1201,8 +1201,9 @@ CoreBuffers fill_core(cfh::CoreArgs& C, const cfh_params* p, const CoreLayout& L
 }
 // one wavefront (= workgroup) per (item, head); the hardware deals them to the compute units as slots free up
 template <typename Kern>
-int launch_core(Kern kern, const cfh::CoreArgs& C, hipStream_t st, const char* what) {
-    const unsigned blocks = (unsigned)C.K.N * (unsigned)C.K.H;
+int launch_core(Kern kern, const cfh::CoreArgs& C, hipStream_t st, const char* what, unsigned waves = 0) {
+    if (waves == 0) waves = (unsigned)C.K.N * (unsigned)C.K.H;
+    const unsigned blocks = (waves + cfh::CORE_WPB - 1) / cfh::CORE_WPB;
     bool timed = false;
     TimedLaunch t;
     {
@@ -1214,7 +1215,7 @@ int launch_core(Kern kern, const cfh::CoreArgs& C, hipStream_t st, const char* w
         timed = hipEventCreate(&t.start) == hipSuccess && hipEventCreate(&t.stop) == hipSuccess &&
                 hipEventRecord(t.start, st) == hipSuccess;
     }
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(cfh::WAVE), 0, st, C);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(cfh::WAVE * cfh::CORE_WPB), 0, st, C);
     if (timed && hipEventRecord(t.stop, st) == hipSuccess) {
         std::lock_guard<std::mutex> lock(g_timing_mutex);
         g_timed.push_back(t);
@@ -1281,7 +1282,31 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
             F.K.counters2 = reinterpret_cast<int32_t*>(ws + QUEUE_OFFSET + QUEUE_SET_BYTES);
             F.K.frames_to_records = 1;
             hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, F.K, 1);
-            if ((rc = launch_core(cfh::frame_axes_sorted_kernel, F, st, "frame_axes"))) return rc;
+            if (F.sorted_tab) {
+                // four heads of an atom per wavefront for the items with the usual box and short rows, the others one
+                // by one, all in one launch
+                const unsigned item_blocks = ((unsigned)N * (unsigned)p->num_heads + cfh::CORE_WPB - 1) / cfh::CORE_WPB;
+                const unsigned quad_waves = (unsigned)N * (unsigned)((p->num_heads + cfh::FQ_ROWS - 1) / cfh::FQ_ROWS);
+                const unsigned quad_blocks = (quad_waves + cfh::CORE_WPB - 1) / cfh::CORE_WPB;
+                bool timed = false;
+                TimedLaunch t;
+                {
+                    std::lock_guard<std::mutex> lock(g_timing_mutex);
+                    timed = g_timing_on;
+                }
+                if (timed) {
+                    t.what = "frame_axes";
+                    timed = hipEventCreate(&t.start) == hipSuccess && hipEventCreate(&t.stop) == hipSuccess &&
+                            hipEventRecord(t.start, st) == hipSuccess;
+                }
+                hipLaunchKernelGGL(cfh::frame_axes_kernel, dim3(item_blocks + quad_blocks), dim3(cfh::WAVE * cfh::CORE_WPB), 0,
+                                   st, F, (int)item_blocks);
+                if (timed && hipEventRecord(t.stop, st) == hipSuccess) {
+                    std::lock_guard<std::mutex> lock(g_timing_mutex);
+                    g_timed.push_back(t);
+                }
+                if ((rc = finish_launch("frame_axes"))) return rc;
+            } else if ((rc = launch_core(cfh::frame_axes_sorted_kernel, F, st, "frame_axes"))) return rc;
             C.K.counters = F.K.counters2;
         } else {
             C.K.frames = has_ang ? frames : nullptr;

@@ -442,6 +442,10 @@ __device__ __forceinline__ Item unpack_item(uint32_t rec) {
     for (int d = 0; d < 9; d++) t.L.t[d] = rec_f(rec, REC_LATTICE + d);
     return t;
 }
+// the same for a wavefront that is not the first of its workgroup
+__device__ __forceinline__ uint32_t load_record_lane(const KernelArgs& P, int it, int h, int lane) {
+    return (it >= 0 && lane < REC_WORDS) ? P.items[((size_t)it * P.H + h) * REC_WORDS + lane] : 0u;
+}
 __device__ __forceinline__ uint32_t load_record(const KernelArgs& P, int it, int h) {
     return (it >= 0 && threadIdx.x < REC_WORDS) ? P.items[((size_t)it * P.H + h) * REC_WORDS + threadIdx.x] : 0u;
 }

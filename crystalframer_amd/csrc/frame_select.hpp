@@ -43,6 +43,26 @@ __device__ __forceinline__ void shift_of(int t, const Box& bx, const Lattice& L,
     vz = fmaf(L.t[8], n3, fmaf(L.t[5], n2, L.t[2] * n1));
 }
 
+// The last steps of every frame search, written once and without contraction of multiply-add pairs, so that every
+// kernel that searches frames rounds them alike (their results are compared bit for bit).
+#pragma clang fp contract(off)
+// unit vector of (x, y, z)
+__device__ __forceinline__ void unit_vector(float& x, float& y, float& z) {
+    const float inv = 1.0f / sqrtf((x * x + y * y) + z * z);
+    x = x * inv; y = y * inv; z = z * inv;
+}
+// Gram-Schmidt and cross product (models/indexed_lattice_multi_head_attention_cuda.py:475-481; F.normalize eps 1e-12):
+// g = normalised part of f2 orthogonal to f1, h = f1 x g
+__device__ __forceinline__ void orthonormal_axes(float f1x, float f1y, float f1z, float f2x, float f2y, float f2z,
+                                                 float& gx, float& gy, float& gz, float& hx, float& hy, float& hz) {
+    const float dot = (f1x * f2x + f1y * f2y) + f1z * f2z;
+    gx = f2x - dot * f1x; gy = f2y - dot * f1y; gz = f2z - dot * f1z;
+    const float inv = 1.0f / fmaxf(sqrtf((gx * gx + gy * gy) + gz * gz), 1e-12f);
+    gx = gx * inv; gy = gy * inv; gz = gz * inv;
+    hx = f1y * gz - f1z * gy; hy = f1z * gx - f1x * gz; hz = f1x * gy - f1y * gx;
+}
+#pragma clang fp contract(fast)
+
 // best candidate of a wavefront: largest score, then lowest pair, then lowest translation
 struct Best { float score; int e; int t; };
 __device__ __forceinline__ bool better(float s1, int e1, int t1, float s2, int e2, int t2) {
@@ -309,8 +329,7 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                     vy = uniform_f(P.rpos[(size_t)best.e * 3 + 1]) + sy;
                     vz = uniform_f(P.rpos[(size_t)best.e * 3 + 2]) + sz;
                 }
-                const float inv = 1.0f / sqrtf(vx * vx + vy * vy + vz * vz);
-                vx *= inv; vy *= inv; vz *= inv;
+                unit_vector(vx, vy, vz);
             }
             if (pass == 0) { f1x = vx; f1y = vy; f1z = vz; }
             else { f2x = vx; f2y = vy; f2z = vz; }
@@ -322,17 +341,12 @@ __global__ __launch_bounds__(WAVE) void frame_axis_kernel(const KernelArgs P) {
                 if (MODE == 0) { o[0] = f1x; o[1] = f1y; o[2] = f1z; }
                 else { o[0] = f2x; o[1] = f2y; o[2] = f2z; }
             } else {
-                // Gram-Schmidt and cross product
-                // (models/indexed_lattice_multi_head_attention_cuda.py:475-481; F.normalize eps 1e-12)
-                const float dot = f1x * f2x + f1y * f2y + f1z * f2z;
-                float gx = f2x - dot * f1x, gy = f2y - dot * f1y, gz = f2z - dot * f1z;
-                const float inv = 1.0f / fmaxf(sqrtf(gx * gx + gy * gy + gz * gz), 1e-12f);
-                gx *= inv; gy *= inv; gz *= inv;
+                float gx, gy, gz, hx, hy, hz;
+                orthonormal_axes(f1x, f1y, f1z, f2x, f2y, f2z, gx, gy, gz, hx, hy, hz);
                 const size_t stride = (size_t)P.N * H * 3;
                 float* o = P.out_frame + ((size_t)i * H + h) * 3;
                 o[0] = f1x; o[1] = f1y; o[2] = f1z;
                 o[stride + 0] = gx; o[stride + 1] = gy; o[stride + 2] = gz;
-                const float hx = f1y * gz - f1z * gy, hy = f1z * gx - f1x * gz, hz = f1x * gy - f1y * gx;
                 o[2 * stride + 0] = hx; o[2 * stride + 1] = hy; o[2 * stride + 2] = hz;
                 if (P.frames_to_records) {
                     // the record of this item (already in registers) becomes that of the kernel that

@@ -25,12 +25,20 @@
 
 namespace cfh {
 
-// shifts t0 .. t0+cnt of the box in the reference's loop order, w = position in the chunk (read like the low bits of
-// the sorted table's packed length: a tiny value that passes every reach test)
-__device__ __forceinline__ void build_shift_table_indexed(float4* tab, int t0, int cnt, const Box& bx, const Lattice& L,
-                                                          int lane) {
-    for (int u = lane; u < cnt; u += WAVE) {
-        const int t = t0 + u;
+constexpr int FQ_ROWS = 4;          // heads of an atom per wavefront, one per 16-lane row
+constexpr int FQ_STAGE = 64;        // pairs staged at a time
+constexpr int FQ_MAX_PAIRS = 16;    // longer rows go one item per wavefront: 64 lanes finish a long item sooner than 16
+
+// Shifts t0 .. t0+cnt (cnt <= 128) of the box, sorted by length within the chunk: w = length with the position in the
+// chunk (loop order of the reference) in its low 7 bits, like the entries of the per-crystal tables.  Items whose box
+// is not the table's thereby get the same bounded prefixes, chunk by chunk (a bound on the distance of a candidate
+// holds for any subset of the translations).  Each lane makes two entries and ranks them against all keys.
+__device__ __forceinline__ void build_sorted_chunk(float4* tab, int t0, int cnt, const Box& bx, const Lattice& L, int lane) {
+    float4 ent[2];
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const int u = lane + k * WAVE;
+        const int t = t0 + min(u, cnt - 1);
         const int i3 = t % bx.s3;
         const int q = t / bx.s3;
         const int i2 = q % bx.s2;
@@ -40,9 +48,22 @@ __device__ __forceinline__ void build_shift_table_indexed(float4* tab, int t0, i
         v.x = fmaf(L.t[6], n3, fmaf(L.t[3], n2, L.t[0] * n1));
         v.y = fmaf(L.t[7], n3, fmaf(L.t[4], n2, L.t[1] * n1));
         v.z = fmaf(L.t[8], n3, fmaf(L.t[5], n2, L.t[2] * n1));
-        v.w = __uint_as_float((uint32_t)u);
+        const float len = sqrtf(fmaf(v.x, v.x, fmaf(v.y, v.y, v.z * v.z)));
+        v.w = u < cnt ? __uint_as_float((__float_as_uint(len) & ~(uint32_t)(FC_TCAP - 1)) | (uint32_t)u) : __builtin_inff();
+        ent[k] = v;
         tab[u] = v;
     }
+    wave_sync();
+    int rank[2] = {0, 0};
+    for (int j = 0; j < cnt; j++) {
+        const float kj = tab[j].w;         // the keys differ in their low bits: no ties
+        rank[0] += kj < ent[0].w ? 1 : 0;
+        rank[1] += kj < ent[1].w ? 1 : 0;
+    }
+    wave_sync();
+    if (lane < cnt) tab[rank[0]] = ent[0];
+    if (lane + WAVE < cnt) tab[rank[1]] = ent[1];
+    for (int u = cnt + lane; u < FC_TCAP; u += WAVE) tab[u] = make_float4(0.f, 0.f, 0.f, __builtin_inff());
 }
 
 // inclusive prefix sum over the 64 lanes (row scans in DPP, row totals by lane reads)
@@ -53,19 +74,25 @@ __device__ __forceinline__ int wave_scan_incl(int x) {
     x += dpp_movei<0x118>(x);
     const int t0 = __builtin_amdgcn_readlane(x, 15), t1 = __builtin_amdgcn_readlane(x, 31);
     const int t2 = __builtin_amdgcn_readlane(x, 47);
-    const int row = (int)threadIdx.x >> 4;
+    const int row = ((int)threadIdx.x & 63) >> 4;
     return x + (row == 0 ? 0 : row == 1 ? t0 : row == 2 ? t0 + t1 : t0 + t1 + t2);
 }
 
-__global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs C) {
-    __shared__ float4 tab[FC_TCAP];
-    __shared__ float4 pq[WAVE];             // rpos and q.k of the staged pairs
-    __shared__ int pstart[WAVE + 1];        // first candidate of every staged pair, then the total
+struct FrameShared {
+    float4 tab[FC_TCAP];
+    float4 pq[WAVE];             // rpos and q.k of the staged pairs
+    int pstart[WAVE + 1];        // first candidate of every staged pair, then the total
+};
+// one wavefront, one item: wid = item * H + head.  `others_only`: only the items that the four-heads-per-wavefront
+// search leaves out (box not the table's, or more pairs than it takes).
+__device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& sh, int wid, int lane, bool others_only) {
+    float4* const tab = sh.tab;
+    float4* const pq = sh.pq;
+    int* const pstart = sh.pstart;
 
     const KernelArgs& P = C.K;
-    const int lane = threadIdx.x;
     const int H = P.H;
-    const int h = blockIdx.x % H;
+    const int h = wid % H;
     const bool noisy = P.noise > 0.0f;
     uint32_t seed_lo = P.seed_lo, seed_hi = P.seed_hi;
     if (noisy && P.seed_dev) {
@@ -74,10 +101,10 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
         seed_hi += (uint32_t)(s >> 32) ^ ((uint32_t)s * 0x85EBCA77u);
     }
 
-    const int it_cur = (int)blockIdx.x / H;      // one wavefront per item, long items first
+    const int it_cur = wid / H;      // one wavefront per item, long items first
     if (it_cur >= P.N) return;
     {
-        const uint32_t rec_cur = load_record(P, it_cur, h);
+        const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
         const Item item = unpack_item(rec_cur);
         const int crystal = __builtin_amdgcn_readlane((int)rec_cur, REC_CRYSTAL);
         const int j0 = __builtin_amdgcn_readlane((int)rec_cur, REC_J0);
@@ -90,6 +117,7 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
         for (int c = 0; c < DH; c++) qi[c] = rec_f(rec_cur, REC_QUERY + c);
         const bool sorted = C.sorted_tab != nullptr && bx.R1 == C.table_R && bx.R2 == C.table_R && bx.R3 == C.table_R &&
                             a < 0.0f;
+        if (others_only && sorted && item.npairs <= FQ_MAX_PAIRS) return;      // searched four heads at a time
         const int nchunks = sorted ? 1 : (bx.T + FC_TCAP - 1) / FC_TCAP;
         const int e0 = item.e0, npairs = item.npairs;
         const float nz = noisy ? P.noise : 0.0f;
@@ -100,7 +128,7 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
             tab[lane] = src[lane];
             tab[lane + WAVE] = src[lane + WAVE];
         } else if (nchunks == 1) {
-            build_shift_table_indexed(tab, 0, bx.T, bx, L, lane);
+            build_sorted_chunk(tab, 0, bx.T, bx, L, lane);
         }
         wave_sync();
         const float s1 = sorted ? tab[1].w : 0.0f;      // shortest non-zero shift (entry 0 is the zero shift)
@@ -114,7 +142,7 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
             Best best;
             best.score = -3.0e38f; best.e = 0x7fffffff; best.t = 0x7fffffff;
             // sweeps: the first axis needs one; the second a first one for the bound and one with the bound
-            const int nsweeps = (pass == 1 && sorted) ? 2 : 1;
+            const int nsweeps = pass == 1 ? 2 : 1;
             for (int sw = 0; sw < nsweeps; sw++) {
                 const float bound = (pass == 1 && sw == 1) ? uniform_f(-wave_min(-best.score)) : -3.0e38f;
                 for (int pb = 0; pb < npairs; pb += WAVE) {
@@ -122,7 +150,8 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
                     // stage rpos and q_i.k_j of the pairs, one per lane (a row that fits stays staged for all sweeps;
                     // the pairs of an atom point at consecutive atoms)
                     float4 rq = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (sw == 0 && C.pair_near && sorted && lane < npc) dvalid = C.pair_near[e0 + pb + lane].y;
+                    // (made for the table's box, which every other box of the launch contains: an upper bound there)
+                    if (sw == 0 && C.pair_near && lane < npc) dvalid = C.pair_near[e0 + pb + lane].y;
                     if (npairs > WAVE || (pass == 0 && sw == 0)) {
                         if (lane < npc) {
                             const int e = e0 + pb + lane;
@@ -146,14 +175,14 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
                     }
                     // how far into the sorted table this lane's pair has to look
                     float reach = 3.0e38f;
-                    if (sorted) {
+                    if (a < 0.0f) {
                         const float r2 = fmaf(rq.x, rq.x, fmaf(rq.y, rq.y, rq.z * rq.z));
                         const float r = hw_sqrt(r2);
                         if (sw == 0) {
                             // nearest valid image at distance d: every candidate within the noise of it has
                             // |s| <= |r| + sqrt(d^2 + noise); without the batch's table of d: d <= |r| (+ |s_1|)
-                            reach = dvalid >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(dvalid + nz), 1e-3f)
-                                                   : fmaf(1.0001f, fmaf(2.0f, r, (r2 > 1e-5f ? 0.0f : s1) + sq_nz), 1e-3f);
+                            if (dvalid >= 0.0f) reach = fmaf(1.0001f, r + hw_sqrt(dvalid + nz), 1e-3f);
+                            else if (sorted) reach = fmaf(1.0001f, fmaf(2.0f, r, (r2 > 1e-5f ? 0.0f : s1) + sq_nz), 1e-3f);
                         } else if (bound > -1.0e38f) {
                             const float need = (bound - rq.w - 0.5f * nz) / a;
                             reach = need >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(need), 1e-3f) : -1.0f;
@@ -164,14 +193,14 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
                         const int cnt = sorted ? bx.T : min(FC_TCAP, bx.T - t0c);
                         if (nchunks > 1) {
                             wave_sync();
-                            build_shift_table_indexed(tab, t0c, cnt, bx, L, lane);
+                            build_sorted_chunk(tab, t0c, cnt, bx, L, lane);
                         }
                         wave_sync();              // pq, the table; the readers of pstart are done
                         // the bound sweep of the second axis looks at the candidates of the first axis' sweep: when
                         // the row is staged as a whole their list is still there
                         const bool relist = !(pass == 1 && sw == 0 && sorted && npairs <= WAVE);
                         int mine = cnt;           // candidates of this lane's pair: entries with length <= reach
-                        if (sorted && relist) {
+                        if (relist) {
                             int lo = 0, hi = FC_TCAP;
 #pragma unroll
                             for (int s = 0; s < 8; s++) {      // the count is one of 0 .. 128: eight halvings
@@ -248,25 +277,19 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
                     vy = uniform_f(P.rpos[(size_t)best.e * 3 + 1]) + sy;
                     vz = uniform_f(P.rpos[(size_t)best.e * 3 + 2]) + sz;
                 }
-                const float inv = 1.0f / sqrtf(vx * vx + vy * vy + vz * vz);
-                vx *= inv; vy *= inv; vz *= inv;
+                unit_vector(vx, vy, vz);
             }
             if (pass == 0) { f1x = vx; f1y = vy; f1z = vz; }
             else { f2x = vx; f2y = vy; f2z = vz; }
         }
 
         if (lane == 0) {
-            // Gram-Schmidt and cross product
-            // (models/indexed_lattice_multi_head_attention_cuda.py:475-481; F.normalize eps 1e-12)
-            const float dot = f1x * f2x + f1y * f2y + f1z * f2z;
-            float gx = f2x - dot * f1x, gy = f2y - dot * f1y, gz = f2z - dot * f1z;
-            const float inv = 1.0f / fmaxf(sqrtf(gx * gx + gy * gy + gz * gz), 1e-12f);
-            gx *= inv; gy *= inv; gz *= inv;
+            float gx, gy, gz, hx, hy, hz;
+            orthonormal_axes(f1x, f1y, f1z, f2x, f2y, f2z, gx, gy, gz, hx, hy, hz);
             const size_t stride = (size_t)P.N * H * 3;
             float* o = P.out_frame + ((size_t)i * H + h) * 3;
             o[0] = f1x; o[1] = f1y; o[2] = f1z;
             o[stride + 0] = gx; o[stride + 1] = gy; o[stride + 2] = gz;
-            const float hx = f1y * gz - f1z * gy, hy = f1z * gx - f1x * gz, hz = f1x * gy - f1y * gx;
             o[2 * stride + 0] = hx; o[2 * stride + 1] = hy; o[2 * stride + 2] = hz;
             if (P.frames_to_records) {
                 // the record of this item becomes that of the kernel that follows: the query makes room for the frames
@@ -278,6 +301,258 @@ __global__ __launch_bounds__(WAVE) void frame_axes_sorted_kernel(const CoreArgs 
         }
         if (P.stats && lane == 0) atomicAdd(P.stats + STAT_FRAME1_RAW, n_seen);      // candidates looked at, both axes
     }
+}
+
+// ---- four heads of one atom per wavefront ----------------------------------------------------------------------
+// The items (atom, head) of an atom share everything but the query, the Gaussian coefficient and therefore the
+// scores: same pairs, same sorted table, same distances.  One wavefront takes four heads of an atom, one per
+// 16-lane row.  The pairs are staged once for all four rows (positions and nearest-image distances, and q.k per head);
+// every row then lays its own candidates end to end and deals them to its 16 lanes, and keeps its own best.  The
+// loops run as long as the longest row needs (the four rows have the same pairs, so nearly the same lengths);
+// reductions stay inside a row (DPP).  Compared with one wavefront per item: a quarter of the staging work per item,
+// lanes filled by four short candidate lists instead of one, four independent items in flight per wavefront.
+// Rows whose box is not the table's are left to frame_axes_sorted_kernel (unsorted_only).
+template <int CTRL>
+__device__ __forceinline__ float row_maxf_step(float x) { return fmaxf(x, dpp_move<CTRL>(x)); }
+__device__ __forceinline__ float row_max(float x) {
+    x = row_maxf_step<0xB1>(x); x = row_maxf_step<0x4E>(x); x = row_maxf_step<0x141>(x); x = row_maxf_step<0x140>(x);
+    return x;
+}
+__device__ __forceinline__ void row_best(Best& b) {
+    best_dpp<0xB1>(b); best_dpp<0x4E>(b); best_dpp<0x141>(b); best_dpp<0x140>(b);
+}
+
+struct FrameQuadShared {
+    float4 tab[FC_TCAP];
+    float4 rp[FQ_STAGE];                 // staged pairs: rpos, d^2 of the nearest valid image (or -1)
+    float qk_s[FQ_ROWS][FQ_STAGE];       // q_h . k_j of the staged pairs, per row
+    int pstart[FQ_ROWS][17];             // per row: first candidate of each of 16 pairs, then the total
+};
+// one wavefront, four heads of one atom: wid = item * groups + group of heads
+__device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShared& sh, int wid, int lane) {
+    float4* const tab = sh.tab;
+    float4* const rp = sh.rp;
+    float (*const qk_s)[FQ_STAGE] = sh.qk_s;
+    int (*const pstart)[17] = sh.pstart;
+
+    const KernelArgs& P = C.K;
+    const int row = lane >> 4, l16 = lane & 15;
+    const int H = P.H;
+    const int groups = (H + FQ_ROWS - 1) / FQ_ROWS;
+    const int it = wid / groups, hg = wid % groups;
+    if (it >= P.N) return;
+    const int h_row = min(hg * FQ_ROWS + row, H - 1);
+    const bool row_exists = hg * FQ_ROWS + row < H;
+    const bool noisy = P.noise > 0.0f;
+    uint32_t seed_lo = P.seed_lo, seed_hi = P.seed_hi;
+    if (noisy && P.seed_dev) {
+        const unsigned long long s = *P.seed_snap;
+        seed_lo ^= (uint32_t)s * 0x9E3779B1u;
+        seed_hi += (uint32_t)(s >> 32) ^ ((uint32_t)s * 0x85EBCA77u);
+    }
+    // record of this row's item: atom, pairs, lattice, first neighbour and crystal are the same in all four
+    const uint32_t* rec = P.items + ((size_t)it * H + h_row) * REC_WORDS;
+    const uint32_t w0 = rec[l16], w1 = rec[16 + l16];
+    const int i = __builtin_amdgcn_readlane((int)w0, REC_ATOM);
+    const int e0 = __builtin_amdgcn_readlane((int)w0, REC_E0);
+    const int npairs = __builtin_amdgcn_readlane((int)w0, REC_NPAIRS);
+    const int j0 = __builtin_amdgcn_readlane((int)w1, REC_J0 - 16);
+    const int crystal = __builtin_amdgcn_readlane((int)w1, REC_CRYSTAL - 16);
+    Lattice L;
+#pragma unroll
+    for (int d = 0; d < 9; d++) L.t[d] = __int_as_float(__builtin_amdgcn_readlane((int)w0, REC_LATTICE + d));
+    const int boxw = (int)rec[REC_BOX];
+    const float a = __uint_as_float(rec[REC_A]);
+    float q[DH];
+    {
+        const float4* qp = reinterpret_cast<const float4*>(rec + REC_QUERY);
+#pragma unroll
+        for (int c4 = 0; c4 < DH / 4; c4++) {
+            const float4 v = qp[c4];
+            q[4 * c4] = v.x; q[4 * c4 + 1] = v.y; q[4 * c4 + 2] = v.z; q[4 * c4 + 3] = v.w;
+        }
+    }
+    const int R0 = C.table_R;
+    // this row is searched here (the others by frame_item_body)
+    const bool mine = row_exists && boxw == (R0 | (R0 << 8) | (R0 << 16)) && a < 0.0f && npairs <= FQ_MAX_PAIRS;
+    if (__ballot(mine) == 0) return;
+    Box bx;
+    bx.R1 = bx.R2 = bx.R3 = R0; bx.s2 = bx.s3 = 2 * R0 + 1; bx.T = bx.s2 * bx.s2 * bx.s2; bx.over = 0;
+    {
+        const float4* src = C.sorted_tab + (size_t)crystal * FC_TCAP;
+        tab[lane] = src[lane];
+        tab[lane + WAVE] = src[lane + WAVE];
+    }
+    const float nz = noisy ? P.noise : 0.0f;
+    const float sq_nz = sqrtf(nz);
+    wave_sync();
+    const float s1 = tab[1].w;          // shortest non-zero shift (entry 0 is the zero shift)
+
+    float f1x = 0.f, f1y = 0.f, f1z = 0.f, f2x = 0.f, f2y = 0.f, f2z = 0.f;
+    unsigned long long n_seen = 0;
+    for (int pass = 0; pass < 2; pass++) {
+        Best best;
+        best.score = -3.0e38f; best.e = 0x7fffffff; best.t = 0x7fffffff;
+        for (int sw = 0; sw < (pass == 1 ? 2 : 1); sw++) {
+            const float bound = (pass == 1 && sw == 1) ? row_max(best.score) : -3.0e38f;      // per row
+            for (int pb = 0; pb < npairs; pb += FQ_STAGE) {
+                const int nst = min(FQ_STAGE, npairs - pb);
+                if (npairs > FQ_STAGE || (pass == 0 && sw == 0)) {
+                    // ---- stage: lane = pair; q.k for the four heads with the query channels read across the rows
+                    wave_sync();
+                    float4 r4 = make_float4(0.f, 0.f, 0.f, -1.0f);
+                    const bool have = lane < nst;
+                    const int e = e0 + pb + min(lane, nst - 1);
+                    if (have) {
+                        r4.x = P.rpos[(size_t)e * 3 + 0]; r4.y = P.rpos[(size_t)e * 3 + 1]; r4.z = P.rpos[(size_t)e * 3 + 2];
+                        if (C.pair_near) r4.w = C.pair_near[e].y;
+                    }
+                    rp[lane] = r4;
+#pragma unroll 1
+                    for (int r = 0; r < FQ_ROWS; r++) {
+                        const int hr = min(hg * FQ_ROWS + r, H - 1);
+                        const float4* kp = reinterpret_cast<const float4*>(C.k + ((size_t)(j0 + pb + min(lane, nst - 1)) * H + hr) * DH);
+                        float acc = 0.0f;
+#pragma unroll
+                        for (int c4 = 0; c4 < DH / 4; c4++) {
+                            const float4 kv = kp[c4];
+                            acc = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(q[4 * c4 + 0]), r * 16)), kv.x, acc);
+                            acc = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(q[4 * c4 + 1]), r * 16)), kv.y, acc);
+                            acc = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(q[4 * c4 + 2]), r * 16)), kv.z, acc);
+                            acc = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(q[4 * c4 + 3]), r * 16)), kv.w, acc);
+                        }
+                        qk_s[r][lane] = acc;
+                    }
+                    wave_sync();
+                }
+                for (int pc = 0; pc < nst; pc += 16) {
+                    // ---- this row's 16 pairs: how far each has to look, its candidates end to end
+                    const int pj = pc + l16;
+                    const bool pair_ok = mine && pj < nst;
+                    const float4 r4 = rp[min(pj, nst - 1)];
+                    const float myqk = qk_s[row][min(pj, nst - 1)];
+                    const float r2 = fmaf(r4.x, r4.x, fmaf(r4.y, r4.y, r4.z * r4.z));
+                    const float r = hw_sqrt(r2);
+                    float reach;
+                    if (sw == 0) {
+                        reach = r4.w >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(r4.w + nz), 1e-3f)
+                                             : fmaf(1.0001f, fmaf(2.0f, r, (r2 > 1e-5f ? 0.0f : s1) + sq_nz), 1e-3f);
+                    } else if (bound > -1.0e38f) {
+                        const float need = (bound - myqk - 0.5f * nz) / a;
+                        reach = need >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(need), 1e-3f) : -1.0f;
+                    } else {
+                        reach = 3.0e38f;
+                    }
+                    int cnt;
+                    {
+                        int lo = 0, hi = FC_TCAP;
+#pragma unroll
+                        for (int s = 0; s < 8; s++) {      // the count is one of 0 .. 128: eight halvings
+                            const int mid = min((lo + hi) >> 1, FC_TCAP - 1);
+                            const bool le = lo < hi && tab[mid].w <= reach;
+                            lo = le ? mid + 1 : lo;
+                            hi = le ? hi : mid;
+                        }
+                        cnt = pair_ok ? min(lo, bx.T) : 0;
+                    }
+                    int incl = cnt;                        // inclusive prefix within the row
+                    incl += dpp_movei<0x111>(incl);
+                    incl += dpp_movei<0x112>(incl);
+                    incl += dpp_movei<0x114>(incl);
+                    incl += dpp_movei<0x118>(incl);
+                    const int t0 = __builtin_amdgcn_readlane(incl, 15), t1 = __builtin_amdgcn_readlane(incl, 31);
+                    const int t2 = __builtin_amdgcn_readlane(incl, 47), t3 = __builtin_amdgcn_readlane(incl, 63);
+                    const int total = row == 0 ? t0 : row == 1 ? t1 : row == 2 ? t2 : t3;
+                    const int longest = max(max(t0, t1), max(t2, t3));
+                    wave_sync();                           // the readers of pstart are done
+                    pstart[row][l16] = incl - cnt;
+                    if (l16 == 0) pstart[row][16] = total;
+                    wave_sync();
+                    n_seen += (unsigned long long)(t0 + t1 + t2 + t3);
+                    for (int base = 0; base < longest; base += 16) {
+                        const int c = base + l16;
+                        const bool in = c < total;
+                        int lo = 0, hi = 16;               // pstart[lo] <= c < pstart[hi]
+#pragma unroll
+                        for (int s = 0; s < 4; s++) {
+                            const int mid = (lo + hi) >> 1;
+                            const bool le = pstart[row][mid] <= c;
+                            lo = le ? mid : lo;
+                            hi = le ? hi : mid;
+                        }
+                        const int pl = in ? lo : 0;
+                        const float4 v = tab[in ? c - pstart[row][pl] : 0];
+                        const int ps = min(pc + pl, nst - 1);
+                        const float4 cq = rp[ps];
+                        const float cqk = qk_s[row][ps];
+                        const int e = e0 + pb + pc + pl;
+                        const int t = (int)(__float_as_uint(v.w) & (uint32_t)(FC_TCAP - 1));
+                        const float dx = cq.x + v.x, dy = cq.y + v.y, dz = cq.z + v.z;
+                        const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+                        float score = fmaf(a, d2, cqk);
+                        bool ok = in && d2 > 1e-5f;
+                        if (pass == 1) {
+                            const float rinv = hw_rsq(d2);
+                            const float ac = fabsf((dx * f1x + dy * f1y + dz * f1z) * rinv);
+                            score += hw_log2(fmaxf(1.0f - ac, 1e-5f)) * LN2;
+                            ok = ok && ac < 0.9999f;
+                        }
+                        if (noisy) {
+                            const float phase = hash_uniform(pass ? seed_hi : seed_lo, pass ? seed_lo : seed_hi,
+                                                             (uint32_t)(e * H + h_row), (uint32_t)pass);
+                            const float un = __builtin_amdgcn_fractf(fmaf((float)t, 0.61803399f, phase));
+                            if (pass == 0) score = fmaf(a, d2 + (un - 0.5f) * P.noise, cqk);
+                            else score += (un - 0.5f) * P.noise;
+                        }
+                        if (ok && better(score, e, t, best.score, best.e, best.t)) {
+                            best.score = score; best.e = e; best.t = t;
+                        }
+                    }
+                }
+            }
+        }
+        row_best(best);
+        float vx = 0.f, vy = 0.f, vz = 0.f;
+        if (best.e != 0x7fffffff) {
+            float sx, sy, sz;
+            shift_of(best.t, bx, L, sx, sy, sz);
+            vx = P.rpos[(size_t)best.e * 3 + 0] + sx;
+            vy = P.rpos[(size_t)best.e * 3 + 1] + sy;
+            vz = P.rpos[(size_t)best.e * 3 + 2] + sz;
+            unit_vector(vx, vy, vz);
+        }
+        if (pass == 0) { f1x = vx; f1y = vy; f1z = vz; }
+        else { f2x = vx; f2y = vy; f2z = vz; }
+    }
+    // lane c < 9 of a row stores component c of that row's frame
+    float gx, gy, gz, hx, hy, hz;
+    orthonormal_axes(f1x, f1y, f1z, f2x, f2y, f2z, gx, gy, gz, hx, hy, hz);
+    if (mine && l16 < 9) {
+        const float val = l16 == 0 ? f1x : l16 == 1 ? f1y : l16 == 2 ? f1z : l16 == 3 ? gx : l16 == 4 ? gy : l16 == 5 ? gz
+                        : l16 == 6 ? hx : l16 == 7 ? hy : hz;
+        const int ax = l16 / 3, d = l16 - 3 * ax;
+        P.out_frame[(((size_t)ax * P.N + i) * H + h_row) * 3 + d] = val;
+        if (P.frames_to_records)      // the record becomes that of the kernel that follows: the query makes room for the frames
+            reinterpret_cast<float*>(P.items + ((size_t)it * H + h_row) * REC_WORDS + REC_FRAMES)[l16] = val;
+    }
+    if (P.stats && lane == 0) atomicAdd(P.stats + STAT_FRAME1_RAW, n_seen);
+}
+
+// One item per wavefront, every item (launches without per-crystal tables).  waves: N * H.
+__global__ __launch_bounds__(WAVE * CORE_WPB) void frame_axes_sorted_kernel(const CoreArgs C) {
+    __shared__ FrameShared shared[CORE_WPB];
+    frame_item_body(C, shared[threadIdx.x >> 6], (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6),
+                    (int)threadIdx.x & (WAVE - 1), false);
+}
+
+// Both ways in one launch.  The first `item_blocks` workgroups go over all items one per wavefront and take those that
+// the four-heads search leaves out (the rest return at once); they come first so that these few, slower items start
+// early and run beside the others.  The remaining workgroups search four heads of an atom per wavefront.
+__global__ __launch_bounds__(WAVE * CORE_WPB) void frame_axes_kernel(const CoreArgs C, int item_blocks) {
+    __shared__ union { FrameShared item; FrameQuadShared quad; } shared[CORE_WPB];
+    const int wv = (int)(threadIdx.x >> 6), lane = (int)threadIdx.x & (WAVE - 1);
+    if ((int)blockIdx.x < item_blocks) frame_item_body(C, shared[wv].item, (int)blockIdx.x * CORE_WPB + wv, lane, true);
+    else frame_quad_body(C, shared[wv].quad, ((int)blockIdx.x - item_blocks) * CORE_WPB + wv, lane);
 }
 
 }  // namespace cfh

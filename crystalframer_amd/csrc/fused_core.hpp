@@ -45,6 +45,8 @@ constexpr int FC_SHIFT = 7;                     // list entry = pair-in-group <<
 #define CFH_NORD 5
 #endif
 constexpr int NORD = CFH_NORD;                  // moments per axis
+constexpr int CORE_WPB = 1;                     // wavefronts per workgroup of the main kernels: each takes an item of its
+                                                // own (no barriers); dispatching one-wavefront workgroups is slower than the items are
 constexpr int FC_LOGCAP = 256;                  // logits of a row kept in LDS until the row is complete
 constexpr int HW_DIST = NBINS;
 constexpr int HW_ANG = NBINS * (1 + 3 * NORD);  // 1024 words per (atom, head) with the angle encoding
@@ -59,7 +61,7 @@ typedef float v4f_c __attribute__((ext_vector_type(4)));
 #ifdef CFH_PHASE_TIMING
 #define CFH_PH_DECL unsigned long long ph_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long ph_last = __builtin_amdgcn_s_memtime(); int ph_cur = 0;
 #define CFH_PH(n) do { const unsigned long long ph_t = __builtin_amdgcn_s_memtime(); ph_acc[ph_cur] += ph_t - ph_last; ph_last = ph_t; ph_cur = (n); } while (0)
-#define CFH_PH_FLUSH(stats) do { CFH_PH(0); if ((stats) && threadIdx.x == 0) for (int u = 0; u < 8; u++) atomicAdd((stats) + 16 + u, ph_acc[u]); } while (0)
+#define CFH_PH_FLUSH(stats) do { CFH_PH(0); if ((stats) && (threadIdx.x & 63) == 0) for (int u = 0; u < 8; u++) atomicAdd((stats) + 16 + u, ph_acc[u]); } while (0)
 #else
 #define CFH_PH_DECL
 #define CFH_PH(n) do { } while (0)
@@ -334,34 +336,46 @@ __device__ __forceinline__ void core_store_table(const CoreItem& ci, const CoreP
 // =================================================================================================================
 // forward
 // =================================================================================================================
+template <int HWK>
+struct CoreFwdShared {
+    float4 tab[FC_TCAP];
+    uint16_t list[FC_LISTCAP];
+    int32_t hist[HWK];
+    float4 pairA[FC_GROUP];      // rx, ry, rz, d2min
+    float pairC[FC_GROUP];       // exp(logit - running max) / S in fixed-point units
+    float logit_s[FC_LOGCAP];    // logits of the row (rows of more pairs park them in the probability array)
+};
 template <int WL, bool HAS_ANG, bool COS_ABS>
-__global__ __launch_bounds__(WAVE) void fused_core_fwd_kernel(const CoreArgs C) {
+__global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const CoreArgs C) {
     constexpr int HWK = HAS_ANG ? HW_ANG : HW_DIST;
-    __shared__ float4 tab[FC_TCAP];
-    __shared__ uint16_t list[FC_LISTCAP];
-    __shared__ int32_t hist[HWK];
-    __shared__ float4 pairA[FC_GROUP];      // rx, ry, rz, d2min
-    __shared__ float pairC[FC_GROUP];       // exp(logit - running max) / S in fixed-point units
-    __shared__ float logit_s[FC_LOGCAP];    // logits of the row (rows of more pairs park them in the probability array)
+    __shared__ CoreFwdShared<HWK> shared[CORE_WPB];
+    CoreFwdShared<HWK>& sh = shared[threadIdx.x >> 6];
+    float4* const tab = sh.tab;
+    uint16_t* const list = sh.list;
+    int32_t* const hist = sh.hist;
+    float4* const pairA = sh.pairA;
+    float* const pairC = sh.pairC;
+    float* const logit_s = sh.logit_s;
 
     const KernelArgs& P = C.K;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & (WAVE - 1);
     const int H = P.H;
-    const int h = blockIdx.x % H;
+    const int wid = (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6);      // this wavefront's (item, head)
+    const int h = wid % H;
     const int pr = lane >> 3;          // pair of the group served by this 8-lane row
     const int sub = lane & 7;          // position in the row
     const BasisConsts bc = P.bc;
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
     const float INF = __builtin_inff();
 
-    const int it_cur = (int)blockIdx.x / H;      // items in descending order of their pair count: the long ones start first
+    const int it_cur = wid / H;      // items in descending order of their pair count: the long ones start first
     if (it_cur >= P.N) return;
     for (int u = lane; u < HWK; u += WAVE) hist[u] = 0;
     wave_sync();
 
     CFH_PH_DECL
     {
-        const uint32_t rec_cur = load_record(P, it_cur, h);
+        const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
         const CorePrefetch pf = core_prefetch(C, rec_cur, it_cur, h, lane);
         CFH_PH(0);
         const CoreItem ci = core_unpack(C, rec_cur, true);
@@ -756,29 +770,41 @@ __global__ void core_zero_kernel(float* p, int n) {
 //     gq_i                 = sum_j gl_ij k_j
 // (the terms A0_j (go . psi_ij) of dL/dz and of the covariance form cancel).  gk and gv are sums over the pairs that
 // point AT an atom and are left to the column kernel of the attention backward (from gl and P).
+template <int HWK>
+struct CoreBwdShared {
+    float4 tab[FC_TCAP];
+    uint16_t list[FC_LISTCAP];
+    float Gs[HWK];
+    float4 pairA[FC_GROUP];      // rx, ry, rz, z log2(e)
+    float pairP[FC_GROUP];       // P_ij
+    int32_t pairB[FC_GROUP];     // sum_n P_ij p_n bg_n in fixed point
+};
 template <int WL, bool HAS_ANG, bool COS_ABS>
-__global__ __launch_bounds__(WAVE) void fused_core_bwd_kernel(const CoreArgs C) {
+__global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const CoreArgs C) {
     constexpr int HWK = HAS_ANG ? HW_ANG : HW_DIST;
-    __shared__ float4 tab[FC_TCAP];
-    __shared__ uint16_t list[FC_LISTCAP];
-    __shared__ float Gs[HWK];
-    __shared__ float4 pairA[FC_GROUP];      // rx, ry, rz, z log2(e)
-    __shared__ float pairP[FC_GROUP];       // P_ij
-    __shared__ int32_t pairB[FC_GROUP];     // sum_n P_ij p_n bg_n in fixed point
+    __shared__ CoreBwdShared<HWK> shared[CORE_WPB];
+    CoreBwdShared<HWK>& sh = shared[threadIdx.x >> 6];
+    float4* const tab = sh.tab;
+    uint16_t* const list = sh.list;
+    float* const Gs = sh.Gs;
+    float4* const pairA = sh.pairA;
+    float* const pairP = sh.pairP;
+    int32_t* const pairB = sh.pairB;
 
     const KernelArgs& P = C.K;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & (WAVE - 1);
     const int H = P.H;
-    const int h = blockIdx.x % H;
+    const int wid = (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6);
+    const int h = wid % H;
     const int pr = lane >> 3, sub = lane & 7;
     const BasisConsts bc = P.bc;
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
     const float INF = __builtin_inff();
 
-    const int it_cur = (int)blockIdx.x / H;      // one wavefront per item, long items first
+    const int it_cur = wid / H;      // one wavefront per item, long items first
     if (it_cur >= P.N) return;
     {
-        const uint32_t rec_cur = load_record(P, it_cur, h);
+        const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
         const CoreItem ci = core_unpack(C, rec_cur, true);
         const int i = ci.item.i;
         const float a2 = ci.item.a * LOG2E;
