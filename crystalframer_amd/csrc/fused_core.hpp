@@ -82,11 +82,11 @@ struct CoreArgs {
     float* out;                   // (N,H,16) sum_j P_ij v_j (core_project_kernel adds W . hist)
     float* prob;                  // (E,H) P_ij
     float* z;                     // (E,H)
-    float* hist;                  // (N,H,hw)
+    float* hist;                  // (H,N,hw)
     // backward operands and results
     const float* go;              // (N,H,16) upstream gradient of out
     const float* outv;            // (N,H,16) the forward's final out
-    const float* G;               // (N,H,hw) Wcat^T go per item
+    const float* G;               // (H,N,hw) Wcat^T go per item
     float* gq;                    // (N,H,16)
     float* glogit;                // (E,H) gradient of the logits (the column kernel turns it into gk)
 };
@@ -604,7 +604,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             // all reads first (one LDS round trip instead of one per word), then clear and store
             constexpr int NW = HWK / WAVE;
             const float sc = inv * (float)max(npairs, 1) * (1.0f / 1073741824.0f);
-            float* dst = C.hist + ih * HWK + lane;
+            float* dst = C.hist + ((size_t)h * P.N + i) * HWK + lane;      // head-major: the rows of a head are contiguous
             int32_t hv[NW];
 #pragma unroll
             for (int u = 0; u < NW; u++) hv[u] = hist[lane + WAVE * u];
@@ -632,7 +632,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
     }
 }
 
-// out (N,H,16) += Wcat_h (16, hw) . hist (N,H,hw): one workgroup of PROJ_WAVES wavefronts per (16 atoms, head); each
+// out (N,H,16) += Wcat_h (16, hw) . hist (H,N,hw): one workgroup of PROJ_WAVES wavefronts per (16 atoms, head); each
 // wavefront takes a slice of the reduction index through MFMA 16x16x4 (a lane owns 16 consecutive words of each
 // 64-word step: 64-byte loads of its row), the slices meet in LDS and are added in a fixed order by the first
 // wavefront (no atomics: the result does not depend on timing).  grid (ceil(N/16), H), block 64 * PROJ_WAVES.
@@ -644,7 +644,7 @@ __global__ __launch_bounds__(WAVE * PROJ_WAVES) void core_project_kernel(const f
     const int lane = threadIdx.x & (WAVE - 1), wv = threadIdx.x >> 6, col = lane & 15, kk = lane >> 4;
     const int h = blockIdx.y, i0 = blockIdx.x * 16;
     const int row = min(i0 + col, N - 1);
-    const float4* ap = reinterpret_cast<const float4*>(hist + ((size_t)row * H + h) * hw) + 4 * kk;
+    const float4* ap = reinterpret_cast<const float4*>(hist + ((size_t)h * N + row) * hw) + 4 * kk;
     const float4* bp = reinterpret_cast<const float4*>(wcat + ((size_t)h * DH + col) * hw) + 4 * kk;
     v4f_c acc = {0.f, 0.f, 0.f, 0.f};
     const int steps = hw / 64, per = (steps + PROJ_WAVES - 1) / PROJ_WAVES;
@@ -677,7 +677,7 @@ __global__ __launch_bounds__(WAVE * PROJ_WAVES) void core_project_kernel(const f
     }
 }
 
-// G (N,H,hw) = go (N,H,16) . Wcat_h (16, hw): wavefront per (16 atoms, head, 64-word block); four MFMA tiles whose
+// G (H,N,hw) = go (N,H,16) . Wcat_h (16, hw): wavefront per (16 atoms, head, 64-word block); four MFMA tiles whose
 // columns are interleaved (tile t, column c <-> word 4 c + t) so that a lane stores 16 consecutive bytes.
 // grid (ceil(N/16), H, hw/64).  `queues`: optional work-queue heads to clear (when no prepare launch does).
 __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restrict__ go, const float* __restrict__ wcat,
@@ -710,13 +710,13 @@ __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restri
         for (int r = 0; r < 4; r++) {
             const int it = i0 + 4 * kk + r;
             if (it < N)
-                *reinterpret_cast<float4*>(G + ((size_t)it * H + h) * hw + w0 + 4 * col) =
+                *reinterpret_cast<float4*>(G + ((size_t)h * N + it) * hw + w0 + 4 * col) =
                     make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
         }
     }
 }
 
-// gwcat (H,16,hw) += sum over a slice of the atoms of go (.,h,16) (x) hist (.,h,hw): wavefront per (head, 64-word
+// gwcat (H,16,hw) += sum over a slice of the atoms of go (.,h,16) (x) hist (h,.,hw): wavefront per (head, 64-word
 // block, slice); four MFMA tiles with interleaved columns as above; float atomics into the cleared result.
 // grid (hw/64, H, nslices).
 __global__ __launch_bounds__(WAVE) void core_gwcat_kernel(const float* __restrict__ go, const float* __restrict__ hist,
@@ -736,7 +736,8 @@ __global__ __launch_bounds__(WAVE) void core_gwcat_kernel(const float* __restric
             const bool live = it < i_end;
             const size_t base = ((size_t)(live ? it : i_begin) * H + h);
             av[j] = live ? go[base * DH + col] : 0.0f;
-            bv[j] = live ? *reinterpret_cast<const float4*>(hist + base * hw + w0 + 4 * col) : make_float4(0.f, 0.f, 0.f, 0.f);
+            bv[j] = live ? *reinterpret_cast<const float4*>(hist + ((size_t)h * N + it) * hw + w0 + 4 * col)
+                         : make_float4(0.f, 0.f, 0.f, 0.f);
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -824,7 +825,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
         core_load_table(C, ci, tab, lane);
         float gabs = 0.0f;
         {
-            const float* src = C.G + ih * HWK;
+            const float* src = C.G + ((size_t)h * P.N + i) * HWK;
             for (int u = lane; u < HWK; u += WAVE) { const float g = src[u]; Gs[u] = g; gabs += fabsf(g); }
         }
         const float2 go2 = *reinterpret_cast<const float2*>(C.go + ih * DH + 2 * sub);

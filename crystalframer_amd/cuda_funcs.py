@@ -612,7 +612,7 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
             fr = None
         z = torch.empty((E, H), dtype=torch.float32, device=dev)
         prob = torch.empty((E, H), dtype=torch.float32, device=dev)
-        hist = torch.empty((N, H, hw), dtype=torch.float32, device=dev)
+        hist = torch.empty((H, N, hw), dtype=torch.float32, device=dev)      # head-major
         out = torch.empty((N, H, Dh), dtype=torch.float32, device=dev)
         # kept for the backward (and, the table, for the other layers of the pass): sorted translations of every
         # crystal, projection weights with the moment matrices folded in, item records

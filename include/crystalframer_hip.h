@@ -292,7 +292,8 @@ int cfh_fused_dpa_backward(const float* q, const float* k, const float* v, const
  * (error < 2e-6 of a basis function's peak for angle_wscale 4; angle_wscale < 3 returns CFH_EINVAL).
  * Needs dist_bins = 64, dist_wscale = 1, angle_bins 0 or 64, and the pairs as the complete n x n block of every
  * crystal (cfh_pair_layout_check).  qs = query / sqrt(Dh).
- * Results kept for the backward: z (E,H), prob (E,H) = P, hist (N,H,words) the normalised histograms
+ * Results kept for the backward: z (E,H), prob (E,H) = P, hist (H,N,words) the normalised histograms
+ * (head-major: the kernels that contract them with the weights read the rows of a head one after the other)
  * (words = cfh_fused_core_hist_words: 64 distance bins, then per axis and order 64 moment bins), out (N,H,Dh).
  * workspace: cfh_fused_core_workspace_bytes(p, N, E, B, 0).
  *
