@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
@@ -76,7 +76,7 @@ class CfhLinearGradJob(ctypes.Structure):
 
 EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_frame_axis1",
            "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_forward_static", "cfh_frame_axes_framed_pe_forward",
-           "cfh_framed_pe_backward",
+           "cfh_framed_pe_backward", "cfh_framed_pe_backward_pairwise",
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
            "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
            "cfh_crystal_geometry", "cfh_small_linear_forward", "cfh_small_linear_dx", "cfh_linear_weight_bias_grad", "cfh_linear_weight_bias_grad_batch", "cfh_attention_inputs_forward",
@@ -131,6 +131,8 @@ def load():
         lib.cfh_layer_bridge_backward.argtypes = [_P] * 7 + [_I64, ctypes.c_int32, ctypes.c_int32] + [_P] * 6
         lib.cfh_framed_pe_backward.restype = ctypes.c_int
         lib.cfh_framed_pe_backward.argtypes = [pp] + [_P] * 17 + [_I64] * 3 + [_P] * 6 + [ctypes.c_size_t, _P]
+        lib.cfh_framed_pe_backward_pairwise.restype = ctypes.c_int
+        lib.cfh_framed_pe_backward_pairwise.argtypes = [pp] + [_P] * 12 + [_I64] * 3 + [_P, _P, ctypes.c_size_t, _P]
         lib.cfh_fused_dpa_forward.restype = ctypes.c_int
         lib.cfh_fused_dpa_forward.argtypes = [_P] * 7 + [_I64] * 4 + [_P] * 3
         lib.cfh_fused_dpa_backward.restype = ctypes.c_int

@@ -626,12 +626,13 @@ static int framed_pe_backward_impl(const cfh_params* p, const float* a_ih, const
                            const float* shat, int64_t N, int64_t E, int64_t B, float* ga, float* gW_dist,
                            float* gW_axis1,
                            float* gW_axis2, float* gW_axis3, void* workspace, size_t workspace_bytes,
-                           void* stream) {
+                           void* stream, const float* g_pair = nullptr) {
     int rc = check_params(p);
     if (rc) return rc;
     if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
-    const bool has_len = p->dist_bins > 0 && W_dist != nullptr;
-    const bool has_ang = has_len && p->angle_bins > 0 && W_axis1 != nullptr;
+    // g_pair: the rows W^T gpsi come per pair from the caller; no weights, no weight gradients
+    const bool has_len = p->dist_bins > 0 && (W_dist != nullptr || g_pair != nullptr);
+    const bool has_ang = has_len && p->angle_bins > 0 && (W_axis1 != nullptr || (g_pair != nullptr && frames != nullptr));
     hipStream_t st = (hipStream_t)stream;
     const size_t wbytes = (size_t)p->num_heads * cfh::DH * cfh::NBINS * sizeof(float);
     if (N == 0) {     // no atoms: the weight gradients are zero
@@ -641,8 +642,8 @@ static int framed_pe_backward_impl(const cfh_params* p, const float* a_ih, const
         return finish_launch("zero_outputs");
     }
     if (!z || !gz || !ga) return fail(CFH_EINVAL, "z, gz and ga must not be NULL");
-    if (has_len && !gpsi) return fail(CFH_EINVAL, "gpsi must not be NULL when dist_bins > 0");
-    if (has_ang && (!W_axis2 || !W_axis3 || !frames))
+    if (has_len && !gpsi && !g_pair) return fail(CFH_EINVAL, "gpsi must not be NULL when dist_bins > 0");
+    if (has_ang && !g_pair && (!W_axis2 || !W_axis3 || !frames))
         return fail(CFH_EINVAL, "W_axis1..3 and frames must be given together");
     int wl = 0, wa = 0;
     if ((rc = window_widths(p, &wl, &wa))) return rc;
@@ -654,7 +655,20 @@ static int framed_pe_backward_impl(const cfh_params* p, const float* a_ih, const
     A.W[0] = W_dist; A.W[1] = W_axis1; A.W[2] = W_axis2; A.W[3] = W_axis3;
     A.frames = frames; A.z = z; A.gz = gz; A.gpsi = gpsi; A.out_ga = ga;
     A.shat = const_cast<float*>(shat);
+    A.g_pair = g_pair;
     A.gw_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + COUNTER_BYTES + items_bytes(N, p->num_heads));
+    if (g_pair) {        // gather-only kernel on this stream; nothing else
+        const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+        const char* what = "framed_pe_backward";
+        if (p->angle_bins == SMALL_ANGLE_BINS && has_ang) {
+            if (wide) rc = p->cos_abs ? launch_persistent(cfh::framed_pe_bwd_saved_kernel<11, SMALL_ANGLE_WINDOW, true, true, true, false>, A, &waves, st, what)
+                                      : launch_persistent(cfh::framed_pe_bwd_saved_kernel<11, SMALL_ANGLE_WINDOW, false, true, true, false>, A, &waves, st, what);
+            else rc = p->cos_abs ? launch_persistent(cfh::framed_pe_bwd_saved_kernel<9, SMALL_ANGLE_WINDOW, true, true, true, false>, A, &waves, st, what)
+                                 : launch_persistent(cfh::framed_pe_bwd_saved_kernel<9, SMALL_ANGLE_WINDOW, false, true, true, false>, A, &waves, st, what);
+        } else if (has_ang) CFH_DISPATCH_PE_NOGW(cfh::framed_pe_bwd_saved_kernel, true);
+        else CFH_DISPATCH_PE_NOGW(cfh::framed_pe_bwd_saved_kernel, false);
+        return rc;
+    }
     if (has_len) {      // cleared by the prepare kernel of this launch, added into by gw_reduce_kernel
         A.gw_out[0] = gW_dist;
         if (has_ang) { A.gw_out[1] = gW_axis1; A.gw_out[2] = gW_axis2; A.gw_out[3] = gW_axis3; }
@@ -783,6 +797,18 @@ int cfh_framed_pe_backward(const cfh_params* p, const float* a_ih, const float* 
     hipLaunchKernelGGL(cfh::unpad_bins_kernel, dim3((3 * per_small + 255) / 256), dim3(256), 0, st, gpad, rows,
                        SMALL_ANGLE_BINS, gW_axis1, gW_axis2, gW_axis3);
     return finish_launch("framed_pe_backward (16-bin angle basis)");
+}
+
+int cfh_framed_pe_backward_pairwise(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,
+                                    const float* rvlen, const int64_t* batch, const int64_t* edges,
+                                    const int64_t* e_start, const int32_t* order, const float* frames, const float* z,
+                                    const float* gz, const float* g_pair, int64_t N, int64_t E, int64_t B, float* ga,
+                                    void* workspace, size_t workspace_bytes, void* stream) {
+    if (!g_pair) return fail(CFH_EINVAL, "g_pair must not be NULL");
+    if (N <= 0) return check_params(p);
+    return framed_pe_backward_impl(p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, nullptr, nullptr, nullptr,
+                                   nullptr, frames, z, gz, nullptr, nullptr, N, E, B, ga, nullptr, nullptr, nullptr,
+                                   nullptr, workspace, workspace_bytes, stream, g_pair);
 }
 
 namespace {

@@ -332,6 +332,8 @@ struct KernelArgs {
     const float* q; const float* k; const float* frame1;
     // value-PE operands
     const float* W[4]; const float* frames; const float* z; const float* gz; const float* gpsi;
+    const float* g_pair;          // backward, optional: (E, H, 4, NBINS) the rows W^T gpsi of every pair, made by the caller
+                                  // (projection weights that differ from pair to pair); the weights are then not read
     // outputs
     float* out_z; float* out_psi; float* out_d2min; float* out_frame; float* out_ga;
     float* gw_partial;            // (waves, 4, DH, NBINS) per-wave weight-gradient partials

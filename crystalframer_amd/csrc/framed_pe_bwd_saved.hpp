@@ -39,7 +39,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
 #pragma unroll
     for (int en = 0; en < NENC; en++) {
 #pragma unroll
-        for (int c = 0; c < DH; c++) Wt[en * DH + c] = P.W[en][((size_t)h * DH + c) * NBINS + lane];
+        for (int c = 0; c < DH; c++) Wt[en * DH + c] = P.g_pair ? 0.0f : P.W[en][((size_t)h * DH + c) * NBINS + lane];
         if constexpr (WITH_GW) {
 #pragma unroll
             for (int cq = 0; cq < 4; cq++) gWacc[en * 4 + cq] = v4f_b{0.f, 0.f, 0.f, 0.f};
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
                 if (NENC > 0) {
                     if ((el_glob & 15) == 0) {             // gpsi of the next 16 pairs: 64 B per pair
                         const int e = e0 + el_glob + (lane >> 2);
-                        if (e < e1)
+                        if (e < e1 && !P.g_pair)
                             pgp = reinterpret_cast<const float4*>(P.gpsi + ((size_t)e * H + h) * DH)[sub];
                     }
                     // the 32 lanes that hold this group's gpsi stage it in both layouts
@@ -205,6 +205,16 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
                     }
                     wave_sync();
                     // G[pair = 4 half + sub][enc][k = 4 blk + r] = sum_c W_enc[c][k] gpsi[pair][c]
+                    if (P.g_pair) {          // given per pair (already scaled by the encodings' coefficients)
+                        for (int half = 0; half * 4 < cur_ng; half++) {
+                            const int pl = half * 4 + sub;
+                            const float4* src = reinterpret_cast<const float4*>(
+                                P.g_pair + (((size_t)(cur_g0 + min(pl, cur_ng - 1)) * H + h) * 4) * NBINS) + blk;
+#pragma unroll
+                            for (int en = 0; en < NENC; en++)
+                                *reinterpret_cast<float4*>(Gs + pl * PAIR_STRIDE + en * HS + 4 * blk) = src[en * (NBINS / 4)];
+                        }
+                    } else
                     for (int half = 0; half * 4 < cur_ng; half++) {
                         const int pl = half * 4 + sub;
                         float gb[DH];

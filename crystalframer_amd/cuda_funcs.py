@@ -198,7 +198,8 @@ def _f32c(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
 
 
 def _proj_weight(W: Optional[torch.Tensor], H: int, what: str) -> Optional[torch.Tensor]:
-    """(1,H,Dh,bins) or (H,Dh,bins) -> contiguous (H,Dh,bins); per-edge / per-atom weights unsupported."""
+    """(1,H,Dh,bins) or (H,Dh,bins) -> contiguous (H,Dh,bins) (weights that differ from pair to pair are handled by
+    the caller, see _weight_sets)."""
     if W is None:
         return None
     if W.dim() not in (3, 4):
@@ -317,6 +318,58 @@ def _stacked_frames(f1, f2, f3):
     return torch.stack([_f32c(f1), _f32c(f2), _f32c(f3)], 0).contiguous()
 
 
+_PAIR_CHUNK = 4096      # pairs per step of the framework products below (bounds their temporaries)
+
+
+def _weight_sets(W_k, E: int, N: int) -> str:
+    """How the projection weights are shared (models/kernels/real_enc_frame_proj_fwd_length.cu:166-173):
+    "shared" (leading dimension 1 or none), "edge" (one set per pair), "atom" (one set per query atom)."""
+    if W_k is None or W_k.dim() == 3 or W_k.shape[0] == 1:
+        return "shared"
+    if W_k.shape[0] == E:
+        return "edge"
+    if W_k.shape[0] == N:
+        return "atom"
+    raise ValueError(f"W_k: leading dimension {W_k.shape[0]} is neither 1, the number of pairs {E} nor of atoms {N}")
+
+
+def _pairwise_psi(Ws, coefs, rows, shat, Dh):
+    """psi (E,H,Dh) = sum_enc coef_enc W_enc[rows[e]] . shat[e,:,enc] for weights that differ from pair to pair
+    (``rows`` None: pair e uses set e).  Device products of the framework over the histograms the kernel made."""
+    E, H = shat.shape[:2]
+    out = torch.zeros((E, H, Dh), dtype=torch.float32, device=shat.device)
+    for s0 in range(0, E, _PAIR_CHUNK):
+        sl = slice(s0, min(E, s0 + _PAIR_CHUNK))
+        for en, (W, c) in enumerate(zip(Ws, coefs)):
+            if W is None:
+                continue
+            Wsel = W[sl] if rows is None else W[rows[sl]]
+            out[sl] += c * torch.einsum("ehck,ehk->ehc", Wsel.to(torch.float32), shat[sl, :, en, :W.shape[-1]])
+    return out
+
+
+def _pairwise_backward(Ws, coefs, rows, shat, gpsi):
+    """(g_pair (E,H,4,64), [gW_enc]) for upstream gpsi (E,H,Dh): the rows W^T gpsi the library's backward takes per
+    pair, and the weight gradients gpsi (x) shat summed over the pairs of a weight set."""
+    E, H = shat.shape[:2]
+    g_pair = torch.zeros((E, H, 4, shat.shape[-1]), dtype=torch.float32, device=shat.device)
+    gWs = [None if W is None else torch.zeros(W.shape, dtype=torch.float32, device=shat.device) for W in Ws]
+    for s0 in range(0, E, _PAIR_CHUNK):
+        sl = slice(s0, min(E, s0 + _PAIR_CHUNK))
+        for en, (W, c) in enumerate(zip(Ws, coefs)):
+            if W is None:
+                continue
+            bins = W.shape[-1]
+            Wsel = (W[sl] if rows is None else W[rows[sl]]).to(torch.float32)
+            g_pair[sl, :, en, :bins] = c * torch.einsum("ehck,ehc->ehk", Wsel, gpsi[sl])
+            outer = c * torch.einsum("ehc,ehk->ehck", gpsi[sl], shat[sl, :, en, :bins])
+            if rows is None:
+                gWs[en][sl] = outer
+            else:
+                gWs[en].index_add_(0, rows[sl], outer)
+    return g_pair, gWs
+
+
 def _framed_pe_forward(ctx, qk, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, W_k, W_k1,
                        W_k2, W_k3, frame_vecs, dim_angle_enc, value_pe_angle_scale, cos_abs, length_rbf_mul,
                        angle_rbf_mul, rvlen_n, cutoff_radius):
@@ -328,9 +381,22 @@ def _framed_pe_forward(ctx, qk, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K,
     E = edge_ij_e.shape[1]
     dev = a_ik.device
     K = int(K) if W_k is not None else 0
-    Wd = _proj_weight(W_k, H, "W_k") if K > 0 else None
+    sets = _weight_sets(W_k, E, N) if K > 0 else "shared"
     use_angle = K > 0 and W_k1 is not None and int(dim_angle_enc) > 0
     A = int(dim_angle_enc) if use_angle else 0
+    pair_W = None
+    if sets != "shared":
+        # One weight set per pair or per query atom (W_num = E or N in the reference's kernels).  The kernels make z
+        # and the histograms with the first set; psi and, in the backward, W^T gpsi and the weight gradients are
+        # products of the framework over those histograms.
+        if KernelManager.GRAD_COEF_QUIRK:
+            raise NotImplementedError("GRAD_COEF_QUIRK with per-pair / per-atom projection weights")
+        pair_W = [W_k] + ([W_k1, W_k2, W_k3] if use_angle else [None, None, None])
+        for w in pair_W:
+            if w is not None and (w.dim() != 4 or w.shape[0] != W_k.shape[0]):
+                raise ValueError("per-pair / per-atom projection weights: every weight needs the same leading dimension")
+        W_k, W_k1, W_k2, W_k3 = [None if w is None else w[:1] for w in pair_W]
+    Wd = _proj_weight(W_k, H, "W_k") if K > 0 else None
     Wa = [_proj_weight(w, H, "W_k%d" % (n + 1)) for n, w in enumerate((W_k1, W_k2, W_k3))] if use_angle \
         else [None, None, None]
     Dh = Wd.shape[-2] if Wd is not None else 16
@@ -343,7 +409,7 @@ def _framed_pe_forward(ctx, qk, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K,
     p = _params(H, Dh, K, A, cos_abs, float(dist_max), wscale, value_pe_angle_scale,
                 length_rbf_mul, angle_rbf_mul, cutoff_radius if rv is not None else None)
     shat = None
-    if KernelManager.SAVE_HISTOGRAMS and K > 0 and any(ctx.needs_input_grad):
+    if K > 0 and (pair_W is not None or (KernelManager.SAVE_HISTOGRAMS and any(ctx.needs_input_grad))):
         shat = torch.empty((E, H, 4, K), dtype=torch.float32, device=dev)
     if qk is None:
         frames = _stacked_frames(*frame_vecs) if use_angle else None
@@ -367,6 +433,17 @@ def _framed_pe_forward(ctx, qk, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K,
                 _lib.ptr(Wa[1]), _lib.ptr(Wa[2]), N, E, tv.shape[0], _lib.ptr(frames), _lib.ptr(z), _lib.ptr(v),
                 None, _lib.ptr(shat), _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
         _lib.check(rc, "cfh_frame_axes_framed_pe_forward")
+    ctx.pairwise = None
+    if pair_W is not None:
+        rows = None if sets == "edge" else edges[0]
+        coefs = (float(length_rbf_mul), float(angle_rbf_mul), float(angle_rbf_mul), float(angle_rbf_mul))
+        v = _pairwise_psi([None if w is None else w.detach() for w in pair_W], coefs, rows, shat, Dh)
+        ctx.pairwise = (sets, coefs)
+        ctx.save_for_backward(a, rpos, tv, rv, batch, edges, e_start, order, *[None if w is None else w.detach() for w in pair_W],
+                              frames if use_angle else None, z, shat)
+        ctx.params = p
+        ctx.w_shapes = [None if w is None else w.shape for w in pair_W]
+        return z, v, frames
     ctx.save_for_backward(a, rpos, tv, rv, batch, edges, e_start, order, Wd, Wa[0], Wa[1], Wa[2],
                           frames if use_angle else None, z, shat)
     ctx.params = p
@@ -383,6 +460,20 @@ def _framed_pe_backward(ctx, gz_ek, gv_ekd):
     E = edges.shape[1]
     dev = a.device
     gz = _f32c(gz_ek) if gz_ek is not None else torch.zeros_like(z)
+    if getattr(ctx, "pairwise", None) is not None:
+        sets, coefs = ctx.pairwise
+        Ws = [Wd, W1, W2, W3]
+        gpsi = _f32c(gv_ekd) if gv_ekd is not None else torch.zeros((E, H, Wd.shape[-2]), dtype=torch.float32, device=dev)
+        g_pair, gWs = _pairwise_backward(Ws, coefs, None if sets == "edge" else edges[0], shat, gpsi)
+        ga = torch.empty((N, H), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev), _timed("framed_pe_backward", dev):
+            ws = _lib.workspace(dev, lib.cfh_workspace_bytes(ctypes.byref(p), N, E))
+            rc = lib.cfh_framed_pe_backward_pairwise(
+                ctypes.byref(p), _lib.ptr(a), _lib.ptr(rpos), _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges),
+                _lib.ptr(e_start), _lib.ptr(order), _lib.ptr(frames), _lib.ptr(z), _lib.ptr(gz), _lib.ptr(g_pair), N, E,
+                tv.shape[0], _lib.ptr(ga), _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
+        _lib.check(rc, "cfh_framed_pe_backward_pairwise")
+        return ga, [g if g is None else g.to(w.dtype) for g, w in zip(gWs, Ws)]
     gv = None
     if Wd is not None:
         gv = _f32c(gv_ekd) if gv_ekd is not None else torch.zeros((E, H, Wd.shape[-2]), dtype=torch.float32, device=dev)

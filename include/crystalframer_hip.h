@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 9
+#define CFH_ABI_VERSION 10
 
 enum {
     CFH_OK = 0,
@@ -276,6 +276,21 @@ int cfh_fused_dpa_backward(const float* q, const float* k, const float* v, const
                            const float* prob, const float* out, const float* gout, int64_t N,
                            int64_t H, int64_t Dh, int64_t E, float* gq, float* gk, float* gv,
                            float* gaij, float* gbij, void* stream);
+
+/*
+ * ga (N,H) of cfh_framed_pe_backward when the projection weights differ from pair to pair (W_num = E or N in
+ * models/kernels/real_enc_frame_proj_bwd_length.cu:166-173, models/cuda_funcs/real_space_framed_proj.py:156): the
+ * kernel needs the weights only through the rows g = W^T gpsi, which the caller makes for every pair,
+ *     g_pair[e,h,0,k] = dist_coef  sum_c W_dist[w(e),h,c,k] gpsi[e,h,c],
+ *     g_pair[e,h,1+axis,k] = angle_coef sum_c W_axis[w(e),h,c,k] gpsi[e,h,c]        (E,H,4,64; unused rows and, for a
+ * 16-bin angle basis, the entries beyond the bins: zero), and the weight gradients are outer products of gpsi and the
+ * histograms of the forward (shat), the caller's as well.  frames NULL: no angle encoding.
+ */
+int cfh_framed_pe_backward_pairwise(const cfh_params* p, const float* a_ih, const float* rpos, const float* tvecs,
+                                    const float* rvlen, const int64_t* batch, const int64_t* edges,
+                                    const int64_t* e_start, const int32_t* order, const float* frames, const float* z,
+                                    const float* gz, const float* g_pair, int64_t N, int64_t E, int64_t B, float* ga,
+                                    void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * The attention core of a layer in one call: lattice sums, softmax over the pairs of every atom and the value

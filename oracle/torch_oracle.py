@@ -190,7 +190,8 @@ def framed_pe(a_ih, rpos, tvecs, batch, edges, W_k, W_axes, frames, *, K=64, dis
     """z (E,H) and psi (E,H,Dh) of RealEncodingWithFramedProjFuncCUDA.forward.
 
     models/cuda_funcs/real_space_framed_proj.py:21-120 with the two kernels it launches.
-    ``W_k`` (1,H,Dh,K) or None; ``W_axes`` sequence of three (1,H,Dh,A) or None;
+    ``W_k`` (W_num,H,Dh,K) or None; ``W_axes`` sequence of three (W_num,H,Dh,A) or None, W_num = 1 (one shared
+    set), E (one set per pair) or N (one per query atom): models/kernels/real_enc_frame_proj_fwd_length.cu:166-173;
     ``frames`` sequence of three (N,H,3).  ``windows``: "reference" (9/33-bin truncation, the
     kernel's), "full" (no truncation, the pure-PyTorch layer's), or an explicit (Wl, Wa).
     Differentiable in ``a_ih``, ``W_k`` and ``W_axes`` (float64 autograd = gradient oracle).
@@ -210,6 +211,18 @@ def framed_pe(a_ih, rpos, tvecs, batch, edges, W_k, W_axes, frames, *, K=64, dis
     R = translation_ranges(a_ih, rvlen, batch, cutoff_radius, lattice_range, minimum_range)
     sizes = torch.bincount(batch, minlength=tvecs.shape[0]).tolist()
     Dh = W_k.shape[-2] if W_k is not None else (W_axes[0].shape[-2] if W_axes is not None else 0)
+
+    def weight_of(W, sl_e, bins):
+        """(e,H,Dh,bins) or (H,Dh,bins): the weight set of every pair of the slice (w_ind = 0, e or i)."""
+        if W.dim() == 3 or W.shape[0] == 1:
+            return W.reshape(H, Dh, bins).to(dt)
+        if W.shape[0] == E:
+            return W[sl_e].to(dt)
+        assert W.shape[0] == N, "W_num must be 1, E or N"
+        return W[edges[0, sl_e]].to(dt)
+
+    def project(W, s):
+        return torch.einsum("hck,ehk->ehc", W, s) if W.dim() == 3 else torch.einsum("ehck,ehk->ehc", W, s)
 
     z_out, psi_out, d2min_out, shat_len, shat_ang = [], [], [], [], []
     n_off = 0
@@ -248,7 +261,7 @@ def framed_pe(a_ih, rpos, tvecs, batch, edges, W_k, W_axes, frames, *, K=64, dis
                 s = torch.einsum("eht,etk->ehk", p, g)
                 if return_parts:
                     shat_len.append(s)
-                psi = psi + c_dist * torch.einsum("hck,ehk->ehc", W_k.reshape(H, Dh, K).to(dt), s)
+                psi = psi + c_dist * project(weight_of(W_k, sl_e, K), s)
             if W_axes is not None and A > 0:
                 valid = d2 > 1e-5
                 dsafe = torch.where(valid, d, torch.ones_like(d))
@@ -259,7 +272,7 @@ def framed_pe(a_ih, rpos, tvecs, batch, edges, W_k, W_axes, frames, *, K=64, dis
                     g = _angle_basis(cosv, valid[:, None, :].expand_as(cosv), A, angle_sigma, cos_abs, wa)
                     s = torch.einsum("eht,ehtm->ehm", p, g)
                     s_axes.append(s)
-                    psi = psi + c_angle * torch.einsum("hcm,ehm->ehc", W_axes[ax].reshape(H, Dh, A).to(dt), s)
+                    psi = psi + c_angle * project(weight_of(W_axes[ax], sl_e, A), s)
                 if return_parts:
                     shat_ang.append(torch.stack(s_axes))
             psi_out.append(psi)

@@ -442,3 +442,39 @@ def test_frames_and_lattice_sums_in_one_call_equal_the_two_calls(noise):
         assert float(Wk.grad.abs().max()) == 0.0 and float(Wax[2].grad.abs().max()) == 0.0
     finally:
         KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE = saved
+
+
+@pytest.mark.parametrize("sets", ["edge", "atom"])
+@pytest.mark.parametrize("angle_bins", [64, 16, 0])
+def test_projection_weights_per_pair_and_per_atom(sets, angle_bins):
+    """W_num = E / N of the reference (models/kernels/real_enc_frame_proj_fwd_length.cu:166-173,
+    models/cuda_funcs/real_space_framed_proj.py:150-156): one weight set per pair or per query atom.  z, psi and the
+    gradients of a and of every weight set against the float64 oracle."""
+    import crystalframer_amd as cf
+    P = Hh.make_problem(num_crystals=7, atoms_hi=5, seed=171)
+    num = P.E if sets == "edge" else P.N
+    gen = torch.Generator().manual_seed(3)
+    mk = lambda bins: (torch.randn(num, Hh.H, Hh.DH, bins, generator=gen, dtype=torch.float64) * 0.3).float().double()
+    Wk64 = mk(64)
+    Wax64 = [mk(angle_bins) for _ in range(3)] if angle_bins else None
+    a = g(P.a).requires_grad_(True)
+    Wk = g(Wk64).requires_grad_(True)
+    Wax = [g(w).requires_grad_(True) for w in Wax64] if angle_bins else [None] * 3
+    fr = [g(f) for f in P.frames] if angle_bins else [None] * 3
+    cd, ca, ws = 0.75, 1.25, (4.0 if angle_bins != 16 else 1.0)
+    z, psi = cf.RealEncodingWithFramedProjFuncCUDA.apply(
+        a, g(P.rpos), None, g(P.tvecs), P.batch.to(dev()), P.edges.to(dev()), 64, Hh.DIST_MAX, 1.0, Wk, Wax[0], Wax[1],
+        Wax[2], fr[0], fr[1], fr[2], angle_bins, ws, 0, cd, ca, g(P.rvlen), CUT)
+    ao = P.a.clone().requires_grad_(True)
+    Wko = Wk64.clone().requires_grad_(True)
+    Waxo = [w.clone().requires_grad_(True) for w in Wax64] if angle_bins else None
+    zo, psio = TO.framed_pe(ao, P.rpos, P.tvecs, P.batch, P.edges, Wko, Waxo, P.frames, K=64, A=angle_bins,
+                            angle_wscale=ws, c_dist=cd, c_angle=ca, rvlen=P.rvlen, cutoff_radius=CUT)
+    assert Hh.rel_err(z, zo) < 2e-5 and Hh.rel_err(psi, psio) < 2e-5
+    ((z * g(P.gz)).sum() + (psi * g(P.gpsi)).sum()).backward()
+    ((zo * P.gz).sum() + (psio * P.gpsi).sum()).backward()
+    assert Hh.rel_err(a.grad, ao.grad) < 5e-5
+    assert Wk.grad.shape == Wk.shape and Hh.rel_err(Wk.grad, Wko.grad) < 5e-5
+    if angle_bins:
+        for x, y in zip(Wax, Waxo):
+            assert Hh.rel_err(x.grad, y.grad) < 5e-5

@@ -424,3 +424,28 @@ def test_gaussian_coefficient_closed_form_facts():
     # other constants: the limit and the slope follow lb and beta
     a2 = TO.gaussian_coefficient(torch.tensor([-1e4, 2.0], dtype=torch.float64), 2.0, 0.25, 0.3)
     assert abs(float(a2[0]) - 0.25 * (-0.125)) < 1e-15 and abs(float(a2[1]) - 1.6 * (-0.125)) < 1e-15
+
+
+def test_per_pair_weight_sets_reduce_to_the_shared_set_and_select_by_pair_or_atom():
+    """W_num = E / N (models/kernels/real_enc_frame_proj_fwd_length.cu:166-173): equal sets give the shared result;
+    with distinct sets pair e uses set e (or the set of its query atom): checked by projecting the shared run's
+    histograms by hand."""
+    P = Hh.make_problem(num_crystals=3, atoms_hi=4, seed=5)
+    kw = dict(rvlen=P.rvlen, cutoff_radius=-3.5)
+    z, psi, parts = TO.framed_pe(P.a, P.rpos, P.tvecs, P.batch, P.edges, P.W_k, P.W_ax, P.frames, return_parts=True, **kw)
+    for num in (P.E, P.N):
+        rep = lambda w: w.expand(num, *w.shape[1:]).clone()
+        z2, psi2 = TO.framed_pe(P.a, P.rpos, P.tvecs, P.batch, P.edges, rep(P.W_k), [rep(w) for w in P.W_ax], P.frames, **kw)
+        assert (z2 - z).abs().max() == 0 and (psi2 - psi).abs().max() < 1e-14
+        gen = torch.Generator().manual_seed(num)
+        Wk = torch.randn(num, Hh.H, Hh.DH, Hh.K, generator=gen, dtype=torch.float64)
+        Wax = [torch.randn(num, Hh.H, Hh.DH, Hh.A, generator=gen, dtype=torch.float64) for _ in range(3)]
+        _, psi3 = TO.framed_pe(P.a, P.rpos, P.tvecs, P.batch, P.edges, Wk, Wax, P.frames, **kw)
+        rows = torch.arange(P.E) if num == P.E else P.edges[0]
+        want = torch.zeros_like(psi3)
+        for e in range(P.E):
+            for h in range(Hh.H):
+                want[e, h] = Wk[rows[e], h] @ parts["shat_len"][e, h]
+                for ax in range(3):
+                    want[e, h] += Wax[ax][rows[e], h] @ parts["shat_ang"][ax, e, h]
+        assert (psi3 - want).abs().max() < 1e-12
