@@ -40,7 +40,8 @@ PEAK_TRANS_TOPS = 9.8                  # quarter-rate transcendental unit
 # FETCH_SIZE / WRITE_SIZE (KiB per dispatch) scaled by what the same counters read for the 256 MiB device copy of
 # --calibrate-copy; the figures and the commands are in TRAFFIC_SOURCE.  Other batch sizes or settings: null.
 TRAFFIC_SOURCE = "profiles/fused_core_hbm_traffic_C3.md"
-TRAFFIC_BYTES_PER_LAUNCH = {"fused_core_forward": None, "fused_core_backward": None, "frame_axes": None}
+# forward 9 303.3 KiB x 2.0 + 92 161.6 KiB; backward 54 966.6 x 2.0 + 9 303.1; frame search 8 197.4 x 2.0 + 2 392.1
+TRAFFIC_BYTES_PER_LAUNCH = {"fused_core_forward": 113.4e6, "fused_core_backward": 122.1e6, "frame_axes": 19.2e6}
 
 
 def parse():
@@ -314,15 +315,16 @@ def main():
     fused = "fused_core_forward" in kern_ms
     traffic = TRAFFIC_BYTES_PER_LAUNCH.get(dom["kernel"][:-len("_kernel")]) if (args.batch == 256 and fused) else None
     roofline = {
-        "kernel": dom["kernel"], "bound": "valu-issue/latency",
+        "kernel": dom["kernel"], "bound": "valu-issue",
         "achieved": dom["achieved"], "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac"], "traffic": traffic,
         "traffic_source": TRAFFIC_SOURCE if traffic is not None else None,
         "bound_detail": "ALGORITHMIC FP32 flop of the reference formulation (what its kernels would execute for the terms "
                         "this kernel evaluates) against the published 157.3 TFLOP/s vector peak.  The kernel does not "
                         "execute that many: the angle encoding is scattered as 5 local moments per axis instead of a "
                         "33-bin window and the projection runs once per (atom, head) in a separate MFMA kernel.  What "
-                        "binds it is instruction issue and latency of small work items (one wavefront per (atom, "
-                        "head), 12.5 pairs on average): vector ALU busy about half of the time, HBM far from its peak",
+                        "binds it is the issue of vector instructions, few of which are multiply-adds (one wavefront per "
+                        "(atom, head), 12.5 pairs on average): vector ALUs issuing 52-66 % of the kernel's time with 86 % "
+                        "of the lanes active, HBM at a fifth of its peak (profiles/fused_core_valu_lds_counters_C3.md)",
         "both_kernels": {k: {"kernel": r["kernel"], "achieved": r["achieved"], "frac": r["frac"],
                              "avg_launch_ms": r["avg_launch_ms"]} for k, r in roof.items()},
         "frac_of_unpacked_fp32_peak": dom["achieved"] / PEAK_FP32_UNPACKED,
