@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
@@ -74,6 +74,12 @@ class CfhLinearGradJob(ctypes.Structure):
                 ("ldy", ctypes.c_int64)]
 
 
+class CfhAdamWJob(ctypes.Structure):
+    """Mirror of ``cfh_adamw_job`` in include/crystalframer_hip.h."""
+    _fields_ = [("param", ctypes.c_void_p), ("grad", ctypes.c_void_p), ("exp_avg", ctypes.c_void_p),
+                ("exp_avg_sq", ctypes.c_void_p), ("n", ctypes.c_int64)]
+
+
 EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_frame_axis1",
            "cfh_frame_axis2", "cfh_frame_axes", "cfh_framed_pe_forward", "cfh_framed_pe_forward_static", "cfh_frame_axes_framed_pe_forward",
            "cfh_framed_pe_backward", "cfh_framed_pe_backward_pairwise",
@@ -83,7 +89,7 @@ EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_fram
            "cfh_attention_inputs_backward", "cfh_layer_bridge_forward", "cfh_layer_bridge_backward",
            "cfh_second_stream_fork", "cfh_second_stream_get", "cfh_second_stream_join",
            "cfh_fused_core_workspace_bytes", "cfh_fused_core_hist_words", "cfh_fused_core_forward",
-           "cfh_fused_core_backward")
+           "cfh_fused_core_backward", "cfh_adamw_step_batch")
 
 _lib = None
 _lock = threading.Lock()
@@ -147,6 +153,9 @@ def load():
         lib.cfh_linear_weight_bias_grad.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P, _P]
         lib.cfh_small_linear_forward.restype = ctypes.c_int
         lib.cfh_small_linear_forward.argtypes = [_P, _P, _P, _I64, _I64, _I64, ctypes.c_int32, _P, _P]
+        lib.cfh_adamw_step_batch.restype = ctypes.c_int
+        lib.cfh_adamw_step_batch.argtypes = [_P, ctypes.c_int32, ctypes.c_float, ctypes.c_float, ctypes.c_float,
+                                             ctypes.c_float, ctypes.c_float, _P, _P]
         lib.cfh_small_linear_dx.restype = ctypes.c_int
         lib.cfh_small_linear_dx.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P]
         lib.cfh_crystal_geometry.restype = ctypes.c_int

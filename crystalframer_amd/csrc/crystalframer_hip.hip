@@ -26,6 +26,7 @@
 #include "linear_grad.hpp"
 #include "small_gemm.hpp"
 #include "layer_bridge.hpp"
+#include "adamw.hpp"
 
 namespace {
 
@@ -1155,6 +1156,41 @@ int cfh_small_linear_dx(const float* dy, const float* W, int64_t M, int64_t N, i
     return finish_launch("small_linear_dx");
 }
 
+int cfh_adamw_step_batch(const cfh_adamw_job* jobs, int32_t njobs, float lr, float beta1, float beta2, float eps,
+                         float weight_decay, uint64_t* step_dev, void* stream) {
+    if (njobs < 0 || (njobs > 0 && !jobs)) return fail(CFH_EINVAL, "jobs is NULL or njobs negative");
+    if (!step_dev) return fail(CFH_EINVAL, "step_dev must not be NULL");
+    if (!(beta1 >= 0.0f && beta1 < 1.0f && beta2 >= 0.0f && beta2 < 1.0f && eps >= 0.0f))
+        return fail(CFH_EINVAL, "adamw: beta1 = %g, beta2 = %g must lie in [0, 1), eps = %g must not be negative", beta1, beta2, eps);
+    for (int32_t j = 0; j < njobs; j++) {
+        const cfh_adamw_job& J = jobs[j];
+        if (J.n < 0 || J.n > 0x7fffffffLL - cfh::ADAMW_BLOCK_ELEMS)
+            return fail(CFH_EINVAL, "adamw job %d: n = %lld out of range", (int)j, (long long)J.n);
+        if (J.n > 0 && (!J.param || !J.grad || !J.exp_avg || !J.exp_avg_sq))
+            return fail(CFH_EINVAL, "adamw job %d: param, grad, exp_avg, exp_avg_sq must not be NULL", (int)j);
+    }
+    hipStream_t st = (hipStream_t)stream;
+    int32_t j = 0;
+    while (j < njobs) {
+        cfh::AdamWJobs T{};
+        T.lr = lr; T.beta1 = beta1; T.beta2 = beta2; T.eps = eps; T.wd = weight_decay;
+        T.step = reinterpret_cast<const unsigned long long*>(step_dev);
+        long blocks = 0;
+        for (; j < njobs && T.njobs < cfh::ADAMW_MAX_JOBS; j++) {
+            if (jobs[j].n == 0) continue;
+            const long nb = (long)((jobs[j].n + cfh::ADAMW_BLOCK_ELEMS - 1) / cfh::ADAMW_BLOCK_ELEMS);
+            if (blocks + nb > 0x7fffffffL) break;
+            cfh::AdamWJob& W = T.job[T.njobs++];
+            W.p = jobs[j].param; W.g = jobs[j].grad; W.m = jobs[j].exp_avg; W.v = jobs[j].exp_avg_sq;
+            W.n = (int)jobs[j].n; W.block0 = (int)blocks;
+            blocks += nb;
+        }
+        if (T.njobs == 0) break;
+        hipLaunchKernelGGL(cfh::adamw_batch_kernel, dim3((unsigned)blocks), dim3(256), 0, st, T);
+    }
+    hipLaunchKernelGGL(cfh::adamw_advance_kernel, dim3(1), dim3(1), 0, st, reinterpret_cast<unsigned long long*>(step_dev));
+    return finish_launch("adamw_step_batch");
+}
 
 }  // extern "C"
 

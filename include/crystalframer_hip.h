@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 10
+#define CFH_ABI_VERSION 11
 
 enum {
     CFH_OK = 0,
@@ -439,6 +439,28 @@ typedef struct cfh_linear_grad_job {
     int64_t N, I, O, ldx, ldy;
 } cfh_linear_grad_job;
 int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t njobs, void* stream);
+
+/*
+ * One AdamW step (decoupled weight decay, bias-corrected moments; the update rule of torch.optim.AdamW without
+ * amsgrad / maximize) for several parameter tensors in one launch:
+ *     p *= 1 - lr wd;  m = b1 m + (1 - b1) g;  v = b2 v + (1 - b2) g^2;
+ *     p -= lr / (1 - b1^t) * m / (sqrt(v) / sqrt(1 - b2^t) + eps),   t = *step_dev + 1
+ * and *step_dev (device memory: the steps taken so far, 0 before the first) is advanced by one afterwards, on the
+ * stream, so that a captured call keeps counting from replay to replay.  Every tensor is contiguous float32 with n
+ * elements.  `jobs` is a host array; it is copied into the kernel arguments, 80 tensors per launch.  The model of
+ * the benchmark has 65 small tensors (0.95 M elements): the framework's multi-tensor kernel takes 2 launches of
+ * 43 us for them, bound by its per-tensor bookkeeping.  No counterpart in the reference (torch.optim.AdamW in its
+ * trainer, train.py); it is here because the measured training step contains the update.
+ */
+typedef struct cfh_adamw_job {
+    float* param;
+    const float* grad;
+    float* exp_avg;
+    float* exp_avg_sq;
+    int64_t n;
+} cfh_adamw_job;
+int cfh_adamw_step_batch(const cfh_adamw_job* jobs, int32_t njobs, float lr, float beta1, float beta2, float eps,
+                         float weight_decay, uint64_t* step_dev, void* stream);
 
 /*
  * Projections with few rows (one per crystal: the head after pooling), where the general GEMM runs on
