@@ -46,7 +46,10 @@ constexpr int FC_SHIFT = 7;                     // list entry = pair-in-group <<
 #endif
 constexpr int NORD = CFH_NORD;                  // moments per axis
 constexpr int CORE_WPB = 1;                     // wavefronts per workgroup of the main kernels: each takes an item of its
-                                                // own (no barriers); dispatching one-wavefront workgroups is slower than the items are
+                                                // own (no barriers).  Workgroups of 4 or 8 items of one head that make the
+                                                // products with the head's weights themselves (projection, G) were slower:
+                                                // +25 us per kernel for the phases behind barriers, against 21 + 20 us for
+                                                // the two separate launches
 constexpr int FC_LOGCAP = 256;                  // logits of a row kept in LDS until the row is complete
 constexpr int HW_DIST = NBINS;
 constexpr int HW_ANG = NBINS * (1 + 3 * NORD);  // 1024 words per (atom, head) with the angle encoding
@@ -104,7 +107,12 @@ __device__ __forceinline__ float rows8_sum(float x) {
     x += dpp_move<0x128>(x);          // row_ror 8: the other half of the 16-lane row
     return rows_sum(x);
 }
-__device__ __forceinline__ int rint_i(float x) { return (int)__builtin_rintf(x); }
+// float -> fixed point, round to nearest (floor(x + 0.5)) in ONE instruction (rintf + conversion are two)
+__device__ __forceinline__ int rint_i(float x) {
+    int r;
+    asm("v_cvt_rpi_i32_f32 %0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
 
 // ---- sorted shifts of the usual box, one table per crystal ---------------------------------------------------
 // block = crystal, 128 threads; entry = (shift, |shift|), ascending length (ties: loop order); entries beyond the
@@ -633,8 +641,8 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
 }
 
 // out (N,H,16) += Wcat_h (16, hw) . hist (H,N,hw): one workgroup of PROJ_WAVES wavefronts per (16 atoms, head); each
-// wavefront takes a slice of the reduction index through MFMA 16x16x4 (a lane owns 16 consecutive words of each
-// 64-word step: 64-byte loads of its row), the slices meet in LDS and are added in a fixed order by the first
+// wavefront takes a slice of the reduction index through MFMA 16x16x4 (the four lanes of a row read 64 consecutive
+// bytes of it per load), the slices meet in LDS and are added in a fixed order by the first
 // wavefront (no atomics: the result does not depend on timing).  grid (ceil(N/16), H), block 64 * PROJ_WAVES.
 constexpr int PROJ_WAVES = 4;
 __global__ __launch_bounds__(WAVE * PROJ_WAVES) void core_project_kernel(const float* __restrict__ hist,
@@ -644,8 +652,10 @@ __global__ __launch_bounds__(WAVE * PROJ_WAVES) void core_project_kernel(const f
     const int lane = threadIdx.x & (WAVE - 1), wv = threadIdx.x >> 6, col = lane & 15, kk = lane >> 4;
     const int h = blockIdx.y, i0 = blockIdx.x * 16;
     const int row = min(i0 + col, N - 1);
-    const float4* ap = reinterpret_cast<const float4*>(hist + ((size_t)h * N + row) * hw) + 4 * kk;
-    const float4* bp = reinterpret_cast<const float4*>(wcat + ((size_t)h * DH + col) * hw) + 4 * kk;
+    // the four lanes (kk) of a row read 64 consecutive bytes per load; which word of the reduction index a lane
+    // holds does not matter as long as both operands agree
+    const float4* ap = reinterpret_cast<const float4*>(hist + ((size_t)h * N + row) * hw) + kk;
+    const float4* bp = reinterpret_cast<const float4*>(wcat + ((size_t)h * DH + col) * hw) + kk;
     v4f_c acc = {0.f, 0.f, 0.f, 0.f};
     const int steps = hw / 64, per = (steps + PROJ_WAVES - 1) / PROJ_WAVES;
     const int s_begin = wv * per, s_end = min(steps, s_begin + per);
@@ -653,7 +663,7 @@ __global__ __launch_bounds__(WAVE * PROJ_WAVES) void core_project_kernel(const f
     for (int s = s_begin; s < s_end; s++) {
         float4 a4[4], b4[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++) { a4[u] = ap[16 * s + u]; b4[u] = bp[16 * s + u]; }
+        for (int u = 0; u < 4; u++) { a4[u] = ap[16 * s + 4 * u]; b4[u] = bp[16 * s + 4 * u]; }
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[u].x, b4[u].x, acc, 0, 0, 0);
@@ -832,8 +842,8 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
         const float2 ov2 = *reinterpret_cast<const float2*>(C.outv + ih * DH + 2 * sub);
         const float c0 = half_sum(fmaf(go2.x, ov2.x, go2.y * ov2.y));          // go . out_i
         const float gnorm = uniform_f(wave_sum(gabs));                          // |bg| <= sum |G|
-        const float bscale = 1073741824.0f / fmaxf(gnorm, 1e-30f);
-        const float binv = fmaxf(gnorm, 1e-30f) * (1.0f / 1073741824.0f);
+        const float bscale = 1073741824.0f / fmaxf(gnorm, 1e-20f);      // (finite: 2^30 / 1e-30 would not be)
+        const float binv = fmaxf(gnorm, 1e-20f) * (1.0f / 1073741824.0f);
         wave_sync();
         float cov = 0.0f;
         float2 gq2 = make_float2(0.f, 0.f);
