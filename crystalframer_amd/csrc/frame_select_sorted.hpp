@@ -55,7 +55,10 @@ __device__ __forceinline__ void build_sorted_chunk(float4* tab, int t0, int cnt,
     }
     wave_sync();
     int rank[2] = {0, 0};
-    for (int j = 0; j < cnt; j++) {
+    // (entries beyond cnt hold +inf and count for nobody; eight reads in flight: the loop waited for one LDS round
+    // trip per key otherwise)
+#pragma unroll 8
+    for (int j = 0; j < FC_TCAP; j++) {
         const float kj = tab[j].w;         // the keys differ in their low bits: no ties
         rank[0] += kj < ent[0].w ? 1 : 0;
         rank[1] += kj < ent[1].w ? 1 : 0;
@@ -79,7 +82,7 @@ __device__ __forceinline__ int wave_scan_incl(int x) {
 }
 
 struct FrameShared {
-    float4 tab[FC_TCAP];
+    float4 tab[2 * FC_TCAP];     // the sorted table, or the sorted chunks of a box of its own (two stay resident)
     float4 pq[WAVE];             // rpos and q.k of the staged pairs
     int pstart[WAVE + 1];        // first candidate of every staged pair, then the total
 };
@@ -103,6 +106,12 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
 
     const int it_cur = wid / H;      // one wavefront per item, long items first
     if (it_cur >= P.N) return;
+#ifdef CFH_FRAME_PHASES
+    unsigned long long fp_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, fp_last = __builtin_amdgcn_s_memtime(); int fp_cur = 0;
+#define FP(n) do { const unsigned long long fp_t = __builtin_amdgcn_s_memtime(); fp_acc[fp_cur] += fp_t - fp_last; fp_last = fp_t; fp_cur = (n); } while (0)
+#else
+#define FP(n) do { } while (0)
+#endif
     {
         const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
         const Item item = unpack_item(rec_cur);
@@ -119,6 +128,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                             a < 0.0f;
         if (others_only && sorted && item.npairs <= FQ_MAX_PAIRS) return;      // searched four heads at a time
         const int nchunks = sorted ? 1 : (bx.T + FC_TCAP - 1) / FC_TCAP;
+        const bool resident = nchunks == 2;             // both chunks of the box fit: sorted once, not once per sweep
         const int e0 = item.e0, npairs = item.npairs;
         const float nz = noisy ? P.noise : 0.0f;
         const float sq_nz = sqrtf(nz);
@@ -149,6 +159,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                     const int npc = min(WAVE, npairs - pb);
                     // stage rpos and q_i.k_j of the pairs, one per lane (a row that fits stays staged for all sweeps;
                     // the pairs of an atom point at consecutive atoms)
+                    FP(1);
                     float4 rq = make_float4(0.f, 0.f, 0.f, 0.f);
                     // (made for the table's box, which every other box of the launch contains: an upper bound there)
                     if (sw == 0 && C.pair_near && lane < npc) dvalid = C.pair_near[e0 + pb + lane].y;
@@ -174,6 +185,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                         rq = pq[lane];
                     }
                     // how far into the sorted table this lane's pair has to look
+                    FP(2);
                     float reach = 3.0e38f;
                     if (a < 0.0f) {
                         const float r2 = fmaf(rq.x, rq.x, fmaf(rq.y, rq.y, rq.z * rq.z));
@@ -191,9 +203,12 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                     for (int ch = 0; ch < nchunks; ch++) {
                         const int t0c = ch * FC_TCAP;
                         const int cnt = sorted ? bx.T : min(FC_TCAP, bx.T - t0c);
-                        if (nchunks > 1) {
+                        float4* const tabc = resident ? tab + ch * FC_TCAP : tab;
+                        if (nchunks > 1 && !(resident && (pass > 0 || sw > 0 || pb > 0))) {
+                            FP(4);
                             wave_sync();
-                            build_sorted_chunk(tab, t0c, cnt, bx, L, lane);
+                            build_sorted_chunk(tabc, t0c, cnt, bx, L, lane);
+                            FP(2);
                         }
                         wave_sync();              // pq, the table; the readers of pstart are done
                         // the bound sweep of the second axis looks at the candidates of the first axis' sweep: when
@@ -205,7 +220,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
 #pragma unroll
                             for (int s = 0; s < 8; s++) {      // the count is one of 0 .. 128: eight halvings
                                 const int mid = min((lo + hi) >> 1, FC_TCAP - 1);
-                                const bool le = lo < hi && tab[mid].w <= reach;
+                                const bool le = lo < hi && tabc[mid].w <= reach;
                                 lo = le ? mid + 1 : lo;
                                 hi = le ? hi : mid;
                             }
@@ -223,7 +238,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                             total = uniform_i(pstart[WAVE]);
                         }
                         n_seen += (unsigned long long)total;
-
+                        FP(3);
                         for (int base = 0; base < total; base += WAVE) {
                             const int c = base + lane;
                             const bool in = c < total;
@@ -236,7 +251,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                                 hi = le ? hi : mid;
                             }
                             const int pl = in ? lo : 0;
-                            const float4 v = tab[in ? c - pstart[pl] : 0];
+                            const float4 v = tabc[in ? c - pstart[pl] : 0];
                             const float4 cq = pq[pl];
                             const int e = e0 + pb + pl;
                             const int t = t0c + (int)(__float_as_uint(v.w) & (uint32_t)(FC_TCAP - 1));
@@ -264,7 +279,9 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                     }
                 }
             }
+            FP(5);
             wave_best(best);
+            FP(6);
             float vx = 0.f, vy = 0.f, vz = 0.f;
             if (best.e != 0x7fffffff) {
                 float sx, sy, sz;
@@ -281,6 +298,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
             }
             if (pass == 0) { f1x = vx; f1y = vy; f1z = vz; }
             else { f2x = vx; f2y = vy; f2z = vz; }
+            FP(7);
         }
 
         if (lane == 0) {
@@ -299,7 +317,20 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                 r[6] = hx; r[7] = hy; r[8] = hz;
             }
         }
+#ifdef CFH_FRAME_PHASES
+        FP(0);
+        {
+            unsigned long long tot = 0;
+            for (int u = 0; u < 8; u++) tot += fp_acc[u];
+            if (P.stats && lane == 0 && tot > 30000ULL && sorted == (CFH_FRAME_PHASES == 1)) {
+                for (int u = 0; u < 8; u++) atomicAdd(P.stats + 16 + u, fp_acc[u]);
+                atomicAdd(P.stats + 24, 1ULL);
+                atomicAdd(P.stats + 25, n_seen);
+            }
+        }
+#else
         if (P.stats && lane == 0) atomicAdd(P.stats + STAT_FRAME1_RAW, n_seen);      // candidates looked at, both axes
+#endif
     }
 }
 
