@@ -251,8 +251,6 @@ def read_stats(device: torch.device, reset: bool = False) -> dict:
     out = dict(zip(STAT_NAMES, vals))
     if any(vals[16:24]):        # cycle counts of a diagnostics build (phase timing of the fused forward kernel)
         out["phase_cycles"] = vals[16:24]
-    if any(vals[24:32]):        # per-wavefront timing of a diagnostics build
-        out["wave_cycles"] = vals[24:32]
     return out
 
 

@@ -106,12 +106,6 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
 
     const int it_cur = wid / H;      // one wavefront per item, long items first
     if (it_cur >= P.N) return;
-#ifdef CFH_FRAME_PHASES
-    unsigned long long fp_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, fp_last = __builtin_amdgcn_s_memtime(); int fp_cur = 0;
-#define FP(n) do { const unsigned long long fp_t = __builtin_amdgcn_s_memtime(); fp_acc[fp_cur] += fp_t - fp_last; fp_last = fp_t; fp_cur = (n); } while (0)
-#else
-#define FP(n) do { } while (0)
-#endif
     {
         const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
         const Item item = unpack_item(rec_cur);
@@ -159,7 +153,6 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                     const int npc = min(WAVE, npairs - pb);
                     // stage rpos and q_i.k_j of the pairs, one per lane (a row that fits stays staged for all sweeps;
                     // the pairs of an atom point at consecutive atoms)
-                    FP(1);
                     float4 rq = make_float4(0.f, 0.f, 0.f, 0.f);
                     // (made for the table's box, which every other box of the launch contains: an upper bound there)
                     if (sw == 0 && C.pair_near && lane < npc) dvalid = C.pair_near[e0 + pb + lane].y;
@@ -185,7 +178,6 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                         rq = pq[lane];
                     }
                     // how far into the sorted table this lane's pair has to look
-                    FP(2);
                     float reach = 3.0e38f;
                     if (a < 0.0f) {
                         const float r2 = fmaf(rq.x, rq.x, fmaf(rq.y, rq.y, rq.z * rq.z));
@@ -205,10 +197,8 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                         const int cnt = sorted ? bx.T : min(FC_TCAP, bx.T - t0c);
                         float4* const tabc = resident ? tab + ch * FC_TCAP : tab;
                         if (nchunks > 1 && !(resident && (pass > 0 || sw > 0 || pb > 0))) {
-                            FP(4);
                             wave_sync();
                             build_sorted_chunk(tabc, t0c, cnt, bx, L, lane);
-                            FP(2);
                         }
                         wave_sync();              // pq, the table; the readers of pstart are done
                         // the bound sweep of the second axis looks at the candidates of the first axis' sweep: when
@@ -238,7 +228,6 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                             total = uniform_i(pstart[WAVE]);
                         }
                         n_seen += (unsigned long long)total;
-                        FP(3);
                         for (int base = 0; base < total; base += WAVE) {
                             const int c = base + lane;
                             const bool in = c < total;
@@ -279,9 +268,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                     }
                 }
             }
-            FP(5);
             wave_best(best);
-            FP(6);
             float vx = 0.f, vy = 0.f, vz = 0.f;
             if (best.e != 0x7fffffff) {
                 float sx, sy, sz;
@@ -298,7 +285,6 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
             }
             if (pass == 0) { f1x = vx; f1y = vy; f1z = vz; }
             else { f2x = vx; f2y = vy; f2z = vz; }
-            FP(7);
         }
 
         if (lane == 0) {
@@ -317,20 +303,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                 r[6] = hx; r[7] = hy; r[8] = hz;
             }
         }
-#ifdef CFH_FRAME_PHASES
-        FP(0);
-        {
-            unsigned long long tot = 0;
-            for (int u = 0; u < 8; u++) tot += fp_acc[u];
-            if (P.stats && lane == 0 && tot > 30000ULL && sorted == (CFH_FRAME_PHASES == 1)) {
-                for (int u = 0; u < 8; u++) atomicAdd(P.stats + 16 + u, fp_acc[u]);
-                atomicAdd(P.stats + 24, 1ULL);
-                atomicAdd(P.stats + 25, n_seen);
-            }
-        }
-#else
         if (P.stats && lane == 0) atomicAdd(P.stats + STAT_FRAME1_RAW, n_seen);      // candidates looked at, both axes
-#endif
     }
 }
 

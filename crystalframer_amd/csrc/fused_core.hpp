@@ -71,21 +71,6 @@ typedef float v4f_c __attribute__((ext_vector_type(4)));
 #define CFH_PH_FLUSH(stats) do { } while (0)
 #endif
 
-// Optional per-wavefront timing (compile with -DCFH_WAVE_TIMING=1 frame search, 2 forward, 3 backward; diagnostics
-// builds only): statistics slots 24.. = sum and maximum of the wavefronts' durations for two kinds of wavefront,
-// the latest start (as its complement: earliest) and end of a wavefront, and the wavefronts that took > 2000 cycles.
-#ifdef CFH_WAVE_TIMING
-#define CFH_WT_BEGIN(which) const unsigned long long wt_t0 = (CFH_WAVE_TIMING == (which)) ? __builtin_amdgcn_s_memtime() : 0ULL;
-#define CFH_WT_END(which, stats, kind) do { if (CFH_WAVE_TIMING == (which) && (stats) && (threadIdx.x & 63) == 0 && ((blockIdx.x & 31) == 0 || blockIdx.x < 64 || blockIdx.x + 64 >= gridDim.x)) { \
-        const unsigned long long wt_t1 = __builtin_amdgcn_s_memtime(), wt_d = wt_t1 - wt_t0; \
-        atomicAdd((stats) + 24 + 2 * (kind), wt_d); atomicMax((stats) + 25 + 2 * (kind), wt_d); \
-        atomicMax((stats) + 28, ~wt_t0); atomicMax((stats) + 29, wt_t1); \
-        if (wt_d > 2000ULL) atomicAdd((stats) + 30 + (kind), 1ULL); } } while (0)
-#else
-#define CFH_WT_BEGIN(which)
-#define CFH_WT_END(which, stats, kind) do { } while (0)
-#endif
-
 struct CoreArgs {
     KernelArgs K;                 // geometry, work queues, item records, basis constants
     const float* qs;              // (N,H,16) query, already divided by sqrt(16)
@@ -367,9 +352,6 @@ struct CoreFwdShared {
     float4 pairA[FC_GROUP];      // rx, ry, rz, d2min
     float pairC[FC_GROUP];       // exp(logit - running max) / S in fixed-point units
     float logit_s[FC_LOGCAP];    // logits of the row (rows of more pairs park them in the probability array)
-#ifdef CFH_EXP_PAD
-    char pad[CFH_EXP_PAD];
-#endif
 };
 template <int WL, bool HAS_ANG, bool COS_ABS>
 __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const CoreArgs C) {
@@ -396,7 +378,6 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
 
     const int it_cur = wid / H;      // items in descending order of their pair count: the long ones start first
     if (it_cur >= P.N) return;
-    CFH_WT_BEGIN(2)
     for (int u = lane; u < HWK; u += WAVE) hist[u] = 0;
     wave_sync();
 
@@ -650,16 +631,13 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             }
         }
         CFH_PH_FLUSH(P.stats);
-#ifndef CFH_WAVE_TIMING
         if (P.stats && lane == 0) {
             atomicAdd(P.stats + STAT_FWD_EVAL, n_eval);
             atomicAdd(P.stats + STAT_FWD_RAW, (unsigned long long)bx.T * (unsigned long long)npairs);
             atomicAdd(P.stats + STAT_FWD_PAIRS, (unsigned long long)npairs);
             atomicAdd(P.stats + STAT_FWD_SEEN, n_seen);
         }
-#endif
     }
-    CFH_WT_END(2, P.stats, 0);
 }
 
 // out (N,H,16) += Wcat_h (16, hw) . hist (H,N,hw): one workgroup of PROJ_WAVES wavefronts per (16 atoms, head); each
@@ -836,7 +814,6 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
 
     const int it_cur = wid / H;      // one wavefront per item, long items first
     if (it_cur >= P.N) return;
-    CFH_WT_BEGIN(3)
     {
         const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
         const CoreItem ci = core_unpack(C, rec_cur, true);
@@ -1019,15 +996,12 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
             if (lane < FC_GROUP) *reinterpret_cast<float2*>(C.gq + ih * DH + 2 * sub) = make_float2(gx, gy);
         }
         if (lane == 0) P.out_ga[ih] = cov;
-#ifndef CFH_WAVE_TIMING
         if (P.stats && lane == 0) {
             atomicAdd(P.stats + STAT_BWD_EVAL, n_eval);
             atomicAdd(P.stats + STAT_BWD_RAW, (unsigned long long)bx.T * (unsigned long long)npairs);
             atomicAdd(P.stats + STAT_BWD_PAIRS, (unsigned long long)npairs);
         }
-#endif
     }
-    CFH_WT_END(3, P.stats, 0);
 }
 
 }  // namespace cfh
