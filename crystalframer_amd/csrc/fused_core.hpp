@@ -378,7 +378,12 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
 
     const int it_cur = wid / H;      // items in descending order of their pair count: the long ones start first
     if (it_cur >= P.N) return;
-    for (int u = lane; u < HWK; u += WAVE) hist[u] = 0;
+    if (HWK >= 4 * WAVE) {
+#pragma unroll
+        for (int u = 0; u < HWK / (4 * WAVE); u++) reinterpret_cast<int4*>(hist)[lane + WAVE * u] = make_int4(0, 0, 0, 0);
+    } else {
+        for (int u = lane; u < HWK; u += WAVE) hist[u] = 0;
+    }
     wave_sync();
 
     CFH_PH_DECL
@@ -550,7 +555,19 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             if (gmax > m_run) {
                 if (m_run > -INF) {
                     const float fac = hw_exp2((m_run - gmax) * LOG2E);
-                    for (int u = lane; u < HWK; u += WAVE) hist[u] = rint_i((float)hist[u] * fac);
+                    if (HWK >= 4 * WAVE) {
+                        constexpr int NW = HWK >= 4 * WAVE ? HWK / (4 * WAVE) : 1;
+                        int4 hv[NW];
+#pragma unroll
+                        for (int u = 0; u < NW; u++) hv[u] = reinterpret_cast<const int4*>(hist)[lane + WAVE * u];
+#pragma unroll
+                        for (int u = 0; u < NW; u++)
+                            reinterpret_cast<int4*>(hist)[lane + WAVE * u] =
+                                make_int4(rint_i((float)hv[u].x * fac), rint_i((float)hv[u].y * fac),
+                                          rint_i((float)hv[u].z * fac), rint_i((float)hv[u].w * fac));
+                    } else {
+                        for (int u = lane; u < HWK; u += WAVE) hist[u] = rint_i((float)hist[u] * fac);
+                    }
                     accv.x *= fac; accv.y *= fac; Dl *= fac;
                 }
                 m_run = gmax;
@@ -609,15 +626,22 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             if (lane < FC_GROUP) *reinterpret_cast<float2*>(C.out + ih * DH + 2 * sub) = make_float2(ox, oy);
         }
         {
-            // all reads first (one LDS round trip instead of one per word), then clear and store
-            constexpr int NW = HWK / WAVE;
+            // all reads first (one LDS round trip instead of one per word), then store; a lane takes four
+            // consecutive words at a time
             const float sc = inv * (float)max(npairs, 1) * (1.0f / 1073741824.0f);
-            float* dst = C.hist + ((size_t)h * P.N + i) * HWK + lane;      // head-major: the rows of a head are contiguous
-            int32_t hv[NW];
+            float* dst = C.hist + ((size_t)h * P.N + i) * HWK;      // head-major: the rows of a head are contiguous
+            if (HWK >= 4 * WAVE) {
+                constexpr int NW = HWK >= 4 * WAVE ? HWK / (4 * WAVE) : 1;
+                int4 hv[NW];
 #pragma unroll
-            for (int u = 0; u < NW; u++) hv[u] = hist[lane + WAVE * u];
+                for (int u = 0; u < NW; u++) hv[u] = reinterpret_cast<const int4*>(hist)[lane + WAVE * u];
 #pragma unroll
-            for (int u = 0; u < NW; u++) dst[WAVE * u] = (float)hv[u] * sc;
+                for (int u = 0; u < NW; u++)
+                    reinterpret_cast<float4*>(dst)[lane + WAVE * u] =
+                        make_float4((float)hv[u].x * sc, (float)hv[u].y * sc, (float)hv[u].z * sc, (float)hv[u].w * sc);
+            } else {
+                for (int u = lane; u < HWK; u += WAVE) dst[u] = (float)hist[u] * sc;
+            }
         }
         if (npairs <= FC_LOGCAP) {                               // logits -> probabilities
             for (int el = lane; el < npairs; el += WAVE)
@@ -836,7 +860,19 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
         float gabs = 0.0f;
         {
             const float* src = C.G + ((size_t)h * P.N + i) * HWK;
-            for (int u = lane; u < HWK; u += WAVE) { const float g = src[u]; Gs[u] = g; gabs += fabsf(g); }
+            if (HWK >= 4 * WAVE) {
+                constexpr int NW = HWK >= 4 * WAVE ? HWK / (4 * WAVE) : 1;
+                float4 g4[NW];
+#pragma unroll
+                for (int u = 0; u < NW; u++) g4[u] = reinterpret_cast<const float4*>(src)[lane + WAVE * u];
+#pragma unroll
+                for (int u = 0; u < NW; u++) {
+                    reinterpret_cast<float4*>(Gs)[lane + WAVE * u] = g4[u];
+                    gabs += (fabsf(g4[u].x) + fabsf(g4[u].y)) + (fabsf(g4[u].z) + fabsf(g4[u].w));
+                }
+            } else {
+                for (int u = lane; u < HWK; u += WAVE) { const float g = src[u]; Gs[u] = g; gabs += fabsf(g); }
+            }
         }
         const float2 go2 = *reinterpret_cast<const float2*>(C.go + ih * DH + 2 * sub);
         const float2 ov2 = *reinterpret_cast<const float2*>(C.outv + ih * DH + 2 * sub);
