@@ -50,7 +50,7 @@ constexpr int CORE_WPB = 1;                     // wavefronts per workgroup of t
                                                 // products with the head's weights themselves (projection, G) were slower:
                                                 // +25 us per kernel for the phases behind barriers, against 21 + 20 us for
                                                 // the two separate launches
-constexpr int FC_LOGCAP = 256;                  // logits of a row kept in LDS until the row is complete
+constexpr int FC_LOGCAP = 64;                   // logits of a row kept in LDS until the row is complete
 constexpr int HW_DIST = NBINS;
 constexpr int HW_ANG = NBINS * (1 + 3 * NORD);  // 1024 words per (atom, head) with the angle encoding
 constexpr int REC_J0 = 30;                      // item record: first neighbour atom (pairs of an atom are j0, j0+1, ...)
