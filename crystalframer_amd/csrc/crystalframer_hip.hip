@@ -1333,9 +1333,13 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
         }
     }
     C.pair_near = buf.near;
+    float* wcat = buf.wcat;
+    const cfh::WcatArgs WA{W_dist, W_axis1, W_axis2, W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat};
     {
         const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
                                                                                           : p->num_heads * cfh::NQUEUE);
+        const int prep_blocks = (threads + 255) / 256;
+        // the item records and the concatenated weights in one launch
         if (search) {
             // records with the query, frame search through the first set of queues; it leaves the frames in the
             // records and the main kernel takes the second set of queues
@@ -1343,7 +1347,8 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
             F.K.q = qs; F.K.k = k; F.K.out_frame = frames;
             F.K.counters2 = reinterpret_cast<int32_t*>(ws + QUEUE_OFFSET + QUEUE_SET_BYTES);
             F.K.frames_to_records = 1;
-            hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, F.K, 1);
+            hipLaunchKernelGGL(cfh::core_prepare_wcat_kernel, dim3(prep_blocks + p->num_heads * cfh::DH), dim3(256), 0, st,
+                               F.K, 1, prep_blocks, WA);
             if (F.sorted_tab) {
                 // four heads of an atom per wavefront for the items with the usual box and short rows, the others one
                 // by one, all in one launch
@@ -1372,12 +1377,10 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
             C.K.counters = F.K.counters2;
         } else {
             C.K.frames = has_ang ? frames : nullptr;
-            hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, C.K, 0);
+            hipLaunchKernelGGL(cfh::core_prepare_wcat_kernel, dim3(prep_blocks + p->num_heads * cfh::DH), dim3(256), 0, st,
+                               C.K, 0, prep_blocks, WA);
         }
     }
-    float* wcat = buf.wcat;
-    hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, W_dist, W_axis1, W_axis2,
-                       W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat);
     C.out = out; C.prob = prob; C.z = z; C.hist = hist;
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "fused_core_forward";
@@ -1474,8 +1477,9 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
 
     // ---- this stream: Wcat, G = Wcat^T go per item, records, tables, the main kernel, gk and gv
     if (!buf.wcat_ready)
-        hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st, W_dist, W_axis1,
-                           W_axis2, W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat);
+        hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st,
+                           cfh::WcatArgs{W_dist, W_axis1, W_axis2, W_axis3, L.hw, p->dist_coef, p->angle_coef,
+                                         p->angle_wscale, wcat});
     // (with records kept from the forward the work queues are all that is left to prepare: gbuild clears them)
     hipLaunchKernelGGL(cfh::core_gbuild_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads, L.hw / 64), dim3(cfh::WAVE), 0,
                        st, gout, wcat, G, (int)N, p->num_heads, L.hw, buf.records_ready ? C.K.counters : nullptr);

@@ -454,8 +454,8 @@ __device__ __forceinline__ uint32_t load_record(const KernelArgs& P, int it, int
 
 // One thread per (item, head): builds the records, clears the work queues of the launch and (backward)
 // the weight-gradient outputs that the reduction after the main kernel adds into.
-__global__ __launch_bounds__(256) void prepare_items_kernel(const KernelArgs P, int with_query) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void prepare_items_block(const KernelArgs& P, int with_query, int block) {
+    const int idx = block * 256 + (int)threadIdx.x;
     if (idx < P.H * NQUEUE) {
         P.counters[idx * QSTRIDE] = 0;
         if (P.counters2) P.counters2[idx * QSTRIDE] = 0;
@@ -496,6 +496,9 @@ __global__ __launch_bounds__(256) void prepare_items_kernel(const KernelArgs P, 
             for (int d = 0; d < 3; d++)
                 rec[REC_FRAMES + ax * 3 + d] = __float_as_uint(P.frames[(((size_t)ax * P.N + i) * P.H + h) * 3 + d]);
     }
+}
+__global__ __launch_bounds__(256) void prepare_items_kernel(const KernelArgs P, int with_query) {
+    prepare_items_block(P, with_query, (int)blockIdx.x);
 }
 
 // Counter-based uniform in [0,1) for the optional tie-breaking noise of the frame search.

@@ -191,13 +191,20 @@ __device__ __forceinline__ void build_moment_table(float* dtab, float ws) {
 }
 // wcat (H,16,hw): [0,64) dist_coef W_dist;  64 + (ax NORD + o) 64 + m': angle_coef sum_m W_ax[c,m] D_o(m - m').
 // grid: H*16 blocks (h, c), 256 threads over the words.
-__global__ __launch_bounds__(256) void core_wcat_kernel(const float* __restrict__ Wd, const float* __restrict__ W1,
-                                                        const float* __restrict__ W2, const float* __restrict__ W3,
-                                                        int hw, float dist_coef, float angle_coef, float ws,
-                                                        float* __restrict__ wcat) {
+struct WcatArgs {
+    const float* Wd; const float* W1; const float* W2; const float* W3;
+    int hw;
+    float dist_coef, angle_coef, ws;
+    float* wcat;
+};
+__device__ __forceinline__ void core_wcat_block(const WcatArgs& A, int hc) {
+    const float* __restrict__ Wd = A.Wd; const float* __restrict__ W1 = A.W1;
+    const float* __restrict__ W2 = A.W2; const float* __restrict__ W3 = A.W3;
+    const int hw = A.hw;
+    const float dist_coef = A.dist_coef, angle_coef = A.angle_coef, ws = A.ws;
+    float* __restrict__ wcat = A.wcat;
     __shared__ float row[3][NBINS];
     __shared__ float dtab[NORD * 128];
-    const int hc = blockIdx.x;
     if (hw > HW_DIST) {
         for (int u = threadIdx.x; u < 3 * NBINS; u += 256) {
             const float* W = u < NBINS ? W1 : (u < 2 * NBINS ? W2 : W3);
@@ -218,6 +225,15 @@ __global__ __launch_bounds__(256) void core_wcat_kernel(const float* __restrict_
         }
         wcat[(size_t)hc * hw + w] = val;
     }
+}
+__global__ __launch_bounds__(256) void core_wcat_kernel(const WcatArgs A) { core_wcat_block(A, (int)blockIdx.x); }
+// The item records of a launch and the concatenated weights in ONE launch (neither depends on the other; both are a
+// few microseconds of work behind a launch): the first prep_blocks workgroups are those of prepare_items_kernel, the
+// following H * 16 those of core_wcat_kernel.
+__global__ __launch_bounds__(256) void core_prepare_wcat_kernel(const KernelArgs P, int with_query, int prep_blocks,
+                                                                const WcatArgs A) {
+    if ((int)blockIdx.x < prep_blocks) prepare_items_block(P, with_query, (int)blockIdx.x);
+    else core_wcat_block(A, (int)blockIdx.x - prep_blocks);
 }
 // The way back: gW_dist = dist_coef gwcat[.., 0:64];  gW_ax[c,m] = angle_coef sum_{o,m'} gwcat[.., ax,o,m'] D_o(m - m').
 // grid: H*16 blocks, 256 threads = (enc 0..3, bin m).
