@@ -14,12 +14,13 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
 FLAG_SINGLE_STREAM = 1      # cfh_params.flags: CFH_FLAG_SINGLE_STREAM
 FLAG_DEFER_JOIN = 2         # cfh_params.flags: CFH_FLAG_DEFER_JOIN
+FLAG_NO_WEIGHT_GRADS = 4    # cfh_params.flags: CFH_FLAG_NO_WEIGHT_GRADS
 
 
 class CfhParams(ctypes.Structure):
@@ -74,6 +75,13 @@ class CfhLinearGradJob(ctypes.Structure):
                 ("ldy", ctypes.c_int64)]
 
 
+class CfhCoreWgradJob(ctypes.Structure):
+    """Mirror of ``cfh_core_wgrad_job`` in include/crystalframer_hip.h."""
+    _fields_ = [("gout", ctypes.c_void_p), ("hist", ctypes.c_void_p), ("N", ctypes.c_int64),
+                ("gW_dist", ctypes.c_void_p), ("gW_axis1", ctypes.c_void_p), ("gW_axis2", ctypes.c_void_p),
+                ("gW_axis3", ctypes.c_void_p)]
+
+
 class CfhAdamWJob(ctypes.Structure):
     """Mirror of ``cfh_adamw_job`` in include/crystalframer_hip.h."""
     _fields_ = [("param", ctypes.c_void_p), ("grad", ctypes.c_void_p), ("exp_avg", ctypes.c_void_p),
@@ -89,7 +97,8 @@ EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_fram
            "cfh_attention_inputs_backward", "cfh_layer_bridge_forward", "cfh_layer_bridge_backward",
            "cfh_second_stream_fork", "cfh_second_stream_get", "cfh_second_stream_join",
            "cfh_fused_core_workspace_bytes", "cfh_fused_core_hist_words", "cfh_fused_core_forward",
-           "cfh_fused_core_backward", "cfh_adamw_step_batch")
+           "cfh_fused_core_backward", "cfh_adamw_step_batch",
+           "cfh_fused_core_weight_gradients_workspace_bytes", "cfh_fused_core_weight_gradients")
 
 _lib = None
 _lock = threading.Lock()
@@ -153,6 +162,10 @@ def load():
         lib.cfh_linear_weight_bias_grad.argtypes = [_P, _P, _I64, _I64, _I64, _P, _P, _P]
         lib.cfh_small_linear_forward.restype = ctypes.c_int
         lib.cfh_small_linear_forward.argtypes = [_P, _P, _P, _I64, _I64, _I64, ctypes.c_int32, _P, _P]
+        lib.cfh_fused_core_weight_gradients_workspace_bytes.restype = ctypes.c_size_t
+        lib.cfh_fused_core_weight_gradients_workspace_bytes.argtypes = [_P, ctypes.c_int32]
+        lib.cfh_fused_core_weight_gradients.restype = ctypes.c_int
+        lib.cfh_fused_core_weight_gradients.argtypes = [_P, _P, ctypes.c_int32, _P, ctypes.c_size_t, _P]
         lib.cfh_adamw_step_batch.restype = ctypes.c_int
         lib.cfh_adamw_step_batch.argtypes = [_P, ctypes.c_int32, ctypes.c_float, ctypes.c_float, ctypes.c_float,
                                              ctypes.c_float, ctypes.c_float, _P, _P]

@@ -1209,7 +1209,7 @@ CoreLayout core_layout(const cfh_params* p, int64_t N, int64_t E, int64_t B, boo
     L.sorted = off; off += align256((size_t)(B > 0 ? B : 1) * cfh::FC_TCAP * sizeof(float4));
     L.near = off; if (!backward) off += align256((size_t)(E > 0 ? E : 1) * sizeof(float2));
     L.wcat = off; off += align256((size_t)p->num_heads * cfh::DH * L.hw * sizeof(float));
-    L.gwcat = off; if (backward) off += align256((size_t)p->num_heads * cfh::DH * L.hw * sizeof(float));
+    L.gwcat = off; if (backward) off += align256((size_t)cfh::CORE_GW_SLICES * p->num_heads * cfh::DH * L.hw * sizeof(float));
     L.G = off; if (backward) off += align256((size_t)(N > 0 ? N : 1) * p->num_heads * L.hw * sizeof(float));
     L.total = off;
     return L;
@@ -1443,7 +1443,8 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
 
     // ---- weight gradients: gwcat = sum_i go_i (x) hist_i, then back through the moment matrices.  They read
     //      nothing that this call makes, so they go to the second stream, beside the kernels below.
-    const bool two = !(p->flags & CFH_FLAG_SINGLE_STREAM);
+    const bool no_wg = (p->flags & CFH_FLAG_NO_WEIGHT_GRADS) != 0;      // the caller makes them later, for several calls at once
+    const bool two = !(p->flags & CFH_FLAG_SINGLE_STREAM) && !no_wg;
     std::unique_lock<std::mutex> side_lock(g_side_mutex, std::defer_lock);
     SideStream* side = nullptr;
     hipStream_t st_w = st;
@@ -1456,20 +1457,20 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         st_w = side->stream;
     }
     auto weight_gradients = [&]() {
-        const int nw = p->num_heads * cfh::DH * L.hw;
-        hipLaunchKernelGGL(cfh::core_zero_kernel, dim3((nw + 255) / 256), dim3(256), 0, st_w, gwcat, nw);
         int cus = device_cus();
         if (cus <= 0) cus = 256;
         const int blocks_per_slice = (L.hw / 64) * p->num_heads;
         int nslices = (cus * 4 + blocks_per_slice - 1) / blocks_per_slice;      // about one wavefront per SIMD
         if (nslices < 1) nslices = 1;
+        if (nslices > cfh::CORE_GW_SLICES) nslices = cfh::CORE_GW_SLICES;
         int per_slice = (int)((N + nslices - 1) / nslices);
         per_slice = (per_slice + 15) & ~15;
         nslices = (int)((N + per_slice - 1) / per_slice);
         hipLaunchKernelGGL(cfh::core_gwcat_kernel, dim3(L.hw / 64, p->num_heads, nslices), dim3(cfh::WAVE), 0, st_w, gout,
                            hist, gwcat, (int)N, p->num_heads, L.hw, per_slice);
-        hipLaunchKernelGGL(cfh::core_gw_finish_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st_w, gwcat, L.hw,
-                           p->dist_coef, p->angle_coef, p->angle_wscale, gW_dist, gW_axis1, gW_axis2, gW_axis3);
+        hipLaunchKernelGGL(cfh::core_gw_finish_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st_w, gwcat, nslices,
+                           p->num_heads, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, gW_dist, gW_axis1, gW_axis2,
+                           gW_axis3);
         return finish_launch("fused_core_weight_gradients");
     };
     int rc_w = CFH_OK;
@@ -1507,13 +1508,73 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
                            dim3(cfh::WAVE * cfh::DPA_WAVES), 0, st, A);
         rc = finish_launch("fused_core_backward");
     }
-    if (!two) rc_w = weight_gradients();
+    if (!two && !no_wg) rc_w = weight_gradients();
     // the join is enqueued whatever happened in between: a stream that was pulled into a capture must come back
     if (two && !(p->flags & CFH_FLAG_DEFER_JOIN) &&
         (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(st, side->join, 0) != hipSuccess) &&
         !rc && !rc_w)
         rc_w = fail(CFH_ELAUNCH, "join of the second stream failed");
     return rc ? rc : rc_w;
+}
+
+
+size_t cfh_fused_core_weight_gradients_workspace_bytes(const cfh_params* p, int32_t njobs) {
+    if (check_core_params(p) != CFH_OK || njobs < 0) return 0;
+    const size_t hw = p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
+    return align256((size_t)cfh::CORE_GW_SLICES * p->num_heads * cfh::DH * hw * sizeof(float)) * (size_t)(njobs > 0 ? njobs : 1);
+}
+
+int cfh_fused_core_weight_gradients(const cfh_params* p, const cfh_core_wgrad_job* jobs, int32_t njobs,
+                                    void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_core_params(p);
+    if (rc) return rc;
+    if (njobs < 0 || (njobs > 0 && !jobs)) return fail(CFH_EINVAL, "jobs is NULL or njobs negative");
+    if (njobs == 0) return CFH_OK;
+    const int hw = p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
+    const size_t per_job = align256((size_t)cfh::CORE_GW_SLICES * p->num_heads * cfh::DH * hw * sizeof(float));
+    if ((rc = check_workspace(workspace, workspace_bytes, per_job * (size_t)njobs))) return rc;
+    for (int32_t j = 0; j < njobs; j++) {
+        if (jobs[j].N < 0 || jobs[j].N > 0x7fffffffLL / 64)
+            return fail(CFH_EINVAL, "weight-gradient job %d: N = %lld out of range", (int)j, (long long)jobs[j].N);
+        if (jobs[j].N > 0 && (!jobs[j].gout || !jobs[j].hist))
+            return fail(CFH_EINVAL, "weight-gradient job %d: gout and hist must not be NULL", (int)j);
+    }
+    hipStream_t st = (hipStream_t)stream;
+    char* ws = reinterpret_cast<char*>(workspace);
+    int cus = device_cus();
+    if (cus <= 0) cus = 256;
+    const int blocks_per_slice = (hw / 64) * p->num_heads;
+    for (int32_t first = 0; first < njobs; first += cfh::CORE_WG_MAX_JOBS) {
+        const int32_t last = njobs < first + cfh::CORE_WG_MAX_JOBS ? njobs : first + cfh::CORE_WG_MAX_JOBS;
+        cfh::CoreWgradJobs T{};
+        T.H = p->num_heads; T.hw = hw;
+        T.dist_coef = p->dist_coef; T.angle_coef = p->angle_coef; T.ws = p->angle_wscale;
+        int slices = 0;
+        for (int32_t j = first; j < last; j++) {
+            cfh::CoreWgradJob& J = T.job[T.njobs++];
+            J.go = jobs[j].gout; J.hist = jobs[j].hist;
+            J.gwcat = reinterpret_cast<float*>(ws + per_job * (size_t)j);
+            J.gW[0] = jobs[j].gW_dist; J.gW[1] = jobs[j].gW_axis1; J.gW[2] = jobs[j].gW_axis2; J.gW[3] = jobs[j].gW_axis3;
+            J.N = (int)jobs[j].N;
+            // about two wavefronts per SIMD over all jobs of the launch
+            int nslices = (cus * 8 / (last - first) + blocks_per_slice - 1) / blocks_per_slice;
+            if (nslices < 1) nslices = 1;
+            if (nslices > cfh::CORE_GW_SLICES) nslices = cfh::CORE_GW_SLICES;
+            int per_slice = (int)((jobs[j].N + nslices - 1) / nslices);
+            per_slice = (per_slice + 15) & ~15;
+            if (per_slice < 16) per_slice = 16;
+            nslices = (int)((jobs[j].N + per_slice - 1) / per_slice);
+            if (nslices < 1) nslices = 1;      // (no atoms: one slice of zeros)
+            J.per_slice = per_slice;
+            J.slice0 = slices;
+            J.nslices = nslices;
+            slices += nslices;
+        }
+        if (slices > 0)
+            hipLaunchKernelGGL(cfh::core_gwcat_multi_kernel, dim3(hw / 64, p->num_heads, slices), dim3(cfh::WAVE), 0, st, T);
+        hipLaunchKernelGGL(cfh::core_gw_finish_multi_kernel, dim3(p->num_heads * cfh::DH, T.njobs), dim3(256), 0, st, T);
+    }
+    return finish_launch("fused_core_weight_gradients");
 }
 
 }  // extern "C"

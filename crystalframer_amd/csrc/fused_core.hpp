@@ -236,21 +236,31 @@ __global__ __launch_bounds__(256) void core_prepare_wcat_kernel(const KernelArgs
     else core_wcat_block(A, (int)blockIdx.x - prep_blocks);
 }
 // The way back: gW_dist = dist_coef gwcat[.., 0:64];  gW_ax[c,m] = angle_coef sum_{o,m'} gwcat[.., ax,o,m'] D_o(m - m').
-// grid: H*16 blocks, 256 threads = (enc 0..3, bin m).
-__global__ __launch_bounds__(256) void core_gw_finish_kernel(const float* __restrict__ gwcat, int hw, float dist_coef,
-                                                             float angle_coef, float ws, float* __restrict__ gWd,
-                                                             float* __restrict__ gW1, float* __restrict__ gW2,
-                                                             float* __restrict__ gW3) {
+// Block hc = (head, channel), 256 threads = (enc 0..3, bin m).  ACC: added to what the destinations hold.
+template <bool ACC>
+__device__ __forceinline__ void core_gw_finish_block(const float* __restrict__ gwcat, int nslices, size_t slice_stride,
+                                                     int hw, float dist_coef, float angle_coef, float ws,
+                                                     float* __restrict__ gWd, float* __restrict__ gW1,
+                                                     float* __restrict__ gW2, float* __restrict__ gW3, int hc) {
     __shared__ float dtab[NORD * 128];
     __shared__ float grow[3 * NORD * NBINS];
-    const int hc = blockIdx.x, enc = threadIdx.x >> 6, m = threadIdx.x & 63;
+    const int enc = threadIdx.x >> 6, m = threadIdx.x & 63;
     const float* g = gwcat + (size_t)hc * hw;
     if (hw > HW_DIST) {
-        for (int u = threadIdx.x; u < 3 * NORD * NBINS; u += 256) grow[u] = g[HW_DIST + u];
+        for (int u = threadIdx.x; u < 3 * NORD * NBINS; u += 256) {
+            float sum = 0.0f;
+            for (int sl = 0; sl < nslices; sl++) sum += g[sl * slice_stride + HW_DIST + u];      // fixed order
+            grow[u] = sum;
+        }
         build_moment_table(dtab, ws);
     }
     if (enc == 0) {
-        if (gWd) gWd[(size_t)hc * NBINS + m] = dist_coef * g[m];
+        if (gWd) {
+            float sum = 0.0f;
+            for (int sl = 0; sl < nslices; sl++) sum += g[sl * slice_stride + m];
+            float* d = gWd + (size_t)hc * NBINS + m;
+            *d = (ACC ? *d : 0.0f) + dist_coef * sum;
+        }
         return;
     }
     if (hw <= HW_DIST) return;
@@ -263,9 +273,33 @@ __global__ __launch_bounds__(256) void core_gw_finish_kernel(const float* __rest
 #pragma unroll 8
         for (int mp = 0; mp < NBINS; mp++) acc = fmaf(gr[mp], dt[-mp], acc);
     }
-    dst[(size_t)hc * NBINS + m] = angle_coef * acc;
+    float* d = dst + (size_t)hc * NBINS + m;
+    *d = (ACC ? *d : 0.0f) + angle_coef * acc;
+}
+// grid: H*16 blocks.
+__global__ __launch_bounds__(256) void core_gw_finish_kernel(const float* __restrict__ gwcat, int nslices, int H, int hw,
+                                                             float dist_coef, float angle_coef, float ws,
+                                                             float* __restrict__ gWd, float* __restrict__ gW1,
+                                                             float* __restrict__ gW2, float* __restrict__ gW3) {
+    core_gw_finish_block<false>(gwcat, nslices, (size_t)H * DH * hw, hw, dist_coef, angle_coef, ws, gWd, gW1, gW2, gW3,
+                                (int)blockIdx.x);
 }
 
+// Weight gradients of several calls of the core (the layers of a backward pass) in one launch each way.
+constexpr int CORE_WG_MAX_JOBS = 8;
+constexpr int CORE_GW_SLICES = 8;      // at most this many slices of the atoms per job (copies of the scratch)
+struct CoreWgradJob {
+    const float* go;       // (N,H,16)
+    const float* hist;     // (H,N,hw)
+    float* gwcat;          // (nslices,H,16,hw) scratch
+    float* gW[4];          // destinations (H,16,64), added to; null: not wanted
+    int N, per_slice, slice0, nslices;      // atoms, atoms per slice, first slice (blockIdx.z) of this job, its slices
+};
+struct CoreWgradJobs {
+    CoreWgradJob job[CORE_WG_MAX_JOBS];
+    int njobs, H, hw;
+    float dist_coef, angle_coef, ws;
+};
 // ---- distance window with round-to-nearest fixed-point adds ---------------------------------------------------
 template <int W>
 __device__ __forceinline__ void window_scatter_rn(int32_t* base, const WindowSeed& s, float cc) {
@@ -766,49 +800,71 @@ __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restri
     }
 }
 
-// gwcat (H,16,hw) += sum over a slice of the atoms of go (.,h,16) (x) hist (h,.,hw): wavefront per (head, 64-word
-// block, slice); four MFMA tiles with interleaved columns as above; float atomics into the cleared result.
-// grid (hw/64, H, nslices).
-__global__ __launch_bounds__(WAVE) void core_gwcat_kernel(const float* __restrict__ go, const float* __restrict__ hist,
-                                                          float* __restrict__ gwcat, int N, int H, int hw, int per_slice) {
+// gwcat (slice,H,16,hw) = sum over a slice of the atoms of go (.,h,16) (x) hist (h,.,hw): wavefront per (head, 64-word
+// block, slice); four MFMA tiles with interleaved columns as above.  grid (hw/64, H, nslices), at most
+// CORE_GW_SLICES slices.
+__device__ __forceinline__ void core_gwcat_block(const float* __restrict__ go, const float* __restrict__ hist,
+                                                 float* __restrict__ gwcat, int N, int H, int hw, int per_slice, int slice) {
     const int lane = threadIdx.x, col = lane & 15, kk = lane >> 4;
     const int w0 = blockIdx.x * 64, h = blockIdx.y;
-    const int i_begin = blockIdx.z * per_slice, i_end = min(N, i_begin + per_slice);
+    const int i_begin = slice * per_slice, i_end = min(N, i_begin + per_slice);
     v4f_c acc[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) acc[t] = v4f_c{0.f, 0.f, 0.f, 0.f};
-    for (int ib = i_begin; ib < i_end; ib += 16) {
-        float av[4];
-        float4 bv[4];
+    // GW_DEPTH x 16 atoms per step, all their loads asked for before the first product: a wavefront keeps 16 KB of
+    // histogram rows in flight (with 4 KB the kernel ran at 40 % of the bandwidth it reaches now)
+    constexpr int GW_DEPTH = 4;
+    for (int ib = i_begin; ib < i_end; ib += 16 * GW_DEPTH) {
+        float av[GW_DEPTH][4];
+        float4 bv[GW_DEPTH][4];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int it = ib + 4 * j + kk;
-            const bool live = it < i_end;
-            const size_t base = ((size_t)(live ? it : i_begin) * H + h);
-            av[j] = live ? go[base * DH + col] : 0.0f;
-            bv[j] = live ? *reinterpret_cast<const float4*>(hist + ((size_t)h * N + it) * hw + w0 + 4 * col)
-                         : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
+        for (int d = 0; d < GW_DEPTH; d++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j].x, acc[0], 0, 0, 0);
-            acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j].y, acc[1], 0, 0, 0);
-            acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j].z, acc[2], 0, 0, 0);
-            acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j].w, acc[3], 0, 0, 0);
-        }
+            for (int j = 0; j < 4; j++) {
+                const int it = ib + 16 * d + 4 * j + kk;
+                const bool live = it < i_end;
+                const size_t base = ((size_t)(live ? it : i_begin) * H + h);
+                av[d][j] = live ? go[base * DH + col] : 0.0f;
+                bv[d][j] = live ? *reinterpret_cast<const float4*>(hist + ((size_t)h * N + it) * hw + w0 + 4 * col)
+                                : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+        for (int d = 0; d < GW_DEPTH; d++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[d][j], bv[d][j].x, acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[d][j], bv[d][j].y, acc[1], 0, 0, 0);
+                acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[d][j], bv[d][j].z, acc[2], 0, 0, 0);
+                acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[d][j], bv[d][j].w, acc[3], 0, 0, 0);
+            }
     }
-    // component r of tile t, lane (kk, col): channel 4 kk + r, word w0 + 4 col + t
+    // component r of tile t, lane (kk, col): channel 4 kk + r, word w0 + 4 col + t.  Every slice writes its own
+    // copy (slice, H, 16, hw) in full: nothing to clear, no atomics, and the sum over the slices that follows is made
+    // in a fixed order
+    float* const part = gwcat + (size_t)slice * H * DH * hw;
 #pragma unroll
     for (int r = 0; r < 4; r++)
-#pragma unroll
-        for (int t = 0; t < 4; t++)
-            atomicAdd(gwcat + ((size_t)h * DH + 4 * kk + r) * hw + w0 + 4 * col + t, acc[t][r]);
+        *reinterpret_cast<float4*>(part + ((size_t)h * DH + 4 * kk + r) * hw + w0 + 4 * col) =
+            make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+}
+__global__ __launch_bounds__(WAVE) void core_gwcat_kernel(const float* __restrict__ go, const float* __restrict__ hist,
+                                                          float* __restrict__ gwcat, int N, int H, int hw, int per_slice) {
+    core_gwcat_block(go, hist, gwcat, N, H, hw, per_slice, (int)blockIdx.z);
+}
+// several jobs: grid (hw/64, H, slices of all jobs); the job of a slice by a scan of the (few) jobs
+__global__ __launch_bounds__(WAVE) void core_gwcat_multi_kernel(const CoreWgradJobs T) {
+    int j = 0;
+    while (j + 1 < T.njobs && (int)blockIdx.z >= T.job[j + 1].slice0) j++;
+    const CoreWgradJob& J = T.job[j];
+    core_gwcat_block(J.go, J.hist, J.gwcat, J.N, T.H, T.hw, J.per_slice, (int)blockIdx.z - J.slice0);
+}
+// grid (H*16, jobs): added to the destinations
+__global__ __launch_bounds__(256) void core_gw_finish_multi_kernel(const CoreWgradJobs T) {
+    const CoreWgradJob& J = T.job[blockIdx.y];
+    core_gw_finish_block<true>(J.gwcat, J.nslices, (size_t)T.H * DH * T.hw, T.hw, T.dist_coef, T.angle_coef, T.ws,
+                               J.gW[0], J.gW[1], J.gW[2], J.gW[3], (int)blockIdx.x);
 }
 
-__global__ void core_zero_kernel(float* p, int n) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx < n) p[idx] = 0.0f;
-}
 
 // =================================================================================================================
 // backward

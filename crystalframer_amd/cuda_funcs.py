@@ -47,6 +47,10 @@ class KernelManager:
     # weight / bias gradients of the linear layers (leaf parameters): all layers of a backward pass in
     # one launch when the pass ends, instead of one launch per layer as the gradient is reached
     DEFER_WEIGHT_GRADS: bool = True
+    # fused attention core: the weight gradients of the value encoding of all layers of a backward pass together when
+    # the pass ends, instead of on the second stream beside every layer's main kernel, which they slow down by as
+    # much as they gain there (False: inside every backward call)
+    DEFER_CORE_WEIGHT_GRADS: bool = True
     COLLECT_STATS: bool = False         # count translations (read with _lib.read_stats)
     EVENT_LOG = None                    # a list: every library call appends (name, start, end) events
     _compiled_for = None
@@ -726,6 +730,7 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
                               z, prob, hist, out, table, wcat, records)
         ctx.params = p
         ctx.w_shapes = [None if w is None else w.shape for w in (W_k, W_k1, W_k2, W_k3)]
+        ctx.weights = (W_k, W_k1 if use_angle else None, W_k2 if use_angle else None, W_k3 if use_angle else None)
         ctx.in_dtype = qs.dtype
         if fr is not None:
             ctx.mark_non_differentiable(fr)
@@ -745,20 +750,39 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
         gq, gk, gv = torch.empty_like(q_), torch.empty_like(k_), torch.empty_like(v_)
         ga = torch.empty((N, H), dtype=torch.float32, device=dev)
         glogit = torch.empty((E, H), dtype=torch.float32, device=dev)
-        gWd = torch.empty_like(Wd)
-        gWa = [torch.empty_like(w) if w is not None else None for w in (W1, W2, W3)]
+        D = _DeferredWeightGrads
+        if D.callback_queued and D.task_id != torch._C._current_graph_task_id():
+            D.reset()                               # left over from a backward pass that raised
+        # the weight gradients: with leaf parameters, zero-filled views of the pass's gradient arena that ONE library
+        # call completes for all layers when the pass ends (see _DeferredWeightGrads); else made by this call
+        defer_core = (KernelManager.DEFER_CORE_WEIGHT_GRADS and N > 0 and D.deferrable(*ctx.weights)
+                      and all(w is None or (w.dtype == torch.float32 and w.numel() == Wd.numel()) for w in ctx.weights))
+        if defer_core:
+            views, refs = [], []
+            for w in ctx.weights:
+                if w is None:
+                    views.append(None); refs.append(None)
+                    continue
+                views.append(D.take(w.numel(), dev))
+                refs.append((D.arena, D.arena_off - ((w.numel() + 63) & ~63), w.numel()))
+            gWd, gWa = views[0], views[1:]
+            del views
+        else:
+            gWd = torch.empty_like(Wd)
+            gWa = [torch.empty_like(w) if w is not None else None for w in (W1, W2, W3)]
         cache = _lib.CfhCoreCache(table.data_ptr(), None, wcat.data_ptr(), records.data_ptr(), 1, 1, 1, 0)
         # The library makes the weight gradients of the value encoding on its second stream, beside its main
         # kernel.  The weight gradients of the linear layers collected so far (those of the layers behind this one)
         # go to that stream as well instead of waiting for the end of the pass; the join is then made here.
-        D = _DeferredWeightGrads
-        second = (N > 0 and not (p.flags & _lib.FLAG_SINGLE_STREAM) and bool(D.pending)
+        second = (N > 0 and not defer_core and not (p.flags & _lib.FLAG_SINGLE_STREAM) and bool(D.pending)
                   and D.task_id == torch._C._current_graph_task_id())
         flags = p.flags
         held = None
         rcj = 0
         with torch.cuda.device(dev):
             try:
+                if defer_core:
+                    p.flags = flags | _lib.FLAG_NO_WEIGHT_GRADS
                 if second:
                     p.flags = flags | _lib.FLAG_DEFER_JOIN
                 with _timed("fused_core_backward", dev):
@@ -768,8 +792,10 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
                         _lib.ptr(tv), _lib.ptr(rv), _lib.ptr(batch), _lib.ptr(edges), _lib.ptr(e_start), _lib.ptr(order),
                         _lib.ptr(Wd), _lib.ptr(W1), _lib.ptr(W2), _lib.ptr(W3), _lib.ptr(fr), _lib.ptr(z), _lib.ptr(prob),
                         _lib.ptr(hist), _lib.ptr(out), _lib.ptr(go), N, E, tv.shape[0], _lib.ptr(gq), _lib.ptr(gk),
-                        _lib.ptr(gv), _lib.ptr(ga), _lib.ptr(glogit), _lib.ptr(gWd), _lib.ptr(gWa[0]), _lib.ptr(gWa[1]),
-                        _lib.ptr(gWa[2]), ctypes.byref(cache), _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
+                        _lib.ptr(gv), _lib.ptr(ga), _lib.ptr(glogit), *([None] * 4 if defer_core else
+                                                                       [_lib.ptr(gWd), _lib.ptr(gWa[0]), _lib.ptr(gWa[1]),
+                                                                        _lib.ptr(gWa[2])]),
+                        ctypes.byref(cache), _lib.ptr(ws), ws.numel(), _lib.current_stream_ptr(dev))
                 if second and rc == 0:
                     held = D.flush(second_stream=True)
             finally:
@@ -780,7 +806,17 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
         if second:
             _lib.check(rcj, "cfh_second_stream_join")
         del held            # what the second stream read is ordered before everything that follows on this one
+        if defer_core:
+            params_copy = _lib.CfhParams.from_buffer_copy(p)
+            params_copy.flags = flags
+            D.core_pending.append((params_copy, go, hist, N, refs, ctx.weights, [D.mark(w) if w is not None else None
+                                                                                for w in ctx.weights]))
+            if not D.callback_queued:
+                torch.autograd.Variable._execution_engine.queue_callback(D.flush)
+                D.callback_queued = True
+                D.task_id = torch._C._current_graph_task_id()
         gws = [g if g is None else g.reshape(s) for g, s in zip([gWd] + gWa, ctx.w_shapes)]
+        del gWd, gWa
         dt = ctx.in_dtype
         return (gq.to(dt), gk.to(dt), gv.to(dt), ga, None, None, None, None, None, None, None, gws[0], gws[1], gws[2],
                 gws[3], None, None, None, None, None, None, None, None)
@@ -850,6 +886,7 @@ class _DeferredWeightGrads:
     (``KernelManager.DEFER_WEIGHT_GRADS = False`` does not change that; the kernel is the same)."""
     ARENA_FLOATS = 1 << 21
     pending = []            # (x2, gy2, col0, O, dW ref, bias-gradient ref, weight, bias, marks)
+    core_pending = []       # fused attention core: (params, gout, hist, N, gradient refs, weights, marks) per call
     arena = None
     arena_off = 0
     arenas = []             # keeps the gradient memory of the pass alive; the views themselves are NOT kept:
@@ -903,6 +940,7 @@ class _DeferredWeightGrads:
     @classmethod
     def reset(cls):
         cls.pending = []
+        cls.core_pending = []
         cls.arena = None
         cls.arena_off = 0
         cls.arenas = []
@@ -914,21 +952,25 @@ class _DeferredWeightGrads:
         what a cfh_framed_pe_backward call that has just been made (with its join deferred) put there, beside
         that call's kernel on the current stream; the caller joins and keeps the list returned here -- the
         tensors the launch reads -- until then; the arena and the callback of the end of the pass stay as
-        they are for the layers still to come."""
+        they are for the layers still to come.  At the end of the pass (``second_stream`` False) the weight
+        gradients of the fused attention cores are made as well: one library call for all layers, behind the
+        linear layers' launch."""
         pending, cls.pending = cls.pending, []
+        core = []
         if not second_stream:
+            core, cls.core_pending = cls.core_pending, []
             arenas, cls.arenas = cls.arenas, []
             cls.arena = None
             cls.arena_off = 0
             cls.callback_queued = False
-        if not pending:
+        if not pending and not core:
             return None
 
         def view(ref):           # (arena, offset, count) -> tensor
             return ref[0][ref[1]:ref[1] + ref[2]]
         lib = _lib.load()
-        dev = pending[0][1].device
-        jobs = (_lib.CfhLinearGradJob * len(pending))()
+        dev = pending[0][1].device if pending else core[0][1].device
+        jobs = (_lib.CfhLinearGradJob * max(len(pending), 1))()
         fixups = []
         for n, (x2, g2, col0, O, dW, db, weight, bias, w_mark, b_mark) in enumerate(pending):
             # dW, db: (arena, offset, count) of the zero-filled tensors handed to autograd (db: of the whole bias)
@@ -969,9 +1011,43 @@ class _DeferredWeightGrads:
                 rc = lib.cfh_linear_weight_bias_grad_batch(jobs, len(pending), side)
             _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
             return pending
-        with torch.cuda.device(dev), _timed("linear_weight_bias_grad_batch", dev):
-            rc = lib.cfh_linear_weight_bias_grad_batch(jobs, len(pending), _lib.current_stream_ptr(dev))
+        # ---- the end of the pass
+        groups = {}                      # calls of the core with the same constants share a library call
+        for params, go, hist, N, refs, weights, marks in core:
+            dst = []
+            for ref, w, mark in zip(refs, weights, marks):
+                if w is None:
+                    dst.append(None)
+                    continue
+                d = ref[0].data_ptr() + 4 * ref[1]
+                wg = w.grad
+                if wg is not None and cls.changed(w, mark) and wg.data_ptr() != d:
+                    if wg.dtype == torch.float32 and wg.is_contiguous() and wg.device == dev:
+                        d = wg.data_ptr()
+                    else:
+                        fixups.append((wg, view(ref).view(wg.shape)))
+                dst.append(d)
+            groups.setdefault(bytes(params), (params, []))[1].append((go, hist, N, dst))
+        # (one after the other on this stream: side by side on two streams the two launches took as long together
+        # and the fork and join came on top)
+        rc = rcc = 0
+        with torch.cuda.device(dev):
+            stream = _lib.current_stream_ptr(dev)
+            if pending:
+                with _timed("linear_weight_bias_grad_batch", dev):
+                    rc = lib.cfh_linear_weight_bias_grad_batch(jobs, len(pending), stream)
+            for params, calls in groups.values():
+                arr = (_lib.CfhCoreWgradJob * len(calls))()
+                for J, (go, hist, N, dst) in zip(arr, calls):
+                    J.gout, J.hist, J.N = go.data_ptr(), hist.data_ptr(), N
+                    J.gW_dist, J.gW_axis1, J.gW_axis2, J.gW_axis3 = dst
+                with _timed("fused_core_weight_gradients", dev):
+                    ws = _lib.workspace(dev, lib.cfh_fused_core_weight_gradients_workspace_bytes(
+                        ctypes.byref(params), len(calls)))
+                    rcc = rcc or lib.cfh_fused_core_weight_gradients(ctypes.byref(params), arr, len(calls),
+                                                                     _lib.ptr(ws), ws.numel(), stream)
         _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
+        _lib.check(rcc, "cfh_fused_core_weight_gradients")
         for grad, part in fixups:
             grad.add_(part.to(grad.dtype))
         return None

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 11
+#define CFH_ABI_VERSION 12
 
 enum {
     CFH_OK = 0,
@@ -98,6 +98,10 @@ typedef struct cfh_params {
  * complete on `stream` before the call) and then MUST call cfh_second_stream_join(stream); until then the
  * weight gradients of the call are not ordered on `stream`. */
 #define CFH_FLAG_DEFER_JOIN 2
+/* cfh_fused_core_backward leaves the four weight gradients out (their pointers may be NULL): the caller collects
+ * (gout, hist) of its calls and makes them together with cfh_fused_core_weight_gradients, e.g. for all layers when a
+ * backward pass ends, away from the main kernels that they would otherwise run beside. */
+#define CFH_FLAG_NO_WEIGHT_GRADS 4
 
 /*
  * The library's second stream of the current device, for a caller that has work of its own to run beside
@@ -370,6 +374,28 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
                             int64_t N, int64_t E, int64_t B, float* gq, float* gk, float* gv, float* ga, float* glogit,
                             float* gW_dist, float* gW_axis1, float* gW_axis2, float* gW_axis3,
                             const cfh_core_cache* cache, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The weight gradients of up to 8 calls of cfh_fused_core_backward made with CFH_FLAG_NO_WEIGHT_GRADS, in one launch
+ * per step (products of gout with the histograms, then the way back through the moment matrices):
+ *     gW_* (H,Dh,64) += sum over the atoms of gout (x) hist   (ADDED to what the destinations hold; NULL: not wanted)
+ * Every job: gout (N,H,Dh) and hist (H,N,words) of one call.  p: the params of those calls (heads, bins, coefficients).
+ * workspace: cfh_fused_core_weight_gradients_workspace_bytes(p, njobs) bytes.  `jobs` is a host array; it is copied
+ * into the kernel arguments.  With float atomics, like the weight gradients inside cfh_fused_core_backward.
+ * No counterpart in the reference (autograd sums its per-atom weight gradients, real_space_framed_proj.py:211-219).
+ */
+typedef struct cfh_core_wgrad_job {
+    const float* gout;
+    const float* hist;
+    int64_t N;
+    float* gW_dist;
+    float* gW_axis1;
+    float* gW_axis2;
+    float* gW_axis3;
+} cfh_core_wgrad_job;
+size_t cfh_fused_core_weight_gradients_workspace_bytes(const cfh_params* p, int32_t njobs);
+int cfh_fused_core_weight_gradients(const cfh_params* p, const cfh_core_wgrad_job* jobs, int32_t njobs,
+                                    void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Sets *flag (device memory) to 0 when edges (2,E) / e_start (N+1) hold, for every crystal, all
