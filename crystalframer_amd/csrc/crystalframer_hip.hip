@@ -1521,7 +1521,9 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
 size_t cfh_fused_core_weight_gradients_workspace_bytes(const cfh_params* p, int32_t njobs) {
     if (check_core_params(p) != CFH_OK || njobs < 0) return 0;
     const size_t hw = p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
-    return align256((size_t)cfh::CORE_GW_SLICES * p->num_heads * cfh::DH * hw * sizeof(float)) * (size_t)(njobs > 0 ? njobs : 1);
+    // (behind the header of every workspace of the library: status word, statistics, work queues)
+    return COUNTER_BYTES +
+           align256((size_t)cfh::CORE_GW_SLICES * p->num_heads * cfh::DH * hw * sizeof(float)) * (size_t)(njobs > 0 ? njobs : 1);
 }
 
 int cfh_fused_core_weight_gradients(const cfh_params* p, const cfh_core_wgrad_job* jobs, int32_t njobs,
@@ -1532,7 +1534,7 @@ int cfh_fused_core_weight_gradients(const cfh_params* p, const cfh_core_wgrad_jo
     if (njobs == 0) return CFH_OK;
     const int hw = p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
     const size_t per_job = align256((size_t)cfh::CORE_GW_SLICES * p->num_heads * cfh::DH * hw * sizeof(float));
-    if ((rc = check_workspace(workspace, workspace_bytes, per_job * (size_t)njobs))) return rc;
+    if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES + per_job * (size_t)njobs))) return rc;
     for (int32_t j = 0; j < njobs; j++) {
         if (jobs[j].N < 0 || jobs[j].N > 0x7fffffffLL / 64)
             return fail(CFH_EINVAL, "weight-gradient job %d: N = %lld out of range", (int)j, (long long)jobs[j].N);
@@ -1540,7 +1542,7 @@ int cfh_fused_core_weight_gradients(const cfh_params* p, const cfh_core_wgrad_jo
             return fail(CFH_EINVAL, "weight-gradient job %d: gout and hist must not be NULL", (int)j);
     }
     hipStream_t st = (hipStream_t)stream;
-    char* ws = reinterpret_cast<char*>(workspace);
+    char* ws = reinterpret_cast<char*>(workspace) + COUNTER_BYTES;
     int cus = device_cus();
     if (cus <= 0) cus = 256;
     const int blocks_per_slice = (hw / 64) * p->num_heads;

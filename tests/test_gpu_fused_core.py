@@ -255,3 +255,31 @@ def test_fused_core_at_batch_256_against_oracle_on_first_crystals():
         assert float(leaves[name].grad[S.N:].abs().max()) == 0.0, name
     for name in ("Wk", "W1", "W2", "W3"):
         assert Hh.rel_err(leaves[name].grad, oleaves[name].grad) < 1e-4, name
+
+
+def test_workspace_header_survives_a_backward_pass():
+    """Status word, statistics and work-queue heads at the head of the shared workspace are not scratch: a forward +
+    backward pass (with the weight gradients made at the end of the pass) leaves the term counters meaningful and the
+    status word clear."""
+    import crystalframer_amd as cf
+    from crystalframer_amd import _lib
+    KM = cf.KernelManager
+    P = Hh.make_problem(num_crystals=12, atoms_hi=6, seed=31)
+    _lib.read_stats(dev(), reset=True)
+    _lib.read_status(dev(), reset=True)
+    saved = KM.COLLECT_STATS
+    KM.COLLECT_STATS = True
+    try:
+        out, _, leaves = run_core(P)
+        (out * g(_gout(P))).sum().backward()
+        torch.cuda.synchronize()
+    finally:
+        KM.COLLECT_STATS = saved
+    st = _lib.read_stats(dev(), reset=True)
+    assert _lib.read_status(dev()) == 0
+    pairs = P.E * Hh.H
+    assert st["fwd_pairs"] == pairs and st["bwd_pairs"] == pairs
+    assert 0 < st["fwd_evaluated"] <= st["fwd_in_box"] <= 343 * 2 * pairs
+    assert 0 < st["bwd_evaluated"] <= st["bwd_in_box"] == st["fwd_in_box"]
+    for name in ("Wk", "W1", "W2", "W3"):
+        assert leaves[name].grad is not None and float(leaves[name].grad.abs().max()) > 0
