@@ -330,14 +330,16 @@ struct FrameQuadShared {
     float4 tab[FC_TCAP];
     float4 rp[FQ_STAGE];                 // staged pairs: rpos, d^2 of the nearest valid image (or -1)
     float qk_s[FQ_ROWS][FQ_STAGE];       // q_h . k_j of the staged pairs, per row
-    int pstart[FQ_ROWS][17];             // per row: first candidate of each of 16 pairs, then the total
+    uint32_t markw[FQ_ROWS][FQ_MAX_PAIRS * FC_TCAP / 32];      // per row: one bit per candidate, set where a pair's run begins
+    uint32_t ent[FQ_ROWS][16];           // per row: the pairs that have candidates, in order: first candidate | pair << 16
 };
 // one wavefront, four heads of one atom: wid = item * groups + group of heads
 __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShared& sh, int wid, int lane) {
     float4* const tab = sh.tab;
     float4* const rp = sh.rp;
     float (*const qk_s)[FQ_STAGE] = sh.qk_s;
-    int (*const pstart)[17] = sh.pstart;
+    uint32_t (*const markw)[FQ_MAX_PAIRS * FC_TCAP / 32] = sh.markw;
+    uint32_t (*const ent)[16] = sh.ent;
 
     const KernelArgs& P = C.K;
     const int row = lane >> 4, l16 = lane & 15;
@@ -468,24 +470,34 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
                     const int t2 = __builtin_amdgcn_readlane(incl, 47), t3 = __builtin_amdgcn_readlane(incl, 63);
                     const int total = row == 0 ? t0 : row == 1 ? t1 : row == 2 ? t2 : t3;
                     const int longest = max(max(t0, t1), max(t2, t3));
-                    wave_sync();                           // the readers of pstart are done
-                    pstart[row][l16] = incl - cnt;
-                    if (l16 == 0) pstart[row][16] = total;
+                    // Which pair a candidate belongs to, without a search: a bit per candidate marks where the run of a
+                    // pair begins, so the pair of candidate c is the number of marks up to c (a population count of
+                    // the 16 marks of the step plus what the steps before counted) into the list of the pairs that
+                    // have candidates.  One read of the marks and one of that list per step, instead of four dependent
+                    // reads of a bisection: the step's latency was what the wavefronts waited for.
+                    const uint32_t nzrow = (uint32_t)(__ballot(cnt > 0) >> (16 * row)) & 0xffffu;
+                    const int kslot = __popc(nzrow & ((1u << l16) - 1u));
+                    const int first = incl - cnt;
+                    wave_sync();                           // the readers of the marks and the list are done
+#pragma unroll
+                    for (int u = 0; u < FQ_MAX_PAIRS * FC_TCAP / 32 / 16; u++) markw[row][l16 + 16 * u] = 0u;
+                    wave_sync();
+                    if (cnt > 0) {
+                        ent[row][kslot] = (uint32_t)first | ((uint32_t)l16 << 16);
+                        atomicOr(&markw[row][first >> 5], 1u << (first & 31));
+                    }
                     wave_sync();
                     n_seen += (unsigned long long)(t0 + t1 + t2 + t3);
+                    int carry = 0;                         // marks in the steps before this one (the same in a row)
                     for (int base = 0; base < longest; base += 16) {
                         const int c = base + l16;
                         const bool in = c < total;
-                        int lo = 0, hi = 16;               // pstart[lo] <= c < pstart[hi]
-#pragma unroll
-                        for (int s = 0; s < 4; s++) {
-                            const int mid = (lo + hi) >> 1;
-                            const bool le = pstart[row][mid] <= c;
-                            lo = le ? mid : lo;
-                            hi = le ? hi : mid;
-                        }
-                        const int pl = in ? lo : 0;
-                        const float4 v = tab[in ? c - pstart[row][pl] : 0];
+                        const uint32_t m16 = (markw[row][base >> 5] >> (base & 16)) & 0xffffu;
+                        const int kk = carry + __popc(m16 & ((2u << l16) - 1u)) - 1;
+                        carry += __popc(m16);
+                        const uint32_t en = ent[row][in ? kk : 0];
+                        const int pl = in ? (int)(en >> 16) : 0;
+                        const float4 v = tab[in ? c - (int)(en & 0xffffu) : 0];
                         const int ps = min(pc + pl, nst - 1);
                         const float4 cq = rp[ps];
                         const float cqk = qk_s[row][ps];
