@@ -84,14 +84,17 @@ __device__ __forceinline__ int wave_scan_incl(int x) {
 struct FrameShared {
     float4 tab[2 * FC_TCAP];     // the sorted table, or the sorted chunks of a box of its own (two stay resident)
     float4 pq[WAVE];             // rpos and q.k of the staged pairs
-    int pstart[WAVE + 1];        // first candidate of every staged pair, then the total
+    uint32_t markw[WAVE * FC_TCAP / 32];      // one bit per candidate, set where the run of a pair begins
+    uint32_t ent[WAVE];          // the staged pairs that have candidates, in order: first candidate | pair << 16
+    int total;                   // candidates of the list that the marks describe
 };
 // one wavefront, one item: wid = item * H + head.  `others_only`: only the items that the four-heads-per-wavefront
 // search leaves out (box not the table's, or more pairs than it takes).
 __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& sh, int wid, int lane, bool others_only) {
     float4* const tab = sh.tab;
     float4* const pq = sh.pq;
-    int* const pstart = sh.pstart;
+    uint32_t* const markw = sh.markw;
+    uint32_t* const ent = sh.ent;
 
     const KernelArgs& P = C.K;
     const int H = P.H;
@@ -200,7 +203,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                             wave_sync();
                             build_sorted_chunk(tabc, t0c, cnt, bx, L, lane);
                         }
-                        wave_sync();              // pq, the table; the readers of pstart are done
+                        wave_sync();              // pq, the table; the readers of the marks are done
                         // the bound sweep of the second axis looks at the candidates of the first axis' sweep: when
                         // the row is staged as a whole their list is still there
                         const bool relist = !(pass == 1 && sw == 0 && sorted && npairs <= WAVE);
@@ -216,31 +219,39 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                             }
                             mine = min(lo, cnt);
                         }
+                        // The candidates of the pairs laid end to end; which pair candidate c belongs to comes without a
+                        // search: a bit per candidate marks where the run of a pair begins, so the pair of c is the
+                        // number of marks up to c (population counts) into the list of the pairs that have candidates.
                         int total;
                         if (relist) {
                             if (lane >= npc) mine = 0;
                             const int incl = wave_scan_incl(mine);
                             total = __builtin_amdgcn_readlane(incl, WAVE - 1);
-                            pstart[lane] = incl - mine;
-                            if (lane == 0) pstart[WAVE] = total;
+                            const int first = incl - mine;
+                            const int kslot = (int)lane_prefix(__ballot(mine > 0));
+#pragma unroll
+                            for (int u = 0; u < FC_TCAP / 32; u++) markw[lane + WAVE * u] = 0u;
+                            wave_sync();
+                            if (mine > 0) {
+                                ent[kslot] = (uint32_t)first | ((uint32_t)lane << 16);
+                                atomicOr(&markw[first >> 5], 1u << (first & 31));
+                            }
+                            if (lane == 0) sh.total = total;
                             wave_sync();
                         } else {
-                            total = uniform_i(pstart[WAVE]);
+                            total = uniform_i(sh.total);
                         }
                         n_seen += (unsigned long long)total;
+                        int carry = 0;              // marks in the steps before this one
                         for (int base = 0; base < total; base += WAVE) {
                             const int c = base + lane;
                             const bool in = c < total;
-                            int lo = 0, hi = WAVE;      // pstart[lo] <= c < pstart[hi]
-#pragma unroll
-                            for (int s = 0; s < 6; s++) {
-                                const int mid = (lo + hi) >> 1;
-                                const bool le = pstart[mid] <= c;
-                                lo = le ? mid : lo;
-                                hi = le ? hi : mid;
-                            }
-                            const int pl = in ? lo : 0;
-                            const float4 v = tabc[in ? c - pstart[pl] : 0];
+                            const uint64_t m64 = (uint64_t)markw[base >> 5] | ((uint64_t)markw[(base >> 5) + 1] << 32);
+                            const int kk = carry + (int)lane_prefix(m64) + (int)((m64 >> lane) & 1ull) - 1;
+                            carry += __popcll(m64);
+                            const uint32_t en = ent[in ? kk : 0];
+                            const int pl = in ? (int)(en >> 16) : 0;
+                            const float4 v = tabc[in ? c - (int)(en & 0xffffu) : 0];
                             const float4 cq = pq[pl];
                             const int e = e0 + pb + pl;
                             const int t = t0c + (int)(__float_as_uint(v.w) & (uint32_t)(FC_TCAP - 1));
