@@ -1042,7 +1042,8 @@ int cfh_layer_bridge_forward(const float* attn, const float* x_res, int64_t N, i
     if (Wqkv && (!lattice_w || !qkv || !qs || !k || !v || !a))
         return fail(CFH_EINVAL, "layer bridge: with Wqkv, lattice_w and qkv, qs, k, v, a must not be NULL");
     const int wide = F > 3 * D ? F : 3 * D;
-    const size_t lds = (size_t)cfh::BR_ROWS * (2 * (D + cfh::BR_PAD) + wide + cfh::BR_PAD) * sizeof(float);
+    const size_t lds = ((size_t)cfh::BR_ROWS * (2 * (D + cfh::BR_PAD) + wide + cfh::BR_PAD) +
+                        (size_t)cfh::BR_WAVES * cfh::BR_STAGE_FLOATS) * sizeof(float);
     if (lds > 160 * 1024) return fail(CFH_EINVAL, "layer bridge: D=%d, F=%d need %zu bytes of LDS", (int)D, (int)F, lds);
     static int lds_set[64] = {0};
     int dev = 0;

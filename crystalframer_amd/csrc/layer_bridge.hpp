@@ -18,9 +18,11 @@
 namespace cfh {
 
 typedef float v4f_b2 __attribute__((ext_vector_type(4)));
+
 constexpr int BR_ROWS = 16;       // rows (atoms) per workgroup
 constexpr int BR_WAVES = 8;
 constexpr int BR_PAD = 4;         // floats of padding per LDS row
+constexpr int BR_STAGE_FLOATS = 64 * (32 + BR_PAD);    // per wavefront: the weights of one batch of products (forward)
 
 struct BridgeArgs {
     const float* attn; const float* xres;         // (N, D)
@@ -43,23 +45,67 @@ template <bool RELU, int T, int U>
 __device__ __forceinline__ void bridge_tiles(const float* in, int K, const float* __restrict__ W,
                                              const float* __restrict__ b, int O, const float* __restrict__ res,
                                              const float* res_lds, int r0, int nrows, float* out_lds,
-                                             float* __restrict__ out_g, int t0) {
+                                             float* __restrict__ out_g, int t0, float* stage) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, kk = lane >> 4;
     const int ldin = K + BR_PAD, ldout = O + BR_PAD;
     const float* const arow = in + col * ldin + 4 * kk;
-    const float* const wrow = W + (size_t)(16 * (t0 + wave) + col) * K + 4 * kk;      // tile tt: + 64 tt K
+    // The weights of the T tiles for 16 U steps of k: (16 T rows) x (16 U floats), T U float4 per lane.  A lane of the
+    // matrix operand needs four consecutive k of ITS row, and the 16 lanes of a quarter wavefront hold 16 different
+    // rows: read straight from memory that is 64 cache lines per load instruction, which the vector cache takes
+    // one per cycle -- twice the time of the products.  So the wavefront reads whole row pieces (16 U floats of a row
+    // by 4 U consecutive lanes) and turns them in a piece of LDS of its own.
+    constexpr int CH = 4 * U;                     // float4 per row piece
+    constexpr int LDS_ROW = 16 * U + BR_PAD;      // floats per staged row (the padding spreads the rows over the banks)
+    const float* wsrc[T * U];
+    int wdst[T * U];
+#pragma unroll
+    for (int i = 0; i < T * U; i++) {
+        const int q = i * 64 + lane, row = q / CH, ch = q % CH;
+        const int tt = row >> 4, j = row & 15;
+        wsrc[i] = W + (size_t)(16 * (t0 + wave + BR_WAVES * tt) + j) * K + 4 * ch;
+        wdst[i] = row * LDS_ROW + 4 * ch;
+    }
+    const float* const srow = stage + col * LDS_ROW + 4 * kk;       // tile tt: + 16 tt LDS_ROW
     v4f_b2 acc[T];
 #pragma unroll
     for (int tt = 0; tt < T; tt++) acc[tt] = v4f_b2{0.f, 0.f, 0.f, 0.f};
-    for (int k0 = 0; k0 < K; k0 += 16 * U) {
+    constexpr int STEP = 16 * U;
+    v4f_b2 g4[T * U];
+#pragma unroll
+    for (int i = 0; i < T * U; i++) g4[i] = *reinterpret_cast<const v4f_b2*>(wsrc[i]);
+    // bias and residual of the lane's outputs: asked for now, used behind the products
+    float add[T][4];
+#pragma unroll
+    for (int tt = 0; tt < T; tt++) {
+        const int n = 16 * (t0 + wave + BR_WAVES * tt) + col;
+        const float bias = b ? b[n] : 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int m = 4 * kk + c;
+            add[tt][c] = bias + (res && m < nrows ? res[(size_t)(r0 + m) * O + n] : 0.f);
+        }
+    }
+    for (int k0 = 0; k0 < K; k0 += STEP) {
+        wave_sync();                               // the products of the step before have read the stage
+#pragma unroll
+        for (int i = 0; i < T * U; i++) *reinterpret_cast<v4f_b2*>(stage + wdst[i]) = g4[i];
+        {   // the next batch is asked for before the products of this one (the last one once more at the end: no
+            // branch around the loads).  Asking two steps ahead gains nothing: a compute unit takes about 20 bytes a
+            // cycle from the L2 however many loads are in flight, and the 768 KB of weights that every workgroup
+            // streams make that the bound of the kernel (18 us), above the 10 us of its matrix instructions.
+            const int kn = k0 + STEP < K ? k0 + STEP : k0;
+#pragma unroll
+            for (int i = 0; i < T * U; i++) g4[i] = *reinterpret_cast<const v4f_b2*>(wsrc[i] + kn);
+        }
+        wave_sync();
         float4 a4[U], w4[U][T];
 #pragma unroll
         for (int u = 0; u < U; u++) {
             a4[u] = *reinterpret_cast<const float4*>(arow + k0 + 16 * u);
 #pragma unroll
             for (int tt = 0; tt < T; tt++)
-                w4[u][tt] = *reinterpret_cast<const float4*>(wrow + (size_t)16 * BR_WAVES * tt * K + k0 + 16 * u);
+                w4[u][tt] = *reinterpret_cast<const float4*>(srow + 16 * tt * LDS_ROW + 16 * u);
         }
 #pragma unroll
         for (int u = 0; u < U; u++)
@@ -74,12 +120,10 @@ __device__ __forceinline__ void bridge_tiles(const float* in, int K, const float
 #pragma unroll
     for (int tt = 0; tt < T; tt++) {
         const int n = 16 * (t0 + wave + BR_WAVES * tt) + col;
-        const float bias = b ? b[n] : 0.f;
 #pragma unroll
         for (int c = 0; c < 4; c++) {
             const int m = 4 * kk + c;
-            float val = acc[tt][c] + bias;
-            if (res && m < nrows) val += res[(size_t)(r0 + m) * O + n];
+            float val = acc[tt][c] + add[tt][c];
             if (res_lds) val += res_lds[m * ldout + n];
             if (RELU) val = fmaxf(val, 0.f);
             if (out_lds) out_lds[m * ldout + n] = val;
@@ -93,15 +137,16 @@ template <bool RELU>
 __device__ __forceinline__ void bridge_stage(const float* in, int K, const float* __restrict__ W,
                                              const float* __restrict__ b, int O, const float* __restrict__ res,
                                              const float* res_lds, int r0, int nrows, float* out_lds,
-                                             float* __restrict__ out_g) {
+                                             float* __restrict__ out_g, float* stage) {
     int t0 = 0;
     int left = O / (16 * BR_WAVES);     // tiles per wavefront still to do
-    while (left >= 4) { bridge_tiles<RELU, 4, 2>(in, K, W, b, O, res, res_lds, r0, nrows, out_lds, out_g, t0); t0 += 4 * BR_WAVES; left -= 4; }
-    if (left >= 2) { bridge_tiles<RELU, 2, 4>(in, K, W, b, O, res, res_lds, r0, nrows, out_lds, out_g, t0); t0 += 2 * BR_WAVES; left -= 2; }
-    if (left >= 1) { bridge_tiles<RELU, 1, 8>(in, K, W, b, O, res, res_lds, r0, nrows, out_lds, out_g, t0); }
+    while (left >= 4) { bridge_tiles<RELU, 4, 2>(in, K, W, b, O, res, res_lds, r0, nrows, out_lds, out_g, t0, stage); t0 += 4 * BR_WAVES; left -= 4; }
+    if (left >= 2) { bridge_tiles<RELU, 2, 4>(in, K, W, b, O, res, res_lds, r0, nrows, out_lds, out_g, t0, stage); t0 += 2 * BR_WAVES; left -= 2; }
+    if (left >= 1) { bridge_tiles<RELU, 1, 8>(in, K, W, b, O, res, res_lds, r0, nrows, out_lds, out_g, t0, stage); }
 }
 
-// grid: ceil(N / 16) workgroups of 512 threads; dynamic LDS: 16 (2 (D + 4) + max(F, 3 D) + 4) floats.
+// grid: ceil(N / 16) workgroups of 512 threads; dynamic LDS: 16 (2 (D + 4) + max(F, 3 D) + 4) floats and
+// BR_STAGE_FLOATS per wavefront.
 // D, F multiples of 128; D = 16 H.
 __global__ __launch_bounds__(64 * BR_WAVES) void layer_bridge_fwd_kernel(const BridgeArgs P) {
     extern __shared__ __attribute__((aligned(16))) float bridge_lds[];
@@ -109,6 +154,7 @@ __global__ __launch_bounds__(64 * BR_WAVES) void layer_bridge_fwd_kernel(const B
     float* const s_a = bridge_lds;                            // [16][D+4]  attention output, later x2
     float* const s_b = s_a + BR_ROWS * (D + BR_PAD);          // [16][D+4]  x1
     float* const s_c = s_b + BR_ROWS * (D + BR_PAD);          // [16][F+4]  h, later [16][3D+4] qkv
+    float* const stage = s_c + BR_ROWS * ((F > Q ? F : Q) + BR_PAD) + (threadIdx.x >> 6) * BR_STAGE_FLOATS;
     const int r0 = blockIdx.x * BR_ROWS;
     const int nrows = min(BR_ROWS, P.N - r0);
     for (int idx = threadIdx.x * 4; idx < BR_ROWS * D; idx += 64 * BR_WAVES * 4) {
@@ -118,14 +164,14 @@ __global__ __launch_bounds__(64 * BR_WAVES) void layer_bridge_fwd_kernel(const B
         *reinterpret_cast<float4*>(s_a + m * (D + BR_PAD) + c) = v;
     }
     __syncthreads();
-    bridge_stage<false>(s_a, D, P.Wo, P.bo, D, P.xres, nullptr, r0, nrows, s_b, P.x1);
+    bridge_stage<false>(s_a, D, P.Wo, P.bo, D, P.xres, nullptr, r0, nrows, s_b, P.x1, stage);
     __syncthreads();
-    bridge_stage<true>(s_b, D, P.W1, P.b1, F, nullptr, nullptr, r0, nrows, s_c, P.h);
+    bridge_stage<true>(s_b, D, P.W1, P.b1, F, nullptr, nullptr, r0, nrows, s_c, P.h, stage);
     __syncthreads();
-    bridge_stage<false>(s_c, F, P.W2, P.b2, D, nullptr, s_b, r0, nrows, s_a, P.x2);
+    bridge_stage<false>(s_c, F, P.W2, P.b2, D, nullptr, s_b, r0, nrows, s_a, P.x2, stage);
     if (!P.Wq) return;
     __syncthreads();
-    bridge_stage<false>(s_a, D, P.Wq, P.bq, Q, nullptr, nullptr, r0, nrows, s_c, P.qkv);
+    bridge_stage<false>(s_a, D, P.Wq, P.bq, Q, nullptr, nullptr, r0, nrows, s_c, P.qkv, stage);
     __syncthreads();
     // split of qkv, query scaling
     const int ldq = Q + BR_PAD;

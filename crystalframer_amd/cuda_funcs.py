@@ -1338,7 +1338,7 @@ class LayerBridgeHIP(torch.autograd.Function):
     def supported(D: int, F: int, H: int) -> bool:
         wide = max(F, 3 * D)
         return (D % 128 == 0 and F % 128 == 0 and D == 16 * H and H <= 32
-                and 16 * (2 * (D + 4) + wide + 4) * 4 <= 160 * 1024)
+                and (16 * (2 * (D + 4) + wide + 4) + 8 * 64 * 36) * 4 <= 160 * 1024)
 
     @staticmethod
     def forward(ctx, attn, x_res, Wo, bo, W1, b1, W2, b2, stacked, in_bias, lattice_w, gauss_scale, H, c1, lb,
