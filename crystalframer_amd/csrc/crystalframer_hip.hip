@@ -986,7 +986,7 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
     for (int32_t j = 0; j < njobs; j++) {
         const cfh_linear_grad_job& J = jobs[j];
         if (J.N < 0 || J.I < 1 || J.O < 1 || J.N > 0x7fffffffLL / 64 || J.I > 65536 || J.O > 65536 || J.ldx < J.I ||
-            J.ldy < J.O || J.ldx > 0x7fffffffLL || J.ldy > 0x7fffffffLL)
+            J.ldy < J.O || J.ldx > (1LL << 26) || J.ldy > (1LL << 26))
             return fail(CFH_EINVAL, "job %d: sizes N=%lld I=%lld O=%lld ldx=%lld ldy=%lld out of range", (int)j,
                         (long long)J.N, (long long)J.I, (long long)J.O, (long long)J.ldx, (long long)J.ldy);
         if ((!J.dW && !J.db) || (J.N > 0 && (!J.dy || (J.dW && !J.x))))
@@ -995,11 +995,29 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
     hipStream_t st = (hipStream_t)stream;
     for (int32_t first = 0; first < njobs; first += cfh::WGRAD_MAX_JOBS) {
         const int32_t last = njobs < first + cfh::WGRAD_MAX_JOBS ? njobs : first + cfh::WGRAD_MAX_JOBS;
+        // a job whose shape and alignment allow it takes the variant with 16-byte loads
+        auto wide = [](const cfh_linear_grad_job& J) {
+            return J.dW && J.O % 64 == 0 && J.I % 64 == 0 && J.ldx % 4 == 0 && J.ldy % 4 == 0 &&
+                   ((uintptr_t)J.x | (uintptr_t)J.dy) % 16 == 0;
+        };
+        auto tiles_of = [&](const cfh_linear_grad_job& J, long& bx, long& by) {
+            bx = J.dW ? (J.I + 63) / 64 : 1;
+            by = (J.O + 63) / 64;
+        };
         long tiles = 0;
         for (int32_t j = first; j < last; j++)
-            if (jobs[j].N > 0) tiles += (long)(jobs[j].dW ? (jobs[j].I + 63) / 64 : 1) * (long)((jobs[j].O + 63) / 64);
+            if (jobs[j].N > 0) {
+                long bx, by;
+                tiles_of(jobs[j], bx, by);
+                tiles += bx * by;
+            }
         if (tiles == 0) continue;
-        const int want = (int)(1900 / tiles > 0 ? 1900 / tiles : 1);   // slices of a job: the workgroups stay below the 2048 that are resident at once
+        // slices of a job: the workgroups stay just below the four per compute unit that are resident at once (a few
+        // more would run as a second round and double the time)
+        int cus = device_cus();
+        if (cus <= 0) cus = 256;
+        const long target = 4L * cus - 24;
+        const int want = (int)(target / tiles > 0 ? target / tiles : 1);   // slices of a job: the workgroups stay below the 2048 that are resident at once
                                                                         // (a few more would run as a second round and double the time)
         cfh::WgradJobs T{};
         int blocks = 0;
@@ -1009,7 +1027,9 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
             cfh::WgradJob& W = T.job[T.njobs++];
             W.x = J.x; W.dy = J.dy; W.dW = J.dW; W.db = J.db;
             W.N = (int)J.N; W.I = (int)J.I; W.O = (int)J.O; W.ldx = (int)J.ldx; W.ldy = (int)J.ldy;
-            W.bx = J.dW ? (int)((J.I + 63) / 64) : 1; W.by = (int)((J.O + 63) / 64);
+            long bx, by;
+            tiles_of(J, bx, by);
+            W.bx = (int)bx; W.by = (int)by; W.wide = wide(J) ? 1 : 0;
             int slices = want;
             const int max_slices = (int)((J.N + 31) / 32);
             if (slices > max_slices) slices = max_slices;
@@ -1021,7 +1041,8 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
             W.block0 = blocks;
             blocks += W.bx * W.by * slices;
         }
-        hipLaunchKernelGGL(cfh::linear_wgrad_batch_kernel, dim3(blocks), dim3(256), 0, st, T);
+        T.blocks = blocks;
+        hipLaunchKernelGGL(cfh::linear_wgrad_batch_kernel, dim3((blocks + 7) & ~7), dim3(256), 0, st, T);
     }
     return finish_launch("linear_weight_bias_grad_batch");
 }

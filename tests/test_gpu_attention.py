@@ -197,7 +197,10 @@ def test_second_stream_fork_and_join_order_a_library_call():
 
 
 @pytest.mark.parametrize("N,I,O,bias", [(2372, 128, 384, True), (2372, 512, 128, True), (2372, 98, 128, False),
-                                        (37, 20, 50, True), (1, 16, 16, True), (0, 16, 32, True)])
+                                        (37, 20, 50, True), (1, 16, 16, True), (0, 16, 32, True),
+                                        # multiples of 64 take the kernel variant with 16-byte loads: few rows (wavefronts
+                                        # of a workgroup without rows), rows that do not fill the last chunk
+                                        (37, 64, 128, True), (5, 128, 64, True), (1001, 64, 64, False), (1, 64, 64, True)])
 def test_linear_weight_and_bias_gradients(N, I, O, bias):
     """The library's weight/bias gradient kernel against float64 autograd of x W^T + b."""
     import crystalframer_amd as cf
