@@ -1488,7 +1488,8 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         int per_slice = (int)((N + nslices - 1) / nslices);
         per_slice = (per_slice + 15) & ~15;
         nslices = (int)((N + per_slice - 1) / per_slice);
-        hipLaunchKernelGGL(cfh::core_gwcat_kernel, dim3(L.hw / 64, p->num_heads, nslices), dim3(cfh::WAVE), 0, st_w, gout,
+        hipLaunchKernelGGL(cfh::core_gwcat_kernel, dim3((L.hw / 64 + cfh::GW_WPB - 1) / cfh::GW_WPB, p->num_heads, nslices),
+                           dim3(cfh::WAVE * cfh::GW_WPB), 0, st_w, gout,
                            hist, gwcat, (int)N, p->num_heads, L.hw, per_slice);
         hipLaunchKernelGGL(cfh::core_gw_finish_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st_w, gwcat, nslices,
                            p->num_heads, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, gW_dist, gW_axis1, gW_axis2,
@@ -1595,7 +1596,8 @@ int cfh_fused_core_weight_gradients(const cfh_params* p, const cfh_core_wgrad_jo
             slices += nslices;
         }
         if (slices > 0)
-            hipLaunchKernelGGL(cfh::core_gwcat_multi_kernel, dim3(hw / 64, p->num_heads, slices), dim3(cfh::WAVE), 0, st, T);
+            hipLaunchKernelGGL(cfh::core_gwcat_multi_kernel, dim3((hw / 64 + cfh::GW_WPB - 1) / cfh::GW_WPB, p->num_heads, slices),
+                               dim3(cfh::WAVE * cfh::GW_WPB), 0, st, T);
         hipLaunchKernelGGL(cfh::core_gw_finish_multi_kernel, dim3(p->num_heads * cfh::DH, T.njobs), dim3(256), 0, st, T);
     }
     return finish_launch("fused_core_weight_gradients");

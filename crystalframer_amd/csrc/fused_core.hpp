@@ -801,12 +801,15 @@ __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restri
 }
 
 // gwcat (slice,H,16,hw) = sum over a slice of the atoms of go (.,h,16) (x) hist (h,.,hw): wavefront per (head, 64-word
-// block, slice); four MFMA tiles with interleaved columns as above.  grid (hw/64, H, nslices), at most
+// block, slice); four MFMA tiles with interleaved columns as above.  grid (ceil(hw/64 / GW_WPB), H, nslices), at most
 // CORE_GW_SLICES slices.
 __device__ __forceinline__ void core_gwcat_block(const float* __restrict__ go, const float* __restrict__ hist,
                                                  float* __restrict__ gwcat, int N, int H, int hw, int per_slice, int slice) {
-    const int lane = threadIdx.x, col = lane & 15, kk = lane >> 4;
-    const int w0 = blockIdx.x * 64, h = blockIdx.y;
+    // the GW_WPB wavefronts of a workgroup take neighbouring pieces of the same rows at the same time: GW_WPB x 256
+    // contiguous bytes of a row instead of 256 bytes every 4 KB (82 -> 70 us for the four layers of the benchmark)
+    const int lane = threadIdx.x & (WAVE - 1), col = lane & 15, kk = lane >> 4;
+    const int w0 = ((int)blockIdx.x * (int)(blockDim.x >> 6) + (int)(threadIdx.x >> 6)) * 64, h = blockIdx.y;
+    if (w0 >= hw) return;
     const int i_begin = slice * per_slice, i_end = min(N, i_begin + per_slice);
     v4f_c acc[4];
 #pragma unroll
@@ -821,13 +824,16 @@ __device__ __forceinline__ void core_gwcat_block(const float* __restrict__ go, c
         for (int d = 0; d < GW_DEPTH; d++)
 #pragma unroll
             for (int j = 0; j < 4; j++) {
+                // (no branch around the loads: an atom past the end reads the slice's first one, with go as zero)
                 const int it = ib + 16 * d + 4 * j + kk;
                 const bool live = it < i_end;
-                const size_t base = ((size_t)(live ? it : i_begin) * H + h);
-                av[d][j] = live ? go[base * DH + col] : 0.0f;
-                bv[d][j] = live ? *reinterpret_cast<const float4*>(hist + ((size_t)h * N + it) * hw + w0 + 4 * col)
-                                : make_float4(0.f, 0.f, 0.f, 0.f);
+                const int itc = live ? it : i_begin;
+                const float g = go[((size_t)itc * H + h) * DH + col];
+                av[d][j] = live ? g : 0.0f;
+                bv[d][j] = *reinterpret_cast<const float4*>(hist + ((size_t)h * N + itc) * hw + w0 + 4 * col);
             }
+        // (without the branches the compiler would put every load next to its product: 113 us instead of 78)
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int d = 0; d < GW_DEPTH; d++)
 #pragma unroll
@@ -847,12 +853,13 @@ __device__ __forceinline__ void core_gwcat_block(const float* __restrict__ go, c
         *reinterpret_cast<float4*>(part + ((size_t)h * DH + 4 * kk + r) * hw + w0 + 4 * col) =
             make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
 }
-__global__ __launch_bounds__(WAVE) void core_gwcat_kernel(const float* __restrict__ go, const float* __restrict__ hist,
+constexpr int GW_WPB = 4;          // wavefronts per workgroup of the two kernels below (8: the same; 16: far slower)
+__global__ __launch_bounds__(WAVE * GW_WPB) void core_gwcat_kernel(const float* __restrict__ go, const float* __restrict__ hist,
                                                           float* __restrict__ gwcat, int N, int H, int hw, int per_slice) {
     core_gwcat_block(go, hist, gwcat, N, H, hw, per_slice, (int)blockIdx.z);
 }
-// several jobs: grid (hw/64, H, slices of all jobs); the job of a slice by a scan of the (few) jobs
-__global__ __launch_bounds__(WAVE) void core_gwcat_multi_kernel(const CoreWgradJobs T) {
+// several jobs: grid (ceil(hw/64 / GW_WPB), H, slices of all jobs); the job of a slice by a scan of the (few) jobs
+__global__ __launch_bounds__(WAVE * GW_WPB) void core_gwcat_multi_kernel(const CoreWgradJobs T) {
     int j = 0;
     while (j + 1 < T.njobs && (int)blockIdx.z >= T.job[j + 1].slice0) j++;
     const CoreWgradJob& J = T.job[j];
