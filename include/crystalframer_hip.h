@@ -451,8 +451,10 @@ int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int6
  * with row stride ldy (so a job may take a column block of a wider dy, e.g. one of the three
  * stacked input projections), dW (O,I) contiguous, db (O) or NULL.  A job with dW == NULL adds only the
  * column sums of dy to db (x is not read, I = ldx = 1): any sum over rows that a backward pass leaves
- * for its end, e.g. the per-block partials of cfh_attention_inputs_backward.  `jobs` is a host array; it is
- * copied into the kernel arguments, 32 jobs per launch.  Deferring the weight gradients of a whole
+ * for its end, e.g. the per-block partials of cfh_attention_inputs_backward.  Row strides up to 2^26 elements.  A
+ * job whose O and I are multiples of 64, whose strides are multiples of 4 and whose x and dy are 16-byte aligned
+ * takes a faster kernel variant (16-byte loads); the results are the same up to the order of the float sums.
+ * `jobs` is a host array; it is copied into the kernel arguments, 32 jobs per launch.  Deferring the weight gradients of a whole
  * backward pass to one call replaces one launch (plus clearing) per layer -- latency-bound at these
  * sizes -- by a launch that fills the chip.  No counterpart in the reference (autograd of
  * torch.nn.functional.linear, one GEMM per layer).
