@@ -1350,7 +1350,7 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
                            buf.table);
         if (buf.near && E > 0) {
             const int s0 = 2 * C.table_R + 1;
-            hipLaunchKernelGGL(cfh::pair_nearest_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0, st, rpos, edges,
+            hipLaunchKernelGGL(cfh::pair_nearest_kernel, dim3((unsigned)((E * 8 + 255) / 256)), dim3(256), 0, st, rpos, edges,
                                batch, buf.table, s0 * s0 * s0, (int)E, buf.near);
         }
     }
