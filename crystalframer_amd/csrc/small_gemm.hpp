@@ -31,9 +31,7 @@ __global__ __launch_bounds__(256) void small_linear_fwd_kernel(const float* __re
     const float4* wb = reinterpret_cast<const float4*>(w + (size_t)cb * K) + kk;
     v4f_g acc00 = {0.f, 0.f, 0.f, 0.f}, acc01 = acc00, acc10 = acc00, acc11 = acc00;
     const int chunks = K / 16;
-#pragma unroll 4
-    for (int c = 0; c < chunks; c++) {
-        const float4 a0 = xa[4 * c], a1 = xb[4 * c], b0 = wa[4 * c], b1 = wb[4 * c];
+    auto products = [&](const float4& a0, const float4& a1, const float4& b0, const float4& b1) {
         const float A0[4] = {a0.x, a0.y, a0.z, a0.w}, A1[4] = {a1.x, a1.y, a1.z, a1.w};
         const float B0[4] = {b0.x, b0.y, b0.z, b0.w}, B1[4] = {b1.x, b1.y, b1.z, b1.w};
 #pragma unroll
@@ -43,7 +41,19 @@ __global__ __launch_bounds__(256) void small_linear_fwd_kernel(const float* __re
             acc10 = __builtin_amdgcn_mfma_f32_16x16x4f32(A1[j], B0[j], acc10, 0, 0, 0);
             acc11 = __builtin_amdgcn_mfma_f32_16x16x4f32(A1[j], B1[j], acc11, 0, 0, 0);
         }
+    };
+    // four chunks at a time, their sixteen loads asked for before the first product (left to itself the compiler puts
+    // every load next to its product: a chain of trips to the L2, and the kernel is nothing but that chain)
+    int c = 0;
+    for (; c + 4 <= chunks; c += 4) {
+        float4 a0[4], a1[4], b0[4], b1[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) { a0[u] = xa[4 * (c + u)]; a1[u] = xb[4 * (c + u)]; b0[u] = wa[4 * (c + u)]; b1[u] = wb[4 * (c + u)]; }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 4; u++) products(a0[u], a1[u], b0[u], b1[u]);
     }
+    for (; c < chunks; c++) products(xa[4 * c], xb[4 * c], wa[4 * c], wb[4 * c]);
     // accumulator component c of lane (kk, col): row 4 kk + c of the 16x16 block, column col
     const float ba = b ? b[ca] : 0.f, bb = b ? b[cb] : 0.f;
     auto put = [&](int r, int n, float v) {
@@ -72,20 +82,37 @@ __global__ __launch_bounds__(256) void small_linear_dx_kernel(const float* __res
     const float4* yb = reinterpret_cast<const float4*>(dy + (size_t)rb * N) + kk;
     v4f_g acc00 = {0.f, 0.f, 0.f, 0.f}, acc01 = acc00, acc10 = acc00, acc11 = acc00;
     const int chunks = N / 16;
-#pragma unroll 2
-    for (int c = 0; c < chunks; c++) {
-        const float4 a0 = ya[4 * c], a1 = yb[4 * c];
-        const float A0[4] = {a0.x, a0.y, a0.z, a0.w}, A1[4] = {a1.x, a1.y, a1.z, a1.w};
+    // two chunks at a time, all their loads asked for before the first product (see small_linear_fwd_kernel)
+    auto step = [&](int c, int nch) {
+        float4 a0[2], a1[2];
+        float b0[2][4], b1[2][4];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const float* wr = w + (size_t)(16 * c + 4 * kk + j) * K;      // row n = 16 c + 4 kk + j of W
-            const float b0 = wr[ca], b1 = wr[cb];
-            acc00 = __builtin_amdgcn_mfma_f32_16x16x4f32(A0[j], b0, acc00, 0, 0, 0);
-            acc01 = __builtin_amdgcn_mfma_f32_16x16x4f32(A0[j], b1, acc01, 0, 0, 0);
-            acc10 = __builtin_amdgcn_mfma_f32_16x16x4f32(A1[j], b0, acc10, 0, 0, 0);
-            acc11 = __builtin_amdgcn_mfma_f32_16x16x4f32(A1[j], b1, acc11, 0, 0, 0);
+        for (int u = 0; u < 2; u++) {
+            const int cu = u < nch ? c + u : c;
+            a0[u] = ya[4 * cu]; a1[u] = yb[4 * cu];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float* wr = w + (size_t)(16 * cu + 4 * kk + j) * K;      // row n = 16 c + 4 kk + j of W
+                b0[u][j] = wr[ca]; b1[u][j] = wr[cb];
+            }
         }
-    }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            if (u >= nch) continue;
+            const float A0[4] = {a0[u].x, a0[u].y, a0[u].z, a0[u].w}, A1[4] = {a1[u].x, a1[u].y, a1[u].z, a1[u].w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                acc00 = __builtin_amdgcn_mfma_f32_16x16x4f32(A0[j], b0[u][j], acc00, 0, 0, 0);
+                acc01 = __builtin_amdgcn_mfma_f32_16x16x4f32(A0[j], b1[u][j], acc01, 0, 0, 0);
+                acc10 = __builtin_amdgcn_mfma_f32_16x16x4f32(A1[j], b0[u][j], acc10, 0, 0, 0);
+                acc11 = __builtin_amdgcn_mfma_f32_16x16x4f32(A1[j], b1[u][j], acc11, 0, 0, 0);
+            }
+        }
+    };
+    int c = 0;
+    for (; c + 2 <= chunks; c += 2) step(c, 2);
+    if (c < chunks) step(c, 1);
     auto put = [&](int r, int n, float v) {
         if (r < M && n < K) dx[(size_t)r * K + n] = v;
     };
