@@ -1219,8 +1219,9 @@ int cfh_adamw_step_batch(const cfh_adamw_job* jobs, int32_t njobs, float lr, flo
 // ---- fused attention core ----------------------------------------------------------------------------------------
 namespace {
 struct CoreLayout {
-    size_t items, sorted, near, wcat, gwcat, G, total;
+    size_t items, sorted, near, wcat, gwcat, G, slow, total;
     int hw;
+    int prep_blocks;      // blocks of 256 threads of the launch that makes the item records
 };
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 CoreLayout core_layout(const cfh_params* p, int64_t N, int64_t E, int64_t B, bool backward) {
@@ -1233,6 +1234,13 @@ CoreLayout core_layout(const cfh_params* p, int64_t N, int64_t E, int64_t B, boo
     L.wcat = off; off += align256((size_t)p->num_heads * cfh::DH * L.hw * sizeof(float));
     L.gwcat = off; if (backward) off += align256((size_t)cfh::CORE_GW_SLICES * p->num_heads * cfh::DH * L.hw * sizeof(float));
     L.G = off; if (backward) off += align256((size_t)(N > 0 ? N : 1) * p->num_heads * L.hw * sizeof(float));
+    {
+        const int64_t threads = N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
+                                                                                       : (int64_t)p->num_heads * cfh::NQUEUE;
+        L.prep_blocks = (int)((threads + 255) / 256);
+    }
+    // the lists of the records that the main kernel takes first (forward: made with the records)
+    L.slow = off; if (!backward) off += align256((size_t)L.prep_blocks * (1 + cfh::SLOW_SLOTS) * sizeof(int32_t));
     L.total = off;
     return L;
 }
@@ -1286,7 +1294,7 @@ CoreBuffers fill_core(cfh::CoreArgs& C, const cfh_params* p, const CoreLayout& L
 // one wavefront (= workgroup) per (item, head); the hardware deals them to the compute units as slots free up
 template <typename Kern>
 int launch_core(Kern kern, const cfh::CoreArgs& C, hipStream_t st, const char* what, unsigned waves = 0) {
-    if (waves == 0) waves = (unsigned)C.K.N * (unsigned)C.K.H;
+    if (waves == 0) waves = (unsigned)C.K.N * (unsigned)C.K.H + (unsigned)C.slow_wgs;
     const unsigned blocks = (waves + cfh::CORE_WPB - 1) / cfh::CORE_WPB;
     bool timed = false;
     TimedLaunch t;
@@ -1358,9 +1366,13 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     float* wcat = buf.wcat;
     const cfh::WcatArgs WA{W_dist, W_axis1, W_axis2, W_axis3, L.hw, p->dist_coef, p->angle_coef, p->angle_wscale, wcat};
     {
-        const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
-                                                                                          : p->num_heads * cfh::NQUEUE);
-        const int prep_blocks = (threads + 255) / 256;
+        const int prep_blocks = L.prep_blocks;
+        // records whose box is not the table's are listed by the launch that makes them and taken first by the main kernel
+        if (buf.table) {
+            C.K.slow_count = reinterpret_cast<int32_t*>(ws + L.slow);
+            C.K.slow_list = C.K.slow_count + prep_blocks;
+            C.K.slow_R = C.table_R;
+        }
         // the item records and the concatenated weights in one launch
         if (search) {
             // records with the query, frame search through the first set of queues; it leaves the frames in the
@@ -1404,6 +1416,7 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
         }
     }
     C.out = out; C.prob = prob; C.z = z; C.hist = hist;
+    C.slow_wgs = C.K.slow_count ? L.prep_blocks * cfh::SLOW_SLOTS : 0;
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "fused_core_forward";
 #define CFH_CORE_DISPATCH(KERNEL)                                                                         \

@@ -346,6 +346,10 @@ struct KernelArgs {
                                   // works through the same item records without a prepare launch of its own
     int32_t frames_to_records;    // frame search: also store the orthonormal frames into the item records
     uint32_t* items;              // (N, H, REC_WORDS) item records of this launch
+    int32_t* slow_count;          // optional: per block of 256 records, how many of them are listed in slow_list
+    int32_t* slow_list;           // (blocks, SLOW_SLOTS) records whose box is not the usual one, for the launches that
+                                  // take those items first (see prepare_items_block)
+    int32_t slow_R;               // half-width of the usual box
     unsigned long long* stats;    // optional running totals (see STAT_* below); never reset by a launch
     int32_t* status;              // word of the workspace header: set to 1 when a box was cut back to RMAX (never cleared)
     int32_t N, E, H;
@@ -417,6 +421,8 @@ __device__ __forceinline__ int first_queue(int H) { return ((int)blockIdx.x / H)
 //   5..13 lattice rows, 14..22 frame axes (frame search: 14..29 the query vector q_ih),
 //   30 first neighbour atom (the pairs of an atom point at consecutive atoms), 31 crystal
 constexpr int REC_WORDS = 32;
+constexpr int SLOW_SLOTS = 64;                 // records per block of 256 that can be listed as slow
+constexpr uint32_t REC_BOX_LISTED = 0x80000000u;      // flag in the box word of a listed record
 enum { REC_ATOM = 0, REC_E0 = 1, REC_NPAIRS = 2, REC_BOX = 3, REC_A = 4, REC_LATTICE = 5, REC_FRAMES = 14,
        REC_QUERY = 14 };
 
@@ -470,32 +476,56 @@ __device__ __forceinline__ void prepare_items_block(const KernelArgs& P, int wit
         for (int en = 0; en < 4; en++)
             if (P.gw_out[en]) P.gw_out[en][idx] = 0.0f;
     }
-    if (idx >= P.N * P.H) return;
-    const int it = idx / P.H, h = idx - it * P.H;
-    const int i = P.order ? P.order[it] : it;
-    const int b = (int)P.batch[i];
-    const float a = P.a_ih[(size_t)i * P.H + h];
-    float rvl1 = 0.f, rvl2 = 0.f, rvl3 = 0.f;
-    if (P.rvlen) { rvl1 = P.rvlen[(size_t)b * 3 + 0]; rvl2 = P.rvlen[(size_t)b * 3 + 1]; rvl3 = P.rvlen[(size_t)b * 3 + 2]; }
-    const Box bx = translation_box(a, rvl1, rvl2, rvl3, P.cutoff_radius, P.lattice_range, P.minimum_range);
-    if (bx.over && P.status) *P.status = 1;
-    uint32_t* rec = P.items + (size_t)idx * REC_WORDS;
-    const int e0 = (int)P.e_start[i];
-    rec[REC_ATOM] = (uint32_t)i;
-    rec[REC_E0] = (uint32_t)e0;
-    rec[REC_NPAIRS] = (uint32_t)((int)P.e_start[i + 1] - e0);
-    rec[REC_BOX] = (uint32_t)(bx.R1 | (bx.R2 << 8) | (bx.R3 << 16));
-    rec[REC_A] = __float_as_uint(a);
-    for (int d = 0; d < 9; d++) rec[REC_LATTICE + d] = __float_as_uint(P.tvecs[(size_t)b * 9 + d]);
-    rec[30] = (uint32_t)(P.e_start[i + 1] > e0 ? (int)P.edges[(size_t)P.E + e0] : i);      // first neighbour atom
-    rec[31] = (uint32_t)b;                                                                  // crystal
-    if (with_query) {
-        for (int c = 0; c < DH; c++) rec[REC_QUERY + c] = __float_as_uint(P.q[((size_t)i * P.H + h) * DH + c]);
-    } else if (P.frames) {
-        for (int ax = 0; ax < 3; ax++)
-            for (int d = 0; d < 3; d++)
-                rec[REC_FRAMES + ax * 3 + d] = __float_as_uint(P.frames[(((size_t)ax * P.N + i) * P.H + h) * 3 + d]);
+    const bool valid = idx < P.N * P.H;
+    bool slow = false;
+    uint32_t* rec = P.items + (size_t)(valid ? idx : 0) * REC_WORDS;
+    uint32_t boxw = 0;
+    if (valid) {
+        const int it = idx / P.H, h = idx - it * P.H;
+        const int i = P.order ? P.order[it] : it;
+        const int b = (int)P.batch[i];
+        const float a = P.a_ih[(size_t)i * P.H + h];
+        float rvl1 = 0.f, rvl2 = 0.f, rvl3 = 0.f;
+        if (P.rvlen) { rvl1 = P.rvlen[(size_t)b * 3 + 0]; rvl2 = P.rvlen[(size_t)b * 3 + 1]; rvl3 = P.rvlen[(size_t)b * 3 + 2]; }
+        const Box bx = translation_box(a, rvl1, rvl2, rvl3, P.cutoff_radius, P.lattice_range, P.minimum_range);
+        if (bx.over && P.status) *P.status = 1;
+        const int e0 = (int)P.e_start[i];
+        rec[REC_ATOM] = (uint32_t)i;
+        rec[REC_E0] = (uint32_t)e0;
+        rec[REC_NPAIRS] = (uint32_t)((int)P.e_start[i + 1] - e0);
+        boxw = (uint32_t)(bx.R1 | (bx.R2 << 8) | (bx.R3 << 16));
+        slow = P.slow_count != nullptr && !(bx.R1 == P.slow_R && bx.R2 == P.slow_R && bx.R3 == P.slow_R);
+        rec[REC_A] = __float_as_uint(a);
+        for (int d = 0; d < 9; d++) rec[REC_LATTICE + d] = __float_as_uint(P.tvecs[(size_t)b * 9 + d]);
+        rec[30] = (uint32_t)(P.e_start[i + 1] > e0 ? (int)P.edges[(size_t)P.E + e0] : i);      // first neighbour atom
+        rec[31] = (uint32_t)b;                                                                  // crystal
+        if (with_query) {
+            for (int c = 0; c < DH; c++) rec[REC_QUERY + c] = __float_as_uint(P.q[((size_t)i * P.H + h) * DH + c]);
+        } else if (P.frames) {
+            for (int ax = 0; ax < 3; ax++)
+                for (int d = 0; d < 3; d++)
+                    rec[REC_FRAMES + ax * 3 + d] = __float_as_uint(P.frames[(((size_t)ax * P.N + i) * P.H + h) * 3 + d]);
+        }
     }
+    // The records whose box is not the usual one take several times as long as the others in the kernels that
+    // follow, and most of them are atoms of small crystals at the END of the work order, where they alone make the
+    // tail of a launch.  The block lists up to SLOW_SLOTS of its own (rank by ballot, no atomics, nothing to clear);
+    // a launch that wants them first starts with one workgroup per slot and skips a listed record in its place.
+    if (P.slow_count) {
+        __shared__ int slow_in_wave[4];
+        const int ln = threadIdx.x & (WAVE - 1), wv = threadIdx.x >> 6;
+        const uint64_t m = __ballot(slow);
+        if (ln == 0) slow_in_wave[wv] = __popcll(m);
+        __syncthreads();
+        int rank = __popcll(m & ((1ull << ln) - 1ull)), total = 0;
+        for (int w = 0; w < 4; w++) { rank += w < wv ? slow_in_wave[w] : 0; total += slow_in_wave[w]; }
+        if (slow && rank < SLOW_SLOTS) {
+            P.slow_list[block * SLOW_SLOTS + rank] = idx;
+            boxw |= REC_BOX_LISTED;
+        }
+        if (threadIdx.x == 0) P.slow_count[block] = min(total, SLOW_SLOTS);
+    }
+    if (valid) rec[REC_BOX] = boxw;
 }
 __global__ __launch_bounds__(256) void prepare_items_kernel(const KernelArgs P, int with_query) {
     prepare_items_block(P, with_query, (int)blockIdx.x);

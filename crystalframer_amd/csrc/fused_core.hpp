@@ -80,6 +80,8 @@ struct CoreArgs {
     const float2* pair_near;      // (E) per pair over that box: smallest d^2 of all images, of the images with
                                   // d^2 > 1e-5 (what the frame search may point at); or null
     int32_t table_R;              // half-width that table was made for
+    int32_t slow_wgs;             // leading workgroups of the main kernels that take the listed slow records first
+                                  // (blocks of the record launch x SLOW_SLOTS; 0: none, records are taken in place)
     float skip_log2;              // images lighter than 2^-skip of the heaviest of their pair are not visited (<= 0: all are)
     // forward results
     float* out;                   // (N,H,16) sum_j P_ij v_j (core_project_kernel adds W . hist)
@@ -399,6 +401,21 @@ __device__ __forceinline__ void core_store_table(const CoreItem& ci, const CoreP
     }
 }
 
+// Which record a wavefront of a main kernel takes.  The first slow_wgs wavefronts are one per slot of the slow lists
+// (empty slots end at once); the others take the records in work order.  -1: nothing to do.
+__device__ __forceinline__ int core_wave_record(const CoreArgs& C, int w) {
+    if (w < C.slow_wgs) {
+        const int b = w / SLOW_SLOTS, j = w - b * SLOW_SLOTS;
+        return j < C.K.slow_count[b] ? C.K.slow_list[b * SLOW_SLOTS + j] : -1;
+    }
+    return w - C.slow_wgs;
+}
+// (a record that is listed is left to the wavefront of its slot)
+__device__ __forceinline__ bool core_record_taken_elsewhere(const CoreArgs& C, uint32_t rec) {
+    return C.slow_wgs > 0 && (int)(blockIdx.x * CORE_WPB + (threadIdx.x >> 6)) >= C.slow_wgs &&
+           ((uint32_t)__builtin_amdgcn_readlane((int)rec, REC_BOX) & REC_BOX_LISTED) != 0u;
+}
+
 // =================================================================================================================
 // forward
 // =================================================================================================================
@@ -426,7 +443,8 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
     const KernelArgs& P = C.K;
     const int lane = threadIdx.x & (WAVE - 1);
     const int H = P.H;
-    const int wid = (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6);      // this wavefront's (item, head)
+    const int wid = core_wave_record(C, (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6));      // this wavefront's (item, head)
+    if (wid < 0) return;
     const int h = wid % H;
     const int pr = lane >> 3;          // pair of the group served by this 8-lane row
     const int sub = lane & 7;          // position in the row
@@ -447,6 +465,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
     CFH_PH_DECL
     {
         const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
+        if (core_record_taken_elsewhere(C, rec_cur)) return;
         const CorePrefetch pf = core_prefetch(C, rec_cur, it_cur, h, lane);
         CFH_PH(0);
         const CoreItem ci = core_unpack(C, rec_cur, true);
