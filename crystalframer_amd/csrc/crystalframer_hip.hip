@@ -1240,7 +1240,9 @@ CoreLayout core_layout(const cfh_params* p, int64_t N, int64_t E, int64_t B, boo
         L.prep_blocks = (int)((threads + 255) / 256);
     }
     // the lists of the records that the main kernel takes first (forward: made with the records)
-    L.slow = off; if (!backward) off += align256((size_t)L.prep_blocks * (1 + cfh::SLOW_SLOTS) * sizeof(int32_t));
+    // (backward: made by the kernel that writes G, one list per 16 atoms)
+    L.slow = off;
+    off += align256((size_t)(backward ? (N + 15) / 16 + 1 : L.prep_blocks) * (1 + cfh::SLOW_SLOTS) * sizeof(int32_t));
     L.total = off;
     return L;
 }
@@ -1417,6 +1419,7 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     }
     C.out = out; C.prob = prob; C.z = z; C.hist = hist;
     C.slow_wgs = C.K.slow_count ? L.prep_blocks * cfh::SLOW_SLOTS : 0;
+    C.slow_flag = cfh::REC_BOX_LISTED;
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "fused_core_forward";
 #define CFH_CORE_DISPATCH(KERNEL)                                                                         \
@@ -1518,8 +1521,21 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
                            cfh::WcatArgs{W_dist, W_axis1, W_axis2, W_axis3, L.hw, p->dist_coef, p->angle_coef,
                                          p->angle_wscale, wcat});
     // (with records kept from the forward the work queues are all that is left to prepare: gbuild clears them)
+    // with the records kept from the forward pass, the same launch lists those that the main kernel is to take first
+    cfh::SlowListArgs SL{};
+    if (buf.records_ready && buf.table) {
+        const int nlists = (int)((N + 15) / 16);
+        SL.items = C.K.items;
+        SL.count = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(workspace) + L.slow);
+        SL.list = SL.count + nlists;
+        SL.R = C.table_R;
+        C.K.slow_count = SL.count;
+        C.K.slow_list = SL.list;
+        C.slow_wgs = nlists * cfh::SLOW_SLOTS;
+        C.slow_flag = cfh::REC_BOX_LISTED_BWD;
+    }
     hipLaunchKernelGGL(cfh::core_gbuild_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads, L.hw / 64), dim3(cfh::WAVE), 0,
-                       st, gout, wcat, G, (int)N, p->num_heads, L.hw, buf.records_ready ? C.K.counters : nullptr);
+                       st, gout, wcat, G, (int)N, p->num_heads, L.hw, buf.records_ready ? C.K.counters : nullptr, SL);
     if (!buf.records_ready) {
         const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
                                                                                           : p->num_heads * cfh::NQUEUE);

@@ -422,7 +422,8 @@ __device__ __forceinline__ int first_queue(int H) { return ((int)blockIdx.x / H)
 //   30 first neighbour atom (the pairs of an atom point at consecutive atoms), 31 crystal
 constexpr int REC_WORDS = 32;
 constexpr int SLOW_SLOTS = 64;                 // records per block of 256 that can be listed as slow
-constexpr uint32_t REC_BOX_LISTED = 0x80000000u;      // flag in the box word of a listed record
+constexpr uint32_t REC_BOX_LISTED = 0x80000000u;      // flag in the box word of a record listed by the launch that made it
+constexpr uint32_t REC_BOX_LISTED_BWD = 0x40000000u;  // ... listed again for the backward pass (see core_gbuild_kernel)
 enum { REC_ATOM = 0, REC_E0 = 1, REC_NPAIRS = 2, REC_BOX = 3, REC_A = 4, REC_LATTICE = 5, REC_FRAMES = 14,
        REC_QUERY = 14 };
 

@@ -81,7 +81,8 @@ struct CoreArgs {
                                   // d^2 > 1e-5 (what the frame search may point at); or null
     int32_t table_R;              // half-width that table was made for
     int32_t slow_wgs;             // leading workgroups of the main kernels that take the listed slow records first
-                                  // (blocks of the record launch x SLOW_SLOTS; 0: none, records are taken in place)
+                                  // (blocks of the listing launch x SLOW_SLOTS; 0: none, records are taken in place)
+    uint32_t slow_flag;           // the flag in the box word of the records listed for this launch
     float skip_log2;              // images lighter than 2^-skip of the heaviest of their pair are not visited (<= 0: all are)
     // forward results
     float* out;                   // (N,H,16) sum_j P_ij v_j (core_project_kernel adds W . hist)
@@ -413,7 +414,7 @@ __device__ __forceinline__ int core_wave_record(const CoreArgs& C, int w) {
 // (a record that is listed is left to the wavefront of its slot)
 __device__ __forceinline__ bool core_record_taken_elsewhere(const CoreArgs& C, uint32_t rec) {
     return C.slow_wgs > 0 && (int)(blockIdx.x * CORE_WPB + (threadIdx.x >> 6)) >= C.slow_wgs &&
-           ((uint32_t)__builtin_amdgcn_readlane((int)rec, REC_BOX) & REC_BOX_LISTED) != 0u;
+           ((uint32_t)__builtin_amdgcn_readlane((int)rec, REC_BOX) & C.slow_flag) != 0u;
 }
 
 // =================================================================================================================
@@ -791,13 +792,46 @@ __global__ __launch_bounds__(WAVE * PROJ_WAVES) void core_project_kernel(const f
 // G (H,N,hw) = go (N,H,16) . Wcat_h (16, hw): wavefront per (16 atoms, head, 64-word block); four MFMA tiles whose
 // columns are interleaved (tile t, column c <-> word 4 c + t) so that a lane stores 16 consecutive bytes.
 // grid (ceil(N/16), H, hw/64).  `queues`: optional work-queue heads to clear (when no prepare launch does).
+// Records kept from the forward pass (`slow.items` not null): the wavefronts (x, 0, 0) also list the records
+// [16 H x, 16 H (x + 1)) whose box is not the usual one, up to SLOW_SLOTS of them, for the main kernel of the backward
+// pass to take first (as prepare_items_block does for the forward, whose lists are gone by now).
+struct SlowListArgs {
+    uint32_t* items;       // (N, H, REC_WORDS) or null
+    int32_t* count;        // (ceil(N / 16))
+    int32_t* list;         // (ceil(N / 16), SLOW_SLOTS)
+    int32_t R;             // half-width of the usual box
+};
 __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restrict__ go, const float* __restrict__ wcat,
                                                            float* __restrict__ G, int N, int H, int hw,
-                                                           int32_t* __restrict__ queues) {
+                                                           int32_t* __restrict__ queues, const SlowListArgs slow) {
     const int lane = threadIdx.x, col = lane & 15, kk = lane >> 4;
     const int h = blockIdx.y, i0 = blockIdx.x * 16;
     if (queues && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0)      // work queues of the launch that follows
         for (int u = lane; u < H * NQUEUE; u += WAVE) queues[u * QSTRIDE] = 0;
+    if (slow.items && blockIdx.y == 0 && blockIdx.z == 0) {
+        const int first = (int)blockIdx.x * 16 * H, last = min(first + 16 * H, N * H);
+        const uint32_t usual = (uint32_t)(slow.R | (slow.R << 8) | (slow.R << 16));
+        int listed = 0;
+        for (int r0 = first; r0 < last; r0 += WAVE) {
+            const int r = r0 + lane;
+            uint32_t boxw = 0;
+            bool own = false;
+            if (r < last) {
+                boxw = slow.items[(size_t)r * REC_WORDS + REC_BOX];
+                own = (boxw & 0x00ffffffu) != usual;
+            }
+            const uint64_t m = __ballot(own);
+            const int rank = listed + __popcll(m & ((1ull << lane) - 1ull));
+            if (r < last) {
+                const bool take = own && rank < SLOW_SLOTS;
+                if (take) slow.list[(size_t)blockIdx.x * SLOW_SLOTS + rank] = r;
+                const uint32_t neww = take ? (boxw | REC_BOX_LISTED_BWD) : (boxw & ~REC_BOX_LISTED_BWD);
+                if (neww != boxw) slow.items[(size_t)r * REC_WORDS + REC_BOX] = neww;
+            }
+            listed += __popcll(m);
+        }
+        if (lane == 0) slow.count[blockIdx.x] = min(listed, SLOW_SLOTS);
+    }
     const int row = min(i0 + col, N - 1);
     const float4 a4 = reinterpret_cast<const float4*>(go + ((size_t)row * H + h) * DH)[kk];      // channels 4 kk ..
     const float A[4] = {a4.x, a4.y, a4.z, a4.w};
@@ -935,7 +969,8 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
     const KernelArgs& P = C.K;
     const int lane = threadIdx.x & (WAVE - 1);
     const int H = P.H;
-    const int wid = (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6);
+    const int wid = core_wave_record(C, (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6));
+    if (wid < 0) return;
     const int h = wid % H;
     const int pr = lane >> 3, sub = lane & 7;
     const BasisConsts bc = P.bc;
@@ -946,6 +981,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
     if (it_cur >= P.N) return;
     {
         const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
+        if (core_record_taken_elsewhere(C, rec_cur)) return;
         const CoreItem ci = core_unpack(C, rec_cur, true);
         const int i = ci.item.i;
         const float a2 = ci.item.a * LOG2E;
