@@ -1524,7 +1524,7 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
     // with the records kept from the forward pass, the same launch lists those that the main kernel is to take first
     cfh::SlowListArgs SL{};
     if (buf.records_ready && buf.table) {
-        const int nlists = (int)((N + 15) / 16);
+        const int nlists = (int)(((N + 15) / 16 + cfh::SLOW_GB_BLOCKS - 1) / cfh::SLOW_GB_BLOCKS);
         SL.items = C.K.items;
         SL.count = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(workspace) + L.slow);
         SL.list = SL.count + nlists;

@@ -792,13 +792,15 @@ __global__ __launch_bounds__(WAVE * PROJ_WAVES) void core_project_kernel(const f
 // G (H,N,hw) = go (N,H,16) . Wcat_h (16, hw): wavefront per (16 atoms, head, 64-word block); four MFMA tiles whose
 // columns are interleaved (tile t, column c <-> word 4 c + t) so that a lane stores 16 consecutive bytes.
 // grid (ceil(N/16), H, hw/64).  `queues`: optional work-queue heads to clear (when no prepare launch does).
-// Records kept from the forward pass (`slow.items` not null): the wavefronts (x, 0, 0) also list the records
-// [16 H x, 16 H (x + 1)) whose box is not the usual one, up to SLOW_SLOTS of them, for the main kernel of the backward
-// pass to take first (as prepare_items_block does for the forward, whose lists are gone by now).
+// Records kept from the forward pass (`slow.items` not null): the wavefronts (x, 0, 0) with x a multiple of
+// SLOW_GB_BLOCKS also list the records of SLOW_GB_BLOCKS x 16 atoms whose box is not the usual one, up to SLOW_SLOTS
+// of them, for the main kernel of the backward pass to take first (as prepare_items_block does for the forward,
+// whose lists are gone by now).
+constexpr int SLOW_GB_BLOCKS = 4;
 struct SlowListArgs {
     uint32_t* items;       // (N, H, REC_WORDS) or null
-    int32_t* count;        // (ceil(N / 16))
-    int32_t* list;         // (ceil(N / 16), SLOW_SLOTS)
+    int32_t* count;        // (lists), lists = ceil(ceil(N / 16) / SLOW_GB_BLOCKS)
+    int32_t* list;         // (lists, SLOW_SLOTS)
     int32_t R;             // half-width of the usual box
 };
 __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restrict__ go, const float* __restrict__ wcat,
@@ -808,8 +810,9 @@ __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restri
     const int h = blockIdx.y, i0 = blockIdx.x * 16;
     if (queues && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0)      // work queues of the launch that follows
         for (int u = lane; u < H * NQUEUE; u += WAVE) queues[u * QSTRIDE] = 0;
-    if (slow.items && blockIdx.y == 0 && blockIdx.z == 0) {
-        const int first = (int)blockIdx.x * 16 * H, last = min(first + 16 * H, N * H);
+    if (slow.items && blockIdx.y == 0 && blockIdx.z == 0 && blockIdx.x % SLOW_GB_BLOCKS == 0) {
+        const int li = (int)blockIdx.x / SLOW_GB_BLOCKS;
+        const int first = (int)blockIdx.x * 16 * H, last = min(first + SLOW_GB_BLOCKS * 16 * H, N * H);
         const uint32_t usual = (uint32_t)(slow.R | (slow.R << 8) | (slow.R << 16));
         int listed = 0;
         for (int r0 = first; r0 < last; r0 += WAVE) {
@@ -824,13 +827,13 @@ __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restri
             const int rank = listed + __popcll(m & ((1ull << lane) - 1ull));
             if (r < last) {
                 const bool take = own && rank < SLOW_SLOTS;
-                if (take) slow.list[(size_t)blockIdx.x * SLOW_SLOTS + rank] = r;
+                if (take) slow.list[(size_t)li * SLOW_SLOTS + rank] = r;
                 const uint32_t neww = take ? (boxw | REC_BOX_LISTED_BWD) : (boxw & ~REC_BOX_LISTED_BWD);
                 if (neww != boxw) slow.items[(size_t)r * REC_WORDS + REC_BOX] = neww;
             }
             listed += __popcll(m);
         }
-        if (lane == 0) slow.count[blockIdx.x] = min(listed, SLOW_SLOTS);
+        if (lane == 0) slow.count[li] = min(listed, SLOW_SLOTS);
     }
     const int row = min(i0 + col, N - 1);
     const float4 a4 = reinterpret_cast<const float4*>(go + ((size_t)row * H + h) * DH)[kk];      // channels 4 kk ..
