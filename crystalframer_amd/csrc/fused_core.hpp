@@ -33,6 +33,7 @@
 // at 64 + (ax NORD + o) 64.  It is accumulated in LDS as signed 32-bit fixed point (round to nearest) in units of
 // 2^30 / npairs relative to the heaviest pair of the row so far, and written out normalised as float32.
 #pragma once
+#include <type_traits>
 #include "device_common.hpp"
 
 namespace cfh {
@@ -41,6 +42,8 @@ constexpr int FC_TCAP = 128;                    // translations per table chunk 
 constexpr int FC_GROUP = 8;                     // pairs per group: one per 8-lane row
 constexpr int FC_LISTCAP = FC_GROUP * FC_TCAP;  // a group's survivors always fit: no overflow handling
 constexpr int FC_SHIFT = 7;                     // list entry = pair-in-group << 7 | table index
+constexpr int FC_BIGSHIFT = 13;                 // ... of an item of several chunks: pair-in-group << 13 | index in its box
+constexpr int FC_BIGT = 1 << FC_BIGSHIFT;       // (boxes of up to 8192 translations)
 #ifndef CFH_NORD
 #define CFH_NORD 5
 #endif
@@ -500,7 +503,15 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
         // operands of the pair served by this row, fetched one group ahead (the first group: with the item)
         float nrx = pf.rx, nry = pf.ry, nrz = pf.rz, nnear = pf.near;
         float2 nk2 = pf.k2, nv2 = pf.v2;
-        const bool near_known = sorted && C.pair_near != nullptr;      // the nearest image of every pair comes with the batch
+        // The nearest image of every pair over the usual box comes with the batch.  An item whose box CONTAINS the usual
+        // one takes it as the reference of its weights as well (any reference gives the same normalised weights and
+        // the same z; only the pruning threshold moves with it, should an image outside the usual box be nearer)
+        const bool contains_usual = C.sorted_tab != nullptr && bx.R1 >= C.table_R && bx.R2 >= C.table_R && bx.R3 >= C.table_R;
+        const bool near_known = (sorted || contains_usual) && C.pair_near != nullptr;
+        // several chunks: the survivors of all chunks go into one list with their index in the whole box, and the
+        // heavy pass makes their shifts from that index instead of reading a table: one sweep, each chunk built once
+        const bool one_list = nchunks > 1 && bx.T <= FC_BIGT;
+        const float inv_s3 = 1.0f / (float)bx.s3, inv_s2 = 1.0f / (float)bx.s2;
         auto fetch = [&](int g0) {
             const int el = g0 + pr;
             if (el < npairs) {
@@ -531,20 +542,34 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
                     const uint64_t inm = __ballot(in);
                     if (sorted && inm == 0) break;               // every row is past its reach (lengths ascend)
                     const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
-                    fn(in, t, fmaf(dx, dx, fmaf(dy, dy, dz * dz)), __popcll(inm));
+                    fn(in, t0c + t, fmaf(dx, dx, fmaf(dy, dy, dz * dz)), __popcll(inm));
                     v = vn;
                 }
             }
         };
 
         // scatter of the current list (entries point into the resident table)
-        auto heavy = [&](int nlist) {
+        auto heavy_impl = [&](int nlist, auto big) {
+            constexpr bool BIG = decltype(big)::value;      // entries (pair << FC_BIGSHIFT | index in the box), no table
             for (int base = 0; base < nlist; base += WAVE) {
                 const int idx = base + lane;
                 if (idx < nlist) {
                     const uint32_t ent = list[idx];
-                    const int pp = ent >> FC_SHIFT;
-                    const float4 v = tab[ent & (FC_TCAP - 1)];
+                    const int pp = BIG ? (int)(ent >> FC_BIGSHIFT) : (int)(ent >> FC_SHIFT);
+                    float4 v;
+                    if (BIG) {
+                        const int tg = (int)(ent & (FC_BIGT - 1));
+                        // (exact: the quotients stay below 2^13 and the fractions at least 1 / (2 s) from an integer)
+                        const int q = (int)(((float)tg + 0.5f) * inv_s3), i3 = tg - q * bx.s3;
+                        const int i1 = (int)(((float)q + 0.5f) * inv_s2), i2 = q - i1 * bx.s2;
+                        const float n1 = (float)(i1 - bx.R1), n2 = (float)(i2 - bx.R2), n3 = (float)(i3 - bx.R3);
+                        v.x = fmaf(L.t[6], n3, fmaf(L.t[3], n2, L.t[0] * n1));      // as build_shift_table makes them
+                        v.y = fmaf(L.t[7], n3, fmaf(L.t[4], n2, L.t[1] * n1));
+                        v.z = fmaf(L.t[8], n3, fmaf(L.t[5], n2, L.t[2] * n1));
+                        v.w = 0.0f;
+                    } else {
+                        v = tab[ent & (FC_TCAP - 1)];
+                    }
                     const float4 pa = pairA[pp];
                     const float dx = pa.x + v.x, dy = pa.y + v.y, dz = pa.z + v.z;
                     const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
@@ -588,6 +613,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             }
             n_eval += (unsigned long long)nlist;
         };
+        auto heavy = [&](int nlist) { heavy_impl(nlist, std::false_type{}); };
 
         for (int g0 = 0; g0 < npairs; g0 += FC_GROUP) {
             const float rx = nrx, ry = nry, rz = nrz;
@@ -597,9 +623,14 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             const bool active = g0 + pr < npairs;
             const float rn = hw_sqrt(fmaf(rx, rx, fmaf(ry, ry, rz * rz)));
 
+            float Sb, S;
+            int nlist;
+            bool spilled;                     // (several chunks) more survivors than the list holds: the chunks again, one by one
+            bool known = near_known;
+            for (;;) {
             // ---- pass A: nearest image (known beforehand for the usual box)
             CFH_PH(1);
-            if (!near_known) {
+            if (!known) {
                 d2min = 3.0e38f;
                 sweep(active, rx, ry, rz, sorted ? fmaf(2.0002f, rn, 1e-4f) : INF,
                       [&](bool in, int, float d2, int cnt_in) { d2min = in ? fminf(d2min, d2) : d2min; n_seen += cnt_in; });
@@ -609,20 +640,42 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             // ---- pass B: weights, normaliser and (one-chunk tables) the survivors
             CFH_PH(2);
             const float reachB = sorted ? fmaf(1.0001f, rn + hw_sqrt(d2min + cutS), 1e-4f) : INF;
-            float Sb = 0.0f;
-            int nlist = 0;
-            sweep(active, rx, ry, rz, reachB, [&](bool in, int t, float d2, int cnt_in) {
-                const float ex = a2 * (d2 - d2min);
-                Sb += in ? hw_exp2(ex) : 0.0f;
-                n_seen += cnt_in;
-                if (nchunks == 1) {
+            Sb = 0.0f;
+            nlist = 0;
+            spilled = false;
+            if (nchunks == 1) {
+                sweep(active, rx, ry, rz, reachB, [&](bool in, int t, float d2, int cnt_in) {
+                    const float ex = a2 * (d2 - d2min);
+                    Sb += in ? hw_exp2(ex) : 0.0f;
+                    n_seen += cnt_in;
                     const bool keep = in && ex >= prune;
                     const uint64_t m = __ballot(keep);
                     if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
                     nlist += __popcll(m);
-                }
-            });
-            const float S = half_sum(Sb);
+                });
+            } else {
+                sweep(active, rx, ry, rz, reachB, [&](bool in, int t, float d2, int cnt_in) {
+                    const float ex = a2 * (d2 - d2min);
+                    Sb += in ? hw_exp2(ex) : 0.0f;
+                    n_seen += cnt_in;
+                    if (one_list && !spilled) {
+                        const bool keep = in && ex >= prune;
+                        const uint64_t m = __ballot(keep);
+                        if (nlist + __popcll(m) > FC_LISTCAP) spilled = true;
+                        else {
+                            if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_BIGSHIFT) | t);
+                            nlist += __popcll(m);
+                        }
+                    }
+                });
+            }
+            S = half_sum(Sb);
+            // a reference borrowed from the usual box may lie far above the nearest image of a larger box (a strongly
+            // sheared cell): a sum of weights of 2^24 and more says so (with the nearest image as the reference it is at
+            // most the number of translations, 2^13), and the group is done again with a sweep for the nearest
+            if (known && !sorted && __ballot(active && !(S < 0x1p24f)) != 0) { known = false; continue; }
+            break;
+            }
 
             // ---- logits, running softmax
             CFH_PH(3);
@@ -669,6 +722,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             // ---- heavy pass
             CFH_PH(4);
             if (nchunks == 1) heavy(nlist);
+            else if (one_list && !spilled) heavy_impl(nlist, std::true_type{});
             else {
                 for (int ch = 0; ch < nchunks; ch++) {
                     const int t0c = ch * FC_TCAP;
@@ -1045,13 +1099,30 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
         };
         fetch(0);
 
-        auto heavy = [&](int nlist) {
+        // several chunks: the survivors of all chunks in one list with their index in the whole box (as in the forward)
+        const bool one_list = nchunks > 1 && bx.T <= FC_BIGT;
+        const float inv_s3 = 1.0f / (float)bx.s3, inv_s2 = 1.0f / (float)bx.s2;
+        auto heavy_impl = [&](int nlist, auto big) {
+            constexpr bool BIG = decltype(big)::value;      // entries (pair << FC_BIGSHIFT | index in the box), no table
             for (int base = 0; base < nlist; base += WAVE) {
                 const int idx = base + lane;
                 if (idx < nlist) {
                     const uint32_t ent = list[idx];
-                    const int pp = ent >> FC_SHIFT;
-                    const float4 v = tab[ent & (FC_TCAP - 1)];
+                    const int pp = BIG ? (int)(ent >> FC_BIGSHIFT) : (int)(ent >> FC_SHIFT);
+                    float4 v;
+                    if (BIG) {
+                        const int tg = (int)(ent & (FC_BIGT - 1));
+                        // (exact: the quotients stay below 2^13 and the fractions at least 1 / (2 s) from an integer)
+                        const int q = (int)(((float)tg + 0.5f) * inv_s3), i3 = tg - q * bx.s3;
+                        const int i1 = (int)(((float)q + 0.5f) * inv_s2), i2 = q - i1 * bx.s2;
+                        const float n1 = (float)(i1 - bx.R1), n2 = (float)(i2 - bx.R2), n3 = (float)(i3 - bx.R3);
+                        v.x = fmaf(L.t[6], n3, fmaf(L.t[3], n2, L.t[0] * n1));      // as build_shift_table makes them
+                        v.y = fmaf(L.t[7], n3, fmaf(L.t[4], n2, L.t[1] * n1));
+                        v.z = fmaf(L.t[8], n3, fmaf(L.t[5], n2, L.t[2] * n1));
+                        v.w = 0.0f;
+                    } else {
+                        v = tab[ent & (FC_TCAP - 1)];
+                    }
                     const float4 pa = pairA[pp];
                     const float dx = pa.x + v.x, dy = pa.y + v.y, dz = pa.z + v.z;
                     const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
@@ -1091,6 +1162,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
             }
             n_eval += (unsigned long long)nlist;
         };
+        auto heavy = [&](int nlist) { heavy_impl(nlist, std::false_type{}); };
 
         for (int g0 = 0; g0 < npairs; g0 += FC_GROUP) {
             const float rx = nrx, ry = nry, rz = nrz;
@@ -1109,14 +1181,9 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
             }
             float Ap = 0.0f;
             int nlist = 0;
-            for (int ch = 0; ch < nchunks; ch++) {
-                const int t0c = ch * FC_TCAP;
-                const int cnt = sorted ? bx.T : min(FC_TCAP, bx.T - t0c);
-                if (nchunks > 1) {
-                    wave_sync();
-                    build_shift_table(tab, t0c, cnt, bx, L, lane);
-                    wave_sync();
-                }
+            bool spilled = false;             // (several chunks) more survivors than the list holds: the chunks again, one by one
+            if (nchunks == 1) {
+                const int cnt = bx.T;
                 for (int t0 = 0; t0 < cnt; t0 += FC_GROUP) {
                     const int t = t0 + sub;
                     const float4 v = tab[min(t, cnt - 1)];
@@ -1126,17 +1193,42 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
                     const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
                     const float ex = fmaf(a2, d2, -z2);
                     Ap += in ? hw_exp2(ex) * d2 : 0.0f;
-                    if (nchunks == 1) {
-                        const bool keep = in && ex >= prune;
-                        const uint64_t m = __ballot(keep);
-                        if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
-                        nlist += __popcll(m);
+                    const bool keep = in && ex >= prune;
+                    const uint64_t m = __ballot(keep);
+                    if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
+                    nlist += __popcll(m);
+                }
+            } else {
+                for (int ch = 0; ch < nchunks; ch++) {
+                    const int t0c = ch * FC_TCAP;
+                    const int cnt = min(FC_TCAP, bx.T - t0c);
+                    wave_sync();
+                    build_shift_table(tab, t0c, cnt, bx, L, lane);
+                    wave_sync();
+                    for (int t0 = 0; t0 < cnt; t0 += FC_GROUP) {
+                        const int t = t0 + sub;
+                        const float4 v = tab[min(t, cnt - 1)];
+                        const bool in = active && t < cnt;
+                        const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
+                        const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+                        const float ex = fmaf(a2, d2, -z2);
+                        Ap += in ? hw_exp2(ex) * d2 : 0.0f;
+                        if (one_list && !spilled) {
+                            const bool keep = in && ex >= prune;
+                            const uint64_t m = __ballot(keep);
+                            if (nlist + __popcll(m) > FC_LISTCAP) spilled = true;
+                            else {
+                                if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_BIGSHIFT) | (t0c + t));
+                                nlist += __popcll(m);
+                            }
+                        }
                     }
                 }
             }
             const float A0 = half_sum(Ap);
             wave_sync();
             if (nchunks == 1) heavy(nlist);
+            else if (one_list && !spilled) heavy_impl(nlist, std::true_type{});
             else {
                 for (int ch = 0; ch < nchunks; ch++) {
                     const int t0c = ch * FC_TCAP;

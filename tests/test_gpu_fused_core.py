@@ -139,6 +139,25 @@ def test_fused_core_small_cells_with_boxes_of_several_chunks():
     compare(P, _gout(P), out, leaves, oo, oleaves)
 
 
+@pytest.mark.parametrize("shear", [1, 4])
+def test_fused_core_sheared_cells(shear):
+    """The same lattices described by sheared cells (second cell vector + shear x the first): boxes that contain
+    the usual one, whose nearest image of a pair may lie outside the usual box (mildly for shear 1, far outside
+    for shear 4)."""
+    P = Hh.make_problem(num_crystals=5, atoms_lo=2, atoms_hi=5, len_lo=2.5, len_hi=4.0, seed=223 + shear)
+    P.tvecs = P.tvecs.clone()
+    P.tvecs[:, 1] += shear * P.tvecs[:, 0]
+    P.tvecs = P.tvecs.float().double()
+    P.edges, P.rpos, recip, P.vcell = TO.geometry(P.pos, P.tvecs, P.sizes)
+    P.rpos = P.rpos.float().double()
+    P.rvlen = torch.norm(recip, 2, dim=-1).float().double()
+    R = TO.translation_ranges(P.a, P.rvlen, P.batch, CUT)
+    assert int(R.max()) > 2 and int((2 * R + 1).prod(-1).max()) <= 8192
+    out, _, leaves = run_core(P)
+    oo, oleaves = oracle_core(P)
+    compare(P, _gout(P), out, leaves, oo, oleaves)
+
+
 def test_fused_core_mixed_boxes_and_long_rows():
     """Crystals of up to 40 atoms (rows of several groups, the running softmax rescales) with cell sizes that
     mix the usual box with larger ones."""
