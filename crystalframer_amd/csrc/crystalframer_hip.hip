@@ -1241,8 +1241,11 @@ CoreLayout core_layout(const cfh_params* p, int64_t N, int64_t E, int64_t B, boo
     }
     // the lists of the records that the main kernel takes first (forward: made with the records)
     // (backward: made by the kernel that writes G, one list per 16 atoms)
+    // (a count per list and a slot per record: forward a list per block of records, backward per SLOW_GB_BLOCKS x 16 atoms)
     L.slow = off;
-    off += align256((size_t)(backward ? (N + 15) / 16 + 1 : L.prep_blocks) * (1 + cfh::SLOW_SLOTS) * sizeof(int32_t));
+    off += align256(((size_t)(backward ? (N + 15) / 16 + 1 : L.prep_blocks) +
+                     (size_t)(backward ? ((N + 15) / 16 + cfh::SLOW_GB_BLOCKS) * 16 * p->num_heads
+                                       : (int64_t)L.prep_blocks * cfh::SLOW_PREP_SLOTS)) * sizeof(int32_t));
     L.total = off;
     return L;
 }
@@ -1292,6 +1295,12 @@ CoreBuffers fill_core(cfh::CoreArgs& C, const cfh_params* p, const CoreLayout& L
     C.table_R = tables ? R0 : 0;
     C.skip_log2 = p->prune_log2 > 0.0f ? (p->prune_log2 + 8.0f > 32.0f ? p->prune_log2 + 8.0f : 32.0f) : 0.0f;
     return b;
+}
+// Leading wavefronts of a main kernel, one per listed slow record (the host does not know how many are listed): a
+// sixteenth of the records, at least 256.  Listed records beyond that are taken in place like the unlisted.
+int slow_wave_count(int64_t N, int H) {
+    const int64_t w = (N * H / 16 + 7) / 8 * 8;
+    return (int)(w < 256 ? 256 : w);
 }
 // one wavefront (= workgroup) per (item, head); the hardware deals them to the compute units as slots free up
 template <typename Kern>
@@ -1402,8 +1411,14 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
                     timed = hipEventCreate(&t.start) == hipSuccess && hipEventCreate(&t.stop) == hipSuccess &&
                             hipEventRecord(t.start, st) == hipSuccess;
                 }
-                hipLaunchKernelGGL(cfh::frame_axes_kernel, dim3(item_blocks + quad_blocks), dim3(cfh::WAVE * cfh::CORE_WPB), 0,
-                                   st, F, (int)item_blocks);
+                if (F.K.slow_count) {
+                    F.slow_lists = prep_blocks;
+                    F.slow_stride = cfh::SLOW_PREP_SLOTS;
+                    F.slow_wgs = slow_wave_count(N, p->num_heads);
+                }
+                const unsigned slow_blocks = ((unsigned)F.slow_wgs + cfh::CORE_WPB - 1) / cfh::CORE_WPB;
+                hipLaunchKernelGGL(cfh::frame_axes_kernel, dim3(slow_blocks + quad_blocks + item_blocks),
+                                   dim3(cfh::WAVE * cfh::CORE_WPB), 0, st, F, (int)slow_blocks, (int)quad_blocks);
                 if (timed && hipEventRecord(t.stop, st) == hipSuccess) {
                     std::lock_guard<std::mutex> lock(g_timing_mutex);
                     g_timed.push_back(t);
@@ -1418,7 +1433,11 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
         }
     }
     C.out = out; C.prob = prob; C.z = z; C.hist = hist;
-    C.slow_wgs = C.K.slow_count ? L.prep_blocks * cfh::SLOW_SLOTS : 0;
+    if (C.K.slow_count) {
+        C.slow_lists = L.prep_blocks;
+        C.slow_stride = cfh::SLOW_PREP_SLOTS;
+        C.slow_wgs = slow_wave_count(N, p->num_heads);
+    }
     C.slow_flag = cfh::REC_BOX_LISTED;
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
     const char* what = "fused_core_forward";
@@ -1531,7 +1550,9 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         SL.R = C.table_R;
         C.K.slow_count = SL.count;
         C.K.slow_list = SL.list;
-        C.slow_wgs = nlists * cfh::SLOW_SLOTS;
+        C.slow_lists = nlists;
+        C.slow_stride = cfh::SLOW_GB_BLOCKS * 16 * p->num_heads;
+        C.slow_wgs = slow_wave_count(N, p->num_heads);
         C.slow_flag = cfh::REC_BOX_LISTED_BWD;
     }
     hipLaunchKernelGGL(cfh::core_gbuild_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads, L.hw / 64), dim3(cfh::WAVE), 0,

@@ -176,6 +176,18 @@ __device__ __forceinline__ Box translation_box(float a, float rvl1, float rvl2, 
 }
 #pragma clang fp contract(fast)
 
+// inclusive prefix sum over the 64 lanes (row scans in DPP, row totals by lane reads)
+__device__ __forceinline__ int wave_scan_incl(int x) {
+    x += dpp_movei<0x111>(x);
+    x += dpp_movei<0x112>(x);
+    x += dpp_movei<0x114>(x);
+    x += dpp_movei<0x118>(x);
+    const int t0 = __builtin_amdgcn_readlane(x, 15), t1 = __builtin_amdgcn_readlane(x, 31);
+    const int t2 = __builtin_amdgcn_readlane(x, 47);
+    const int row = ((int)threadIdx.x & 63) >> 4;
+    return x + (row == 0 ? 0 : row == 1 ? t0 : row == 2 ? t0 + t1 : t0 + t1 + t2);
+}
+
 struct Lattice { float t[9]; };   // rows = lattice vectors
 
 // Fill tab[0..cnt) with the Cartesian shifts of translations t0..t0+cnt in the reference's loop
@@ -347,8 +359,8 @@ struct KernelArgs {
     int32_t frames_to_records;    // frame search: also store the orthonormal frames into the item records
     uint32_t* items;              // (N, H, REC_WORDS) item records of this launch
     int32_t* slow_count;          // optional: per block of 256 records, how many of them are listed in slow_list
-    int32_t* slow_list;           // (blocks, SLOW_SLOTS) records whose box is not the usual one, for the launches that
-                                  // take those items first (see prepare_items_block)
+    int32_t* slow_list;           // (blocks, SLOW_PREP_SLOTS) records whose box is not the usual one, for the launches that
+                                  // follow to take first
     int32_t slow_R;               // half-width of the usual box
     unsigned long long* stats;    // optional running totals (see STAT_* below); never reset by a launch
     int32_t* status;              // word of the workspace header: set to 1 when a box was cut back to RMAX (never cleared)
@@ -421,7 +433,7 @@ __device__ __forceinline__ int first_queue(int H) { return ((int)blockIdx.x / H)
 //   5..13 lattice rows, 14..22 frame axes (frame search: 14..29 the query vector q_ih),
 //   30 first neighbour atom (the pairs of an atom point at consecutive atoms), 31 crystal
 constexpr int REC_WORDS = 32;
-constexpr int SLOW_SLOTS = 64;                 // records per block of 256 that can be listed as slow
+constexpr int SLOW_PREP_SLOTS = 256;           // slots of a list of slow records: every record of the block that makes it
 constexpr uint32_t REC_BOX_LISTED = 0x80000000u;      // flag in the box word of a record listed by the launch that made it
 constexpr uint32_t REC_BOX_LISTED_BWD = 0x40000000u;  // ... listed again for the backward pass (see core_gbuild_kernel)
 enum { REC_ATOM = 0, REC_E0 = 1, REC_NPAIRS = 2, REC_BOX = 3, REC_A = 4, REC_LATTICE = 5, REC_FRAMES = 14,
@@ -510,8 +522,9 @@ __device__ __forceinline__ void prepare_items_block(const KernelArgs& P, int wit
     }
     // The records whose box is not the usual one take several times as long as the others in the kernels that
     // follow, and most of them are atoms of small crystals at the END of the work order, where they alone make the
-    // tail of a launch.  The block lists up to SLOW_SLOTS of its own (rank by ballot, no atomics, nothing to clear);
-    // a launch that wants them first starts with one workgroup per slot and skips a listed record in its place.
+    // tail of a launch.  The block lists its own (rank by ballot, no atomics, nothing to clear); a launch that wants
+    // them first starts with a few wavefronts that take the listed records by their rank over all lists, and skips a
+    // listed record in its place.
     if (P.slow_count) {
         __shared__ int slow_in_wave[4];
         const int ln = threadIdx.x & (WAVE - 1), wv = threadIdx.x >> 6;
@@ -520,11 +533,11 @@ __device__ __forceinline__ void prepare_items_block(const KernelArgs& P, int wit
         __syncthreads();
         int rank = __popcll(m & ((1ull << ln) - 1ull)), total = 0;
         for (int w = 0; w < 4; w++) { rank += w < wv ? slow_in_wave[w] : 0; total += slow_in_wave[w]; }
-        if (slow && rank < SLOW_SLOTS) {
-            P.slow_list[block * SLOW_SLOTS + rank] = idx;
+        if (slow) {
+            P.slow_list[block * SLOW_PREP_SLOTS + rank] = idx;
             boxw |= REC_BOX_LISTED;
         }
-        if (threadIdx.x == 0) P.slow_count[block] = min(total, SLOW_SLOTS);
+        if (threadIdx.x == 0) P.slow_count[block] = total;
     }
     if (valid) rec[REC_BOX] = boxw;
 }

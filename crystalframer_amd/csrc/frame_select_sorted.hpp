@@ -69,18 +69,6 @@ __device__ __forceinline__ void build_sorted_chunk(float4* tab, int t0, int cnt,
     for (int u = cnt + lane; u < FC_TCAP; u += WAVE) tab[u] = make_float4(0.f, 0.f, 0.f, __builtin_inff());
 }
 
-// inclusive prefix sum over the 64 lanes (row scans in DPP, row totals by lane reads)
-__device__ __forceinline__ int wave_scan_incl(int x) {
-    x += dpp_movei<0x111>(x);
-    x += dpp_movei<0x112>(x);
-    x += dpp_movei<0x114>(x);
-    x += dpp_movei<0x118>(x);
-    const int t0 = __builtin_amdgcn_readlane(x, 15), t1 = __builtin_amdgcn_readlane(x, 31);
-    const int t2 = __builtin_amdgcn_readlane(x, 47);
-    const int row = ((int)threadIdx.x & 63) >> 4;
-    return x + (row == 0 ? 0 : row == 1 ? t0 : row == 2 ? t0 + t1 : t0 + t1 + t2);
-}
-
 struct FrameShared {
     float4 tab[2 * FC_TCAP];     // the sorted table, or the sorted chunks of a box of its own (two stay resident)
     float4 pq[WAVE];             // rpos and q.k of the staged pairs
@@ -90,7 +78,9 @@ struct FrameShared {
 };
 // one wavefront, one item: wid = item * H + head.  `others_only`: only the items that the four-heads-per-wavefront
 // search leaves out (box not the table's, or more pairs than it takes).
-__device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& sh, int wid, int lane, bool others_only) {
+// `skip_listed`: the records listed for the first wavefronts of the launch are theirs.
+__device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& sh, int wid, int lane, bool others_only,
+                                                bool skip_listed) {
     float4* const tab = sh.tab;
     float4* const pq = sh.pq;
     uint32_t* const markw = sh.markw;
@@ -111,6 +101,9 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
     if (it_cur >= P.N) return;
     {
         const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
+        if (skip_listed && ((uint32_t)__builtin_amdgcn_readlane((int)rec_cur, REC_BOX) & REC_BOX_LISTED) != 0u &&
+            core_slow_rank(C, wid, lane) < C.slow_wgs)
+            return;      // (a listed record of higher rank stays here)
         const Item item = unpack_item(rec_cur);
         const int crystal = __builtin_amdgcn_readlane((int)rec_cur, REC_CRYSTAL);
         const int j0 = __builtin_amdgcn_readlane((int)rec_cur, REC_J0);
@@ -569,17 +562,30 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
 __global__ __launch_bounds__(WAVE * CORE_WPB) void frame_axes_sorted_kernel(const CoreArgs C) {
     __shared__ FrameShared shared[CORE_WPB];
     frame_item_body(C, shared[threadIdx.x >> 6], (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6),
-                    (int)threadIdx.x & (WAVE - 1), false);
+                    (int)threadIdx.x & (WAVE - 1), false, false);
 }
 
-// Both ways in one launch.  The first `item_blocks` workgroups go over all items one per wavefront and take those that
-// the four-heads search leaves out (the rest return at once); they come first so that these few, slower items start
-// early and run beside the others.  The remaining workgroups search four heads of an atom per wavefront.
-__global__ __launch_bounds__(WAVE * CORE_WPB) void frame_axes_kernel(const CoreArgs C, int item_blocks) {
+// Both ways in one launch, the slowest work first.  Wavefronts in the order of the grid:
+//   1. one per listed record with a box of their own, by rank over the lists (made by the launch that wrote the
+//      records; no record of that rank: the wavefront ends): several sorted chunks, the longest of the launch;
+//   2. the four-heads search over all atoms;
+//   3. one per item, for the items that neither of the two takes (usual box, longer rows: they are at the start of the
+//      work order, so the wavefronts that find nothing to do come last and only pass through).
+// With the items of (3) and their many passing wavefronts in front, the four-heads search started after a third of
+// the launch's time, and the records with a box of their own, scattered over the work order, later still.
+__global__ __launch_bounds__(WAVE * CORE_WPB) void frame_axes_kernel(const CoreArgs C, int slow_blocks, int quad_blocks) {
     __shared__ union { FrameShared item; FrameQuadShared quad; } shared[CORE_WPB];
     const int wv = (int)(threadIdx.x >> 6), lane = (int)threadIdx.x & (WAVE - 1);
-    if ((int)blockIdx.x < item_blocks) frame_item_body(C, shared[wv].item, (int)blockIdx.x * CORE_WPB + wv, lane, true);
-    else frame_quad_body(C, shared[wv].quad, ((int)blockIdx.x - item_blocks) * CORE_WPB + wv, lane);
+    const int blk = (int)blockIdx.x;
+    if (blk < slow_blocks) {
+        const int wid = core_slow_record(C, blk * CORE_WPB + wv, lane);
+        if (wid < 0) return;
+        frame_item_body(C, shared[wv].item, wid, lane, false, false);
+    } else if (blk < slow_blocks + quad_blocks) {
+        frame_quad_body(C, shared[wv].quad, (blk - slow_blocks) * CORE_WPB + wv, lane);
+    } else {
+        frame_item_body(C, shared[wv].item, (blk - slow_blocks - quad_blocks) * CORE_WPB + wv, lane, true, slow_blocks > 0);
+    }
 }
 
 }  // namespace cfh

@@ -83,8 +83,11 @@ struct CoreArgs {
     const float2* pair_near;      // (E) per pair over that box: smallest d^2 of all images, of the images with
                                   // d^2 > 1e-5 (what the frame search may point at); or null
     int32_t table_R;              // half-width that table was made for
-    int32_t slow_wgs;             // leading workgroups of the main kernels that take the listed slow records first
-                                  // (blocks of the listing launch x SLOW_SLOTS; 0: none, records are taken in place)
+    int32_t slow_wgs;             // leading wavefronts of the main kernels that take the listed slow records first, by
+                                  // rank over all lists: wavefront w the rank w; the listed records of higher rank are
+                                  // taken in place, like the others (0: no lists)
+    int32_t slow_lists;           // lists (K.slow_count, K.slow_list)
+    int32_t slow_stride;          // slots per list
     uint32_t slow_flag;           // the flag in the box word of the records listed for this launch
     float skip_log2;              // images lighter than 2^-skip of the heaviest of their pair are not visited (<= 0: all are)
     // forward results
@@ -405,19 +408,46 @@ __device__ __forceinline__ void core_store_table(const CoreItem& ci, const CoreP
     }
 }
 
-// Which record a wavefront of a main kernel takes.  The first slow_wgs wavefronts are one per slot of the slow lists
-// (empty slots end at once); the others take the records in work order.  -1: nothing to do.
-__device__ __forceinline__ int core_wave_record(const CoreArgs& C, int w) {
-    if (w < C.slow_wgs) {
-        const int b = w / SLOW_SLOTS, j = w - b * SLOW_SLOTS;
-        return j < C.K.slow_count[b] ? C.K.slow_list[b * SLOW_SLOTS + j] : -1;
+// The record of rank r over the slow lists (list after list, a list's records in order), or -1 past the last.  The
+// counts of 64 lists at a time, one per lane, and a prefix sum over the wavefront; r is the same in all lanes.
+__device__ __forceinline__ int core_slow_record(const CoreArgs& C, int r, int lane) {
+    int base = 0;
+    for (int c0 = 0; c0 < C.slow_lists; c0 += WAVE) {
+        const int c = c0 + lane < C.slow_lists ? C.K.slow_count[c0 + lane] : 0;
+        const int incl = wave_scan_incl(c);
+        const int tot = __builtin_amdgcn_readlane(incl, WAVE - 1);
+        if (r < base + tot) {
+            const uint64_t m = __ballot(base + incl > r);
+            const int l = __builtin_amdgcn_readfirstlane(__ffsll((unsigned long long)m) - 1);
+            const int excl = __builtin_amdgcn_readlane(incl - c, l);
+            return C.K.slow_list[(size_t)(c0 + l) * C.slow_stride + (r - base - excl)];
+        }
+        base += tot;
     }
-    return w - C.slow_wgs;
+    return -1;
 }
-// (a record that is listed is left to the wavefront of its slot)
-__device__ __forceinline__ bool core_record_taken_elsewhere(const CoreArgs& C, uint32_t rec) {
-    return C.slow_wgs > 0 && (int)(blockIdx.x * CORE_WPB + (threadIdx.x >> 6)) >= C.slow_wgs &&
-           ((uint32_t)__builtin_amdgcn_readlane((int)rec, REC_BOX) & C.slow_flag) != 0u;
+// Which record a wavefront of a main kernel starts with: the first slow_wgs wavefronts a listed one (-1: none left),
+// the others the records in work order.
+__device__ __forceinline__ int core_wave_record(const CoreArgs& C, int w, int lane) {
+    return w < C.slow_wgs ? core_slow_record(C, w, lane) : w - C.slow_wgs;
+}
+// The rank over the slow lists of the listed record `wid`: the counts of the lists before its own, and its place in its
+// own list (records in ascending order: the entries below it).
+__device__ __forceinline__ int core_slow_rank(const CoreArgs& C, int wid, int lane) {
+    const int li = wid / C.slow_stride;
+    int part = 0;
+    for (int c0 = lane; c0 < li; c0 += WAVE) part += C.K.slow_count[c0];
+    const int n = C.K.slow_count[li];
+    const int32_t* lst = C.K.slow_list + (size_t)li * C.slow_stride;
+    for (int k = lane; k < n; k += WAVE) part += lst[k] < wid ? 1 : 0;
+    return __builtin_amdgcn_readlane(wave_scan_incl(part), WAVE - 1);
+}
+// A listed record is left to the leading wavefront of its rank; ranks past the leading wavefronts stay in place.
+// `wave_id`: this wavefront's number in the launch.
+__device__ __forceinline__ bool core_record_taken_elsewhere(const CoreArgs& C, uint32_t rec, int wid, int lane) {
+    if (C.slow_wgs == 0 || (int)(blockIdx.x * CORE_WPB + (threadIdx.x >> 6)) < C.slow_wgs) return false;
+    if (((uint32_t)__builtin_amdgcn_readlane((int)rec, REC_BOX) & C.slow_flag) == 0u) return false;
+    return core_slow_rank(C, wid, lane) < C.slow_wgs;
 }
 
 // =================================================================================================================
@@ -447,7 +477,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
     const KernelArgs& P = C.K;
     const int lane = threadIdx.x & (WAVE - 1);
     const int H = P.H;
-    const int wid = core_wave_record(C, (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6));      // this wavefront's (item, head)
+    const int wid = core_wave_record(C, (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6), lane);      // this wavefront's (item, head)
     if (wid < 0) return;
     const int h = wid % H;
     const int pr = lane >> 3;          // pair of the group served by this 8-lane row
@@ -469,7 +499,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
     CFH_PH_DECL
     {
         const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
-        if (core_record_taken_elsewhere(C, rec_cur)) return;
+        if (core_record_taken_elsewhere(C, rec_cur, wid, lane)) return;
         const CorePrefetch pf = core_prefetch(C, rec_cur, it_cur, h, lane);
         CFH_PH(0);
         const CoreItem ci = core_unpack(C, rec_cur, true);
@@ -847,14 +877,13 @@ __global__ __launch_bounds__(WAVE * PROJ_WAVES) void core_project_kernel(const f
 // columns are interleaved (tile t, column c <-> word 4 c + t) so that a lane stores 16 consecutive bytes.
 // grid (ceil(N/16), H, hw/64).  `queues`: optional work-queue heads to clear (when no prepare launch does).
 // Records kept from the forward pass (`slow.items` not null): the wavefronts (x, 0, 0) with x a multiple of
-// SLOW_GB_BLOCKS also list the records of SLOW_GB_BLOCKS x 16 atoms whose box is not the usual one, up to SLOW_SLOTS
-// of them, for the main kernel of the backward pass to take first (as prepare_items_block does for the forward,
+// SLOW_GB_BLOCKS also list the records of SLOW_GB_BLOCKS x 16 atoms whose box is not the usual one, for the main kernel of the backward pass to take first (as prepare_items_block does for the forward,
 // whose lists are gone by now).
 constexpr int SLOW_GB_BLOCKS = 4;
 struct SlowListArgs {
     uint32_t* items;       // (N, H, REC_WORDS) or null
     int32_t* count;        // (lists), lists = ceil(ceil(N / 16) / SLOW_GB_BLOCKS)
-    int32_t* list;         // (lists, SLOW_SLOTS)
+    int32_t* list;         // (lists, SLOW_GB_BLOCKS x 16 x H)
     int32_t R;             // half-width of the usual box
 };
 __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restrict__ go, const float* __restrict__ wcat,
@@ -880,14 +909,13 @@ __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restri
             const uint64_t m = __ballot(own);
             const int rank = listed + __popcll(m & ((1ull << lane) - 1ull));
             if (r < last) {
-                const bool take = own && rank < SLOW_SLOTS;
-                if (take) slow.list[(size_t)li * SLOW_SLOTS + rank] = r;
-                const uint32_t neww = take ? (boxw | REC_BOX_LISTED_BWD) : (boxw & ~REC_BOX_LISTED_BWD);
+                if (own) slow.list[(size_t)li * (SLOW_GB_BLOCKS * 16 * H) + rank] = r;
+                const uint32_t neww = own ? (boxw | REC_BOX_LISTED_BWD) : (boxw & ~REC_BOX_LISTED_BWD);
                 if (neww != boxw) slow.items[(size_t)r * REC_WORDS + REC_BOX] = neww;
             }
             listed += __popcll(m);
         }
-        if (lane == 0) slow.count[li] = min(listed, SLOW_SLOTS);
+        if (lane == 0) slow.count[li] = listed;
     }
     const int row = min(i0 + col, N - 1);
     const float4 a4 = reinterpret_cast<const float4*>(go + ((size_t)row * H + h) * DH)[kk];      // channels 4 kk ..
@@ -1026,7 +1054,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
     const KernelArgs& P = C.K;
     const int lane = threadIdx.x & (WAVE - 1);
     const int H = P.H;
-    const int wid = core_wave_record(C, (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6));
+    const int wid = core_wave_record(C, (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6), lane);
     if (wid < 0) return;
     const int h = wid % H;
     const int pr = lane >> 3, sub = lane & 7;
@@ -1038,7 +1066,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
     if (it_cur >= P.N) return;
     {
         const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
-        if (core_record_taken_elsewhere(C, rec_cur)) return;
+        if (core_record_taken_elsewhere(C, rec_cur, wid, lane)) return;
         const CoreItem ci = core_unpack(C, rec_cur, true);
         const int i = ci.item.i;
         const float a2 = ci.item.a * LOG2E;

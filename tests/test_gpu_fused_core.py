@@ -158,6 +158,21 @@ def test_fused_core_sheared_cells(shear):
     compare(P, _gout(P), out, leaves, oo, oleaves)
 
 
+def test_fused_core_more_records_with_boxes_of_their_own_than_leading_wavefronts():
+    """28 crystals of small cells: some 600 records whose box is not the usual one, more than the 256 wavefronts
+    that take such records first, so the rest are taken in place.  Frames from the search of the same call (equal to
+    those of the box search), out and every gradient against the oracle with those frames."""
+    P = Hh.make_problem(num_crystals=28, atoms_lo=2, atoms_hi=4, len_lo=2.2, len_hi=3.0, ang_lo=80, ang_hi=100, seed=229)
+    R = TO.translation_ranges(P.a, P.rvlen, P.batch, CUT)
+    assert int((R.reshape(-1, 3).max(-1).values > 2).sum()) > 300
+    fr, ref = _frames_both_ways(P)
+    assert torch.equal(fr, ref)
+    out, fr2, leaves = run_core(P, frames="search")
+    assert torch.equal(fr2, ref)
+    oo, oleaves = oracle_core(P, frames=[f.double().cpu() for f in fr2])
+    compare(P, _gout(P), out, leaves, oo, oleaves)
+
+
 def test_fused_core_mixed_boxes_and_long_rows():
     """Crystals of up to 40 atoms (rows of several groups, the running softmax rescales) with cell sizes that
     mix the usual box with larger ones."""
