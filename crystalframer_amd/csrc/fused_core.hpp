@@ -408,19 +408,28 @@ __device__ __forceinline__ void core_store_table(const CoreItem& ci, const CoreP
     }
 }
 
-// The record of rank r over the slow lists (list after list, a list's records in order), or -1 past the last.  The
-// counts of 64 lists at a time, one per lane, and a prefix sum over the wavefront; r is the same in all lanes.
+// The record of rank r over the slow lists (list after list, a list's records in order), or -1 past the last; r is
+// the same in all lanes.  Two levels, so that the wavefront waits for memory twice whatever the number of lists: every
+// lane adds the counts of its own run of consecutive lists (loads that do not depend on each other), a prefix sum over
+// the lanes names the run that holds rank r, and a second prefix sum over the counts of that run names the list.
 __device__ __forceinline__ int core_slow_record(const CoreArgs& C, int r, int lane) {
-    int base = 0;
-    for (int c0 = 0; c0 < C.slow_lists; c0 += WAVE) {
-        const int c = c0 + lane < C.slow_lists ? C.K.slow_count[c0 + lane] : 0;
-        const int incl = wave_scan_incl(c);
-        const int tot = __builtin_amdgcn_readlane(incl, WAVE - 1);
+    const int n = C.slow_lists;
+    const int run = (n + WAVE - 1) / WAVE;
+    int mine = 0;
+    for (int k = 0; k < run; k++) mine += lane * run + k < n ? C.K.slow_count[lane * run + k] : 0;
+    const int incl = wave_scan_incl(mine);
+    if (r >= __builtin_amdgcn_readlane(incl, WAVE - 1)) return -1;
+    const int seg = __builtin_amdgcn_readfirstlane(__ffsll((unsigned long long)__ballot(incl > r)) - 1);
+    int base = __builtin_amdgcn_readlane(incl - mine, seg);
+    for (int k0 = 0; k0 < run; k0 += WAVE) {
+        const int li = seg * run + k0 + lane;
+        const int c = (k0 + lane < run && li < n) ? C.K.slow_count[li] : 0;
+        const int inc2 = wave_scan_incl(c);
+        const int tot = __builtin_amdgcn_readlane(inc2, WAVE - 1);
         if (r < base + tot) {
-            const uint64_t m = __ballot(base + incl > r);
-            const int l = __builtin_amdgcn_readfirstlane(__ffsll((unsigned long long)m) - 1);
-            const int excl = __builtin_amdgcn_readlane(incl - c, l);
-            return C.K.slow_list[(size_t)(c0 + l) * C.slow_stride + (r - base - excl)];
+            const int l = __builtin_amdgcn_readfirstlane(__ffsll((unsigned long long)__ballot(base + inc2 > r)) - 1);
+            const int excl = __builtin_amdgcn_readlane(inc2 - c, l);
+            return C.K.slow_list[(size_t)(seg * run + k0 + l) * C.slow_stride + (r - base - excl)];
         }
         base += tot;
     }
