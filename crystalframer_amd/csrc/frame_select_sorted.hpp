@@ -577,15 +577,14 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void frame_axes_kernel(const CoreA
     __shared__ union { FrameShared item; FrameQuadShared quad; } shared[CORE_WPB];
     const int wv = (int)(threadIdx.x >> 6), lane = (int)threadIdx.x & (WAVE - 1);
     const int blk = (int)blockIdx.x;
-    if (blk < slow_blocks) {
-        const int wid = core_slow_record(C, blk * CORE_WPB + wv, lane);
-        if (wid < 0) return;
-        frame_item_body(C, shared[wv].item, wid, lane, false, false);
-    } else if (blk < slow_blocks + quad_blocks) {
+    if (blk >= slow_blocks && blk < slow_blocks + quad_blocks) {
         frame_quad_body(C, shared[wv].quad, (blk - slow_blocks) * CORE_WPB + wv, lane);
-    } else {
-        frame_item_body(C, shared[wv].item, (blk - slow_blocks - quad_blocks) * CORE_WPB + wv, lane, true, slow_blocks > 0);
+        return;
     }
+    const bool listed = blk < slow_blocks;
+    const int wid = listed ? core_slow_record(C, blk * CORE_WPB + wv, lane) : (blk - slow_blocks - quad_blocks) * CORE_WPB + wv;
+    if (wid < 0) return;
+    frame_item_body(C, shared[wv].item, wid, lane, !listed, !listed && slow_blocks > 0);
 }
 
 }  // namespace cfh

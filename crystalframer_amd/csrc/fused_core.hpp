@@ -472,7 +472,9 @@ struct CoreFwdShared {
     float logit_s[FC_LOGCAP];    // logits of the row (rows of more pairs park them in the probability array)
 };
 template <int WL, bool HAS_ANG, bool COS_ABS>
-__global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const CoreArgs C) {
+// (distance encoding alone: 4.8 KB of LDS per item allow eight wavefronts per SIMD, which 64 registers keep)
+__global__ __launch_bounds__(WAVE * CORE_WPB) __attribute__((amdgpu_waves_per_eu(HAS_ANG ? 1 : 8)))
+void fused_core_fwd_kernel(const CoreArgs C) {
     constexpr int HWK = HAS_ANG ? HW_ANG : HW_DIST;
     __shared__ CoreFwdShared<HWK> shared[CORE_WPB];
     CoreFwdShared<HWK>& sh = shared[threadIdx.x >> 6];
@@ -550,7 +552,6 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
         // several chunks: the survivors of all chunks go into one list with their index in the whole box, and the
         // heavy pass makes their shifts from that index instead of reading a table: one sweep, each chunk built once
         const bool one_list = nchunks > 1 && bx.T <= FC_BIGT;
-        const float inv_s3 = 1.0f / (float)bx.s3, inv_s2 = 1.0f / (float)bx.s2;
         auto fetch = [&](int g0) {
             const int el = g0 + pr;
             if (el < npairs) {
@@ -563,7 +564,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             }
         };
 
-        // one sweep of this row's pair over the table(s): fn(inside, table index, d^2)
+        // one sweep of this row's pair over the table(s): fn(inside, index in the chunk, first index of the chunk, d^2, rows inside)
         auto sweep = [&](bool active, float rx, float ry, float rz, float reach, auto&& fn) {
             for (int ch = 0; ch < nchunks; ch++) {
                 const int t0c = ch * FC_TCAP;
@@ -581,7 +582,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
                     const uint64_t inm = __ballot(in);
                     if (sorted && inm == 0) break;               // every row is past its reach (lengths ascend)
                     const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
-                    fn(in, t0c + t, fmaf(dx, dx, fmaf(dy, dy, dz * dz)), __popcll(inm));
+                    fn(in, t, t0c, fmaf(dx, dx, fmaf(dy, dy, dz * dz)), __popcll(inm));
                     v = vn;
                 }
             }
@@ -590,6 +591,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
         // scatter of the current list (entries point into the resident table)
         auto heavy_impl = [&](int nlist, auto big) {
             constexpr bool BIG = decltype(big)::value;      // entries (pair << FC_BIGSHIFT | index in the box), no table
+            const float inv_s3 = BIG ? 1.0f / (float)bx.s3 : 0.0f, inv_s2 = BIG ? 1.0f / (float)bx.s2 : 0.0f;
             for (int base = 0; base < nlist; base += WAVE) {
                 const int idx = base + lane;
                 if (idx < nlist) {
@@ -672,7 +674,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             if (!known) {
                 d2min = 3.0e38f;
                 sweep(active, rx, ry, rz, sorted ? fmaf(2.0002f, rn, 1e-4f) : INF,
-                      [&](bool in, int, float d2, int cnt_in) { d2min = in ? fminf(d2min, d2) : d2min; n_seen += cnt_in; });
+                      [&](bool in, int, int, float d2, int cnt_in) { d2min = in ? fminf(d2min, d2) : d2min; n_seen += cnt_in; });
                 d2min = half_min(d2min);
             }
 
@@ -683,7 +685,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
             nlist = 0;
             spilled = false;
             if (nchunks == 1) {
-                sweep(active, rx, ry, rz, reachB, [&](bool in, int t, float d2, int cnt_in) {
+                sweep(active, rx, ry, rz, reachB, [&](bool in, int t, int, float d2, int cnt_in) {
                     const float ex = a2 * (d2 - d2min);
                     Sb += in ? hw_exp2(ex) : 0.0f;
                     n_seen += cnt_in;
@@ -693,7 +695,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
                     nlist += __popcll(m);
                 });
             } else {
-                sweep(active, rx, ry, rz, reachB, [&](bool in, int t, float d2, int cnt_in) {
+                sweep(active, rx, ry, rz, reachB, [&](bool in, int t, int t0c, float d2, int cnt_in) {
                     const float ex = a2 * (d2 - d2min);
                     Sb += in ? hw_exp2(ex) : 0.0f;
                     n_seen += cnt_in;
@@ -702,7 +704,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_fwd_kernel(const C
                         const uint64_t m = __ballot(keep);
                         if (nlist + __popcll(m) > FC_LISTCAP) spilled = true;
                         else {
-                            if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_BIGSHIFT) | t);
+                            if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_BIGSHIFT) | (t0c + t));
                             nlist += __popcll(m);
                         }
                     }
@@ -1138,9 +1140,9 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
 
         // several chunks: the survivors of all chunks in one list with their index in the whole box (as in the forward)
         const bool one_list = nchunks > 1 && bx.T <= FC_BIGT;
-        const float inv_s3 = 1.0f / (float)bx.s3, inv_s2 = 1.0f / (float)bx.s2;
         auto heavy_impl = [&](int nlist, auto big) {
             constexpr bool BIG = decltype(big)::value;      // entries (pair << FC_BIGSHIFT | index in the box), no table
+            const float inv_s3 = BIG ? 1.0f / (float)bx.s3 : 0.0f, inv_s2 = BIG ? 1.0f / (float)bx.s2 : 0.0f;
             for (int base = 0; base < nlist; base += WAVE) {
                 const int idx = base + lane;
                 if (idx < nlist) {
