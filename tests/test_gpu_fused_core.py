@@ -291,6 +291,42 @@ def test_fused_core_at_batch_256_against_oracle_on_first_crystals():
         assert Hh.rel_err(leaves[name].grad, oleaves[name].grad) < 1e-4, name
 
 
+def test_fused_core_4096_crystals_equals_the_same_crystals_in_reverse_order():
+    """4096 crystals (22 375 atoms, 179 000 items, 700 lists of records taken first): every item's result depends on
+    its own crystal alone, so the batch with its crystals in reverse order, where every item has another place in the
+    work order and in the lists, must give the same frames, the same rows of out and the same gradients."""
+    from crystalframer_amd import synthetic
+    cb = synthetic.make_config("C5")
+    P = Hh.problem_from_batch(cb, seed=11)
+    B = len(P.sizes)
+    starts = torch.tensor([0] + P.sizes).cumsum(0)
+    perm = torch.cat([torch.arange(int(starts[b]), int(starts[b + 1])) for b in reversed(range(B))])
+    Q = Hh.Problem()
+    Q.sizes = P.sizes[::-1]
+    Q.pos, Q.tvecs = P.pos[perm], P.tvecs.flip(0)
+    Q.batch = torch.repeat_interleave(torch.arange(B), torch.tensor(Q.sizes))
+    Q.edges, Q.rpos, recip, Q.vcell = TO.geometry(Q.pos, Q.tvecs, Q.sizes)
+    Q.rvlen = torch.norm(recip, 2, dim=-1)
+    Q.N, Q.E = P.N, P.E
+    Q.a, Q.q, Q.k, Q.v = P.a[perm], P.q[perm], P.k[perm], P.v[perm]
+    Q.W_k, Q.W_ax, Q.frames = P.W_k, P.W_ax, [f[perm] for f in P.frames]
+    gout = _gout(P, seed=13)
+    res = []
+    for prob, go in ((P, gout), (Q, gout[perm])):
+        out, fr, leaves = run_core(prob, frames="search")
+        assert torch.isfinite(out).all()
+        (out * g(go)).sum().backward()
+        res.append((out.detach(), fr, {n: t.grad for n, t in leaves.items()}))
+    (o1, f1, g1), (o2, f2, g2) = res
+    pd = perm.to(dev())
+    assert torch.equal(f2, f1[:, pd])
+    assert Hh.rel_err(o2, o1[pd]) < 1e-6
+    for name in ("q", "k", "v", "a"):
+        assert Hh.rel_err(g2[name], g1[name][pd]) < 1e-6, name
+    for name in ("Wk", "W1", "W2", "W3"):
+        assert Hh.rel_err(g2[name], g1[name]) < 1e-5, name
+
+
 def test_workspace_header_survives_a_backward_pass():
     """Status word, statistics and work-queue heads at the head of the shared workspace are not scratch: a forward +
     backward pass (with the weight gradients made at the end of the pass) leaves the term counters meaningful and the
