@@ -27,6 +27,7 @@ namespace cfh {
 
 constexpr int FQ_ROWS = 4;          // heads of an atom per wavefront, one per 16-lane row
 constexpr int FQ_STAGE = 64;        // pairs staged at a time
+constexpr int FQ_PAIR_GROUP = 16;   // pairs of a row whose candidates are laid end to end at a time (one per lane of the row)
 constexpr int FQ_MAX_PAIRS = 16;    // longer rows go one item per wavefront: 64 lanes finish a long item sooner than 16
 
 // Shifts t0 .. t0+cnt (cnt <= 128) of the box, sorted by length within the chunk: w = length with the position in the
@@ -334,7 +335,7 @@ struct FrameQuadShared {
     float4 tab[FC_TCAP];
     float4 rp[FQ_STAGE];                 // staged pairs: rpos, d^2 of the nearest valid image (or -1)
     float qk_s[FQ_ROWS][FQ_STAGE];       // q_h . k_j of the staged pairs, per row
-    uint32_t markw[FQ_ROWS][FQ_MAX_PAIRS * FC_TCAP / 32];      // per row: one bit per candidate, set where a pair's run begins
+    uint32_t markw[FQ_ROWS][FQ_PAIR_GROUP * FC_TCAP / 32];      // per row: one bit per candidate, set where a pair's run begins
     uint32_t ent[FQ_ROWS][16];           // per row: the pairs that have candidates, in order: first candidate | pair << 16
 };
 // one wavefront, four heads of one atom: wid = item * groups + group of heads
@@ -342,7 +343,7 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
     float4* const tab = sh.tab;
     float4* const rp = sh.rp;
     float (*const qk_s)[FQ_STAGE] = sh.qk_s;
-    uint32_t (*const markw)[FQ_MAX_PAIRS * FC_TCAP / 32] = sh.markw;
+    uint32_t (*const markw)[FQ_PAIR_GROUP * FC_TCAP / 32] = sh.markw;
     uint32_t (*const ent)[16] = sh.ent;
 
     const KernelArgs& P = C.K;
@@ -484,7 +485,7 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
                     const int first = incl - cnt;
                     wave_sync();                           // the readers of the marks and the list are done
 #pragma unroll
-                    for (int u = 0; u < FQ_MAX_PAIRS * FC_TCAP / 32 / 16; u++) markw[row][l16 + 16 * u] = 0u;
+                    for (int u = 0; u < FQ_PAIR_GROUP * FC_TCAP / 32 / 16; u++) markw[row][l16 + 16 * u] = 0u;
                     wave_sync();
                     if (cnt > 0) {
                         ent[row][kslot] = (uint32_t)first | ((uint32_t)l16 << 16);
