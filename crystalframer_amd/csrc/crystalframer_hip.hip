@@ -1576,6 +1576,7 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         A.q = qs; A.k = k; A.v = v; A.edges = edges; A.e_start = e_start;
         A.prob = const_cast<float*>(prob); A.go = gout; A.gk = gk; A.gv = gv; A.gaij = glogit;
         A.N = (int32_t)N; A.H = p->num_heads; A.E = (int32_t)E;
+        A.items = C.K.items;
         const int64_t items = N * p->num_heads;
         hipLaunchKernelGGL(cfh::dpa_bwd_col_kernel, dim3((unsigned)((items + cfh::DPA_WAVES - 1) / cfh::DPA_WAVES)),
                            dim3(cfh::WAVE * cfh::DPA_WAVES), 0, st, A);

@@ -909,22 +909,27 @@ __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restri
         const int first = (int)blockIdx.x * 16 * H, last = min(first + SLOW_GB_BLOCKS * 16 * H, N * H);
         const uint32_t usual = (uint32_t)(slow.R | (slow.R << 8) | (slow.R << 16));
         int listed = 0;
-        for (int r0 = first; r0 < last; r0 += WAVE) {
-            const int r = r0 + lane;
-            uint32_t boxw = 0;
-            bool own = false;
-            if (r < last) {
-                boxw = slow.items[(size_t)r * REC_WORDS + REC_BOX];
-                own = (boxw & 0x00ffffffu) != usual;
+        for (int r0 = first; r0 < last; r0 += 4 * WAVE) {
+            // (four loads that do not wait for each other, then their ranks)
+            uint32_t boxw[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int r = r0 + u * WAVE + lane;
+                boxw[u] = r < last ? slow.items[(size_t)r * REC_WORDS + REC_BOX] : usual;
             }
-            const uint64_t m = __ballot(own);
-            const int rank = listed + __popcll(m & ((1ull << lane) - 1ull));
-            if (r < last) {
-                if (own) slow.list[(size_t)li * (SLOW_GB_BLOCKS * 16 * H) + rank] = r;
-                const uint32_t neww = own ? (boxw | REC_BOX_LISTED_BWD) : (boxw & ~REC_BOX_LISTED_BWD);
-                if (neww != boxw) slow.items[(size_t)r * REC_WORDS + REC_BOX] = neww;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int r = r0 + u * WAVE + lane;
+                const bool own = r < last && (boxw[u] & 0x00ffffffu) != usual;
+                const uint64_t m = __ballot(own);
+                const int rank = listed + __popcll(m & ((1ull << lane) - 1ull));
+                if (r < last) {
+                    if (own) slow.list[(size_t)li * (SLOW_GB_BLOCKS * 16 * H) + rank] = r;
+                    const uint32_t neww = own ? (boxw[u] | REC_BOX_LISTED_BWD) : (boxw[u] & ~REC_BOX_LISTED_BWD);
+                    if (neww != boxw[u]) slow.items[(size_t)r * REC_WORDS + REC_BOX] = neww;
+                }
+                listed += __popcll(m);
             }
-            listed += __popcll(m);
         }
         if (lane == 0) slow.count[li] = listed;
     }

@@ -40,6 +40,8 @@ struct DpaArgs {
     float* gaij;             // (E,H): always written by the row kernel, read by the column kernel
     float* gbij;             // (E,H,16) or null
     int32_t N, H, E;
+    const uint32_t* items;   // optional (column kernel): the item records (N, H, REC_WORDS) of the launch before, in work
+                             // order; they hold an atom's first pair, pair count and first neighbour in one place
 };
 
 constexpr int DPA_WAVES = 4;     // wavefronts (items) per workgroup
@@ -199,12 +201,22 @@ __global__ __launch_bounds__(WAVE * DPA_WAVES) void dpa_bwd_col_kernel(const Dpa
     const int item = blockIdx.x * DPA_WAVES + (threadIdx.x >> 6);
     if (item >= P.N * P.H) return;
     const int H = P.H;
-    const int j = item / H, h = item - j * H;
+    int j = item / H;
+    const int h = item - j * H;
     const int slot = lane >> 2, qd = lane & 3;
-    const int e0 = (int)P.e_start[j], n = (int)P.e_start[j + 1] - e0;
+    int e0, n, first = 0;
+    if (P.items) {
+        // (the atoms in work order instead of atom order: one read where the arrays need two that wait for each other)
+        const uint4 r4 = *reinterpret_cast<const uint4*>(P.items + (size_t)item * REC_WORDS);
+        j = (int)r4.x; e0 = (int)r4.y; n = (int)r4.z;
+        first = (int)P.items[(size_t)item * REC_WORDS + 30];
+    } else {
+        e0 = (int)P.e_start[j];
+        n = (int)P.e_start[j + 1] - e0;
+        if (n > 0) first = (int)P.edges[(size_t)P.E + e0];      // first atom of the crystal
+    }
     float4 gk = make_float4(0.f, 0.f, 0.f, 0.f), gv = gk;
     if (n > 0) {
-        const int first = (int)P.edges[(size_t)P.E + e0];      // first atom of the crystal
         const int col = j - first;
         const size_t eblock = (size_t)e0 - (size_t)col * n;    // first pair of the crystal
         for (int ib = 0; ib < n; ib += DPA_SLOTS) {
