@@ -64,6 +64,9 @@ __device__ __forceinline__ float row_sum(float x) {
 // scan in DPP, four lane reads and a short loop over the largest number of flags of any lane replace
 // a ballot / prefix / branch per k.  `code` = pair-in-group << shift | tl.  Returns the number of
 // flagged entries of the wavefront.
+// The lanes for which p holds, as a mask.  (HIP's __ballot takes an int: the condition is first made into 0 / 1 in a
+// vector register and then compared with zero again, two vector instructions that this form does not need.)
+__device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_ballot_w64(p); }
 template <int CTRL>
 __device__ __forceinline__ int dpp_movei(int x) { return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xf, 0xf, false); }
 __device__ __forceinline__ int append_flagged(uint16_t* list, int nlist, int room, int skip, uint32_t bits,
@@ -78,7 +81,7 @@ __device__ __forceinline__ int append_flagged(uint16_t* list, int nlist, int roo
     const int t2 = __builtin_amdgcn_readlane(x, 47), t3 = __builtin_amdgcn_readlane(x, 63);
     const int base = slot == 0 ? 0 : slot == 1 ? t0 : slot == 2 ? t0 + t1 : t0 + t1 + t2;
     int pos = base + x - own - skip;
-    while (__ballot(bits != 0u)) {
+    while (ballot(bits != 0u)) {
         if (bits != 0u) {
             const int k = __builtin_ctz(bits);
             bits &= bits - 1u;
@@ -413,7 +416,7 @@ __device__ __forceinline__ int queue_pop(const KernelArgs& P, int h, int& q) {
         const int ql = (int)threadIdx.x & (NQUEUE - 1);
         const int c = __hip_atomic_load(P.counters + (h * NQUEUE + ql) * QSTRIDE, __ATOMIC_RELAXED,
                                         __HIP_MEMORY_SCOPE_AGENT);
-        const uint64_t m = __ballot(c * NQUEUE + ql < P.N) & ((1ull << NQUEUE) - 1ull);
+        const uint64_t m = ballot(c * NQUEUE + ql < P.N) & ((1ull << NQUEUE) - 1ull);
         if (m == 0) return -1;
         q = __builtin_ctzll(m);
     }
@@ -528,7 +531,7 @@ __device__ __forceinline__ void prepare_items_block(const KernelArgs& P, int wit
     if (P.slow_count) {
         __shared__ int slow_in_wave[4];
         const int ln = threadIdx.x & (WAVE - 1), wv = threadIdx.x >> 6;
-        const uint64_t m = __ballot(slow);
+        const uint64_t m = ballot(slow);
         if (ln == 0) slow_in_wave[wv] = __popcll(m);
         __syncthreads();
         int rank = __popcll(m & ((1ull << ln) - 1ull)), total = 0;

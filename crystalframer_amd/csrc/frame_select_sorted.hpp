@@ -222,7 +222,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                             const int incl = wave_scan_incl(mine);
                             total = __builtin_amdgcn_readlane(incl, WAVE - 1);
                             const int first = incl - mine;
-                            const int kslot = (int)lane_prefix(__ballot(mine > 0));
+                            const int kslot = (int)lane_prefix(ballot(mine > 0));
 #pragma unroll
                             for (int u = 0; u < FC_TCAP / 32; u++) markw[lane + WAVE * u] = 0u;
                             wave_sync();
@@ -386,7 +386,7 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
     const int R0 = C.table_R;
     // this row is searched here (the others by frame_item_body)
     const bool mine = row_exists && boxw == (R0 | (R0 << 8) | (R0 << 16)) && a < 0.0f && npairs <= FQ_MAX_PAIRS;
-    if (__ballot(mine) == 0) return;
+    if (ballot(mine) == 0) return;
     Box bx;
     bx.R1 = bx.R2 = bx.R3 = R0; bx.s2 = bx.s3 = 2 * R0 + 1; bx.T = bx.s2 * bx.s2 * bx.s2; bx.over = 0;
     {
@@ -480,7 +480,7 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
                     // the 16 marks of the step plus what the steps before counted) into the list of the pairs that
                     // have candidates.  One read of the marks and one of that list per step, instead of four dependent
                     // reads of a bisection: the step's latency was what the wavefronts waited for.
-                    const uint32_t nzrow = (uint32_t)(__ballot(cnt > 0) >> (16 * row)) & 0xffffu;
+                    const uint32_t nzrow = (uint32_t)(ballot(cnt > 0) >> (16 * row)) & 0xffffu;
                     const int kslot = __popc(nzrow & ((1u << l16) - 1u));
                     const int first = incl - cnt;
                     wave_sync();                           // the readers of the marks and the list are done

@@ -349,11 +349,22 @@ __device__ __forceinline__ CoreItem core_unpack(const CoreArgs& C, uint32_t rec,
     return ci;
 }
 // table of the item's first (or only) chunk
+// build_shift_table with the rest of the last group of FC_GROUP entries filled with length +inf: a sweep then needs
+// one comparison per entry, length <= limit, for "inside the table", "the row has a pair" and "within reach" together
+// (the sorted tables end in such entries as well; built tables have length 0 in every real entry).
+__device__ __forceinline__ void build_shift_table_padded(float4* tab, int t0, int cnt, const Box& bx, const Lattice& L,
+                                                         int lane) {
+    build_shift_table(tab, t0, cnt, bx, L, lane);
+    const int u = cnt + lane;
+    if (lane < 8 && u < ((cnt + 7) & ~7)) tab[u] = make_float4(0.f, 0.f, 0.f, __builtin_inff());
+}
+constexpr float FC_REACH_ALL = 3.0e38f;       // a reach that every real entry is within, and no padding entry
+
 __device__ __forceinline__ void core_load_table(const CoreArgs& C, const CoreItem& ci, float4* tab, int lane) {
     if (ci.sorted) {
         for (int u = lane; u < FC_TCAP; u += WAVE) tab[u] = C.sorted_tab[(size_t)ci.crystal * FC_TCAP + u];
     } else if (ci.nchunks == 1) {
-        build_shift_table(tab, 0, ci.item.bx.T, ci.item.bx, ci.item.L, lane);
+        build_shift_table_padded(tab, 0, ci.item.bx.T, ci.item.bx, ci.item.L, lane);
     }
 }
 
@@ -404,7 +415,7 @@ __device__ __forceinline__ void core_store_table(const CoreItem& ci, const CoreP
         tab[lane] = pf.t0;
         tab[lane + WAVE] = pf.t1;
     } else if (ci.nchunks == 1) {
-        build_shift_table(tab, 0, ci.item.bx.T, ci.item.bx, ci.item.L, lane);
+        build_shift_table_padded(tab, 0, ci.item.bx.T, ci.item.bx, ci.item.L, lane);
     }
 }
 
@@ -419,7 +430,7 @@ __device__ __forceinline__ int core_slow_record(const CoreArgs& C, int r, int la
     for (int k = 0; k < run; k++) mine += lane * run + k < n ? C.K.slow_count[lane * run + k] : 0;
     const int incl = wave_scan_incl(mine);
     if (r >= __builtin_amdgcn_readlane(incl, WAVE - 1)) return -1;
-    const int seg = __builtin_amdgcn_readfirstlane(__ffsll((unsigned long long)__ballot(incl > r)) - 1);
+    const int seg = __builtin_amdgcn_readfirstlane(__ffsll((unsigned long long)ballot(incl > r)) - 1);
     int base = __builtin_amdgcn_readlane(incl - mine, seg);
     for (int k0 = 0; k0 < run; k0 += WAVE) {
         const int li = seg * run + k0 + lane;
@@ -427,7 +438,7 @@ __device__ __forceinline__ int core_slow_record(const CoreArgs& C, int r, int la
         const int inc2 = wave_scan_incl(c);
         const int tot = __builtin_amdgcn_readlane(inc2, WAVE - 1);
         if (r < base + tot) {
-            const int l = __builtin_amdgcn_readfirstlane(__ffsll((unsigned long long)__ballot(base + inc2 > r)) - 1);
+            const int l = __builtin_amdgcn_readfirstlane(__ffsll((unsigned long long)ballot(base + inc2 > r)) - 1);
             const int excl = __builtin_amdgcn_readlane(inc2 - c, l);
             return C.K.slow_list[(size_t)(seg * run + k0 + l) * C.slow_stride + (r - base - excl)];
         }
@@ -566,20 +577,21 @@ void fused_core_fwd_kernel(const CoreArgs C) {
 
         // one sweep of this row's pair over the table(s): fn(inside, index in the chunk, first index of the chunk, d^2, rows inside)
         auto sweep = [&](bool active, float rx, float ry, float rz, float reach, auto&& fn) {
+            const float lim = active ? fminf(reach, FC_REACH_ALL) : -1.0f;      // (lengths are >= 0; padding: +inf)
             for (int ch = 0; ch < nchunks; ch++) {
                 const int t0c = ch * FC_TCAP;
                 const int cnt = sorted ? bx.T : min(FC_TCAP, bx.T - t0c);
                 if (nchunks > 1) {
                     wave_sync();
-                    build_shift_table(tab, t0c, cnt, bx, L, lane);
+                    build_shift_table_padded(tab, t0c, cnt, bx, L, lane);
                     wave_sync();
                 }
-                float4 v = tab[min(sub, cnt - 1)];
+                float4 v = tab[sub];
                 for (int t0 = 0; t0 < cnt; t0 += FC_GROUP) {
                     const int t = t0 + sub;
-                    const float4 vn = tab[min(t + FC_GROUP, cnt - 1)];      // the next step's entry, in flight meanwhile
-                    const bool in = active && t < cnt && v.w <= reach;
-                    const uint64_t inm = __ballot(in);
+                    const float4 vn = tab[min(t + FC_GROUP, FC_TCAP - 1)];      // the next step's entry, in flight meanwhile
+                    const bool in = v.w <= lim;
+                    const uint64_t inm = ballot(in);
                     if (sorted && inm == 0) break;               // every row is past its reach (lengths ascend)
                     const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
                     fn(in, t, t0c, fmaf(dx, dx, fmaf(dy, dy, dz * dz)), __popcll(inm));
@@ -673,35 +685,35 @@ void fused_core_fwd_kernel(const CoreArgs C) {
             CFH_PH(1);
             if (!known) {
                 d2min = 3.0e38f;
-                sweep(active, rx, ry, rz, sorted ? fmaf(2.0002f, rn, 1e-4f) : INF,
+                sweep(active, rx, ry, rz, sorted ? fmaf(2.0002f, rn, 1e-4f) : FC_REACH_ALL,
                       [&](bool in, int, int, float d2, int cnt_in) { d2min = in ? fminf(d2min, d2) : d2min; n_seen += cnt_in; });
                 d2min = half_min(d2min);
             }
 
             // ---- pass B: weights, normaliser and (one-chunk tables) the survivors
             CFH_PH(2);
-            const float reachB = sorted ? fmaf(1.0001f, rn + hw_sqrt(d2min + cutS), 1e-4f) : INF;
+            const float reachB = sorted ? fmaf(1.0001f, rn + hw_sqrt(d2min + cutS), 1e-4f) : FC_REACH_ALL;
             Sb = 0.0f;
             nlist = 0;
             spilled = false;
             if (nchunks == 1) {
                 sweep(active, rx, ry, rz, reachB, [&](bool in, int t, int, float d2, int cnt_in) {
-                    const float ex = a2 * (d2 - d2min);
-                    Sb += in ? hw_exp2(ex) : 0.0f;
+                    const float ex = in ? a2 * (d2 - d2min) : -INF;      // (2^-inf = 0, and -inf is below every threshold)
+                    Sb += hw_exp2(ex);
                     n_seen += cnt_in;
-                    const bool keep = in && ex >= prune;
-                    const uint64_t m = __ballot(keep);
+                    const bool keep = ex >= prune;
+                    const uint64_t m = ballot(keep);
                     if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
                     nlist += __popcll(m);
                 });
             } else {
                 sweep(active, rx, ry, rz, reachB, [&](bool in, int t, int t0c, float d2, int cnt_in) {
-                    const float ex = a2 * (d2 - d2min);
-                    Sb += in ? hw_exp2(ex) : 0.0f;
+                    const float ex = in ? a2 * (d2 - d2min) : -INF;
+                    Sb += hw_exp2(ex);
                     n_seen += cnt_in;
                     if (one_list && !spilled) {
-                        const bool keep = in && ex >= prune;
-                        const uint64_t m = __ballot(keep);
+                        const bool keep = ex >= prune;
+                        const uint64_t m = ballot(keep);
                         if (nlist + __popcll(m) > FC_LISTCAP) spilled = true;
                         else {
                             if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_BIGSHIFT) | (t0c + t));
@@ -714,7 +726,7 @@ void fused_core_fwd_kernel(const CoreArgs C) {
             // a reference borrowed from the usual box may lie far above the nearest image of a larger box (a strongly
             // sheared cell): a sum of weights of 2^24 and more says so (with the nearest image as the reference it is at
             // most the number of translations, 2^13), and the group is done again with a sweep for the nearest
-            if (known && !sorted && __ballot(active && !(S < 0x1p24f)) != 0) { known = false; continue; }
+            if (known && !sorted && ballot(active && !(S < 0x1p24f)) != 0) { known = false; continue; }
             break;
             }
 
@@ -778,7 +790,7 @@ void fused_core_fwd_kernel(const CoreArgs C) {
                         const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
                         const float ex = a2 * (fmaf(dx, dx, fmaf(dy, dy, dz * dz)) - d2min);
                         const bool keep = active && t < cnt && ex >= prune;
-                        const uint64_t m = __ballot(keep);
+                        const uint64_t m = ballot(keep);
                         if (keep) list[nl + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
                         nl += __popcll(m);
                     }
@@ -921,7 +933,7 @@ __global__ __launch_bounds__(WAVE) void core_gbuild_kernel(const float* __restri
             for (int u = 0; u < 4; u++) {
                 const int r = r0 + u * WAVE + lane;
                 const bool own = r < last && (boxw[u] & 0x00ffffffu) != usual;
-                const uint64_t m = __ballot(own);
+                const uint64_t m = ballot(own);
                 const int rank = listed + __popcll(m & ((1ull << lane) - 1ull));
                 if (r < last) {
                     if (own) slow.list[(size_t)li * (SLOW_GB_BLOCKS * 16 * H) + rank] = r;
@@ -1217,7 +1229,8 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
             const float rn = hw_sqrt(fmaf(rx, rx, fmaf(ry, ry, rz * rz)));
             // images with a d^2 log2 e - z2 >= -skip: d^2 <= (z2 - skip) / (a log2 e)
             const float dmax2 = (C.skip_log2 > 0.0f && a2 < 0.0f) ? fmaxf((z2 - C.skip_log2) / a2, 0.0f) : INF;
-            const float reach = sorted ? fmaf(1.0001f, rn + hw_sqrt(dmax2), 1e-4f) : INF;
+            const float reach = sorted ? fmaf(1.0001f, rn + hw_sqrt(dmax2), 1e-4f) : FC_REACH_ALL;
+            const float lim = active ? fminf(reach, FC_REACH_ALL) : -1.0f;      // (lengths are >= 0; padding: +inf)
             if (lane < FC_GROUP) pairB[lane] = 0;
             if (sub == 0 && active) {
                 pairA[pr] = make_float4(rx, ry, rz, z2);
@@ -1230,15 +1243,15 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
                 const int cnt = bx.T;
                 for (int t0 = 0; t0 < cnt; t0 += FC_GROUP) {
                     const int t = t0 + sub;
-                    const float4 v = tab[min(t, cnt - 1)];
-                    const bool in = active && t < cnt && v.w <= reach;
-                    if (sorted && __ballot(in) == 0) break;
+                    const float4 v = tab[t];
+                    const bool in = v.w <= lim;
+                    if (sorted && ballot(in) == 0) break;
                     const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
                     const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
-                    const float ex = fmaf(a2, d2, -z2);
-                    Ap += in ? hw_exp2(ex) * d2 : 0.0f;
-                    const bool keep = in && ex >= prune;
-                    const uint64_t m = __ballot(keep);
+                    const float ex = in ? fmaf(a2, d2, -z2) : -INF;      // (2^-inf = 0, and -inf is below every threshold)
+                    Ap = fmaf(hw_exp2(ex), d2, Ap);
+                    const bool keep = ex >= prune;
+                    const uint64_t m = ballot(keep);
                     if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
                     nlist += __popcll(m);
                 }
@@ -1247,19 +1260,19 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
                     const int t0c = ch * FC_TCAP;
                     const int cnt = min(FC_TCAP, bx.T - t0c);
                     wave_sync();
-                    build_shift_table(tab, t0c, cnt, bx, L, lane);
+                    build_shift_table_padded(tab, t0c, cnt, bx, L, lane);
                     wave_sync();
                     for (int t0 = 0; t0 < cnt; t0 += FC_GROUP) {
                         const int t = t0 + sub;
-                        const float4 v = tab[min(t, cnt - 1)];
-                        const bool in = active && t < cnt;
+                        const float4 v = tab[t];
+                        const bool in = v.w <= lim;
                         const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
                         const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
-                        const float ex = fmaf(a2, d2, -z2);
-                        Ap += in ? hw_exp2(ex) * d2 : 0.0f;
+                        const float ex = in ? fmaf(a2, d2, -z2) : -INF;
+                        Ap = fmaf(hw_exp2(ex), d2, Ap);
                         if (one_list && !spilled) {
-                            const bool keep = in && ex >= prune;
-                            const uint64_t m = __ballot(keep);
+                            const bool keep = ex >= prune;
+                            const uint64_t m = ballot(keep);
                             if (nlist + __popcll(m) > FC_LISTCAP) spilled = true;
                             else {
                                 if (keep) list[nlist + lane_prefix(m)] = (uint16_t)((pr << FC_BIGSHIFT) | (t0c + t));
@@ -1287,7 +1300,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
                         const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
                         const float ex = fmaf(a2, fmaf(dx, dx, fmaf(dy, dy, dz * dz)), -z2);
                         const bool keep = active && t < cnt && ex >= prune;
-                        const uint64_t m = __ballot(keep);
+                        const uint64_t m = ballot(keep);
                         if (keep) list[nl + lane_prefix(m)] = (uint16_t)((pr << FC_SHIFT) | t);
                         nl += __popcll(m);
                     }
