@@ -483,8 +483,9 @@ struct CoreFwdShared {
     float logit_s[FC_LOGCAP];    // logits of the row (rows of more pairs park them in the probability array)
 };
 template <int WL, bool HAS_ANG, bool COS_ABS>
-// (distance encoding alone: 4.8 KB of LDS per item allow eight wavefronts per SIMD, which 64 registers keep)
-__global__ __launch_bounds__(WAVE * CORE_WPB) __attribute__((amdgpu_waves_per_eu(HAS_ANG ? 1 : 8)))
+// (distance encoding alone: 4.8 KB of LDS per item allow eight wavefronts per SIMD; seven, with 72 registers and
+// nothing spilled, ran faster than eight with 64 and nine spilled)
+__global__ __launch_bounds__(WAVE * CORE_WPB) __attribute__((amdgpu_waves_per_eu(HAS_ANG ? 1 : 7)))
 void fused_core_fwd_kernel(const CoreArgs C) {
     constexpr int HWK = HAS_ANG ? HW_ANG : HW_DIST;
     __shared__ CoreFwdShared<HWK> shared[CORE_WPB];
