@@ -26,9 +26,10 @@
 namespace cfh {
 
 constexpr int FQ_ROWS = 4;          // heads of an atom per wavefront, one per 16-lane row
-constexpr int FQ_STAGE = 64;        // pairs staged at a time
+constexpr int FQ_STAGE = 16;        // pairs staged at a time (the rows of this search have no more)
 constexpr int FQ_PAIR_GROUP = 16;   // pairs of a row whose candidates are laid end to end at a time (one per lane of the row)
 constexpr int FQ_MAX_PAIRS = 16;    // longer rows go one item per wavefront: 64 lanes finish a long item sooner than 16
+static_assert(FQ_MAX_PAIRS <= FQ_STAGE && FQ_STAGE <= WAVE, "a row of the four-heads search is staged as a whole");
 
 // Shifts t0 .. t0+cnt (cnt <= 128) of the box, sorted by length within the chunk: w = length with the position in the
 // chunk (loop order of the reference) in its low 7 bits, like the entries of the per-crystal tables.  Items whose box
@@ -75,6 +76,7 @@ struct FrameShared {
     float4 pq[WAVE];             // rpos and q.k of the staged pairs
     uint32_t markw[WAVE * FC_TCAP / 32];      // one bit per candidate, set where the run of a pair begins
     uint32_t ent[WAVE];          // the staged pairs that have candidates, in order: first candidate | pair << 16
+    float ph[WAVE];              // phase of the tie-breaking noise of the staged pairs in the current pass
     int total;                   // candidates of the list that the marks describe
 };
 // one wavefront, one item: wid = item * H + head.  `others_only`: only the items that the four-heads-per-wavefront
@@ -174,6 +176,13 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                     } else {
                         rq = pq[lane];
                     }
+                    // the noise of a candidate is a hash of (pair, head, pass) shifted by the translation: the hash once per
+                    // pair here (three integer multiplications), not once per candidate
+                    if (noisy) {
+                        wave_sync();
+                        sh.ph[lane] = hash_uniform(pass ? seed_hi : seed_lo, pass ? seed_lo : seed_hi,
+                                                   (uint32_t)((e0 + pb + lane) * H + h), (uint32_t)pass);
+                    }
                     // how far into the sorted table this lane's pair has to look
                     float reach = 3.0e38f;
                     if (a < 0.0f) {
@@ -260,8 +269,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                                 ok = ok && ac < 0.9999f;
                             }
                             if (noisy) {
-                                const float phase = hash_uniform(pass ? seed_hi : seed_lo, pass ? seed_lo : seed_hi,
-                                                                 (uint32_t)(e * H + h), (uint32_t)pass);
+                                const float phase = sh.ph[pl];
                                 const float un = __builtin_amdgcn_fractf(fmaf((float)t, 0.61803399f, phase));
                                 if (pass == 0) score = fmaf(a, d2 + (un - 0.5f) * P.noise, cq.w);
                                 else score += (un - 0.5f) * P.noise;
@@ -335,6 +343,7 @@ struct FrameQuadShared {
     float4 tab[FC_TCAP];
     float4 rp[FQ_STAGE];                 // staged pairs: rpos, d^2 of the nearest valid image (or -1)
     float qk_s[FQ_ROWS][FQ_STAGE];       // q_h . k_j of the staged pairs, per row
+    float ph_s[2][FQ_ROWS][FQ_STAGE];    // phase of the tie-breaking noise of the staged pairs, per pass and row
     uint32_t markw[FQ_ROWS][FQ_PAIR_GROUP * FC_TCAP / 32];      // per row: one bit per candidate, set where a pair's run begins
     uint32_t ent[FQ_ROWS][16];           // per row: the pairs that have candidates, in order: first candidate | pair << 16
 };
@@ -418,7 +427,7 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
                         r4.x = P.rpos[(size_t)e * 3 + 0]; r4.y = P.rpos[(size_t)e * 3 + 1]; r4.z = P.rpos[(size_t)e * 3 + 2];
                         if (C.pair_near) r4.w = C.pair_near[e].y;
                     }
-                    rp[lane] = r4;
+                    if (lane < FQ_STAGE) rp[lane] = r4;
 #pragma unroll 1
                     for (int r = 0; r < FQ_ROWS; r++) {
                         const int hr = min(hg * FQ_ROWS + r, H - 1);
@@ -432,7 +441,14 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
                             acc = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(q[4 * c4 + 2]), r * 16)), kv.z, acc);
                             acc = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(q[4 * c4 + 3]), r * 16)), kv.w, acc);
                         }
-                        qk_s[r][lane] = acc;
+                        if (lane < FQ_STAGE) qk_s[r][lane] = acc;
+                    }
+                    // the noise of a candidate is a hash of (pair, head, pass) shifted by the translation: the hash once per
+                    // pair and pass here (three integer multiplications), not once per candidate
+                    if (noisy) {
+                        const uint32_t key = (uint32_t)((e0 + pb + min(l16, nst - 1)) * H + h_row);
+                        sh.ph_s[0][row][l16] = hash_uniform(seed_lo, seed_hi, key, 0u);
+                        sh.ph_s[1][row][l16] = hash_uniform(seed_hi, seed_lo, key, 1u);
                     }
                     wave_sync();
                 }
@@ -519,8 +535,7 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
                             ok = ok && ac < 0.9999f;
                         }
                         if (noisy) {
-                            const float phase = hash_uniform(pass ? seed_hi : seed_lo, pass ? seed_lo : seed_hi,
-                                                             (uint32_t)(e * H + h_row), (uint32_t)pass);
+                            const float phase = sh.ph_s[pass][row][ps];
                             const float un = __builtin_amdgcn_fractf(fmaf((float)t, 0.61803399f, phase));
                             if (pass == 0) score = fmaf(a, d2 + (un - 0.5f) * P.noise, cqk);
                             else score += (un - 0.5f) * P.noise;
