@@ -220,6 +220,18 @@ void fill_common(cfh::KernelArgs& A, const cfh_params* p, const float* a_ih, con
     A.items = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(workspace) + COUNTER_BYTES);
     A.stats = p->collect_stats ? reinterpret_cast<unsigned long long*>(reinterpret_cast<char*>(workspace) + STATS_OFFSET) : nullptr;
     A.N = (int32_t)N; A.E = (int32_t)E; A.H = p->num_heads;
+    {
+        // n / H = (n * m) >> (31 + l) with l = ceil(log2 H), m = ceil(2^(31 + l) / H) < 2^32: exact for 0 <= n < 2^31
+        const uint32_t d = (uint32_t)p->num_heads;
+        if (d <= 1) { A.h_magic = 0; A.h_shift = 0; }
+        else {
+            int l = 0;
+            while ((1u << l) < d) l++;
+            const unsigned long long two = 1ull << (31 + l);
+            A.h_magic = (uint32_t)((two + d - 1) / d);
+            A.h_shift = l - 1;
+        }
+    }
     A.cutoff_radius = rvlen ? p->cutoff_radius : 0.0f;
     A.lattice_range = p->lattice_range; A.minimum_range = p->minimum_range;
     A.prune_log2 = p->prune_log2;

@@ -368,6 +368,7 @@ struct KernelArgs {
     unsigned long long* stats;    // optional running totals (see STAT_* below); never reset by a launch
     int32_t* status;              // word of the workspace header: set to 1 when a box was cut back to RMAX (never cleared)
     int32_t N, E, H;
+    uint32_t h_magic; int32_t h_shift;      // n / H for 0 <= n < 2^31 as (n * h_magic) >> (32 + h_shift); h_magic 0: H = 1
     float cutoff_radius; int32_t lattice_range, minimum_range;
     float prune_log2;             // <= 0: keep every translation
     float dist_coef, angle_coef, gz_coef, gw_dist_coef;
@@ -467,6 +468,10 @@ __device__ __forceinline__ Item unpack_item(uint32_t rec) {
     return t;
 }
 // the same for a wavefront that is not the first of its workgroup
+// wid / H without a division (the heads are a launch argument, and a 32-bit division is some 25 vector instructions)
+__device__ __forceinline__ int div_heads(const KernelArgs& P, int wid) {
+    return P.h_magic ? (int)(__umulhi((uint32_t)wid, P.h_magic) >> P.h_shift) : wid;
+}
 __device__ __forceinline__ uint32_t load_record_lane(const KernelArgs& P, int it, int h, int lane) {
     return (it >= 0 && lane < REC_WORDS) ? P.items[((size_t)it * P.H + h) * REC_WORDS + lane] : 0u;
 }

@@ -91,7 +91,8 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
 
     const KernelArgs& P = C.K;
     const int H = P.H;
-    const int h = wid % H;
+    const int it_cur = div_heads(P, wid);      // one wavefront per item, long items first
+    const int h = wid - it_cur * H;
     const bool noisy = P.noise > 0.0f;
     uint32_t seed_lo = P.seed_lo, seed_hi = P.seed_hi;
     if (noisy && P.seed_dev) {
@@ -100,7 +101,6 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
         seed_hi += (uint32_t)(s >> 32) ^ ((uint32_t)s * 0x85EBCA77u);
     }
 
-    const int it_cur = wid / H;      // one wavefront per item, long items first
     if (it_cur >= P.N) return;
     {
         const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);

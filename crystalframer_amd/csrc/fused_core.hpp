@@ -502,14 +502,14 @@ void fused_core_fwd_kernel(const CoreArgs C) {
     const int H = P.H;
     const int wid = core_wave_record(C, (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6), lane);      // this wavefront's (item, head)
     if (wid < 0) return;
-    const int h = wid % H;
+    const int it_cur = div_heads(P, wid);      // items in descending order of their pair count: the long ones start first
+    const int h = wid - it_cur * H;
     const int pr = lane >> 3;          // pair of the group served by this 8-lane row
     const int sub = lane & 7;          // position in the row
     const BasisConsts bc = P.bc;
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
     const float INF = __builtin_inff();
 
-    const int it_cur = wid / H;      // items in descending order of their pair count: the long ones start first
     if (it_cur >= P.N) return;
     if (HWK >= 4 * WAVE) {
 #pragma unroll
@@ -547,7 +547,7 @@ void fused_core_fwd_kernel(const CoreArgs C) {
         const size_t ih = (size_t)i * H + h;
         const float2 q2 = pf.q2;
         const float fixs = 1073741824.0f / (float)max(npairs, 1);      // 2^30 / npairs: sums of weights <= 1 each fit
-        const float cutS = (C.skip_log2 > 0.0f && a2 < 0.0f) ? C.skip_log2 / (-a2) : INF;
+        const float cutS = (C.skip_log2 > 0.0f && a2 < 0.0f) ? C.skip_log2 * hw_rcp(-a2) : INF;      // (a bound with margins)
         float m_run = -INF;                   // running maximum of the logits (wave-uniform)
         float Dl = 0.0f;                      // this lane's share of the softmax denominator
         float2 accv = make_float2(0.f, 0.f);  // sum_j exp(logit_j - m_run) v_j, channels 2 sub, 2 sub + 1
@@ -604,7 +604,8 @@ void fused_core_fwd_kernel(const CoreArgs C) {
         // scatter of the current list (entries point into the resident table)
         auto heavy_impl = [&](int nlist, auto big) {
             constexpr bool BIG = decltype(big)::value;      // entries (pair << FC_BIGSHIFT | index in the box), no table
-            const float inv_s3 = BIG ? 1.0f / (float)bx.s3 : 0.0f, inv_s2 = BIG ? 1.0f / (float)bx.s2 : 0.0f;
+            // (hardware reciprocals, within an ulp: the quotients below stay exact all the same)
+            const float inv_s3 = BIG ? hw_rcp((float)bx.s3) : 0.0f, inv_s2 = BIG ? hw_rcp((float)bx.s2) : 0.0f;
             for (int base = 0; base < nlist; base += WAVE) {
                 const int idx = base + lane;
                 if (idx < nlist) {
@@ -1085,13 +1086,13 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
     const int H = P.H;
     const int wid = core_wave_record(C, (int)blockIdx.x * CORE_WPB + (int)(threadIdx.x >> 6), lane);
     if (wid < 0) return;
-    const int h = wid % H;
+    const int it_cur = div_heads(P, wid);      // one wavefront per item, long items first
+    const int h = wid - it_cur * H;
     const int pr = lane >> 3, sub = lane & 7;
     const BasisConsts bc = P.bc;
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
     const float INF = __builtin_inff();
 
-    const int it_cur = wid / H;      // one wavefront per item, long items first
     if (it_cur >= P.N) return;
     {
         const uint32_t rec_cur = load_record_lane(P, it_cur, h, lane);
@@ -1134,6 +1135,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
         const float2 ov2 = *reinterpret_cast<const float2*>(C.outv + ih * DH + 2 * sub);
         const float c0 = half_sum(fmaf(go2.x, ov2.x, go2.y * ov2.y));          // go . out_i
         const float gnorm = uniform_f(wave_sum(gabs));                          // |bg| <= sum |G|
+        const float inv_a2 = a2 < 0.0f ? hw_rcp(a2) : 0.0f;             // (for a bound with margins)
         const float bscale = 1073741824.0f / fmaxf(gnorm, 1e-20f);      // (finite: 2^30 / 1e-30 would not be)
         const float binv = fmaxf(gnorm, 1e-20f) * (1.0f / 1073741824.0f);
         wave_sync();
@@ -1160,7 +1162,8 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
         const bool one_list = nchunks > 1 && bx.T <= FC_BIGT;
         auto heavy_impl = [&](int nlist, auto big) {
             constexpr bool BIG = decltype(big)::value;      // entries (pair << FC_BIGSHIFT | index in the box), no table
-            const float inv_s3 = BIG ? 1.0f / (float)bx.s3 : 0.0f, inv_s2 = BIG ? 1.0f / (float)bx.s2 : 0.0f;
+            // (hardware reciprocals, within an ulp: the quotients below stay exact all the same)
+            const float inv_s3 = BIG ? hw_rcp((float)bx.s3) : 0.0f, inv_s2 = BIG ? hw_rcp((float)bx.s2) : 0.0f;
             for (int base = 0; base < nlist; base += WAVE) {
                 const int idx = base + lane;
                 if (idx < nlist) {
@@ -1229,7 +1232,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
             const bool active = g0 + pr < npairs;
             const float rn = hw_sqrt(fmaf(rx, rx, fmaf(ry, ry, rz * rz)));
             // images with a d^2 log2 e - z2 >= -skip: d^2 <= (z2 - skip) / (a log2 e)
-            const float dmax2 = (C.skip_log2 > 0.0f && a2 < 0.0f) ? fmaxf((z2 - C.skip_log2) / a2, 0.0f) : INF;
+            const float dmax2 = (C.skip_log2 > 0.0f && a2 < 0.0f) ? fmaxf((z2 - C.skip_log2) * inv_a2, 0.0f) : INF;
             const float reach = sorted ? fmaf(1.0001f, rn + hw_sqrt(dmax2), 1e-4f) : FC_REACH_ALL;
             const float lim = active ? fminf(reach, FC_REACH_ALL) : -1.0f;      // (lengths are >= 0; padding: +inf)
             if (lane < FC_GROUP) pairB[lane] = 0;
