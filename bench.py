@@ -41,7 +41,7 @@ PEAK_TRANS_TOPS = 9.8                  # quarter-rate transcendental unit
 # --calibrate-copy; the figures and the commands are in TRAFFIC_SOURCE.  Other batch sizes or settings: null.
 TRAFFIC_SOURCE = "profiles/fused_core_hbm_traffic_C3.md"
 # forward 9 303.6 KiB x 2.0 + 92 229.7 KiB; backward 54 969.4 x 2.0 + 9 393.4; frame search 8 191.6 x 2.0 + 2 392.5
-TRAFFIC_BYTES_PER_LAUNCH = {"fused_core_forward": 113.9e6, "fused_core_backward": 122.6e6, "frame_axes": 19.6e6}
+TRAFFIC_BYTES_PER_LAUNCH = {"fused_core_forward": 113.9e6, "fused_core_backward": 122.5e6, "frame_axes": 19.4e6}
 
 
 def parse():
@@ -328,7 +328,7 @@ def main():
                         "execute that many: the angle encoding is scattered as 5 local moments per axis instead of a "
                         "33-bin window and the projection runs once per (atom, head) in a separate MFMA kernel.  What "
                         "binds it is the issue of vector instructions, few of which are multiply-adds (one wavefront per "
-                        "(atom, head), 12.5 pairs on average): vector ALUs issuing 80 % of the kernel's time with 86 % "
+                        "(atom, head), 12.5 pairs on average): vector ALUs issuing 76 % of the kernel's time with 79 % "
                         "of the lanes active, HBM at a quarter of its peak (profiles/fused_core_valu_lds_counters_C3.md)",
         "both_kernels": {k: {"kernel": r["kernel"], "achieved": r["achieved"], "frac": r["frac"],
                              "avg_launch_ms": r["avg_launch_ms"]} for k, r in roof.items()},
