@@ -36,7 +36,7 @@ __device__ __forceinline__ void box_coords(int t, const Box& bx, float inv_s2, f
 __device__ __forceinline__ void shift_of(int t, const Box& bx, const Lattice& L, float& vx, float& vy,
                                          float& vz) {
     int m1, m2, m3;
-    box_coords(t, bx, 1.0f / (float)bx.s2, 1.0f / (float)bx.s3, m1, m2, m3);
+    box_coords(t, bx, hw_rcp((float)bx.s2), hw_rcp((float)bx.s3), m1, m2, m3);      // (within an ulp: the quotients stay exact)
     const float n1 = (float)m1, n2 = (float)m2, n3 = (float)m3;
     vx = fmaf(L.t[6], n3, fmaf(L.t[3], n2, L.t[0] * n1));
     vy = fmaf(L.t[7], n3, fmaf(L.t[4], n2, L.t[1] * n1));

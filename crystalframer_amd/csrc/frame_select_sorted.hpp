@@ -112,6 +112,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
         const int j0 = __builtin_amdgcn_readlane((int)rec_cur, REC_J0);
         const int i = item.i;
         const float a = item.a;
+        const float inv_a = a < 0.0f ? hw_rcp(a) : 0.0f;      // (for a reach with margins: the hardware reciprocal will do)
         const Lattice L = item.L;
         const Box bx = item.bx;
         float qi[DH];
@@ -194,7 +195,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                             if (dvalid >= 0.0f) reach = fmaf(1.0001f, r + hw_sqrt(dvalid + nz), 1e-3f);
                             else if (sorted) reach = fmaf(1.0001f, fmaf(2.0f, r, (r2 > 1e-5f ? 0.0f : s1) + sq_nz), 1e-3f);
                         } else if (bound > -1.0e38f) {
-                            const float need = (bound - rq.w - 0.5f * nz) / a;
+                            const float need = (bound - rq.w - 0.5f * nz) * inv_a;
                             reach = need >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(need), 1e-3f) : -1.0f;
                         }
                     }
@@ -359,7 +360,9 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
     const int row = lane >> 4, l16 = lane & 15;
     const int H = P.H;
     const int groups = (H + FQ_ROWS - 1) / FQ_ROWS;
-    const int it = wid / groups, hg = wid % groups;
+    // (groups of heads: a power of two for 4, 8, 16 ... heads, then without a division)
+    const bool pow2 = (groups & (groups - 1)) == 0;
+    const int it = pow2 ? wid >> (__ffs(groups) - 1) : wid / groups, hg = wid - it * groups;
     if (it >= P.N) return;
     const int h_row = min(hg * FQ_ROWS + row, H - 1);
     const bool row_exists = hg * FQ_ROWS + row < H;
@@ -383,6 +386,7 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
     for (int d = 0; d < 9; d++) L.t[d] = __int_as_float(__builtin_amdgcn_readlane((int)w0, REC_LATTICE + d));
     const int boxw = (int)rec[REC_BOX];
     const float a = __uint_as_float(rec[REC_A]);
+    const float inv_a = a < 0.0f ? hw_rcp(a) : 0.0f;      // (for a reach with margins: the hardware reciprocal will do)
     float q[DH];
     {
         const float4* qp = reinterpret_cast<const float4*>(rec + REC_QUERY);
@@ -465,7 +469,7 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
                         reach = r4.w >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(r4.w + nz), 1e-3f)
                                              : fmaf(1.0001f, fmaf(2.0f, r, (r2 > 1e-5f ? 0.0f : s1) + sq_nz), 1e-3f);
                     } else if (bound > -1.0e38f) {
-                        const float need = (bound - myqk - 0.5f * nz) / a;
+                        const float need = (bound - myqk - 0.5f * nz) * inv_a;
                         reach = need >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(need), 1e-3f) : -1.0f;
                     } else {
                         reach = 3.0e38f;
