@@ -163,6 +163,8 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
         self._gauss_ready = None      # host-side cache of "gauss_scale[0] > 0"
         self._in_proj_stack = None    # the storage q/k/v_proj_weight share once they are adjacent
         self.frame_sink = None        # a list: every forward appends its (f1, f2, f3) (diagnostics)
+        self.grad_sink = None         # a dict: the backward pass leaves the gradients of the attention core's operands
+                                      # (scaled query "q", "k", "v", Gaussian coefficient "a") in it (diagnostics)
         self._reset_parameters()
 
     def _reset_parameters(self):
@@ -305,6 +307,12 @@ class CrystalformerMultiheadAttentionCUDA(nn.Module):
         coefficients a (N,H): the heads' outputs side by side (N, H Dv), before the output projection,
         and psi."""
         P = self.params
+        if not q_is_scaled:
+            q, q_is_scaled = q / math.sqrt(q.shape[-1]), True
+        if self.grad_sink is not None:
+            for name, t in (("q", q), ("k", k), ("v", v), ("a", a)):
+                if t.requires_grad:
+                    t.register_hook(lambda grad, name=name: self.grad_sink.__setitem__(name, grad.detach()))
         if (FUSED_CORE and q.is_cuda and P.frame_method == "max" and batch_q is batch_kv and self.pe_dist_proj is not None
                 and cuda_funcs.PeriodicAttentionCoreHIP.supported(
                     P.value_pe_dist_real, P.value_pe_angle_real, P.value_pe_dist_wscale, P.value_pe_angle_wscale,

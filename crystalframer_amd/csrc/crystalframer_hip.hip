@@ -277,6 +277,33 @@ struct TimedLaunch { std::string what; hipEvent_t start, stop; };
 std::mutex g_timing_mutex;
 bool g_timing_on = false;
 std::vector<TimedLaunch> g_timed;
+// set by an entry point that must not allocate (events are allocations): its launches are never timed
+thread_local bool t_timing_blocked = false;
+// Brackets the launches made during its lifetime with a pair of events on their stream, when timing is on.
+struct TimedScope {
+    TimedLaunch t;
+    hipStream_t st;
+    bool on = false;
+    TimedScope(const char* what, hipStream_t stream) : st(stream) {
+        if (t_timing_blocked) return;
+        {
+            std::lock_guard<std::mutex> lock(g_timing_mutex);
+            on = g_timing_on;
+        }
+        if (!on) return;
+        t.what = what;
+        on = hipEventCreate(&t.start) == hipSuccess && hipEventCreate(&t.stop) == hipSuccess &&
+             hipEventRecord(t.start, st) == hipSuccess;
+    }
+    ~TimedScope() {
+        if (on && hipEventRecord(t.stop, st) == hipSuccess) {
+            std::lock_guard<std::mutex> lock(g_timing_mutex);
+            g_timed.push_back(t);
+        }
+    }
+    TimedScope(const TimedScope&) = delete;
+    TimedScope& operator=(const TimedScope&) = delete;
+};
 
 // `waves`: in = upper bound, out = wavefronts actually launched
 template <typename Kern>
@@ -288,21 +315,9 @@ int launch_persistent(Kern kern, const cfh::KernelArgs& A, int* waves, hipStream
         if (threads < A.gw_out_n) threads = A.gw_out_n;
         hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, A, A.q != nullptr ? 1 : 0);
     }
-    bool timed = false;
-    TimedLaunch t;
     {
-        std::lock_guard<std::mutex> lock(g_timing_mutex);
-        timed = g_timing_on;
-    }
-    if (timed) {
-        t.what = what;
-        timed = hipEventCreate(&t.start) == hipSuccess && hipEventCreate(&t.stop) == hipSuccess &&
-                hipEventRecord(t.start, st) == hipSuccess;
-    }
-    hipLaunchKernelGGL(kern, dim3(*waves), dim3(cfh::WAVE), 0, st, A);
-    if (timed && hipEventRecord(t.stop, st) == hipSuccess) {
-        std::lock_guard<std::mutex> lock(g_timing_mutex);
-        g_timed.push_back(t);
+        TimedScope timed(what, st);
+        hipLaunchKernelGGL(kern, dim3(*waves), dim3(cfh::WAVE), 0, st, A);
     }
     return finish_launch(what);
 }
@@ -612,7 +627,10 @@ int cfh_framed_pe_forward_static(const cfh_params* p, const float* a_ih, const f
         return fail(CFH_EINVAL, "the 16-bin angle basis needs workspace for padded weights: use cfh_framed_pe_forward");
     void* ptr = static_scratch();
     if (!ptr) return CFH_EDEVICE;
-    // the work-queue heads are cleared by the prepare kernel of every launch; nothing else must start at zero
+    // the work-queue heads are cleared by the prepare kernel of every launch; nothing else must start at zero.
+    // The timing diagnostics create events, i.e. allocate: they are off for this call whatever cfh_timing_enable says.
+    struct Unblock { ~Unblock() { t_timing_blocked = false; } } unblock;
+    t_timing_blocked = true;
     return framed_pe_forward_impl(p, nullptr, nullptr, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, W_dist,
                                   W_axis1, W_axis2, W_axis3, frames, nullptr, N, E, B, z, psi, d2min_out, shat_out,
                                   ptr, STATIC_SCRATCH_BYTES, stream);
@@ -1319,21 +1337,9 @@ template <typename Kern>
 int launch_core(Kern kern, const cfh::CoreArgs& C, hipStream_t st, const char* what, unsigned waves = 0) {
     if (waves == 0) waves = (unsigned)C.K.N * (unsigned)C.K.H + (unsigned)C.slow_wgs;
     const unsigned blocks = (waves + cfh::CORE_WPB - 1) / cfh::CORE_WPB;
-    bool timed = false;
-    TimedLaunch t;
     {
-        std::lock_guard<std::mutex> lock(g_timing_mutex);
-        timed = g_timing_on;
-    }
-    if (timed) {
-        t.what = what;
-        timed = hipEventCreate(&t.start) == hipSuccess && hipEventCreate(&t.stop) == hipSuccess &&
-                hipEventRecord(t.start, st) == hipSuccess;
-    }
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(cfh::WAVE * cfh::CORE_WPB), 0, st, C);
-    if (timed && hipEventRecord(t.stop, st) == hipSuccess) {
-        std::lock_guard<std::mutex> lock(g_timing_mutex);
-        g_timed.push_back(t);
+        TimedScope timed(what, st);
+        hipLaunchKernelGGL(kern, dim3(blocks), dim3(cfh::WAVE * cfh::CORE_WPB), 0, st, C);
     }
     return finish_launch(what);
 }
@@ -1377,6 +1383,7 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     const CoreBuffers buf = fill_core(C, p, L, qs, k, v, rvlen != nullptr, cache, workspace);
     const bool search = has_ang && search_frames != 0;
     if (buf.table && !buf.table_ready) {
+        TimedScope timed("core_tables", st);
         hipLaunchKernelGGL(cfh::sorted_shifts_kernel, dim3((unsigned)B), dim3(cfh::FC_TCAP), 0, st, tvecs, C.table_R,
                            buf.table);
         if (buf.near && E > 0) {
@@ -1404,42 +1411,34 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
             F.K.q = qs; F.K.k = k; F.K.out_frame = frames;
             F.K.counters2 = reinterpret_cast<int32_t*>(ws + QUEUE_OFFSET + QUEUE_SET_BYTES);
             F.K.frames_to_records = 1;
-            hipLaunchKernelGGL(cfh::core_prepare_wcat_kernel, dim3(prep_blocks + p->num_heads * cfh::DH), dim3(256), 0, st,
-                               F.K, 1, prep_blocks, WA);
+            {
+                TimedScope timed("core_prepare", st);
+                hipLaunchKernelGGL(cfh::core_prepare_wcat_kernel, dim3(prep_blocks + p->num_heads * cfh::DH), dim3(256), 0, st,
+                                   F.K, 1, prep_blocks, WA);
+            }
             if (F.sorted_tab) {
                 // four heads of an atom per wavefront for the items with the usual box and short rows, the others one
                 // by one, all in one launch
                 const unsigned item_blocks = ((unsigned)N * (unsigned)p->num_heads + cfh::CORE_WPB - 1) / cfh::CORE_WPB;
                 const unsigned quad_waves = (unsigned)N * (unsigned)((p->num_heads + cfh::FQ_ROWS - 1) / cfh::FQ_ROWS);
                 const unsigned quad_blocks = (quad_waves + cfh::CORE_WPB - 1) / cfh::CORE_WPB;
-                bool timed = false;
-                TimedLaunch t;
-                {
-                    std::lock_guard<std::mutex> lock(g_timing_mutex);
-                    timed = g_timing_on;
-                }
-                if (timed) {
-                    t.what = "frame_axes";
-                    timed = hipEventCreate(&t.start) == hipSuccess && hipEventCreate(&t.stop) == hipSuccess &&
-                            hipEventRecord(t.start, st) == hipSuccess;
-                }
                 if (F.K.slow_count) {
                     F.slow_lists = prep_blocks;
                     F.slow_stride = cfh::SLOW_PREP_SLOTS;
                     F.slow_wgs = slow_wave_count(N, p->num_heads);
                 }
                 const unsigned slow_blocks = ((unsigned)F.slow_wgs + cfh::CORE_WPB - 1) / cfh::CORE_WPB;
-                hipLaunchKernelGGL(cfh::frame_axes_kernel, dim3(slow_blocks + quad_blocks + item_blocks),
-                                   dim3(cfh::WAVE * cfh::CORE_WPB), 0, st, F, (int)slow_blocks, (int)quad_blocks);
-                if (timed && hipEventRecord(t.stop, st) == hipSuccess) {
-                    std::lock_guard<std::mutex> lock(g_timing_mutex);
-                    g_timed.push_back(t);
+                {
+                    TimedScope timed("frame_axes", st);
+                    hipLaunchKernelGGL(cfh::frame_axes_kernel, dim3(slow_blocks + quad_blocks + item_blocks),
+                                       dim3(cfh::WAVE * cfh::CORE_WPB), 0, st, F, (int)slow_blocks, (int)quad_blocks);
                 }
                 if ((rc = finish_launch("frame_axes"))) return rc;
             } else if ((rc = launch_core(cfh::frame_axes_sorted_kernel, F, st, "frame_axes"))) return rc;
             C.K.counters = F.K.counters2;
         } else {
             C.K.frames = has_ang ? frames : nullptr;
+            TimedScope timed("core_prepare", st);
             hipLaunchKernelGGL(cfh::core_prepare_wcat_kernel, dim3(prep_blocks + p->num_heads * cfh::DH), dim3(256), 0, st,
                                C.K, 0, prep_blocks, WA);
         }
@@ -1467,8 +1466,11 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     } while (0)
     CFH_CORE_DISPATCH(cfh::fused_core_fwd_kernel);
     if (rc) return rc;
-    hipLaunchKernelGGL(cfh::core_project_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads),
-                       dim3(cfh::WAVE * cfh::PROJ_WAVES), 0, st, hist, wcat, out, (int)N, p->num_heads, L.hw);
+    {
+        TimedScope timed("core_project", st);
+        hipLaunchKernelGGL(cfh::core_project_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads),
+                           dim3(cfh::WAVE * cfh::PROJ_WAVES), 0, st, hist, wcat, out, (int)N, p->num_heads, L.hw);
+    }
     return finish_launch("fused_core_project");
 }
 
@@ -1535,6 +1537,7 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         int per_slice = (int)((N + nslices - 1) / nslices);
         per_slice = (per_slice + 15) & ~15;
         nslices = (int)((N + per_slice - 1) / per_slice);
+        TimedScope timed("core_weight_gradients", st_w);
         hipLaunchKernelGGL(cfh::core_gwcat_kernel, dim3((L.hw / 64 + cfh::GW_WPB - 1) / cfh::GW_WPB, p->num_heads, nslices),
                            dim3(cfh::WAVE * cfh::GW_WPB), 0, st_w, gout,
                            hist, gwcat, (int)N, p->num_heads, L.hw, per_slice);
@@ -1547,10 +1550,12 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
     if (two) rc_w = weight_gradients();
 
     // ---- this stream: Wcat, G = Wcat^T go per item, records, tables, the main kernel, gk and gv
-    if (!buf.wcat_ready)
+    if (!buf.wcat_ready) {
+        TimedScope timed("core_prepare_bwd", st);
         hipLaunchKernelGGL(cfh::core_wcat_kernel, dim3(p->num_heads * cfh::DH), dim3(256), 0, st,
                            cfh::WcatArgs{W_dist, W_axis1, W_axis2, W_axis3, L.hw, p->dist_coef, p->angle_coef,
                                          p->angle_wscale, wcat});
+    }
     // (with records kept from the forward the work queues are all that is left to prepare: gbuild clears them)
     // with the records kept from the forward pass, the same launch lists those that the main kernel is to take first
     cfh::SlowListArgs SL{};
@@ -1567,9 +1572,13 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         C.slow_wgs = slow_wave_count(N, p->num_heads);
         C.slow_flag = cfh::REC_BOX_LISTED_BWD;
     }
-    hipLaunchKernelGGL(cfh::core_gbuild_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads, L.hw / 64), dim3(cfh::WAVE), 0,
-                       st, gout, wcat, G, (int)N, p->num_heads, L.hw, buf.records_ready ? C.K.counters : nullptr, SL);
+    {
+        TimedScope timed("core_gbuild", st);
+        hipLaunchKernelGGL(cfh::core_gbuild_kernel, dim3((unsigned)((N + 15) / 16), p->num_heads, L.hw / 64), dim3(cfh::WAVE), 0,
+                           st, gout, wcat, G, (int)N, p->num_heads, L.hw, buf.records_ready ? C.K.counters : nullptr, SL);
+    }
     if (!buf.records_ready) {
+        TimedScope timed("core_prepare_bwd", st);
         const int threads = (int)(N * p->num_heads > (int64_t)p->num_heads * cfh::NQUEUE ? N * p->num_heads
                                                                                           : p->num_heads * cfh::NQUEUE);
         hipLaunchKernelGGL(cfh::prepare_items_kernel, dim3((threads + 255) / 256), dim3(256), 0, st, C.K, 0);
@@ -1590,8 +1599,11 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         A.N = (int32_t)N; A.H = p->num_heads; A.E = (int32_t)E;
         A.items = C.K.items;
         const int64_t items = N * p->num_heads;
-        hipLaunchKernelGGL(cfh::dpa_bwd_col_kernel, dim3((unsigned)((items + cfh::DPA_WAVES - 1) / cfh::DPA_WAVES)),
-                           dim3(cfh::WAVE * cfh::DPA_WAVES), 0, st, A);
+        {
+            TimedScope timed("core_bwd_col", st);
+            hipLaunchKernelGGL(cfh::dpa_bwd_col_kernel, dim3((unsigned)((items + cfh::DPA_WAVES - 1) / cfh::DPA_WAVES)),
+                               dim3(cfh::WAVE * cfh::DPA_WAVES), 0, st, A);
+        }
         rc = finish_launch("fused_core_backward");
     }
     if (!two && !no_wg) rc_w = weight_gradients();
@@ -1632,6 +1644,7 @@ int cfh_fused_core_weight_gradients(const cfh_params* p, const cfh_core_wgrad_jo
     int cus = device_cus();
     if (cus <= 0) cus = 256;
     const int blocks_per_slice = (hw / 64) * p->num_heads;
+    TimedScope timed("core_weight_gradients", st);
     for (int32_t first = 0; first < njobs; first += cfh::CORE_WG_MAX_JOBS) {
         const int32_t last = njobs < first + cfh::CORE_WG_MAX_JOBS ? njobs : first + cfh::CORE_WG_MAX_JOBS;
         cfh::CoreWgradJobs T{};

@@ -34,6 +34,13 @@ class KernelManager:
     NOISE_SEED_DEVICE: Optional[torch.Tensor] = None
     # options of this implementation (no reference counterpart)
     WINDOW_MODE: int = _lib.CFH_WINDOW_REFERENCE
+    # distance window of the fused attention core (PeriodicAttentionCoreHIP).  Its angle encoding is the untruncated
+    # Gaussian basis whatever this says; with the wide window (11 bins, +-5 sigma: a dropped bin is below 4e-6 of a
+    # basis function's peak) the distance encoding is the untruncated basis as well to within that bound, i.e. the
+    # core computes the reference's pure-PyTorch formulation
+    # (models/indexed_lattice_multi_head_attention.py:580-588), which is what its results are held to (1e-4).
+    # CFH_WINDOW_REFERENCE: the 9-bin window of the reference's CUDA kernels (+-4 sigma, dropped bin up to e^-8).
+    CORE_WINDOW_MODE: int = _lib.CFH_WINDOW_WIDE
     # skip translations lighter than 2^-24 of their pair's heaviest: below the float32 resolution of the
     # normalised sum (measured on 256 crystals: every output within 1e-6 of the unpruned result); 0 keeps all
     PRUNE_LOG2: float = 24.0
@@ -664,7 +671,7 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
     (the reference's sequence, models/indexed_lattice_multi_head_attention_cuda.py:589-734 and :144-185), computed
     with one histogram per (atom, head) instead of one per (pair, head): psi (E,H,Dh) is never formed.  The angle
     encoding uses the full Gaussian basis (no +-4 sigma window; a 5-term series around the nearest bin), the
-    distance encoding the window of ``KernelManager.WINDOW_MODE``.  No counterpart class in the reference."""
+    distance encoding the window of ``KernelManager.CORE_WINDOW_MODE``.  No counterpart class in the reference."""
 
     @staticmethod
     def supported(K, dim_angle_enc, wscale, angle_wscale, W_k, W_k1) -> bool:
@@ -697,6 +704,7 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
         _require_complete_blocks(edge_ij_e, e_start, N)
         p = _params(H, Dh, int(K), A, cos_abs, float(dist_max), wscale, value_pe_angle_scale, length_rbf_mul,
                     angle_rbf_mul, cutoff_radius if rv is not None else None)
+        p.window_mode = int(KernelManager.CORE_WINDOW_MODE)
         hw = int(lib.cfh_fused_core_hist_words(ctypes.byref(p)))
         if hw <= 0:
             _lib.check(-1, "cfh_fused_core_hist_words")

@@ -32,6 +32,7 @@ def attention_layer(x, sd: Dict[str, torch.Tensor], prefix: str, geo, lp, *, win
     k = F.linear(x, w("k_proj_weight"), b[kdim:2 * kdim]).view(N, H, -1)
     v = F.linear(x, w("v_proj_weight"), b[2 * kdim:]).view(N, H, -1)
     Dh = q.shape[-1]
+    qs = q / math.sqrt(Dh)          # the query as the attention core takes it
     alpha = (q * w("lattice_pos_weights").view(1, H, Dh)).sum(-1)
     if lp.normalize_gauss:
         gs = gauss_scale if gauss_scale is not None else sd[prefix + "gauss_scale"]
@@ -54,18 +55,17 @@ def attention_layer(x, sd: Dict[str, torch.Tensor], prefix: str, geo, lp, *, win
         if frames_override is not None:
             frames = frames_override
         else:
-            qs = (q / math.sqrt(Dh)).detach()
-            f1, f2m = TO.frame_axes_max_vec(qs, k.detach(), a.detach(), geo["rpos"], geo["tvecs"], geo["batch"],
+            f1, f2m = TO.frame_axes_max_vec(qs.detach(), k.detach(), a.detach(), geo["rpos"], geo["tvecs"], geo["batch"],
                                             geo["edges"], **rng)
             frames = TO.orthonormal_frame(f1, f2m)
     z, psi = TO.framed_pe(a, geo["rpos"], geo["tvecs"], geo["batch"], geo["edges"], W_k, W_ax, frames,
                           K=K, dist_max=dist_max, wscale=lp.value_pe_dist_wscale, A=A if W_ax is not None else 0,
                           angle_wscale=lp.value_pe_angle_wscale, cos_abs=lp.cos_abs,
                           c_dist=lp.value_pe_dist_coef, c_angle=lp.value_pe_angle_coef, windows=windows, **rng)
-    out, _ = TO.softmax_attention(q / math.sqrt(Dh), k, v, z, psi if K > 0 else None, geo["batch"], geo["edges"])
+    out, _ = TO.softmax_attention(qs, k, v, z, psi if K > 0 else None, geo["batch"], geo["edges"])
     out = F.linear(out.reshape(N, -1), w("out_proj.weight"), w("out_proj.bias"))
     if return_aux:
-        return out, dict(a=a, z=z, psi=psi, frames=frames, q=q, k=k, v=v)
+        return out, dict(a=a, z=z, psi=psi, frames=frames, q=q, qs=qs, k=k, v=v)
     return out
 
 

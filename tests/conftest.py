@@ -24,11 +24,14 @@ def pytest_collection_modifyitems(config, items):
 
 @pytest.fixture(params=["fused", "two_step"])
 def core_mode(request):
-    """Runs a model test with both attention cores: the fused one (one histogram per (atom, head); its angle
-    encoding is the untruncated Gaussian basis) and the reference's sequence of operators (33-bin angle windows).
-    Yields the ``windows`` argument that makes the CPU oracle compute the same thing."""
-    from crystalframer_amd import attention
-    saved = attention.FUSED_CORE
+    """Runs a model test with both attention cores: the fused one (one histogram per (atom, head); untruncated
+    angle basis and, in its default mode, a +-5 sigma distance window: the reference's pure-PyTorch formulation
+    with full Gaussian bases) and the reference's sequence of operators (9- and 33-bin windows of its CUDA kernels).
+    Yields the ``windows`` argument that makes the CPU oracle compute what the path is held to."""
+    import crystalframer_amd as cf
+    from crystalframer_amd import attention, _lib
+    saved = attention.FUSED_CORE, cf.KernelManager.CORE_WINDOW_MODE
     attention.FUSED_CORE = request.param == "fused"
-    yield (9, None) if attention.FUSED_CORE else "reference"
-    attention.FUSED_CORE = saved
+    cf.KernelManager.CORE_WINDOW_MODE = _lib.CFH_WINDOW_WIDE
+    yield "full" if attention.FUSED_CORE else "reference"
+    attention.FUSED_CORE, cf.KernelManager.CORE_WINDOW_MODE = saved

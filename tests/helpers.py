@@ -100,3 +100,27 @@ def first_crystals(P, nb):
     S.rvlen, S.W_k, S.W_ax = P.rvlen[:nb], P.W_k, P.W_ax
     S.frames = [f[:n_at] for f in P.frames]
     return S
+
+
+def check_model_gradients(model, leaves, auxes, n_at=None, tol=1e-4, min_checked=20):
+    """Every parameter gradient of ``model`` (GPU) against the float64 leaves of the CPU model, and the gradients
+    of the attention core's operands (scaled query, k, v, Gaussian coefficient) of every layer against the
+    retained gradients of the CPU model's ``auxes``; ``n_at``: the CPU model ran on the first n_at atoms only.
+    Tensor-scale bound ``tol`` and the element-wise bound |x - ref| <= tol |ref| + tol/10 max|ref|."""
+    checked = 0
+    for name, p in model.named_parameters():
+        if p.grad is None:
+            continue
+        g_ref = leaves[name].grad
+        assert g_ref is not None, name
+        assert rel_err(p.grad, g_ref) < tol, (name, rel_err(p.grad, g_ref))
+        assert elem_err(p.grad, g_ref, rtol=tol, atol_frac=tol / 10) <= 1.0, name
+        checked += 1
+    assert checked >= min_checked
+    for li, (layer, aux) in enumerate(zip(model.encoder.layers, auxes)):
+        sink = layer.self_attn.grad_sink
+        for gpu_name, cpu_name in (("q", "qs"), ("k", "k"), ("v", "v"), ("a", "a")):
+            got = sink[gpu_name] if n_at is None else sink[gpu_name][:n_at]
+            ref = aux[cpu_name].grad
+            assert rel_err(got, ref) < tol, (li, gpu_name, rel_err(got, ref))
+            assert elem_err(got, ref, rtol=tol, atol_frac=tol / 10) <= 1.0, (li, gpu_name)

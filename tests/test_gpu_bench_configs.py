@@ -6,7 +6,9 @@
   * C2  256 crystals (log-normal atom counts), one max-frame layer: backward of the lattice sums on the whole
         batch, checked on its first crystals, with the weight gradients on the second stream and without;
   * C3  the 4-layer model at batch 256 (what bench.py times): outputs of the first crystals and the parameter
-        gradients of a loss on those crystals against the CPU model run on those crystals alone.
+        gradients of a loss on those crystals against the CPU model run on those crystals alone; the fused core
+        (the default path, +-5 sigma distance window, untruncated angle basis) against the FULL Gaussian bases of
+        the pure-PyTorch formulation, the two-step operators against the windows of the reference's CUDA kernels.
 
 Tolerances: 1e-4 against the full-basis oracle with the 5-sigma windows, 5e-4 with the reference's own
 4-sigma windows (its truncation, exp(-8) per dropped bin), both also as an ELEMENTWISE bound
@@ -144,6 +146,7 @@ def test_c3_four_layer_model_at_batch_256_against_cpu_model_on_first_crystals(co
     target = torch.linspace(-1, 1, nb, device=dev())[:, None]
     for layer in model.encoder.layers:
         layer.self_attn.frame_sink = []
+        layer.self_attn.grad_sink = {}
     for _ in range(2):      # the first training pass measures and stores the normalisation of alpha
         model.zero_grad(set_to_none=True)
         for layer in model.encoder.layers:
@@ -158,15 +161,15 @@ def test_c3_four_layer_model_at_batch_256_against_cpu_model_on_first_crystals(co
     frames = [[f.detach().cpu().double()[:n_at] for f in layer.self_attn.frame_sink[0]]
               for layer in model.encoder.layers]
     sub = synthetic.CrystalBatch(cb.x[:n_at], cb.pos[:n_at], cb.batch[:n_at], cb.trans_vec[:nb], cb.sizes[:nb])
-    ref = cpu_model.model_forward(leaves, sub, mp, dtype=torch.float64, frames_per_layer=frames, windows=core_mode)
+    ref, auxes = cpu_model.model_forward(leaves, sub, mp, dtype=torch.float64, frames_per_layer=frames,
+                                         windows=core_mode, return_aux=True)
+    for aux in auxes:
+        for n in ("qs", "k", "v", "a"):
+            aux[n].retain_grad()
     torch.nn.functional.mse_loss(ref, target.cpu().double()).backward()
-    assert Hh.rel_err(out[:nb], ref) < 1e-4
-    checked = 0
-    for name, p in model.named_parameters():
-        if p.grad is None:
-            continue
-        g_ref = leaves[name].grad
-        assert g_ref is not None, name
-        assert Hh.rel_err(p.grad, g_ref) < 2e-4, name
-        checked += 1
-    assert checked >= 40
+    assert Hh.rel_err(out[:nb], ref) < 1e-4 and Hh.elem_err(out[:nb], ref, rtol=1e-4, atol_frac=1e-5) <= 1.0
+    # every parameter gradient and, per layer, the gradients of the attention core's operands: 1e-4, element-wise too
+    Hh.check_model_gradients(model, leaves, auxes, n_at=n_at, tol=1e-4, min_checked=40)
+    for layer in model.encoder.layers:          # atoms outside the 12 crystals: no upstream gradient, no gradient
+        for n in ("q", "k", "v", "a"):
+            assert float(layer.self_attn.grad_sink[n][n_at:].abs().max()) == 0.0

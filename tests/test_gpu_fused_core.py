@@ -2,7 +2,8 @@
 float64 oracle composition  TO.framed_pe -> TO.softmax_attention  (autograd for every gradient), and against the
 two-step operators of the library.  The fused core sums the same translation sets and uses the same distance
 windows as the two-step path; its angle encoding is the FULL Gaussian basis (a 5-term series around the nearest
-bin), so the oracle runs with windows = (9, None): 9-bin distance window, untruncated angle basis.
+bin), so the oracle runs with windows = (9, None): 9-bin distance window (KernelManager.CORE_WINDOW_MODE = 0 in
+this file; the default is the 11-bin window), untruncated angle basis.
 
 Tolerances (relative to the largest magnitude of the tensor): 2e-5 forward, 1e-4 gradients."""
 import math
@@ -22,10 +23,11 @@ CUT = -3.5
 def _defaults():
     import crystalframer_amd as cf
     KM = cf.KernelManager
-    names = ("SYMM_BREAK_NOISE", "PRUNE_LOG2", "WINDOW_MODE", "GRAD_COEF_QUIRK", "LATTICE_RANGE", "MINIMUM_RANGE",
-             "SAVE_HISTOGRAMS", "SECOND_STREAM", "NOISE_SEED", "NOISE_SEED_DEVICE")
+    names = ("SYMM_BREAK_NOISE", "PRUNE_LOG2", "WINDOW_MODE", "CORE_WINDOW_MODE", "GRAD_COEF_QUIRK", "LATTICE_RANGE",
+             "MINIMUM_RANGE", "SAVE_HISTOGRAMS", "SECOND_STREAM", "NOISE_SEED", "NOISE_SEED_DEVICE")
     saved = {n: getattr(KM, n) for n in names}
     KM.SYMM_BREAK_NOISE, KM.PRUNE_LOG2, KM.WINDOW_MODE, KM.GRAD_COEF_QUIRK = 0.0, 24.0, 0, False
+    KM.CORE_WINDOW_MODE = 0        # 9-bin distance window unless a test says otherwise (oracle: windows=(9, None))
     KM.LATTICE_RANGE, KM.MINIMUM_RANGE = 2, 2
     yield
     for n, v in saved.items():
@@ -116,7 +118,7 @@ def test_fused_core_distance_encoding_only():
 
 def test_fused_core_fixed_box_and_wide_distance_window():
     import crystalframer_amd as cf
-    cf.KernelManager.WINDOW_MODE = 1
+    cf.KernelManager.CORE_WINDOW_MODE = 1
     P = Hh.make_problem(num_crystals=8, atoms_hi=5, seed=213)
     out, _, leaves = run_core(P, cutoff=None)
     oo, oleaves = oracle_core(P, cutoff=None, wl=11)
@@ -188,7 +190,7 @@ def test_fused_core_with_frame_search_equals_two_step_path():
     bit for bit, and out equals the two-step operators with those frames up to the truncation of their angle
     windows (5-sigma windows: 1e-4)."""
     import crystalframer_amd as cf
-    cf.KernelManager.WINDOW_MODE = 1
+    cf.KernelManager.WINDOW_MODE = cf.KernelManager.CORE_WINDOW_MODE = 1
     P = Hh.make_problem(num_crystals=12, atoms_hi=6, seed=83)
     out, fr, leaves = run_core(P, frames="search")
     ref_fr = cf.ComputeFramesMaximumMethodCUDA.apply(g(P.q), g(P.k), None, g(P.a), g(P.rpos), None, g(P.tvecs),

@@ -8,7 +8,7 @@ columns.
 Oracle: the scalar C port in float64 for z, psi and their backward (the tensor oracle needs minutes and tens of
 GB at these sizes), composed with the float64 softmax attention of the tensor oracle, whose autograd gives the
 gradients of q, k, v and the upstream gradients (gz, gpsi) of the C port's backward.  The frames are those the
-call itself searched.  Windows as the core computes them: the distance window of KernelManager.WINDOW_MODE,
+call itself searched.  Windows as the core computes them: the distance window of KernelManager.CORE_WINDOW_MODE,
 the angle basis untruncated (C port: angle_range = 0).
 
 Tolerances (relative to the tensor's largest magnitude): forward 2e-5, gradients 1e-4; element-wise bound too."""
@@ -28,7 +28,7 @@ CUT = -3.5
 def _defaults():
     import crystalframer_amd as cf
     KM = cf.KernelManager
-    names = ("SYMM_BREAK_NOISE", "PRUNE_LOG2", "WINDOW_MODE", "GRAD_COEF_QUIRK", "LATTICE_RANGE", "MINIMUM_RANGE",
+    names = ("SYMM_BREAK_NOISE", "PRUNE_LOG2", "CORE_WINDOW_MODE", "GRAD_COEF_QUIRK", "LATTICE_RANGE", "MINIMUM_RANGE",
              "NOISE_SEED", "NOISE_SEED_DEVICE")
     saved = {n: getattr(KM, n) for n in names}
     KM.SYMM_BREAK_NOISE, KM.PRUNE_LOG2, KM.GRAD_COEF_QUIRK = 0.0, 24.0, False
@@ -97,7 +97,7 @@ def _gout(N, seed):
 @pytest.mark.parametrize("window_mode,wl", [(0, 9), (1, 11)])
 def test_fused_core_rows_of_66_to_90_pairs(window_mode, wl):
     import crystalframer_amd as cf
-    cf.KernelManager.WINDOW_MODE = window_mode
+    cf.KernelManager.CORE_WINDOW_MODE = window_mode
     P = Hh.make_problem(num_crystals=2, atoms_lo=66, atoms_hi=90, len_lo=8.0, len_hi=14.0, seed=301)
     assert min(P.sizes) > 64
     P.q = P.q * 3.0            # sharper attention: the running maximum moves over the groups of a row
@@ -109,7 +109,7 @@ def test_fused_core_rows_of_66_to_90_pairs(window_mode, wl):
 
 def test_fused_core_row_of_200_pairs():
     import crystalframer_amd as cf
-    cf.KernelManager.WINDOW_MODE = 0
+    cf.KernelManager.CORE_WINDOW_MODE = 0
     P = Hh.make_problem(num_crystals=1, atoms_lo=200, atoms_hi=200, len_lo=14.0, len_hi=18.0, seed=305)
     gout = _gout(P.N, 19)
     out, fr, grads = run_core(P, gout)
@@ -148,7 +148,7 @@ def test_fused_core_large_cell_stress_case_at_full_size():
     float64 oracle, with an upstream gradient that is zero outside that crystal so that the weight gradients can be
     compared too; the backward pass is linear in the upstream gradient over the whole batch; frames orthonormal."""
     import crystalframer_amd as cf
-    cf.KernelManager.WINDOW_MODE = 0
+    cf.KernelManager.CORE_WINDOW_MODE = 0
     P = _large_cell_problem()
     assert len(P.sizes) == 32 and min(P.sizes) >= 40 and max(P.sizes) > 150 and P.E > 300_000
     g1, g2 = _gout(P.N, 43), _gout(P.N, 44)

@@ -19,6 +19,7 @@ def _run(mp, cb, seed=0, passes=1, windows="reference"):
     model = latticeformer.Latticeformer(mp).to(dev)
     for layer in model.encoder.layers:
         layer.self_attn.frame_sink = []
+        layer.self_attn.grad_sink = {}
     target = torch.linspace(-1, 1, cb.num_crystals, device=dev)[:, None]
     for _ in range(passes):
         # the first training-mode pass measures and stores the normalisation of alpha with framework
@@ -35,9 +36,14 @@ def _run(mp, cb, seed=0, passes=1, windows="reference"):
     frames = None
     if mp.value_pe_angle_real > 0:
         frames = [[f.detach().cpu().double() for f in layer.self_attn.frame_sink[0]] for layer in model.encoder.layers]
-    ref = cpu_model.model_forward(leaves, cb, mp, dtype=torch.float64, frames_per_layer=frames, windows=windows)
+    ref, auxes = cpu_model.model_forward(leaves, cb, mp, dtype=torch.float64, frames_per_layer=frames, windows=windows,
+                                         return_aux=True)
+    for aux in auxes:
+        for n in ("qs", "k", "v", "a"):
+            aux[n].retain_grad()
     ref_loss = torch.nn.functional.mse_loss(ref, target.cpu().double())
     ref_loss.backward()
+    model.oracle_auxes = auxes
     return model, out, ref, leaves
 
 
@@ -49,15 +55,7 @@ def test_model_forward_backward_matches_cpu_oracle(angle_bins, passes, core_mode
                               ang_lo=65.0, ang_hi=115.0, seed=11)
     model, out, ref, leaves = _run(mp, cb, passes=passes, windows=core_mode)
     assert Hh.rel_err(out, ref) < 1e-4
-    checked = 0
-    for name, p in model.named_parameters():
-        if p.grad is None:
-            continue
-        g_ref = leaves[name].grad
-        assert g_ref is not None, name
-        assert Hh.rel_err(p.grad, g_ref) < 2e-4, name
-        checked += 1
-    assert checked >= 20
+    Hh.check_model_gradients(model, leaves, model.oracle_auxes, tol=1e-4, min_checked=20)
     # the first training-mode forward stored the normalisation of alpha
     for layer in model.encoder.layers:
         assert float(layer.self_attn.gauss_scale[0]) > 0
@@ -146,8 +144,15 @@ def test_training_step_as_hip_graph_matches_eager_on_every_replay():
             assert abs(le - lg) < 2e-4 * abs(le), (replay, le, lg)
             junk = torch.tanh(junk @ junk / 512.0)          # eager work between the replays
             assert torch.isfinite(junk).all()
+        # The two twins are not bit-equal: the weight gradients of the linear layers are summed with float atomics, and
+        # AdamW's first steps move every element by about lr whatever the size of its gradient, so an element whose
+        # tiny gradient differs in the last bits (or in sign) drifts by up to 2 lr per step.  Bound: two such steps
+        # for any element, a hundredth of a step on average.
+        lr = 1e-3
         for (n, pe), (_, pg) in zip(model_e.named_parameters(), model_g.named_parameters()):
-            assert Hh.rel_err(pg, pe.detach().cpu()) < 5e-3, n
+            diff = (pg.detach() - pe.detach()).abs()
+            assert float(diff.max()) <= 4 * lr, n
+            assert float(diff.mean()) <= 0.02 * lr, n
     finally:
         KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE = saved
 
