@@ -44,8 +44,9 @@ __global__ __launch_bounds__(256) void adamw_batch_kernel(const AdamWJobs T) {
     }
     const AdamWJob J = T.job[lo];
     const float t = (float)(*T.step + 1ULL);
-    const float bc1 = 1.0f - exp2f(t * log2f(T.beta1));
-    const float bc2 = 1.0f - exp2f(t * log2f(T.beta2));
+    // 1 - beta^t in double: for beta close to 1 and the first steps the float form cancels (1 - 0.999 has three digits)
+    const float bc1 = (float)(-expm1((double)t * log((double)T.beta1)));
+    const float bc2 = (float)(-expm1((double)t * log((double)T.beta2)));
     const float step_size = T.lr / bc1;
     const float inv_sqrt_bc2 = rsqrtf(bc2);
     const float decay = 1.0f - T.lr * T.wd;

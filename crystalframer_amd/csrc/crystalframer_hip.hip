@@ -1380,6 +1380,7 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     cfh::CoreArgs C;
     std::memset(&C, 0, sizeof(C));
     fill_common(C.K, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
+    C.K.contiguous_neighbours = 1;
     const CoreBuffers buf = fill_core(C, p, L, qs, k, v, rvlen != nullptr, cache, workspace);
     const bool search = has_ang && search_frames != 0;
     if (buf.table && !buf.table_ready) {
@@ -1505,6 +1506,7 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
     cfh::CoreArgs C;
     std::memset(&C, 0, sizeof(C));
     fill_common(C.K, p, a_ih, rpos, tvecs, rvlen, batch, edges, e_start, order, N, E, workspace);
+    C.K.contiguous_neighbours = 1;
     const CoreBuffers buf = fill_core(C, p, L, qs, k, v, rvlen != nullptr, cache, workspace);
     float* wcat = buf.wcat;
     C.K.frames = has_ang ? frames : nullptr;

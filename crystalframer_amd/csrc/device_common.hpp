@@ -360,13 +360,16 @@ struct KernelArgs {
     int32_t* counters2;           // optional second set, cleared along with the first: for a second kernel that
                                   // works through the same item records without a prepare launch of its own
     int32_t frames_to_records;    // frame search: also store the orthonormal frames into the item records
+    int32_t contiguous_neighbours;      // the kernels of this launch take the neighbours of an atom as j0, j0 + 1, ... (the
+                                        // complete n x n block per crystal, sorted by i then j): the record step checks it
     uint32_t* items;              // (N, H, REC_WORDS) item records of this launch
     int32_t* slow_count;          // optional: per block of 256 records, how many of them are listed in slow_list
     int32_t* slow_list;           // (blocks, SLOW_PREP_SLOTS) records whose box is not the usual one, for the launches that
                                   // follow to take first
     int32_t slow_R;               // half-width of the usual box
     unsigned long long* stats;    // optional running totals (see STAT_* below); never reset by a launch
-    int32_t* status;              // word of the workspace header: set to 1 when a box was cut back to RMAX (never cleared)
+    int32_t* status;              // word of the workspace header (bits, never cleared): 1 a box was cut back to RMAX;
+                                  // 2 the pairs of an atom are not the consecutive neighbours j0, j0 + 1, ...
     int32_t N, E, H;
     uint32_t h_magic; int32_t h_shift;      // n / H for 0 <= n < 2^31 as (n * h_magic) >> (32 + h_shift); h_magic 0: H = 1
     float cutoff_radius; int32_t lattice_range, minimum_range;
@@ -509,7 +512,7 @@ __device__ __forceinline__ void prepare_items_block(const KernelArgs& P, int wit
         float rvl1 = 0.f, rvl2 = 0.f, rvl3 = 0.f;
         if (P.rvlen) { rvl1 = P.rvlen[(size_t)b * 3 + 0]; rvl2 = P.rvlen[(size_t)b * 3 + 1]; rvl3 = P.rvlen[(size_t)b * 3 + 2]; }
         const Box bx = translation_box(a, rvl1, rvl2, rvl3, P.cutoff_radius, P.lattice_range, P.minimum_range);
-        if (bx.over && P.status) *P.status = 1;
+        if (bx.over && P.status) atomicOr(P.status, 1);
         const int e0 = (int)P.e_start[i];
         rec[REC_ATOM] = (uint32_t)i;
         rec[REC_E0] = (uint32_t)e0;
@@ -518,7 +521,18 @@ __device__ __forceinline__ void prepare_items_block(const KernelArgs& P, int wit
         slow = P.slow_count != nullptr && !(bx.R1 == P.slow_R && bx.R2 == P.slow_R && bx.R3 == P.slow_R);
         rec[REC_A] = __float_as_uint(a);
         for (int d = 0; d < 9; d++) rec[REC_LATTICE + d] = __float_as_uint(P.tvecs[(size_t)b * 9 + d]);
-        rec[30] = (uint32_t)(P.e_start[i + 1] > e0 ? (int)P.edges[(size_t)P.E + e0] : i);      // first neighbour atom
+        int j0 = P.e_start[i + 1] > e0 ? (int)P.edges[(size_t)P.E + e0] : i;      // first neighbour atom
+        if (P.contiguous_neighbours) {
+            // a layout other than whole n x n blocks would make the kernels read other atoms than the pairs name, or
+            // past the last atom: say so in the status word and keep every read inside the arrays
+            const int np = (int)P.e_start[i + 1] - e0;
+            const bool bad = j0 < 0 || j0 + np > P.N || (np > 0 && (int)P.edges[(size_t)P.E + e0 + np - 1] != j0 + np - 1);
+            if (bad) {
+                if (P.status) atomicOr(P.status, 2);
+                j0 = max(0, min(j0, P.N - np));
+            }
+        }
+        rec[30] = (uint32_t)j0;
         rec[31] = (uint32_t)b;                                                                  // crystal
         if (with_query) {
             for (int c = 0; c < DH; c++) rec[REC_QUERY + c] = __float_as_uint(P.q[((size_t)i * P.H + h) * DH + c]);

@@ -114,3 +114,25 @@ class Latticeformer(nn.Module):
         x = _run_head(self.proj_before_pooling, x)
         x = self.pooling_layer(x, data.batch, data.sizes)
         return _run_head(self.mlp, x)
+
+
+def load_reference_checkpoint(model: Latticeformer, state_dict, prefix: str = "swa_model.module.",
+                              fold_target_statistics: bool = True) -> Latticeformer:
+    """Load the weights of a checkpoint written by the reference's trainer into ``model``, the way the reference's
+    demo does (demo.py:67-88): ``state_dict`` is the checkpoint's ``"state_dict"`` entry (read it with
+    ``torch.load(path, weights_only=True)["state_dict"]``); the entries of the averaged model carry ``prefix``, which
+    is stripped; the load is strict, i.e. every parameter name and shape must match (they are the reference's).
+    With ``fold_target_statistics`` the checkpoint's ``target_std`` / ``target_mean`` are folded into the last linear
+    layer so that the model predicts in the target's units."""
+    own = {key[len(prefix):]: value for key, value in state_dict.items() if key.startswith(prefix)}
+    if not own:
+        raise KeyError(f"no entry of the checkpoint starts with {prefix!r}")
+    model.load_state_dict(own)
+    if fold_target_statistics and "target_std" in state_dict and "target_mean" in state_dict:
+        last = model.mlp[-1]
+        std = state_dict["target_std"].to(last.weight.device, last.weight.dtype)
+        mean = state_dict["target_mean"].to(last.weight.device, last.weight.dtype)
+        with torch.no_grad():
+            last.weight.mul_(std[:, None])
+            last.bias.mul_(std).add_(mean)
+    return model

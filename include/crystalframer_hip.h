@@ -135,9 +135,11 @@ int cfh_timing_read(const char* what, double* total_ms, int64_t* launches);
 
 /* Bytes of device scratch the four entry points below need for (N atoms, E pairs).  The first 512 bytes of
  * a workspace are a header that the caller zeroes once: bytes 0..7 the snapshot of the noise seed, the int32
- * at byte 16 a status word that a launch sets to 1 when the box rule asked for a half-width beyond 32 (the
- * largest the kernels sum; the box was cut back and the result differs from the reference's), bytes 256..511
- * the statistics of collect_stats.  Launches never clear the status word. */
+ * at byte 16 a status word of flag bits that launches set and never clear: 1 when the box rule asked for a
+ * half-width beyond 32 (the largest the kernels sum; the box was cut back and the result differs from the
+ * reference's), 2 when a call of the fused core found pairs that are not the complete n x n block of every crystal
+ * sorted by i then j (every read stays inside the arrays, the results are meaningless); bytes 256..511 the
+ * statistics of collect_stats. */
 size_t cfh_workspace_bytes(const cfh_params* p, int64_t N, int64_t E);
 
 /*

@@ -355,3 +355,34 @@ def test_workspace_header_survives_a_backward_pass():
     assert 0 < st["bwd_evaluated"] <= st["bwd_in_box"] == st["fwd_in_box"]
     for name in ("Wk", "W1", "W2", "W3"):
         assert leaves[name].grad is not None and float(leaves[name].grad.abs().max()) > 0
+
+
+def test_fused_core_reports_pairs_that_are_not_whole_blocks():
+    """A caller of the C ABI that hands over another pair layout than the complete n x n block per crystal (here: the
+    neighbours of every atom in descending order, declared complete to get past the Python check): the call sets bit 2
+    of the workspace's status word, reads inside the arrays and returns finite numbers; with the right layout the bit
+    stays clear."""
+    from crystalframer_amd import _lib, cuda_funcs as F
+    P = Hh.make_problem(num_crystals=6, atoms_lo=2, atoms_hi=5, seed=47)
+    _lib.read_status(dev(), reset=True)
+    out, _, _ = run_core(P, need_grad=False)
+    torch.cuda.synchronize()
+    assert _lib.read_status(dev(), reset=True) & 2 == 0
+    # reverse the neighbours within every row
+    e_dev = P.edges.to(dev())
+    rows = torch.bincount(P.edges[0], minlength=P.N)
+    start = torch.cumsum(rows, 0) - rows
+    pos_in_row = torch.arange(P.E) - start[P.edges[0]]
+    perm = start[P.edges[0]] + rows[P.edges[0]] - 1 - pos_in_row
+    Q = Hh.Problem()
+    Q.__dict__.update(P.__dict__)
+    Q.edges, Q.rpos = P.edges[:, perm].contiguous(), P.rpos[perm].contiguous()
+    edges_dev = Q.edges.to(dev())
+    F.declare_complete_blocks(edges_dev)
+    leaves = [g(t) for t in (Q.q, Q.k, Q.v, Q.a)]
+    out2, _ = F.PeriodicAttentionCoreHIP.apply(
+        *leaves, g(Q.rpos), g(Q.tvecs), Q.batch.to(dev()), edges_dev, 64, Hh.DIST_MAX, 1.0, g(Q.W_k), g(Q.W_ax[0]),
+        g(Q.W_ax[1]), g(Q.W_ax[2]), 64, 4.0, 0, 1.0, 1.0, g(Q.rvlen), CUT, torch.stack([g(f) for f in Q.frames], 0))
+    torch.cuda.synchronize()
+    assert _lib.read_status(dev(), reset=True) & 2 == 2
+    assert torch.isfinite(out2).all()

@@ -37,13 +37,16 @@ def _grads(params, step, seed=100):
         p.grad = (torch.randn(p.shape, generator=gen) * (0.1 + k)).to(p.device)
 
 
+@pytest.mark.parametrize("betas", [(0.9, 0.98), (0.9, 0.999)])
 @pytest.mark.parametrize("wd", [0.0, 1e-2])
-def test_adamw_matches_torch(wd):
+def test_adamw_matches_torch(wd, betas):
+    """(0.9, 0.999), the default of both optimizers: 1 - beta2^t cancels in float32 during the first steps, so the
+    kernel makes the bias corrections in double, as the framework does on the host."""
     from crystalframer_amd import optim
     dev = torch.device("cuda:0")
     mine, ref = _twin(dev), _twin(dev)
-    o1 = optim.AdamW(mine, lr=3e-3, betas=(0.9, 0.98), eps=1e-8, weight_decay=wd)
-    o2 = torch.optim.AdamW(ref, lr=3e-3, betas=(0.9, 0.98), eps=1e-8, weight_decay=wd)
+    o1 = optim.AdamW(mine, lr=3e-3, betas=betas, eps=1e-8, weight_decay=wd)
+    o2 = torch.optim.AdamW(ref, lr=3e-3, betas=betas, eps=1e-8, weight_decay=wd)
     for step in range(6):
         _grads(mine, step); _grads(ref, step)
         before = mine[3].detach().clone()
@@ -58,7 +61,7 @@ def test_adamw_matches_torch(wd):
     assert torch.equal(mine[-1], torch.ones(5, device=dev))
     # the moments are visible under torch's names and survive a round trip through state_dict
     sd = o1.state_dict()
-    o3 = optim.AdamW(mine, lr=3e-3, betas=(0.9, 0.98), eps=1e-8, weight_decay=wd)
+    o3 = optim.AdamW(mine, lr=3e-3, betas=betas, eps=1e-8, weight_decay=wd)
     o3.load_state_dict(sd)
     assert torch.equal(o3.state[mine[0]]["exp_avg"], o1.state[mine[0]]["exp_avg"])
     assert int(o3.state[mine[0]]["step"]) == 6

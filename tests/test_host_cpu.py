@@ -127,6 +127,48 @@ def test_model_has_reference_parameter_names_and_count():
     assert lp.scale_real == 1.4 and lp.layer_index == 2 and lp.cos_abs == 0 and lp.value_pe_angle_real == 64
 
 
+def test_a_reference_checkpoint_loads_strictly():
+    """The names and shapes below are what the reference's modules register for its default configuration
+    (models/latticeformer.py:113,189; models/indexed_latticeformer_encoder.py:796-804;
+    models/indexed_lattice_multi_head_attention_cuda.py:1042-1098), under the prefix its trainer's averaged model
+    gives them (demo.py:75-79), next to entries a checkpoint also holds and the loader must ignore."""
+    from crystalframer_amd import latticeformer
+    gen = torch.Generator().manual_seed(5)
+    shapes = {"input_embeddings.weight": (128, 98), "mlp.0.weight": (128, 128), "mlp.0.bias": (128,),
+              "mlp.3.weight": (1, 128), "mlp.3.bias": (1,)}
+    for li in range(4):
+        pre = f"encoder.layers.{li}."
+        shapes.update({pre + "linear1.weight": (512, 128), pre + "linear1.bias": (512,),
+                       pre + "linear2.weight": (128, 512), pre + "linear2.bias": (128,)})
+        at = pre + "self_attn."
+        shapes.update({at + "gauss_scale": (2,), at + "atten_scale": (1,), at + "q_proj_weight": (128, 128),
+                       at + "k_proj_weight": (128, 128), at + "v_proj_weight": (128, 128), at + "in_proj_bias": (384,),
+                       at + "out_proj.weight": (128, 128), at + "out_proj.bias": (128,),
+                       at + "lattice_pos_weights": (128,), at + "pe_dist_proj": (1, 8, 16, 64),
+                       at + "proj_angle1": (1, 8, 16, 64), at + "proj_angle2": (1, 8, 16, 64),
+                       at + "proj_angle3": (1, 8, 16, 64)})
+    ckpt = {"swa_model.module." + k: torch.randn(v, generator=gen) for k, v in shapes.items()}
+    ckpt.update({"model." + k: torch.zeros(v) for k, v in shapes.items()})
+    ckpt["swa_model.n_averaged"] = torch.tensor(7)
+    ckpt["target_std"], ckpt["target_mean"] = torch.tensor([2.5]), torch.tensor([-0.75])
+    model = latticeformer.Latticeformer(params.ModelParams())
+    assert set(model.state_dict()) == set(shapes)
+    latticeformer.load_reference_checkpoint(model, ckpt)
+    sd = model.state_dict()
+    for k in shapes:
+        if k.startswith("mlp.3"):
+            continue
+        assert torch.equal(sd[k], ckpt["swa_model.module." + k]), k
+    assert torch.allclose(sd["mlp.3.weight"], ckpt["swa_model.module.mlp.3.weight"] * 2.5)
+    assert torch.allclose(sd["mlp.3.bias"], ckpt["swa_model.module.mlp.3.bias"] * 2.5 - 0.75)
+    # the three input projections are re-packed into one storage on first use without changing what was loaded
+    at = model.encoder.layers[2].self_attn
+    at._stacked_in_proj()
+    assert torch.equal(at.k_proj_weight, ckpt["swa_model.module.encoder.layers.2.self_attn.k_proj_weight"])
+    with pytest.raises(KeyError):
+        latticeformer.load_reference_checkpoint(model, {"model.x": torch.zeros(1)})
+
+
 def test_vectorised_frame_oracle_matches_loop_oracle():
     import helpers as Hh
     P = Hh.make_problem(num_crystals=5, atoms_hi=4, seed=71)
