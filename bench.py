@@ -210,7 +210,7 @@ def instrumented(fn, nprof: int, dev, count_terms: bool = True):
     return kern_ms, kern_launches, stats, calls
 
 
-def lattice_roofline(kern_ms, kern_launches, stats, angle: bool, items_per_launch: int):
+def lattice_roofline(kern_ms, kern_launches, stats, angle: bool, items_per_launch: int, angle_bins: int = 64):
     """Per pass (all layers of one step), forward and backward: algorithmic flop over the SUM of the durations of
     every kernel that executes part of that work, each measured by the library with HIP events on its launch stream.
     Algorithmic flop = the per-term counts above x the terms actually evaluated, 87 flop per candidate the frame
@@ -221,6 +221,10 @@ def lattice_roofline(kern_ms, kern_launches, stats, angle: bool, items_per_launc
     fused = "fused_core_forward" in kern_ms
     kind = "fused" if fused else "two_step"
     f_fwd, f_bwd, epi = (F_FWD, F_BWD, EPI_FWD) if angle else (F_FWD_DIST, F_BWD_DIST, EPI_FWD_DIST)
+    if angle and angle_bins == 16:      # the whole 16-bin basis per axis instead of a 33-bin window
+        f_fwd, f_bwd, epi = 56 + 4 * WL + 12 * 16, 61 + 6 * WL + 18 * 16, 2 * 16 * (64 + 3 * 16)
+    if not angle:
+        angle_bins = 0
     out = {}
     for path, (ev, pairs) in (("forward", ("fwd_evaluated", "fwd_pairs")), ("backward", ("bwd_evaluated", "bwd_pairs"))):
         names = [k for k in PATHS[path][kind] if k in kern_ms]
@@ -240,7 +244,7 @@ def lattice_roofline(kern_ms, kern_launches, stats, angle: bool, items_per_launc
         # per (atom, head) over its histogram of hw words (64 distance bins + 3 axes x 5 moments x 64 bins)
         flop_epi_reference = stats[pairs] * epi * passes
         if fused:
-            hw = 1024 if angle else 64
+            hw = {64: 1024, 16: 128}.get(angle_bins, 64)
             flop_epi = items_per_launch * n * 2 * 16 * hw * passes
         else:
             flop_epi = flop_epi_reference
@@ -258,12 +262,12 @@ def lattice_roofline(kern_ms, kern_launches, stats, angle: bool, items_per_launc
     return out
 
 
-def other_config(name: str, dev, *, layers: int, backward: bool, angle_bins: int, steps: int):
+def other_config(name: str, dev, *, layers: int, backward: bool, angle_bins: int, steps: int, **model_kw):
     """One of the large configurations beside the headline one: the step as one HIP graph, timed by the host clock
     around ``steps`` replays; then the lattice kernels' own durations and term counts from instrumented eager runs."""
     from crystalframer_amd import latticeformer, params, synthetic
     torch.manual_seed(11)
-    mp = params.ModelParams(num_layers=layers, value_pe_angle_real=angle_bins)
+    mp = params.ModelParams(num_layers=layers, value_pe_angle_real=angle_bins, **model_kw)
     model = latticeformer.Latticeformer(mp).to(dev)
     cb_cpu = synthetic.make_config(name, seed=123)
     cb = cb_cpu.to(dev)
@@ -288,7 +292,7 @@ def other_config(name: str, dev, *, layers: int, backward: bool, angle_bins: int
     run = graphed(fn, 2)
     sec = timed(run, steps)
     kern_ms, kern_launches, stats, _ = instrumented(fn, 2, dev)
-    roof = lattice_roofline(kern_ms, kern_launches, stats, angle_bins > 0, int(cb_cpu.pos.shape[0]) * mp.head_num)
+    roof = lattice_roofline(kern_ms, kern_launches, stats, angle_bins > 0, int(cb_cpu.pos.shape[0]) * mp.head_num, angle_bins)
     return {"workload": f"{name}: {B} crystals, {int(cb_cpu.pos.shape[0])} atoms, {int((cb_cpu.sizes ** 2).sum())} atom pairs; "
                         f"{layers}-layer max-frame model ({'64 + %d bins' % angle_bins if angle_bins else '64 distance bins, no angle encoding'}), "
                         f"{'forward + backward' if backward else 'forward only'}, one HIP graph per pass",
@@ -511,6 +515,9 @@ def main():
                                                               "instead of the +-5 sigma one (11 bins)",
                                                   "ms": sec9 * 1e3, "crystals_per_s": args.batch / sec9, "steps": args.steps}
             del step9
+        # the reference's lightweight setting (train_jarvis_time.sh:40-57): 16 angle bins, sigma one bin
+        other["C3_lightweight"] = other_config("C3", dev, layers=4, backward=True, angle_bins=16, steps=20,
+                                               value_pe_angle_wscale=1.0, value_pe_dist_coef=1.5, value_pe_angle_coef=6.0)
         other["C2"] = other_config("C2", dev, layers=1, backward=True, angle_bins=64, steps=20)
         other["C4"] = other_config("C4", dev, layers=1, backward=True, angle_bins=64, steps=10)
         other["C5"] = other_config("C5", dev, layers=4, backward=False, angle_bins=64, steps=10)

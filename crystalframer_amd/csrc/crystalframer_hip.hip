@@ -1256,7 +1256,7 @@ struct CoreLayout {
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 CoreLayout core_layout(const cfh_params* p, int64_t N, int64_t E, int64_t B, bool backward) {
     CoreLayout L;
-    L.hw = p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
+    L.hw = cfh::core_hist_words(p->angle_bins);
     size_t off = COUNTER_BYTES;
     L.items = off; off += items_bytes(N > 0 ? N : 1, p->num_heads);
     L.sorted = off; off += align256((size_t)(B > 0 ? B : 1) * cfh::FC_TCAP * sizeof(float4));
@@ -1285,9 +1285,11 @@ int check_core_params(const cfh_params* p) {
     if (p->dist_bins != cfh::NBINS) return fail(CFH_EINVAL, "fused core: dist_bins must be %d", cfh::NBINS);
     if (p->dist_wscale != 1.0f) return fail(CFH_EINVAL, "fused core: only dist_wscale 1.0 is compiled");
     if (p->grad_coef_quirk) return fail(CFH_EINVAL, "fused core: grad_coef_quirk is not available (exact gradients only)");
-    if (p->angle_bins > 0 && p->angle_wscale < 3.0f)
-        return fail(CFH_EINVAL, "fused core: angle_wscale %g < 3: the moment expansion of the angle basis (5 terms) "
-                    "is not accurate enough; use the two-step operators", (double)p->angle_wscale);
+    if (p->angle_bins == cfh::NBINS && p->angle_wscale < 3.0f)
+        return fail(CFH_EINVAL, "fused core: angle_wscale %g < 3 with 64 angle bins: the moment expansion of the angle "
+                    "basis (5 terms) is not accurate enough; use the two-step operators", (double)p->angle_wscale);
+    if (p->angle_bins == cfh::SMALL_A && p->angle_wscale < 1.0f)
+        return fail(CFH_EINVAL, "fused core: angle_wscale %g < 1 with 16 angle bins is not compiled", (double)p->angle_wscale);
     return CFH_OK;
 }
 // the kernels' launch-wide arguments that both directions share; buffers of the caller's cache replace the
@@ -1354,7 +1356,7 @@ size_t cfh_fused_core_workspace_bytes(const cfh_params* p, int64_t N, int64_t E,
 
 int32_t cfh_fused_core_hist_words(const cfh_params* p) {
     if (check_core_params(p) != CFH_OK) return 0;
-    return p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
+    return cfh::core_hist_words(p->angle_bins);
 }
 
 int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k, const float* v, const float* a_ih,
@@ -1455,14 +1457,19 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     const char* what = "fused_core_forward";
 #define CFH_CORE_DISPATCH(KERNEL)                                                                         \
     do {                                                                                                  \
-        if (has_ang) {                                                                                    \
-            if (wide) rc = p->cos_abs ? launch_core(KERNEL<11, true, true>, C, st, what)             \
-                                      : launch_core(KERNEL<11, true, false>, C, st, what);           \
-            else rc = p->cos_abs ? launch_core(KERNEL<9, true, true>, C, st, what)                   \
-                                 : launch_core(KERNEL<9, true, false>, C, st, what);                 \
+        if (p->angle_bins == cfh::SMALL_A) {                                                              \
+            if (wide) rc = p->cos_abs ? launch_core(KERNEL<11, cfh::SMALL_A, true>, C, st, what)          \
+                                      : launch_core(KERNEL<11, cfh::SMALL_A, false>, C, st, what);        \
+            else rc = p->cos_abs ? launch_core(KERNEL<9, cfh::SMALL_A, true>, C, st, what)                \
+                                 : launch_core(KERNEL<9, cfh::SMALL_A, false>, C, st, what);              \
+        } else if (has_ang) {                                                                             \
+            if (wide) rc = p->cos_abs ? launch_core(KERNEL<11, cfh::NBINS, true>, C, st, what)            \
+                                      : launch_core(KERNEL<11, cfh::NBINS, false>, C, st, what);          \
+            else rc = p->cos_abs ? launch_core(KERNEL<9, cfh::NBINS, true>, C, st, what)                  \
+                                 : launch_core(KERNEL<9, cfh::NBINS, false>, C, st, what);                \
         } else {                                                                                          \
-            rc = wide ? launch_core(KERNEL<11, false, false>, C, st, what)                           \
-                      : launch_core(KERNEL<9, false, false>, C, st, what);                           \
+            rc = wide ? launch_core(KERNEL<11, 0, false>, C, st, what)                                    \
+                      : launch_core(KERNEL<9, 0, false>, C, st, what);                                    \
         }                                                                                                 \
     } while (0)
     CFH_CORE_DISPATCH(cfh::fused_core_fwd_kernel);
@@ -1490,8 +1497,12 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
     const bool has_ang = p->angle_bins > 0;
     const int per_enc = p->num_heads * cfh::DH * cfh::NBINS;
     if (N == 0) {
+        const int per_axis = p->num_heads * cfh::DH * p->angle_bins;      // (the axes' rows have angle_bins words)
         hipLaunchKernelGGL(cfh::zero_outputs_kernel, dim3((per_enc + 255) / 256), dim3(256), 0, st, per_enc, gW_dist,
-                           gW_axis1, gW_axis2, gW_axis3);
+                           (float*)nullptr, (float*)nullptr, (float*)nullptr);
+        if (per_axis > 0)
+            hipLaunchKernelGGL(cfh::zero_outputs_kernel, dim3((per_axis + 255) / 256), dim3(256), 0, st, per_axis,
+                               (float*)nullptr, gW_axis1, gW_axis2, gW_axis3);
         return finish_launch("zero_outputs");
     }
     if (!qs || !k || !v || !W_dist || !z || !prob || !hist || !out || !gout || !gq || !gk || !gv || !ga || !glogit)
@@ -1620,7 +1631,7 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
 
 size_t cfh_fused_core_weight_gradients_workspace_bytes(const cfh_params* p, int32_t njobs) {
     if (check_core_params(p) != CFH_OK || njobs < 0) return 0;
-    const size_t hw = p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
+    const size_t hw = (size_t)cfh::core_hist_words(p->angle_bins);
     // (behind the header of every workspace of the library: status word, statistics, work queues)
     return COUNTER_BYTES +
            align256((size_t)cfh::CORE_GW_SLICES * p->num_heads * cfh::DH * hw * sizeof(float)) * (size_t)(njobs > 0 ? njobs : 1);
@@ -1632,7 +1643,7 @@ int cfh_fused_core_weight_gradients(const cfh_params* p, const cfh_core_wgrad_jo
     if (rc) return rc;
     if (njobs < 0 || (njobs > 0 && !jobs)) return fail(CFH_EINVAL, "jobs is NULL or njobs negative");
     if (njobs == 0) return CFH_OK;
-    const int hw = p->angle_bins > 0 ? cfh::HW_ANG : cfh::HW_DIST;
+    const int hw = cfh::core_hist_words(p->angle_bins);
     const size_t per_job = align256((size_t)cfh::CORE_GW_SLICES * p->num_heads * cfh::DH * hw * sizeof(float));
     if ((rc = check_workspace(workspace, workspace_bytes, COUNTER_BYTES + per_job * (size_t)njobs))) return rc;
     for (int32_t j = 0; j < njobs; j++) {

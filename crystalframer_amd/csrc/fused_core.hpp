@@ -55,7 +55,14 @@ constexpr int CORE_WPB = 1;                     // wavefronts per workgroup of t
                                                 // the two separate launches
 constexpr int FC_LOGCAP = 64;                   // logits of a row kept in LDS until the row is complete
 constexpr int HW_DIST = NBINS;
-constexpr int HW_ANG = NBINS * (1 + 3 * NORD);  // 1024 words per (atom, head) with the angle encoding
+constexpr int HW_ANG = NBINS * (1 + 3 * NORD);  // 1024 words per (atom, head) with the 64-bin angle encoding
+constexpr int SMALL_A = 16;                     // the 16-bin angle basis (the reference's lightweight setting): sigma is
+                                                // one bin or more, far too wide a step for the moment series, and the
+                                                // basis is small: every image adds its 16 basis values per axis directly
+                                                // (the whole basis, as the reference evaluates it for 16 bins)
+constexpr int HW_ANG16 = 2 * NBINS;             // 64 distance bins + 3 axes x 16 bins, padded to whole 64-word blocks
+// words of an item's histogram for `ang` angle bins (0: distance encoding alone)
+__host__ __device__ constexpr int core_hist_words(int ang) { return ang == NBINS ? HW_ANG : (ang == SMALL_A ? HW_ANG16 : HW_DIST); }
 constexpr int REC_J0 = 30;                      // item record: first neighbour atom (pairs of an atom are j0, j0+1, ...)
 constexpr int REC_CRYSTAL = 31;                 // item record: crystal of the atom
 static_assert(FC_TCAP == (1 << FC_SHIFT) && (FC_GROUP << FC_SHIFT) <= 65536, "list entry is 16 bits");
@@ -209,7 +216,7 @@ __device__ __forceinline__ void build_moment_table(float* dtab, float ws) {
 // wcat (H,16,hw): [0,64) dist_coef W_dist;  64 + (ax NORD + o) 64 + m': angle_coef sum_m W_ax[c,m] D_o(m - m').
 // grid: H*16 blocks (h, c), 256 threads over the words.
 struct WcatArgs {
-    const float* Wd; const float* W1; const float* W2; const float* W3;
+    const float* Wd; const float* W1; const float* W2; const float* W3;      // (H,16,64) and (H,16,A) x 3
     int hw;
     float dist_coef, angle_coef, ws;
     float* wcat;
@@ -222,6 +229,20 @@ __device__ __forceinline__ void core_wcat_block(const WcatArgs& A, int hc) {
     float* __restrict__ wcat = A.wcat;
     __shared__ float row[3][NBINS];
     __shared__ float dtab[NORD * 128];
+    if (hw == HW_ANG16) {
+        // 16-bin basis: the weights themselves behind the distance block, zeros in the padding
+        for (int w = threadIdx.x; w < hw; w += 256) {
+            float val = 0.0f;
+            if (w < HW_DIST) val = dist_coef * Wd[(size_t)hc * NBINS + w];
+            else if (w < HW_DIST + 3 * SMALL_A) {
+                const int u = w - HW_DIST, ax = u / SMALL_A, m = u % SMALL_A;
+                const float* W = ax == 0 ? W1 : (ax == 1 ? W2 : W3);
+                val = angle_coef * W[(size_t)hc * SMALL_A + m];
+            }
+            wcat[(size_t)hc * hw + w] = val;
+        }
+        return;
+    }
     if (hw > HW_DIST) {
         for (int u = threadIdx.x; u < 3 * NBINS; u += 256) {
             const float* W = u < NBINS ? W1 : (u < 2 * NBINS ? W2 : W3);
@@ -263,6 +284,18 @@ __device__ __forceinline__ void core_gw_finish_block(const float* __restrict__ g
     __shared__ float grow[3 * NORD * NBINS];
     const int enc = threadIdx.x >> 6, m = threadIdx.x & 63;
     const float* g = gwcat + (size_t)hc * hw;
+    if (hw == HW_ANG16) {
+        // 16-bin basis: thread (enc, m) sums the slices of its word; the axes' rows have 16 bins
+        if (enc > 0 && m >= SMALL_A) return;
+        float* dst = enc == 0 ? gWd : (enc == 1 ? gW1 : (enc == 2 ? gW2 : gW3));
+        if (!dst) return;
+        const int word = enc == 0 ? m : HW_DIST + (enc - 1) * SMALL_A + m;
+        float sum = 0.0f;
+        for (int sl = 0; sl < nslices; sl++) sum += g[sl * slice_stride + word];      // fixed order
+        float* d = dst + (size_t)hc * (enc == 0 ? NBINS : SMALL_A) + m;
+        *d = (ACC ? *d : 0.0f) + (enc == 0 ? dist_coef : angle_coef) * sum;
+        return;
+    }
     if (hw > HW_DIST) {
         for (int u = threadIdx.x; u < 3 * NORD * NBINS; u += 256) {
             float sum = 0.0f;
@@ -482,12 +515,14 @@ struct CoreFwdShared {
     float pairC[FC_GROUP];       // exp(logit - running max) / S in fixed-point units
     float logit_s[FC_LOGCAP];    // logits of the row (rows of more pairs park them in the probability array)
 };
-template <int WL, bool HAS_ANG, bool COS_ABS>
+template <int WL, int ANG, bool COS_ABS>
+// ANG: angle bins, 0 (distance encoding alone), 64 (moment series) or 16 (basis values added directly)
 // (distance encoding alone: 4.8 KB of LDS per item allow eight wavefronts per SIMD; seven, with 72 registers and
 // nothing spilled, ran faster than eight with 64 and nine spilled)
-__global__ __launch_bounds__(WAVE * CORE_WPB) __attribute__((amdgpu_waves_per_eu(HAS_ANG ? 1 : 7)))
+__global__ __launch_bounds__(WAVE * CORE_WPB) __attribute__((amdgpu_waves_per_eu(ANG > 0 ? 1 : 7)))
 void fused_core_fwd_kernel(const CoreArgs C) {
-    constexpr int HWK = HAS_ANG ? HW_ANG : HW_DIST;
+    constexpr bool HAS_ANG = ANG > 0;
+    constexpr int HWK = core_hist_words(ANG);
     __shared__ CoreFwdShared<HWK> shared[CORE_WPB];
     CoreFwdShared<HWK>& sh = shared[threadIdx.x >> 6];
     float4* const tab = sh.tab;
@@ -650,6 +685,13 @@ void fused_core_fwd_kernel(const CoreArgs C) {
                                 float cs = (dx * f[ax][0] + dy * f[ax][1] + dz * f[ax][2]) * rinv;
                                 if (COS_ABS) cs = fabsf(cs);
                                 const float uu = (cs - bc.ang_mu0) * bc.ang_inv_interval;      // in bin units
+                                if (ANG == SMALL_A) {
+                                    // all 16 basis values, outwards from bin 8 by the two-sided recurrence (sigma >= 1
+                                    // bin: the value at bin 8 is at least e^-32 of the peak, no underflow)
+                                    const WindowSeed sa = window_seed(((float)(SMALL_A / 2) - uu) * bc.ang_step, bc.ang_step, w);
+                                    window_scatter_rn<SMALL_A>(hist + HW_DIST + ax * SMALL_A, sa, bc.ang_cc);
+                                    continue;
+                                }
                                 const float mf = clampf(__builtin_rintf(uu), 0.0f, (float)(NBINS - 1));
                                 const float eps = 2.0f * (uu - mf);
 #ifndef CFH_EXP_NOCONFLICT
@@ -1069,9 +1111,10 @@ struct CoreBwdShared {
     float pairP[FC_GROUP];       // P_ij
     int32_t pairB[FC_GROUP];     // sum_n P_ij p_n bg_n in fixed point
 };
-template <int WL, bool HAS_ANG, bool COS_ABS>
+template <int WL, int ANG, bool COS_ABS>
 __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const CoreArgs C) {
-    constexpr int HWK = HAS_ANG ? HW_ANG : HW_DIST;
+    constexpr bool HAS_ANG = ANG > 0;
+    constexpr int HWK = core_hist_words(ANG);
     __shared__ CoreBwdShared<HWK> shared[CORE_WPB];
     CoreBwdShared<HWK>& sh = shared[threadIdx.x >> 6];
     float4* const tab = sh.tab;
@@ -1205,6 +1248,11 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
                                 float cs = (dx * f[ax][0] + dy * f[ax][1] + dz * f[ax][2]) * rinv;
                                 if (COS_ABS) cs = fabsf(cs);
                                 const float uu = (cs - bc.ang_mu0) * bc.ang_inv_interval;
+                                if (ANG == SMALL_A) {
+                                    const WindowSeed sa = window_seed(((float)(SMALL_A / 2) - uu) * bc.ang_step, bc.ang_step, 1.0f);
+                                    bg += window_gather<SMALL_A>(Gs + HW_DIST + ax * SMALL_A, sa, bc.ang_cc);
+                                    continue;
+                                }
                                 const float mf = clampf(__builtin_rintf(uu), 0.0f, (float)(NBINS - 1));
                                 const float eps = 2.0f * (uu - mf);
                                 const float* gb = Gs + HW_DIST + ax * NORD * NBINS + (int)mf;

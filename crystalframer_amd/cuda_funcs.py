@@ -670,8 +670,9 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
     divided by sqrt(Dh).  Same result as RealEncodingWithMaxFramesFuncHIP followed by FusedDotProductAttentionCUDA
     (the reference's sequence, models/indexed_lattice_multi_head_attention_cuda.py:589-734 and :144-185), computed
     with one histogram per (atom, head) instead of one per (pair, head): psi (E,H,Dh) is never formed.  The angle
-    encoding uses the full Gaussian basis (no +-4 sigma window; a 5-term series around the nearest bin), the
-    distance encoding the window of ``KernelManager.CORE_WINDOW_MODE``.  No counterpart class in the reference."""
+    encoding uses the full Gaussian basis (no +-4 sigma window: 64 bins as a 5-term series around the nearest bin,
+    16 bins by adding all 16 basis values), the distance encoding the window of
+    ``KernelManager.CORE_WINDOW_MODE``.  No counterpart class in the reference."""
 
     @staticmethod
     def supported(K, dim_angle_enc, wscale, angle_wscale, W_k, W_k1) -> bool:
@@ -680,7 +681,9 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
         if W_k.dim() == 4 and W_k.shape[0] != 1:
             return False
         A = int(dim_angle_enc) if W_k1 is not None else 0
-        return A == 0 or (A == 64 and float(angle_wscale) >= 3.0)
+        # 64 angle bins: moment series, accurate for sigma >= 3 bins; 16 bins (the lightweight setting): the whole
+        # basis added directly, sigma >= 1 bin
+        return A == 0 or (A == 64 and float(angle_wscale) >= 3.0) or (A == 16 and float(angle_wscale) >= 1.0)
 
     @staticmethod
     def forward(ctx, qs, k, v, a_ik, rpos_ij_e, tvecs_n, batch_i, edge_ij_e, K, dist_max, wscale, W_k, W_k1, W_k2,

@@ -308,14 +308,19 @@ int cfh_framed_pe_backward_pairwise(const cfh_params* p, const float* a_ih, cons
  * computed differently: because out is linear in psi = W . s, the basis values of all images of all pairs of an
  * atom are scattered, weighted by P_ij p_n, into ONE histogram per (atom, head), which is projected once.
  * psi (E,H,Dh) and the per-pair histograms are never formed.  The distance basis keeps the truncated window of
- * window_mode; the angle basis is the FULL Gaussian basis (no truncation: the pure-PyTorch formulation,
- * models/indexed_lattice_multi_head_attention.py:580-588), evaluated as a 5-term series around the nearest bin
- * (error < 2e-6 of a basis function's peak for angle_wscale 4; angle_wscale < 3 returns CFH_EINVAL).
- * Needs dist_bins = 64, dist_wscale = 1, angle_bins 0 or 64, and the pairs as the complete n x n block of every
- * crystal (cfh_pair_layout_check).  qs = query / sqrt(Dh).
+ * window_mode (CFH_WINDOW_WIDE, +-5 sigma: full-basis results to within 4e-6 of a basis function's peak); the angle
+ * basis is the FULL Gaussian basis (no truncation: the pure-PyTorch formulation,
+ * models/indexed_lattice_multi_head_attention.py:580-588): with 64 bins evaluated as a 5-term series around the
+ * nearest bin (error < 2e-6 of a basis function's peak for angle_wscale 4; angle_wscale < 3 returns CFH_EINVAL), with
+ * 16 bins (the reference's lightweight setting, train_jarvis_time.sh:40-57; angle_wscale >= 1) by adding all 16
+ * basis values of every image, as the reference evaluates that basis.
+ * Needs dist_bins = 64, dist_wscale = 1, angle_bins 0, 16 or 64, and the pairs as the complete n x n block of every
+ * crystal (cfh_pair_layout_check; a call that finds another layout sets bit 2 of the workspace's status word).
+ * qs = query / sqrt(Dh).
  * Results kept for the backward: z (E,H), prob (E,H) = P, hist (H,N,words) the normalised histograms
  * (head-major: the kernels that contract them with the weights read the rows of a head one after the other)
- * (words = cfh_fused_core_hist_words: 64 distance bins, then per axis and order 64 moment bins), out (N,H,Dh).
+ * (words = cfh_fused_core_hist_words: 64 distance bins, then per axis and order 64 moment bins = 1024; with 16
+ * angle bins 64 + 3 x 16 padded to 128), out (N,H,Dh).
  * workspace: cfh_fused_core_workspace_bytes(p, N, E, B, 0).
  *
  * cache (may be NULL, as may every pointer in it): buffers the caller keeps so that later calls need not make

@@ -5,8 +5,8 @@ With 16 bins the reference's window (ANGLE_RANGE = ceil(8 wscale + 1), models/cu
 at most 7 bins out, and its kernels then evaluate the WHOLE basis (the windowed branch needs more than 8,
 models/kernels/real_enc_frame_proj_fwd_angle.cu:154,168-175), for |cos| as well.  The oracles apply the same rule.
 
-Tolerances (relative to the tensor's largest magnitude): forward 2e-5, gradients 5e-5, float32 port of the kernel
-text 5e-5, model output 1e-4 and parameter gradients 2e-4."""
+Tolerances (relative to the tensor's largest magnitude): forward 2e-5, gradients 5e-5 (fused core: 1e-4), float32
+port of the kernel text 5e-5, model output and parameter gradients 1e-4."""
 import pytest
 import torch
 
@@ -100,8 +100,45 @@ def test_sixteen_angle_bins_match_the_port_of_the_kernel_text(cos_abs):
     assert Hh.rel_err(psi, psic) < 5e-5
 
 
-def test_lightweight_model_forward_backward_matches_cpu_model():
-    """Two layers with the lightweight setting against the float64 CPU model, output and every parameter gradient."""
+@pytest.mark.parametrize("cos_abs", [0, 1])
+@pytest.mark.parametrize("wscale,sizes", [(1.0, (1, 6)), (2.0, (1, 6)), (1.0, (20, 40))])
+def test_sixteen_angle_bins_fused_core(cos_abs, wscale, sizes):
+    """The fused attention core with the 16-bin basis (every image adds all 16 basis values per axis into the
+    item's histogram of 64 + 3 x 16 words) against the composition of the float64 oracles, whole angle basis and
+    the core's default +-5 sigma distance window; rows of up to 40 pairs (several groups: the running softmax
+    rescales the histogram) and one-atom crystals."""
+    from crystalframer_amd import cuda_funcs as F
+    P = Hh.make_problem(num_crystals=10 if sizes[1] < 10 else 4, atoms_lo=sizes[0], atoms_hi=sizes[1],
+                        len_lo=3.0 if sizes[1] < 10 else 2.5, len_hi=8.0, seed=150 + cos_abs)
+    if sizes[1] >= 10:
+        P.q = P.q * 4.0
+    W16 = _weights16(P, seed=7)
+    cd, ca = 1.5, 6.0
+    names = ("q", "k", "v", "a", "Wk", "W1", "W2", "W3")
+    src = dict(q=P.q, k=P.k, v=P.v, a=P.a, Wk=P.W_k, W1=W16[0], W2=W16[1], W3=W16[2])
+    lv = {n: g(src[n]).requires_grad_(True) for n in names}
+    out, fr = F.PeriodicAttentionCoreHIP.apply(
+        lv["q"], lv["k"], lv["v"], lv["a"], g(P.rpos), g(P.tvecs), P.batch.to(dev()), P.edges.to(dev()), 64, Hh.DIST_MAX,
+        1.0, lv["Wk"], lv["W1"], lv["W2"], lv["W3"], A16, wscale, cos_abs, cd, ca, g(P.rvlen), CUT,
+        torch.stack([g(f) for f in P.frames], 0))
+    lo = {n: src[n].clone().requires_grad_(True) for n in names}
+    zo, psio = TO.framed_pe(lo["a"], P.rpos, P.tvecs, P.batch, P.edges, lo["Wk"], [lo["W1"], lo["W2"], lo["W3"]], P.frames,
+                            K=64, A=A16, angle_wscale=wscale, cos_abs=cos_abs, c_dist=cd, c_angle=ca, rvlen=P.rvlen,
+                            cutoff_radius=CUT, windows=(11, None))
+    oo, _ = TO.softmax_attention(lo["q"], lo["k"], lo["v"], zo, psio, P.batch, P.edges)
+    assert torch.isfinite(out).all()
+    assert Hh.rel_err(out, oo) < 2e-5 and Hh.elem_err(out, oo, rtol=1e-4, atol_frac=1e-5) <= 1.0
+    gout = torch.randn(P.N, Hh.H, Hh.DH, generator=torch.Generator().manual_seed(3), dtype=torch.float64)
+    (out * g(gout)).sum().backward()
+    (oo * gout).sum().backward()
+    for n in names:
+        assert lv[n].grad.shape == lo[n].grad.shape, n
+        assert Hh.rel_err(lv[n].grad, lo[n].grad) < 1e-4, n
+
+
+def test_lightweight_model_forward_backward_matches_cpu_model(core_mode):
+    """Two layers with the lightweight setting against the float64 CPU model, output and every parameter gradient,
+    through the fused core (whole bases) and through the two-step operators (the reference's windows)."""
     import crystalframer_amd as cf
     from crystalframer_amd import latticeformer, params, synthetic
     mp = params.ModelParams(num_layers=2, value_pe_angle_real=A16, value_pe_angle_wscale=1.0, value_pe_dist_coef=1.5,
@@ -120,13 +157,13 @@ def test_lightweight_model_forward_backward_matches_cpu_model():
     leaves = {k: v.clone().requires_grad_("scale" not in k) for k, v in sd.items()}
     assert leaves["encoder.layers.0.self_attn.proj_angle1"].shape[-1] == A16
     frames = [[f.detach().cpu().double() for f in layer.self_attn.frame_sink[0]] for layer in model.encoder.layers]
-    ref = cpu_model.model_forward(leaves, cb, mp, dtype=torch.float64, frames_per_layer=frames, windows="reference")
+    ref = cpu_model.model_forward(leaves, cb, mp, dtype=torch.float64, frames_per_layer=frames, windows=core_mode)
     torch.nn.functional.mse_loss(ref, target.cpu().double()).backward()
     assert Hh.rel_err(out, ref) < 1e-4
     checked = 0
     for name, p in model.named_parameters():
         if p.grad is None:
             continue
-        assert Hh.rel_err(p.grad, leaves[name].grad) < 2e-4, name
+        assert Hh.rel_err(p.grad, leaves[name].grad) < 1e-4, name
         checked += 1
     assert checked >= 20
