@@ -61,6 +61,15 @@ constexpr int SMALL_A = 16;                     // the 16-bin angle basis (the r
                                                 // basis is small: every image adds its 16 basis values per axis directly
                                                 // (the whole basis, as the reference evaluates it for 16 bins)
 constexpr int HW_ANG16 = 2 * NBINS;             // 64 distance bins + 3 axes x 16 bins, padded to whole 64-word blocks
+// In LDS the 3 x 16 angle bins of an item exist A16_COPIES times, one copy per value of lane & 15: every image adds
+// to ALL 16 bins of an axis in the same order, so with one copy the 64 lanes of an atomic instruction would meet on
+// one word (128 clocks instead of 6).  A copy has an odd number of words so that the copies start in different banks.
+constexpr int A16_COPIES = 16;
+constexpr int A16_STRIDE = 3 * SMALL_A + 1;
+// words of an item's histogram in LDS
+__host__ __device__ constexpr int core_hist_lds_words(int ang) {
+    return ang == SMALL_A ? HW_DIST + A16_COPIES * A16_STRIDE : (ang == NBINS ? HW_ANG : HW_DIST);
+}
 // words of an item's histogram for `ang` angle bins (0: distance encoding alone)
 __host__ __device__ constexpr int core_hist_words(int ang) { return ang == NBINS ? HW_ANG : (ang == SMALL_A ? HW_ANG16 : HW_DIST); }
 constexpr int REC_J0 = 30;                      // item record: first neighbour atom (pairs of an atom are j0, j0+1, ...)
@@ -522,9 +531,11 @@ template <int WL, int ANG, bool COS_ABS>
 __global__ __launch_bounds__(WAVE * CORE_WPB) __attribute__((amdgpu_waves_per_eu(ANG > 0 ? 1 : 7)))
 void fused_core_fwd_kernel(const CoreArgs C) {
     constexpr bool HAS_ANG = ANG > 0;
-    constexpr int HWK = core_hist_words(ANG);
-    __shared__ CoreFwdShared<HWK> shared[CORE_WPB];
-    CoreFwdShared<HWK>& sh = shared[threadIdx.x >> 6];
+    constexpr int HWK = core_hist_words(ANG);          // words per item in memory
+    constexpr int HWL = core_hist_lds_words(ANG);      // ... and in LDS
+    constexpr bool VEC = HWL == HWK && HWK >= 4 * WAVE;      // clear, rescale and store four words per lane at a time
+    __shared__ CoreFwdShared<HWL> shared[CORE_WPB];
+    CoreFwdShared<HWL>& sh = shared[threadIdx.x >> 6];
     float4* const tab = sh.tab;
     uint16_t* const list = sh.list;
     int32_t* const hist = sh.hist;
@@ -546,11 +557,11 @@ void fused_core_fwd_kernel(const CoreArgs C) {
     const float INF = __builtin_inff();
 
     if (it_cur >= P.N) return;
-    if (HWK >= 4 * WAVE) {
+    if (VEC) {
 #pragma unroll
         for (int u = 0; u < HWK / (4 * WAVE); u++) reinterpret_cast<int4*>(hist)[lane + WAVE * u] = make_int4(0, 0, 0, 0);
     } else {
-        for (int u = lane; u < HWK; u += WAVE) hist[u] = 0;
+        for (int u = lane; u < HWL; u += WAVE) hist[u] = 0;
     }
     wave_sync();
 
@@ -689,7 +700,8 @@ void fused_core_fwd_kernel(const CoreArgs C) {
                                     // all 16 basis values, outwards from bin 8 by the two-sided recurrence (sigma >= 1
                                     // bin: the value at bin 8 is at least e^-32 of the peak, no underflow)
                                     const WindowSeed sa = window_seed(((float)(SMALL_A / 2) - uu) * bc.ang_step, bc.ang_step, w);
-                                    window_scatter_rn<SMALL_A>(hist + HW_DIST + ax * SMALL_A, sa, bc.ang_cc);
+                                    window_scatter_rn<SMALL_A>(hist + HW_DIST + (lane & (A16_COPIES - 1)) * A16_STRIDE + ax * SMALL_A,
+                                                               sa, bc.ang_cc);
                                     continue;
                                 }
                                 const float mf = clampf(__builtin_rintf(uu), 0.0f, (float)(NBINS - 1));
@@ -783,8 +795,8 @@ void fused_core_fwd_kernel(const CoreArgs C) {
             if (gmax > m_run) {
                 if (m_run > -INF) {
                     const float fac = hw_exp2((m_run - gmax) * LOG2E);
-                    if (HWK >= 4 * WAVE) {
-                        constexpr int NW = HWK >= 4 * WAVE ? HWK / (4 * WAVE) : 1;
+                    if (VEC) {
+                        constexpr int NW = VEC ? HWK / (4 * WAVE) : 1;
                         int4 hv[NW];
 #pragma unroll
                         for (int u = 0; u < NW; u++) hv[u] = reinterpret_cast<const int4*>(hist)[lane + WAVE * u];
@@ -794,7 +806,7 @@ void fused_core_fwd_kernel(const CoreArgs C) {
                                 make_int4(rint_i((float)hv[u].x * fac), rint_i((float)hv[u].y * fac),
                                           rint_i((float)hv[u].z * fac), rint_i((float)hv[u].w * fac));
                     } else {
-                        for (int u = lane; u < HWK; u += WAVE) hist[u] = rint_i((float)hist[u] * fac);
+                        for (int u = lane; u < HWL; u += WAVE) hist[u] = rint_i((float)hist[u] * fac);
                     }
                     accv.x *= fac; accv.y *= fac; Dl *= fac;
                 }
@@ -859,8 +871,19 @@ void fused_core_fwd_kernel(const CoreArgs C) {
             // consecutive words at a time
             const float sc = inv * (float)max(npairs, 1) * (1.0f / 1073741824.0f);
             float* dst = C.hist + ((size_t)h * P.N + i) * HWK;      // head-major: the rows of a head are contiguous
-            if (HWK >= 4 * WAVE) {
-                constexpr int NW = HWK >= 4 * WAVE ? HWK / (4 * WAVE) : 1;
+            if (ANG == SMALL_A) {
+                // distance bins as they are, every angle bin as the sum of its copies (integers: any order), zeros behind
+                for (int u = lane; u < HWK; u += WAVE) {
+                    int32_t sum = 0;
+                    if (u < HW_DIST) sum = hist[u];
+                    else if (u < HW_DIST + 3 * SMALL_A) {
+#pragma unroll
+                        for (int c = 0; c < A16_COPIES; c++) sum += hist[HW_DIST + c * A16_STRIDE + (u - HW_DIST)];
+                    }
+                    dst[u] = (float)sum * sc;
+                }
+            } else if (VEC) {
+                constexpr int NW = VEC ? HWK / (4 * WAVE) : 1;
                 int4 hv[NW];
 #pragma unroll
                 for (int u = 0; u < NW; u++) hv[u] = reinterpret_cast<const int4*>(hist)[lane + WAVE * u];
