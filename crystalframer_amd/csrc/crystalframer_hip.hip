@@ -146,16 +146,33 @@ int check_params(const cfh_params* p) {
     return CFH_OK;
 }
 
-// window widths for the configured scales; only (9,33) and (11,41) are instantiated
+// Bins of the distance window for the configured scale: ceil(2 wscale cut + 1) (LENGTH_RANGE of
+// models/cuda_funcs/kernel_manager.py:146 for cut = 4), or the whole basis when that leaves at most 8 bins out
+// (models/kernels/real_enc_frame_proj_fwd_length.cu:139-142: the windowed branch needs K - LENGTH_RANGE > 8).
+int dist_window_bins(const cfh_params* p) {
+    const int cut = (p->window_mode == CFH_WINDOW_WIDE) ? 5 : 4;
+    int wl = (int)std::ceil(2.0 * (double)p->dist_wscale * cut + 1.0);
+    if (wl < 1) wl = 1;
+    if (p->dist_bins - wl <= 8) wl = p->dist_bins;
+    return wl;
+}
+// The kernels are compiled for the widths of wscale 1 (9 bins, 11 for the wide mode) and once more for a width that
+// is known at run time only (any other scale).
+bool dist_window_dynamic(const cfh_params* p) {
+    return p->dist_bins > 0 && dist_window_bins(p) != ((p->window_mode == CFH_WINDOW_WIDE) ? 11 : 9);
+}
+// window widths for the configured scales; the angle windows are instantiated for (33) and (41) only
 int window_widths(const cfh_params* p, int* wl, int* wa) {
     const int cut = (p->window_mode == CFH_WINDOW_WIDE) ? 5 : 4;
-    *wl = (int)std::ceil(2.0 * (double)p->dist_wscale * cut + 1.0);
+    *wl = dist_window_bins(p);
     *wa = (int)std::ceil(2.0 * (double)p->angle_wscale * cut + 1.0);
-    const int want_l = cut == 4 ? 9 : 11, want_a = cut == 4 ? 33 : 41;
+    const int want_a = cut == 4 ? 33 : 41;
     if (p->angle_bins == SMALL_ANGLE_BINS) *wa = want_a;      // the whole basis whatever the scale
-    if (p->dist_bins > 0 && *wl != want_l)
-        return fail(CFH_EINVAL, "dist_wscale %g gives a %d-bin window; only wscale 1.0 (%d bins) is compiled",
-                    (double)p->dist_wscale, *wl, want_l);
+    if (p->dist_bins > 0 && !(p->dist_wscale > 0.0f))
+        return fail(CFH_EINVAL, "dist_wscale %g must be positive", (double)p->dist_wscale);
+    if (p->angle_bins == SMALL_ANGLE_BINS && dist_window_dynamic(p))
+        return fail(CFH_EINVAL, "dist_wscale %g with 16 angle bins is not compiled for the two-step operators",
+                    (double)p->dist_wscale);
     if (p->angle_bins > 0 && *wa != want_a)
         return fail(CFH_EINVAL, "angle_wscale %g gives a %d-bin window; only wscale 4.0 (%d bins) is compiled",
                     (double)p->angle_wscale, *wa, want_a);
@@ -174,6 +191,7 @@ cfh::BasisConsts basis_consts(const cfh_params* p) {
         const double step = sl2e / ((double)p->dist_wscale * std::sqrt(2.0));
         bc.len_step = (float)step;
         bc.len_cc = (float)std::exp2(-2.0 * step * step);
+        bc.len_window = dist_window_bins(p);
     }
     if (p->angle_bins > 0) {
         const int A = p->angle_bins;
@@ -463,22 +481,22 @@ int cfh_frame_axes(const cfh_params* p, const float* q, const float* k, const fl
 #define CFH_DISPATCH_PE(KERNEL, HAS_LEN, HAS_ANG)                                                   \
     do {                                                                                            \
         if (wide) {                                                                                 \
-            if (p->cos_abs) rc = launch_persistent(KERNEL<11, 41, true, HAS_LEN, HAS_ANG>, A, &waves, st, what);  \
-            else rc = launch_persistent(KERNEL<11, 41, false, HAS_LEN, HAS_ANG>, A, &waves, st, what);            \
+            if (p->cos_abs) rc = (dyn ? launch_persistent(KERNEL<0, 41, true, HAS_LEN, HAS_ANG>, A, &waves, st, what) : launch_persistent(KERNEL<11, 41, true, HAS_LEN, HAS_ANG>, A, &waves, st, what));  \
+            else rc = (dyn ? launch_persistent(KERNEL<0, 41, false, HAS_LEN, HAS_ANG>, A, &waves, st, what) : launch_persistent(KERNEL<11, 41, false, HAS_LEN, HAS_ANG>, A, &waves, st, what));            \
         } else {                                                                                    \
-            if (p->cos_abs) rc = launch_persistent(KERNEL<9, 33, true, HAS_LEN, HAS_ANG>, A, &waves, st, what);   \
-            else rc = launch_persistent(KERNEL<9, 33, false, HAS_LEN, HAS_ANG>, A, &waves, st, what);             \
+            if (p->cos_abs) rc = (dyn ? launch_persistent(KERNEL<0, 33, true, HAS_LEN, HAS_ANG>, A, &waves, st, what) : launch_persistent(KERNEL<9, 33, true, HAS_LEN, HAS_ANG>, A, &waves, st, what));   \
+            else rc = (dyn ? launch_persistent(KERNEL<0, 33, false, HAS_LEN, HAS_ANG>, A, &waves, st, what) : launch_persistent(KERNEL<9, 33, false, HAS_LEN, HAS_ANG>, A, &waves, st, what));             \
         }                                                                                           \
     } while (0)
 
 #define CFH_DISPATCH_PE_NOGW(KERNEL, HAS_ANG)                                                       \
     do {                                                                                            \
         if (wide) {                                                                                 \
-            if (p->cos_abs) rc = launch_persistent(KERNEL<11, 41, true, true, HAS_ANG, false>, A, &waves, st, what);  \
-            else rc = launch_persistent(KERNEL<11, 41, false, true, HAS_ANG, false>, A, &waves, st, what);            \
+            if (p->cos_abs) rc = (dyn ? launch_persistent(KERNEL<0, 41, true, true, HAS_ANG, false>, A, &waves, st, what) : launch_persistent(KERNEL<11, 41, true, true, HAS_ANG, false>, A, &waves, st, what));  \
+            else rc = (dyn ? launch_persistent(KERNEL<0, 41, false, true, HAS_ANG, false>, A, &waves, st, what) : launch_persistent(KERNEL<11, 41, false, true, HAS_ANG, false>, A, &waves, st, what));            \
         } else {                                                                                    \
-            if (p->cos_abs) rc = launch_persistent(KERNEL<9, 33, true, true, HAS_ANG, false>, A, &waves, st, what);   \
-            else rc = launch_persistent(KERNEL<9, 33, false, true, HAS_ANG, false>, A, &waves, st, what);             \
+            if (p->cos_abs) rc = (dyn ? launch_persistent(KERNEL<0, 33, true, true, HAS_ANG, false>, A, &waves, st, what) : launch_persistent(KERNEL<9, 33, true, true, HAS_ANG, false>, A, &waves, st, what));   \
+            else rc = (dyn ? launch_persistent(KERNEL<0, 33, false, true, HAS_ANG, false>, A, &waves, st, what) : launch_persistent(KERNEL<9, 33, false, true, HAS_ANG, false>, A, &waves, st, what));             \
         }                                                                                           \
     } while (0)
 
@@ -533,16 +551,17 @@ static int framed_pe_forward_impl(const cfh_params* p, const float* q, const flo
     A.frames = frames; A.out_z = z; A.out_psi = psi; A.out_d2min = d2min_out; A.shat = shat_out;
     int waves = launch_waves(N, p->num_heads);
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+    const bool dyn = dist_window_dynamic(p);      // a distance window whose width is not one of the compiled ones
     const char* what = "framed_pe_forward";
     const bool prep = !search;
 #define CFH_DISPATCH_FWD(HAS_LEN, HAS_ANG)                                                                      \
     do {                                                                                                        \
         if (wide) {                                                                                             \
-            if (p->cos_abs) rc = launch_persistent(cfh::framed_pe_fwd_kernel<11, 41, true, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep);  \
-            else rc = launch_persistent(cfh::framed_pe_fwd_kernel<11, 41, false, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep);            \
+            if (p->cos_abs) rc = (dyn ? launch_persistent(cfh::framed_pe_fwd_kernel<0, 41, true, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep) : launch_persistent(cfh::framed_pe_fwd_kernel<11, 41, true, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep));  \
+            else rc = (dyn ? launch_persistent(cfh::framed_pe_fwd_kernel<0, 41, false, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep) : launch_persistent(cfh::framed_pe_fwd_kernel<11, 41, false, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep));            \
         } else {                                                                                                \
-            if (p->cos_abs) rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, true, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep);   \
-            else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep);             \
+            if (p->cos_abs) rc = (dyn ? launch_persistent(cfh::framed_pe_fwd_kernel<0, 33, true, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep) : launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, true, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep));   \
+            else rc = (dyn ? launch_persistent(cfh::framed_pe_fwd_kernel<0, 33, false, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep) : launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, HAS_LEN, HAS_ANG>, A, &waves, st, what, prep));             \
         }                                                                                                       \
     } while (0)
     if (has_ang && p->angle_bins == SMALL_ANGLE_BINS) {
@@ -555,7 +574,7 @@ static int framed_pe_forward_impl(const cfh_params* p, const float* q, const flo
         }
     } else if (has_ang) CFH_DISPATCH_FWD(true, true);
     else if (has_len) CFH_DISPATCH_FWD(true, false);
-    else rc = launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, false, false>, A, &waves, st, what, prep);
+    else rc = (dyn ? launch_persistent(cfh::framed_pe_fwd_kernel<0, 33, false, false, false>, A, &waves, st, what, prep) : launch_persistent(cfh::framed_pe_fwd_kernel<9, 33, false, false, false>, A, &waves, st, what, prep));
 #undef CFH_DISPATCH_FWD
     return rc;
 }
@@ -690,6 +709,7 @@ static int framed_pe_backward_impl(const cfh_params* p, const float* a_ih, const
     A.gw_partial = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + COUNTER_BYTES + items_bytes(N, p->num_heads));
     if (g_pair) {        // gather-only kernel on this stream; nothing else
         const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+        const bool dyn = dist_window_dynamic(p);      // a distance window whose width is not one of the compiled ones
         const char* what = "framed_pe_backward";
         if (p->angle_bins == SMALL_ANGLE_BINS && has_ang) {
             if (wide) rc = p->cos_abs ? launch_persistent(cfh::framed_pe_bwd_saved_kernel<11, SMALL_ANGLE_WINDOW, true, true, true, false>, A, &waves, st, what)
@@ -706,6 +726,7 @@ static int framed_pe_backward_impl(const cfh_params* p, const float* a_ih, const
         A.gw_out_n = p->num_heads * cfh::DH * cfh::NBINS;
     }
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+    const bool dyn = dist_window_dynamic(p);      // a distance window whose width is not one of the compiled ones
     const char* what = "framed_pe_backward";
     if (has_len && shat && !(p->flags & CFH_FLAG_SINGLE_STREAM) && p->angle_bins != SMALL_ANGLE_BINS) {
         // The forward kept its histograms and the weight gradients need nothing else: they are summed by a
@@ -773,7 +794,7 @@ static int framed_pe_backward_impl(const cfh_params* p, const float* a_ih, const
         else CFH_DISPATCH_PE(cfh::framed_pe_bwd_saved_kernel, true, false);
     } else if (has_ang) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, true);
     else if (has_len) CFH_DISPATCH_PE(cfh::framed_pe_bwd_kernel, true, false);
-    else rc = launch_persistent(cfh::framed_pe_bwd_kernel<9, 33, false, false, false>, A, &waves, st, what);
+    else rc = (dyn ? launch_persistent(cfh::framed_pe_bwd_kernel<0, 33, false, false, false>, A, &waves, st, what) : launch_persistent(cfh::framed_pe_bwd_kernel<9, 33, false, false, false>, A, &waves, st, what));
     if (rc) return rc;
     if (has_len) {
         const int nenc = has_ang ? 4 : 1;
@@ -1283,7 +1304,7 @@ int check_core_params(const cfh_params* p) {
     int rc = check_params(p);
     if (rc) return rc;
     if (p->dist_bins != cfh::NBINS) return fail(CFH_EINVAL, "fused core: dist_bins must be %d", cfh::NBINS);
-    if (p->dist_wscale != 1.0f) return fail(CFH_EINVAL, "fused core: only dist_wscale 1.0 is compiled");
+    if (!(p->dist_wscale > 0.0f)) return fail(CFH_EINVAL, "fused core: dist_wscale %g must be positive", (double)p->dist_wscale);
     if (p->grad_coef_quirk) return fail(CFH_EINVAL, "fused core: grad_coef_quirk is not available (exact gradients only)");
     if (p->angle_bins == cfh::NBINS && p->angle_wscale < 3.0f)
         return fail(CFH_EINVAL, "fused core: angle_wscale %g < 3 with 64 angle bins: the moment expansion of the angle "
@@ -1454,22 +1475,23 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     }
     C.slow_flag = cfh::REC_BOX_LISTED;
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+    const bool dyn = dist_window_dynamic(p);      // a distance window whose width is not one of the compiled ones
     const char* what = "fused_core_forward";
 #define CFH_CORE_DISPATCH(KERNEL)                                                                         \
     do {                                                                                                  \
         if (p->angle_bins == cfh::SMALL_A) {                                                              \
-            if (wide) rc = p->cos_abs ? launch_core(KERNEL<11, cfh::SMALL_A, true>, C, st, what)          \
-                                      : launch_core(KERNEL<11, cfh::SMALL_A, false>, C, st, what);        \
-            else rc = p->cos_abs ? launch_core(KERNEL<9, cfh::SMALL_A, true>, C, st, what)                \
-                                 : launch_core(KERNEL<9, cfh::SMALL_A, false>, C, st, what);              \
+            if (wide) rc = p->cos_abs ? (dyn ? launch_core(KERNEL<0, cfh::SMALL_A, true>, C, st, what) : launch_core(KERNEL<11, cfh::SMALL_A, true>, C, st, what))          \
+                                      : (dyn ? launch_core(KERNEL<0, cfh::SMALL_A, false>, C, st, what) : launch_core(KERNEL<11, cfh::SMALL_A, false>, C, st, what));        \
+            else rc = p->cos_abs ? (dyn ? launch_core(KERNEL<0, cfh::SMALL_A, true>, C, st, what) : launch_core(KERNEL<9, cfh::SMALL_A, true>, C, st, what))                \
+                                 : (dyn ? launch_core(KERNEL<0, cfh::SMALL_A, false>, C, st, what) : launch_core(KERNEL<9, cfh::SMALL_A, false>, C, st, what));              \
         } else if (has_ang) {                                                                             \
-            if (wide) rc = p->cos_abs ? launch_core(KERNEL<11, cfh::NBINS, true>, C, st, what)            \
-                                      : launch_core(KERNEL<11, cfh::NBINS, false>, C, st, what);          \
-            else rc = p->cos_abs ? launch_core(KERNEL<9, cfh::NBINS, true>, C, st, what)                  \
-                                 : launch_core(KERNEL<9, cfh::NBINS, false>, C, st, what);                \
+            if (wide) rc = p->cos_abs ? (dyn ? launch_core(KERNEL<0, cfh::NBINS, true>, C, st, what) : launch_core(KERNEL<11, cfh::NBINS, true>, C, st, what))            \
+                                      : (dyn ? launch_core(KERNEL<0, cfh::NBINS, false>, C, st, what) : launch_core(KERNEL<11, cfh::NBINS, false>, C, st, what));          \
+            else rc = p->cos_abs ? (dyn ? launch_core(KERNEL<0, cfh::NBINS, true>, C, st, what) : launch_core(KERNEL<9, cfh::NBINS, true>, C, st, what))                  \
+                                 : (dyn ? launch_core(KERNEL<0, cfh::NBINS, false>, C, st, what) : launch_core(KERNEL<9, cfh::NBINS, false>, C, st, what));                \
         } else {                                                                                          \
-            rc = wide ? launch_core(KERNEL<11, 0, false>, C, st, what)                                    \
-                      : launch_core(KERNEL<9, 0, false>, C, st, what);                                    \
+            rc = wide ? (dyn ? launch_core(KERNEL<0, 0, false>, C, st, what) : launch_core(KERNEL<11, 0, false>, C, st, what))                                    \
+                      : (dyn ? launch_core(KERNEL<0, 0, false>, C, st, what) : launch_core(KERNEL<9, 0, false>, C, st, what));                                    \
         }                                                                                                 \
     } while (0)
     CFH_CORE_DISPATCH(cfh::fused_core_fwd_kernel);
@@ -1600,6 +1622,7 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
         hipLaunchKernelGGL(cfh::sorted_shifts_kernel, dim3((unsigned)B), dim3(cfh::FC_TCAP), 0, st, tvecs, C.table_R,
                            buf.table);
     const bool wide = p->window_mode == CFH_WINDOW_WIDE;
+    const bool dyn = dist_window_dynamic(p);      // a distance window whose width is not one of the compiled ones
     const char* what = "fused_core_backward";
     CFH_CORE_DISPATCH(cfh::fused_core_bwd_kernel);
 #undef CFH_CORE_DISPATCH

@@ -253,13 +253,16 @@ constexpr float FIX_ONE = 2147483648.0f;          // 2^31
 constexpr float FIX_INV = 1.0f / 2147483648.0f;
 static_assert(TCAP <= (1 << (16 - GROUP_BITS)) && GROUP <= (1 << GROUP_BITS), "list entry is 16 bits");
 
+// Window helpers.  W > 0: the width is a compile-time constant (the loops unroll); W == 0: the width is `wrt`, the same
+// in all lanes (a distance scale other than 1: any width from 2 bins to the whole basis).  The recurrence starts at
+// bin C = width / 2 of the window and walks upwards to the last bin and downwards to the first.
 template <int W>
-__device__ __forceinline__ void window_scatter(uint32_t* base, const WindowSeed& s, float cc) {
-    constexpr int C = W / 2;
+__device__ __forceinline__ void window_scatter(uint32_t* base, const WindowSeed& s, float cc, int wrt = 0) {
+    const int Wd = W > 0 ? W : wrt, C = Wd / 2;
     atomicAdd(base + C, (uint32_t)s.gc);
     float g = s.gc, r = s.rr;
 #pragma unroll
-    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; atomicAdd(base + m, (uint32_t)g); }
+    for (int m = C + 1; m < Wd; m++) { g *= r; r *= cc; atomicAdd(base + m, (uint32_t)g); }
     g = s.gc; r = s.rl;
 #pragma unroll
     for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; atomicAdd(base + m, (uint32_t)g); }
@@ -269,30 +272,31 @@ __device__ __forceinline__ void window_scatter(uint32_t* base, const WindowSeed&
 // downwards, then upwards): lanes whose windows coincide (clamped windows of one pair) then add to
 // different words at the same time instead of queueing on one.
 template <int W>
-__device__ __forceinline__ void window_scatter_dir(uint32_t* base, const WindowSeed& s, float cc, int dir) {
-    constexpr int C = W / 2;
-    static_assert(W == 2 * C + 1, "window width must be odd");
+__device__ __forceinline__ void window_scatter_dir(uint32_t* base, const WindowSeed& s, float cc, int dir, int wrt = 0) {
+    const int Wd = W > 0 ? W : wrt, C = Wd / 2;
+    const int up = Wd - 1 - C, down = C;            // bins above and below the centre (equal for an odd width)
     uint32_t* const centre = base + C;
     atomicAdd(centre, (uint32_t)s.gc);
     float g = s.gc, r = dir > 0 ? s.rr : s.rl;
     uint32_t* p = centre;
+    const int n1 = dir > 0 ? up : down, n2 = dir > 0 ? down : up;
 #pragma unroll
-    for (int m = 1; m <= C; m++) { p += dir; g *= r; r *= cc; atomicAdd(p, (uint32_t)g); }
+    for (int m = 1; m <= n1; m++) { p += dir; g *= r; r *= cc; atomicAdd(p, (uint32_t)g); }
     g = s.gc; r = dir > 0 ? s.rl : s.rr; p = centre;
 #pragma unroll
-    for (int m = 1; m <= C; m++) { p -= dir; g *= r; r *= cc; atomicAdd(p, (uint32_t)g); }
+    for (int m = 1; m <= n2; m++) { p -= dir; g *= r; r *= cc; atomicAdd(p, (uint32_t)g); }
 }
 
 // Scatter weight*g_m into hbase[m] and return sum_m weight*g_m*gbase[m].
 template <int W>
 __device__ __forceinline__ float window_scatter_gather(uint32_t* hbase, const float* gbase,
-                                                       const WindowSeed& s, float cc) {
-    constexpr int C = W / 2;
+                                                       const WindowSeed& s, float cc, int wrt = 0) {
+    const int Wd = W > 0 ? W : wrt, C = Wd / 2;
     float acc = s.gc * gbase[C];
     atomicAdd(hbase + C, (uint32_t)s.gc);
     float g = s.gc, r = s.rr;
 #pragma unroll
-    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); atomicAdd(hbase + m, (uint32_t)g); }
+    for (int m = C + 1; m < Wd; m++) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); atomicAdd(hbase + m, (uint32_t)g); }
     g = s.gc; r = s.rl;
 #pragma unroll
     for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); atomicAdd(hbase + m, (uint32_t)g); }
@@ -301,12 +305,12 @@ __device__ __forceinline__ float window_scatter_gather(uint32_t* hbase, const fl
 
 // sum_m weight*g_m*gbase[m] alone (the histograms come from the forward pass).
 template <int W>
-__device__ __forceinline__ float window_gather(const float* gbase, const WindowSeed& s, float cc) {
-    constexpr int C = W / 2;
+__device__ __forceinline__ float window_gather(const float* gbase, const WindowSeed& s, float cc, int wrt = 0) {
+    const int Wd = W > 0 ? W : wrt, C = Wd / 2;
     float acc = s.gc * gbase[C];
     float g = s.gc, r = s.rr;
 #pragma unroll
-    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); }
+    for (int m = C + 1; m < Wd; m++) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); }
     g = s.gc; r = s.rl;
 #pragma unroll
     for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; acc = fmaf(g, gbase[m], acc); }
@@ -327,6 +331,7 @@ struct BasisConsts {
     float start_off;       // 4*wscale + 1  : start = trunc(d*inv_interval - start_off)
     float len_step;        // sqrt(log2 e)/(wscale*sqrt 2) : scaled offset between neighbouring bins
     float len_cc;          // 2^(-2 len_step^2)
+    int32_t len_window;    // bins of the distance window (the kernels compiled for a fixed width do not read it)
     // angle basis
     float ang_inv_interval;  // (A-1)/2 (cos_abs: A-1)
     float ang_end_off;       // 1 + 4*sigma_a

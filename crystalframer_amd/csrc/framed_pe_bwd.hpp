@@ -64,6 +64,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
         for (int cq = 0; cq < 4; cq++) gWacc[en * 4 + cq] = v4f_b{0.f, 0.f, 0.f, 0.f};
     }
     const BasisConsts bc = P.bc;
+    const int WLr = WL > 0 ? WL : bc.len_window;      // bins of the distance window (WL == 0: known at run time only)
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
 
     for (int u = lane; u < GROUP_BWD * PAIR_STRIDE; u += WAVE) { hist[u] = 0u; Gs[u] = 0.0f; }
@@ -125,10 +126,10 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_kernel(const KernelArgs P)
                             const float d = hw_sqrt(d2);
                             const float u = d * bc.inv_interval;
                             int start = (int)(u - bc.start_off);
-                            start = max(0, min(start, NBINS - WL));
-                            const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
+                            start = max(0, min(start, NBINS - WLr));
+                            const float beta_c = ((float)(start + WLr / 2 + 1) - u) * bc.len_step;
                             const WindowSeed s = window_seed(beta_c, bc.len_step, pf);
-                            pbg += window_scatter_gather<WL>(myhist + start, myG + start, s, bc.len_cc);
+                            pbg += window_scatter_gather<WL>(myhist + start, myG + start, s, bc.len_cc, WLr);
                         }
                         if (HAS_ANG) {
                             if (d2 > 1e-5f) {

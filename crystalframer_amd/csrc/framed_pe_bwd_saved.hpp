@@ -46,6 +46,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
         }
     }
     const BasisConsts bc = P.bc;
+    const int WLr = WL > 0 ? WL : bc.len_window;      // bins of the distance window (WL == 0: known at run time only)
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
 
     for (int u = lane; u < GROUP_SAVED * PAIR_STRIDE; u += WAVE) Gs[u] = 0.0f;
@@ -106,10 +107,10 @@ __global__ __launch_bounds__(WAVE) void framed_pe_bwd_saved_kernel(const KernelA
                             const float d = hw_sqrt(d2);
                             const float u = d * bc.inv_interval;
                             int start = (int)(u - bc.start_off);
-                            start = max(0, min(start, NBINS - WL));
-                            const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
+                            start = max(0, min(start, NBINS - WLr));
+                            const float beta_c = ((float)(start + WLr / 2 + 1) - u) * bc.len_step;
                             const WindowSeed s = window_seed(beta_c, bc.len_step, pf);
-                            pbg += window_gather<WL>(myG + start, s, bc.len_cc);
+                            pbg += window_gather<WL>(myG + start, s, bc.len_cc, WLr);
                         }
                         if (HAS_ANG) {
                             if (d2 > 1e-5f) {

@@ -60,6 +60,7 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
     }
     const float enc_scale = ((enc == 0) ? P.dist_coef : P.angle_coef) * FIX_INV;
     const BasisConsts bc = P.bc;
+    const int WLr = WL > 0 ? WL : bc.len_window;      // bins of the distance window (WL == 0: known at run time only)
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
 
     for (int u = lane; u < GROUP * PAIR_STRIDE; u += WAVE) hist[u] = 0u;
@@ -130,11 +131,11 @@ __global__ __launch_bounds__(WAVE) void framed_pe_fwd_kernel(const KernelArgs P)
                             const float d = hw_sqrt(d2);
                             const float u = d * bc.inv_interval;
                             int start = (int)(u - bc.start_off);          // truncation toward zero
-                            start = max(0, min(start, NBINS - WL));
+                            start = max(0, min(start, NBINS - WLr));
                             // bin k has centre (k+1)*interval: scaled offset ((k+1) - u)*len_step
-                            const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
+                            const float beta_c = ((float)(start + WLr / 2 + 1) - u) * bc.len_step;
                             const WindowSeed s = window_seed(beta_c, bc.len_step, w);
-                            window_scatter_dir<WL>(myhist + start, s, bc.len_cc, dir);
+                            window_scatter_dir<WL>(myhist + start, s, bc.len_cc, dir, WLr);
                         }
                         if (HAS_ANG) {
                             if (d2 > 1e-5f) {       // the self image contributes to S only

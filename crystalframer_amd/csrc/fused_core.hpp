@@ -361,12 +361,12 @@ struct CoreWgradJobs {
 };
 // ---- distance window with round-to-nearest fixed-point adds ---------------------------------------------------
 template <int W>
-__device__ __forceinline__ void window_scatter_rn(int32_t* base, const WindowSeed& s, float cc) {
-    constexpr int C = W / 2;
+__device__ __forceinline__ void window_scatter_rn(int32_t* base, const WindowSeed& s, float cc, int wrt = 0) {
+    const int Wd = W > 0 ? W : wrt, C = Wd / 2;      // (W == 0: the width is known at run time only)
     atomicAdd(base + C, rint_i(s.gc));
     float g = s.gc, r = s.rr;
 #pragma unroll
-    for (int m = C + 1; m < W; m++) { g *= r; r *= cc; atomicAdd(base + m, rint_i(g)); }
+    for (int m = C + 1; m < Wd; m++) { g *= r; r *= cc; atomicAdd(base + m, rint_i(g)); }
     g = s.gc; r = s.rl;
 #pragma unroll
     for (int m = C - 1; m >= 0; m--) { g *= r; r *= cc; atomicAdd(base + m, rint_i(g)); }
@@ -491,7 +491,8 @@ __device__ __forceinline__ int core_slow_record(const CoreArgs& C, int r, int la
 // Which record a wavefront of a main kernel starts with: the first slow_wgs wavefronts a listed one (-1: none left),
 // the others the records in work order.
 __device__ __forceinline__ int core_wave_record(const CoreArgs& C, int w, int lane) {
-    return w < C.slow_wgs ? core_slow_record(C, w, lane) : w - C.slow_wgs;
+    // (the same in all lanes: said so, the index arithmetic that follows stays on the scalar unit)
+    return __builtin_amdgcn_readfirstlane(w < C.slow_wgs ? core_slow_record(C, w, lane) : w - C.slow_wgs);
 }
 // The rank over the slow lists of the listed record `wid`: the counts of the lists before its own, and its place in its
 // own list (records in ascending order: the entries below it).
@@ -553,6 +554,7 @@ void fused_core_fwd_kernel(const CoreArgs C) {
     const int pr = lane >> 3;          // pair of the group served by this 8-lane row
     const int sub = lane & 7;          // position in the row
     const BasisConsts bc = P.bc;
+    const int WLr = WL > 0 ? WL : bc.len_window;      // bins of the distance window (WL == 0: known at run time only)
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
     const float INF = __builtin_inff();
 
@@ -592,7 +594,9 @@ void fused_core_fwd_kernel(const CoreArgs C) {
         wave_sync();
         const size_t ih = (size_t)i * H + h;
         const float2 q2 = pf.q2;
-        const float fixs = 1073741824.0f / (float)max(npairs, 1);      // 2^30 / npairs: sums of weights <= 1 each fit
+        // 2^30 / npairs: sums of weights <= 1 each fit (hardware reciprocal: any scale near it will do, the histogram
+        // is divided by the same number when it is written)
+        const float fixs = 1073741824.0f * hw_rcp((float)max(npairs, 1));
         const float cutS = (C.skip_log2 > 0.0f && a2 < 0.0f) ? C.skip_log2 * hw_rcp(-a2) : INF;      // (a bound with margins)
         float m_run = -INF;                   // running maximum of the logits (wave-uniform)
         float Dl = 0.0f;                      // this lane's share of the softmax denominator
@@ -679,13 +683,13 @@ void fused_core_fwd_kernel(const CoreArgs C) {
                         const float d = hw_sqrt(d2);
                         const float u = d * bc.inv_interval;
                         int start = (int)(u - bc.start_off);          // truncation toward zero
-                        start = max(0, min(start, NBINS - WL));
-                        const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
+                        start = max(0, min(start, NBINS - WLr));
+                        const float beta_c = ((float)(start + WLr / 2 + 1) - u) * bc.len_step;
                         const WindowSeed s = window_seed(beta_c, bc.len_step, w);
 #ifndef CFH_EXP_NOCONFLICT
-                        window_scatter_rn<WL>(hist + start, s, bc.len_cc);
+                        window_scatter_rn<WL>(hist + start, s, bc.len_cc, WLr);
 #else
-                        window_scatter_rn<WL>(hist + (start & 0) + lane, s, bc.len_cc);
+                        window_scatter_rn<WL>(hist + (start & 0) + lane, s, bc.len_cc, WLr);
 #endif
                     }
                     if (HAS_ANG) {
@@ -869,7 +873,7 @@ void fused_core_fwd_kernel(const CoreArgs C) {
         {
             // all reads first (one LDS round trip instead of one per word), then store; a lane takes four
             // consecutive words at a time
-            const float sc = inv * (float)max(npairs, 1) * (1.0f / 1073741824.0f);
+            const float sc = inv * hw_rcp(fixs);
             float* dst = C.hist + ((size_t)h * P.N + i) * HWK;      // head-major: the rows of a head are contiguous
             if (ANG == SMALL_A) {
                 // distance bins as they are, every angle bin as the sum of its copies (integers: any order), zeros behind
@@ -1156,6 +1160,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
     const int h = wid - it_cur * H;
     const int pr = lane >> 3, sub = lane & 7;
     const BasisConsts bc = P.bc;
+    const int WLr = WL > 0 ? WL : bc.len_window;      // bins of the distance window (WL == 0: known at run time only)
     const float prune = (P.prune_log2 > 0.0f) ? -P.prune_log2 : -3.0e38f;
     const float INF = __builtin_inff();
 
@@ -1258,10 +1263,10 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
                         const float d = hw_sqrt(d2);
                         const float u = d * bc.inv_interval;
                         int start = (int)(u - bc.start_off);
-                        start = max(0, min(start, NBINS - WL));
-                        const float beta_c = ((float)(start + WL / 2 + 1) - u) * bc.len_step;
+                        start = max(0, min(start, NBINS - WLr));
+                        const float beta_c = ((float)(start + WLr / 2 + 1) - u) * bc.len_step;
                         const WindowSeed s = window_seed(beta_c, bc.len_step, 1.0f);
-                        bg = window_gather<WL>(Gs + start, s, bc.len_cc);
+                        bg = window_gather<WL>(Gs + start, s, bc.len_cc, WLr);
                     }
                     if (HAS_ANG) {
                         if (d2 > 1e-5f) {

@@ -75,8 +75,11 @@ def compile_kernels(lattice_range: int, head_num: int, key_head_dim: int, value_
     if value_pe_dim not in (0, 64) or dim_angle_enc not in (0, 16, 64):
         raise NotImplementedError(f"value_pe_dist_real={value_pe_dim}, value_pe_angle_real={dim_angle_enc}: "
                                   "compiled are 0 or 64 distance bins and 0, 16 or 64 angle bins")
-    if value_pe_dim > 0 and float(value_pe_dist_wscale) != 1.0:
-        raise NotImplementedError("value_pe_dist_wscale: only 1.0 is compiled")
+    if value_pe_dim > 0 and not float(value_pe_dist_wscale) > 0.0:
+        raise ValueError("value_pe_dist_wscale must be positive")
+    if value_pe_dim > 0 and float(value_pe_dist_wscale) != 1.0 and dim_angle_enc == 16 and not _fused_core_default():
+        # (kernels for a window width known at run time only exist for 0 and 64 angle bins in the two-step operators)
+        raise NotImplementedError("value_pe_dist_wscale != 1 with 16 angle bins: only through the fused attention core")
     if dim_angle_enc == 64 and float(value_pe_angle_wscale) != 4.0:
         raise NotImplementedError("value_pe_angle_wscale: only 4.0 is compiled for 64 angle bins")
     if dim_angle_enc == 16 and float(value_pe_angle_wscale) < 1.0:
@@ -88,6 +91,11 @@ def compile_kernels(lattice_range: int, head_num: int, key_head_dim: int, value_
     KernelManager.SYMM_BREAK_NOISE = float(symm_break_noise)
     KernelManager._compiled_for = dict(head_num=head_num, cos_abs=cos_abs)
     _lib.load()
+
+
+def _fused_core_default() -> bool:
+    from . import attention
+    return bool(attention.FUSED_CORE)
 
 
 # --------------------------------------------------------------------------------------------------
@@ -676,7 +684,7 @@ class PeriodicAttentionCoreHIP(torch.autograd.Function):
 
     @staticmethod
     def supported(K, dim_angle_enc, wscale, angle_wscale, W_k, W_k1) -> bool:
-        if W_k is None or int(K) != 64 or float(wscale) != 1.0 or KernelManager.GRAD_COEF_QUIRK:
+        if W_k is None or int(K) != 64 or not float(wscale) > 0.0 or KernelManager.GRAD_COEF_QUIRK:
             return False
         if W_k.dim() == 4 and W_k.shape[0] != 1:
             return False

@@ -308,6 +308,32 @@ def test_crystal_indices_with_an_offset_give_the_same_output():
     assert torch.equal(out, ref)
 
 
+def test_a_bare_batch_object_with_the_reference_fields_only():
+    """What the reference's data loader hands the model (dataloaders/dataset_latticeformer.py:32-37): an object with
+    x, pos, batch, trans_vec and sizes and nothing else (no host-known pair count, no zero-based flag).  Same output
+    and gradients as the CrystalBatch that carries the extras."""
+    import types
+    from crystalframer_amd import latticeformer, params, synthetic
+    dev = torch.device("cuda:0")
+    mp = params.ModelParams(num_layers=2, symm_break_noise=0.0)
+    cb = synthetic.make_batch(7, atoms="uniform", atoms_lo=1, atoms_hi=6, len_lo=3.0, len_hi=9.0,
+                              ang_lo=65.0, ang_hi=115.0, seed=33).to(dev)
+    bare = types.SimpleNamespace(x=cb.x, pos=cb.pos, batch=cb.batch, trans_vec=cb.trans_vec, sizes=cb.sizes)
+    torch.manual_seed(2)
+    model = latticeformer.Latticeformer(mp).to(dev)
+    model.train()
+    model(cb)                      # stores the normalisation of alpha
+    results = []
+    for data in (cb, bare):
+        model.zero_grad(set_to_none=True)
+        out = model(data)
+        out.square().sum().backward()
+        results.append((out.detach().clone(), {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None}))
+    assert torch.equal(results[0][0], results[1][0])
+    for n, gr in results[0][1].items():
+        assert Hh.rel_err(results[1][1][n], gr) < 1e-6, n
+
+
 def test_hooked_parameter_and_reused_weight_get_complete_gradients():
     """Deferred weight gradients must not be visible as zeros: a parameter with a tensor hook or a
     post-accumulate hook is not deferred (its hook sees the finished gradient), and a weight used by two
