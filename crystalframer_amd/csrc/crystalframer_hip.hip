@@ -1313,6 +1313,14 @@ int check_core_params(const cfh_params* p) {
         return fail(CFH_EINVAL, "fused core: angle_wscale %g < 1 with 16 angle bins is not compiled", (double)p->angle_wscale);
     return CFH_OK;
 }
+// The main kernels address q, k, v, rpos, z and the probabilities with 32-bit byte offsets.
+int check_core_sizes(const cfh_params* p, int64_t N, int64_t E) {
+    const int64_t lim = (int64_t)1 << 30;      // elements of 4 bytes
+    if (N * p->num_heads * cfh::DH >= lim || E * p->num_heads >= lim || E * 3 >= lim)
+        return fail(CFH_EINVAL, "fused core: N = %lld atoms or E = %lld pairs beyond the 32-bit offsets of its kernels "
+                    "(N x heads x 16 and E x heads must stay below 2^30)", (long long)N, (long long)E);
+    return CFH_OK;
+}
 // the kernels' launch-wide arguments that both directions share; buffers of the caller's cache replace the
 // workspace regions of the same content
 struct CoreBuffers {
@@ -1390,6 +1398,7 @@ int cfh_fused_core_forward(const cfh_params* p, const float* qs, const float* k,
     int rc = check_core_params(p);
     if (rc) return rc;
     if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
+    if ((rc = check_core_sizes(p, N, E))) return rc;
     if (N == 0) return CFH_OK;
     const bool has_ang = p->angle_bins > 0;
     if (!qs || !k || !v || !W_dist || !z || !prob || !hist || !out)
@@ -1515,6 +1524,7 @@ int cfh_fused_core_backward(const cfh_params* p, const float* qs, const float* k
     int rc = check_core_params(p);
     if (rc) return rc;
     if ((rc = check_geometry(a_ih, rpos, tvecs, batch, edges, e_start, N, E, B))) return rc;
+    if ((rc = check_core_sizes(p, N, E))) return rc;
     hipStream_t st = (hipStream_t)stream;
     const bool has_ang = p->angle_bins > 0;
     const int per_enc = p->num_heads * cfh::DH * cfh::NBINS;

@@ -119,6 +119,14 @@ struct CoreArgs {
     float* glogit;                // (E,H) gradient of the logits (the column kernel turns it into gk)
 };
 
+// Loads at a 32-bit BYTE offset from a base that is the same in all lanes: the address is (scalar base + vector offset),
+// one instruction's operands, where an element index of 64 bits costs two or three vector instructions per address
+// (the entry points refuse sizes whose offsets would not fit).
+template <typename T>
+__device__ __forceinline__ T load_at(const void* base, uint32_t byte_off) {
+    return *reinterpret_cast<const T*>(reinterpret_cast<const char*>(base) + byte_off);
+}
+
 // ---- reductions over an 8-lane row (half of a DPP row) -------------------------------------------------------
 __device__ __forceinline__ float half_sum(float x) {
     x += dpp_move<0xB1>(x); x += dpp_move<0x4E>(x); x += dpp_move<0x141>(x); return x;
@@ -440,14 +448,17 @@ __device__ __forceinline__ CorePrefetch core_prefetch(const CoreArgs& C, uint32_
         pf.t0 = src[lane];
         pf.t1 = src[lane + WAVE];
     }
-    pf.q2 = *reinterpret_cast<const float2*>(C.qs + ((size_t)i * H + h) * DH + 2 * sub);
-    if (pr < npairs) {
-        const size_t e = (size_t)(e0 + pr);
-        const size_t jh = ((size_t)(j0 + pr) * H + h) * DH + 2 * sub;
-        pf.rx = P.rpos[e * 3 + 0]; pf.ry = P.rpos[e * 3 + 1]; pf.rz = P.rpos[e * 3 + 2];
-        pf.k2 = *reinterpret_cast<const float2*>(C.k + jh);
-        pf.v2 = *reinterpret_cast<const float2*>(C.v + jh);
-        if (C.pair_near) pf.near = C.pair_near[e].x;
+    pf.q2 = load_at<float2>(C.qs, (((uint32_t)i * (uint32_t)H + (uint32_t)h) * DH + 2u * sub) * 4u);
+    if (npairs > 0) {
+        // (no branch per row: a row past the end re-reads the row's last pair; nothing of it is used)
+        const uint32_t el = (uint32_t)min(pr, npairs - 1);
+        const uint32_t e = min((uint32_t)e0 + el, (uint32_t)(P.E - 1));
+        const uint32_t jh = ((((uint32_t)j0 + el) * (uint32_t)H + (uint32_t)h) * DH + 2u * sub) * 4u;
+        const float3 r3 = load_at<float3>(P.rpos, e * 12u);
+        pf.rx = r3.x; pf.ry = r3.y; pf.rz = r3.z;
+        pf.k2 = load_at<float2>(C.k, jh);
+        pf.v2 = load_at<float2>(C.v, jh);
+        if (C.pair_near) pf.near = load_at<float>(C.pair_near, e * 8u);
     }
     return pf;
 }
@@ -615,15 +626,15 @@ void fused_core_fwd_kernel(const CoreArgs C) {
         // heavy pass makes their shifts from that index instead of reading a table: one sweep, each chunk built once
         const bool one_list = nchunks > 1 && bx.T <= FC_BIGT;
         auto fetch = [&](int g0) {
-            const int el = g0 + pr;
-            if (el < npairs) {
-                const size_t e = (size_t)(e0 + el);
-                const size_t jh = ((size_t)(ci.j0 + el) * H + h) * DH + 2 * sub;
-                nrx = P.rpos[e * 3 + 0]; nry = P.rpos[e * 3 + 1]; nrz = P.rpos[e * 3 + 2];
-                nk2 = *reinterpret_cast<const float2*>(C.k + jh);
-                nv2 = *reinterpret_cast<const float2*>(C.v + jh);
-                if (near_known) nnear = C.pair_near[e].x;
-            }
+            // (no branch per row: a row past the end re-reads the row's last pair; nothing of it is used)
+            const uint32_t el = (uint32_t)min(g0 + pr, npairs - 1);
+            const uint32_t e = min((uint32_t)e0 + el, (uint32_t)(P.E - 1));
+            const uint32_t jh = ((((uint32_t)ci.j0 + el) * (uint32_t)H + (uint32_t)h) * DH + 2u * sub) * 4u;
+            const float3 r3 = load_at<float3>(P.rpos, e * 12u);
+            nrx = r3.x; nry = r3.y; nrz = r3.z;
+            nk2 = load_at<float2>(C.k, jh);
+            nv2 = load_at<float2>(C.v, jh);
+            if (near_known) nnear = load_at<float>(C.pair_near, e * 8u);
         };
 
         // one sweep of this row's pair over the table(s): fn(inside, index in the chunk, first index of the chunk, d^2, rows inside)
@@ -820,14 +831,12 @@ void fused_core_fwd_kernel(const CoreArgs C) {
             accv.x = fmaf(ew, v2.x, accv.x);
             accv.y = fmaf(ew, v2.y, accv.y);
             if (sub == 0 && active) {
-                const size_t eh = (size_t)(e0 + g0 + pr) * H + h;
+                const uint32_t eh = ((uint32_t)(e0 + g0 + pr) * (uint32_t)H + (uint32_t)h) * 4u;      // byte offset
                 pairA[pr] = make_float4(rx, ry, rz, d2min);
                 pairC[pr] = ew * hw_rcp(S) * fixs;
-#ifndef CFH_EXP_NOZ
-                C.z[eh] = z;
-#endif
+                *reinterpret_cast<float*>(reinterpret_cast<char*>(C.z) + eh) = z;
                 if (npairs <= FC_LOGCAP) logit_s[g0 + pr] = logit;
-                else C.prob[eh] = logit;         // the logit for now; normalised when the row is complete
+                else *reinterpret_cast<float*>(reinterpret_cast<char*>(C.prob) + eh) = logit;      // the logit for now; normalised when the row is complete
                 Dl += ew;
             }
             wave_sync();
@@ -1217,17 +1226,18 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
         float nrx = 0.f, nry = 0.f, nrz = 0.f, nz = 0.f, npb = 0.f;
         float2 nk2 = make_float2(0.f, 0.f), nv2 = nk2;
         auto fetch = [&](int g0) {
-            const int el = g0 + pr;
-            if (el < npairs) {
-                const size_t e = (size_t)(e0 + el);
-                const size_t jh = ((size_t)(ci.j0 + el) * H + h) * DH + 2 * sub;
-                nrx = P.rpos[e * 3 + 0]; nry = P.rpos[e * 3 + 1]; nrz = P.rpos[e * 3 + 2];
-                nz = C.z[e * H + h]; npb = C.prob[e * H + h];
-                nk2 = *reinterpret_cast<const float2*>(C.k + jh);
-                nv2 = *reinterpret_cast<const float2*>(C.v + jh);
-            }
+            // (no branch per row: a row past the end re-reads the row's last pair; nothing of it is used)
+            const uint32_t el = (uint32_t)min(g0 + pr, npairs - 1);
+            const uint32_t e = min((uint32_t)e0 + el, (uint32_t)(P.E - 1));
+            const uint32_t jh = ((((uint32_t)ci.j0 + el) * (uint32_t)H + (uint32_t)h) * DH + 2u * sub) * 4u;
+            const uint32_t eh = (e * (uint32_t)H + (uint32_t)h) * 4u;
+            const float3 r3 = load_at<float3>(P.rpos, e * 12u);
+            nrx = r3.x; nry = r3.y; nrz = r3.z;
+            nz = load_at<float>(C.z, eh); npb = load_at<float>(C.prob, eh);
+            nk2 = load_at<float2>(C.k, jh);
+            nv2 = load_at<float2>(C.v, jh);
         };
-        fetch(0);
+        if (npairs > 0) fetch(0);
 
         // several chunks: the survivors of all chunks in one list with their index in the whole box (as in the forward)
         const bool one_list = nchunks > 1 && bx.T <= FC_BIGT;
@@ -1395,7 +1405,7 @@ __global__ __launch_bounds__(WAVE * CORE_WPB) void fused_core_bwd_kernel(const C
             gq2.x = fmaf(gl, k2.x, gq2.x);
             gq2.y = fmaf(gl, k2.y, gq2.y);
             if (sub == 0 && active) {
-                C.glogit[(size_t)(e0 + g0 + pr) * H + h] = gl;
+                *reinterpret_cast<float*>(reinterpret_cast<char*>(C.glogit) + ((uint32_t)(e0 + g0 + pr) * (uint32_t)H + (uint32_t)h) * 4u) = gl;
                 cov = fmaf(pij * (gov - c0), A0, cov);
             }
             wave_sync();                      // pair data, sums and list may be rewritten
