@@ -422,7 +422,7 @@ def main():
         """What the main kernel of a path executed, by the counter profile: fraction of its time the vector ALUs
         issue, lanes active, transcendental rate against the quarter-rate unit."""
         pre = "counters." + ("fused_core_forward" if path == "forward" else "fused_core_backward") + "."
-        keys = ("valu_issue_frac", "valu_lanes_active_frac", "valu_wave_insts_per_launch", "trans_wave_insts_per_launch",
+        keys = ("valu_issue_frac", "valu_issue_frac_of_busy_cycles", "valu_lanes_active_frac", "valu_wave_insts_per_launch", "trans_wave_insts_per_launch",
                 "salu_wave_insts_per_launch", "mfma_wave_insts_per_launch", "avg_launch_us")
         got = {k: ct[pre + k] for k in keys if pre + k in ct}
         if "trans_wave_insts_per_launch" in got and "avg_launch_us" in got:
