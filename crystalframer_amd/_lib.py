@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libcrystalframer_hip.so")
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 CFH_WINDOW_REFERENCE = 0
 CFH_WINDOW_WIDE = 1
@@ -93,7 +93,7 @@ EXPORTS = ("cfh_abi_version", "cfh_last_error", "cfh_workspace_bytes", "cfh_fram
            "cfh_framed_pe_backward", "cfh_framed_pe_backward_pairwise",
            "cfh_fused_dpa_forward", "cfh_fused_dpa_backward", "cfh_pair_layout_check",
            "cfh_crystal_mean_forward", "cfh_crystal_mean_backward", "cfh_timing_enable", "cfh_timing_read",
-           "cfh_crystal_geometry", "cfh_small_linear_forward", "cfh_small_linear_dx", "cfh_linear_weight_bias_grad", "cfh_linear_weight_bias_grad_batch", "cfh_attention_inputs_forward",
+           "cfh_crystal_geometry", "cfh_small_linear_forward", "cfh_small_linear_dx", "cfh_linear_weight_bias_grad", "cfh_linear_weight_bias_grad_batch", "cfh_linear_weight_bias_grad_batch_workspace_bytes", "cfh_attention_inputs_forward",
            "cfh_attention_inputs_backward", "cfh_layer_bridge_forward", "cfh_layer_bridge_backward",
            "cfh_second_stream_fork", "cfh_second_stream_get", "cfh_second_stream_join",
            "cfh_fused_core_workspace_bytes", "cfh_fused_core_hist_words", "cfh_fused_core_forward",
@@ -174,7 +174,11 @@ def load():
         lib.cfh_crystal_geometry.restype = ctypes.c_int
         lib.cfh_crystal_geometry.argtypes = [_P, _P, _P, _P, _I64, _I64, _I64] + [_P] * 8 + [_P, ctypes.c_size_t, _P]
         lib.cfh_linear_weight_bias_grad_batch.restype = ctypes.c_int
-        lib.cfh_linear_weight_bias_grad_batch.argtypes = [ctypes.POINTER(CfhLinearGradJob), ctypes.c_int32, _P]
+        lib.cfh_linear_weight_bias_grad_batch.argtypes = [ctypes.POINTER(CfhLinearGradJob), ctypes.c_int32, _P,
+                                                          ctypes.c_size_t, _P]
+        lib.cfh_linear_weight_bias_grad_batch_workspace_bytes.restype = ctypes.c_size_t
+        lib.cfh_linear_weight_bias_grad_batch_workspace_bytes.argtypes = [ctypes.POINTER(CfhLinearGradJob),
+                                                                          ctypes.c_int32]
         _F, _I32 = ctypes.c_float, ctypes.c_int32
         lib.cfh_attention_inputs_forward.restype = ctypes.c_int
         lib.cfh_attention_inputs_forward.argtypes = [_P, _P, _P, _F, _F, _F, _F, _I64, _I32, _I32, _P, _P, _P, _P, _P]
@@ -248,6 +252,22 @@ def workspace(device: torch.device, nbytes: int) -> torch.Tensor:
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         buf[:512].zero_()          # work-queue heads and the statistics block
         _workspaces[key] = buf
+    return buf
+
+
+_wgrad_scratch = {}
+
+
+def wgrad_scratch(device: torch.device, stream_ptr, nbytes: int) -> torch.Tensor:
+    """Scratch of cfh_linear_weight_bias_grad_batch for launches on ``stream_ptr`` (which need not be the framework's
+    current stream, whose buffer ``workspace`` hands out): one buffer per (device, stream), grown on demand."""
+    key = (device.type, device.index, int(getattr(stream_ptr, "value", stream_ptr) or 0))
+    buf = _wgrad_scratch.get(key)
+    if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            _superseded.append(buf)      # a captured graph may still hold its address
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _wgrad_scratch[key] = buf
     return buf
 
 

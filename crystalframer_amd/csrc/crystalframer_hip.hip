@@ -1032,7 +1032,9 @@ int cfh_attention_inputs_backward(const float* qkv, const float* lattice_w, cons
     return finish_launch("attention_inputs_backward");
 }
 
-int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t njobs, void* stream) {
+}  // extern "C"
+namespace {
+int check_wgrad_jobs(const cfh_linear_grad_job* jobs, int32_t njobs) {
     if (njobs < 0 || (njobs > 0 && !jobs)) return fail(CFH_EINVAL, "jobs is NULL or njobs negative");
     for (int32_t j = 0; j < njobs; j++) {
         const cfh_linear_grad_job& J = jobs[j];
@@ -1043,57 +1045,141 @@ int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t n
         if ((!J.dW && !J.db) || (J.N > 0 && (!J.dy || (J.dW && !J.x))))
             return fail(CFH_EINVAL, "job %d: dy, one of dW and db, and x with dW must not be NULL", (int)j);
     }
-    hipStream_t st = (hipStream_t)stream;
-    for (int32_t first = 0; first < njobs; first += cfh::WGRAD_MAX_JOBS) {
-        const int32_t last = njobs < first + cfh::WGRAD_MAX_JOBS ? njobs : first + cfh::WGRAD_MAX_JOBS;
-        // a job whose shape and alignment allow it takes the variant with 16-byte loads
-        auto wide = [](const cfh_linear_grad_job& J) {
-            return J.dW && J.O % 64 == 0 && J.I % 64 == 0 && J.ldx % 4 == 0 && J.ldy % 4 == 0 &&
-                   ((uintptr_t)J.x | (uintptr_t)J.dy) % 16 == 0;
-        };
-        auto tiles_of = [&](const cfh_linear_grad_job& J, long& bx, long& by) {
-            bx = J.dW ? (J.I + 63) / 64 : 1;
-            by = (J.O + 63) / 64;
-        };
-        long tiles = 0;
-        for (int32_t j = first; j < last; j++)
-            if (jobs[j].N > 0) {
-                long bx, by;
-                tiles_of(jobs[j], bx, by);
-                tiles += bx * by;
-            }
-        if (tiles == 0) continue;
-        // slices of a job: the workgroups stay just below the four per compute unit that are resident at once (a few
-        // more would run as a second round and double the time)
-        int cus = device_cus();
-        if (cus <= 0) cus = 256;
-        const long target = 4L * cus - 24;
-        const int want = (int)(target / tiles > 0 ? target / tiles : 1);   // slices of a job: the workgroups stay below the 2048 that are resident at once
-                                                                        // (a few more would run as a second round and double the time)
-        cfh::WgradJobs T{};
-        int blocks = 0;
-        for (int32_t j = first; j < last; j++) {
-            const cfh_linear_grad_job& J = jobs[j];
-            if (J.N == 0) continue;
-            cfh::WgradJob& W = T.job[T.njobs++];
-            W.x = J.x; W.dy = J.dy; W.dW = J.dW; W.db = J.db;
-            W.N = (int)J.N; W.I = (int)J.I; W.O = (int)J.O; W.ldx = (int)J.ldx; W.ldy = (int)J.ldy;
+    return CFH_OK;
+}
+// The launch of the jobs [first, last): slices and workgroup numbers of every job; returns the number of tiles that
+// several slices share.
+int plan_wgrad(const cfh_linear_grad_job* jobs, int32_t first, int32_t last, cfh::WgradJobs& T) {
+    // a job whose shape and alignment allow it takes the variant with 16-byte loads
+    auto wide = [](const cfh_linear_grad_job& J) {
+        return J.dW && J.O % 64 == 0 && J.I % 64 == 0 && J.ldx % 4 == 0 && J.ldy % 4 == 0 &&
+               ((uintptr_t)J.x | (uintptr_t)J.dy) % 16 == 0;
+    };
+    auto tiles_of = [&](const cfh_linear_grad_job& J, long& bx, long& by) {
+        bx = J.dW ? (J.I + 63) / 64 : 1;
+        by = (J.O + 63) / 64;
+    };
+    long tiles = 0;
+    for (int32_t j = first; j < last; j++)
+        if (jobs[j].N > 0) {
             long bx, by;
-            tiles_of(J, bx, by);
-            W.bx = (int)bx; W.by = (int)by; W.wide = wide(J) ? 1 : 0;
-            int slices = want;
-            const int max_slices = (int)((J.N + 31) / 32);
-            if (slices > max_slices) slices = max_slices;
-            if (slices < 1) slices = 1;
-            int rows = (int)((J.N + slices - 1) / slices);
-            rows = (rows + 3) & ~3;
-            slices = (int)((J.N + rows - 1) / rows);
-            W.rows_per_slice = rows;
-            W.block0 = blocks;
-            blocks += W.bx * W.by * slices;
+            tiles_of(jobs[j], bx, by);
+            tiles += bx * by;
         }
-        T.blocks = blocks;
-        hipLaunchKernelGGL(cfh::linear_wgrad_batch_kernel, dim3((blocks + 7) & ~7), dim3(256), 0, st, T);
+    T = cfh::WgradJobs{};
+    if (tiles == 0) return 0;
+    // slices of a job: the workgroups stay just below the four per compute unit that are resident at once (a few
+    // more would run as a second round and double the time)
+    int cus = device_cus();
+    if (cus <= 0) cus = 256;
+    const long target = 4L * cus - 24;
+    const int want = (int)(target / tiles > 0 ? target / tiles : 1);
+    int blocks = 0, tile0 = 0;
+    for (int32_t j = first; j < last; j++) {
+        const cfh_linear_grad_job& J = jobs[j];
+        if (J.N == 0) continue;
+        cfh::WgradJob& W = T.job[T.njobs++];
+        W.x = J.x; W.dy = J.dy; W.dW = J.dW; W.db = J.db;
+        W.N = (int)J.N; W.I = (int)J.I; W.O = (int)J.O; W.ldx = (int)J.ldx; W.ldy = (int)J.ldy;
+        long bx, by;
+        tiles_of(J, bx, by);
+        W.bx = (int)bx; W.by = (int)by; W.wide = wide(J) ? 1 : 0;
+        int slices = want;
+        const int max_slices = (int)((J.N + 31) / 32);
+        if (slices > max_slices) slices = max_slices;
+        if (slices < 1) slices = 1;
+        int rows = (int)((J.N + slices - 1) / slices);
+        rows = (rows + 3) & ~3;
+        slices = (int)((J.N + rows - 1) / rows);
+        W.rows_per_slice = rows;
+        W.slices = slices;
+        W.block0 = blocks;
+        W.tile0 = tile0;
+        blocks += W.bx * W.by * slices;
+        if (slices > 1) tile0 += W.bx * W.by;
+    }
+    T.blocks = blocks;
+    T.split_tiles = tile0;
+    return tile0;
+}
+// Order of the jobs of a call and where one launch ends and the next begins.  With float atomics: the caller's
+// order, 32 jobs a launch.  For sums in a fixed order two jobs that add to the same memory (a weight used twice in
+// one pass) must not share a launch -- the sums reach the outputs without atomics -- so a job goes
+// to the launch after the last one that holds a job whose dW or db overlaps its own.
+void wgrad_launches(const cfh_linear_grad_job* jobs, int32_t njobs, bool fixed_order,
+                    std::vector<cfh_linear_grad_job>& ordered, std::vector<int32_t>& ends) {
+    std::vector<int> round(njobs, 0);
+    int rounds = 1;
+    if (fixed_order) {
+        auto overlap = [](const float* a, size_t na, const float* b, size_t nb) {
+            return a && b && (uintptr_t)a < (uintptr_t)(b + nb) && (uintptr_t)b < (uintptr_t)(a + na);
+        };
+        for (int32_t j = 1; j < njobs; j++)
+            for (int32_t i = 0; i < j; i++) {
+                const cfh_linear_grad_job &A = jobs[i], &B = jobs[j];
+                if (round[i] >= round[j] &&
+                    (overlap(A.dW, (size_t)A.O * A.I, B.dW, (size_t)B.O * B.I) || overlap(A.db, A.O, B.db, B.O)))
+                    round[j] = round[i] + 1;
+            }
+        for (int32_t j = 0; j < njobs; j++) rounds = round[j] + 1 > rounds ? round[j] + 1 : rounds;
+    }
+    ordered.clear();
+    ends.clear();
+    for (int r = 0; r < rounds; r++) {
+        int in_launch = 0;
+        for (int32_t j = 0; j < njobs; j++) {
+            if (round[j] != r) continue;
+            if (in_launch == cfh::WGRAD_MAX_JOBS) { ends.push_back((int32_t)ordered.size()); in_launch = 0; }
+            ordered.push_back(jobs[j]);
+            in_launch++;
+        }
+        if (in_launch) ends.push_back((int32_t)ordered.size());
+    }
+}
+}  // namespace
+extern "C" {
+
+size_t cfh_linear_weight_bias_grad_batch_workspace_bytes(const cfh_linear_grad_job* jobs, int32_t njobs) {
+    if (check_wgrad_jobs(jobs, njobs) != CFH_OK) return 0;
+    std::vector<cfh_linear_grad_job> ordered;
+    std::vector<int32_t> ends;
+    wgrad_launches(jobs, njobs, true, ordered, ends);
+    size_t need = 256;
+    int32_t first = 0;
+    for (int32_t last : ends) {
+        cfh::WgradJobs T;
+        plan_wgrad(ordered.data(), first, last, T);
+        const size_t bytes = (size_t)T.blocks * cfh::WG_PART * sizeof(float);
+        if (bytes > need) need = bytes;
+        first = last;
+    }
+    return need;
+}
+
+int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t njobs, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+    int rc = check_wgrad_jobs(jobs, njobs);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    std::vector<cfh_linear_grad_job> ordered;
+    std::vector<int32_t> ends;
+    wgrad_launches(jobs, njobs, workspace != nullptr, ordered, ends);
+    int32_t first = 0;
+    for (int32_t last : ends) {
+        cfh::WgradJobs T;
+        plan_wgrad(ordered.data(), first, last, T);
+        first = last;
+        if (T.blocks == 0) continue;
+        if (workspace) {
+            // scratch for the sums in a fixed order: a stored tile per workgroup; the launches of one call run one
+            // after the other and share it
+            if ((rc = check_workspace(workspace, workspace_bytes, (size_t)T.blocks * cfh::WG_PART * sizeof(float))))
+                return rc;
+            T.scratch.partials = reinterpret_cast<float*>(workspace);
+        }
+        hipLaunchKernelGGL(cfh::linear_wgrad_batch_kernel, dim3((T.blocks + 7) & ~7), dim3(256), 0, st, T);
+        if (workspace && T.split_tiles > 0)
+            hipLaunchKernelGGL(cfh::linear_wgrad_sum_kernel, dim3(4 * T.split_tiles), dim3(256), 0, st, T);
     }
     return finish_launch("linear_weight_bias_grad_batch");
 }

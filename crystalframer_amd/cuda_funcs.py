@@ -41,6 +41,9 @@ class KernelManager:
     # (models/indexed_lattice_multi_head_attention.py:580-588), which is what its results are held to (1e-4).
     # CFH_WINDOW_REFERENCE: the 9-bin window of the reference's CUDA kernels (+-4 sigma, dropped bin up to e^-8).
     CORE_WINDOW_MODE: int = _lib.CFH_WINDOW_WIDE
+    # weight and bias gradients of the linear layers summed in a fixed order (per-workgroup partial tiles, added by
+    # the last workgroup of a tile): the same bits from run to run.  False: float atomics, no scratch traffic.
+    DETERMINISTIC_WEIGHT_GRADIENTS: bool = True
     # skip translations lighter than 2^-24 of their pair's heaviest: below the float32 resolution of the
     # normalised sum (measured on 256 crystals: every output within 1e-6 of the unpruned result); 0 keeps all
     PRUNE_LOG2: float = 24.0
@@ -1027,7 +1030,7 @@ class _DeferredWeightGrads:
                 # no new fork: the stream was forked when the library call began, and what these jobs read
                 # was complete before that
                 _lib.check(lib.cfh_second_stream_get(ctypes.byref(side)), "cfh_second_stream_get")
-                rc = lib.cfh_linear_weight_bias_grad_batch(jobs, len(pending), side)
+                rc = _wgrad_batch(lib, jobs, len(pending), dev, side)
             _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
             return pending
         # ---- the end of the pass
@@ -1054,7 +1057,7 @@ class _DeferredWeightGrads:
             stream = _lib.current_stream_ptr(dev)
             if pending:
                 with _timed("linear_weight_bias_grad_batch", dev):
-                    rc = lib.cfh_linear_weight_bias_grad_batch(jobs, len(pending), stream)
+                    rc = _wgrad_batch(lib, jobs, len(pending), dev, stream)
             for params, calls in groups.values():
                 arr = (_lib.CfhCoreWgradJob * len(calls))()
                 for J, (go, hist, N, dst) in zip(arr, calls):
@@ -1070,6 +1073,15 @@ class _DeferredWeightGrads:
         for grad, part in fixups:
             grad.add_(part.to(grad.dtype))
         return None
+
+
+def _wgrad_batch(lib, jobs, njobs, dev, stream):
+    """cfh_linear_weight_bias_grad_batch with the scratch that makes its sums run in a fixed order (the same bits
+    from run to run); KernelManager.DETERMINISTIC_WEIGHT_GRADIENTS = False leaves the scratch out (float atomics)."""
+    if not KernelManager.DETERMINISTIC_WEIGHT_GRADIENTS:
+        return lib.cfh_linear_weight_bias_grad_batch(jobs, njobs, None, 0, stream)
+    ws = _lib.wgrad_scratch(dev, stream, lib.cfh_linear_weight_bias_grad_batch_workspace_bytes(jobs, njobs))
+    return lib.cfh_linear_weight_bias_grad_batch(jobs, njobs, _lib.ptr(ws), ws.numel(), stream)
 
 
 def _linear_param_grads(x2, g2, weights, bias):
@@ -1126,7 +1138,7 @@ def _linear_param_grads(x2, g2, weights, bias):
             J.db = None if db is None else db[0].data_ptr() + 4 * (db[1] + c0)
             J.N, J.I, J.O, J.ldx, J.ldy = x2_.shape[0], I, O, x2_.stride(0), g2_.stride(0)
         with torch.cuda.device(dev), _timed("linear_weight_bias_grad", dev):
-            rc = lib.cfh_linear_weight_bias_grad_batch(arr, len(jobs), _lib.current_stream_ptr(dev))
+            rc = _wgrad_batch(lib, arr, len(jobs), dev, _lib.current_stream_ptr(dev))
         _lib.check(rc, "cfh_linear_weight_bias_grad_batch")
     gws = [g.to(w.dtype) if g.dtype != w.dtype else g for g, w in zip(gws, weights)]
     gb_out = None if gb is None else (gb if gb.dtype == bias.dtype else gb.to(bias.dtype))

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define CFH_ABI_VERSION 12
+#define CFH_ABI_VERSION 13
 
 enum {
     CFH_OK = 0,
@@ -465,6 +465,13 @@ int cfh_linear_weight_bias_grad(const float* x, const float* dy, int64_t N, int6
  * backward pass to one call replaces one launch (plus clearing) per layer -- latency-bound at these
  * sizes -- by a launch that fills the chip.  No counterpart in the reference (autograd of
  * torch.nn.functional.linear, one GEMM per layer).
+ *
+ * The rows of a job are split over several workgroups per 64x64 tile of dW.  With workspace == NULL they add
+ * their parts with float atomics (the sums differ in the last bits from run to run).  With a workspace of at
+ * least cfh_linear_weight_bias_grad_batch_workspace_bytes(jobs, njobs) bytes every workgroup stores its part
+ * there and a second kernel adds the parts in the order of the row slices: the same bits on every run with the
+ * same jobs on the same device.  Jobs whose dW or db overlap (a weight used twice in one pass) then go to
+ * separate launches, in the jobs' order.  The workspace needs no initialisation and holds nothing between calls.
  */
 typedef struct cfh_linear_grad_job {
     const float* x;
@@ -473,7 +480,9 @@ typedef struct cfh_linear_grad_job {
     float* db;
     int64_t N, I, O, ldx, ldy;
 } cfh_linear_grad_job;
-int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t njobs, void* stream);
+size_t cfh_linear_weight_bias_grad_batch_workspace_bytes(const cfh_linear_grad_job* jobs, int32_t njobs);
+int cfh_linear_weight_bias_grad_batch(const cfh_linear_grad_job* jobs, int32_t njobs, void* workspace,
+                                      size_t workspace_bytes, void* stream);
 
 /*
  * One AdamW step (decoupled weight decay, bias-corrected moments; the update rule of torch.optim.AdamW without

@@ -299,14 +299,90 @@ def test_weight_gradient_batch_job_without_weight_sums_columns():
     jobs[0].N, jobs[0].I, jobs[0].O, jobs[0].ldx, jobs[0].ldy = 297, 1, 128, 1, 128
     jobs[1].x, jobs[1].dy, jobs[1].dW, jobs[1].db = x.data_ptr(), dy.data_ptr(), dW.data_ptr(), db.data_ptr()
     jobs[1].N, jobs[1].I, jobs[1].O, jobs[1].ldx, jobs[1].ldy = 150, 48, 40, 48, 40
-    _lib.check(lib.cfh_linear_weight_bias_grad_batch(jobs, 2, _lib.current_stream_ptr(part.device)), "batch")
+    _lib.check(lib.cfh_linear_weight_bias_grad_batch(jobs, 2, None, 0, _lib.current_stream_ptr(part.device)), "batch")
     torch.cuda.synchronize()
     assert Hh.rel_err(out, 0.5 + part.double().sum(0)) < 1e-5
     assert Hh.rel_err(dW, dy.double().t() @ x.double()) < 1e-5
     assert Hh.rel_err(db, dy.double().sum(0)) < 1e-5
     # neither output given: refused
     jobs[0].db = None
-    assert lib.cfh_linear_weight_bias_grad_batch(jobs, 1, _lib.current_stream_ptr(part.device)) != 0
+    assert lib.cfh_linear_weight_bias_grad_batch(jobs, 1, None, 0, _lib.current_stream_ptr(part.device)) != 0
+
+
+def test_weight_gradient_batch_sums_in_a_fixed_order_with_scratch():
+    """With scratch the batched weight-gradient launch adds the row slices of every tile in a fixed order: the same
+    bits on every run, the values those of the float64 products, accumulated into what dW and db held.  Jobs of both
+    kernel variants (16-byte loads: O and I multiples of 64; scalar loads with ragged edges), a bias-only job, a job
+    with a single slice (16 rows), and a second call with fewer jobs on the same scratch."""
+    from crystalframer_amd import _lib
+    lib = _lib.load()
+    gen = torch.Generator().manual_seed(78)
+    rnd = lambda *s: f32(torch.randn(*s, generator=gen, dtype=torch.float64))
+    shapes = [(3001, 128, 128, True), (3001, 128, 384, True), (1777, 48, 40, True), (16, 64, 64, True), (2500, 1, 128, False),
+              (2222, 100, 70, False)]
+    ops = []
+    for N, I, O, has_b in shapes:
+        x, dy = rnd(N, I), rnd(N, O)
+        ops.append((x, dy, rnd(O, I) if I > 1 else None, rnd(O)))
+
+    def run(n_jobs):
+        outs = []
+        jobs = (_lib.CfhLinearGradJob * n_jobs)()
+        for J, (x, dy, w0, b0) in zip(jobs, ops):
+            dW = None if w0 is None else w0.clone()
+            db = b0.clone()
+            J.x, J.dy = (None if w0 is None else x.data_ptr()), dy.data_ptr()
+            J.dW, J.db = (None if dW is None else dW.data_ptr()), db.data_ptr()
+            J.N, J.I, J.O, J.ldx, J.ldy = x.shape[0], x.shape[1], dy.shape[1], x.shape[1], dy.shape[1]
+            outs.append((dW, db))
+        need = lib.cfh_linear_weight_bias_grad_batch_workspace_bytes(jobs, n_jobs)
+        assert need > 0
+        ws = _lib.wgrad_scratch(dev(), _lib.current_stream_ptr(dev()), need)
+        _lib.check(lib.cfh_linear_weight_bias_grad_batch(jobs, n_jobs, _lib.ptr(ws), ws.numel(),
+                                                         _lib.current_stream_ptr(dev())), "batch")
+        torch.cuda.synchronize()
+        # too small a scratch is refused
+        assert lib.cfh_linear_weight_bias_grad_batch(jobs, n_jobs, _lib.ptr(ws), 256,
+                                                     _lib.current_stream_ptr(dev())) != 0
+        return outs
+
+    first = run(len(ops))
+    for (dW, db), (x, dy, w0, b0) in zip(first, ops):
+        if dW is not None:
+            assert Hh.rel_err(dW, w0.double() + dy.double().t() @ x.double()) < 1e-5
+        assert Hh.rel_err(db, b0.double() + dy.double().sum(0)) < 1e-5
+    for _ in range(3):
+        again = run(len(ops))
+        for (dW, db), (dW2, db2) in zip(first, again):
+            assert dW is None or torch.equal(dW, dW2)
+            assert torch.equal(db, db2)
+    # fewer jobs: other slice counts per tile, the same scratch
+    fewer = run(2)
+    for (dW, db), (x, dy, w0, b0) in zip(fewer, ops):
+        assert Hh.rel_err(dW, w0.double() + dy.double().t() @ x.double()) < 1e-5
+        assert Hh.rel_err(db, b0.double() + dy.double().sum(0)) < 1e-5
+    assert all(torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) for a, b in zip(fewer, run(2)))
+
+    # two jobs that add to the same dW and db (a weight used twice in one pass): both arrive, in the jobs' order
+    def shared():
+        x, dy, w0, b0 = ops[0]
+        x2, dy2 = ops[1][0], ops[1][1][:, :128].contiguous()
+        dW, db = w0.clone(), b0.clone()
+        jobs = (_lib.CfhLinearGradJob * 2)()
+        for J, (xx, yy) in zip(jobs, ((x, dy), (x2, dy2))):
+            J.x, J.dy, J.dW, J.db = xx.data_ptr(), yy.data_ptr(), dW.data_ptr(), db.data_ptr()
+            J.N, J.I, J.O, J.ldx, J.ldy = xx.shape[0], 128, 128, 128, 128
+        ws = _lib.wgrad_scratch(dev(), _lib.current_stream_ptr(dev()),
+                                lib.cfh_linear_weight_bias_grad_batch_workspace_bytes(jobs, 2))
+        _lib.check(lib.cfh_linear_weight_bias_grad_batch(jobs, 2, _lib.ptr(ws), ws.numel(),
+                                                         _lib.current_stream_ptr(dev())), "batch")
+        torch.cuda.synchronize()
+        ref = w0.double() + dy.double().t() @ x.double() + dy2.double().t() @ x2.double()
+        assert Hh.rel_err(dW, ref) < 1e-5
+        assert Hh.rel_err(db, b0.double() + dy.double().sum(0) + dy2.double().sum(0)) < 1e-5
+        return dW, db
+    s1, s2 = shared(), shared()
+    assert torch.equal(s1[0], s2[0]) and torch.equal(s1[1], s2[1])
 
 
 def test_linear_deferred_gradients_stacked_accumulated_and_nonleaf():

@@ -86,15 +86,20 @@ def test_model_frames_agree_with_oracle_frames(core_mode):
     assert (used[0].cpu().double() - f1)[clear].abs().max() < 1e-4
 
 
-def test_training_step_as_hip_graph_matches_eager_on_every_replay():
+@pytest.mark.parametrize("fixed_order", [True, False])
+def test_training_step_as_hip_graph_matches_eager_on_every_replay(fixed_order):
     """The whole training step (geometry, forward, loss, backward, AdamW) captured as one HIP graph:
     every replay is compared with an eager twin of the same model, with eager work and
-    synchronisations between the replays."""
+    synchronisations between the replays.  With the weight gradients of the linear layers summed in a fixed order
+    (KernelManager.DETERMINISTIC_WEIGHT_GRADIENTS, the default) every kernel of the step adds in a fixed order and
+    the twins stay bit-equal; with float atomics they drift apart as bounded below."""
     import crystalframer_amd as cf
     from crystalframer_amd import latticeformer, params, synthetic
     KM = cf.KernelManager
     dev = torch.device("cuda:0")
     saved = (KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE)
+    saved_order = KM.DETERMINISTIC_WEIGHT_GRADIENTS
+    KM.DETERMINISTIC_WEIGHT_GRADIENTS = fixed_order
     mp = params.ModelParams(num_layers=2)
     cb = synthetic.make_batch(24, atoms="uniform", atoms_lo=1, atoms_hi=9, len_lo=3.0, len_hi=9.0,
                               ang_lo=65.0, ang_hi=115.0, seed=21).to(dev)
@@ -142,19 +147,22 @@ def test_training_step_as_hip_graph_matches_eager_on_every_replay():
             torch.cuda.synchronize()
             le, lg = float(loss_e), float(loss_g)
             assert abs(le - lg) < 2e-4 * abs(le), (replay, le, lg)
+            assert le == lg or not fixed_order, (replay, le, lg)
             junk = torch.tanh(junk @ junk / 512.0)          # eager work between the replays
             assert torch.isfinite(junk).all()
-        # The two twins are not bit-equal: the weight gradients of the linear layers are summed with float atomics, and
-        # AdamW's first steps move every element by about lr whatever the size of its gradient, so an element whose
-        # tiny gradient differs in the last bits (or in sign) drifts by up to 2 lr per step.  Bound: two such steps
-        # for any element, a hundredth of a step on average.
+        # With float atomics the twins are not bit-equal, and AdamW's first steps move every element by about lr
+        # whatever the size of its gradient, so an element whose tiny gradient differs in the last bits (or in sign)
+        # drifts by up to 2 lr per step.  Bound: two such steps for any element, a hundredth of a step on average.
         lr = 1e-3
         for (n, pe), (_, pg) in zip(model_e.named_parameters(), model_g.named_parameters()):
             diff = (pg.detach() - pe.detach()).abs()
+            if fixed_order:
+                assert float(diff.max()) == 0.0, n
             assert float(diff.max()) <= 4 * lr, n
             assert float(diff.mean()) <= 0.02 * lr, n
     finally:
         KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE = saved
+        KM.DETERMINISTIC_WEIGHT_GRADIENTS = saved_order
 
 
 def test_bridged_encoder_equals_the_modules_own_forward():
