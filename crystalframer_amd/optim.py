@@ -5,7 +5,10 @@ The reference trains with ``torch.optim.AdamW`` (models/regression.py:298-301). 
 kernel for all parameter tensors of a group (``cfh_adamw_step_batch``) instead of the framework's multi-tensor
 machinery, which for a model of many small tensors is bound by its bookkeeping.  The step count lives on the device,
 so a captured step keeps counting from replay to replay; ``lr`` and the other scalars are read on the host when
-``step`` is called (a captured step replays the values of its capture).
+``step`` is called (a captured step replays the values of its capture: a learning-rate scheduler, as the
+reference's trainer uses, needs the step captured again, or run eagerly, whenever it changes ``lr``).  The step
+count is one word per parameter GROUP, not per parameter as in torch.optim.AdamW: all parameters of a group take
+their first step together (a parameter that gets its first gradient later is bias-corrected with the group's count).
 """
 import ctypes
 
