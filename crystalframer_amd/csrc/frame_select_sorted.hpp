@@ -8,8 +8,13 @@
 //   * first axis: the best candidate of a pair is its nearest valid image (d^2 > 1e-5).  The unshifted image is at
 //     distance |r|, so the nearest one has |s| <= 2 |r|; when the unshifted image is the atom itself (|r| = 0) the
 //     shortest non-zero shift s_1 gives d <= |r| + |s_1|, hence |s| <= 2 |r| + |s_1|.  Only that prefix is read.
-//   * second axis: score = q.k + a d^2 + log(max(1 - |cos|, 1e-5)) <= q.k + a d^2.  A first sweep over the same
-//     prefixes gives a lower bound `best` of the maximum; a candidate of pair j can then only matter if
+//     With the batch's table of every pair's nearest valid image (pair_nearest_kernel: its d^2 and its position in
+//     the sorted table) most pairs are not looked at at all: no candidate of pair j scores above
+//     hi_j = q.k_j + a (d_j^2 - noise / 2), and its nearest valid image scores at least lo_j = q.k_j + a (d_j^2 + noise / 2),
+//     so only the pairs with hi_j >= max_j lo_j can hold the maximum -- one or two of a row, unless images tie.
+//   * second axis: score = q.k + a d^2 + log(max(1 - |cos|, 1e-5)) <= q.k + a d^2.  A first sweep -- over every
+//     pair's nearest valid image when the batch's table names it, else over the first axis' prefixes -- gives a
+//     lower bound `best` of the maximum; a candidate of pair j can then only matter if
 //     a d^2 >= best - q.k_j, i.e. d^2 <= need_j = (best - q.k_j) / a: no candidate when need_j < 0, else only
 //     shifts with |s| <= |r| + sqrt(need_j).  The second sweep reads those prefixes.
 // The tie-breaking noise moves a score by at most |a| noise / 2 (first axis) or noise / 2 (second): the bounds are
@@ -138,6 +143,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
         const float s1 = sorted ? tab[1].w : 0.0f;      // shortest non-zero shift (entry 0 is the zero shift)
 
         float dvalid = -1.0f;                           // this lane's pair: d^2 of its nearest valid image, when known
+        float dvraw = -1.0f;                            // ... as the batch's table holds it (table position in the low bits)
         float f1x = 0.f, f1y = 0.f, f1z = 0.f;          // first axis
         float f2x = 0.f, f2y = 0.f, f2z = 0.f;          // second axis before orthogonalisation
         unsigned long long n_seen = 0;
@@ -145,6 +151,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
         for (int pass = 0; pass < 2; pass++) {
             Best best;
             best.score = -3.0e38f; best.e = 0x7fffffff; best.t = 0x7fffffff;
+            float row_lb = -3.0e38f;      // first axis: the best score that some pair of the row is known to reach
             // sweeps: the first axis needs one; the second a first one for the bound and one with the bound
             const int nsweeps = pass == 1 ? 2 : 1;
             for (int sw = 0; sw < nsweeps; sw++) {
@@ -155,7 +162,11 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                     // the pairs of an atom point at consecutive atoms)
                     float4 rq = make_float4(0.f, 0.f, 0.f, 0.f);
                     // (made for the table's box, which every other box of the launch contains: an upper bound there)
-                    if (sw == 0 && C.pair_near && lane < npc) dvalid = C.pair_near[e0 + pb + lane].y;
+                    // (the table's value is rounded down by up to 2^-16 of itself: an upper bound is wanted here)
+                    if (sw == 0 && C.pair_near && lane < npc) {
+                        dvraw = C.pair_near[e0 + pb + lane].y;
+                        dvalid = dvraw * (1.0f + 0x1p-15f);
+                    }
                     if (npairs > WAVE || (pass == 0 && sw == 0)) {
                         if (lane < npc) {
                             const int e = e0 + pb + lane;
@@ -199,6 +210,45 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                             reach = need >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(need), 1e-3f) : -1.0f;
                         }
                     }
+                    // With the usual box the batch's table names every pair's nearest valid image (d^2 within
+                    // [dv_lo, dv_hi], position near_t in the sorted table).
+                    const bool near_known = sorted && C.pair_near != nullptr && lane < npc && dvraw >= 0.0f && dvraw < 1.0e37f;
+                    const float dv_lo = __uint_as_float(__float_as_uint(dvraw) & ~(uint32_t)(FC_TCAP - 1));
+                    const float dv_hi = dv_lo * (1.0f + 0x1p-15f);
+                    if (pass == 1 && sw == 0 && sorted && C.pair_near) {
+                        // ---- lower bound of the second axis' best score: every pair's nearest valid image, one per lane
+                        // (the same arithmetic as in the loop over candidates below, which meets this image again)
+                        wave_sync();              // pq (and the phases of the noise) are staged
+                        const float4 v = tab[near_known ? (int)(__float_as_uint(dvraw) & (uint32_t)(FC_TCAP - 1)) : 0];
+                        const int t = (int)(__float_as_uint(v.w) & (uint32_t)(FC_TCAP - 1));
+                        const float dx = rq.x + v.x, dy = rq.y + v.y, dz = rq.z + v.z;
+                        const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+                        const float rinv = hw_rsq(d2);
+                        const float ac = fabsf((dx * f1x + dy * f1y + dz * f1z) * rinv);
+                        float score = fmaf(a, d2, rq.w) + hw_log2(fmaxf(1.0f - ac, 1e-5f)) * LN2;
+                        if (noisy) {
+                            const float un = __builtin_amdgcn_fractf(fmaf((float)t, 0.61803399f, sh.ph[lane]));
+                            score += (un - 0.5f) * P.noise;
+                        }
+                        const int e = e0 + pb + lane;
+                        if (near_known && d2 > 1e-5f && ac < 0.9999f && better(score, e, t, best.score, best.e, best.t)) {
+                            best.score = score; best.e = e; best.t = t;
+                        }
+                        n_seen += (unsigned long long)npc;
+                        continue;
+                    }
+                    // First axis: no candidate of a pair scores above hi (its nearest valid image with the noise at its
+                    // most favourable), and that image scores at least lo.  A pair whose hi stays below the best lo seen
+                    // so far in the row cannot hold the maximum: its candidates are left out.  (The margins cover the
+                    // rounding of d^2 in the table of nearest images and of the scores.)
+                    bool contender = true;
+                    if (pass == 0 && sorted && C.pair_near) {
+                        const float hi = near_known ? fmaf(a, dv_lo - 0.5f * nz, rq.w) : 3.0e38f;
+                        const float lo_s = near_known ? fmaf(a, dv_hi + 0.5f * nz, rq.w) : -3.0e38f;
+                        const float mg = 2e-6f * (fabsf(rq.w) + fabsf(a) * (dv_hi + nz)) + 1e-30f;
+                        row_lb = fmaxf(row_lb, uniform_f(wave_maxf(near_known ? lo_s - mg : -3.0e38f)));
+                        contender = hi + mg >= row_lb;
+                    }
                     for (int ch = 0; ch < nchunks; ch++) {
                         const int t0c = ch * FC_TCAP;
                         const int cnt = sorted ? bx.T : min(FC_TCAP, bx.T - t0c);
@@ -221,7 +271,7 @@ __device__ __forceinline__ void frame_item_body(const CoreArgs& C, FrameShared& 
                                 lo = le ? mid + 1 : lo;
                                 hi = le ? hi : mid;
                             }
-                            mine = min(lo, cnt);
+                            mine = contender ? min(lo, cnt) : 0;
                         }
                         // The candidates of the pairs laid end to end; which pair candidate c belongs to comes without a
                         // search: a bit per candidate marks where the run of a pair begins, so the pair of c is the
@@ -464,10 +514,38 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
                     const float myqk = qk_s[row][min(pj, nst - 1)];
                     const float r2 = fmaf(r4.x, r4.x, fmaf(r4.y, r4.y, r4.z * r4.z));
                     const float r = hw_sqrt(r2);
+                    // the pair's nearest valid image, when the batch's table of them is there: its d^2 lies in
+                    // [dv_lo, dv_hi], its position in the sorted table is near_t
+                    const bool near_known = r4.w >= 0.0f && r4.w < 1.0e37f;
+                    const float dv_lo = __uint_as_float(__float_as_uint(r4.w) & ~(uint32_t)(FC_TCAP - 1));
+                    const float dv_hi = dv_lo * (1.0f + 0x1p-15f);
+                    const int near_t = (int)(__float_as_uint(r4.w) & (uint32_t)(FC_TCAP - 1));
+                    if (pass == 1 && sw == 0 && C.pair_near) {
+                        // ---- lower bound of the second axis' best score: every pair's nearest valid image, one per lane
+                        // (the same arithmetic as in the loop over candidates below, which meets this image again)
+                        const float4 v = tab[near_known ? near_t : 0];
+                        const int t = (int)(__float_as_uint(v.w) & (uint32_t)(FC_TCAP - 1));
+                        const float dx = r4.x + v.x, dy = r4.y + v.y, dz = r4.z + v.z;
+                        const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
+                        const float rinv = hw_rsq(d2);
+                        const float ac = fabsf((dx * f1x + dy * f1y + dz * f1z) * rinv);
+                        float score = fmaf(a, d2, myqk) + hw_log2(fmaxf(1.0f - ac, 1e-5f)) * LN2;
+                        if (noisy) {
+                            const float phase = sh.ph_s[1][row][min(pj, nst - 1)];
+                            const float un = __builtin_amdgcn_fractf(fmaf((float)t, 0.61803399f, phase));
+                            score += (un - 0.5f) * P.noise;
+                        }
+                        const int e = e0 + pb + pj;
+                        if (pair_ok && near_known && d2 > 1e-5f && ac < 0.9999f && better(score, e, t, best.score, best.e, best.t)) {
+                            best.score = score; best.e = e; best.t = t;
+                        }
+                        n_seen += (unsigned long long)__popcll(ballot(pair_ok));
+                        continue;
+                    }
                     float reach;
                     if (sw == 0) {
-                        reach = r4.w >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(r4.w + nz), 1e-3f)
-                                             : fmaf(1.0001f, fmaf(2.0f, r, (r2 > 1e-5f ? 0.0f : s1) + sq_nz), 1e-3f);
+                        reach = near_known ? fmaf(1.0001f, r + hw_sqrt(dv_hi + nz), 1e-3f)
+                                           : fmaf(1.0001f, fmaf(2.0f, r, (r2 > 1e-5f ? 0.0f : s1) + sq_nz), 1e-3f);
                     } else if (bound > -1.0e38f) {
                         const float need = (bound - myqk - 0.5f * nz) * inv_a;
                         reach = need >= 0.0f ? fmaf(1.0001f, r + hw_sqrt(need), 1e-3f) : -1.0f;
@@ -485,6 +563,17 @@ __device__ __forceinline__ void frame_quad_body(const CoreArgs& C, FrameQuadShar
                             hi = le ? hi : mid;
                         }
                         cnt = pair_ok ? min(lo, bx.T) : 0;
+                    }
+                    if (pass == 0 && C.pair_near) {
+                        // First axis: no candidate of a pair scores above hi (its nearest valid image with the noise at
+                        // its most favourable), and its nearest valid image scores at least lo.  A pair whose hi stays
+                        // below the best lo of the row cannot hold the maximum: its candidates are left out.  (The
+                        // margins cover the rounding of d^2 in the table of nearest images and of the scores.)
+                        const float hi = near_known ? fmaf(a, dv_lo - 0.5f * nz, myqk) : 3.0e38f;
+                        const float lo_s = near_known ? fmaf(a, dv_hi + 0.5f * nz, myqk) : -3.0e38f;
+                        const float mg = 2e-6f * (fabsf(myqk) + fabsf(a) * (dv_hi + nz)) + 1e-30f;
+                        const float lb = row_max(pair_ok ? lo_s - mg : -3.0e38f);
+                        if (!(hi + mg >= lb)) cnt = 0;
                     }
                     int incl = cnt;                        // inclusive prefix within the row
                     incl += dpp_movei<0x111>(incl);

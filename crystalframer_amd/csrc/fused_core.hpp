@@ -97,7 +97,8 @@ struct CoreArgs {
     const float* v;               // (N,H,16)
     const float4* sorted_tab;     // (B, FC_TCAP) shifts of the usual box sorted by length, w = length; or null
     const float2* pair_near;      // (E) per pair over that box: smallest d^2 of all images, of the images with
-                                  // d^2 > 1e-5 (what the frame search may point at); or null
+                                  // d^2 > 1e-5 (what the frame search may point at; low 7 bits: that image's
+                                  // position in the sorted table); or null
     int32_t table_R;              // half-width that table was made for
     int32_t slow_wgs;             // leading wavefronts of the main kernels that take the listed slow records first, by
                                   // rank over all lists: wavefront w the rank w; the listed records of higher rank are
@@ -177,7 +178,7 @@ __global__ __launch_bounds__(FC_TCAP) void sorted_shifts_kernel(const float* __r
 }
 
 // Per pair, over the usual box of its crystal: the smallest squared distance of all images and of the images with
-// d^2 > 1e-5.  Both depend on the geometry alone, not on the head or the layer, so they are made once per batch:
+// d^2 > 1e-5, the latter with the position of that image in the sorted table in its low 7 bits.  Both depend on the geometry alone, not on the head or the layer, so they are made once per batch:
 // the lattice sums of an item with the usual box then need no sweep for the nearest image, and the frame search
 // knows how far into the sorted table a pair's best first-axis candidate can sit.  Eight lanes per pair, eight
 // entries of the sorted table at a time; the sorted order ends the loop once |s| - |r| exceeds the larger of the
@@ -194,6 +195,8 @@ __global__ __launch_bounds__(256) void pair_nearest_kernel(const float* __restri
     const float4* tab = sorted_tab + (size_t)b * FC_TCAP;
     const float rx = rpos[(size_t)e * 3 + 0], ry = rpos[(size_t)e * 3 + 1], rz = rpos[(size_t)e * 3 + 2];
     const float r = sqrtf(fmaf(rx, rx, fmaf(ry, ry, rz * rz)));
+    // (dval carries the table position of its image in its low 7 bits -- it is rounded down by at most 2^-16 of itself,
+    // which the margins of every test that uses it cover -- so that the minimum over the lanes brings the position along)
     float dall = 3.0e38f, dval = 3.0e38f;
     for (int t0 = 0; t0 < T0; t0 += 8) {
         // the first entry of the group decides for all eight lanes whether the walk goes on
@@ -203,7 +206,8 @@ __global__ __launch_bounds__(256) void pair_nearest_kernel(const float* __restri
             const float dx = rx + v.x, dy = ry + v.y, dz = rz + v.z;
             const float d2 = fmaf(dx, dx, fmaf(dy, dy, dz * dz));
             dall = fminf(dall, d2);
-            if (d2 > 1e-5f) dval = fminf(dval, d2);
+            if (d2 > 1e-5f)
+                dval = fminf(dval, __uint_as_float((__float_as_uint(d2) & ~(uint32_t)(FC_TCAP - 1)) | (uint32_t)(t0 + sub)));
         }
         dall = half_min(dall);
         dval = half_min(dval);
