@@ -252,6 +252,49 @@ def test_sorted_frame_search_mixed_boxes_fixed_box_and_long_rows(noise):
     assert torch.equal(fr, ref)
 
 
+@pytest.mark.parametrize("noise", [0.0, 1e-5])
+def test_sorted_frame_search_on_symmetric_crystals_with_exact_ties(noise):
+    """Cubic cells with atoms at special positions (simple cubic, body-centred, face-centred, a 2 x 1 x 1 supercell) and
+    the SAME query, key and Gaussian width on every atom: several pairs and several translations reach exactly the
+    same best score, so the winner is whatever the tie rule says (lowest pair, then lowest translation in the
+    reference's loop order).  The sorted search -- which looks only at the pairs whose nearest valid image can hold
+    the maximum -- must keep every tied candidate: its frames equal the box search's bit for bit."""
+    import crystalframer_amd as cf
+    from oracle import torch_oracle as TO
+    KM = cf.KernelManager
+    KM.SYMM_BREAK_NOISE, KM.NOISE_SEED, KM.NOISE_SEED_DEVICE = noise, 4321, None
+    cells = [
+        (4.0, [[0, 0, 0]]),
+        (3.5, [[0, 0, 0], [0.5, 0.5, 0.5]]),
+        (5.0, [[0, 0, 0], [0.5, 0.5, 0], [0.5, 0, 0.5], [0, 0.5, 0.5]]),
+        (4.5, [[0, 0, 0], [0.5, 0, 0], [0.25, 0.5, 0.5], [0.75, 0.5, 0.5]]),
+        (6.0, [[0.25, 0.25, 0.25], [0.75, 0.75, 0.25], [0.75, 0.25, 0.75], [0.25, 0.75, 0.75],
+               [0.75, 0.75, 0.75], [0.25, 0.25, 0.75], [0.25, 0.75, 0.25], [0.75, 0.25, 0.25]]),
+    ]
+    P = Hh.make_problem(num_crystals=len(cells), atoms_lo=1, atoms_hi=1, seed=77)
+    sizes = [len(f) for _, f in cells]
+    P.sizes = sizes
+    P.tvecs = torch.stack([torch.eye(3, dtype=torch.float64) * a for a, _ in cells])
+    P.pos = torch.cat([torch.tensor(f, dtype=torch.float64) * a for a, f in cells])
+    P.batch = torch.repeat_interleave(torch.arange(len(cells)), torch.tensor(sizes))
+    P.edges, P.rpos, recip, P.vcell = TO.geometry(P.pos, P.tvecs, P.sizes)
+    P.rpos = P.rpos.float().double()
+    P.rvlen = torch.norm(recip, 2, dim=-1).float().double()
+    P.N, P.E = P.pos.shape[0], P.edges.shape[1]
+    gen = torch.Generator().manual_seed(5)
+    one = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64).float().double()
+    P.q = (one(1, Hh.H, Hh.DH) / 4).expand(P.N, -1, -1).contiguous()
+    P.k = one(1, Hh.H, Hh.DH).expand(P.N, -1, -1).contiguous()
+    P.v = one(P.N, Hh.H, Hh.DH)
+    P.a = TO.gaussian_coefficient(one(1, Hh.H)).float().double().expand(P.N, -1).contiguous()
+    fr, ref = _frames_both_ways(P)
+    assert torch.equal(fr, ref)
+    fr, ref = _frames_both_ways(P, cutoff=None)
+    assert torch.equal(fr, ref)
+    det = torch.linalg.det(fr.permute(1, 2, 0, 3).double())
+    assert float((det - 1).abs().max()) < 1e-4
+
+
 def test_fused_core_one_atom_crystals_and_empty_batch():
     from crystalframer_amd import cuda_funcs as F
     P = Hh.make_problem(num_crystals=5, atoms_lo=1, atoms_hi=1, seed=41)
