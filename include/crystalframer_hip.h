@@ -331,7 +331,9 @@ int cfh_framed_pe_backward_pairwise(const cfh_params* p, const float* a_ih, cons
  *                           reads it (filled by an earlier call, forward or backward, with the same tvecs and
  *                           params), else it fills it.
  *   pair_near (E,2)         per pair over that box: the smallest squared distance of all images and of the images
- *                           with d^2 > 1e-5 (geometry alone: made once per batch, together with shift_table and
+ *                           with d^2 > 1e-5, the second with the position of its image in shift_table in its low
+ *                           7 bits (an opaque buffer: the library writes and reads it; geometry alone: made once
+ *                           per batch, together with shift_table and
  *                           under the same ready word; the lattice sums then skip their sweep for the nearest
  *                           image and the frame search reads shorter prefixes of the table).  Only the forward
  *                           uses it; without it the forward makes it in its workspace.
